@@ -1,0 +1,227 @@
+/*
+ * tqhip.h -- C ABI of libtqhip.so: the PolarQuant KV-cache hot path on MI355X (gfx950).
+ *
+ * One entry point per GPU kernel launcher of the reference (each of which is a
+ * Python wrapper around mx.fast.metal_kernel); the citation on each declaration
+ * is the reference interface it replaces.  A reference-side binding is a ctypes
+ * stub that passes device pointers and sizes.
+ *
+ * Conventions
+ *  - every pointer is a DEVICE pointer unless the comment says "host"; the two small tables,
+ *    `boundaries` and `centroids` (at most 16 floats), are always HOST pointers: they travel
+ *    to the kernels by value;
+ *  - the library never allocates or frees device memory: outputs and workspace
+ *    are caller-owned;
+ *  - launches are asynchronous on `stream` (a hipStream_t passed as void*);
+ *  - every function returns 0 on success or a negative tq_status; the text of
+ *    the last failure on the calling thread is tq_last_error();
+ *  - packed layout: element e of a vector lives in uint32 word e / vpw at bit
+ *    offset (e % vpw) * bits, vpw = 32/16/10/8 for bits = 1/2/3/4
+ *    (reference turboquant_mlx/packing.py:16-56);
+ *  - "KV addressing": sequence s, kv head h, position p of a packed / norm / fp16-K
+ *    tensor is the row  s * seq_stride + h * head_stride + (first[s] + p)
+ *    where strides are counted in ROWS (a row = pdim words, 1 norm, or dim halfs),
+ *    first[s] = seq_offsets ? seq_offsets[s] : 0 and the sequence length is
+ *    seq_offsets ? seq_offsets[s+1] - seq_offsets[s] : seq_len.
+ *    A cache tensor [B, H, T_alloc, *] uses seq_stride = H*T_alloc, head_stride =
+ *    T_alloc, seq_offsets = NULL; a ragged batch [H, sum(L), *] uses seq_stride = 0,
+ *    head_stride = sum(L) and seq_offsets[n_seq+1].
+ */
+#ifndef TQHIP_H
+#define TQHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* tq_stream_t;
+
+enum tq_dtype { TQ_F32 = 0, TQ_F16 = 1, TQ_BF16 = 2 };
+
+enum tq_status {
+  TQ_OK = 0,
+  TQ_ERR_NULL = -1,       /* a required pointer is NULL */
+  TQ_ERR_DIM = -2,        /* dim not a power of two or out of range */
+  TQ_ERR_BITS = -3,       /* bits not in 1..4 */
+  TQ_ERR_NREP = -4,       /* n_q_heads != n_kv_heads * n_rep, or n_rep < 1 */
+  TQ_ERR_ALIGN = -5,      /* pointer not aligned for its element type */
+  TQ_ERR_DTYPE = -6,      /* unknown tq_dtype */
+  TQ_ERR_BLOCK = -7,      /* block_size outside 1..32 */
+  TQ_ERR_WORKSPACE = -8,  /* workspace too small */
+  TQ_ERR_ARG = -9,        /* other invalid argument (negative size, ...) */
+  TQ_ERR_UNSUPPORTED = -10, /* valid request this build has no kernel for */
+  TQ_ERR_HIP = -100       /* a HIP call failed; tq_last_error() holds hipGetErrorString */
+};
+
+/* encode variants */
+enum tq_encode_variant {
+  TQ_ENCODE_MLX = 0,   /* bits equal to PolarQuantizer.quantize (quantizer.py:85-106):
+                          compares (w*s)/s, s = float32(1/sqrt(dim)) */
+  TQ_ENCODE_METAL = 1  /* bits equal to the fused Metal encoder (metal.py:66-77):
+                          compares the raw butterfly output w */
+};
+
+/* which fused decode kernel a workspace query is for */
+enum tq_op {
+  TQ_OP_SPARSE_V = 0,
+  TQ_OP_FLASH_DECODE = 1,
+  TQ_OP_VONLY_DECODE = 2
+};
+
+int tq_version(void);
+const char* tq_last_error(void);            /* host string, valid until the next failing call on this thread */
+const char* tq_status_string(int status);   /* host string */
+
+/*
+ * Fused encode: per-vector L2 norm -> x/max(n,1e-8) -> sign flip -> Walsh-Hadamard
+ * butterfly -> Lloyd-Max boundary count -> bit packing.
+ * Replaces fused_quantize (reference turboquant_mlx/metal.py:147-196, kernel 14-101) and,
+ * with TQ_ENCODE_MLX, PolarQuantizer.quantize + pack_indices (quantizer.py:75-106,
+ * packing.py:26-56).
+ *   x          [n_groups*rows_per_group, dim] contiguous, dtype x_dtype
+ *   signs      [dim] float, +-1 (device);  boundaries [2^bits - 1] float, ascending (HOST)
+ *   packed     row r = (g, i) is written at packed + (g*packed_group_stride + i) * pdim words
+ *   norms      row r is written at norms + g*norms_group_stride + i   (float32, un-clamped norm)
+ * With n_groups = 1 this is the plain (n_vecs, dim) -> (n_vecs, pdim), (n_vecs,) call.
+ */
+int tq_encode(const void* x, int x_dtype, const float* signs, const float* boundaries,
+              uint32_t* packed, float* norms,
+              int64_t n_groups, int64_t rows_per_group,
+              int64_t packed_group_stride, int64_t norms_group_stride,
+              int dim, int bits, int variant, tq_stream_t stream);
+
+/*
+ * Dequantise packed rows: out = ((butterfly(c[idx]*s) * s) * signs) * norm, s = 1/sqrt(dim).
+ * Replaces packed_dequantize (kernels.py:123-155, kernel 14-55; out_dtype TQ_F32) and
+ * dequant_fp16 (metal.py:199-232, kernel 104-141; out_dtype TQ_F16).  TQ_BF16 also accepted.
+ * Row addressing as in tq_encode, plus out_group_stride (rows of dim elements).
+ */
+int tq_dequant(const uint32_t* packed, const float* norms, const float* centroids,
+               const float* signs, void* out, int out_dtype,
+               int64_t n_groups, int64_t rows_per_group,
+               int64_t packed_group_stride, int64_t norms_group_stride, int64_t out_group_stride,
+               int dim, int bits, tq_stream_t stream);
+
+/*
+ * q_rot[h] = butterfly(q[h] * signs), no 1/sqrt(dim).
+ * Replaces prerotate_query (metal_kernels_v4.py:119-150, kernel 37-62).
+ *   q [n_heads, dim] dtype q_dtype -> q_rot [n_heads, dim] float32
+ */
+int tq_prerotate_query(const void* q, int q_dtype, const float* signs, float* q_rot,
+                       int64_t n_heads, int dim, tq_stream_t stream);
+
+/*
+ * scores[h, p] = (sum_e c[idx[h/n_rep, p, e]] * q_rot[h, e]) * k_norms[h/n_rep, p] * (1/dim).
+ * Replaces prerot_fused_qk_scores (metal_kernels_v4.py:153-221, kernel 71-113).
+ *   q_rot [n_kv*n_rep, dim] f32; k_packed / k_norms: one sequence, head_stride in rows;
+ *   scores [n_kv*n_rep, seq_len] f32 contiguous.
+ */
+int tq_prerot_qk_scores(const float* q_rot, const uint32_t* k_packed, const float* k_norms,
+                        const float* centroids, float* scores,
+                        int n_kv_heads, int n_rep, int64_t seq_len,
+                        int64_t packed_head_stride, int64_t norms_head_stride,
+                        int dim, int bits, tq_stream_t stream);
+
+/*
+ * scores[h, p] = <dequant(K[h, p]), query[h]>, one butterfly per K row (MHA only).
+ * Replaces packed_fused_qk_scores (kernels.py:158-196, kernel 58-117); kept because the
+ * reference uses it as the cross-check of the pre-rotated path (tests/test_prerot.py:81-88).
+ */
+int tq_packed_qk_scores(const float* query, const uint32_t* k_packed, const float* k_norms,
+                        const float* centroids, const float* signs, float* scores,
+                        int n_heads, int64_t seq_len,
+                        int64_t packed_head_stride, int64_t norms_head_stride,
+                        int dim, int bits, tq_stream_t stream);
+
+/*
+ * scores[h, p] = <q[h], K[h/n_rep, p]> * scale for fp16 keys (the K side of a V-only cache,
+ * v_only_cache.py:24-38; the reference computes this inside the stock SDPA).
+ *   q [n_kv*n_rep, dim] dtype q_dtype; k fp16 rows of dim halfs, head_stride in rows.
+ */
+int tq_dense_qk_scores(const void* q, int q_dtype, const void* k_f16, float* scores,
+                       int n_kv_heads, int n_rep, int64_t seq_len, int64_t k_head_stride,
+                       int dim, float scale, tq_stream_t stream);
+
+/*
+ * weights[r, :] = softmax(scores[r, :] * scale + mask[r * mask_row_stride, :]).
+ * Replaces the `* attn_scale`, `+ mask`, mx.softmax steps of turboquant_attention
+ * (fused_attention.py:78-94).  mask may be NULL; mask_row_stride is 0 for a mask shared by
+ * all rows or seq_len for one row per score row.  In-place (weights == scores) is allowed.
+ */
+int tq_softmax_rows(const float* scores, const float* mask, int64_t mask_row_stride,
+                    float* weights, int64_t n_rows, int64_t seq_len, float scale,
+                    tq_stream_t stream);
+
+/*
+ * out[h] = butterfly(sum_{p: !(w[h,p] < thr)} w[h,p] * norm[h/n_rep,p] * c[idx[h/n_rep,p,:]])
+ *          * signs * (1/dim),   thr = max(threshold, 0).
+ * Replaces sparse_v_matvec (sparse_v.py:94-186, kernel 32-88).  KV positions are split
+ * across workgroups; partial sums go through `workspace` and a second pass applies the one
+ * butterfly.   weights [n_kv*n_rep, seq_len] f32; out [n_kv*n_rep, dim] f32.
+ */
+int tq_sparse_v_matvec(const float* weights, const uint32_t* v_packed, const float* v_norms,
+                       const float* centroids, const float* signs, float* out,
+                       void* workspace, size_t workspace_bytes,
+                       int n_kv_heads, int n_rep, int64_t seq_len,
+                       int64_t packed_head_stride, int64_t norms_head_stride,
+                       int dim, int bits, float threshold, tq_stream_t stream);
+
+/* Shapes and addressing shared by the two fused decode-attention entry points. */
+typedef struct tq_decode_shape {
+  int32_t n_seq;             /* sequences in the batch (>= 1) */
+  int32_t n_kv_heads;
+  int32_t n_rep;             /* query heads per kv head */
+  int32_t dim;               /* head dimension */
+  int32_t bits;
+  int32_t block_size;        /* accepted for interface parity (1..32); the result does not depend on it */
+  int64_t seq_len;           /* uniform length, or the maximum length when seq_offsets != NULL */
+  const int32_t* seq_offsets;/* device, [n_seq+1], or NULL */
+  int64_t k_seq_stride, k_head_stride;   /* rows; K packed and K fp16 share the row count */
+  int64_t kn_seq_stride, kn_head_stride; /* K norms (unused by the V-only kernel) */
+  int64_t v_seq_stride, v_head_stride;   /* V packed */
+  int64_t vn_seq_stride, vn_head_stride; /* V norms */
+  const float* mask;         /* optional additive mask, device, or NULL */
+  int64_t mask_seq_stride;   /* floats between sequences */
+  int64_t mask_head_stride;  /* floats between query heads (0 = shared) */
+  float attn_scale;
+  int32_t out_dtype;         /* TQ_F32 or TQ_F16 */
+} tq_decode_shape;
+
+/*
+ * Single-pass SDPA for one query token per head over packed K and packed V, online softmax in
+ * float32:  s = (sum_e c_k[idx_k] * q_rot) * k_norm * (1/dim) * attn_scale (+ mask),
+ *           out = butterfly(sum_p e^{s-m} * v_norm * c_v[idx_v]) * v_signs * (1/dim) / l.
+ * Replaces flash_attention_turboquant (flash_attention.py:168-274, kernel 36-163), extended
+ * with a batch of sequences of ragged length.
+ *   q_rot [n_seq, n_kv*n_rep, dim] f32;  out [n_seq, n_kv*n_rep, dim] out_dtype.
+ */
+int tq_flash_decode(const float* q_rot,
+                    const uint32_t* k_packed, const float* k_norms,
+                    const uint32_t* v_packed, const float* v_norms,
+                    const float* k_centroids, const float* v_centroids, const float* v_signs,
+                    void* out, void* workspace, size_t workspace_bytes,
+                    const tq_decode_shape* shape /* host */, tq_stream_t stream);
+
+/*
+ * Decode attention for a V-only cache: fp16 keys, packed values, dense softmax (threshold 0):
+ *   out = butterfly(sum_p softmax_p(<q,K_p>*attn_scale + mask) * v_norm * c_v[idx_v]) * v_signs / dim.
+ * The composition dense-K scores -> softmax -> sparse_v_matvec of hybrid_attention.py:52-88 /
+ * fused_attention.py:50-121 in one launch for the cache of v_only_cache.py:24-127.
+ *   q [n_seq, n_kv*n_rep, dim] dtype q_dtype;  k_f16 rows of dim halfs;  out as tq_flash_decode.
+ */
+int tq_vonly_decode_attn(const void* q, int q_dtype, const void* k_f16,
+                         const uint32_t* v_packed, const float* v_norms,
+                         const float* v_centroids, const float* v_signs,
+                         void* out, void* workspace, size_t workspace_bytes,
+                         const tq_decode_shape* shape /* host */, tq_stream_t stream);
+
+/* Bytes of workspace the fused op needs for this shape (host computation, no GPU call). */
+size_t tq_workspace_bytes(int op, int n_seq, int n_q_heads, int64_t max_seq_len, int dim);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TQHIP_H */

@@ -1,0 +1,316 @@
+"""GPU tests of the cache objects and the decode-step compositions, following the reference's
+tests/test_core.py:112-181, tests/test_v_only_cache.py and tests/test_fused_attn.py, with the
+packed state additionally compared bit-for-bit against the oracle."""
+import math
+
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+
+from oracle import polarquant_oracle as o  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+F32 = np.float32
+
+
+@pytest.fixture(scope="module")
+def tq():
+    if not torch.cuda.is_available():
+        pytest.fail("GPU tests need a GPU: torch.cuda.is_available() is False")
+    import tqhip
+    return tqhip
+
+
+def rand(shape, seed, dtype=torch.float16):
+    rng = np.random.default_rng(seed)
+    return torch.from_numpy(rng.standard_normal(shape).astype(F32)).to(dtype).cuda()
+
+
+def host(t):
+    return t.detach().float().cpu().numpy()
+
+
+def cos(a, b):
+    a, b = a.astype(np.float64).ravel(), b.astype(np.float64).ravel()
+    return float(a @ b / np.linalg.norm(a) / np.linalg.norm(b))
+
+
+def oracle_pack(x, seed, bits=3, variant="mlx"):
+    """x: [B,H,T,D] numpy -> packed [B,H,T,pd], norms [B,H,T] by the oracle."""
+    B, H, T, D = x.shape
+    c = o.gaussian_codebook(bits)
+    p, n = o.fused_quantize(x.reshape(-1, D), o.random_diagonal_sign(D, seed), o.gaussian_boundaries(c), D, bits, variant)
+    return p.reshape(B, H, T, -1), n.reshape(B, H, T)
+
+
+# ------------------------------------------------------------------ TurboQuantKVCache
+
+def test_cache_decode_and_prefill_shapes(tq):
+    cache = tq.TurboQuantKVCache(bits=3)
+    assert cache.empty() and cache.size() == 0 and cache.state == []
+    k, v = rand((1, 4, 8, 128), 0), rand((1, 4, 8, 128), 1)
+    ko, vo = cache.update_and_fetch(k, v)                                  # prefill
+    assert ko.shape == (1, 4, 8, 128) and vo.shape == (1, 4, 8, 128) and cache.offset == 8
+    assert ko.dtype == torch.float16 and not cache.empty()
+    assert cache.k_packed.shape == (1, 4, 256, 13) and cache.k_packed.dtype == torch.uint32
+    assert cache.k_norms.shape == (1, 4, 256) and cache.k_norms.dtype == torch.float32
+    for i in range(5):                                                      # decode
+        ko, vo = cache.update_and_fetch(rand((1, 4, 1, 128), 10 + i), rand((1, 4, 1, 128), 20 + i))
+    assert cache.offset == 13 and ko.shape == (1, 4, 13, 128)
+    assert cos(host(ko[..., :8, :]), host(k)) > 0.7 and cos(host(vo[..., :8, :]), host(v)) > 0.7
+    assert cache.compression_ratio > 1.5
+    assert abs(cache.compression_ratio - 512 / 112) < 1e-9
+    assert cache.nbytes == 1 * 4 * 13 * 56 * 2
+    assert cache.is_trimmable() and cache.size() == 13
+
+
+def test_cache_packed_state_bit_exact_and_incremental_equals_full(tq):
+    B, H, D = 2, 4, 128
+    k, v = rand((B, H, 300, D), 2), rand((B, H, 300, D), 3)
+    cache = tq.TurboQuantKVCache(bits=3, seed=42)
+    cache.update_and_fetch(k[..., :290, :], v[..., :290, :])               # grows to 512
+    for t in range(290, 300, 2):
+        ko, vo = cache.update_and_fetch(k[..., t:t + 2, :], v[..., t:t + 2, :])
+    assert cache.offset == 300 and cache.k_packed.shape[2] == 512
+    wkp, wkn = oracle_pack(k.cpu().numpy(), 42)
+    wvp, wvn = oracle_pack(v.cpu().numpy(), 43)
+    st = cache.state
+    assert len(st) == 4
+    assert np.array_equal(st[0].cpu().numpy(), wkp) and np.array_equal(st[1].cpu().numpy(), wkn)
+    assert np.array_equal(st[2].cpu().numpy(), wvp) and np.array_equal(st[3].cpu().numpy(), wvn)
+    # incremental buffer == one-shot dequantisation of the same packed data, bit for bit
+    c = o.gaussian_codebook(3)
+    wk = o.packed_dequantize(wkp.reshape(-1, 13), wkn.reshape(-1), c, o.random_diagonal_sign(D, 42), D, 3)
+    assert np.array_equal(ko.cpu().numpy(), wk.reshape(B, H, 300, D).astype(np.float16))
+    fresh = tq.TurboQuantKVCache(bits=3, seed=42)
+    k2, v2 = fresh.update_and_fetch(k, v)
+    assert torch.equal(k2, ko) and torch.equal(v2, vo)
+
+
+def test_cache_growth_across_step_keeps_old_rows(tq):
+    cache = tq.TurboQuantKVCache(bits=3)
+    k, v = rand((1, 2, 700, 128), 4), rand((1, 2, 700, 128), 5)
+    cache.update_and_fetch(k[..., :250, :], v[..., :250, :])
+    cache.update_and_fetch(k[..., 250:260, :], v[..., 250:260, :])          # crosses 256
+    cache.update_and_fetch(k[..., 260:700, :], v[..., 260:700, :])          # crosses 512, lands in 768
+    assert cache.v_packed.shape[2] == 768
+    wvp, wvn = oracle_pack(v.cpu().numpy(), 43)
+    assert np.array_equal(cache.state[2].cpu().numpy(), wvp)
+    assert np.array_equal(cache.state[3].cpu().numpy(), wvn)
+
+
+def test_cache_fused_mode_returns_placeholders(tq):
+    cache = tq.TurboQuantKVCache(bits=3, fused=True)
+    ko, vo = cache.update_and_fetch(rand((1, 4, 16, 128), 6), rand((1, 4, 16, 128), 7))
+    assert ko.shape == (1, 4, 16, 128) and float(ko.abs().max()) == 0.0 and float(vo.abs().max()) == 0.0
+    assert cache._k_deq_buf is None and cache.k_packed is not None
+
+
+def test_cache_trim_then_extend(tq):
+    cache = tq.TurboQuantKVCache(bits=3)
+    k, v = rand((1, 2, 20, 128), 8), rand((1, 2, 20, 128), 9)
+    cache.update_and_fetch(k[..., :16, :], v[..., :16, :])
+    assert cache.trim(4) == 4 and cache.offset == 12 and cache._v_deq_buf is None
+    assert cache.trim(100) == 12 and cache.offset == 0
+    cache.update_and_fetch(k[..., :12, :], v[..., :12, :])
+    ko, vo = cache.update_and_fetch(k[..., 12:20, :], v[..., 12:20, :])     # S=8 > 4: full dequant path
+    wkp, _ = oracle_pack(k.cpu().numpy(), 42)
+    assert np.array_equal(cache.state[0].cpu().numpy(), wkp)
+    assert ko.shape == (1, 2, 20, 128)
+
+
+def test_cache_serialisation_roundtrip(tq):
+    cache = tq.TurboQuantKVCache(bits=3, seed=7)
+    k, v = rand((1, 4, 12, 128), 10), rand((1, 4, 12, 128), 11)
+    cache.update_and_fetch(k[..., :8, :], v[..., :8, :])
+    assert cache.meta_state == "8,3,7,128,128,float16"
+    rest = tq.TurboQuantKVCache.from_state(cache.state, cache.meta_state)
+    assert rest.offset == 8 and rest.quant_bits == 3 and rest.seed == 7 and rest.v_only is False
+    assert torch.equal(rest.k_packed, cache.state[0])
+    ko, vo = rest.update_and_fetch(k[..., 8:12, :], v[..., 8:12, :])        # restored cache extends
+    assert rest.offset == 12 and ko.shape == (1, 4, 12, 128)
+    wkp, wkn = oracle_pack(k.cpu().numpy(), 7)
+    assert np.array_equal(rest.state[0].cpu().numpy(), wkp) and np.array_equal(rest.state[1].cpu().numpy(), wkn)
+    with pytest.raises(ValueError, match="Expected 2"):
+        tq.TurboQuantKVCache.from_state(cache.state[:3], cache.meta_state)
+    bf = tq.TurboQuantKVCache(bits=4)
+    bf.update_and_fetch(rand((1, 2, 3, 64), 12, torch.bfloat16), rand((1, 2, 3, 64), 13, torch.bfloat16))
+    assert bf.meta_state == "3,4,42,64,64,bfloat16"
+
+
+def test_cache_masks(tq):
+    cache = tq.TurboQuantKVCache(bits=3)
+    cache.update_and_fetch(rand((1, 2, 5, 128), 14), rand((1, 2, 5, 128), 15))
+    assert cache.make_mask(1) is None and cache.make_mask(4) == "causal"
+    m = cache.make_mask(3, return_array=True)
+    assert m.shape == (3, 8) and m.dtype == torch.bool
+    want = np.array([[j <= 5 + i for j in range(8)] for i in range(3)])
+    assert np.array_equal(m.cpu().numpy(), want)
+    mw = cache.make_mask(3, window_size=2)
+    want_w = np.array([[(j <= 5 + i) and (j > 5 + i - 2) for j in range(8)] for i in range(3)])
+    assert np.array_equal(mw.cpu().numpy(), want_w)
+
+
+def test_cache_from_kvcache(tq):
+    kv = tq.KVCache()
+    k, v = rand((1, 4, 40, 128), 16), rand((1, 4, 40, 128), 17)
+    kv.update_and_fetch(k, v)
+    assert kv.keys.shape[2] == 256 and kv.offset == 40
+    a = tq.TurboQuantKVCache.from_kvcache(kv, bits=3, seed=42)
+    b = tq.TurboQuantKVCache(bits=3, seed=42)
+    b.update_and_fetch(k, v)
+    assert a.offset == 40 and all(torch.equal(x, y) for x, y in zip(a.state, b.state))
+    vo = tq.VOnlyTurboQuantCache.from_kvcache(kv, bits=3)
+    assert vo.offset == 40 and torch.equal(vo.state[0], k)
+    assert tq.TurboQuantKVCache.from_kvcache(tq.KVCache()).offset == 0
+
+
+@pytest.mark.parametrize("variant", ["mlx", "metal"])
+def test_cache_encode_variant(tq, variant):
+    cache = tq.TurboQuantKVCache(bits=3, encode_variant=variant)
+    k, v = rand((1, 2, 64, 128), 18), rand((1, 2, 64, 128), 19)
+    cache.update_and_fetch(k, v)
+    wvp, _ = oracle_pack(v.cpu().numpy(), 43, variant=variant)
+    assert np.array_equal(cache.state[2].cpu().numpy(), wvp)
+
+
+# ------------------------------------------------------------------ VOnlyTurboQuantCache
+
+def test_vonly_cache_roundtrip_and_protocol(tq):
+    cache = tq.VOnlyTurboQuantCache(bits=3)
+    assert cache.empty()
+    k, v = rand((1, 4, 16, 128), 20), rand((1, 4, 16, 128), 21)
+    ko, vo = cache.update_and_fetch(k[..., :8, :], v[..., :8, :])
+    assert cos(host(ko), host(k[..., :8, :])) > 0.999 and cos(host(vo), host(v[..., :8, :])) > 0.95
+    assert torch.equal(ko, k[..., :8, :])
+    assert cache.offset == 8 and not cache.empty()
+    ko, vo = cache.update_and_fetch(k[..., 8:12, :], v[..., 8:12, :])
+    assert cache.offset == 12 and vo.shape == (1, 4, 12, 128)
+    assert len(cache.state) == 4 and cache.meta_state.startswith("VOnlyTQ,3,")
+    assert cache.meta_state == "VOnlyTQ,3,42,12,3,42,0,128,float16"
+    ko, vo = cache.update_and_fetch(k[..., 12:16, :], v[..., 12:16, :])
+    assert cache.trim(4) == 4 and cache.offset == 12 and cache.size() == 12
+    assert cache.make_mask(1) is None and cache.is_trimmable()
+    wvp, wvn = oracle_pack(v.cpu().numpy(), 43)
+    assert np.array_equal(cache.state[2].cpu().numpy(), wvp[..., :12, :])
+    assert np.array_equal(cache.state[3].cpu().numpy(), wvn[..., :12])
+
+
+def test_vonly_cache_no_v_buffer(tq):
+    a = tq.VOnlyTurboQuantCache(bits=3, no_v_buffer=True)
+    b = tq.VOnlyTurboQuantCache(bits=3)
+    k, v = rand((1, 4, 12, 128), 22), rand((1, 4, 12, 128), 23)
+    for lo, hi in ((0, 8), (8, 9), (9, 12)):
+        ka, va = a.update_and_fetch(k[..., lo:hi, :], v[..., lo:hi, :])
+        kb, vb = b.update_and_fetch(k[..., lo:hi, :], v[..., lo:hi, :])
+    assert a._v_tq._v_deq_buf is None
+    assert torch.equal(va, vb) and cos(host(va), host(v)) > 0.95            # test_v_only_cache.py:70-75
+
+
+def test_vonly_cache_from_state(tq):
+    cache = tq.VOnlyTurboQuantCache(bits=3, seed=5)
+    k, v = rand((1, 4, 12, 128), 24), rand((1, 4, 12, 128), 25)
+    cache.update_and_fetch(k[..., :8, :], v[..., :8, :])
+    rest = tq.VOnlyTurboQuantCache.from_state(cache.state, cache.meta_state)
+    assert rest.offset == 8 and rest._v_bits == 3 and rest._v_tq.seed == 5
+    assert torch.equal(rest._v_tq.v_packed, cache.state[2])                # test_v_only_cache.py:98-118
+    ko, vo = rest.update_and_fetch(k[..., 8:12, :], v[..., 8:12, :])
+    assert rest.offset == 12 and vo.shape == (1, 4, 12, 128)               # test_v_only_cache.py:120-134
+    wvp, _ = oracle_pack(v.cpu().numpy(), 6)
+    assert np.array_equal(rest.state[2].cpu().numpy(), wvp)
+
+
+def test_adaptive_cache_layout(tq):
+    caches = tq.make_adaptive_cache(12, bits=3, fp16_layers=2, fused=True)
+    kinds = [type(c).__name__ for c in caches]
+    assert kinds == ["KVCache"] * 2 + ["TurboQuantKVCache"] * 8 + ["KVCache"] * 2
+    assert all(c.fused for c in caches[2:10])
+
+    class Odd:
+        def make_cache(self):
+            return [object()]
+    with pytest.raises(ValueError, match="Incompatible cache type"):
+        tq.make_adaptive_cache(4, model=Odd())
+
+
+# ------------------------------------------------------------------ attention compositions
+
+@pytest.mark.parametrize("fused", [False, True])
+@pytest.mark.parametrize("thr", [None, 1e-5])
+def test_turboquant_attention_vs_dense_sdpa(tq, fused, thr):
+    """tests/test_fused_attn.py:67-112: attention over the packed cache vs plain SDPA on the
+    dequantised K/V, cosine > 0.999; and against the oracle within 2e-3 rel / 1e-3 abs."""
+    B, n_q, n_kv, S, D = 2, 8, 4, 512, 128
+    sc = 1 / math.sqrt(D)
+    k, v = rand((B, n_kv, S, D), 26), rand((B, n_kv, S, D), 27)
+    q = rand((B, n_q, 1, D), 28)
+    cache = tq.TurboQuantKVCache(bits=3, fused=True)
+    cache.update_and_fetch(k, v)
+    out = tq.turboquant_attention(q, cache, sc, sparse_v_threshold=thr, fused=fused)
+    assert out.shape == (B, n_q, 1, D) and out.dtype == q.dtype
+    plain = tq.TurboQuantKVCache(bits=3)
+    kd, vd = plain.update_and_fetch(k, v)
+    ref = o.dense_attention(host(q)[0], host(kd)[0], host(vd)[0], sc)
+    assert cos(host(out)[0], ref) > 0.999
+    kp, kn, vp, vn = [t.cpu().numpy() for t in cache.state]
+    c = o.gaussian_codebook(3)
+    for b in range(B):
+        want = o.turboquant_attention_single(host(q)[b, :, 0], kp[b], kn[b], vp[b], vn[b], c,
+                                             o.random_diagonal_sign(D, 42), c, o.random_diagonal_sign(D, 43),
+                                             D, 3, sc, sparse_v_threshold=thr)
+        err = np.abs(host(out)[b, :, 0] - want)
+        assert (err <= 1e-3 + 2e-3 * np.abs(want)).all()
+
+
+def test_turboquant_attention_masks_and_v_buffer(tq):
+    B, n_q, n_kv, S, D = 2, 4, 2, 200, 128
+    sc = 1 / math.sqrt(D)
+    k, v = rand((B, n_kv, S, D), 29), rand((B, n_kv, S, D), 30)
+    q = rand((B, n_q, 1, D), 31, torch.float32)
+    cache = tq.TurboQuantKVCache(bits=3, fused=True)
+    cache.update_and_fetch(k, v)
+    rng = np.random.default_rng(0)
+    m4 = torch.from_numpy(np.where(rng.random((B, 1, 1, S)) < 0.3, -np.inf, 0).astype(F32)).cuda()
+    a = tq.turboquant_attention(q, cache, sc, mask=m4)
+    b = tq.turboquant_attention(q, cache, sc, mask=m4, fused=True)
+    assert np.abs(host(a) - host(b)).max() < 1e-4
+    kp, kn, vp, vn = [t.cpu().numpy() for t in cache.state]
+    c = o.gaussian_codebook(3)
+    for i in range(B):
+        want = o.turboquant_attention_single(host(q)[i, :, 0], kp[i], kn[i], vp[i], vn[i], c,
+                                             o.random_diagonal_sign(D, 42), c, o.random_diagonal_sign(D, 43),
+                                             D, 3, sc, mask=host(m4)[i, 0])
+        assert np.abs(host(a)[i, :, 0] - want).max() < 1e-4
+    m3 = m4[:, 0]                                                            # (B, 1, S)
+    assert np.abs(host(tq.turboquant_attention(q, cache, sc, mask=m3)) - host(a)).max() < 1e-6
+    plain = tq.TurboQuantKVCache(bits=3)
+    kd, vd = plain.update_and_fetch(k, v)
+    vb = tq.turboquant_attention(q, cache, sc, v_buffer=vd.float())
+    nb = tq.turboquant_attention(q, cache, sc)
+    assert np.abs(host(vb) - host(nb)).max() < 5e-3
+
+
+@pytest.mark.parametrize("thr", [None, 1e-5])
+def test_vonly_decode_attention_on_cache(tq, thr):
+    B, n_q, n_kv, S, D = 2, 28, 4, 1500, 128
+    sc = 1 / math.sqrt(D)
+    k, v = rand((B, n_kv, S, D), 32), rand((B, n_kv, S, D), 33)
+    q = rand((B, n_q, 1, D), 34)
+    cache = tq.VOnlyTurboQuantCache(bits=3)
+    cache.update_and_fetch(k[..., :1498, :], v[..., :1498, :])
+    cache.update_and_fetch(k[..., 1498:, :], v[..., 1498:, :])
+    out = tq.vonly_decode_attention(q, cache, sc, sparse_v_threshold=thr)
+    assert out.shape == (B, n_q, 1, D) and out.dtype == torch.float16
+    st = cache.state
+    c = o.gaussian_codebook(3)
+    for b in range(B):
+        want = o.vonly_decode_attention(host(q)[b, :, 0], host(st[0])[b], st[2].cpu().numpy()[b],
+                                        st[3].cpu().numpy()[b], c, o.random_diagonal_sign(D, 43), D, 3, sc,
+                                        threshold=thr or 0.0)
+        err = np.abs(host(out)[b, :, 0] - want)
+        assert (err <= 1e-3 + 2e-3 * np.abs(want)).all()
+    # against attention on the cache's own (fp16 K, dequantised V) outputs: cosine > 0.999
+    ko, vo = cache._k_cache.keys[..., :S, :], cache._v_tq._v_deq_buf[..., :S, :]
+    ref = o.dense_attention(host(q)[0], host(ko)[0], host(vo)[0], sc)
+    assert cos(host(out)[0], ref) > 0.999

@@ -1,0 +1,496 @@
+"""GPU parity tests: every HIP kernel, called through the C-ABI library, against the CPU oracle
+on the same seeded inputs.  Integer outputs (packed indices) must be bit-exact; float outputs are
+held to the tolerance written in each test.  Cases mirror the reference's own test parameters
+(tests/test_prerot.py, tests/test_sparse_v.py, tests/test_flash_attention.py, tests/test_core.py).
+"""
+import math
+
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+
+from oracle import polarquant_oracle as o  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+
+F32 = np.float32
+REL, ABS = 2e-3, 1e-3          # attention-output tolerance of the task statement
+
+
+@pytest.fixture(scope="module")
+def tq():
+    if not torch.cuda.is_available():
+        pytest.fail("GPU tests need a GPU: torch.cuda.is_available() is False")
+    import tqhip
+    return tqhip
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    return t.detach().cpu().numpy()
+
+
+def tables(bits):
+    c = o.gaussian_codebook(bits)
+    return c, o.gaussian_boundaries(c)
+
+
+def close(got, want, rel=REL, abs_=ABS):
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    ok = err <= abs_ + rel * np.abs(want)
+    assert ok.all(), f"max err {err.max():.3e} (want scale {np.abs(want).max():.3e}), {(~ok).sum()} bad"
+
+
+# ------------------------------------------------------------------ encode
+
+@pytest.mark.parametrize("variant", ["mlx", "metal"])
+@pytest.mark.parametrize("dim,bits", [(128, 3), (128, 4), (128, 2), (128, 1), (64, 4), (64, 3), (32, 2),
+                                      (32, 3), (256, 3), (256, 4)])
+def test_encode_bit_exact(tq, dim, bits, variant):
+    rng = np.random.default_rng(dim * 10 + bits)
+    x = rng.standard_normal((1037, dim)).astype(np.float16)       # ragged count: not a multiple of 4
+    s = o.random_diagonal_sign(dim, 43)
+    c, b = tables(bits)
+    wp, wn = o.fused_quantize(x, s, b, dim, bits, variant)
+    gp, gn = tq.fused_quantize(dev(x), dev(s), b, dim, bits, variant=variant)
+    assert gp.dtype == torch.uint32 and gp.shape == wp.shape
+    assert np.array_equal(host(gp), wp)
+    assert np.array_equal(host(gn), wn)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_encode_dtypes_and_scales(tq, dtype):
+    rng = np.random.default_rng(1)
+    x = (rng.standard_normal((513, 128)) * rng.choice([1e-3, 1.0, 300.0], size=(513, 1))).astype(dtype)
+    s = o.random_diagonal_sign(128, 42)
+    c, b = tables(3)
+    wp, wn = o.fused_quantize(x, s, b, 128, 3)
+    gp, gn = tq.fused_quantize(dev(x), dev(s), b, 128, 3)
+    assert np.array_equal(host(gp), wp) and np.array_equal(host(gn), wn)
+
+
+def test_encode_bf16_input(tq):
+    rng = np.random.default_rng(2)
+    xt = torch.from_numpy(rng.standard_normal((200, 128)).astype(F32)).to(torch.bfloat16)
+    s = o.random_diagonal_sign(128, 42)
+    c, b = tables(3)
+    wp, wn = o.fused_quantize(xt.float().numpy(), s, b, 128, 3)
+    gp, gn = tq.fused_quantize(xt.cuda(), dev(s), b, 128, 3)
+    assert np.array_equal(host(gp), wp) and np.array_equal(host(gn), wn)
+
+
+def test_encode_known_answers(tq):
+    c, b = tables(3)
+    ones = np.ones(128, F32)
+    x = np.zeros((3, 128), np.float16)
+    x[1, 5] = 3.0
+    x[2, :] = np.nan
+    gp, gn = tq.fused_quantize(dev(x), dev(ones), b, 128, 3)
+    gp, gn = host(gp), host(gn)
+    assert [int(w) for w in gp[0]] == [0x1B6DB6DB] * 12 + [0x006DB6DB] and gn[0] == 0.0
+    assert [int(w) for w in gp[1][:3]] == [0x15AAA555, 0x1556AA95, 0x2A555AAA] and gn[1] == 3.0
+    assert (gp[2] == 0).all() and np.isnan(gn[2])
+    # empty input
+    ep, en = tq.fused_quantize(torch.zeros((0, 128), dtype=torch.float16, device="cuda"), dev(ones), b, 128, 3)
+    assert ep.shape == (0, 13) and en.shape == (0,)
+
+
+def test_encode_near_boundary_values(tq):
+    """Vectors built so that butterfly outputs sit within a few ulp of decision boundaries: the
+    double-rounding rule of the pure-array quantiser and the raw rule of the Metal encoder must
+    each be reproduced exactly."""
+    c, b = tables(3)
+    ones = np.ones(128, F32)
+    rng = np.random.default_rng(3)
+    rows = []
+    H = np.array([[1.0 if bin(j & k).count("1") % 2 == 0 else -1.0 for k in range(128)] for j in range(128)])
+    for _ in range(400):
+        z = rng.standard_normal(128)
+        k = rng.integers(0, 128)
+        z[k] = float(b[rng.integers(0, 7)]) * (1 + rng.integers(-3, 4) * 2.0 ** -23)
+        z *= math.sqrt(128) / np.linalg.norm(z)
+        rows.append((H @ z) / 128.0)
+    x = np.array(rows, dtype=F32)
+    for variant in ("mlx", "metal"):
+        wp, wn = o.fused_quantize(x, ones, b, 128, 3, variant)
+        gp, gn = tq.fused_quantize(dev(x), dev(ones), b, 128, 3, variant=variant)
+        assert np.array_equal(host(gp), wp) and np.array_equal(host(gn), wn)
+
+
+def test_config1_roundtrip(tq):
+    """BASELINE config 1: [1,4,1024,128] fp16 N(0,1): indices bit-exact, reconstruction MSE equal."""
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((1, 4, 1024, 128)).astype(np.float16)
+    s = o.random_diagonal_sign(128, 43)
+    c, b = tables(3)
+    wp, wn = o.fused_quantize(x.reshape(-1, 128), s, b, 128, 3)
+    gp, gn = tq.fused_quantize(dev(x.reshape(-1, 128)), dev(s), b, 128, 3)
+    assert np.array_equal(host(gp), wp) and np.array_equal(host(gn), wn)
+    wd = o.packed_dequantize(wp, wn, c, s, 128, 3)
+    gd = host(tq.packed_dequantize(gp, gn, c, dev(s), 128, 3))
+    assert np.array_equal(gd, wd)
+    x32 = x.reshape(-1, 128).astype(F32)
+    assert abs(float(((gd - x32) ** 2).mean()) - float(((wd - x32) ** 2).mean())) == 0.0
+    assert 0.032 < float(((gd - x32) ** 2).mean()) < 0.036
+    # fp16 norms, as the config text allows: a cast of the float32 norms
+    assert np.array_equal(host(gn.to(torch.float16)), wn.astype(np.float16))
+
+
+# ------------------------------------------------------------------ dequant / prerotate
+
+@pytest.mark.parametrize("dim,bits", [(128, 3), (64, 4), (32, 2), (256, 3), (128, 1)])
+def test_dequant_bit_exact(tq, dim, bits):
+    rng = np.random.default_rng(4)
+    c, b = tables(bits)
+    s = o.random_diagonal_sign(dim, 42)
+    p = o.pack_indices(rng.integers(0, 2 ** bits, size=(333, dim)).astype(np.uint8), bits)
+    n = (rng.random(333) * 10 + 0.1).astype(F32)
+    want = o.packed_dequantize(p, n, c, s, dim, bits)
+    got = host(tq.packed_dequantize(dev(p), dev(n), c, dev(s), dim, bits))
+    assert got.dtype == F32 and np.array_equal(got, want)
+    got16 = host(tq.dequant_fp16(dev(p), dev(n), c, dev(s), dim, bits))
+    assert got16.dtype == np.float16 and np.array_equal(got16, want.astype(np.float16))
+
+
+@pytest.mark.parametrize("dim", [32, 64, 128, 256])
+def test_prerotate_query_bit_exact(tq, dim):
+    rng = np.random.default_rng(5)
+    q = rng.standard_normal((28, dim)).astype(F32)
+    s = o.random_diagonal_sign(dim, 1)
+    want = o.prerotate_query(q, s)
+    assert np.array_equal(host(tq.prerotate_query(dev(q), dev(s))), want)
+    q16 = q.astype(np.float16)
+    assert np.array_equal(host(tq.prerotate_query(dev(q16), dev(s))), o.prerotate_query(q16, s))
+    with pytest.raises(ValueError, match="expects"):
+        tq.prerotate_query(dev(q[0]), dev(s))
+
+
+def test_rotation_helpers(tq):
+    rng = np.random.default_rng(6)
+    x = rng.standard_normal((8, 128)).astype(F32)
+    s = o.random_diagonal_sign(128, 42)
+    assert np.array_equal(host(tq.random_diagonal_sign(128, 42, device="cuda")), s)
+    y = tq.walsh_hadamard_transform(dev(x))
+    assert np.array_equal(host(y), o.walsh_hadamard_transform(x))
+    assert np.abs(host(tq.walsh_hadamard_transform(y)) - x).max() < 1e-5
+    z = tq.inverse_randomized_hadamard(tq.randomized_hadamard_transform(dev(x), dev(s)), dev(s))
+    assert np.abs(host(z) - x).max() < 1e-4
+
+
+def test_polar_quantizer_object(tq):
+    rng = np.random.default_rng(7)
+    x = rng.standard_normal((2, 50, 128)).astype(F32)
+    pq = tq.PolarQuantizer(128, bits=3, seed=42)
+    idx, n = pq.quantize(dev(x))
+    wi, wn = o.quantize(x, o.random_diagonal_sign(128, 42), o.gaussian_boundaries(o.gaussian_codebook(3)))
+    assert idx.dtype == torch.uint8 and np.array_equal(host(idx), wi) and np.array_equal(host(n), wn)
+    xh = host(pq.dequantize(idx, n))
+    assert np.array_equal(xh, o.dequantize(wi, wn, o.gaussian_codebook(3), o.random_diagonal_sign(128, 42)))
+    cos = (xh * x).sum(-1) / np.linalg.norm(xh, axis=-1) / np.linalg.norm(x, axis=-1)
+    assert cos.mean() > 0.97
+
+
+# ------------------------------------------------------------------ scores
+
+@pytest.mark.parametrize("H,S,D,bits", [(4, 64, 128, 3), (8, 256, 128, 3), (2, 16, 64, 4), (1, 128, 32, 2),
+                                        (3, 1000, 128, 3)])
+def test_prerot_scores_match_oracle_and_full_kernel(tq, H, S, D, bits):
+    rng = np.random.default_rng(8)
+    c, b = tables(bits)
+    s = o.random_diagonal_sign(D, 42)
+    kp = o.pack_indices(rng.integers(0, 2 ** bits, size=(H, S, D)).astype(np.uint8), bits)
+    kn = (rng.random((H, S)) * 10 + 1).astype(F32)
+    q = rng.standard_normal((H, D)).astype(F32)
+    q_rot = tq.prerotate_query(dev(q), dev(s))
+    pre = host(tq.prerot_fused_qk_scores(q_rot, dev(kp), dev(kn), c, D, bits))
+    full = host(tq.packed_fused_qk_scores(dev(q), dev(kp), dev(kn), c, dev(s), D, bits))
+    want = o.prerot_fused_qk_scores(o.prerotate_query(q, s), kp, kn, c, D, bits)
+    scale = max(1.0, np.abs(want).max())
+    assert np.abs(pre - want).max() < 1e-5 * scale
+    assert np.abs(full - want).max() < 1e-5 * scale
+    assert np.abs(pre - full).max() < 1e-4 * scale                       # test_prerot.py:62-97
+
+
+@pytest.mark.parametrize("n_kv,n_rep", [(4, 2), (2, 4), (4, 7), (1, 12)])
+def test_prerot_scores_gqa(tq, n_kv, n_rep):
+    rng = np.random.default_rng(9)
+    D, S, bits = 128, 300, 3
+    c, b = tables(bits)
+    kp = o.pack_indices(rng.integers(0, 8, size=(n_kv, S, D)).astype(np.uint8), bits)
+    kn = (rng.random((n_kv, S)) + 0.5).astype(F32)
+    qr = rng.standard_normal((n_kv * n_rep, D)).astype(F32)
+    got = host(tq.prerot_fused_qk_scores(dev(qr), dev(kp), dev(kn), c, D, bits, n_rep=n_rep))
+    want = o.prerot_fused_qk_scores(qr, kp, kn, c, D, bits, n_rep)
+    assert np.abs(got - want).max() < 1e-5 * max(1.0, np.abs(want).max())
+    with pytest.raises(ValueError, match="must equal n_kv_heads"):
+        tq.prerot_fused_qk_scores(dev(qr[:-1]), dev(kp), dev(kn), c, D, bits, n_rep=n_rep)
+
+
+def test_scores_on_cache_slices(tq):
+    """k_packed[b, :, :total] slices of cache storage are strided views: no copy must be needed."""
+    rng = np.random.default_rng(10)
+    D, bits, n_kv, T_alloc, total = 128, 3, 4, 512, 300
+    c, b = tables(bits)
+    kp = o.pack_indices(rng.integers(0, 8, size=(2, n_kv, T_alloc, D)).astype(np.uint8), bits)
+    kn = (rng.random((2, n_kv, T_alloc)) + 0.5).astype(F32)
+    qr = rng.standard_normal((n_kv * 2, D)).astype(F32)
+    kpt, knt = dev(kp), dev(kn)
+    got = host(tq.prerot_fused_qk_scores(dev(qr), kpt[1, :, :total, :], knt[1, :, :total], c, D, bits, n_rep=2))
+    want = o.prerot_fused_qk_scores(qr, kp[1, :, :total], kn[1, :, :total], c, D, bits, 2)
+    assert np.abs(got - want).max() < 1e-5 * max(1.0, np.abs(want).max())
+
+
+def test_dense_scores_and_softmax(tq):
+    rng = np.random.default_rng(11)
+    n_kv, n_rep, T, D = 4, 7, 700, 128
+    K = rng.standard_normal((n_kv, T, D)).astype(np.float16)
+    q = rng.standard_normal((n_kv * n_rep, D)).astype(np.float16)
+    sc = 1 / math.sqrt(D)
+    got = host(tq.dense_qk_scores(dev(q), dev(K), sc, n_rep=n_rep))
+    want = np.einsum("grd,gtd->grt", q.reshape(n_kv, n_rep, D).astype(np.float64), K.astype(np.float64))
+    want = want.reshape(n_kv * n_rep, T) * sc
+    assert np.abs(got - want).max() < 1e-5 * np.abs(want).max()
+    mask = np.where(rng.random((1, T)) < 0.2, -np.inf, 0.0).astype(F32)
+    w = host(tq.softmax_rows(dev(got), 1.0, dev(mask)))
+    ref = o._softmax64(got.astype(np.float64) + mask)
+    assert np.abs(w - ref).max() < 1e-6 and np.abs(w.sum(-1) - 1).max() < 1e-5
+    assert (w[:, mask[0] == -np.inf] == 0).all()
+
+
+# ------------------------------------------------------------------ sparse V
+
+def v_fixture(rng, n_kv, S, D, bits):
+    c, b = tables(bits)
+    s = o.random_diagonal_sign(D, 43)
+    vp = o.pack_indices(rng.integers(0, 2 ** bits, size=(n_kv, S, D)).astype(np.uint8), bits)
+    vn = (rng.random((n_kv, S)) + 0.1).astype(F32)
+    return c, s, vp, vn
+
+
+def softmax_np(x):
+    e = np.exp(x - x.max(-1, keepdims=True))
+    return (e / e.sum(-1, keepdims=True)).astype(F32)
+
+
+@pytest.mark.parametrize("H,S,D,bits", [(4, 128, 128, 3), (2, 512, 128, 3), (8, 64, 64, 4), (2, 777, 256, 3),
+                                        (3, 100, 32, 2), (1, 5000, 128, 3)])
+def test_sparse_v_dense_threshold(tq, H, S, D, bits):
+    rng = np.random.default_rng(12)
+    c, s, vp, vn = v_fixture(rng, H, S, D, bits)
+    w = softmax_np(rng.standard_normal((H, S)) * 3)
+    want = o.sparse_v_matvec(w, vp, vn, c, s, D, bits, threshold=0.0)
+    got = host(tq.sparse_v_matvec(dev(w), dev(vp), dev(vn), c, dev(s), D, bits, threshold=0.0))
+    assert np.abs(got - want).max() / np.abs(want).max() < 1e-5         # test_sparse_v.py:47-76
+
+
+def test_sparse_v_threshold_semantics(tq):
+    rng = np.random.default_rng(13)
+    H, S, D, bits = 4, 2048, 128, 3
+    c, s, vp, vn = v_fixture(rng, H, S, D, bits)
+    w = softmax_np(rng.standard_normal((H, S)) * 5)
+    args = (dev(vp), dev(vn), c, dev(s), D, bits)
+    for thr in (1e-5, 1e-4, 1e-3):
+        want = o.sparse_v_matvec(w, vp, vn, c, s, D, bits, threshold=thr)
+        got = host(tq.sparse_v_matvec(dev(w), *args, threshold=thr))
+        assert np.abs(got - want).max() < 1e-5 * np.abs(want).max()
+    dense = host(tq.sparse_v_matvec(dev(w), *args, threshold=0.0))
+    sp = host(tq.sparse_v_matvec(dev(w), *args))                         # default threshold 1e-5
+    assert (sp * dense).sum() / np.linalg.norm(sp) / np.linalg.norm(dense) > 0.999
+    zero = host(tq.sparse_v_matvec(dev(w), *args, threshold=2.0))
+    assert (zero == 0).all()                                             # test_sparse_v.py:150-168
+    neg = host(tq.sparse_v_matvec(dev(w), *args, threshold=-1.0))
+    assert np.array_equal(neg, dense)
+    assert tq.count_active_positions(dev(w), 1e-5) == o.count_active_positions(w, 1e-5)
+
+
+@pytest.mark.parametrize("n_kv,n_rep", [(4, 2), (2, 4), (4, 7), (2, 9)])
+def test_sparse_v_gqa(tq, n_kv, n_rep):
+    rng = np.random.default_rng(14)
+    S, D, bits = 400, 128, 3
+    c, s, vp, vn = v_fixture(rng, n_kv, S, D, bits)
+    w = softmax_np(rng.standard_normal((n_kv * n_rep, S)))
+    want = o.sparse_v_matvec(w, vp, vn, c, s, D, bits, 0.0, n_rep)
+    got = host(tq.sparse_v_matvec(dev(w), dev(vp), dev(vn), c, dev(s), D, bits, threshold=0.0, n_rep=n_rep))
+    assert np.abs(got - want).max() < 1e-5 * np.abs(want).max()
+    with pytest.raises(ValueError, match="power of 2"):
+        tq.sparse_v_matvec(dev(w), dev(vp), dev(vn), c, dev(s), 96, bits)
+    with pytest.raises(ValueError, match="dim > 256"):
+        tq.sparse_v_matvec(dev(w), dev(vp), dev(vn), c, dev(s), 512, bits)
+    with pytest.raises(ValueError, match="must equal n_kv_heads"):
+        tq.sparse_v_matvec(dev(w[:-1]), dev(vp), dev(vn), c, dev(s), D, bits, n_rep=n_rep)
+
+
+# ------------------------------------------------------------------ flash decode
+
+def kv_fixture(rng, n_kv, S, D, bits, outliers=False):
+    c, b = tables(bits)
+    ks, vs = o.random_diagonal_sign(D, 42), o.random_diagonal_sign(D, 43)
+    K = rng.standard_normal((n_kv, S, D)).astype(np.float16)
+    V = rng.standard_normal((n_kv, S, D)).astype(np.float16)
+    if outliers:
+        K[..., 7] *= 20
+        V[..., 19] *= 20
+    kp, kn = o.fused_quantize(K.reshape(-1, D), ks, b, D, bits)
+    vp, vn = o.fused_quantize(V.reshape(-1, D), vs, b, D, bits)
+    pd = o.packed_dim(D, bits)
+    return (c, ks, vs, K, V, kp.reshape(n_kv, S, pd), kn.reshape(n_kv, S),
+            vp.reshape(n_kv, S, pd), vn.reshape(n_kv, S))
+
+
+@pytest.mark.parametrize("n_kv,n_rep,S,D,bits,bc", [(4, 1, 64, 128, 3, 16), (2, 1, 96, 128, 3, 32),
+                                                    (8, 1, 256, 128, 3, 16), (2, 1, 33, 64, 4, 8),
+                                                    (1, 1, 128, 32, 2, 1), (4, 2, 300, 128, 3, 16),
+                                                    (2, 4, 1025, 128, 3, 16), (4, 7, 2000, 128, 3, 16)])
+def test_flash_matches_oracle(tq, n_kv, n_rep, S, D, bits, bc):
+    rng = np.random.default_rng(15)
+    c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, n_kv, S, D, bits)
+    q = rng.standard_normal((n_kv * n_rep, D)).astype(F32)
+    sc = 1 / math.sqrt(D)
+    want = o.flash_attention_turboquant(o.prerotate_query(q, ks), kp, kn, vp, vn, c, c, vs, D, bits, sc, bc, n_rep)
+    q_rot = tq.prerotate_query(dev(q), dev(ks))
+    got = host(tq.flash_attention_turboquant(q_rot, dev(kp), dev(kn), dev(vp), dev(vn), c, c, dev(vs),
+                                             D, bits, sc, block_size=bc, n_rep=n_rep))
+    assert np.abs(got - want).max() < 1e-3 * np.abs(want).max()          # test_flash_attention.py:38-137
+    close(got, want)
+    # equals the unfused composition on the GPU as well
+    scores = tq.prerot_fused_qk_scores(q_rot, dev(kp), dev(kn), c, D, bits, n_rep=n_rep)
+    w = tq.softmax_rows(scores, sc)
+    comp = host(tq.sparse_v_matvec(w, dev(vp), dev(vn), c, dev(vs), D, bits, threshold=0.0, n_rep=n_rep))
+    assert np.abs(got - comp).max() < 1e-3 * np.abs(comp).max()
+
+
+def test_flash_argument_errors(tq):
+    rng = np.random.default_rng(16)
+    c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, 2, 32, 128, 3)
+    q = dev(rng.standard_normal((2, 128)).astype(F32))
+    a = (dev(kp), dev(kn), dev(vp), dev(vn), c, c, dev(vs))
+    with pytest.raises(ValueError, match="block_size must be in 1..32"):
+        tq.flash_attention_turboquant(q, *a, 128, 3, 0.1, block_size=33)
+    with pytest.raises(ValueError, match="<= 128"):
+        tq.flash_attention_turboquant(q, *a, 256, 3, 0.1)
+    with pytest.raises(ValueError, match="must equal n_kv_heads"):
+        tq.flash_attention_turboquant(q, *a, 128, 3, 0.1, n_rep=2)
+
+
+def test_flash_ragged_batch(tq):
+    """A batch of sequences of different lengths in one launch (BASELINE config 4 shape, scaled down):
+    32 q heads, 8 kv heads, lengths drawn from the seed, fp16 output."""
+    rng = np.random.default_rng(17)
+    n_kv, n_rep, D, bits, n_seq = 8, 4, 128, 3, 5
+    lens = rng.integers(40, 700, size=n_seq)
+    offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, n_kv, int(offs[-1]), D, bits)
+    q = rng.standard_normal((n_seq, n_kv * n_rep, D)).astype(np.float16)
+    sc = 1 / math.sqrt(D)
+    q_rot = tq.prerotate_query(dev(q.reshape(-1, D)), dev(ks)).reshape(n_seq, n_kv * n_rep, D)
+    got = tq.flash_decode(q_rot, dev(kp), dev(kn), dev(vp), dev(vn), c, c, dev(vs), D, bits, sc, n_rep=n_rep,
+                          seq_offsets=dev(offs), max_seq_len=int(lens.max()), out_dtype=torch.float16)
+    assert got.dtype == torch.float16
+    got = host(got).astype(F32)
+    for i in range(n_seq):
+        a, e = offs[i], offs[i + 1]
+        want = o.flash_attention_turboquant(o.prerotate_query(q[i], ks), kp[:, a:e], kn[:, a:e], vp[:, a:e],
+                                            vn[:, a:e], c, c, vs, D, bits, sc, 16, n_rep)
+        close(got[i], want)
+
+
+def test_flash_mask_and_cache_layout(tq):
+    rng = np.random.default_rng(18)
+    n_kv, n_rep, D, bits, B, T_alloc, total = 2, 2, 128, 3, 3, 512, 301
+    sc = 1 / math.sqrt(D)
+    c, b = tables(bits)
+    ks, vs = o.random_diagonal_sign(D, 42), o.random_diagonal_sign(D, 43)
+    kp = o.pack_indices(rng.integers(0, 8, size=(B, n_kv, T_alloc, D)).astype(np.uint8), bits)
+    vp = o.pack_indices(rng.integers(0, 8, size=(B, n_kv, T_alloc, D)).astype(np.uint8), bits)
+    kn = (rng.random((B, n_kv, T_alloc)) + 0.5).astype(F32)
+    vn = (rng.random((B, n_kv, T_alloc)) + 0.5).astype(F32)
+    q = rng.standard_normal((B, n_kv * n_rep, D)).astype(F32)
+    mask = np.where(rng.random((B, 1, total)) < 0.3, -np.inf, 0.0).astype(F32)
+    q_rot = tq.prerotate_query(dev(q.reshape(-1, D)), dev(ks)).reshape(B, -1, D)
+    got = host(tq.flash_decode(q_rot, dev(kp), dev(kn), dev(vp), dev(vn), c, c, dev(vs), D, bits, sc,
+                               n_rep=n_rep, seq_len=total, mask=dev(mask)))
+    for i in range(B):
+        want = o.turboquant_attention_single(q[i], kp[i, :, :total], kn[i, :, :total], vp[i, :, :total],
+                                             vn[i, :, :total], c, ks, c, vs, D, bits, sc, mask=mask[i])
+        close(got[i], want)
+
+
+# ------------------------------------------------------------------ V-only decode
+
+@pytest.mark.parametrize("n_kv,n_rep,T,D", [(4, 7, 1000, 128), (2, 1, 64, 128), (8, 4, 513, 128), (2, 3, 300, 64),
+                                           (1, 9, 257, 128)])
+def test_vonly_decode_matches_oracle(tq, n_kv, n_rep, T, D):
+    rng = np.random.default_rng(19)
+    bits = 3
+    c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, n_kv, T, D, bits)
+    q = rng.standard_normal((1, n_kv * n_rep, D)).astype(np.float16)
+    sc = 1 / math.sqrt(D)
+    got = host(tq.vonly_decode(dev(q), dev(K), dev(vp), dev(vn), c, dev(vs), D, bits, sc, n_rep=n_rep))
+    want = o.vonly_decode_attention(q[0], K, vp, vn, c, vs, D, bits, sc)
+    close(got[0], want)
+
+
+def test_vonly_decode_ragged_and_mask(tq):
+    rng = np.random.default_rng(20)
+    n_kv, n_rep, D, bits, n_seq = 4, 7, 128, 3, 4
+    lens = rng.integers(10, 900, size=n_seq)
+    offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, n_kv, int(offs[-1]), D, bits)
+    q = rng.standard_normal((n_seq, n_kv * n_rep, D)).astype(np.float16)
+    sc = 1 / math.sqrt(D)
+    got = host(tq.vonly_decode(dev(q), dev(K), dev(vp), dev(vn), c, dev(vs), D, bits, sc, n_rep=n_rep,
+                               seq_offsets=dev(offs), max_seq_len=int(lens.max())))
+    for i in range(n_seq):
+        a, e = offs[i], offs[i + 1]
+        want = o.vonly_decode_attention(q[i], K[:, a:e], vp[:, a:e], vn[:, a:e], c, vs, D, bits, sc)
+        close(got[i], want)
+
+
+def test_config2_full_size(tq):
+    """BASELINE config 2 at full size: 28 q / 4 kv heads, d=128, 32768 positions; V encoded on the
+    GPU (bit-exact against the oracle), then the fused V-only decode step against the oracle."""
+    rng = np.random.default_rng(2)
+    n_kv, n_rep, T, D, bits = 4, 7, 32768, 128, 3
+    c, b = tables(bits)
+    vs = o.random_diagonal_sign(D, 43)
+    K = rng.standard_normal((n_kv, T, D)).astype(np.float16)
+    V = rng.standard_normal((n_kv, T, D)).astype(np.float16)
+    q = rng.standard_normal((1, n_kv * n_rep, D)).astype(np.float16)
+    sc = 1 / math.sqrt(D)
+    wp, wn = o.fused_quantize(V.reshape(-1, D), vs, b, D, bits)
+    gp, gn = tq.fused_quantize(dev(V.reshape(-1, D)), dev(vs), b, D, bits)
+    assert np.array_equal(host(gp), wp) and np.array_equal(host(gn), wn)
+    vp, vn = gp.reshape(n_kv, T, -1), gn.reshape(n_kv, T)
+    got = host(tq.vonly_decode(dev(q), dev(K), vp, vn, c, dev(vs), D, bits, sc, n_rep=n_rep))
+    want = o.vonly_decode_attention(q[0], K, wp.reshape(n_kv, T, -1), wn.reshape(n_kv, T), c, vs, D, bits, sc)
+    close(got[0], want)
+    # unfused sparse path with the default threshold stays within cosine 0.999 of dense
+    scores = tq.dense_qk_scores(dev(q[0]), dev(K), 1.0, n_rep=n_rep)
+    w = tq.softmax_rows(scores, sc)
+    sp = host(tq.sparse_v_matvec(w, vp, vn, c, dev(vs), D, bits, threshold=1e-5, n_rep=n_rep))
+    want_sp = o.vonly_decode_attention(q[0], K, wp.reshape(n_kv, T, -1), wn.reshape(n_kv, T), c, vs, D, bits,
+                                       sc, threshold=1e-5)
+    close(sp, want_sp)
+    assert (sp * want).sum() / np.linalg.norm(sp) / np.linalg.norm(want) > 0.999
+
+
+@pytest.mark.parametrize("T", [4096, 16384, 65536])
+def test_config3_scores(tq, T):
+    """BASELINE config 3: pre-rotated-Q scoring over packed K, 28/4 heads, d=128."""
+    rng = np.random.default_rng(3)
+    n_kv, n_rep, D, bits = 4, 7, 128, 3
+    c, b = tables(bits)
+    ks = o.random_diagonal_sign(D, 42)
+    K = rng.standard_normal((n_kv * T, D)).astype(np.float16)
+    q = rng.standard_normal((n_kv * n_rep, D)).astype(np.float16)
+    gp, gn = tq.fused_quantize(dev(K), dev(ks), b, D, bits)
+    q_rot = tq.prerotate_query(dev(q), dev(ks))
+    got = host(tq.prerot_fused_qk_scores(q_rot, gp.reshape(n_kv, T, -1), gn.reshape(n_kv, T), c, D, bits, n_rep=n_rep))
+    want = o.prerot_fused_qk_scores(o.prerotate_query(q, ks), host(gp).reshape(n_kv, T, -1),
+                                    host(gn).reshape(n_kv, T), c, D, bits, n_rep)
+    assert got.shape == (28, T) and got.dtype == F32
+    close(got, want, rel=1e-4, abs_=1e-4)

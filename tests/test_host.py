@@ -1,0 +1,121 @@
+"""CPU-side tests: the C-ABI library loads and exports every declared symbol, argument errors are
+raised before any launch, and the host logic (sign generator, tables, packing, meta strings,
+masks) matches the oracle.  No kernel is launched here."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+
+import tqhip  # noqa: E402
+from tqhip import _lib, ops  # noqa: E402
+from oracle import polarquant_oracle as o  # noqa: E402
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    header = open(os.path.join(ROOT, "include", "tqhip.h")).read()
+    declared = set(re.findall(r"\b(tq_[a-z0-9_]+)\s*\(", header))
+    assert declared, "no declarations parsed"
+    assert declared == set(_lib.PROTOTYPES), declared ^ set(_lib.PROTOTYPES)
+    for name in declared:
+        assert getattr(lib, name) is not None
+    assert lib.tq_version() >= 100
+    assert lib.tq_status_string(-3) == b"bad bits"
+
+
+def test_decode_shape_struct_matches_header_size():
+    # 6 int32 + int64 + ptr + 8 int64 + ptr + 2 int64 + float + int32
+    assert ctypes.sizeof(_lib.DecodeShape) == 6 * 4 + 8 + 8 + 8 * 8 + 8 + 2 * 8 + 4 + 4
+
+
+def test_argument_errors_without_launch():
+    lib = _lib.load()
+    null = ctypes.c_void_p(0)
+    b = _lib.host_floats([0.0] * 7)
+    assert lib.tq_encode(null, 1, null, b, null, null, 1, 4, 0, 0, 128, 5, 0, null) == -3
+    assert b"Unsupported bit width: 5" in lib.tq_last_error()
+    assert lib.tq_encode(null, 1, null, b, null, null, 1, 4, 0, 0, 96, 3, 0, null) == -2
+    assert b"power of 2" in lib.tq_last_error()
+    assert lib.tq_encode(null, 7, null, b, null, null, 1, 4, 0, 0, 128, 3, 0, null) == -6
+    assert lib.tq_encode(null, 1, null, b, null, null, 1, 4, 0, 0, 128, 3, 0, null) == -1
+    assert lib.tq_encode(null, 1, null, b, null, null, 0, 4, 0, 0, 128, 3, 0, null) == 0   # empty: no-op
+    assert lib.tq_prerot_qk_scores(null, null, null, b, null, 4, 0, 16, 0, 0, 128, 3, null) == -4
+    assert lib.tq_sparse_v_matvec(null, null, null, b, null, null, null, 0, 4, 7, 16, 0, 0, 512, 3, 0.0, null) == -2
+    assert b"dim > 256" in lib.tq_last_error()
+    sh = _lib.DecodeShape()
+    sh.n_seq, sh.n_kv_heads, sh.n_rep, sh.dim, sh.bits, sh.block_size, sh.seq_len = 1, 2, 1, 128, 3, 33, 8
+    rc = lib.tq_flash_decode(null, null, null, null, null, b, b, null, null, null, 0, ctypes.byref(sh), null)
+    assert rc == -7 and b"block_size must be in 1..32" in lib.tq_last_error()
+    with pytest.raises(ValueError, match="block_size must be in 1..32"):
+        _lib.check(rc)
+    sh.block_size, sh.dim = 16, 256
+    assert lib.tq_flash_decode(null, null, null, null, null, b, b, null, null, null, 0, ctypes.byref(sh), null) == -2
+    with pytest.raises(RuntimeError):
+        _lib.check(-8)
+    assert lib.tq_workspace_bytes(2, 1, 28, 32768, 128) == 28 * 128 * 130 * 4
+
+
+def test_kernels_refuse_cpu_tensors():
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        tqhip.fused_quantize(torch.zeros(2, 128), torch.ones(128), [0.0] * 7, 128, 3)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        tqhip.prerotate_query(torch.zeros(2, 128), torch.ones(128))
+    with pytest.raises(ValueError, match="expects"):
+        tqhip.prerotate_query(torch.zeros(128), torch.ones(128))
+    with pytest.raises(KeyError):
+        tqhip.fused_quantize(torch.zeros(2, 128), torch.ones(128), [0.0], 128, 5)
+    with pytest.raises(ValueError, match="power of 2"):
+        tqhip.sparse_v_matvec(torch.zeros(2, 4), torch.zeros(2, 4, 13), torch.zeros(2, 4), [0.0] * 8,
+                              torch.ones(96), 96, 3)
+
+
+def test_sign_generator_and_tables_match_oracle():
+    for d, seed in ((128, 42), (128, 43), (64, 7), (256, 0)):
+        assert np.array_equal(tqhip.random_diagonal_sign(d, seed).numpy(), o.random_diagonal_sign(d, seed))
+    from tqhip.quantizer import gaussian_boundaries, gaussian_codebook
+    for bits in (1, 2, 3, 4):
+        c = gaussian_codebook(bits)
+        assert np.array_equal(c.numpy(), o.gaussian_codebook(bits))
+        assert np.array_equal(gaussian_boundaries(c).numpy(), o.gaussian_boundaries(o.gaussian_codebook(bits)))
+    with pytest.raises(ValueError, match="Unsupported bit width"):
+        gaussian_codebook(5)
+
+
+@pytest.mark.parametrize("bits,dim", [(1, 128), (2, 32), (3, 128), (3, 64), (4, 64)])
+def test_pack_unpack_match_oracle(bits, dim):
+    rng = np.random.default_rng(bits)
+    idx = rng.integers(0, 2 ** bits, size=(3, 7, dim)).astype(np.uint8)
+    p = tqhip.pack_indices(torch.from_numpy(idx), bits)
+    assert p.dtype == torch.uint32 and p.shape == (3, 7, tqhip.packed_dim(dim, bits))
+    assert np.array_equal(p.numpy(), o.pack_indices(idx, bits))
+    assert np.array_equal(tqhip.unpack_indices(p, bits, dim).numpy(), idx)
+    assert tqhip.packed_dim(128, 3) == 13
+
+
+def test_cache_meta_state_and_masks_on_host():
+    c = tqhip.TurboQuantKVCache(bits=3, seed=9)
+    assert c.meta_state == "0,3,9,0,0,float16" and c.state == [] and c.empty() and c.nbytes == 0
+    assert c.compression_ratio == 1.0
+    c.meta_state = "12,4,5,64,128,bfloat16"
+    assert (c.offset, c.quant_bits, c.seed, c._k_dim, c._v_dim, c._dtype) == (12, 4, 5, 64, 128, torch.bfloat16)
+    c.meta_state = "3,2,1,0,128"
+    assert c._k_dim is None and c._dtype == torch.float16
+    v = tqhip.VOnlyTurboQuantCache(bits=2, seed=11)
+    assert v.meta_state == "VOnlyTQ,2,11,0,2,11,0,0,float16" and v.empty() and v.state == []
+    m = tqhip.create_causal_mask(3, offset=2)
+    assert m.tolist() == [[True, True, True, False, False], [True] * 4 + [False], [True] * 5]
+    kv = tqhip.KVCache()
+    k = torch.randn(1, 2, 300, 16)
+    ko, vo = kv.update_and_fetch(k, k)
+    assert kv.keys.shape[2] == 512 and kv.offset == 300 and torch.equal(ko, k)
+    kv.update_and_fetch(k[..., :5, :], k[..., :5, :])
+    assert kv.offset == 305 and kv.trim(10) == 10 and kv.size() == 295
+    assert kv.make_mask(1) is None and kv.make_mask(2) == "causal"
+    r = tqhip.KVCache.from_state(kv.state)
+    assert r.offset == 295 and torch.equal(r.keys, k[..., :295, :])

@@ -1,0 +1,626 @@
+// Decode-attention kernels over packed PolarQuant K/V for gfx950, float32 vector-ALU path.
+//
+// KV positions are the parallel axis: a workgroup owns one tile of kTile positions of ONE kv
+// head and serves all n_rep query heads of that kv head from a single read of the tile.  The
+// V side accumulates sum_p w_p * norm_p * c[idx_p] in the rotated domain (no butterfly per
+// position); partial sums (and the online-softmax statistics m, l) go to a workspace and a
+// second pass merges the tiles, applies the ONE Walsh-Hadamard butterfly per output row, the
+// signs and the 1/dim factor.
+#include "tq_common.h"
+
+#include <math.h>
+
+namespace {
+
+using namespace tqd;
+
+constexpr int kTile = 256;          // positions per workgroup, one per thread in the score phase
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / TQ_WAVE;
+constexpr int kRMax = 8;            // query heads per kv head served by one workgroup
+
+enum KMode { kWeights = 0, kPackedK = 1, kDenseK = 2 };
+
+struct DecodeArgs {
+  // query side
+  const void* q;                // kPackedK: q_rot f32; kDenseK: q (dtype QT); kWeights: weights f32 [n_q, T]
+  // key side
+  const uint32_t* k_packed;
+  const float* k_norms;
+  const __half* k_dense;
+  // value side
+  const uint32_t* v_packed;
+  const float* v_norms;
+  const int32_t* seq_offsets;
+  const float* mask;
+  float* ws_S;                  // [n_seq*n_q, n_tiles_max, D]
+  float* ws_ml;                 // [n_seq*n_q, n_tiles_max, 2]
+  int64_t seq_len;
+  int64_t k_seq_stride, k_head_stride, kn_seq_stride, kn_head_stride;
+  int64_t v_seq_stride, v_head_stride, vn_seq_stride, vn_head_stride;
+  int64_t mask_seq_stride, mask_head_stride;
+  int32_t n_kv, n_rep, n_rgroups, n_tiles_max;
+  float attn_scale, inv_dim, threshold;
+};
+
+__device__ __forceinline__ void seq_range(const int32_t* seq_offsets, int64_t seq_len, int seq,
+                                          int64_t& first, int64_t& len) {
+  if (seq_offsets) {
+    first = seq_offsets[seq];
+    len = (int64_t)seq_offsets[seq + 1] - first;
+  } else {
+    first = 0;
+    len = seq_len;
+  }
+}
+
+// ---- score of one position against up to kRMax query heads, packed keys:
+//      acc[r] = sum_e c[idx_e] * q_rot[r][e]           (q_s is [D][kRMax] in LDS)
+template <int D, int BITS>
+__device__ __forceinline__ void score_packed(const uint32_t* __restrict__ krow, const float* cb,
+                                             const float (*q_s)[kRMax], float (&acc)[kRMax]) {
+  constexpr int VPW = Pk<BITS>::VPW;
+  constexpr int PDIM = Pk<BITS>::pdim(D);
+#pragma unroll
+  for (int r = 0; r < kRMax; ++r) acc[r] = 0.0f;
+#pragma unroll 1
+  for (int w = 0; w < PDIM; ++w) {
+    const uint32_t word = krow[w];
+#pragma unroll
+    for (int i = 0; i < VPW; ++i) {
+      const int e = w * VPW + i;
+      if (e < D) {
+        const float c = cb[(word >> (i * BITS)) & Pk<BITS>::MASK];
+        const float4 qa = *reinterpret_cast<const float4*>(&q_s[e][0]);
+        const float4 qb = *reinterpret_cast<const float4*>(&q_s[e][4]);
+        acc[0] += c * qa.x; acc[1] += c * qa.y; acc[2] += c * qa.z; acc[3] += c * qa.w;
+        acc[4] += c * qb.x; acc[5] += c * qb.y; acc[6] += c * qb.z; acc[7] += c * qb.w;
+      }
+    }
+  }
+}
+
+// ---- same for fp16 keys: acc[r] = sum_e K[e] * q[r][e]
+template <int D>
+__device__ __forceinline__ void score_dense(const __half* __restrict__ krow, const float (*q_s)[kRMax],
+                                            float (&acc)[kRMax]) {
+#pragma unroll
+  for (int r = 0; r < kRMax; ++r) acc[r] = 0.0f;
+#pragma unroll 1
+  for (int e0 = 0; e0 < D; e0 += 8) {
+    const uint4 raw = *reinterpret_cast<const uint4*>(krow + e0);
+    const __half2* h2 = reinterpret_cast<const __half2*>(&raw);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float2 kf = __half22float2(h2[j]);
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const float kv = u ? kf.y : kf.x;
+        const int e = e0 + 2 * j + u;
+        const float4 qa = *reinterpret_cast<const float4*>(&q_s[e][0]);
+        const float4 qb = *reinterpret_cast<const float4*>(&q_s[e][4]);
+        acc[0] += kv * qa.x; acc[1] += kv * qa.y; acc[2] += kv * qa.z; acc[3] += kv * qa.w;
+        acc[4] += kv * qb.x; acc[5] += kv * qb.y; acc[6] += kv * qb.z; acc[7] += kv * qb.w;
+      }
+    }
+  }
+}
+
+template <typename QT, int D>
+__device__ __forceinline__ void load_q_tile(const QT* __restrict__ q, int64_t q_row0, int n_local,
+                                            float (*q_s)[kRMax]) {
+  for (int i = threadIdx.x; i < D * kRMax; i += kThreads) {
+    const int r = i / D, e = i % D;
+    q_s[e][r] = (r < n_local) ? load_as_float<QT>(q + (q_row0 + r) * D + e) : 0.0f;
+  }
+}
+
+// ---------------------------------------------------------------- stand-alone score kernels
+template <int D, int BITS>
+__global__ __launch_bounds__(kThreads) void prerot_scores_kernel(const float* __restrict__ q_rot,
+                                                                 const uint32_t* __restrict__ k_packed,
+                                                                 const float* __restrict__ k_norms,
+                                                                 Codebook cbk, float* __restrict__ scores,
+                                                                 int n_rep, int n_rgroups, int64_t seq_len,
+                                                                 int64_t p_head_stride, int64_t n_head_stride,
+                                                                 float inv_dim) {
+  constexpr int PDIM = Pk<BITS>::pdim(D);
+  __shared__ float cb[16];
+  __shared__ __align__(16) float q_s[D][kRMax];
+  const int kvh = blockIdx.y / n_rgroups;
+  const int r0 = (blockIdx.y % n_rgroups) * kRMax;
+  const int n_local = min(kRMax, n_rep - r0);
+  const int64_t q_row0 = (int64_t)kvh * n_rep + r0;
+  if (threadIdx.x < 16) cb[threadIdx.x] = cbk.c[threadIdx.x];
+  load_q_tile<float, D>(q_rot, q_row0, n_local, q_s);
+  __syncthreads();
+  const int64_t p = (int64_t)blockIdx.x * kTile + threadIdx.x;
+  if (p >= seq_len) return;
+  float acc[kRMax];
+  score_packed<D, BITS>(k_packed + ((int64_t)kvh * p_head_stride + p) * PDIM, cb, q_s, acc);
+  const float nrm = k_norms[(int64_t)kvh * n_head_stride + p];
+#pragma unroll
+  for (int r = 0; r < kRMax; ++r)
+    if (r < n_local) scores[(q_row0 + r) * seq_len + p] = (acc[r] * nrm) * inv_dim;
+}
+
+template <int D, typename QT>
+__global__ __launch_bounds__(kThreads) void dense_scores_kernel(const QT* __restrict__ q,
+                                                                const __half* __restrict__ k,
+                                                                float* __restrict__ scores, int n_rep,
+                                                                int n_rgroups, int64_t seq_len,
+                                                                int64_t k_head_stride, float scale) {
+  __shared__ __align__(16) float q_s[D][kRMax];
+  const int kvh = blockIdx.y / n_rgroups;
+  const int r0 = (blockIdx.y % n_rgroups) * kRMax;
+  const int n_local = min(kRMax, n_rep - r0);
+  const int64_t q_row0 = (int64_t)kvh * n_rep + r0;
+  load_q_tile<QT, D>(q, q_row0, n_local, q_s);
+  __syncthreads();
+  const int64_t p = (int64_t)blockIdx.x * kTile + threadIdx.x;
+  if (p >= seq_len) return;
+  float acc[kRMax];
+  score_dense<D>(k + ((int64_t)kvh * k_head_stride + p) * D, q_s, acc);
+#pragma unroll
+  for (int r = 0; r < kRMax; ++r)
+    if (r < n_local) scores[(q_row0 + r) * seq_len + p] = acc[r] * scale;
+}
+
+// ---------------------------------------------------------------- row softmax
+__global__ __launch_bounds__(kThreads) void softmax_rows_kernel(const float* __restrict__ scores,
+                                                                const float* __restrict__ mask,
+                                                                int64_t mask_row_stride,
+                                                                float* __restrict__ weights, int64_t seq_len,
+                                                                float scale) {
+  __shared__ float red[kWaves];
+  const int64_t row = blockIdx.x;
+  const float* s = scores + row * seq_len;
+  const float* mk = mask ? mask + row * mask_row_stride : nullptr;
+  float* w = weights + row * seq_len;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float m = -INFINITY;
+  for (int64_t p = threadIdx.x; p < seq_len; p += kThreads) {
+    float v = s[p] * scale;
+    if (mk) v += mk[p];
+    m = fmaxf(m, v);
+  }
+  m = wave_max(m);
+  if (lane == 0) red[wave] = m;
+  __syncthreads();
+  m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  __syncthreads();
+  if (m == -INFINITY) m = 0.0f;
+  float l = 0.0f;
+  for (int64_t p = threadIdx.x; p < seq_len; p += kThreads) {
+    float v = s[p] * scale;
+    if (mk) v += mk[p];
+    l += expf(v - m);
+  }
+  l = wave_sum(l);
+  if (lane == 0) red[wave] = l;
+  __syncthreads();
+  l = (red[0] + red[1]) + (red[2] + red[3]);
+  for (int64_t p = threadIdx.x; p < seq_len; p += kThreads) {
+    float v = s[p] * scale;
+    if (mk) v += mk[p];
+    w[p] = expf(v - m) / l;
+  }
+}
+
+// ---------------------------------------------------------------- fused tile pass
+// grid = (n_tiles_max, n_kv * n_rgroups, n_seq)
+template <int D, int BITS, int KMODE, typename QT>
+__global__ __launch_bounds__(kThreads) void decode_tile_kernel(DecodeArgs a, Codebook kcb, Codebook vcb) {
+  constexpr int EPL = Lay<D>::EPL;
+  constexpr int VPW = Pk<BITS>::VPW;
+  constexpr int PDIM = Pk<BITS>::pdim(D);
+  __shared__ float cbk_s[16], cbv_s[16];
+  __shared__ __align__(16) float q_s[KMODE == kWeights ? 1 : D][kRMax];
+  __shared__ float p_s[kRMax][kTile];
+  __shared__ float red_s[kWaves][kRMax];
+  __shared__ float acc_s[kWaves][kRMax][D >= 64 ? D : 64];
+
+  const int tile = blockIdx.x;
+  const int kvh = blockIdx.y / a.n_rgroups;
+  const int r0 = (blockIdx.y % a.n_rgroups) * kRMax;
+  const int n_local = min(kRMax, a.n_rep - r0);
+  const int seq = blockIdx.z;
+  const int n_q = a.n_kv * a.n_rep;
+  const int64_t q_row0 = (int64_t)seq * n_q + (int64_t)kvh * a.n_rep + r0;   // row in [n_seq*n_q]
+  int64_t first, len;
+  seq_range(a.seq_offsets, a.seq_len, seq, first, len);
+  const int64_t p0 = (int64_t)tile * kTile;
+  if (p0 >= len) return;     // tile past the end of this sequence: the merge pass never reads it
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+
+  if (threadIdx.x < 16) {
+    cbk_s[threadIdx.x] = kcb.c[threadIdx.x];
+    cbv_s[threadIdx.x] = vcb.c[threadIdx.x];
+  }
+  if (KMODE != kWeights) load_q_tile<QT, D>(reinterpret_cast<const QT*>(a.q), q_row0, n_local, q_s);
+  __syncthreads();
+
+  // ---- phase 1: one position per thread -> up to kRMax scores / weights
+  const int64_t p = p0 + threadIdx.x;
+  const bool live = p < len;
+  float sc[kRMax];
+  if (KMODE == kWeights) {
+    const float* wts = reinterpret_cast<const float*>(a.q);
+#pragma unroll
+    for (int r = 0; r < kRMax; ++r) {
+      float w = 0.0f;
+      if (live && r < n_local) {
+        w = wts[(q_row0 + r) * len + p];
+        if (w < a.threshold) w = 0.0f;
+      }
+      p_s[r][threadIdx.x] = w;
+    }
+  } else {
+    if (live) {
+      if (KMODE == kPackedK) {
+        const int64_t row = (int64_t)seq * a.k_seq_stride + (int64_t)kvh * a.k_head_stride + first + p;
+        score_packed<D, BITS>(a.k_packed + row * PDIM, cbk_s, q_s, sc);
+        const float nrm = a.k_norms[(int64_t)seq * a.kn_seq_stride + (int64_t)kvh * a.kn_head_stride + first + p];
+#pragma unroll
+        for (int r = 0; r < kRMax; ++r) sc[r] = ((sc[r] * nrm) * a.inv_dim) * a.attn_scale;
+      } else {
+        const int64_t row = (int64_t)seq * a.k_seq_stride + (int64_t)kvh * a.k_head_stride + first + p;
+        score_dense<D>(a.k_dense + row * D, q_s, sc);
+#pragma unroll
+        for (int r = 0; r < kRMax; ++r) sc[r] = sc[r] * a.attn_scale;
+      }
+      if (a.mask) {
+#pragma unroll
+        for (int r = 0; r < kRMax; ++r)
+          if (r < n_local)
+            sc[r] += a.mask[(int64_t)seq * a.mask_seq_stride +
+                            ((int64_t)kvh * a.n_rep + r0 + r) * a.mask_head_stride + p];
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < kRMax; ++r) sc[r] = -INFINITY;
+    }
+    // ---- phase 2: tile-local softmax statistics
+    float mx[kRMax];
+#pragma unroll
+    for (int r = 0; r < kRMax; ++r) {
+      float m = wave_max(sc[r]);
+      if (lane == 0) red_s[wave][r] = m;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < kRMax; ++r)
+      mx[r] = fmaxf(fmaxf(red_s[0][r], red_s[1][r]), fmaxf(red_s[2][r], red_s[3][r]));
+    __syncthreads();
+    float ls[kRMax];
+#pragma unroll
+    for (int r = 0; r < kRMax; ++r) {
+      const float e = (mx[r] == -INFINITY) ? 0.0f : expf(sc[r] - mx[r]);
+      p_s[r][threadIdx.x] = e;
+      ls[r] = wave_sum(e);
+      if (lane == 0) red_s[wave][r] = ls[r];
+    }
+    __syncthreads();
+    if (threadIdx.x < kRMax && threadIdx.x < n_local) {
+      const int r = threadIdx.x;
+      const float l = (red_s[0][r] + red_s[1][r]) + (red_s[2][r] + red_s[3][r]);
+      float* ml = a.ws_ml + ((q_row0 + r) * a.n_tiles_max + tile) * 2;
+      ml[0] = mx[r];
+      ml[1] = l;
+    }
+  }
+  __syncthreads();
+
+  // ---- phase 3: V accumulation in the rotated domain; wave w walks positions [64w, 64w+64)
+  float acc[kRMax][EPL];
+#pragma unroll
+  for (int r = 0; r < kRMax; ++r)
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) acc[r][i] = 0.0f;
+  int widx[EPL], wsh[EPL];
+#pragma unroll
+  for (int i = 0; i < EPL; ++i) {
+    const int e = lane + 64 * i;
+    widx[i] = (e < D) ? e / VPW : 0;
+    wsh[i] = (e % VPW) * BITS;
+  }
+  const int t_begin = wave * TQ_WAVE;
+  const int t_end = (int)min((int64_t)(t_begin + TQ_WAVE), len - p0);
+  const int64_t vrow0 = (int64_t)seq * a.v_seq_stride + (int64_t)kvh * a.v_head_stride + first + p0;
+  const int64_t vnrow0 = (int64_t)seq * a.vn_seq_stride + (int64_t)kvh * a.vn_head_stride + first + p0;
+  for (int t = t_begin; t < t_end; ++t) {
+    const uint32_t* vrow = a.v_packed + (vrow0 + t) * PDIM;
+    const float nrm = a.v_norms[vnrow0 + t];
+    float c[EPL];
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) c[i] = cbv_s[(vrow[widx[i]] >> wsh[i]) & Pk<BITS>::MASK];
+#pragma unroll
+    for (int r = 0; r < kRMax; ++r) {
+      const float wn = p_s[r][t] * nrm;
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) acc[r][i] += wn * c[i];
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < kRMax; ++r)
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) {
+      const int e = lane + 64 * i;
+      if (e < D) acc_s[wave][r][e] = acc[r][i];
+    }
+  __syncthreads();
+  // ---- phase 4: merge the four waves, fixed order, and emit the tile partial
+  for (int i = threadIdx.x; i < n_local * D; i += kThreads) {
+    const int r = i / D, e = i % D;
+    const float v = ((acc_s[0][r][e] + acc_s[1][r][e]) + acc_s[2][r][e]) + acc_s[3][r][e];
+    a.ws_S[((q_row0 + r) * a.n_tiles_max + tile) * D + e] = v;
+  }
+}
+
+// ---------------------------------------------------------------- merge pass
+// grid = (n_q, n_seq), one wavefront each.
+template <int D, int KMODE, typename TO>
+__global__ __launch_bounds__(TQ_WAVE) void decode_merge_kernel(const float* __restrict__ ws_S,
+                                                               const float* __restrict__ ws_ml,
+                                                               const int32_t* __restrict__ seq_offsets,
+                                                               int64_t seq_len, int n_tiles_max,
+                                                               const float* __restrict__ signs, float inv_dim,
+                                                               TO* __restrict__ out) {
+  constexpr int EPL = Lay<D>::EPL;
+  const int lane = threadIdx.x;
+  const int64_t row = (int64_t)blockIdx.y * gridDim.x + blockIdx.x;
+  int64_t first, len;
+  seq_range(seq_offsets, seq_len, blockIdx.y, first, len);
+  const int n_tiles = (int)((len + kTile - 1) / kTile);
+  const float* S = ws_S + row * n_tiles_max * D;
+  const float* ml = ws_ml + row * n_tiles_max * 2;
+  float v[EPL];
+#pragma unroll
+  for (int i = 0; i < EPL; ++i) v[i] = 0.0f;
+  float L = 1.0f;
+  if (KMODE == kWeights) {
+    for (int t = 0; t < n_tiles; ++t)
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) {
+        const int e = lane + 64 * i;
+        if (e < D) v[i] += S[(int64_t)t * D + e];
+      }
+  } else {
+    float M = -INFINITY;
+    for (int t = 0; t < n_tiles; ++t) M = fmaxf(M, ml[2 * t]);
+    L = 0.0f;
+    for (int t = 0; t < n_tiles; ++t) {
+      const float mt = ml[2 * t];
+      const float alpha = (mt == -INFINITY) ? 0.0f : expf(mt - M);
+      L += alpha * ml[2 * t + 1];
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) {
+        const int e = lane + 64 * i;
+        if (e < D) v[i] += alpha * S[(int64_t)t * D + e];
+      }
+    }
+  }
+  raw_butterfly<D>(v, lane);
+#pragma unroll
+  for (int i = 0; i < EPL; ++i) {
+    const int e = lane + 64 * i;
+    if (e < D) {
+      float o = (v[i] * signs[e]) * inv_dim;
+      if (KMODE != kWeights) o = (L > 0.0f) ? o / L : 0.0f;
+      store_from_float<TO>(out + row * D + e, o);
+    }
+  }
+}
+
+// ---------------------------------------------------------------- host side
+
+int n_tiles_for(int64_t len) { return (int)((len + kTile - 1) / kTile); }
+
+size_t ws_bytes(int n_seq, int n_q, int64_t max_len, int dim) {
+  const size_t tiles = (size_t)(n_tiles_for(max_len) > 0 ? n_tiles_for(max_len) : 1);
+  return (size_t)n_seq * n_q * tiles * ((size_t)dim + 2) * sizeof(float);
+}
+
+void fill_codebook(Codebook& cb, const float* c, int bits) {
+  for (int i = 0; i < 16; ++i) cb.c[i] = (c && i < (1 << bits)) ? c[i] : 0.0f;
+}
+
+int check_heads(int n_kv, int n_rep, const char* who) {
+  if (n_kv < 1) return tq::fail(TQ_ERR_ARG, "%s: n_kv_heads must be >= 1, got %d", who, n_kv);
+  if (n_rep < 1) return tq::fail(TQ_ERR_NREP, "%s: n_rep must be >= 1, got %d", who, n_rep);
+  return 0;
+}
+
+template <int KMODE>
+int launch_decode(const void* q, int q_dtype, const uint32_t* k_packed, const float* k_norms,
+                  const void* k_dense, const uint32_t* v_packed, const float* v_norms,
+                  const float* k_centroids, const float* v_centroids, const float* v_signs, void* out,
+                  void* workspace, size_t workspace_bytes, const tq_decode_shape& sh, float threshold,
+                  hipStream_t stream, const char* who) {
+  const int n_q = sh.n_kv_heads * sh.n_rep;
+  const size_t need = ws_bytes(sh.n_seq, n_q, sh.seq_len, sh.dim);
+  if (!workspace || workspace_bytes < need)
+    return tq::fail(TQ_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, need, workspace_bytes);
+  if (!tq::aligned(workspace, 16)) return tq::fail(TQ_ERR_ALIGN, "%s: workspace must be 16-byte aligned", who);
+  const int n_tiles = n_tiles_for(sh.seq_len);
+  const int n_tiles_max = n_tiles > 0 ? n_tiles : 1;
+  DecodeArgs a{};
+  a.q = q;
+  a.k_packed = k_packed; a.k_norms = k_norms; a.k_dense = (const __half*)k_dense;
+  a.v_packed = v_packed; a.v_norms = v_norms;
+  a.seq_offsets = sh.seq_offsets; a.mask = sh.mask;
+  a.ws_S = (float*)workspace;
+  a.ws_ml = a.ws_S + (size_t)sh.n_seq * n_q * n_tiles_max * sh.dim;
+  a.seq_len = sh.seq_len;
+  a.k_seq_stride = sh.k_seq_stride; a.k_head_stride = sh.k_head_stride;
+  a.kn_seq_stride = sh.kn_seq_stride; a.kn_head_stride = sh.kn_head_stride;
+  a.v_seq_stride = sh.v_seq_stride; a.v_head_stride = sh.v_head_stride;
+  a.vn_seq_stride = sh.vn_seq_stride; a.vn_head_stride = sh.vn_head_stride;
+  a.mask_seq_stride = sh.mask_seq_stride; a.mask_head_stride = sh.mask_head_stride;
+  a.n_kv = sh.n_kv_heads; a.n_rep = sh.n_rep;
+  a.n_rgroups = (sh.n_rep + kRMax - 1) / kRMax;
+  a.n_tiles_max = n_tiles_max;
+  a.attn_scale = sh.attn_scale;
+  a.inv_dim = 1.0f / (float)sh.dim;
+  a.threshold = threshold;
+  Codebook kcb, vcb;
+  fill_codebook(kcb, k_centroids, sh.bits);
+  fill_codebook(vcb, v_centroids, sh.bits);
+  if (n_tiles > 0) {
+    dim3 grid(n_tiles, sh.n_kv_heads * a.n_rgroups, sh.n_seq);
+#define LAUNCH_TILE(QT)                                                                              \
+  TQ_DISPATCH_DIM(sh.dim, TQ_DISPATCH_BITS(sh.bits, (decode_tile_kernel<D_, B_, KMODE, QT>            \
+                                                        <<<grid, kThreads, 0, stream>>>(a, kcb, vcb))))
+    if (KMODE == kDenseK && q_dtype == TQ_F16) { LAUNCH_TILE(__half); }
+    else if (KMODE == kDenseK && q_dtype == TQ_BF16) { LAUNCH_TILE(__hip_bfloat16); }
+    else { LAUNCH_TILE(float); }
+#undef LAUNCH_TILE
+    TQ_CHECK_LAUNCH(who);
+  }
+  dim3 mgrid(n_q, sh.n_seq);
+#define LAUNCH_MERGE(TO)                                                                              \
+  TQ_DISPATCH_DIM(sh.dim, (decode_merge_kernel<D_, KMODE, TO><<<mgrid, TQ_WAVE, 0, stream>>>(          \
+                              a.ws_S, a.ws_ml, sh.seq_offsets, sh.seq_len, n_tiles_max, v_signs,       \
+                              a.inv_dim, (TO*)out)))
+  if (sh.out_dtype == TQ_F16) { LAUNCH_MERGE(__half); }
+  else if (sh.out_dtype == TQ_BF16) { LAUNCH_MERGE(__hip_bfloat16); }
+  else { LAUNCH_MERGE(float); }
+#undef LAUNCH_MERGE
+  TQ_CHECK_LAUNCH(who);
+  return TQ_OK;
+}
+
+int check_shape(const tq_decode_shape* sh, const char* who, int max_dim) {
+  if (!sh) return tq::fail(TQ_ERR_NULL, "%s: null shape", who);
+  if (int rc = tq::check_dim_bits(sh->dim, sh->bits)) return rc;
+  if (sh->dim > max_dim)
+    return tq::fail(TQ_ERR_DIM, "dim must be a power of 2 and <= %d, got %d", max_dim, sh->dim);
+  if (int rc = check_heads(sh->n_kv_heads, sh->n_rep, who)) return rc;
+  if (sh->n_seq < 1) return tq::fail(TQ_ERR_ARG, "%s: n_seq must be >= 1, got %d", who, sh->n_seq);
+  if (sh->seq_len < 0) return tq::fail(TQ_ERR_ARG, "%s: negative seq_len", who);
+  if (sh->block_size < 1 || sh->block_size > 32)
+    return tq::fail(TQ_ERR_BLOCK, "block_size must be in 1..32, got %d", sh->block_size);
+  if (tq::check_dtype(sh->out_dtype)) return tq::fail(TQ_ERR_DTYPE, "%s: unknown out_dtype %d", who, sh->out_dtype);
+  return 0;
+}
+
+}  // namespace
+
+// ------------------------------------------------------------------ C ABI
+
+extern "C" size_t tq_workspace_bytes(int op, int n_seq, int n_q_heads, int64_t max_seq_len, int dim) {
+  (void)op;
+  if (n_seq < 1 || n_q_heads < 1 || max_seq_len < 0 || dim < 1) return 0;
+  return ws_bytes(n_seq, n_q_heads, max_seq_len, dim);
+}
+
+extern "C" int tq_prerot_qk_scores(const float* q_rot, const uint32_t* k_packed, const float* k_norms,
+                                   const float* centroids, float* scores, int n_kv_heads, int n_rep,
+                                   int64_t seq_len, int64_t packed_head_stride, int64_t norms_head_stride,
+                                   int dim, int bits, tq_stream_t stream_) {
+  if (int rc = tq::check_dim_bits(dim, bits)) return rc;
+  if (int rc = check_heads(n_kv_heads, n_rep, "tq_prerot_qk_scores")) return rc;
+  if (seq_len < 0) return tq::fail(TQ_ERR_ARG, "tq_prerot_qk_scores: negative seq_len");
+  if (seq_len == 0) return TQ_OK;
+  if (!q_rot || !k_packed || !k_norms || !centroids || !scores)
+    return tq::fail(TQ_ERR_NULL, "tq_prerot_qk_scores: null pointer");
+  Codebook cb;
+  fill_codebook(cb, centroids, bits);
+  const int n_rgroups = (n_rep + kRMax - 1) / kRMax;
+  dim3 grid(n_tiles_for(seq_len), n_kv_heads * n_rgroups);
+  hipStream_t stream = (hipStream_t)stream_;
+  TQ_DISPATCH_DIM(dim, TQ_DISPATCH_BITS(bits, (prerot_scores_kernel<D_, B_><<<grid, kThreads, 0, stream>>>(
+                                                  q_rot, k_packed, k_norms, cb, scores, n_rep, n_rgroups,
+                                                  seq_len, packed_head_stride, norms_head_stride,
+                                                  1.0f / (float)dim))));
+  TQ_CHECK_LAUNCH("tq_prerot_qk_scores launch");
+  return TQ_OK;
+}
+
+extern "C" int tq_dense_qk_scores(const void* q, int q_dtype, const void* k_f16, float* scores, int n_kv_heads,
+                                  int n_rep, int64_t seq_len, int64_t k_head_stride, int dim, float scale,
+                                  tq_stream_t stream_) {
+  if (int rc = tq::check_dim_bits(dim, 3)) return rc;
+  if (int rc = check_heads(n_kv_heads, n_rep, "tq_dense_qk_scores")) return rc;
+  if (tq::check_dtype(q_dtype)) return tq::fail(TQ_ERR_DTYPE, "tq_dense_qk_scores: unknown q_dtype %d", q_dtype);
+  if (seq_len < 0) return tq::fail(TQ_ERR_ARG, "tq_dense_qk_scores: negative seq_len");
+  if (seq_len == 0) return TQ_OK;
+  if (!q || !k_f16 || !scores) return tq::fail(TQ_ERR_NULL, "tq_dense_qk_scores: null pointer");
+  if (!tq::aligned(k_f16, 16)) return tq::fail(TQ_ERR_ALIGN, "tq_dense_qk_scores: k must be 16-byte aligned");
+  const int n_rgroups = (n_rep + kRMax - 1) / kRMax;
+  dim3 grid(n_tiles_for(seq_len), n_kv_heads * n_rgroups);
+  hipStream_t stream = (hipStream_t)stream_;
+#define LAUNCH_DS(QT)                                                                                   \
+  TQ_DISPATCH_DIM(dim, (dense_scores_kernel<D_, QT><<<grid, kThreads, 0, stream>>>(                       \
+                           (const QT*)q, (const __half*)k_f16, scores, n_rep, n_rgroups, seq_len,         \
+                           k_head_stride, scale)))
+  if (q_dtype == TQ_F32) { LAUNCH_DS(float); }
+  else if (q_dtype == TQ_F16) { LAUNCH_DS(__half); }
+  else { LAUNCH_DS(__hip_bfloat16); }
+#undef LAUNCH_DS
+  TQ_CHECK_LAUNCH("tq_dense_qk_scores launch");
+  return TQ_OK;
+}
+
+extern "C" int tq_softmax_rows(const float* scores, const float* mask, int64_t mask_row_stride, float* weights,
+                               int64_t n_rows, int64_t seq_len, float scale, tq_stream_t stream_) {
+  if (n_rows < 0 || seq_len < 0) return tq::fail(TQ_ERR_ARG, "tq_softmax_rows: negative size");
+  if (n_rows == 0 || seq_len == 0) return TQ_OK;
+  if (!scores || !weights) return tq::fail(TQ_ERR_NULL, "tq_softmax_rows: null pointer");
+  if (n_rows > 0x7FFFFFFF) return tq::fail(TQ_ERR_ARG, "tq_softmax_rows: too many rows");
+  softmax_rows_kernel<<<(int)n_rows, kThreads, 0, (hipStream_t)stream_>>>(scores, mask, mask_row_stride, weights,
+                                                                         seq_len, scale);
+  TQ_CHECK_LAUNCH("tq_softmax_rows launch");
+  return TQ_OK;
+}
+
+extern "C" int tq_sparse_v_matvec(const float* weights, const uint32_t* v_packed, const float* v_norms,
+                                  const float* centroids, const float* signs, float* out, void* workspace,
+                                  size_t workspace_bytes, int n_kv_heads, int n_rep, int64_t seq_len,
+                                  int64_t packed_head_stride, int64_t norms_head_stride, int dim, int bits,
+                                  float threshold, tq_stream_t stream_) {
+  if (!tq::is_pow2(dim)) return tq::fail(TQ_ERR_DIM, "dim must be a power of 2, got %d", dim);
+  if (dim > 256) return tq::fail(TQ_ERR_DIM, "dim > 256 not supported by threadgroup layout, got %d", dim);
+  tq_decode_shape sh{};
+  sh.n_seq = 1; sh.n_kv_heads = n_kv_heads; sh.n_rep = n_rep; sh.dim = dim; sh.bits = bits;
+  sh.block_size = 16; sh.seq_len = seq_len;
+  sh.v_head_stride = packed_head_stride; sh.vn_head_stride = norms_head_stride;
+  sh.out_dtype = TQ_F32;
+  if (int rc = check_shape(&sh, "tq_sparse_v_matvec", 256)) return rc;
+  if (!signs || !out || !centroids) return tq::fail(TQ_ERR_NULL, "tq_sparse_v_matvec: null pointer");
+  if (seq_len > 0 && (!weights || !v_packed || !v_norms))
+    return tq::fail(TQ_ERR_NULL, "tq_sparse_v_matvec: null pointer");
+  const float thr = threshold > 0.0f ? threshold : 0.0f;
+  return launch_decode<kWeights>(weights, TQ_F32, nullptr, nullptr, nullptr, v_packed, v_norms, nullptr,
+                                 centroids, signs, out, workspace, workspace_bytes, sh, thr,
+                                 (hipStream_t)stream_, "tq_sparse_v_matvec");
+}
+
+extern "C" int tq_flash_decode(const float* q_rot, const uint32_t* k_packed, const float* k_norms,
+                               const uint32_t* v_packed, const float* v_norms, const float* k_centroids,
+                               const float* v_centroids, const float* v_signs, void* out, void* workspace,
+                               size_t workspace_bytes, const tq_decode_shape* shape, tq_stream_t stream_) {
+  if (int rc = check_shape(shape, "tq_flash_decode", 128)) return rc;
+  if (!q_rot || !k_centroids || !v_centroids || !v_signs || !out)
+    return tq::fail(TQ_ERR_NULL, "tq_flash_decode: null pointer");
+  if (shape->seq_len > 0 && (!k_packed || !k_norms || !v_packed || !v_norms))
+    return tq::fail(TQ_ERR_NULL, "tq_flash_decode: null pointer");
+  return launch_decode<kPackedK>(q_rot, TQ_F32, k_packed, k_norms, nullptr, v_packed, v_norms, k_centroids,
+                                 v_centroids, v_signs, out, workspace, workspace_bytes, *shape, 0.0f,
+                                 (hipStream_t)stream_, "tq_flash_decode");
+}
+
+extern "C" int tq_vonly_decode_attn(const void* q, int q_dtype, const void* k_f16, const uint32_t* v_packed,
+                                    const float* v_norms, const float* v_centroids, const float* v_signs,
+                                    void* out, void* workspace, size_t workspace_bytes,
+                                    const tq_decode_shape* shape, tq_stream_t stream_) {
+  if (int rc = check_shape(shape, "tq_vonly_decode_attn", 256)) return rc;
+  if (tq::check_dtype(q_dtype)) return tq::fail(TQ_ERR_DTYPE, "tq_vonly_decode_attn: unknown q_dtype %d", q_dtype);
+  if (!q || !v_centroids || !v_signs || !out) return tq::fail(TQ_ERR_NULL, "tq_vonly_decode_attn: null pointer");
+  if (shape->seq_len > 0 && (!k_f16 || !v_packed || !v_norms))
+    return tq::fail(TQ_ERR_NULL, "tq_vonly_decode_attn: null pointer");
+  if (!tq::aligned(k_f16, 16)) return tq::fail(TQ_ERR_ALIGN, "tq_vonly_decode_attn: k must be 16-byte aligned");
+  return launch_decode<kDenseK>(q, q_dtype, nullptr, nullptr, k_f16, v_packed, v_norms, nullptr, v_centroids,
+                                v_signs, out, workspace, workspace_bytes, *shape, 0.0f, (hipStream_t)stream_,
+                                "tq_vonly_decode_attn");
+}

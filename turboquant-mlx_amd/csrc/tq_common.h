@@ -1,0 +1,184 @@
+// Shared host/device helpers for libtqhip (gfx950, wave64).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <hip/hip_bf16.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/tqhip.h"
+
+#define TQ_WAVE 64
+#define TQ_VERSION 100
+
+// ------------------------------------------------------------------ host side
+
+namespace tq {
+
+// thread-local message of the last failure
+inline char* err_buf() {
+  static thread_local char buf[512] = {0};
+  return buf;
+}
+
+inline int fail(int status, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(err_buf(), 512, fmt, ap);
+  va_end(ap);
+  return status;
+}
+
+inline int hip_fail(hipError_t e, const char* what) {
+  return fail(TQ_ERR_HIP - (int)e, "%s: %s", what, hipGetErrorString(e));
+}
+
+inline int vals_per_word(int bits) {
+  switch (bits) { case 1: return 32; case 2: return 16; case 3: return 10; case 4: return 8; }
+  return 0;
+}
+
+inline int packed_dim(int dim, int bits) {
+  int vpw = vals_per_word(bits);
+  return (dim + vpw - 1) / vpw;
+}
+
+inline bool is_pow2(int d) { return d > 0 && (d & (d - 1)) == 0; }
+
+inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+inline int check_dtype(int dt) { return (dt == TQ_F32 || dt == TQ_F16 || dt == TQ_BF16) ? 0 : 1; }
+
+inline size_t dtype_size(int dt) { return dt == TQ_F32 ? 4 : 2; }
+
+inline int check_dim_bits(int dim, int bits) {
+  if (bits < 1 || bits > 4) return fail(TQ_ERR_BITS, "Unsupported bit width: %d. Use 1-4.", bits);
+  if (!is_pow2(dim)) return fail(TQ_ERR_DIM, "dim must be a power of 2, got %d", dim);
+  if (dim < 32 || dim > 256) return fail(TQ_ERR_DIM, "dim %d outside the supported range 32..256", dim);
+  return 0;
+}
+
+#define TQ_DISPATCH_DIM(dim, ...)                                  \
+  switch (dim) {                                                   \
+    case 32: { constexpr int D_ = 32; __VA_ARGS__; } break;        \
+    case 64: { constexpr int D_ = 64; __VA_ARGS__; } break;        \
+    case 128: { constexpr int D_ = 128; __VA_ARGS__; } break;      \
+    case 256: { constexpr int D_ = 256; __VA_ARGS__; } break;      \
+  }
+#define TQ_DISPATCH_BITS(bits, ...)                                \
+  switch (bits) {                                                  \
+    case 1: { constexpr int B_ = 1; __VA_ARGS__; } break;          \
+    case 2: { constexpr int B_ = 2; __VA_ARGS__; } break;          \
+    case 3: { constexpr int B_ = 3; __VA_ARGS__; } break;          \
+    case 4: { constexpr int B_ = 4; __VA_ARGS__; } break;          \
+  }
+
+#define TQ_CHECK_LAUNCH(what)                                   \
+  do {                                                          \
+    hipError_t e__ = hipGetLastError();                         \
+    if (e__ != hipSuccess) return tq::hip_fail(e__, what);      \
+  } while (0)
+
+}  // namespace tq
+
+// ------------------------------------------------------------------ device side
+
+namespace tqd {
+
+// centroid table passed to kernels by value
+struct Codebook { float c[16]; };
+
+template <int BITS> struct Pk {
+  static constexpr int VPW = BITS == 1 ? 32 : BITS == 2 ? 16 : BITS == 3 ? 10 : 8;
+  static constexpr uint32_t MASK = (1u << BITS) - 1u;
+  static constexpr int pdim(int d) { return (d + VPW - 1) / VPW; }
+};
+
+// A 128-float (or shorter) vector is spread over one wavefront: lane l, slot i holds
+// element l + 64*i.  EPL = slots per lane.
+template <int D> struct Lay { static constexpr int EPL = (D >= 64) ? D / 64 : 1; };
+
+__device__ __forceinline__ float shfl_xor_f(float v, int m) { return __shfl_xor(v, m, TQ_WAVE); }
+
+// Raw (un-normalised) Walsh-Hadamard butterfly, stages h = 1, 2, ..., D/2; the element whose
+// index has bit h clear receives a+b, its partner a-b.  Stages below 64 exchange lanes, stages
+// from 64 up are register-to-register.  Float adds only, so the result is the same expression
+// tree as a serial loop over h.
+template <int D>
+__device__ __forceinline__ void raw_butterfly(float (&v)[Lay<D>::EPL], int lane) {
+  constexpr int EPL = Lay<D>::EPL;
+#pragma unroll
+  for (int h = 1; h < 64 && h < D; h <<= 1) {
+    const bool upper = (lane & h) != 0;
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) {
+      float p = shfl_xor_f(v[i], h);
+      v[i] = upper ? (p - v[i]) : (v[i] + p);
+    }
+  }
+#pragma unroll
+  for (int h = 64; h < D; h <<= 1) {
+    const int hs = h / 64;
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) {
+      if ((i & hs) == 0) {
+        float a = v[i], b = v[i + hs];
+        v[i] = a + b;
+        v[i + hs] = a - b;
+      }
+    }
+  }
+}
+
+// Sum over the D elements in stride-halving tree order: ns[e] += ns[e + stride] for
+// stride = D/2, D/4, ..., 1.  Every lane ends with the value of ns[0].
+template <int D>
+__device__ __forceinline__ float tree_sum(float (&s)[Lay<D>::EPL]) {
+  constexpr int EPL = Lay<D>::EPL;
+#pragma unroll
+  for (int hs = EPL / 2; hs >= 1; hs >>= 1) {
+#pragma unroll
+    for (int i = 0; i < hs; ++i) s[i] = s[i] + s[i + hs];
+  }
+  float v = s[0];
+#pragma unroll
+  for (int m = (D >= 64 ? 32 : D / 2); m >= 1; m >>= 1) v = v + shfl_xor_f(v, m);
+  return v;
+}
+
+template <typename T> __device__ __forceinline__ float load_as_float(const T* p);
+template <> __device__ __forceinline__ float load_as_float<float>(const float* p) { return *p; }
+template <> __device__ __forceinline__ float load_as_float<__half>(const __half* p) { return __half2float(*p); }
+template <> __device__ __forceinline__ float load_as_float<__hip_bfloat16>(const __hip_bfloat16* p) {
+  return __bfloat162float(*p);
+}
+
+template <typename T> __device__ __forceinline__ void store_from_float(T* p, float v);
+template <> __device__ __forceinline__ void store_from_float<float>(float* p, float v) { *p = v; }
+// The value is rounded to float32 first and to the 16-bit type second, as a cast of a float
+// variable does.  The empty asm keeps the compiler from folding the producing multiply into a
+// mixed-precision multiply-convert, which would round only once.
+template <> __device__ __forceinline__ void store_from_float<__half>(__half* p, float v) {
+  asm volatile("" : "+v"(v));
+  *p = __float2half_rn(v);
+}
+template <> __device__ __forceinline__ void store_from_float<__hip_bfloat16>(__hip_bfloat16* p, float v) {
+  asm volatile("" : "+v"(v));
+  *p = __float2bfloat16(v);
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, shfl_xor_f(v, m));
+  return v;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) v += shfl_xor_f(v, m);
+  return v;
+}
+
+}  // namespace tqd

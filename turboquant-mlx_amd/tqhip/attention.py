@@ -1,0 +1,119 @@
+"""Decode-step attention over PolarQuant caches.
+
+`turboquant_attention` is the reference composition (fused_attention.py:20-125): pre-rotate the
+query, score it against the packed keys, scale, mask, softmax, then the butterfly-pulled-out
+weighted sum over packed values.  `vonly_decode_attention` is the same for a V-only cache, whose
+keys are fp16.  Both can run as ONE fused launch per step when no positive sparse-V threshold is
+asked for (the threshold is defined on final softmax weights, so it needs the unfused passes).
+"""
+from __future__ import annotations
+
+import torch
+
+from . import ops
+
+
+def _mask_rows(mask, b: int, n_q: int, total: int):
+    """The mask rank cases of fused_attention.py:81-92, returning a (rows, total) float tensor."""
+    m = mask
+    if m.dim() == 4:
+        m = m[min(b, m.shape[0] - 1)]
+        m = m[:, 0, :]
+        if m.shape[0] == 1:
+            m = m.expand(n_q, total)
+    elif m.dim() == 3:
+        m = m[min(b, m.shape[0] - 1), 0, :].reshape(1, -1).expand(n_q, total)
+    elif m.dim() == 1:
+        m = m.reshape(1, -1)
+    if m.dtype == torch.bool:
+        m = torch.zeros(m.shape, dtype=torch.float32, device=m.device).masked_fill_(~m, float("-inf"))
+    return m
+
+
+def turboquant_attention(queries: torch.Tensor, cache, attn_scale: float, mask=None, v_buffer=None,
+                         sparse_v_threshold: float | None = None, fused: bool = False) -> torch.Tensor:
+    """fused_attention.py:20-125.  queries (B, n_heads, 1, dim) against a TurboQuantKVCache holding
+    packed K and V; returns (B, n_heads, 1, dim) in queries.dtype.
+
+    fused=True runs the whole step as one launch (pre-rotation aside) when neither a v_buffer nor a
+    positive sparse-V threshold is requested; the result is the same up to float32 summation order.
+    """
+    B, n_q, S_q, dim = queries.shape
+    if S_q != 1:
+        raise ValueError(f"turboquant_attention is a decode step: expected one query token, got {S_q}")
+    total = cache.offset
+    n_kv = cache.k_packed.shape[1]
+    n_rep = n_q // n_kv
+    bits = cache.quant_bits
+    kq, vq = cache._k_q, cache._v_q
+    thr = sparse_v_threshold if (sparse_v_threshold is not None and sparse_v_threshold >= 0.0) else 0.0
+
+    if fused and v_buffer is None and thr == 0.0:
+        q_rot = ops.prerotate_query(queries.reshape(B * n_q, dim), kq.signs).reshape(B, n_q, dim)
+        m = None
+        if mask is not None:
+            m = torch.stack([_mask_rows(mask, b, n_q, total).expand(n_q, total) for b in range(B)])
+        out = ops.flash_decode(q_rot, cache.k_packed, cache.k_norms, cache.v_packed, cache.v_norms,
+                               kq.centroids, vq.centroids, vq.signs, dim, bits, attn_scale, n_rep=n_rep,
+                               seq_len=total, mask=m)
+        return out[:, :, None, :].to(queries.dtype)
+
+    outputs = []
+    for b in range(B):
+        kp = cache.k_packed[b, :, :total, :]
+        kn = cache.k_norms[b, :, :total]
+        q_rot = ops.prerotate_query(queries[b, :, 0, :], kq.signs)
+        scores = ops.prerot_fused_qk_scores(q_rot, kp, kn, kq.centroids, dim, bits, n_rep=n_rep)
+        m = _mask_rows(mask, b, n_q, total) if mask is not None else None
+        weights = ops.softmax_rows(scores, attn_scale, m)
+        if v_buffer is not None:
+            v_deq = v_buffer[b]
+            if n_rep > 1:
+                v_deq = v_deq.repeat_interleave(n_rep, dim=0)
+            out = weights[:, None, :].to(queries.dtype) @ v_deq.to(queries.dtype)
+        else:
+            vp = cache.v_packed[b, :, :total, :]
+            vn = cache.v_norms[b, :, :total]
+            mv = ops.sparse_v_matvec(weights, vp, vn, vq.centroids, vq.signs, cache._v_dim, bits,
+                                     threshold=thr, n_rep=n_rep)
+            out = mv[:, None, :].to(queries.dtype)
+        outputs.append(out)
+    return torch.stack(outputs, dim=0)
+
+
+def vonly_decode_attention(queries: torch.Tensor, cache, attn_scale: float, mask=None,
+                           sparse_v_threshold: float | None = None) -> torch.Tensor:
+    """Decode attention straight off a VOnlyTurboQuantCache: softmax(q K^T * scale + mask) over the
+    fp16 keys, then the weighted sum over the packed values without ever dequantising them
+    (the dense-K-scores -> softmax -> sparse_v_matvec shape of hybrid_attention.py:52-88).
+
+    queries (B, n_heads, 1, dim) -> (B, n_heads, 1, dim) in queries.dtype.  With no positive
+    threshold the step is one fused launch; otherwise scores, softmax and sparse-V run separately
+    so that the threshold applies to the final weights (sparse_v.py:60-61).
+    """
+    B, n_q, S_q, dim = queries.shape
+    if S_q != 1:
+        raise ValueError(f"vonly_decode_attention is a decode step: expected one query token, got {S_q}")
+    kc, tq = cache._k_cache, cache._v_tq
+    total = kc.offset
+    n_kv = kc.keys.shape[1]
+    n_rep = n_q // n_kv
+    vq = tq._v_q
+    bits = tq.quant_bits
+    thr = sparse_v_threshold if (sparse_v_threshold is not None and sparse_v_threshold >= 0.0) else 0.0
+    if thr == 0.0:
+        m = None
+        if mask is not None:
+            m = torch.stack([_mask_rows(mask, b, n_q, total).expand(n_q, total) for b in range(B)])
+        out = ops.vonly_decode(queries[:, :, 0, :], kc.keys, tq.v_packed, tq.v_norms, vq.centroids, vq.signs,
+                               dim, bits, attn_scale, n_rep=n_rep, seq_len=total, mask=m)
+        return out[:, :, None, :].to(queries.dtype)
+    outputs = []
+    for b in range(B):
+        scores = ops.dense_qk_scores(queries[b, :, 0, :], kc.keys[b, :, :total, :], 1.0, n_rep=n_rep)
+        m = _mask_rows(mask, b, n_q, total) if mask is not None else None
+        weights = ops.softmax_rows(scores, attn_scale, m)
+        mv = ops.sparse_v_matvec(weights, tq.v_packed[b, :, :total, :], tq.v_norms[b, :, :total],
+                                 vq.centroids, vq.signs, tq._v_dim, bits, threshold=thr, n_rep=n_rep)
+        outputs.append(mv[:, None, :].to(queries.dtype))
+    return torch.stack(outputs, dim=0)

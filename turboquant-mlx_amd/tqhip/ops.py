@@ -1,0 +1,530 @@
+"""Kernel wrappers: the reference's operator API on torch tensors.
+
+Each function has the name, argument order and error behaviour of the reference
+wrapper it stands in for (cited per function; paths relative to the reference's
+turboquant_mlx/ package), takes `torch.Tensor` where the reference takes
+`mx.array`, and launches the HIP kernel of libtqhip.so on torch's current stream.
+Tensors must live on a GPU; there is no CPU implementation behind these calls.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+
+import torch
+
+from . import _lib
+from ._lib import DecodeShape, TQ_BF16, TQ_F16, TQ_F32
+
+VALS_PER_WORD = {1: 32, 2: 16, 3: 10, 4: 8}       # packing.py:16
+BIT_MASK = {1: 0x1, 2: 0x3, 3: 0x7, 4: 0xF}       # packing.py:17
+
+_DTYPES = {torch.float32: TQ_F32, torch.float16: TQ_F16, torch.bfloat16: TQ_BF16}
+_TORCH_OF = {TQ_F32: torch.float32, TQ_F16: torch.float16, TQ_BF16: torch.bfloat16}
+
+
+def packed_dim(dim: int, bits: int) -> int:
+    """packing.py:20-23."""
+    vpw = VALS_PER_WORD[bits]
+    return (dim + vpw - 1) // vpw
+
+
+# ------------------------------------------------------------------ helpers
+
+def _need_gpu(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError(
+                "tqhip kernels run on the GPU only: got a tensor on "
+                f"{t.device}; there is no CPU fallback")
+
+
+def _stream(t: torch.Tensor):
+    return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _ptr(t):
+    return C.c_void_p(t.data_ptr()) if t is not None else C.c_void_p(0)
+
+
+def _dt(t: torch.Tensor) -> int:
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise ValueError(f"unsupported dtype {t.dtype}; use float32, float16 or bfloat16") from None
+
+
+def _host_table(x):
+    """Small table (boundaries / centroids) as a ctypes float array.  Accepts tensors, lists."""
+    if isinstance(x, torch.Tensor):
+        key = (x.data_ptr(), x._version, x.numel(), str(x.device))
+        hit = _host_table.cache.get(key)
+        if hit is None:
+            hit = _lib.host_floats(x.detach().float().cpu().tolist())
+            if len(_host_table.cache) > 256:
+                _host_table.cache.clear()
+            _host_table.cache[key] = hit
+        return hit
+    return _lib.host_floats(x)
+
+
+_host_table.cache = {}
+
+
+def _as_f32_dev(x, like: torch.Tensor) -> torch.Tensor:
+    if not isinstance(x, torch.Tensor):
+        x = torch.tensor(list(x), dtype=torch.float32)
+    return x.to(device=like.device, dtype=torch.float32).contiguous()
+
+
+_workspaces = {}
+
+
+def _workspace(device, stream_id: int, nbytes: int) -> torch.Tensor:
+    key = (device, stream_id)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1 << 16), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def _u32(t: torch.Tensor) -> torch.Tensor:
+    """View / convert an integer tensor of packed words as uint32."""
+    if t.dtype == torch.uint32:
+        return t
+    if t.dtype == torch.int32:
+        return t.view(torch.uint32)
+    return (t.to(torch.int64) & 0xFFFFFFFF).to(torch.int32).view(torch.uint32)
+
+
+def _rows_view(t: torch.Tensor, inner: int):
+    """(head_stride_in_rows, ok) for a [H, T, inner] view whose rows are contiguous."""
+    if t.dim() != 3 or t.stride(2) != 1 or t.stride(1) != inner or t.stride(0) % inner:
+        return None
+    return t.stride(0) // inner
+
+
+def _head_layout_3d(t: torch.Tensor, inner: int) -> tuple[torch.Tensor, int]:
+    hs = _rows_view(t, inner)
+    if hs is None:
+        t = t.contiguous()
+        hs = t.stride(0) // inner
+    return t, hs
+
+
+def _head_layout_2d(t: torch.Tensor) -> tuple[torch.Tensor, int]:
+    if t.dim() != 2 or t.stride(1) != 1:
+        t = t.contiguous()
+    return t, t.stride(0)
+
+
+# ------------------------------------------------------------------ packing (integer plumbing)
+
+def pack_indices(indices: torch.Tensor, bits: int) -> torch.Tensor:
+    """packing.py:26-56.  (..., dim) integer indices -> (..., packed_dim) uint32."""
+    vpw = VALS_PER_WORD[bits]
+    shape = indices.shape
+    dim = shape[-1]
+    pd = packed_dim(dim, bits)
+    flat = indices.reshape(-1, dim).to(torch.int64)
+    if dim % vpw:
+        flat = torch.nn.functional.pad(flat, (0, pd * vpw - dim))
+    flat = flat.reshape(-1, pd, vpw)
+    shifts = torch.arange(vpw, device=flat.device, dtype=torch.int64) * bits
+    words = (flat << shifts).sum(dim=-1)            # disjoint bit fields: sum == OR
+    return words.to(torch.int32).view(torch.uint32).reshape(*shape[:-1], pd)
+
+
+def unpack_indices(packed: torch.Tensor, bits: int, dim: int) -> torch.Tensor:
+    """packing.py:59-87.  (..., packed_dim) uint32 -> (..., dim) uint8."""
+    vpw = VALS_PER_WORD[bits]
+    shape = packed.shape
+    w = _u32(packed).contiguous().view(torch.int32).to(torch.int64) & 0xFFFFFFFF
+    shifts = torch.arange(vpw, device=w.device, dtype=torch.int64) * bits
+    vals = (w.unsqueeze(-1) >> shifts) & BIT_MASK[bits]
+    vals = vals.reshape(*shape[:-1], shape[-1] * vpw)[..., :dim]
+    return vals.to(torch.uint8)
+
+
+# ------------------------------------------------------------------ encode / dequant
+
+def encode_into(x: torch.Tensor, signs: torch.Tensor, boundaries, packed: torch.Tensor,
+                norms: torch.Tensor, *, n_groups: int, rows_per_group: int,
+                packed_group_stride: int, norms_group_stride: int, dim: int, bits: int,
+                variant: str = "mlx", packed_row_offset: int = 0, norms_row_offset: int = 0) -> None:
+    """Encode rows of `x` straight into caller-owned packed / norm storage (tq_encode)."""
+    _need_gpu(x, signs, packed, norms)
+    x = x.contiguous()
+    pd = packed_dim(dim, bits)
+    var = {"mlx": _lib.TQ_ENCODE_MLX, "metal": _lib.TQ_ENCODE_METAL}[variant]
+    lib = _lib.load()
+    _lib.check(lib.tq_encode(
+        _ptr(x), _dt(x), _ptr(signs), _host_table(boundaries),
+        C.c_void_p(packed.data_ptr() + packed_row_offset * pd * 4),
+        C.c_void_p(norms.data_ptr() + norms_row_offset * 4),
+        n_groups, rows_per_group, packed_group_stride, norms_group_stride,
+        dim, bits, var, _stream(x)))
+
+
+def fused_quantize(vectors: torch.Tensor, signs: torch.Tensor, boundaries, dim: int, bits: int,
+                   variant: str = "mlx"):
+    """metal.py:147-196.  (n_vecs, dim) fp16/bf16/fp32 -> packed (n_vecs, pdim) uint32, norms (n_vecs,) f32.
+
+    variant="mlx" reproduces the bits of PolarQuantizer.quantize + pack_indices
+    (quantizer.py:85-106); variant="metal" those of the Metal encoder (metal.py:66-77).
+    """
+    if bits not in VALS_PER_WORD:
+        raise KeyError(bits)                                    # packing.py:22 via metal.py:177
+    _need_gpu(vectors)
+    n_vecs = vectors.shape[0]
+    vectors = vectors.reshape(n_vecs, dim)
+    signs = _as_f32_dev(signs, vectors)
+    pd = packed_dim(dim, bits)
+    packed = torch.empty((n_vecs, pd), dtype=torch.uint32, device=vectors.device)
+    norms = torch.empty((n_vecs,), dtype=torch.float32, device=vectors.device)
+    encode_into(vectors, signs, boundaries, packed, norms, n_groups=1, rows_per_group=n_vecs,
+                packed_group_stride=0, norms_group_stride=0, dim=dim, bits=bits, variant=variant)
+    return packed, norms
+
+
+def dequant_into(packed: torch.Tensor, norms: torch.Tensor, centroids, signs: torch.Tensor,
+                 out: torch.Tensor, *, n_groups: int, rows_per_group: int, packed_group_stride: int,
+                 norms_group_stride: int, out_group_stride: int, dim: int, bits: int,
+                 packed_row_offset: int = 0, norms_row_offset: int = 0, out_row_offset: int = 0) -> None:
+    """Dequantise rows of caller-owned packed storage into caller-owned `out` (tq_dequant)."""
+    _need_gpu(packed, norms, signs, out)
+    pd = packed_dim(dim, bits)
+    lib = _lib.load()
+    _lib.check(lib.tq_dequant(
+        C.c_void_p(packed.data_ptr() + packed_row_offset * pd * 4),
+        C.c_void_p(norms.data_ptr() + norms_row_offset * 4),
+        _host_table(centroids), _ptr(signs),
+        C.c_void_p(out.data_ptr() + out_row_offset * dim * out.element_size()), _dt(out),
+        n_groups, rows_per_group, packed_group_stride, norms_group_stride, out_group_stride,
+        dim, bits, _stream(out)))
+
+
+def _dequant(packed, norms, centroids, signs, dim, bits, dtype):
+    _need_gpu(packed, norms)
+    seq_len = norms.shape[0]
+    packed = _u32(packed).reshape(seq_len, -1).contiguous()
+    norms = norms.to(torch.float32).contiguous()
+    signs = _as_f32_dev(signs, packed)
+    out = torch.empty((seq_len, dim), dtype=dtype, device=packed.device)
+    dequant_into(packed, norms, centroids, signs, out, n_groups=1, rows_per_group=seq_len,
+                 packed_group_stride=0, norms_group_stride=0, out_group_stride=0, dim=dim, bits=bits)
+    return out
+
+
+def packed_dequantize(packed, norms, centroids, signs, dim: int, bits: int) -> torch.Tensor:
+    """kernels.py:123-155.  (seq, pdim) uint32 + (seq,) -> (seq, dim) float32."""
+    return _dequant(packed, norms, centroids, signs, dim, bits, torch.float32)
+
+
+prerot_packed_dequantize = packed_dequantize      # metal_kernels_v4.py:27
+
+
+def dequant_fp16(packed, norms, centroids, signs, dim: int, bits: int) -> torch.Tensor:
+    """metal.py:199-232.  Same arithmetic, half-precision output."""
+    return _dequant(packed, norms, centroids, signs, dim, bits, torch.float16)
+
+
+# ------------------------------------------------------------------ scores
+
+def prerotate_query(q: torch.Tensor, signs) -> torch.Tensor:
+    """metal_kernels_v4.py:119-150.  (n_heads, dim) -> raw butterfly of signs*q, float32."""
+    if q.dim() != 2:
+        raise ValueError(f"prerotate_query expects (n_heads, dim), got {tuple(q.shape)}")
+    _need_gpu(q)
+    n_heads, dim = q.shape
+    if q.dtype not in _DTYPES:
+        q = q.float()
+    q = q.contiguous()
+    signs = _as_f32_dev(signs, q)
+    out = torch.empty((n_heads, dim), dtype=torch.float32, device=q.device)
+    _lib.check(_lib.load().tq_prerotate_query(_ptr(q), _dt(q), _ptr(signs), _ptr(out), n_heads, dim, _stream(q)))
+    return out
+
+
+def _check_gqa(n_q: int, n_kv: int, n_rep: int):
+    if n_q != n_kv * n_rep:
+        raise ValueError(f"n_q_heads ({n_q}) must equal n_kv_heads ({n_kv}) * n_rep ({n_rep})")
+
+
+def prerot_fused_qk_scores(q_rot: torch.Tensor, k_packed: torch.Tensor, k_norms: torch.Tensor,
+                           centroids, dim: int, bits: int, n_rep: int = 1) -> torch.Tensor:
+    """metal_kernels_v4.py:153-221.  Scores of pre-rotated queries against packed K, GQA-aware.
+
+    q_rot (n_q, dim); k_packed (n_kv, seq, pdim); k_norms (n_kv, seq) -> (n_q, seq) float32.
+    """
+    _need_gpu(q_rot, k_packed, k_norms)
+    n_q = q_rot.shape[0]
+    n_kv, seq_len = k_norms.shape
+    _check_gqa(n_q, n_kv, n_rep)
+    pd = packed_dim(dim, bits)
+    q_rot = q_rot.to(torch.float32).contiguous()
+    k_packed, phs = _head_layout_3d(_u32(k_packed), pd)
+    k_norms, nhs = _head_layout_2d(k_norms.to(torch.float32))
+    out = torch.empty((n_q, seq_len), dtype=torch.float32, device=q_rot.device)
+    _lib.check(_lib.load().tq_prerot_qk_scores(
+        _ptr(q_rot), _ptr(k_packed), _ptr(k_norms), _host_table(centroids), _ptr(out),
+        n_kv, n_rep, seq_len, phs, nhs, dim, bits, _stream(q_rot)))
+    return out
+
+
+def packed_fused_qk_scores(query: torch.Tensor, k_packed: torch.Tensor, k_norms: torch.Tensor,
+                           centroids, signs, dim: int, bits: int) -> torch.Tensor:
+    """kernels.py:158-196.  One butterfly per K row, MHA only: (H, D), (H, S, pdim), (H, S) -> (H, S)."""
+    _need_gpu(query, k_packed, k_norms)
+    n_heads, seq_len = k_norms.shape
+    pd = packed_dim(dim, bits)
+    query = query.to(torch.float32).contiguous()
+    k_packed, phs = _head_layout_3d(_u32(k_packed), pd)
+    k_norms, nhs = _head_layout_2d(k_norms.to(torch.float32))
+    signs = _as_f32_dev(signs, query)
+    out = torch.empty((n_heads, seq_len), dtype=torch.float32, device=query.device)
+    _lib.check(_lib.load().tq_packed_qk_scores(
+        _ptr(query), _ptr(k_packed), _ptr(k_norms), _host_table(centroids), _ptr(signs), _ptr(out),
+        n_heads, seq_len, phs, nhs, dim, bits, _stream(query)))
+    return out
+
+
+def dense_qk_scores(q: torch.Tensor, k: torch.Tensor, scale: float, n_rep: int = 1) -> torch.Tensor:
+    """<q[h], K[h // n_rep, p]> * scale for fp16 keys: (n_q, D), (n_kv, T, D) fp16 -> (n_q, T) f32."""
+    _need_gpu(q, k)
+    n_q, dim = q.shape
+    n_kv, seq_len, _ = k.shape
+    _check_gqa(n_q, n_kv, n_rep)
+    if k.dtype != torch.float16:
+        raise ValueError(f"dense keys must be float16, got {k.dtype}")
+    if q.dtype not in _DTYPES:
+        q = q.float()
+    q = q.contiguous()
+    k, khs = _head_layout_3d(k, dim)
+    out = torch.empty((n_q, seq_len), dtype=torch.float32, device=q.device)
+    _lib.check(_lib.load().tq_dense_qk_scores(_ptr(q), _dt(q), _ptr(k), _ptr(out), n_kv, n_rep, seq_len,
+                                               khs, dim, float(scale), _stream(q)))
+    return out
+
+
+def softmax_rows(scores: torch.Tensor, scale: float = 1.0, mask: torch.Tensor | None = None) -> torch.Tensor:
+    """softmax(scores * scale + mask) along the last axis of a (rows, T) float32 tensor
+    (fused_attention.py:78-94).  mask: (T,), (1, T) or (rows, T)."""
+    _need_gpu(scores, mask)
+    scores = scores.to(torch.float32).contiguous()
+    n_rows, seq_len = scores.shape
+    mrs = 0
+    if mask is not None:
+        mask = mask.to(torch.float32)
+        if mask.dim() == 1:
+            mask = mask.reshape(1, -1)
+        if mask.shape[-1] != seq_len or mask.shape[0] not in (1, n_rows):
+            raise ValueError(f"mask shape {tuple(mask.shape)} does not match scores {tuple(scores.shape)}")
+        mask = mask.contiguous()
+        mrs = seq_len if mask.shape[0] == n_rows and n_rows > 1 else 0
+    out = torch.empty_like(scores)
+    _lib.check(_lib.load().tq_softmax_rows(_ptr(scores), _ptr(mask), mrs, _ptr(out), n_rows, seq_len,
+                                            float(scale), _stream(scores)))
+    return out
+
+
+# ------------------------------------------------------------------ sparse V
+
+def sparse_v_matvec(weights: torch.Tensor, v_packed: torch.Tensor, v_norms: torch.Tensor, centroids,
+                    signs, dim: int, bits: int, threshold: float = 1e-5, n_rep: int = 1) -> torch.Tensor:
+    """sparse_v.py:94-186.  Weighted sum of dequantised V rows with the butterfly pulled out of
+    the position loop; positions with weight < threshold are skipped; threshold <= 0 is dense.
+
+    weights (n_q, seq); v_packed (n_kv, seq, pdim); v_norms (n_kv, seq) -> (n_q, dim) float32.
+    """
+    if dim & (dim - 1):
+        raise ValueError(f"dim must be a power of 2, got {dim}")
+    if dim > 256:
+        raise ValueError(f"dim > 256 not supported by threadgroup layout, got {dim}")
+    _need_gpu(weights, v_packed, v_norms)
+    n_q, seq_len = weights.shape
+    n_kv = v_packed.shape[0]
+    _check_gqa(n_q, n_kv, n_rep)
+    pd = packed_dim(dim, bits)
+    weights = weights.to(torch.float32).contiguous()
+    v_packed, phs = _head_layout_3d(_u32(v_packed), pd)
+    v_norms, nhs = _head_layout_2d(v_norms.to(torch.float32))
+    signs = _as_f32_dev(signs, weights)
+    out = torch.empty((n_q, dim), dtype=torch.float32, device=weights.device)
+    lib = _lib.load()
+    need = lib.tq_workspace_bytes(_lib.TQ_OP_SPARSE_V, 1, n_q, seq_len, dim)
+    stream = _stream(weights)
+    ws = _workspace(weights.device, stream.value or 0, need)
+    _lib.check(lib.tq_sparse_v_matvec(
+        _ptr(weights), _ptr(v_packed), _ptr(v_norms), _host_table(centroids), _ptr(signs), _ptr(out),
+        _ptr(ws), ws.numel(), n_kv, n_rep, seq_len, phs, nhs, dim, bits, float(max(threshold, 0.0)), stream))
+    return out
+
+
+def count_active_positions(weights: torch.Tensor, threshold: float = 1e-5) -> int:
+    """sparse_v.py:189-191 (diagnostics only)."""
+    return int((weights > threshold).sum().item())
+
+
+# ------------------------------------------------------------------ fused decode attention
+
+def _decode_shape(*, n_seq, n_kv, n_rep, dim, bits, block_size, seq_len, seq_offsets, k_strides, kn_strides,
+                  v_strides, vn_strides, mask, mask_strides, attn_scale, out_dtype) -> DecodeShape:
+    sh = DecodeShape()
+    sh.n_seq, sh.n_kv_heads, sh.n_rep, sh.dim, sh.bits, sh.block_size = n_seq, n_kv, n_rep, dim, bits, block_size
+    sh.seq_len = seq_len
+    sh.seq_offsets = seq_offsets.data_ptr() if seq_offsets is not None else None
+    sh.k_seq_stride, sh.k_head_stride = k_strides
+    sh.kn_seq_stride, sh.kn_head_stride = kn_strides
+    sh.v_seq_stride, sh.v_head_stride = v_strides
+    sh.vn_seq_stride, sh.vn_head_stride = vn_strides
+    sh.mask = mask.data_ptr() if mask is not None else None
+    sh.mask_seq_stride, sh.mask_head_stride = mask_strides
+    sh.attn_scale = float(attn_scale)
+    sh.out_dtype = _DTYPES[out_dtype]
+    return sh
+
+
+def _kv_layout(t: torch.Tensor, inner: int, ragged: bool):
+    """Strides in rows for KV addressing.  Accepts [H, T, inner] (one sequence or ragged batch) or
+    [B, H, T, inner] (cache layout); the last two axes must be row-contiguous."""
+    if t.dim() == 3:
+        t, hs = _head_layout_3d(t, inner)
+        return t, (0, hs)
+    if t.dim() != 4:
+        raise ValueError(f"expected a 3-D or 4-D KV tensor, got shape {tuple(t.shape)}")
+    if t.stride(3) != 1 or t.stride(2) != inner or t.stride(1) % inner or t.stride(0) % inner:
+        t = t.contiguous()
+    return t, (t.stride(0) // inner, t.stride(1) // inner)
+
+
+def _norm_layout(t: torch.Tensor):
+    if t.dim() == 2:
+        t, hs = _head_layout_2d(t)
+        return t, (0, hs)
+    if t.dim() != 3:
+        raise ValueError(f"expected a 2-D or 3-D norm tensor, got shape {tuple(t.shape)}")
+    if t.stride(2) != 1:
+        t = t.contiguous()
+    return t, (t.stride(0), t.stride(1))
+
+
+def _mask_layout(mask, n_seq: int, n_q: int, seq_len: int, device):
+    """Additive float mask broadcastable to (n_seq, n_q, seq_len) -> (tensor, (seq_stride, head_stride))."""
+    if mask is None:
+        return None, (0, 0)
+    m = mask.to(device=device, dtype=torch.float32)
+    while m.dim() < 3:
+        m = m.unsqueeze(0)
+    if m.shape[-1] != seq_len or m.shape[0] not in (1, n_seq) or m.shape[1] not in (1, n_q):
+        raise ValueError(f"mask shape {tuple(mask.shape)} not broadcastable to ({n_seq}, {n_q}, {seq_len})")
+    m = m.contiguous()
+    ss = m.shape[1] * seq_len if m.shape[0] == n_seq and n_seq > 1 else 0
+    hs = seq_len if m.shape[1] == n_q and n_q > 1 else 0
+    return m, (ss, hs)
+
+
+def flash_decode(q_rot: torch.Tensor, k_packed, k_norms, v_packed, v_norms, k_centroids, v_centroids,
+                 v_signs, dim: int, bits: int, attn_scale: float, *, n_rep: int = 1, block_size: int = 16,
+                 seq_len: int | None = None, seq_offsets: torch.Tensor | None = None,
+                 max_seq_len: int | None = None, mask=None, out_dtype=torch.float32) -> torch.Tensor:
+    """Batched form of flash_attention_turboquant (tq_flash_decode).
+
+    q_rot (n_seq, n_q, dim) float32.  K/V either cache layout [n_seq, n_kv, T_alloc, *] with the
+    uniform valid length `seq_len`, or ragged [n_kv, sum(L), *] with int32 `seq_offsets`
+    (n_seq + 1 entries on the GPU) and `max_seq_len`.  Returns (n_seq, n_q, dim) `out_dtype`.
+    """
+    _need_gpu(q_rot, k_packed, k_norms, v_packed, v_norms, seq_offsets)
+    if dim > 128 or dim & (dim - 1):
+        raise ValueError(f"dim must be a power of 2 and <= 128, got {dim}")
+    if block_size < 1 or block_size > 32:
+        raise ValueError(f"block_size must be in 1..32, got {block_size}")
+    n_seq, n_q, _ = q_rot.shape
+    ragged = seq_offsets is not None
+    n_kv = k_norms.shape[-2]
+    _check_gqa(n_q, n_kv, n_rep)
+    pd = packed_dim(dim, bits)
+    q_rot = q_rot.to(torch.float32).contiguous()
+    k_packed, ks = _kv_layout(_u32(k_packed), pd, ragged)
+    v_packed, vs = _kv_layout(_u32(v_packed), pd, ragged)
+    k_norms, kns = _norm_layout(k_norms.to(torch.float32))
+    v_norms, vns = _norm_layout(v_norms.to(torch.float32))
+    if ragged:
+        if max_seq_len is None:
+            raise ValueError("max_seq_len is required with seq_offsets")
+        if seq_offsets.dtype != torch.int32 or seq_offsets.numel() != n_seq + 1:
+            raise ValueError("seq_offsets must be int32 with n_seq + 1 entries")
+        T = int(max_seq_len)
+    else:
+        T = int(seq_len if seq_len is not None else k_norms.shape[-1])
+    v_signs = _as_f32_dev(v_signs, q_rot)
+    mask, ms = _mask_layout(mask, n_seq, n_q, T, q_rot.device)
+    out = torch.empty((n_seq, n_q, dim), dtype=out_dtype, device=q_rot.device)
+    sh = _decode_shape(n_seq=n_seq, n_kv=n_kv, n_rep=n_rep, dim=dim, bits=bits, block_size=block_size,
+                       seq_len=T, seq_offsets=seq_offsets, k_strides=ks, kn_strides=kns, v_strides=vs,
+                       vn_strides=vns, mask=mask, mask_strides=ms, attn_scale=attn_scale, out_dtype=out_dtype)
+    lib = _lib.load()
+    need = lib.tq_workspace_bytes(_lib.TQ_OP_FLASH_DECODE, n_seq, n_q, T, dim)
+    stream = _stream(q_rot)
+    ws = _workspace(q_rot.device, stream.value or 0, need)
+    _lib.check(lib.tq_flash_decode(
+        _ptr(q_rot), _ptr(k_packed), _ptr(k_norms), _ptr(v_packed), _ptr(v_norms),
+        _host_table(k_centroids), _host_table(v_centroids), _ptr(v_signs), _ptr(out),
+        _ptr(ws), ws.numel(), C.byref(sh), stream))
+    return out
+
+
+def flash_attention_turboquant(q_rot, k_packed, k_norms, v_packed, v_norms, k_centroids, v_centroids,
+                               v_signs, dim: int, bits: int, attn_scale: float, block_size: int = 16,
+                               n_rep: int = 1) -> torch.Tensor:
+    """flash_attention.py:168-274.  One sequence: q_rot (n_q, dim); K/V (n_kv, seq, pdim) + (n_kv, seq)
+    -> (n_q, dim) float32 = softmax(QK * scale) @ V over the packed cache."""
+    out = flash_decode(q_rot.unsqueeze(0), k_packed, k_norms, v_packed, v_norms, k_centroids, v_centroids,
+                       v_signs, dim, bits, attn_scale, n_rep=n_rep, block_size=block_size)
+    return out[0]
+
+
+def vonly_decode(q: torch.Tensor, k: torch.Tensor, v_packed, v_norms, v_centroids, v_signs, dim: int,
+                 bits: int, attn_scale: float, *, n_rep: int = 1, seq_len: int | None = None,
+                 seq_offsets: torch.Tensor | None = None, max_seq_len: int | None = None, mask=None,
+                 out_dtype=torch.float32) -> torch.Tensor:
+    """Dense-softmax decode attention over fp16 keys and packed values (tq_vonly_decode_attn).
+
+    q (n_seq, n_q, dim) fp16/bf16/fp32; k [n_seq, n_kv, T_alloc, dim] or ragged [n_kv, sum(L), dim] fp16;
+    V as in flash_decode.  Returns (n_seq, n_q, dim) `out_dtype`.
+    """
+    _need_gpu(q, k, v_packed, v_norms, seq_offsets)
+    if k.dtype != torch.float16:
+        raise ValueError(f"dense keys must be float16, got {k.dtype}")
+    n_seq, n_q, _ = q.shape
+    ragged = seq_offsets is not None
+    n_kv = v_norms.shape[-2]
+    _check_gqa(n_q, n_kv, n_rep)
+    pd = packed_dim(dim, bits)
+    if q.dtype not in _DTYPES:
+        q = q.float()
+    q = q.contiguous()
+    k, ks = _kv_layout(k, dim, ragged)
+    v_packed, vs = _kv_layout(_u32(v_packed), pd, ragged)
+    v_norms, vns = _norm_layout(v_norms.to(torch.float32))
+    if ragged:
+        if max_seq_len is None:
+            raise ValueError("max_seq_len is required with seq_offsets")
+        T = int(max_seq_len)
+    else:
+        T = int(seq_len if seq_len is not None else v_norms.shape[-1])
+    v_signs = _as_f32_dev(v_signs, q)
+    mask, ms = _mask_layout(mask, n_seq, n_q, T, q.device)
+    out = torch.empty((n_seq, n_q, dim), dtype=out_dtype, device=q.device)
+    sh = _decode_shape(n_seq=n_seq, n_kv=n_kv, n_rep=n_rep, dim=dim, bits=bits, block_size=16, seq_len=T,
+                       seq_offsets=seq_offsets, k_strides=ks, kn_strides=(0, 0), v_strides=vs, vn_strides=vns,
+                       mask=mask, mask_strides=ms, attn_scale=attn_scale, out_dtype=out_dtype)
+    lib = _lib.load()
+    need = lib.tq_workspace_bytes(_lib.TQ_OP_VONLY_DECODE, n_seq, n_q, T, dim)
+    stream = _stream(q)
+    ws = _workspace(q.device, stream.value or 0, need)
+    _lib.check(lib.tq_vonly_decode_attn(
+        _ptr(q), _dt(q), _ptr(k), _ptr(v_packed), _ptr(v_norms), _host_table(v_centroids), _ptr(v_signs),
+        _ptr(out), _ptr(ws), ws.numel(), C.byref(sh), stream))
+    return out

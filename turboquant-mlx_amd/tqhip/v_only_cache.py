@@ -1,0 +1,96 @@
+"""VOnlyTurboQuantCache (reference turboquant_mlx/v_only_cache.py:24-127): fp16 keys in a plain
+KVCache, values PolarQuant-compressed in a TurboQuantKVCache(v_only=True)."""
+from __future__ import annotations
+
+import torch
+
+from .cache import TurboQuantKVCache
+from .kvcache import KVCache
+
+
+class VOnlyTurboQuantCache:
+    """update_and_fetch stores K in fp16, compresses V and returns (K_fp16, V_dequantised).
+    With no_v_buffer=True the fp16 V buffer is not kept: V is re-dequantised from the packed
+    storage on every call (v_only_cache.py:41-49)."""
+
+    def __init__(self, bits: int = 3, seed: int = 42, no_v_buffer: bool = False):
+        self._k_cache = KVCache()
+        self._v_tq = TurboQuantKVCache(bits=bits, seed=seed, v_only=True)
+        self._v_bits = bits
+        self._no_v_buffer = no_v_buffer
+
+    def update_and_fetch(self, keys: torch.Tensor, values: torch.Tensor):
+        k_out, _ = self._k_cache.update_and_fetch(keys, values)
+        if self._no_v_buffer:                                    # v_only_cache.py:54-75
+            tq = self._v_tq
+            B, H, S, v_dim = values.shape
+            tq._dtype = keys.dtype
+            tq._ensure_quantizer(keys.shape[-1], v_dim, values.device)
+            tq._ensure_storage(B, H, S, values.device)
+            prev = tq.offset
+            tq._encode(values, tq._v_q, tq.v_packed, tq.v_norms, B, H, S, v_dim, prev)
+            tq.offset += S
+            v_out = tq._full_dequant(tq.v_packed, tq.v_norms, tq._v_q, v_dim, B, H, tq.offset, values.dtype)
+        else:
+            _, v_out = self._v_tq.update_and_fetch(keys, values)
+        return k_out, v_out
+
+    @property
+    def offset(self):
+        return self._k_cache.offset
+
+    @property
+    def state(self):
+        k_state = list(self._k_cache.state) if self._k_cache.state else []
+        v_state = list(self._v_tq.state) if self._v_tq.state else []
+        return k_state + v_state
+
+    @property
+    def meta_state(self):
+        return f"VOnlyTQ,{self._v_bits},{self._v_tq.seed},{self._v_tq.meta_state}"
+
+    @classmethod
+    def from_state(cls, state, meta_state):
+        parts = meta_state.split(",", 3)                        # v_only_cache.py:95-111
+        bits = int(parts[1])
+        seed = int(parts[2])
+        obj = cls(bits=bits, seed=seed)
+        if len(state) >= 2:
+            obj._k_cache.keys = state[0]
+            obj._k_cache.values = state[1]
+            obj._k_cache.offset = state[0].shape[2]
+        if len(state) > 2:
+            obj._v_tq.state = state[2:]
+            obj._v_tq.meta_state = parts[3]
+        return obj
+
+    @classmethod
+    def from_kvcache(cls, kv, bits: int = 3, seed: int = 42, **kwargs):
+        """Construct empty, then insert the valid prefix of an uncompressed cache (see
+        TurboQuantKVCache.from_kvcache)."""
+        obj = cls(bits=bits, seed=seed, **kwargs)
+        if kv.keys is not None and kv.offset > 0:
+            obj.update_and_fetch(kv.keys[..., :kv.offset, :], kv.values[..., :kv.offset, :])
+        return obj
+
+    def make_mask(self, *args, **kwargs):
+        return self._k_cache.make_mask(*args, **kwargs)
+
+    def empty(self):
+        return self._k_cache.offset == 0
+
+    def is_trimmable(self):
+        return True
+
+    def trim(self, n):
+        self._k_cache.trim(n)
+        return self._v_tq.trim(n)
+
+    def size(self):
+        return self._k_cache.offset
+
+    @property
+    def nbytes(self):
+        ks = self._k_cache
+        k_bytes = 0 if ks.keys is None else ks.keys[..., :ks.offset, :].numel() * ks.keys.element_size()
+        return k_bytes + self._v_tq.nbytes
