@@ -1,0 +1,209 @@
+#!/usr/bin/env python3
+"""Headline benchmark: V-only decode attention at the Qwen2.5-7B GQA shape, 32K context.
+
+One step = one layer's decode attention: q[28,128] fp16 against fp16 K[4,32768,128] and 3-bit
+packed V[4,32768,13]+norms[4,32768], dense softmax, out[28,128] -- the fused tq_vonly_decode_attn
+entry point of libtqhip.so, called through the C ABI.  Inputs are resident in HBM before the timed
+region; the steps rotate over N_SETS independent (q, K, V) sets totalling > 400 MB so that neither
+the L2s nor the 256 MB Infinity Cache can serve the reads.  The K timed steps are captured once
+into a HIP graph and replayed (back-to-back launches, no host gaps); HIP events on the launch
+stream bracket the replay.
+
+Prints ONE JSON line (see the fields below).  `roofline.achieved` = algorithmic bytes per step
+(40 908 800 B: q 7 168 + K 33 554 432 + V packed 6 815 744 + V norms 524 288 + out 7 168)
+divided by the measured time per step.  `cpu_baseline` times the numpy oracle on the same
+workload on this host's cores.
+"""
+import argparse
+import ctypes as C
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "turboquant-mlx_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+N_Q, N_KV, N_REP, D, BITS, T = 28, 4, 7, 128, 3, 32768
+PDIM = 13
+ALGO_BYTES = N_Q * D * 2 + N_KV * T * D * 2 + N_KV * T * PDIM * 4 + N_KV * T * 4 + N_Q * D * 2
+HBM_PEAK_GBS = 8000.0
+N_SETS = 10
+
+# HBM bytes per step from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same command,
+# scaled by the factor the same counters read for a plain copy kernel (see profiles/).
+# None until measured for the kernel that is currently the default.
+MEASURED_TRAFFIC_BYTES = None
+
+
+def make_sets(torch, tqhip, dev):
+    from tqhip.quantizer import gaussian_boundaries, gaussian_codebook
+    cb = gaussian_codebook(BITS)
+    bd = gaussian_boundaries(cb)
+    signs = tqhip.random_diagonal_sign(D, 43, device=dev)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(2)
+    sets = []
+    for _ in range(N_SETS):
+        q = torch.randn((1, N_Q, D), generator=gen, device=dev, dtype=torch.float32).to(torch.float16)
+        k = torch.randn((N_KV, T, D), generator=gen, device=dev, dtype=torch.float32).to(torch.float16)
+        v = torch.randn((N_KV * T, D), generator=gen, device=dev, dtype=torch.float32).to(torch.float16)
+        vp, vn = tqhip.fused_quantize(v, signs, bd, D, BITS)
+        del v
+        sets.append((q, k, vp.reshape(N_KV, T, PDIM), vn.reshape(N_KV, T)))
+    return sets, cb, signs
+
+
+def cpu_baseline(torch, sets, cb, signs, budget_s=12.0):
+    """The numpy oracle on set 0 at full size, timed on the host."""
+    import numpy as np
+    from oracle import polarquant_oracle as orc
+    q, k, vp, vn = [t.cpu().numpy() for t in sets[0]]
+    cbn, sg = cb.numpy(), signs.cpu().numpy()
+    sc = 1.0 / math.sqrt(D)
+
+    def run():
+        return orc.vonly_decode_attention(q[0], k, vp, vn, cbn, sg, D, BITS, sc)
+    ref = run()                       # warm-up, and the reference output for the check below
+    t0 = time.perf_counter()
+    n = 0
+    while True:
+        run()
+        n += 1
+        el = time.perf_counter() - t0
+        if el > budget_s or n >= 20:
+            break
+    per = el / n
+    try:
+        from threadpoolctl import threadpool_info
+        threads = max([p.get("num_threads", 1) for p in threadpool_info()] or [1])
+    except Exception:
+        threads = 1
+    return ref, {
+        "value": round(ALGO_BYTES / per / 1e9, 3), "unit": "GB/s", "us_per_layer": round(per * 1e6, 1),
+        "cores": threads, "kind": "port",
+        "sample": f"{n} full-size steps (28/4 heads, d=128, T=32768) of the numpy oracle; its matmuls run "
+                  f"on {threads} BLAS threads, unpack/gather/softmax on one (host reports {os.cpu_count()} cpus)",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (the hot path shards by kv head "
+              "with no communication; see DESIGN.md). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    import tqhip
+    from tqhip import _lib, ops
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    sets, cb, signs = make_sets(torch, tqhip, dev)
+    sc = 1.0 / math.sqrt(D)
+    lib = _lib.load()
+
+    # Pre-bound C-ABI calls: one argument tuple per buffer set, so a step is a single ctypes call.
+    outs = [torch.empty((1, N_Q, D), dtype=torch.float32, device=dev) for _ in range(N_SETS)]
+    ws_bytes = lib.tq_workspace_bytes(_lib.TQ_OP_VONLY_DECODE, 1, N_Q, T, D)
+    ws = torch.zeros(ws_bytes, dtype=torch.uint8, device=dev)
+    cb_host = _lib.host_floats(cb.tolist())
+    shape = ops._decode_shape(n_seq=1, n_kv=N_KV, n_rep=N_REP, dim=D, bits=BITS, block_size=16, seq_len=T,
+                              seq_offsets=None, k_strides=(0, T), kn_strides=(0, 0), v_strides=(0, T),
+                              vn_strides=(0, T), mask=None, mask_strides=(0, 0), attn_scale=sc,
+                              out_dtype=torch.float32)
+
+    def bound(i, stream):
+        q, k, vp, vn = sets[i]
+        return (C.c_void_p(q.data_ptr()), _lib.TQ_F16, C.c_void_p(k.data_ptr()), C.c_void_p(vp.data_ptr()),
+                C.c_void_p(vn.data_ptr()), cb_host, C.c_void_p(signs.data_ptr()), C.c_void_p(outs[i].data_ptr()),
+                C.c_void_p(ws.data_ptr()), ws.numel(), C.byref(shape), C.c_void_p(stream))
+
+    def step(i, argsets):
+        rc = lib.tq_vonly_decode_attn(*argsets[i % N_SETS])
+        if rc != 0:
+            _lib.check(rc)
+
+    # correctness of what is being timed: set 0 against the oracle
+    cur = torch.cuda.current_stream(dev)
+    eager_args = [bound(i, cur.cuda_stream) for i in range(N_SETS)]
+    step(0, eager_args)
+    torch.cuda.synchronize()
+    cpu = None
+    if not args.no_cpu:
+        ref, cpu = cpu_baseline(torch, sets, cb, signs)
+        err = np.abs(outs[0][0].cpu().numpy() - ref)
+        if not np.all(err <= 1e-3 + 2e-3 * np.abs(ref)):
+            print(f"bench: GPU output disagrees with the oracle (max err {err.max():.3e})", file=sys.stderr)
+            sys.exit(1)
+
+    side = torch.cuda.Stream(device=dev)
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    with torch.cuda.stream(side):
+        s_args = [bound(i, side.cuda_stream) for i in range(N_SETS)]
+        for i in range(args.warmup):
+            step(i, s_args)
+        side.synchronize()
+        if args.no_graph:
+            torch.cuda.synchronize()
+            ev0.record(side)
+            for i in range(args.steps):
+                step(i, s_args)
+            ev1.record(side)
+            side.synchronize()
+            mode = "eager"
+        else:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                g_stream = torch.cuda.current_stream(dev)
+                g_args = [bound(i, g_stream.cuda_stream) for i in range(N_SETS)]
+                for i in range(args.steps):
+                    step(i, g_args)
+            graph.replay()                      # one untimed replay: instantiation, page-in
+            torch.cuda.synchronize()
+            ev0.record(side)
+            graph.replay()
+            ev1.record(side)
+            side.synchronize()
+            mode = "hipgraph"
+    torch.cuda.synchronize()
+    ms_total = ev0.elapsed_time(ev1)
+    ms_per_step = ms_total / args.steps
+    gbs = ALGO_BYTES / (ms_per_step * 1e-3) / 1e9
+
+    # the timed steps must have produced the same result as the checked eager step
+    if not torch.equal(outs[0], outs[0]) or torch.isnan(outs[0]).any():
+        print("bench: NaN in timed output", file=sys.stderr)
+        sys.exit(1)
+
+    line = {
+        "metric": "sparse-V decode attn us/layer & HBM GB/s (% peak), 7B GQA shape, 32K ctx",
+        "value": round(gbs, 1), "unit": "GB/s",
+        "us_per_layer": round(ms_per_step * 1e3, 3), "pct_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2),
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16 in, f32 accumulate",
+        "data": "synthetic (seeded N(0,1) fp16 q/K; V = 3-bit PolarQuant of seeded N(0,1) fp16)",
+        "config": {"workload": "config 2: V-only decode attention, 28 q / 4 kv heads (n_rep 7), d=128, "
+                               "batch 1, 1 query token, 32768 cached positions, dense softmax (threshold 0)",
+                   "launch": mode, "buffer_sets": N_SETS, "algorithmic_bytes_per_step": ALGO_BYTES},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
+                     "kernel": "tq_vonly_decode_attn (tile pass + merge pass per step)"},
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -290,7 +290,7 @@ def prerot_fused_qk_scores(q_rot, k_packed, k_norms, centroids, dim: int, bits: 
     idx = unpack_indices(k_packed, bits, dim).astype(np.int64)      # (n_kv, seq, dim)
     cv = c[idx].astype(np.float64)
     qg = q_rot.reshape(n_kv, n_rep, dim).astype(np.float64)
-    dots = np.einsum("gsd,grd->grs", cv, qg)                         # (n_kv, n_rep, seq)
+    dots = np.matmul(qg, cv.transpose(0, 2, 1))                      # (n_kv, n_rep, seq)
     out = dots.astype(F32) * k_norms[:, None, :] * F32(1.0 / dim)
     return out.reshape(n_q, seq).astype(F32)
 
@@ -322,7 +322,7 @@ def sparse_v_matvec(weights, v_packed, v_norms, centroids, signs, dim: int, bits
     cv = c[idx].astype(np.float64)                                   # (n_kv, seq, dim)
     wn = np.where(w < thr, F32(0), w).reshape(n_kv, n_rep, seq).astype(np.float64)
     wn = wn * np.asarray(v_norms, dtype=F32).astype(np.float64)[:, None, :]
-    S = np.einsum("grs,gsd->grd", wn, cv).reshape(n_q, dim).astype(F32)
+    S = np.matmul(wn, cv).reshape(n_q, dim).astype(F32)
     return raw_butterfly(S) * np.asarray(signs, dtype=F32) * F32(1.0 / dim)
 
 
@@ -395,7 +395,7 @@ def vonly_decode_attention(q, k, v_packed, v_norms, v_centroids, v_signs, dim: i
         raise ValueError(
             f"n_q_heads ({n_q}) must equal n_kv_heads ({n_kv}) * n_rep ({n_rep})")
     qg = q.reshape(n_kv, n_rep, dim).astype(np.float64)
-    s = np.einsum("grd,gtd->grt", qg, k.astype(np.float64)).reshape(n_q, T) * float(attn_scale)
+    s = np.matmul(qg, k.astype(np.float64).transpose(0, 2, 1)).reshape(n_q, T) * float(attn_scale)
     if mask is not None:
         s = s + np.asarray(mask, dtype=np.float64)
     w = _softmax64(s).astype(F32)
