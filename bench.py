@@ -199,7 +199,7 @@ def main():
                    "launch": mode, "buffer_sets": N_SETS, "algorithmic_bytes_per_step": ALGO_BYTES},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
-                     "kernel": "tq_vonly_decode_attn (tile pass + merge pass per step)"},
+                     "kernel": "tqm::vonly_tile_mfma_kernel (+ tqm::decode_merge_rows_kernel, both inside the timed step)"},
         "cpu_baseline": cpu,
     }
     print(json.dumps(line))

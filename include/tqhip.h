@@ -218,7 +218,12 @@ int tq_vonly_decode_attn(const void* q, int q_dtype, const void* k_f16,
                          void* out, void* workspace, size_t workspace_bytes,
                          const tq_decode_shape* shape /* host */, tq_stream_t stream);
 
-/* Bytes of workspace the fused op needs for this shape (host computation, no GPU call). */
+/*
+ * Bytes of workspace the op needs for this shape (host computation, no GPU call).  The workspace
+ * holds per-tile partial results between the two passes of a call; its contents need not be
+ * preserved or cleared between calls.  Calls that share a workspace must be ordered (same stream);
+ * concurrent calls need separate workspaces.
+ */
 size_t tq_workspace_bytes(int op, int n_seq, int n_q_heads, int64_t max_seq_len, int dim);
 
 #ifdef __cplusplus

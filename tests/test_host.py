@@ -58,6 +58,7 @@ def test_argument_errors_without_launch():
     assert lib.tq_flash_decode(null, null, null, null, null, b, b, null, null, null, 0, ctypes.byref(sh), null) == -2
     with pytest.raises(RuntimeError):
         _lib.check(-8)
+    assert lib.tq_workspace_bytes(0, 1, 28, 32768, 128) == 28 * 128 * 130 * 4
     assert lib.tq_workspace_bytes(2, 1, 28, 32768, 128) == 28 * 128 * 130 * 4
 
 

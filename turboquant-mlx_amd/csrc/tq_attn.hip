@@ -7,6 +7,7 @@
 // second pass merges the tiles, applies the ONE Walsh-Hadamard butterfly per output row, the
 // signs and the 1/dim factor.
 #include "tq_common.h"
+#include "tq_decode_mfma.h"
 
 #include <math.h>
 
@@ -490,6 +491,55 @@ int launch_decode(const void* q, int q_dtype, const uint32_t* k_packed, const fl
   return TQ_OK;
 }
 
+// Matrix-core path: tile pass (partials of 512-position tiles) + merge pass.
+int launch_vonly_mfma(const void* q, const void* k_f16, const uint32_t* v_packed, const float* v_norms,
+                      const float* v_centroids, const float* v_signs, void* out, void* workspace,
+                      size_t workspace_bytes, const tq_decode_shape& sh, hipStream_t stream) {
+  const char* who = "tq_vonly_decode_attn";
+  const int n_q = sh.n_kv_heads * sh.n_rep;
+  const int n_tiles = (int)((sh.seq_len + tqm::kTilePos - 1) / tqm::kTilePos);
+  const size_t need = (size_t)sh.n_seq * n_q * n_tiles * (tqm::kD + 2) * sizeof(float);
+  if (!workspace || workspace_bytes < need)
+    return tq::fail(TQ_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, need, workspace_bytes);
+  if (!tq::aligned(workspace, 16)) return tq::fail(TQ_ERR_ALIGN, "%s: workspace must be 16-byte aligned", who);
+  tqm::MfmaArgs a{};
+  a.q = (const __half*)q; a.k = (const __half*)k_f16;
+  a.v_packed = v_packed; a.v_norms = v_norms;
+  a.seq_offsets = sh.seq_offsets; a.mask = sh.mask;
+  a.ws_S = (float*)workspace;
+  a.ws_ml = a.ws_S + (size_t)sh.n_seq * n_q * n_tiles * tqm::kD;
+  a.seq_len = sh.seq_len;
+  a.k_seq_stride = sh.k_seq_stride; a.k_head_stride = sh.k_head_stride;
+  a.v_seq_stride = sh.v_seq_stride; a.v_head_stride = sh.v_head_stride;
+  a.vn_seq_stride = sh.vn_seq_stride; a.vn_head_stride = sh.vn_head_stride;
+  a.mask_seq_stride = sh.mask_seq_stride; a.mask_head_stride = sh.mask_head_stride;
+  a.n_kv = sh.n_kv_heads; a.n_rep = sh.n_rep; a.n_tiles_max = n_tiles;
+  a.attn_scale = sh.attn_scale;
+#ifdef TQ_TRACE
+  {  // timeline goes behind the regular workspace when the caller left room for it
+    const size_t tbytes = (size_t)n_tiles * sh.n_kv_heads * sh.n_seq * 16 * sizeof(unsigned long long);
+    const size_t off = (need + 255) / 256 * 256;
+    a.trace = (workspace_bytes >= off + tbytes) ? (unsigned long long*)((char*)workspace + off) : nullptr;
+  }
+#endif
+  Codebook vcb;
+  fill_codebook(vcb, v_centroids, sh.bits);
+  dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
+  tqm::vonly_tile_mfma_kernel<<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb);
+  TQ_CHECK_LAUNCH(who);
+  dim3 mgrid(n_q, sh.n_seq);
+  const float inv_dim = 1.0f / (float)sh.dim;
+#define LAUNCH_MERGE_M(TO)                                                                                \
+  tqm::decode_merge_rows_kernel<TO><<<mgrid, tqm::kMergeThreads, 0, stream>>>(                              \
+      a.ws_S, a.ws_ml, sh.seq_offsets, sh.seq_len, n_tiles, sh.n_kv_heads, sh.n_rep, v_signs, inv_dim, (TO*)out)
+  if (sh.out_dtype == TQ_F16) { LAUNCH_MERGE_M(__half); }
+  else if (sh.out_dtype == TQ_BF16) { LAUNCH_MERGE_M(__hip_bfloat16); }
+  else { LAUNCH_MERGE_M(float); }
+#undef LAUNCH_MERGE_M
+  TQ_CHECK_LAUNCH(who);
+  return TQ_OK;
+}
+
 int check_shape(const tq_decode_shape* sh, const char* who, int max_dim) {
   if (!sh) return tq::fail(TQ_ERR_NULL, "%s: null shape", who);
   if (int rc = tq::check_dim_bits(sh->dim, sh->bits)) return rc;
@@ -509,8 +559,10 @@ int check_shape(const tq_decode_shape* sh, const char* who, int max_dim) {
 // ------------------------------------------------------------------ C ABI
 
 extern "C" size_t tq_workspace_bytes(int op, int n_seq, int n_q_heads, int64_t max_seq_len, int dim) {
-  (void)op;
   if (n_seq < 1 || n_q_heads < 1 || max_seq_len < 0 || dim < 1) return 0;
+  // Partials of the float32 kernels (tiles of kTile positions) bound those of the matrix-core
+  // kernels (larger tiles), so one size serves every op.
+  (void)op;
   return ws_bytes(n_seq, n_q_heads, max_seq_len, dim);
 }
 
@@ -620,6 +672,11 @@ extern "C" int tq_vonly_decode_attn(const void* q, int q_dtype, const void* k_f1
   if (shape->seq_len > 0 && (!k_f16 || !v_packed || !v_norms))
     return tq::fail(TQ_ERR_NULL, "tq_vonly_decode_attn: null pointer");
   if (!tq::aligned(k_f16, 16)) return tq::fail(TQ_ERR_ALIGN, "tq_vonly_decode_attn: k must be 16-byte aligned");
+  // d = 128, 3-bit, fp16 queries, at most 16 query heads per kv head: matrix-core tile pass.
+  if (shape->dim == 128 && shape->bits == 3 && q_dtype == TQ_F16 && shape->n_rep <= tqm::kHeadsMax &&
+      tq::aligned(q, 16) && shape->seq_len > 0)
+    return launch_vonly_mfma(q, k_f16, v_packed, v_norms, v_centroids, v_signs, out, workspace, workspace_bytes,
+                             *shape, (hipStream_t)stream_);
   return launch_decode<kDenseK>(q, q_dtype, nullptr, nullptr, k_f16, v_packed, v_norms, nullptr, v_centroids,
                                 v_signs, out, workspace, workspace_bytes, *shape, 0.0f, (hipStream_t)stream_,
                                 "tq_vonly_decode_attn");

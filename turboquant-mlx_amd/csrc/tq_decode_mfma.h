@@ -1,0 +1,470 @@
+// Decode attention on the matrix cores for the common shape d = 128, 3-bit values, fp16 queries,
+// n_rep <= 16 query heads per kv head.  Included by tq_attn.hip.
+//
+// Tile pass.  A workgroup of 8 wavefronts owns 512 consecutive KV positions of one kv head; a
+// wavefront owns 64 of them and serves all n_rep query heads that share the kv head.  A CU can only
+// start one wave-wide load instruction every ~24 clocks, so the pass is built to need few of them
+// (22 per wave) and to have all of them in flight before any arithmetic starts:
+//
+//   K rows   16 x 16-byte loads per lane, fully coalesced (an instruction reads 4 whole rows), then
+//            turned into matrix-operand layout (one row per lane) through a 4 KB per-wave LDS buffer
+//            with an XOR swizzle on the 16-byte piece index: writes and reads are conflict-free.
+//   V words  the wave's 64 packed rows are one contiguous 3328-byte block: 4 coalesced 16-byte loads
+//            per lane, copied into the same LDS buffer, from which each lane picks the two words
+//            that hold its 8 three-bit fields of a position.
+//   Q, norms one 4-byte load per thread each, shared through LDS.
+//   scores   D[p][h] = sum_e K[p][e] * Q[h][e]: per 16 positions 4 x v_mfma_f32_16x16x32_f16
+//            (A = K rows, B = Q columns, heads padded to 16).
+//   softmax  over the wave's 64 positions per head, in registers plus two lane exchanges.
+//   values   S[h][e] += sum_p P[h][p] * c[idx[p][e]]: A = P * v_norm, taken straight from the score
+//            accumulators (the D layout of the first product is the A layout of the second);
+//            B = centroid pairs looked up in a 64-entry LDS table indexed by two 3-bit fields --
+//            the look-ups are done while K is still arriving.
+//   output   the 8 waves combine (m, l, S) through LDS; one partial per workgroup goes to the
+//            workspace.
+//
+// Merge pass.  One workgroup per query head folds the tile partials (running-maximum rescale),
+// applies the ONE Walsh-Hadamard butterfly per output row, signs, 1/dim and 1/l.  As a dependent
+// launch it costs about 1.3 us plus its own ~1 us; merging inside the tile pass instead (last
+// workgroup to arrive) was measured slower, because a single CU cannot pull the ~230 KB of partials
+// of a kv head quickly and the counter/visibility round trips sit on the critical path.
+//
+// The contraction index of a matrix instruction may be permuted freely as long as A and B use the
+// same permutation; that freedom is what lets K be read in 16-byte pieces and lets positions inside
+// a 32-position block keep the order the score accumulators come in.
+#pragma once
+
+#include "tq_common.h"
+
+namespace tqm {
+
+using namespace tqd;
+
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u4 __attribute__((ext_vector_type(4)));   // plain vector: stays in registers
+
+constexpr int kD = 128;
+constexpr int kPdim = 13;
+constexpr int kWaves = 8;
+constexpr int kWavePos = 64;
+constexpr int kTilePos = kWaves * kWavePos;      // 512 positions per workgroup
+constexpr int kMfmaThreads = kWaves * 64;
+constexpr int kHeadsMax = 16;
+constexpr int kMergeThreads = 256;
+
+struct MfmaArgs {
+  const __half* q;            // [n_seq, n_q, 128] fp16
+  const __half* k;            // dense keys, rows of 128 halfs
+  const uint32_t* v_packed;
+  const float* v_norms;
+  const int32_t* seq_offsets;
+  const float* mask;
+  float* ws_S;                // [n_seq * n_kv, n_tiles_max, n_rep, 128]
+  float* ws_ml;               // [n_seq * n_kv, n_tiles_max, n_rep, 2]
+  int64_t seq_len;
+  int64_t k_seq_stride, k_head_stride;
+  int64_t v_seq_stride, v_head_stride, vn_seq_stride, vn_head_stride;
+  int64_t mask_seq_stride, mask_head_stride;
+  int32_t n_kv, n_rep, n_tiles_max;
+  float attn_scale;
+#ifdef TQ_TRACE
+  unsigned long long* trace;
+#endif
+};
+
+// Optional phase timeline for tuning (compile with -DTQ_TRACE): thread 0 of every workgroup
+// stores the 100 MHz real-time counter at each phase boundary into a.trace[workgroup][16].
+#ifdef TQ_TRACE
+#define TQ_STAMP(slot)                                                                              \
+  do {                                                                                              \
+    if (a.trace && threadIdx.x == 0)                                                                \
+      a.trace[((blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 16 + (slot)] =     \
+          __builtin_amdgcn_s_memrealtime();                                                         \
+  } while (0)
+#else
+#define TQ_STAMP(slot) do {} while (0)
+#endif
+
+__device__ __forceinline__ uint32_t pack_h2(float a, float b) {
+  __half2 h = __floats2half2_rn(a, b);
+  return *reinterpret_cast<uint32_t*>(&h);
+}
+
+// grid = (n_tiles_max, n_kv, n_seq), 512 threads.
+__global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
+  // 32 KB used three ways: per-wave staging (8 x 4 KB) first for the packed V block, then for K
+  // tiles; finally the cross-wave merge buffer S_s[4][16][128].
+  __shared__ __align__(16) unsigned char big_s[32768];
+  __shared__ uint32_t lut_s[64];                       // half2(c[i & 7], c[i >> 3])
+  __shared__ __align__(16) uint32_t q_s[kHeadsMax][kD / 2];   // fp16 pairs, rows >= n_rep are zero
+  __shared__ __align__(16) float nrm_s[kWaves][kWavePos];
+  __shared__ float m_s[kWaves][kHeadsMax], l_s[kWaves][kHeadsMax];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int n16 = lane & 15, g = lane >> 4;
+  const int tile = blockIdx.x, kvh = blockIdx.y, seq = blockIdx.z;
+  const int n_rep = a.n_rep;
+  const int n_q = a.n_kv * n_rep;
+  const int64_t q_row0 = (int64_t)seq * n_q + (int64_t)kvh * n_rep;
+
+  int64_t first = 0, len = a.seq_len;
+  if (a.seq_offsets) {
+    first = a.seq_offsets[seq];
+    len = (int64_t)a.seq_offsets[seq + 1] - first;
+  }
+  const int64_t tile_p0 = (int64_t)tile * kTilePos;
+  TQ_STAMP(0);
+  if (tile_p0 >= len) return;                          // the merge pass never reads this tile
+  const int rows_here = (int)min((int64_t)kTilePos, len - tile_p0);   // valid rows of this tile
+  const int last_row = rows_here - 1;
+  const int wrow0 = wave * kWavePos;                                  // wave's first row inside the tile
+
+  // ---- issue every global load of this wave, small ones first -------------------------------------
+  uint32_t my_q[2];                                    // Q rows of this kv head: n_rep x 64 words, <= 1024
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int w = tid + i * kMfmaThreads;
+    my_q[i] = (w < n_rep * (kD / 2)) ? reinterpret_cast<const uint32_t*>(a.q + q_row0 * kD)[w] : 0u;
+  }
+  float my_norm;
+  {
+    const float* nb = a.v_norms + (int64_t)seq * a.vn_seq_stride + (int64_t)kvh * a.vn_head_stride + first + tile_p0;
+    int row = wrow0 + lane;
+    row = row < last_row ? row : last_row;
+    my_norm = nb[(unsigned)row];
+  }
+  // packed V of the wave: 64 rows x 52 bytes, contiguous.  Full, 16-byte aligned blocks take four
+  // 16-byte loads per lane; ragged or unaligned ones take thirteen 4-byte loads with the index
+  // clamped to the last valid word.  Either way the LDS image is the plain copy of the block.
+  const uint32_t* vblock = a.v_packed +
+      ((int64_t)seq * a.v_seq_stride + (int64_t)kvh * a.v_head_stride + first + tile_p0 + wrow0) * kPdim;
+  const bool v_wide = (wrow0 + kWavePos <= rows_here) && ((reinterpret_cast<uintptr_t>(vblock) & 15) == 0);
+  u4 vq[4];
+  uint32_t vd[13];
+  if (v_wide) {
+    const u4* vb4 = reinterpret_cast<const u4*>(vblock);
+#pragma unroll
+    for (int i = 0; i < 3; ++i) vq[i] = vb4[i * 64 + lane];
+    vq[3] = vb4[192 + (lane & 15)];                      // 208 pieces in all; lanes >= 16 repeat
+  } else {
+    const int valid_words = max(0, rows_here - wrow0) * kPdim;       // words of the block inside the sequence
+    const uint32_t* tile_base = vblock - (int64_t)wrow0 * kPdim;     // row 0 of the tile: always valid
+#pragma unroll
+    for (int i = 0; i < 13; ++i) {
+      const int w = i * 64 + lane;
+      vd[i] = (w < valid_words) ? vblock[w] : tile_base[0];
+    }
+  }
+  // K: instruction i reads rows 4i .. 4i+3 of the wave; lane L takes 16-byte piece (L & 15) ^ (row & 7)
+  // of row 4i + (L >> 4) -- any order of the 16 pieces covers the same 256 contiguous bytes.
+  // A wave cannot run ahead of a load it is unable to issue, and the CU's memory pipeline is busy
+  // for the whole pass, so the K loads are issued in three instalments with the V decode (pure
+  // ALU / LDS work) placed between them; scheduling barriers keep the compiler from regrouping.
+  const u4* kbase = reinterpret_cast<const u4*>(
+      a.k + ((int64_t)seq * a.k_seq_stride + (int64_t)kvh * a.k_head_stride + first + tile_p0) * kD);
+  u4 kreg[16];
+  auto issue_k = [&](int i) {
+    const int r = 4 * i + (lane >> 4);
+    const int piece = (lane & 15) ^ (r & 7);
+    int row = wrow0 + r;
+    row = row < last_row ? row : last_row;
+    kreg[i] = kbase[(unsigned)(row * 16 + piece)];
+  };
+#pragma unroll
+  for (int i = 0; i < 4; ++i) issue_k(i);
+  __builtin_amdgcn_sched_barrier(0);
+  TQ_STAMP(15);
+  if (tid < 64) {
+    float clo = 0.0f, chi = 0.0f;                        // selects, not a dynamic index into kernel arguments
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      clo = ((tid & 7) == i) ? vcb.c[i] : clo;
+      chi = ((tid >> 3) == i) ? vcb.c[i] : chi;
+    }
+    lut_s[tid] = pack_h2(clo, chi);
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) (&q_s[0][0])[tid + i * kMfmaThreads] = my_q[i];
+  nrm_s[wave][lane] = my_norm;
+  __syncthreads();
+  TQ_STAMP(1);
+
+  // ---- Q operand and the V norms of this lane's 16 positions ----------------------------------------
+  u4 qreg[4];
+#pragma unroll
+  for (int kb = 0; kb < 4; ++kb) qreg[kb] = *reinterpret_cast<const u4*>(&q_s[n16][(4 * kb + g) * 4]);
+  float vn[4][4];
+  float nmax = 0.0f;
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const float4 n4 = *reinterpret_cast<const float4*>(&nrm_s[wave][16 * t + 4 * g]);
+    vn[t][0] = n4.x; vn[t][1] = n4.y; vn[t][2] = n4.z; vn[t][3] = n4.w;
+    nmax = fmaxf(nmax, fmaxf(fmaxf(n4.x, n4.y), fmaxf(n4.z, n4.w)));
+  }
+  nmax = fmaxf(nmax, shfl_xor_f(nmax, 16));
+  nmax = fmaxf(nmax, shfl_xor_f(nmax, 32));
+  // power-of-two scale 2^-floor(log2 nmax): keeps P * norm inside half range whatever the norms are
+  int ex = (int)((__float_as_uint(nmax) >> 23) & 0xFF);
+  ex = ex < 1 ? 127 : (ex > 253 ? 253 : ex);
+  const float tscale = __uint_as_float((uint32_t)(254 - ex) << 23);
+  const float inv_tscale = __uint_as_float((uint32_t)ex << 23);
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) vn[t][j] *= tscale;
+
+  // ---- packed V -> B operands of the value product, while K is still on its way -------------------
+  uint32_t* stage = reinterpret_cast<uint32_t*>(big_s) + wave * 1024;   // this wave's 4 KB
+  if (v_wide) {
+    u4* st4 = reinterpret_cast<u4*>(stage);
+#pragma unroll
+    for (int i = 0; i < 3; ++i) st4[i * 64 + lane] = vq[i];
+    if (lane < 16) st4[192 + lane] = vq[3];
+  } else {
+#pragma unroll
+    for (int i = 0; i < 13; ++i) stage[i * 64 + lane] = vd[i];
+  }
+  // lane (n16, g) decodes elements 8*n16 .. 8*n16+7 of positions 16t + 4g + j: 24 bits that start in
+  // word w0 at field s0 and may spill into word w0 + 1 (lane 15 reads words 11, 12 and takes
+  // everything from the second).  X / Y interleave the even / odd fields of two positions into
+  // 6-bit table indices at bit offsets 0, 6, 12, 18; each index fetches a centroid pair.
+  const int w0 = (n16 == 15) ? 11 : (8 * n16) / 10;
+  const int s0 = (n16 == 15) ? 10 : (8 * n16) % 10;
+  const int sh_lo = 3 * s0, sh_hi = 30 - 3 * s0;
+  constexpr uint32_t kEven = 0x1C71C7u;        // fields 0, 2, 4, 6
+  u4 breg[2][8];
+#pragma unroll
+  for (int kb2 = 0; kb2 < 2; ++kb2) {
+    if (kb2 == 1) {                                      // second instalment of K
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 4; i < 8; ++i) issue_k(i);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    uint32_t X[4], Y[4];
+#pragma unroll
+    for (int qd = 0; qd < 4; ++qd) {
+      const int t = 2 * kb2 + (qd >> 1), jp = qd & 1;
+      const uint32_t* ra = stage + (16 * t + 4 * g + 2 * jp) * kPdim + w0;
+      const uint32_t fa = ((ra[0] >> sh_lo) | (ra[1] << sh_hi)) & 0xFFFFFFu;
+      const uint32_t fb = ((ra[kPdim] >> sh_lo) | (ra[kPdim + 1] << sh_hi)) & 0xFFFFFFu;
+      X[qd] = (fa & kEven) | ((fb & kEven) << 3);
+      Y[qd] = ((fa >> 3) & kEven) | (fb & (kEven << 3));
+    }
+#pragma unroll
+    for (int et = 0; et < 8; ++et)
+#pragma unroll
+      for (int qd = 0; qd < 4; ++qd) {
+        const uint32_t src = (et & 1) ? Y[qd] : X[qd];
+        breg[kb2][et][qd] = lut_s[(src >> (6 * (et >> 1))) & 63u];
+      }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int i = 8; i < 16; ++i) issue_k(i);               // last instalment of K
+  __builtin_amdgcn_sched_barrier(0);
+  TQ_STAMP(7);
+
+  // ---- scores, tile by tile as K arrives ----------------------------------------------------------------
+  float s[4][4];
+  {
+    u4* kst = reinterpret_cast<u4*>(stage);                           // 256 pieces of 16 bytes
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+#pragma unroll
+      for (int ii = 0; ii < 4; ++ii) kst[ii * 64 + lane] = kreg[4 * t + ii];
+      f4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb) {
+        const u4 ka = kst[n16 * 16 + ((4 * kb + g) ^ (n16 & 7))];     // piece 4kb+g of row n16
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, ka), __builtin_bit_cast(h8, qreg[kb]),
+                                                     acc, 0, 0, 0);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int row = wrow0 + 16 * t + 4 * g + j;                    // accumulator row 4g + j of tile t
+        float v = acc[j] * a.attn_scale;
+        if (a.mask && row < rows_here && n16 < n_rep)
+          v += a.mask[(int64_t)seq * a.mask_seq_stride + ((int64_t)kvh * n_rep + n16) * a.mask_head_stride +
+                      tile_p0 + row];
+        s[t][j] = (row < rows_here) ? v : -INFINITY;
+      }
+    }
+  }
+  TQ_STAMP(2);
+
+  // ---- softmax statistics of head n16 over the wave's 64 positions ----------------------------------
+  float m = -INFINITY;
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) m = fmaxf(m, s[t][j]);
+  m = fmaxf(m, shfl_xor_f(m, 16));
+  m = fmaxf(m, shfl_xor_f(m, 32));
+  const float msafe = (m == -INFINITY) ? 0.0f : m;
+  float l = 0.0f;
+  uint32_t pa[2][4];                                     // A operands of the value product
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    float p[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      p[j] = __expf(s[t][j] - msafe);
+      l += p[j];
+      p[j] *= vn[t][j];
+    }
+    pa[t >> 1][2 * (t & 1)] = pack_h2(p[0], p[1]);
+    pa[t >> 1][2 * (t & 1) + 1] = pack_h2(p[2], p[3]);
+  }
+  l += shfl_xor_f(l, 16);
+  l += shfl_xor_f(l, 32);
+
+  // ---- values ------------------------------------------------------------------------------------------
+  f4 accS[8];
+#pragma unroll
+  for (int et = 0; et < 8; ++et) accS[et] = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int kb2 = 0; kb2 < 2; ++kb2) {
+    const u4 A = {pa[kb2][0], pa[kb2][1], pa[kb2][2], pa[kb2][3]};
+#pragma unroll
+    for (int et = 0; et < 8; ++et)
+      accS[et] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, A), __builtin_bit_cast(h8, breg[kb2][et]),
+                                                        accS[et], 0, 0, 0);
+  }
+  TQ_STAMP(3);
+
+  // ---- merge the eight waves ---------------------------------------------------------------------------
+  if (g == 0) {
+    m_s[wave][n16] = m;
+    l_s[wave][n16] = l;
+  }
+  __syncthreads();                                       // also: every wave is done with its staging area
+  TQ_STAMP(8);
+  float (*S_s)[kHeadsMax][kD] = reinterpret_cast<float (*)[kHeadsMax][kD]>(big_s);   // [4][16][128]
+  float alpha[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int h = 4 * g + j;                             // accumulator row -> head
+    float M = m_s[0][h];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) M = fmaxf(M, m_s[w][h]);
+    const float mw = m_s[wave][h];
+    alpha[j] = (mw == -INFINITY) ? 0.0f : __expf(mw - M) * inv_tscale;
+  }
+  if (wave >= 4) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float4* dst = reinterpret_cast<float4*>(&S_s[wave - 4][4 * g + j][8 * n16]);
+      dst[0] = make_float4(accS[0][j] * alpha[j], accS[1][j] * alpha[j], accS[2][j] * alpha[j], accS[3][j] * alpha[j]);
+      dst[1] = make_float4(accS[4][j] * alpha[j], accS[5][j] * alpha[j], accS[6][j] * alpha[j], accS[7][j] * alpha[j]);
+    }
+  }
+  __syncthreads();
+  if (wave < 4) {                                        // same lanes, same addresses as wave + 4 used
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float4* dst = reinterpret_cast<float4*>(&S_s[wave][4 * g + j][8 * n16]);
+      const float4 a0 = dst[0], a1 = dst[1];
+      dst[0] = make_float4(accS[0][j] * alpha[j] + a0.x, accS[1][j] * alpha[j] + a0.y,
+                           accS[2][j] * alpha[j] + a0.z, accS[3][j] * alpha[j] + a0.w);
+      dst[1] = make_float4(accS[4][j] * alpha[j] + a1.x, accS[5][j] * alpha[j] + a1.y,
+                           accS[6][j] * alpha[j] + a1.z, accS[7][j] * alpha[j] + a1.w);
+    }
+  }
+  __syncthreads();
+  TQ_STAMP(9);
+  const int64_t grp = (int64_t)seq * a.n_kv + kvh;
+  float* pS = a.ws_S + (grp * a.n_tiles_max + tile) * (int64_t)(n_rep * kD);
+  float* pml = a.ws_ml + (grp * a.n_tiles_max + tile) * (int64_t)(n_rep * 2);
+  for (int i = tid; i < n_rep * kD; i += kMfmaThreads) {
+    const int h = i >> 7, e = i & 127;
+    pS[i] = (S_s[0][h][e] + S_s[1][h][e]) + (S_s[2][h][e] + S_s[3][h][e]);
+  }
+  if (tid < n_rep) {
+    const int h = tid;
+    float M = m_s[0][h];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) M = fmaxf(M, m_s[w][h]);
+    float L = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) L += (m_s[w][h] == -INFINITY) ? 0.0f : __expf(m_s[w][h] - M) * l_s[w][h];
+    pml[2 * h] = M;
+    pml[2 * h + 1] = L;
+  }
+  TQ_STAMP(10);
+}
+
+// Merge pass: grid = (n_q, n_seq), 256 threads.  Lane group ph = tid / 32 folds tiles ph, ph + 8, ...
+// (4 elements per lane) with a running maximum; the 8 groups are then combined through LDS and wave 0
+// finishes the row.
+template <typename TO>
+__global__ __launch_bounds__(kMergeThreads) void decode_merge_rows_kernel(
+    const float* __restrict__ ws_S, const float* __restrict__ ws_ml, const int32_t* __restrict__ seq_offsets,
+    int64_t seq_len, int n_tiles_max, int n_kv, int n_rep, const float* __restrict__ signs, float inv_dim,
+    TO* __restrict__ out) {
+  __shared__ __align__(16) float acc_s[8][kD];
+  __shared__ float ml_s[8][2];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int eq = tid & 31, ph = tid >> 5;
+  const int head = blockIdx.x, seq = blockIdx.y;
+  const int kvh = head / n_rep, r = head - kvh * n_rep;
+  int64_t len = seq_len;
+  if (seq_offsets) len = (int64_t)seq_offsets[seq + 1] - seq_offsets[seq];
+  const int n_tiles = (int)((len + kTilePos - 1) / kTilePos);
+  const int64_t grp = (int64_t)seq * n_kv + kvh;
+  const float* gS = ws_S + grp * n_tiles_max * (int64_t)(n_rep * kD) + r * kD + 4 * eq;
+  const float* gml = ws_ml + grp * n_tiles_max * (int64_t)(n_rep * 2) + r * 2;
+  float M = -INFINITY, L = 0.0f;
+  f4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int t0 = ph; t0 < n_tiles; t0 += 64) {            // 8 tiles per lane group and round
+    f4 x[8];
+    float2 ml[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int t = min(t0 + 8 * u, n_tiles - 1);
+      x[u] = *reinterpret_cast<const f4*>(gS + (int64_t)t * (n_rep * kD));
+      ml[u] = *reinterpret_cast<const float2*>(gml + (int64_t)t * (n_rep * 2));
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (t0 + 8 * u < n_tiles && ml[u].x != -INFINITY) {
+        const float Mn = fmaxf(M, ml[u].x);
+        const float fo = (M == -INFINITY) ? 0.0f : __expf(M - Mn);
+        const float fc = __expf(ml[u].x - Mn);
+        acc = acc * fo + x[u] * fc;
+        L = L * fo + ml[u].y * fc;
+        M = Mn;
+      }
+    }
+  }
+  *reinterpret_cast<f4*>(&acc_s[ph][4 * eq]) = acc;
+  if (eq == 0) { ml_s[ph][0] = M; ml_s[ph][1] = L; }
+  __syncthreads();
+  if (tid >= 64) return;
+  float Mt = ml_s[0][0];
+#pragma unroll
+  for (int p = 1; p < 8; ++p) Mt = fmaxf(Mt, ml_s[p][0]);
+  float Lt = 0.0f;
+  float v[2] = {0.0f, 0.0f};
+#pragma unroll
+  for (int p = 0; p < 8; ++p) {
+    const float f = (ml_s[p][0] == -INFINITY) ? 0.0f : __expf(ml_s[p][0] - Mt);
+    Lt += f * ml_s[p][1];
+    v[0] += f * acc_s[p][lane];
+    v[1] += f * acc_s[p][lane + 64];
+  }
+  raw_butterfly<kD>(v, lane);
+  TO* o = out + ((int64_t)seq * gridDim.x + head) * kD;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int e = lane + 64 * i;
+    float val = (v[i] * signs[e]) * inv_dim;
+    val = (Lt > 0.0f) ? val / Lt : 0.0f;
+    store_from_float<TO>(o + e, val);
+  }
+}
+
+}  // namespace tqm

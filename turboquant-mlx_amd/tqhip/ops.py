@@ -81,6 +81,7 @@ _workspaces = {}
 
 
 def _workspace(device, stream_id: int, nbytes: int) -> torch.Tensor:
+    """Per (device, stream) scratch buffer for tile partials, grown on demand."""
     key = (device, stream_id)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
