@@ -33,10 +33,13 @@ ALGO_BYTES = N_Q * D * 2 + N_KV * T * D * 2 + N_KV * T * PDIM * 4 + N_KV * T * 4
 HBM_PEAK_GBS = 8000.0
 N_SETS = 10
 
-# HBM bytes per step from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same command,
-# scaled by the factor the same counters read for a plain copy kernel (see profiles/).
-# None until measured for the kernel that is currently the default.
-MEASURED_TRAFFIC_BYTES = None
+# HBM bytes per launch of the dominant kernel (the tile pass), from two rocprofv3 --pmc runs of
+# `python bench.py --steps 60 --warmup 6 --no-cpu --no-graph` (FETCH_SIZE, then WRITE_SIZE), each
+# scaled by what the same counter reads for `python bench.py --calibrate-copy --steps 40`, a plain
+# copy of ALGO_BYTES bytes (FETCH_SIZE reads 19986.6 for 39950 KiB -> factor 1.9988; WRITE_SIZE
+# reads 39950.0 -> factor 1.0000).  Tile pass: FETCH_SIZE 20080.5 -> 40137 KiB, WRITE_SIZE 916.0
+# -> 916 KiB.  Summary: profiles/vonly_decode_c2_pmc_traffic.md.
+MEASURED_TRAFFIC_BYTES = int((20080.5 * 39950.0 / 19986.6 + 916.0) * 1024)
 
 
 def make_sets(torch, tqhip, dev):
@@ -97,6 +100,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="instead of the benchmark, run --steps plain device copies of ALGO_BYTES bytes each "
+                         "(known traffic: ALGO_BYTES read + ALGO_BYTES written) to scale rocprofv3's "
+                         "FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the hot path shards by kv head "
@@ -110,6 +117,15 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.calibrate_copy:
+        srcs = [torch.full((ALGO_BYTES,), i + 1, dtype=torch.uint8, device=dev) for i in range(N_SETS)]
+        dst = torch.empty(ALGO_BYTES, dtype=torch.uint8, device=dev)
+        for i in range(args.steps):
+            dst.copy_(srcs[i % N_SETS])
+        torch.cuda.synchronize()
+        print(json.dumps({"calibrate_copy": True, "copies": args.steps, "bytes_read_each": ALGO_BYTES,
+                          "bytes_written_each": ALGO_BYTES}))
+        return
     sets, cb, signs = make_sets(torch, tqhip, dev)
     sc = 1.0 / math.sqrt(D)
     lib = _lib.load()
@@ -130,8 +146,9 @@ def main():
                 C.c_void_p(vn.data_ptr()), cb_host, C.c_void_p(signs.data_ptr()), C.c_void_p(outs[i].data_ptr()),
                 C.c_void_p(ws.data_ptr()), ws.numel(), C.byref(shape), C.c_void_p(stream))
 
-    def step(i, argsets):
-        rc = lib.tq_vonly_decode_attn(*argsets[i % N_SETS])
+    def step(i, argsets, phases=3):
+        a = argsets[i % N_SETS]
+        rc = lib.tq_vonly_decode_attn_phases(*a[:-1], phases, a[-1])
         if rc != 0:
             _lib.check(rc)
 
@@ -149,38 +166,45 @@ def main():
             sys.exit(1)
 
     side = torch.cuda.Stream(device=dev)
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    with torch.cuda.stream(side):
-        s_args = [bound(i, side.cuda_stream) for i in range(N_SETS)]
-        for i in range(args.warmup):
-            step(i, s_args)
-        side.synchronize()
-        if args.no_graph:
-            torch.cuda.synchronize()
-            ev0.record(side)
-            for i in range(args.steps):
-                step(i, s_args)
-            ev1.record(side)
+
+    def timed(phases):
+        """ms per launch of `args.steps` back-to-back calls (HIP graph replay unless --no-graph),
+        bracketed by HIP events on the launch stream."""
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        with torch.cuda.stream(side):
+            s_args = [bound(i, side.cuda_stream) for i in range(N_SETS)]
+            for i in range(args.warmup):
+                step(i, s_args, phases)
             side.synchronize()
-            mode = "eager"
-        else:
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, stream=side):
-                g_stream = torch.cuda.current_stream(dev)
-                g_args = [bound(i, g_stream.cuda_stream) for i in range(N_SETS)]
+            if args.no_graph:
+                ev0.record(side)
                 for i in range(args.steps):
-                    step(i, g_args)
-            graph.replay()                      # one untimed replay: instantiation, page-in
-            torch.cuda.synchronize()
-            ev0.record(side)
-            graph.replay()
-            ev1.record(side)
-            side.synchronize()
-            mode = "hipgraph"
-    torch.cuda.synchronize()
-    ms_total = ev0.elapsed_time(ev1)
-    ms_per_step = ms_total / args.steps
+                    step(i, s_args, phases)
+                ev1.record(side)
+                side.synchronize()
+            else:
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, stream=side):
+                    g_stream = torch.cuda.current_stream(dev)
+                    g_args = [bound(i, g_stream.cuda_stream) for i in range(N_SETS)]
+                    for i in range(args.steps):
+                        step(i, g_args, phases)
+                graph.replay()                  # one untimed replay: instantiation, page-in
+                torch.cuda.synchronize()
+                ev0.record(side)
+                graph.replay()
+                ev1.record(side)
+                side.synchronize()
+        torch.cuda.synchronize()
+        return ev0.elapsed_time(ev1) / args.steps
+
+    mode = "eager" if args.no_graph else "hipgraph"
+    ms_per_step = timed(3)                      # whole step: tile pass + merge pass
+    ms_tile = timed(1)                          # dominant kernel alone, same launch pattern
     gbs = ALGO_BYTES / (ms_per_step * 1e-3) / 1e9
+    gbs_tile = ALGO_BYTES / (ms_tile * 1e-3) / 1e9
+    step(0, eager_args)                         # leave outs[0] = the full result of set 0
+    torch.cuda.synchronize()
 
     # the timed steps must have produced the same result as the checked eager step
     if not torch.equal(outs[0], outs[0]) or torch.isnan(outs[0]).any():
@@ -197,9 +221,11 @@ def main():
         "config": {"workload": "config 2: V-only decode attention, 28 q / 4 kv heads (n_rep 7), d=128, "
                                "batch 1, 1 query token, 32768 cached positions, dense softmax (threshold 0)",
                    "launch": mode, "buffer_sets": N_SETS, "algorithmic_bytes_per_step": ALGO_BYTES},
-        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
-                     "kernel": "tqm::vonly_tile_mfma_kernel (+ tqm::decode_merge_rows_kernel, both inside the timed step)"},
+        "roofline": {"bound": "hbm", "achieved": round(gbs_tile, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs_tile / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
+                     "kernel": "tqm::vonly_tile_mfma_kernel", "us_per_launch": round(ms_tile * 1e3, 3),
+                     "note": "algorithmic bytes / event-timed launch period of the tile pass alone; "
+                             "`value` covers the whole step (tile pass + merge pass)"},
         "cpu_baseline": cpu,
     }
     print(json.dumps(line))

@@ -219,6 +219,18 @@ int tq_vonly_decode_attn(const void* q, int q_dtype, const void* k_f16,
                          const tq_decode_shape* shape /* host */, tq_stream_t stream);
 
 /*
+ * The same call with its two passes selectable: phases = 1 runs only the tile pass (per-tile
+ * partial sums and softmax statistics into `workspace`), phases = 2 only the merge pass (workspace
+ * -> out), phases = 3 both (= tq_vonly_decode_attn).  For callers that time or overlap the passes;
+ * the reference has a single kernel per call (sparse_v.py:169-185) and no counterpart to the split.
+ */
+int tq_vonly_decode_attn_phases(const void* q, int q_dtype, const void* k_f16,
+                                const uint32_t* v_packed, const float* v_norms,
+                                const float* v_centroids, const float* v_signs,
+                                void* out, void* workspace, size_t workspace_bytes,
+                                const tq_decode_shape* shape /* host */, int phases, tq_stream_t stream);
+
+/*
  * Bytes of workspace the op needs for this shape (host computation, no GPU call).  The workspace
  * holds per-tile partial results between the two passes of a call; its contents need not be
  * preserved or cleared between calls.  Calls that share a workspace must be ordered (same stream);

@@ -437,7 +437,7 @@ int launch_decode(const void* q, int q_dtype, const uint32_t* k_packed, const fl
                   const void* k_dense, const uint32_t* v_packed, const float* v_norms,
                   const float* k_centroids, const float* v_centroids, const float* v_signs, void* out,
                   void* workspace, size_t workspace_bytes, const tq_decode_shape& sh, float threshold,
-                  hipStream_t stream, const char* who) {
+                  hipStream_t stream, const char* who, int phases = 3) {
   const int n_q = sh.n_kv_heads * sh.n_rep;
   const size_t need = ws_bytes(sh.n_seq, n_q, sh.seq_len, sh.dim);
   if (!workspace || workspace_bytes < need)
@@ -467,7 +467,7 @@ int launch_decode(const void* q, int q_dtype, const uint32_t* k_packed, const fl
   Codebook kcb, vcb;
   fill_codebook(kcb, k_centroids, sh.bits);
   fill_codebook(vcb, v_centroids, sh.bits);
-  if (n_tiles > 0) {
+  if (n_tiles > 0 && (phases & 1)) {
     dim3 grid(n_tiles, sh.n_kv_heads * a.n_rgroups, sh.n_seq);
 #define LAUNCH_TILE(QT)                                                                              \
   TQ_DISPATCH_DIM(sh.dim, TQ_DISPATCH_BITS(sh.bits, (decode_tile_kernel<D_, B_, KMODE, QT>            \
@@ -478,6 +478,7 @@ int launch_decode(const void* q, int q_dtype, const uint32_t* k_packed, const fl
 #undef LAUNCH_TILE
     TQ_CHECK_LAUNCH(who);
   }
+  if (!(phases & 2)) return TQ_OK;
   dim3 mgrid(n_q, sh.n_seq);
 #define LAUNCH_MERGE(TO)                                                                              \
   TQ_DISPATCH_DIM(sh.dim, (decode_merge_kernel<D_, KMODE, TO><<<mgrid, TQ_WAVE, 0, stream>>>(          \
@@ -494,7 +495,7 @@ int launch_decode(const void* q, int q_dtype, const uint32_t* k_packed, const fl
 // Matrix-core path: tile pass (partials of 512-position tiles) + merge pass.
 int launch_vonly_mfma(const void* q, const void* k_f16, const uint32_t* v_packed, const float* v_norms,
                       const float* v_centroids, const float* v_signs, void* out, void* workspace,
-                      size_t workspace_bytes, const tq_decode_shape& sh, hipStream_t stream) {
+                      size_t workspace_bytes, const tq_decode_shape& sh, hipStream_t stream, int phases) {
   const char* who = "tq_vonly_decode_attn";
   const int n_q = sh.n_kv_heads * sh.n_rep;
   const int n_tiles = (int)((sh.seq_len + tqm::kTilePos - 1) / tqm::kTilePos);
@@ -524,9 +525,12 @@ int launch_vonly_mfma(const void* q, const void* k_f16, const uint32_t* v_packed
 #endif
   Codebook vcb;
   fill_codebook(vcb, v_centroids, sh.bits);
-  dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
-  tqm::vonly_tile_mfma_kernel<<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb);
-  TQ_CHECK_LAUNCH(who);
+  if (phases & 1) {
+    dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
+    tqm::vonly_tile_mfma_kernel<<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb);
+    TQ_CHECK_LAUNCH(who);
+  }
+  if (!(phases & 2)) return TQ_OK;
   dim3 mgrid(n_q, sh.n_seq);
   const float inv_dim = 1.0f / (float)sh.dim;
 #define LAUNCH_MERGE_M(TO)                                                                                \
@@ -662,11 +666,12 @@ extern "C" int tq_flash_decode(const float* q_rot, const uint32_t* k_packed, con
                                  (hipStream_t)stream_, "tq_flash_decode");
 }
 
-extern "C" int tq_vonly_decode_attn(const void* q, int q_dtype, const void* k_f16, const uint32_t* v_packed,
-                                    const float* v_norms, const float* v_centroids, const float* v_signs,
-                                    void* out, void* workspace, size_t workspace_bytes,
-                                    const tq_decode_shape* shape, tq_stream_t stream_) {
+extern "C" int tq_vonly_decode_attn_phases(const void* q, int q_dtype, const void* k_f16, const uint32_t* v_packed,
+                                           const float* v_norms, const float* v_centroids, const float* v_signs,
+                                           void* out, void* workspace, size_t workspace_bytes,
+                                           const tq_decode_shape* shape, int phases, tq_stream_t stream_) {
   if (int rc = check_shape(shape, "tq_vonly_decode_attn", 256)) return rc;
+  if (phases < 1 || phases > 3) return tq::fail(TQ_ERR_ARG, "tq_vonly_decode_attn: phases must be 1, 2 or 3");
   if (tq::check_dtype(q_dtype)) return tq::fail(TQ_ERR_DTYPE, "tq_vonly_decode_attn: unknown q_dtype %d", q_dtype);
   if (!q || !v_centroids || !v_signs || !out) return tq::fail(TQ_ERR_NULL, "tq_vonly_decode_attn: null pointer");
   if (shape->seq_len > 0 && (!k_f16 || !v_packed || !v_norms))
@@ -674,10 +679,18 @@ extern "C" int tq_vonly_decode_attn(const void* q, int q_dtype, const void* k_f1
   if (!tq::aligned(k_f16, 16)) return tq::fail(TQ_ERR_ALIGN, "tq_vonly_decode_attn: k must be 16-byte aligned");
   // d = 128, 3-bit, fp16 queries, at most 16 query heads per kv head: matrix-core tile pass.
   if (shape->dim == 128 && shape->bits == 3 && q_dtype == TQ_F16 && shape->n_rep <= tqm::kHeadsMax &&
-      tq::aligned(q, 16) && shape->seq_len > 0)
+      tq::aligned(q, 4) && shape->seq_len > 0)
     return launch_vonly_mfma(q, k_f16, v_packed, v_norms, v_centroids, v_signs, out, workspace, workspace_bytes,
-                             *shape, (hipStream_t)stream_);
+                             *shape, (hipStream_t)stream_, phases);
   return launch_decode<kDenseK>(q, q_dtype, nullptr, nullptr, k_f16, v_packed, v_norms, nullptr, v_centroids,
                                 v_signs, out, workspace, workspace_bytes, *shape, 0.0f, (hipStream_t)stream_,
-                                "tq_vonly_decode_attn");
+                                "tq_vonly_decode_attn", phases);
+}
+
+extern "C" int tq_vonly_decode_attn(const void* q, int q_dtype, const void* k_f16, const uint32_t* v_packed,
+                                    const float* v_norms, const float* v_centroids, const float* v_signs,
+                                    void* out, void* workspace, size_t workspace_bytes,
+                                    const tq_decode_shape* shape, tq_stream_t stream_) {
+  return tq_vonly_decode_attn_phases(q, q_dtype, k_f16, v_packed, v_norms, v_centroids, v_signs, out, workspace,
+                                     workspace_bytes, shape, 3, stream_);
 }
