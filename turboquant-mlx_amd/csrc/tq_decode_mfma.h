@@ -95,12 +95,12 @@ __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
 __global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
   // 32 KB used three ways: per-wave staging (8 x 4 KB) first for the packed V block, then for K
-  // tiles; finally the cross-wave merge buffer S_s[4][16][128].
+  // tiles; finally the cross-wave merge buffer S_all[8][8][128].
   __shared__ __align__(16) unsigned char big_s[32768];
   __shared__ uint32_t lut_s[64];                       // half2(c[i & 7], c[i >> 3])
   __shared__ __align__(16) uint32_t q_s[kHeadsMax][kD / 2];   // fp16 pairs, rows >= n_rep are zero
   __shared__ __align__(16) float nrm_s[kWaves][kWavePos];
-  __shared__ float m_s[kWaves][kHeadsMax], l_s[kWaves][kHeadsMax];
+  __shared__ float m_s[kWaves][kHeadsMax], l_s[kWaves][kHeadsMax], t_s[kWaves];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -174,7 +174,7 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
     kreg[i] = kbase[(unsigned)(row * 16 + piece)];
   };
 #pragma unroll
-  for (int i = 0; i < 4; ++i) issue_k(i);
+  for (int i = 0; i < 8; ++i) issue_k(i);
   __builtin_amdgcn_sched_barrier(0);
   TQ_STAMP(15);
   if (tid < 64) {
@@ -216,7 +216,7 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) vn[t][j] *= tscale;
 
-  // ---- packed V -> B operands of the value product, while K is still on its way -------------------
+  // ---- packed V -> table indices (registers), then look-ups interleaved with the score tiles -----------
   uint32_t* stage = reinterpret_cast<uint32_t*>(big_s) + wave * 1024;   // this wave's 4 KB
   if (v_wide) {
     u4* st4 = reinterpret_cast<u4*>(stage);
@@ -235,65 +235,70 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
   const int s0 = (n16 == 15) ? 10 : (8 * n16) % 10;
   const int sh_lo = 3 * s0, sh_hi = 30 - 3 * s0;
   constexpr uint32_t kEven = 0x1C71C7u;        // fields 0, 2, 4, 6
-  u4 breg[2][8];
+  uint32_t X[2][4], Y[2][4];
 #pragma unroll
-  for (int kb2 = 0; kb2 < 2; ++kb2) {
-    if (kb2 == 1) {                                      // second instalment of K
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int i = 4; i < 8; ++i) issue_k(i);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    uint32_t X[4], Y[4];
+  for (int kb2 = 0; kb2 < 2; ++kb2)
 #pragma unroll
     for (int qd = 0; qd < 4; ++qd) {
       const int t = 2 * kb2 + (qd >> 1), jp = qd & 1;
       const uint32_t* ra = stage + (16 * t + 4 * g + 2 * jp) * kPdim + w0;
       const uint32_t fa = ((ra[0] >> sh_lo) | (ra[1] << sh_hi)) & 0xFFFFFFu;
       const uint32_t fb = ((ra[kPdim] >> sh_lo) | (ra[kPdim + 1] << sh_hi)) & 0xFFFFFFu;
-      X[qd] = (fa & kEven) | ((fb & kEven) << 3);
-      Y[qd] = ((fa >> 3) & kEven) | (fb & (kEven << 3));
+      X[kb2][qd] = (fa & kEven) | ((fb & kEven) << 3);
+      Y[kb2][qd] = ((fa >> 3) & kEven) | (fb & (kEven << 3));
     }
+  u4 breg[2][8];
+  auto lookups = [&](int kb2) {
 #pragma unroll
     for (int et = 0; et < 8; ++et)
 #pragma unroll
       for (int qd = 0; qd < 4; ++qd) {
-        const uint32_t src = (et & 1) ? Y[qd] : X[qd];
+        const uint32_t src = (et & 1) ? Y[kb2][qd] : X[kb2][qd];
         breg[kb2][et][qd] = lut_s[(src >> (6 * (et >> 1))) & 63u];
       }
-  }
+  };
+  // one 16-position score tile: K pieces through the wave's staging area, 4 matrix instructions
+  float s[4][4];
+  u4* kst = reinterpret_cast<u4*>(stage);                             // 256 pieces of 16 bytes
+  auto qk_tile = [&](int t) {
+#pragma unroll
+    for (int ii = 0; ii < 4; ++ii) kst[ii * 64 + lane] = kreg[4 * t + ii];
+    f4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+      const u4 ka = kst[n16 * 16 + ((4 * kb + g) ^ (n16 & 7))];       // piece 4kb+g of row n16
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, ka), __builtin_bit_cast(h8, qreg[kb]),
+                                                   acc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int row = wrow0 + 16 * t + 4 * g + j;                      // accumulator row 4g + j of tile t
+      float v = acc[j] * a.attn_scale;
+      if (a.mask && row < rows_here && n16 < n_rep)
+        v += a.mask[(int64_t)seq * a.mask_seq_stride + ((int64_t)kvh * n_rep + n16) * a.mask_head_stride +
+                    tile_p0 + row];
+      s[t][j] = (row < rows_here) ? v : -INFINITY;
+    }
+  };
+  // schedule: look-ups (ALU + LDS) alternate with K instalments and score tiles, so the memory
+  // pipeline, the LDS and the ALUs all stay busy while K streams in
+  __builtin_amdgcn_sched_barrier(0);
+  lookups(0);
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-  for (int i = 8; i < 16; ++i) issue_k(i);               // last instalment of K
+  for (int i = 8; i < 12; ++i) issue_k(i);
+  __builtin_amdgcn_sched_barrier(0);
+  qk_tile(0);
+  __builtin_amdgcn_sched_barrier(0);
+  lookups(1);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int i = 12; i < 16; ++i) issue_k(i);
   __builtin_amdgcn_sched_barrier(0);
   TQ_STAMP(7);
-
-  // ---- scores, tile by tile as K arrives ----------------------------------------------------------------
-  float s[4][4];
-  {
-    u4* kst = reinterpret_cast<u4*>(stage);                           // 256 pieces of 16 bytes
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-#pragma unroll
-      for (int ii = 0; ii < 4; ++ii) kst[ii * 64 + lane] = kreg[4 * t + ii];
-      f4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int kb = 0; kb < 4; ++kb) {
-        const u4 ka = kst[n16 * 16 + ((4 * kb + g) ^ (n16 & 7))];     // piece 4kb+g of row n16
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, ka), __builtin_bit_cast(h8, qreg[kb]),
-                                                     acc, 0, 0, 0);
-      }
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int row = wrow0 + 16 * t + 4 * g + j;                    // accumulator row 4g + j of tile t
-        float v = acc[j] * a.attn_scale;
-        if (a.mask && row < rows_here && n16 < n_rep)
-          v += a.mask[(int64_t)seq * a.mask_seq_stride + ((int64_t)kvh * n_rep + n16) * a.mask_head_stride +
-                      tile_p0 + row];
-        s[t][j] = (row < rows_here) ? v : -INFINITY;
-      }
-    }
-  }
+  qk_tile(1);
+  qk_tile(2);
+  qk_tile(3);
   TQ_STAMP(2);
 
   // ---- softmax statistics of head n16 over the wave's 64 positions ----------------------------------
@@ -336,53 +341,47 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
   }
   TQ_STAMP(3);
 
-  // ---- merge the eight waves ---------------------------------------------------------------------------
+  // ---- merge the eight waves: one barrier ------------------------------------------------------------
+  // Every wave deposits its unscaled accumulator rows together with (m, l, 2^k scale); the
+  // cooperative sum below rescales while it adds.  Eight query heads fit the 32 KB buffer per round.
+  float (*S_all)[8][kD] = reinterpret_cast<float (*)[8][kD]>(big_s);    // [wave][head in round][128]
+  const int64_t grp = (int64_t)seq * a.n_kv + kvh;
+  float* pS = a.ws_S + (grp * a.n_tiles_max + tile) * (int64_t)(n_rep * kD);
+  float* pml = a.ws_ml + (grp * a.n_tiles_max + tile) * (int64_t)(n_rep * 2);
   if (g == 0) {
     m_s[wave][n16] = m;
     l_s[wave][n16] = l;
   }
-  __syncthreads();                                       // also: every wave is done with its staging area
-  TQ_STAMP(8);
-  float (*S_s)[kHeadsMax][kD] = reinterpret_cast<float (*)[kHeadsMax][kD]>(big_s);   // [4][16][128]
-  float alpha[4];
+  if (lane == 0) t_s[wave] = inv_tscale;
+  for (int h0 = 0; h0 < n_rep; h0 += 8) {
+    __syncthreads();                                     // staging area (or the previous round) is free
+    if ((g >> 1) == (h0 >> 3)) {                         // lanes whose rows 4g+j fall in this round
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int h = 4 * g + j;                             // accumulator row -> head
-    float M = m_s[0][h];
+      for (int j = 0; j < 4; ++j) {
+        float4* dst = reinterpret_cast<float4*>(&S_all[wave][(4 * g + j) & 7][8 * n16]);
+        dst[0] = make_float4(accS[0][j], accS[1][j], accS[2][j], accS[3][j]);
+        dst[1] = make_float4(accS[4][j], accS[5][j], accS[6][j], accS[7][j]);
+      }
+    }
+    __syncthreads();
+    TQ_STAMP(8);
+    const int rows = min(8, n_rep - h0);
+    for (int i = tid; i < rows * kD; i += kMfmaThreads) {
+      const int hl = i >> 7, e = i & 127, h = h0 + hl;
+      float M = m_s[0][h];
 #pragma unroll
-    for (int w = 1; w < kWaves; ++w) M = fmaxf(M, m_s[w][h]);
-    const float mw = m_s[wave][h];
-    alpha[j] = (mw == -INFINITY) ? 0.0f : __expf(mw - M) * inv_tscale;
-  }
-  if (wave >= 4) {
+      for (int w = 1; w < kWaves; ++w) M = fmaxf(M, m_s[w][h]);
+      float sum = 0.0f;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      float4* dst = reinterpret_cast<float4*>(&S_s[wave - 4][4 * g + j][8 * n16]);
-      dst[0] = make_float4(accS[0][j] * alpha[j], accS[1][j] * alpha[j], accS[2][j] * alpha[j], accS[3][j] * alpha[j]);
-      dst[1] = make_float4(accS[4][j] * alpha[j], accS[5][j] * alpha[j], accS[6][j] * alpha[j], accS[7][j] * alpha[j]);
+      for (int w = 0; w < kWaves; ++w) {
+        const float mw = m_s[w][h];
+        const float f = (mw == -INFINITY) ? 0.0f : __expf(mw - M) * t_s[w];
+        sum += f * S_all[w][hl][e];
+      }
+      pS[h * kD + e] = sum;
     }
   }
-  __syncthreads();
-  if (wave < 4) {                                        // same lanes, same addresses as wave + 4 used
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      float4* dst = reinterpret_cast<float4*>(&S_s[wave][4 * g + j][8 * n16]);
-      const float4 a0 = dst[0], a1 = dst[1];
-      dst[0] = make_float4(accS[0][j] * alpha[j] + a0.x, accS[1][j] * alpha[j] + a0.y,
-                           accS[2][j] * alpha[j] + a0.z, accS[3][j] * alpha[j] + a0.w);
-      dst[1] = make_float4(accS[4][j] * alpha[j] + a1.x, accS[5][j] * alpha[j] + a1.y,
-                           accS[6][j] * alpha[j] + a1.z, accS[7][j] * alpha[j] + a1.w);
-    }
-  }
-  __syncthreads();
   TQ_STAMP(9);
-  const int64_t grp = (int64_t)seq * a.n_kv + kvh;
-  float* pS = a.ws_S + (grp * a.n_tiles_max + tile) * (int64_t)(n_rep * kD);
-  float* pml = a.ws_ml + (grp * a.n_tiles_max + tile) * (int64_t)(n_rep * 2);
-  for (int i = tid; i < n_rep * kD; i += kMfmaThreads) {
-    const int h = i >> 7, e = i & 127;
-    pS[i] = (S_s[0][h][e] + S_s[1][h][e]) + (S_s[2][h][e] + S_s[3][h][e]);
-  }
   if (tid < n_rep) {
     const int h = tid;
     float M = m_s[0][h];
