@@ -118,12 +118,15 @@ int tq_prerotate_query(const void* q, int q_dtype, const float* signs, float* q_
  * Replaces prerot_fused_qk_scores (metal_kernels_v4.py:153-221, kernel 71-113).
  *   q_rot [n_kv*n_rep, dim] f32; k_packed / k_norms: one sequence, head_stride in rows;
  *   scores [n_kv*n_rep, seq_len] f32 contiguous.
+ * allow_mma = 0: float32 arithmetic throughout (the reference's numerics); 1: q_rot and the
+ * centroids are rounded to fp16 and multiplied on the matrix cores with float32 accumulation
+ * (about 3e-4 relative per score) where the shape allows (d = 128, 3-bit, n_rep <= 16).
  */
 int tq_prerot_qk_scores(const float* q_rot, const uint32_t* k_packed, const float* k_norms,
                         const float* centroids, float* scores,
                         int n_kv_heads, int n_rep, int64_t seq_len,
                         int64_t packed_head_stride, int64_t norms_head_stride,
-                        int dim, int bits, tq_stream_t stream);
+                        int dim, int bits, int allow_mma, tq_stream_t stream);
 
 /*
  * scores[h, p] = <dequant(K[h, p]), query[h]>, one butterfly per K row (MHA only).
@@ -161,13 +164,14 @@ int tq_softmax_rows(const float* scores, const float* mask, int64_t mask_row_str
  * Replaces sparse_v_matvec (sparse_v.py:94-186, kernel 32-88).  KV positions are split
  * across workgroups; partial sums go through `workspace` and a second pass applies the one
  * butterfly.   weights [n_kv*n_rep, seq_len] f32; out [n_kv*n_rep, dim] f32.
+ * allow_mma as in tq_prerot_qk_scores (weights * norm and centroids rounded to fp16).
  */
 int tq_sparse_v_matvec(const float* weights, const uint32_t* v_packed, const float* v_norms,
                        const float* centroids, const float* signs, float* out,
                        void* workspace, size_t workspace_bytes,
                        int n_kv_heads, int n_rep, int64_t seq_len,
                        int64_t packed_head_stride, int64_t norms_head_stride,
-                       int dim, int bits, float threshold, tq_stream_t stream);
+                       int dim, int bits, float threshold, int allow_mma, tq_stream_t stream);
 
 /* Shapes and addressing shared by the two fused decode-attention entry points. */
 typedef struct tq_decode_shape {
@@ -187,7 +191,10 @@ typedef struct tq_decode_shape {
   int64_t mask_seq_stride;   /* floats between sequences */
   int64_t mask_head_stride;  /* floats between query heads (0 = shared) */
   float attn_scale;
-  int32_t out_dtype;         /* TQ_F32 or TQ_F16 */
+  int32_t out_dtype;         /* TQ_F32, TQ_F16 or TQ_BF16 */
+  int32_t allow_mma;         /* 1: use the fp16 matrix-core kernels where the shape allows (d = 128,
+                                3-bit, n_rep <= 16; operands rounded to fp16, float32 accumulation);
+                                0: float32 vector-ALU kernels only */
 } tq_decode_shape;
 
 /*

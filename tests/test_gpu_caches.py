@@ -273,8 +273,8 @@ def test_turboquant_attention_masks_and_v_buffer(tq):
     rng = np.random.default_rng(0)
     m4 = torch.from_numpy(np.where(rng.random((B, 1, 1, S)) < 0.3, -np.inf, 0).astype(F32)).cuda()
     a = tq.turboquant_attention(q, cache, sc, mask=m4)
-    b = tq.turboquant_attention(q, cache, sc, mask=m4, fused=True)
-    assert np.abs(host(a) - host(b)).max() < 1e-4
+    b = tq.turboquant_attention(q, cache, sc, mask=m4, fused=True)      # fp16 matrix-core kernel
+    assert (np.abs(host(a) - host(b)) <= 1e-3 + 2e-3 * np.abs(host(a))).all()
     kp, kn, vp, vn = [t.cpu().numpy() for t in cache.state]
     c = o.gaussian_codebook(3)
     for i in range(B):

@@ -39,9 +39,14 @@ def tables(bits):
     return c, o.gaussian_boundaries(c)
 
 
-def close(got, want, rel=REL, abs_=ABS):
+def close(got, want, rel=REL, abs_=ABS, row_scale=False):
+    """|err| <= abs + rel * |want| elementwise; with row_scale the relative part is taken against the
+    largest magnitude of the output row (the reference's own measure, tests/test_flash_attention.py:
+    max_abs / max_ref), which is the meaningful one when an outlier channel dominates a row: the
+    Hadamard mixing spreads any operand rounding over all elements of the row."""
     err = np.abs(got.astype(np.float64) - want.astype(np.float64))
-    ok = err <= abs_ + rel * np.abs(want)
+    ref = np.abs(want).max(axis=-1, keepdims=True) if row_scale else np.abs(want)
+    ok = err <= abs_ + rel * ref
     assert ok.all(), f"max err {err.max():.3e} (want scale {np.abs(want).max():.3e}), {(~ok).sum()} bad"
 
 
@@ -497,3 +502,73 @@ def test_config3_scores(tq, T):
                                     host(gn).reshape(n_kv, T), c, D, bits, n_rep)
     assert got.shape == (28, T) and got.dtype == F32
     close(got, want, rel=1e-4, abs_=1e-4)
+
+
+# ------------------------------------------------------------------ fp16 matrix-core variants vs float32
+
+@pytest.mark.parametrize("n_kv,n_rep,T", [(4, 7, 2000), (8, 4, 513), (2, 16, 700), (1, 1, 64)])
+def test_scores_and_sparse_v_fp16_paths(tq, n_kv, n_rep, T):
+    """precision="fp16": operands rounded to half, float32 accumulation.  Scores within 2e-3 of the
+    score scale, sparse-V within the attention bar; precision="fp32" stays at 1e-5."""
+    rng = np.random.default_rng(21)
+    D, bits = 128, 3
+    c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, n_kv, T, D, bits)
+    q = rng.standard_normal((n_kv * n_rep, D)).astype(F32)
+    q_rot = tq.prerotate_query(dev(q), dev(ks))
+    want = o.prerot_fused_qk_scores(o.prerotate_query(q, ks), kp, kn, c, D, bits, n_rep)
+    s16 = host(tq.prerot_fused_qk_scores(q_rot, dev(kp), dev(kn), c, D, bits, n_rep=n_rep, precision="fp16"))
+    s32 = host(tq.prerot_fused_qk_scores(q_rot, dev(kp), dev(kn), c, D, bits, n_rep=n_rep, precision="fp32"))
+    scale = np.abs(want).max()
+    assert np.abs(s32 - want).max() < 1e-5 * scale
+    assert np.abs(s16 - want).max() < 2e-3 * scale
+    w = softmax_np(want / math.sqrt(D))
+    for thr in (0.0, 1e-4):
+        ws = o.sparse_v_matvec(w, vp, vn, c, vs, D, bits, thr, n_rep)
+        g16 = host(tq.sparse_v_matvec(dev(w), dev(vp), dev(vn), c, dev(vs), D, bits, threshold=thr, n_rep=n_rep,
+                                      precision="fp16"))
+        close(g16, ws)
+    z = host(tq.sparse_v_matvec(dev(w), dev(vp), dev(vn), c, dev(vs), D, bits, threshold=2.0, n_rep=n_rep,
+                                precision="fp16"))
+    assert (z == 0).all()
+    with pytest.raises(ValueError, match="precision"):
+        tq.sparse_v_matvec(dev(w), dev(vp), dev(vn), c, dev(vs), D, bits, n_rep=n_rep, precision="bf16")
+
+
+@pytest.mark.parametrize("precision", ["fp16", "fp32"])
+def test_flash_and_vonly_both_precisions(tq, precision):
+    rng = np.random.default_rng(22)
+    n_kv, n_rep, T, D, bits = 4, 7, 3000, 128, 3
+    c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, n_kv, T, D, bits, outliers=True)
+    q = rng.standard_normal((n_kv * n_rep, D)).astype(np.float16)
+    sc = 1 / math.sqrt(D)
+    q_rot = tq.prerotate_query(dev(q), dev(ks))
+    got = host(tq.flash_attention_turboquant(q_rot, dev(kp), dev(kn), dev(vp), dev(vn), c, c, dev(vs), D, bits, sc,
+                                             n_rep=n_rep, precision=precision))
+    want = o.flash_attention_turboquant(o.prerotate_query(q, ks), kp, kn, vp, vn, c, c, vs, D, bits, sc, 16, n_rep)
+    close(got, want, row_scale=True)                    # outlier channels: rows span 0.01 .. 17
+    err = np.abs(got - want).max() / np.abs(want).max()
+    assert err < (1e-3 if precision == "fp16" else 1e-5), err
+    got = host(tq.vonly_decode(dev(q[None]), dev(K), dev(vp), dev(vn), c, dev(vs), D, bits, sc, n_rep=n_rep,
+                               precision=precision))[0]
+    close(got, o.vonly_decode_attention(q, K, vp, vn, c, vs, D, bits, sc), row_scale=True)
+
+
+def test_config4_flash_ragged_full_heads(tq):
+    """BASELINE config 4 shape (scaled in length): 32 q / 8 kv heads, 16 sequences of ragged length,
+    fp16 output, packed K and V."""
+    rng = np.random.default_rng(4)
+    n_kv, n_rep, D, bits, n_seq = 8, 4, 128, 3, 16
+    lens = rng.integers(300, 2100, size=n_seq)
+    offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, n_kv, int(offs[-1]), D, bits)
+    q = rng.standard_normal((n_seq, n_kv * n_rep, D)).astype(np.float16)
+    sc = 1 / math.sqrt(D)
+    q_rot = tq.prerotate_query(dev(q.reshape(-1, D)), dev(ks)).reshape(n_seq, n_kv * n_rep, D)
+    got = host(tq.flash_decode(q_rot, dev(kp), dev(kn), dev(vp), dev(vn), c, c, dev(vs), D, bits, sc, n_rep=n_rep,
+                               seq_offsets=dev(offs), max_seq_len=int(lens.max()),
+                               out_dtype=torch.float16)).astype(F32)
+    for i in range(n_seq):
+        a, e = offs[i], offs[i + 1]
+        want = o.flash_attention_turboquant(o.prerotate_query(q[i], ks), kp[:, a:e], kn[:, a:e], vp[:, a:e],
+                                            vn[:, a:e], c, c, vs, D, bits, sc, 16, n_rep)
+        close(got[i], want)

@@ -30,8 +30,8 @@ def test_library_exports_every_declared_symbol():
 
 
 def test_decode_shape_struct_matches_header_size():
-    # 6 int32 + int64 + ptr + 8 int64 + ptr + 2 int64 + float + int32
-    assert ctypes.sizeof(_lib.DecodeShape) == 6 * 4 + 8 + 8 + 8 * 8 + 8 + 2 * 8 + 4 + 4
+    # 6 int32 + int64 + ptr + 8 int64 + ptr + 2 int64 + float + 2 int32 (+ 4 bytes tail padding)
+    assert ctypes.sizeof(_lib.DecodeShape) == 6 * 4 + 8 + 8 + 8 * 8 + 8 + 2 * 8 + 4 + 4 + 4 + 4
 
 
 def test_argument_errors_without_launch():
@@ -45,8 +45,8 @@ def test_argument_errors_without_launch():
     assert lib.tq_encode(null, 7, null, b, null, null, 1, 4, 0, 0, 128, 3, 0, null) == -6
     assert lib.tq_encode(null, 1, null, b, null, null, 1, 4, 0, 0, 128, 3, 0, null) == -1
     assert lib.tq_encode(null, 1, null, b, null, null, 0, 4, 0, 0, 128, 3, 0, null) == 0   # empty: no-op
-    assert lib.tq_prerot_qk_scores(null, null, null, b, null, 4, 0, 16, 0, 0, 128, 3, null) == -4
-    assert lib.tq_sparse_v_matvec(null, null, null, b, null, null, null, 0, 4, 7, 16, 0, 0, 512, 3, 0.0, null) == -2
+    assert lib.tq_prerot_qk_scores(null, null, null, b, null, 4, 0, 16, 0, 0, 128, 3, 0, null) == -4
+    assert lib.tq_sparse_v_matvec(null, null, null, b, null, null, null, 0, 4, 7, 16, 0, 0, 512, 3, 0.0, 0, null) == -2
     assert b"dim > 256" in lib.tq_last_error()
     sh = _lib.DecodeShape()
     sh.n_seq, sh.n_kv_heads, sh.n_rep, sh.dim, sh.bits, sh.block_size, sh.seq_len = 1, 2, 1, 128, 3, 33, 8

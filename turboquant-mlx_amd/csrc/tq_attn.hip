@@ -8,8 +8,12 @@
 // signs and the 1/dim factor.
 #include "tq_common.h"
 #include "tq_decode_mfma.h"
+#include "tq_packed_mfma.h"
 
 #include <math.h>
+#include <cmath>
+#include <cstring>
+#include <mutex>
 
 namespace {
 
@@ -359,46 +363,79 @@ __global__ __launch_bounds__(kThreads) void decode_tile_kernel(DecodeArgs a, Cod
 }
 
 // ---------------------------------------------------------------- merge pass
-// grid = (n_q, n_seq), one wavefront each.
+// grid = (n_q, n_seq), 256 threads.  Lane group ph = tid / (D/4) folds tiles ph, ph + P, ... (4
+// elements per lane, P = 1024 / D groups) -- with a running maximum for the softmax modes, a plain
+// sum for given weights -- the groups are combined through LDS in a fixed order and wave 0 applies
+// the one butterfly, the signs, 1/dim (and 1/l).
 template <int D, int KMODE, typename TO>
-__global__ __launch_bounds__(TQ_WAVE) void decode_merge_kernel(const float* __restrict__ ws_S,
-                                                               const float* __restrict__ ws_ml,
-                                                               const int32_t* __restrict__ seq_offsets,
-                                                               int64_t seq_len, int n_tiles_max,
-                                                               const float* __restrict__ signs, float inv_dim,
-                                                               TO* __restrict__ out) {
+__global__ __launch_bounds__(kThreads) void decode_merge_kernel(const float* __restrict__ ws_S,
+                                                                const float* __restrict__ ws_ml,
+                                                                const int32_t* __restrict__ seq_offsets,
+                                                                int64_t seq_len, int n_tiles_max,
+                                                                const float* __restrict__ signs, float inv_dim,
+                                                                TO* __restrict__ out) {
   constexpr int EPL = Lay<D>::EPL;
-  const int lane = threadIdx.x;
+  constexpr int LPG = D / 4;                 // lanes per group
+  constexpr int P = kThreads / LPG;          // groups
+  typedef float f4 __attribute__((ext_vector_type(4)));
+  __shared__ __align__(16) float acc_s[P][D];
+  __shared__ float ml_s[P][2];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int eq = tid % LPG, ph = tid / LPG;
   const int64_t row = (int64_t)blockIdx.y * gridDim.x + blockIdx.x;
   int64_t first, len;
   seq_range(seq_offsets, seq_len, blockIdx.y, first, len);
   const int n_tiles = (int)((len + kTile - 1) / kTile);
-  const float* S = ws_S + row * n_tiles_max * D;
+  const float* S = ws_S + row * n_tiles_max * D + 4 * eq;
   const float* ml = ws_ml + row * n_tiles_max * 2;
+  float M = -INFINITY, L = 0.0f;
+  f4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int t0 = ph; t0 < n_tiles; t0 += 4 * P) {
+    f4 x[4];
+    float2 st[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int t = min(t0 + u * P, n_tiles - 1);
+      x[u] = *reinterpret_cast<const f4*>(S + (int64_t)t * D);
+      st[u] = (KMODE == kWeights) ? make_float2(0.f, 0.f) : *reinterpret_cast<const float2*>(ml + 2 * t);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (t0 + u * P >= n_tiles) continue;
+      if (KMODE == kWeights) {
+        acc += x[u];
+      } else if (st[u].x != -INFINITY) {
+        const float Mn = fmaxf(M, st[u].x);
+        const float fo = (M == -INFINITY) ? 0.0f : expf(M - Mn);
+        const float fc = expf(st[u].x - Mn);
+        acc = acc * fo + x[u] * fc;
+        L = L * fo + st[u].y * fc;
+        M = Mn;
+      }
+    }
+  }
+  *reinterpret_cast<f4*>(&acc_s[ph][4 * eq]) = acc;
+  if (eq == 0) { ml_s[ph][0] = M; ml_s[ph][1] = L; }
+  __syncthreads();
+  if (tid >= TQ_WAVE) return;
+  float Mt = -INFINITY, Lt = 1.0f;
   float v[EPL];
 #pragma unroll
   for (int i = 0; i < EPL; ++i) v[i] = 0.0f;
-  float L = 1.0f;
-  if (KMODE == kWeights) {
-    for (int t = 0; t < n_tiles; ++t)
+  if (KMODE != kWeights) {
+    for (int p = 0; p < P; ++p) Mt = fmaxf(Mt, ml_s[p][0]);
+    Lt = 0.0f;
+  }
+  for (int p = 0; p < P; ++p) {
+    float f = 1.0f;
+    if (KMODE != kWeights) {
+      f = (ml_s[p][0] == -INFINITY) ? 0.0f : expf(ml_s[p][0] - Mt);
+      Lt += f * ml_s[p][1];
+    }
 #pragma unroll
-      for (int i = 0; i < EPL; ++i) {
-        const int e = lane + 64 * i;
-        if (e < D) v[i] += S[(int64_t)t * D + e];
-      }
-  } else {
-    float M = -INFINITY;
-    for (int t = 0; t < n_tiles; ++t) M = fmaxf(M, ml[2 * t]);
-    L = 0.0f;
-    for (int t = 0; t < n_tiles; ++t) {
-      const float mt = ml[2 * t];
-      const float alpha = (mt == -INFINITY) ? 0.0f : expf(mt - M);
-      L += alpha * ml[2 * t + 1];
-#pragma unroll
-      for (int i = 0; i < EPL; ++i) {
-        const int e = lane + 64 * i;
-        if (e < D) v[i] += alpha * S[(int64_t)t * D + e];
-      }
+    for (int i = 0; i < EPL; ++i) {
+      const int e = lane + 64 * i;
+      if (e < D) v[i] += f * acc_s[p][e];
     }
   }
   raw_butterfly<D>(v, lane);
@@ -407,7 +444,7 @@ __global__ __launch_bounds__(TQ_WAVE) void decode_merge_kernel(const float* __re
     const int e = lane + 64 * i;
     if (e < D) {
       float o = (v[i] * signs[e]) * inv_dim;
-      if (KMODE != kWeights) o = (L > 0.0f) ? o / L : 0.0f;
+      if (KMODE != kWeights) o = (Lt > 0.0f) ? o / Lt : 0.0f;
       store_from_float<TO>(out + row * D + e, o);
     }
   }
@@ -424,6 +461,44 @@ size_t ws_bytes(int n_seq, int n_q, int64_t max_len, int dim) {
 
 void fill_codebook(Codebook& cb, const float* c, int bits) {
   for (int i = 0; i < 16; ++i) cb.c[i] = (c && i < (1 << bits)) ? c[i] : 0.0f;
+}
+
+// The matrix-core kernels hold the codebook as fp16.  Rounding the 2^bits levels to fp16 is a
+// systematic error (the same few values at every position, so it does not average out over a
+// sequence); multiplying the table by a scale a in [1, 2) first and dividing the result by a
+// afterwards (in float32) leaves the mathematics alone, and a can be chosen so that every a*c[i]
+// lies within a few 2^-16 of an fp16 value.  Returns 1/a; the search result is kept for the last
+// table seen.
+float fill_codebook_fp16(Codebook& cb, const float* c, int bits) {
+  static std::mutex mu;
+  static float last_c[16], last_scale = 0.0f;
+  static int last_n = 0;
+  const int n = 1 << bits;
+  float scale = 1.0f;
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    if (last_n == n && last_scale != 0.0f && std::memcmp(last_c, c, n * sizeof(float)) == 0) {
+      scale = last_scale;
+    } else {
+      double best = 1e30;
+      for (int j = 0; j < 65536; ++j) {
+        const float a = 1.0f + (float)j * (1.0f / 65536.0f);
+        double worst = 0.0;
+        for (int i = 0; i < n && worst < best; ++i) {
+          const float v = a * c[i];
+          if (v == 0.0f) continue;
+          const float r = (float)(_Float16)v;
+          worst = std::fmax(worst, std::fabs(((double)r - (double)v) / (double)v));
+        }
+        if (worst < best) { best = worst; scale = a; }
+      }
+      std::memcpy(last_c, c, n * sizeof(float));
+      last_n = n;
+      last_scale = scale;
+    }
+  }
+  for (int i = 0; i < 16; ++i) cb.c[i] = (i < n) ? scale * c[i] : 0.0f;
+  return 1.0f / scale;
 }
 
 int check_heads(int n_kv, int n_rep, const char* who) {
@@ -481,7 +556,7 @@ int launch_decode(const void* q, int q_dtype, const uint32_t* k_packed, const fl
   if (!(phases & 2)) return TQ_OK;
   dim3 mgrid(n_q, sh.n_seq);
 #define LAUNCH_MERGE(TO)                                                                              \
-  TQ_DISPATCH_DIM(sh.dim, (decode_merge_kernel<D_, KMODE, TO><<<mgrid, TQ_WAVE, 0, stream>>>(          \
+  TQ_DISPATCH_DIM(sh.dim, (decode_merge_kernel<D_, KMODE, TO><<<mgrid, kThreads, 0, stream>>>(         \
                               a.ws_S, a.ws_ml, sh.seq_offsets, sh.seq_len, n_tiles_max, v_signs,       \
                               a.inv_dim, (TO*)out)))
   if (sh.out_dtype == TQ_F16) { LAUNCH_MERGE(__half); }
@@ -524,7 +599,7 @@ int launch_vonly_mfma(const void* q, const void* k_f16, const uint32_t* v_packed
   }
 #endif
   Codebook vcb;
-  fill_codebook(vcb, v_centroids, sh.bits);
+  a.v_unscale = fill_codebook_fp16(vcb, v_centroids, sh.bits);
   if (phases & 1) {
     dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
     tqm::vonly_tile_mfma_kernel<<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb);
@@ -534,7 +609,7 @@ int launch_vonly_mfma(const void* q, const void* k_f16, const uint32_t* v_packed
   dim3 mgrid(n_q, sh.n_seq);
   const float inv_dim = 1.0f / (float)sh.dim;
 #define LAUNCH_MERGE_M(TO)                                                                                \
-  tqm::decode_merge_rows_kernel<TO><<<mgrid, tqm::kMergeThreads, 0, stream>>>(                              \
+  tqm::decode_merge_rows_kernel<TO, true><<<mgrid, tqm::kMergeThreads, 0, stream>>>(                        \
       a.ws_S, a.ws_ml, sh.seq_offsets, sh.seq_len, n_tiles, sh.n_kv_heads, sh.n_rep, v_signs, inv_dim, (TO*)out)
   if (sh.out_dtype == TQ_F16) { LAUNCH_MERGE_M(__half); }
   else if (sh.out_dtype == TQ_BF16) { LAUNCH_MERGE_M(__hip_bfloat16); }
@@ -542,6 +617,59 @@ int launch_vonly_mfma(const void* q, const void* k_f16, const uint32_t* v_packed
 #undef LAUNCH_MERGE_M
   TQ_CHECK_LAUNCH(who);
   return TQ_OK;
+}
+
+// Matrix-core path over packed keys/values: MODE = tqm::kFlash (tq_flash_decode) or tqm::kWeights
+// (tq_sparse_v_matvec): tile pass + merge pass.
+template <int MODE>
+int launch_packed_mfma(const float* q_rot_or_weights, const uint32_t* k_packed, const float* k_norms,
+                       const uint32_t* v_packed, const float* v_norms, const float* k_centroids,
+                       const float* v_centroids, const float* v_signs, void* out, void* workspace,
+                       size_t workspace_bytes, const tq_decode_shape& sh, float threshold, hipStream_t stream,
+                       const char* who) {
+  const int n_q = sh.n_kv_heads * sh.n_rep;
+  const int n_tiles = (int)((sh.seq_len + tqm::kTilePos - 1) / tqm::kTilePos);
+  const size_t need = (size_t)sh.n_seq * n_q * n_tiles * (tqm::kD + 2) * sizeof(float);
+  if (!workspace || workspace_bytes < need)
+    return tq::fail(TQ_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, need, workspace_bytes);
+  if (!tq::aligned(workspace, 16)) return tq::fail(TQ_ERR_ALIGN, "%s: workspace must be 16-byte aligned", who);
+  tqm::PackedArgs a{};
+  if (MODE == tqm::kWeights) a.weights = q_rot_or_weights; else a.q_rot = q_rot_or_weights;
+  a.k_packed = k_packed; a.k_norms = k_norms; a.v_packed = v_packed; a.v_norms = v_norms;
+  a.seq_offsets = sh.seq_offsets; a.mask = sh.mask;
+  a.ws_S = (float*)workspace;
+  a.ws_ml = a.ws_S + (size_t)sh.n_seq * n_q * n_tiles * tqm::kD;
+  a.seq_len = sh.seq_len;
+  a.k_seq_stride = sh.k_seq_stride; a.k_head_stride = sh.k_head_stride;
+  a.kn_seq_stride = sh.kn_seq_stride; a.kn_head_stride = sh.kn_head_stride;
+  a.v_seq_stride = sh.v_seq_stride; a.v_head_stride = sh.v_head_stride;
+  a.vn_seq_stride = sh.vn_seq_stride; a.vn_head_stride = sh.vn_head_stride;
+  a.mask_seq_stride = sh.mask_seq_stride; a.mask_head_stride = sh.mask_head_stride;
+  a.n_kv = sh.n_kv_heads; a.n_rep = sh.n_rep; a.n_tiles_max = n_tiles;
+  a.score_scale = sh.attn_scale / (float)sh.dim;
+  a.threshold = threshold;
+  Codebook kcb, vcb;
+  fill_codebook(kcb, nullptr, sh.bits);
+  if (MODE != tqm::kWeights) a.score_scale *= fill_codebook_fp16(kcb, k_centroids, sh.bits);
+  a.v_unscale = fill_codebook_fp16(vcb, v_centroids, sh.bits);
+  dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
+  tqm::packed_tile_mfma_kernel<MODE><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, kcb, vcb);
+  TQ_CHECK_LAUNCH(who);
+  dim3 mgrid(n_q, sh.n_seq);
+  const float inv_dim = 1.0f / (float)sh.dim;
+#define LAUNCH_MERGE_P(TO)                                                                                    \
+  tqm::decode_merge_rows_kernel<TO, MODE == tqm::kFlash><<<mgrid, tqm::kMergeThreads, 0, stream>>>(            \
+      a.ws_S, a.ws_ml, sh.seq_offsets, sh.seq_len, n_tiles, sh.n_kv_heads, sh.n_rep, v_signs, inv_dim, (TO*)out)
+  if (sh.out_dtype == TQ_F16) { LAUNCH_MERGE_P(__half); }
+  else if (sh.out_dtype == TQ_BF16) { LAUNCH_MERGE_P(__hip_bfloat16); }
+  else { LAUNCH_MERGE_P(float); }
+#undef LAUNCH_MERGE_P
+  TQ_CHECK_LAUNCH(who);
+  return TQ_OK;
+}
+
+bool mma_shape(const tq_decode_shape& sh) {
+  return sh.allow_mma && sh.dim == 128 && sh.bits == 3 && sh.n_rep <= tqm::kHeadsMax && sh.seq_len > 0;
 }
 
 int check_shape(const tq_decode_shape* sh, const char* who, int max_dim) {
@@ -573,7 +701,7 @@ extern "C" size_t tq_workspace_bytes(int op, int n_seq, int n_q_heads, int64_t m
 extern "C" int tq_prerot_qk_scores(const float* q_rot, const uint32_t* k_packed, const float* k_norms,
                                    const float* centroids, float* scores, int n_kv_heads, int n_rep,
                                    int64_t seq_len, int64_t packed_head_stride, int64_t norms_head_stride,
-                                   int dim, int bits, tq_stream_t stream_) {
+                                   int dim, int bits, int allow_mma, tq_stream_t stream_) {
   if (int rc = tq::check_dim_bits(dim, bits)) return rc;
   if (int rc = check_heads(n_kv_heads, n_rep, "tq_prerot_qk_scores")) return rc;
   if (seq_len < 0) return tq::fail(TQ_ERR_ARG, "tq_prerot_qk_scores: negative seq_len");
@@ -582,6 +710,18 @@ extern "C" int tq_prerot_qk_scores(const float* q_rot, const uint32_t* k_packed,
     return tq::fail(TQ_ERR_NULL, "tq_prerot_qk_scores: null pointer");
   Codebook cb;
   fill_codebook(cb, centroids, bits);
+  if (allow_mma && dim == 128 && bits == 3 && n_rep <= tqm::kHeadsMax && tq::aligned(q_rot, 8)) {
+    tqm::PackedArgs a{};
+    a.q_rot = q_rot; a.k_packed = k_packed; a.k_norms = k_norms; a.scores = scores;
+    a.seq_len = seq_len; a.k_head_stride = packed_head_stride; a.kn_head_stride = norms_head_stride;
+    a.n_kv = n_kv_heads; a.n_rep = n_rep; a.n_tiles_max = 1;
+    Codebook cbh;
+    a.score_scale = fill_codebook_fp16(cbh, centroids, bits) / (float)dim;
+    dim3 grid((unsigned)((seq_len + tqm::kTilePos - 1) / tqm::kTilePos), n_kv_heads, 1);
+    tqm::packed_tile_mfma_kernel<tqm::kScores><<<grid, tqm::kMfmaThreads, 0, (hipStream_t)stream_>>>(a, cbh, cbh);
+    TQ_CHECK_LAUNCH("tq_prerot_qk_scores launch");
+    return TQ_OK;
+  }
   const int n_rgroups = (n_rep + kRMax - 1) / kRMax;
   dim3 grid(n_tiles_for(seq_len), n_kv_heads * n_rgroups);
   hipStream_t stream = (hipStream_t)stream_;
@@ -634,7 +774,7 @@ extern "C" int tq_sparse_v_matvec(const float* weights, const uint32_t* v_packed
                                   const float* centroids, const float* signs, float* out, void* workspace,
                                   size_t workspace_bytes, int n_kv_heads, int n_rep, int64_t seq_len,
                                   int64_t packed_head_stride, int64_t norms_head_stride, int dim, int bits,
-                                  float threshold, tq_stream_t stream_) {
+                                  float threshold, int allow_mma, tq_stream_t stream_) {
   if (!tq::is_pow2(dim)) return tq::fail(TQ_ERR_DIM, "dim must be a power of 2, got %d", dim);
   if (dim > 256) return tq::fail(TQ_ERR_DIM, "dim > 256 not supported by threadgroup layout, got %d", dim);
   tq_decode_shape sh{};
@@ -647,6 +787,11 @@ extern "C" int tq_sparse_v_matvec(const float* weights, const uint32_t* v_packed
   if (seq_len > 0 && (!weights || !v_packed || !v_norms))
     return tq::fail(TQ_ERR_NULL, "tq_sparse_v_matvec: null pointer");
   const float thr = threshold > 0.0f ? threshold : 0.0f;
+  sh.allow_mma = allow_mma;
+  if (mma_shape(sh))
+    return launch_packed_mfma<tqm::kWeights>(weights, nullptr, nullptr, v_packed, v_norms, centroids, centroids,
+                                             signs, out, workspace, workspace_bytes, sh, thr,
+                                             (hipStream_t)stream_, "tq_sparse_v_matvec");
   return launch_decode<kWeights>(weights, TQ_F32, nullptr, nullptr, nullptr, v_packed, v_norms, nullptr,
                                  centroids, signs, out, workspace, workspace_bytes, sh, thr,
                                  (hipStream_t)stream_, "tq_sparse_v_matvec");
@@ -661,6 +806,10 @@ extern "C" int tq_flash_decode(const float* q_rot, const uint32_t* k_packed, con
     return tq::fail(TQ_ERR_NULL, "tq_flash_decode: null pointer");
   if (shape->seq_len > 0 && (!k_packed || !k_norms || !v_packed || !v_norms))
     return tq::fail(TQ_ERR_NULL, "tq_flash_decode: null pointer");
+  if (mma_shape(*shape) && tq::aligned(q_rot, 8))
+    return launch_packed_mfma<tqm::kFlash>(q_rot, k_packed, k_norms, v_packed, v_norms, k_centroids, v_centroids,
+                                           v_signs, out, workspace, workspace_bytes, *shape, 0.0f,
+                                           (hipStream_t)stream_, "tq_flash_decode");
   return launch_decode<kPackedK>(q_rot, TQ_F32, k_packed, k_norms, nullptr, v_packed, v_norms, k_centroids,
                                  v_centroids, v_signs, out, workspace, workspace_bytes, *shape, 0.0f,
                                  (hipStream_t)stream_, "tq_flash_decode");
@@ -678,8 +827,7 @@ extern "C" int tq_vonly_decode_attn_phases(const void* q, int q_dtype, const voi
     return tq::fail(TQ_ERR_NULL, "tq_vonly_decode_attn: null pointer");
   if (!tq::aligned(k_f16, 16)) return tq::fail(TQ_ERR_ALIGN, "tq_vonly_decode_attn: k must be 16-byte aligned");
   // d = 128, 3-bit, fp16 queries, at most 16 query heads per kv head: matrix-core tile pass.
-  if (shape->dim == 128 && shape->bits == 3 && q_dtype == TQ_F16 && shape->n_rep <= tqm::kHeadsMax &&
-      tq::aligned(q, 4) && shape->seq_len > 0)
+  if (mma_shape(*shape) && q_dtype == TQ_F16 && tq::aligned(q, 4))
     return launch_vonly_mfma(q, k_f16, v_packed, v_norms, v_centroids, v_signs, out, workspace, workspace_bytes,
                              *shape, (hipStream_t)stream_, phases);
   return launch_decode<kDenseK>(q, q_dtype, nullptr, nullptr, k_f16, v_packed, v_norms, nullptr, v_centroids,

@@ -68,6 +68,7 @@ struct MfmaArgs {
   int64_t mask_seq_stride, mask_head_stride;
   int32_t n_kv, n_rep, n_tiles_max;
   float attn_scale;
+  float v_unscale;            // 1 / the scale the value table was multiplied by on the host
 #ifdef TQ_TRACE
   unsigned long long* trace;
 #endif
@@ -352,7 +353,7 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
     m_s[wave][n16] = m;
     l_s[wave][n16] = l;
   }
-  if (lane == 0) t_s[wave] = inv_tscale;
+  if (lane == 0) t_s[wave] = inv_tscale * a.v_unscale;
   for (int h0 = 0; h0 < n_rep; h0 += 8) {
     __syncthreads();                                     // staging area (or the previous round) is free
     if ((g >> 1) == (h0 >> 3)) {                         // lanes whose rows 4g+j fall in this round
@@ -398,8 +399,8 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
 
 // Merge pass: grid = (n_q, n_seq), 256 threads.  Lane group ph = tid / 32 folds tiles ph, ph + 8, ...
 // (4 elements per lane) with a running maximum; the 8 groups are then combined through LDS and wave 0
-// finishes the row.
-template <typename TO>
+// finishes the row.  NORM = false (given weights, all maxima zero) skips the division by l.
+template <typename TO, bool NORM>
 __global__ __launch_bounds__(kMergeThreads) void decode_merge_rows_kernel(
     const float* __restrict__ ws_S, const float* __restrict__ ws_ml, const int32_t* __restrict__ seq_offsets,
     int64_t seq_len, int n_tiles_max, int n_kv, int n_rep, const float* __restrict__ signs, float inv_dim,
@@ -461,7 +462,7 @@ __global__ __launch_bounds__(kMergeThreads) void decode_merge_rows_kernel(
   for (int i = 0; i < 2; ++i) {
     const int e = lane + 64 * i;
     float val = (v[i] * signs[e]) * inv_dim;
-    val = (Lt > 0.0f) ? val / Lt : 0.0f;
+    if (NORM) val = (Lt > 0.0f) ? val / Lt : 0.0f;
     store_from_float<TO>(o + e, val);
   }
 }

@@ -1,0 +1,384 @@
+// Matrix-core tile pass over PACKED keys and/or values (d = 128, 3-bit, n_rep <= 16).
+// Included by tq_attn.hip after tq_decode_mfma.h, whose conventions it shares: a workgroup of 8
+// waves owns 512 positions of one kv head, a wave 64 of them; partials go to the workspace and
+// the merge pass finishes.  Three modes:
+//
+//   kFlash    packed K and packed V: scores from the pre-rotated query, online-softmax partials
+//             (tq_flash_decode);
+//   kScores   packed K only: the scores themselves are the output (tq_prerot_qk_scores);
+//   kWeights  packed V only: the weights are given, positions below the threshold contribute
+//             nothing (tq_sparse_v_matvec).
+//
+// Packed rows are 52 bytes, so the wave's 64 rows of K (and of V) are one contiguous 3328-byte
+// block: 4 coalesced 16-byte loads per lane, copied into the wave's LDS area.  A lane then needs, per
+// row, the 24 bits holding 8 consecutive elements: two words, one shift-or.  For K the 8 elements
+// are 4 ADJACENT pairs, i.e. four contiguous 6-bit fields, each of which indexes the centroid-pair
+// table directly and yields one register of the A operand; for V two positions are interleaved
+// first (see tq_decode_mfma.h).  Scores are (sum_e c_k[idx] q_rot[e]) * k_norm * (1/d) [* scale].
+#pragma once
+
+#include "tq_decode_mfma.h"
+
+namespace tqm {
+
+enum PackedMode { kFlash = 0, kScores = 1, kWeights = 2 };
+
+struct PackedArgs {
+  const float* q_rot;         // kFlash / kScores: [n_seq, n_q, 128] f32
+  const float* weights;       // kWeights: [n_q, T] f32 (one sequence)
+  const uint32_t* k_packed;
+  const float* k_norms;
+  const uint32_t* v_packed;
+  const float* v_norms;
+  const int32_t* seq_offsets;
+  const float* mask;
+  float* scores;              // kScores: [n_q, T] f32
+  float* ws_S;
+  float* ws_ml;
+  int64_t seq_len;
+  int64_t k_seq_stride, k_head_stride, kn_seq_stride, kn_head_stride;
+  int64_t v_seq_stride, v_head_stride, vn_seq_stride, vn_head_stride;
+  int64_t mask_seq_stride, mask_head_stride;
+  int32_t n_kv, n_rep, n_tiles_max;
+  float score_scale;          // (1/d) * attn_scale for kFlash, 1/d for kScores; times 1/key-table scale
+  float v_unscale;            // 1 / the scale the value table was multiplied by on the host
+  float threshold;            // kWeights
+};
+
+// copy one wave's 64 packed rows (3328 bytes) from global memory into its LDS area
+struct PackedBlock {
+  u4 q[4];
+  uint32_t d[13];
+  bool wide;
+};
+
+__device__ __forceinline__ void load_block(PackedBlock& b, const uint32_t* block, int lane, int wrow0, int rows_here) {
+  b.wide = (wrow0 + kWavePos <= rows_here) && ((reinterpret_cast<uintptr_t>(block) & 15) == 0);
+  if (b.wide) {
+    const u4* b4 = reinterpret_cast<const u4*>(block);
+#pragma unroll
+    for (int i = 0; i < 3; ++i) b.q[i] = b4[i * 64 + lane];
+    b.q[3] = b4[192 + (lane & 15)];
+  } else {
+    const int valid_words = max(0, rows_here - wrow0) * kPdim;
+    const uint32_t* tile_base = block - (int64_t)wrow0 * kPdim;       // row 0 of the tile: always valid
+#pragma unroll
+    for (int i = 0; i < 13; ++i) {
+      const int w = i * 64 + lane;
+      b.d[i] = (w < valid_words) ? block[w] : tile_base[0];
+    }
+  }
+}
+
+__device__ __forceinline__ void stage_block(const PackedBlock& b, uint32_t* stage, int lane) {
+  if (b.wide) {
+    u4* st4 = reinterpret_cast<u4*>(stage);
+#pragma unroll
+    for (int i = 0; i < 3; ++i) st4[i * 64 + lane] = b.q[i];
+    if (lane < 16) st4[192 + lane] = b.q[3];
+  } else {
+#pragma unroll
+    for (int i = 0; i < 13; ++i) stage[i * 64 + lane] = b.d[i];
+  }
+}
+
+// word index / shifts of the 24 bits that hold elements 8*pc .. 8*pc+7 of a packed row
+__device__ __forceinline__ void piece_bits(int pc, int& w0, int& sh_lo, int& sh_hi) {
+  w0 = (pc == 15) ? 11 : (8 * pc) / 10;
+  const int s0 = (pc == 15) ? 10 : (8 * pc) % 10;
+  sh_lo = 3 * s0;
+  sh_hi = 30 - 3 * s0;
+}
+
+__device__ __forceinline__ void fill_lut(uint32_t* lut, const Codebook& cb, int tid) {
+  if (tid < 64) {
+    float clo = 0.0f, chi = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      clo = ((tid & 7) == i) ? cb.c[i] : clo;
+      chi = ((tid >> 3) == i) ? cb.c[i] : chi;
+    }
+    lut[tid] = pack_h2(clo, chi);
+  }
+}
+
+// grid = (n_tiles_max, n_kv, n_seq), 512 threads.
+template <int MODE>
+__global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(2, 4)))
+void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
+  constexpr bool HAS_K = MODE != kWeights;
+  constexpr bool HAS_V = MODE != kScores;
+  __shared__ __align__(16) unsigned char big_s[32768];      // per-wave 4 KB areas, later S_all[8][8][128]
+  __shared__ uint32_t lutk_s[64], lutv_s[64];
+  __shared__ __align__(16) uint32_t q_s[kHeadsMax][kD / 2];      // rotated queries as half2: rounded value ...
+  __shared__ __align__(16) uint32_t ql_s[kHeadsMax][kD / 2];     // ... and what the rounding lost
+  __shared__ __align__(16) float kn_s[kWaves][kWavePos], vn_s[kWaves][kWavePos];
+  __shared__ float m_s[kWaves][kHeadsMax], l_s[kWaves][kHeadsMax], t_s[kWaves];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int n16 = lane & 15, g = lane >> 4;
+  const int tile = blockIdx.x, kvh = blockIdx.y, seq = blockIdx.z;
+  const int n_rep = a.n_rep;
+  const int n_q = a.n_kv * n_rep;
+  const int64_t q_row0 = (int64_t)seq * n_q + (int64_t)kvh * n_rep;
+
+  int64_t first = 0, len = a.seq_len;
+  if (a.seq_offsets) {
+    first = a.seq_offsets[seq];
+    len = (int64_t)a.seq_offsets[seq + 1] - first;
+  }
+  const int64_t tile_p0 = (int64_t)tile * kTilePos;
+  if (tile_p0 >= len) return;
+  const int rows_here = (int)min((int64_t)kTilePos, len - tile_p0);
+  const int last_row = rows_here - 1;
+  const int wrow0 = wave * kWavePos;
+  int crow = wrow0 + lane;
+  crow = crow < last_row ? crow : last_row;                           // clamped row of this lane
+
+  // ---- loads ----------------------------------------------------------------------------------------
+  float2 my_q[2];
+  if (HAS_K) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int w = tid + i * kMfmaThreads;                           // word = 2 consecutive elements
+      my_q[i] = (w < n_rep * (kD / 2)) ? reinterpret_cast<const float2*>(a.q_rot + q_row0 * kD)[w]
+                                       : make_float2(0.f, 0.f);
+    }
+  }
+  float my_kn = 0.0f, my_vn = 0.0f;
+  PackedBlock kb_, vb_;
+  if (HAS_V) {
+    my_vn = a.v_norms[(int64_t)seq * a.vn_seq_stride + (int64_t)kvh * a.vn_head_stride + first + tile_p0 + crow];
+    load_block(vb_, a.v_packed + ((int64_t)seq * a.v_seq_stride + (int64_t)kvh * a.v_head_stride + first +
+                                  tile_p0 + wrow0) * kPdim, lane, wrow0, rows_here);
+  }
+  if (HAS_K) {
+    my_kn = a.k_norms[(int64_t)seq * a.kn_seq_stride + (int64_t)kvh * a.kn_head_stride + first + tile_p0 + crow];
+    load_block(kb_, a.k_packed + ((int64_t)seq * a.k_seq_stride + (int64_t)kvh * a.k_head_stride + first +
+                                  tile_p0 + wrow0) * kPdim, lane, wrow0, rows_here);
+  }
+  // given weights: lane (head n16, group g) takes positions 16t + 4g + j
+  float wgt[4][4];
+  if (MODE == kWeights) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int row = wrow0 + 16 * t + 4 * g + j;
+        float w = 0.0f;
+        if (row < rows_here && n16 < n_rep) w = a.weights[((int64_t)kvh * n_rep + n16) * len + tile_p0 + row];
+        wgt[t][j] = (w < a.threshold) ? 0.0f : w;
+      }
+  }
+  if (HAS_K) fill_lut(lutk_s, kcb, tid);
+  if (HAS_V) fill_lut(lutv_s, vcb, tid);
+  if (HAS_K) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const __half2 h = __floats2half2_rn(my_q[i].x, my_q[i].y);
+      const float2 back = __half22float2(h);
+      (&q_s[0][0])[tid + i * kMfmaThreads] = *reinterpret_cast<const uint32_t*>(&h);
+      (&ql_s[0][0])[tid + i * kMfmaThreads] = pack_h2(my_q[i].x - back.x, my_q[i].y - back.y);
+    }
+    kn_s[wave][lane] = my_kn;
+  }
+  if (HAS_V) vn_s[wave][lane] = my_vn;
+  __syncthreads();
+
+  uint32_t* stage = reinterpret_cast<uint32_t*>(big_s) + wave * 1024;
+
+  // ---- V: norms, table indices --------------------------------------------------------------------------
+  float vn[4][4];
+  float inv_tscale = 1.0f;
+  uint32_t X[2][4], Y[2][4];
+  if (HAS_V) {
+    float nmax = 0.0f;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const float4 n4 = *reinterpret_cast<const float4*>(&vn_s[wave][16 * t + 4 * g]);
+      vn[t][0] = n4.x; vn[t][1] = n4.y; vn[t][2] = n4.z; vn[t][3] = n4.w;
+      nmax = fmaxf(nmax, fmaxf(fmaxf(n4.x, n4.y), fmaxf(n4.z, n4.w)));
+    }
+    nmax = fmaxf(nmax, shfl_xor_f(nmax, 16));
+    nmax = fmaxf(nmax, shfl_xor_f(nmax, 32));
+    int ex = (int)((__float_as_uint(nmax) >> 23) & 0xFF);
+    ex = ex < 1 ? 127 : (ex > 253 ? 253 : ex);
+    const float tscale = __uint_as_float((uint32_t)(254 - ex) << 23);
+    inv_tscale = __uint_as_float((uint32_t)ex << 23);
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) vn[t][j] *= tscale;
+
+    stage_block(vb_, stage, lane);
+    int w0, sh_lo, sh_hi;
+    piece_bits(n16, w0, sh_lo, sh_hi);
+    constexpr uint32_t kEven = 0x1C71C7u;
+#pragma unroll
+    for (int kb2 = 0; kb2 < 2; ++kb2)
+#pragma unroll
+      for (int qd = 0; qd < 4; ++qd) {
+        const int t = 2 * kb2 + (qd >> 1), jp = qd & 1;
+        const uint32_t* ra = stage + (16 * t + 4 * g + 2 * jp) * kPdim + w0;
+        const uint32_t fa = ((ra[0] >> sh_lo) | (ra[1] << sh_hi)) & 0xFFFFFFu;
+        const uint32_t fb = ((ra[kPdim] >> sh_lo) | (ra[kPdim + 1] << sh_hi)) & 0xFFFFFFu;
+        X[kb2][qd] = (fa & kEven) | ((fb & kEven) << 3);
+        Y[kb2][qd] = ((fa >> 3) & kEven) | (fb & (kEven << 3));
+      }
+  }
+
+  // ---- K: scores ----------------------------------------------------------------------------------------
+  float s[4][4];
+  if (HAS_K) {
+    u4 qreg[4], qlow[4];
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+      qreg[kb] = *reinterpret_cast<const u4*>(&q_s[n16][(4 * kb + g) * 4]);
+      qlow[kb] = *reinterpret_cast<const u4*>(&ql_s[n16][(4 * kb + g) * 4]);
+    }
+    stage_block(kb_, stage, lane);                       // the V image has been consumed
+    int kw0[4], ksl[4], ksh[4];
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) piece_bits(4 * kb + g, kw0[kb], ksl[kb], ksh[kb]);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      f4 acc = {0.f, 0.f, 0.f, 0.f};
+      const uint32_t* krow = stage + (16 * t + n16) * kPdim;
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb) {
+        const uint32_t f = ((krow[kw0[kb]] >> ksl[kb]) | (krow[kw0[kb] + 1] << ksh[kb])) & 0xFFFFFFu;
+        u4 ka;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) ka[k] = lutk_s[(f >> (6 * k)) & 63u];
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, ka), __builtin_bit_cast(h8, qreg[kb]),
+                                                     acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, ka), __builtin_bit_cast(h8, qlow[kb]),
+                                                     acc, 0, 0, 0);
+      }
+      const float4 kn4 = *reinterpret_cast<const float4*>(&kn_s[wave][16 * t + 4 * g]);
+      const float knv[4] = {kn4.x, kn4.y, kn4.z, kn4.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int row = wrow0 + 16 * t + 4 * g + j;
+        float v = (acc[j] * knv[j]) * a.score_scale;
+        if (MODE == kFlash && a.mask && row < rows_here && n16 < n_rep)
+          v += a.mask[(int64_t)seq * a.mask_seq_stride + ((int64_t)kvh * n_rep + n16) * a.mask_head_stride +
+                      tile_p0 + row];
+        s[t][j] = (row < rows_here) ? v : -INFINITY;
+      }
+    }
+    if (MODE == kScores) {
+      if (n16 < n_rep) {
+        float* orow = a.scores + ((int64_t)kvh * n_rep + n16) * len + tile_p0;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int row = wrow0 + 16 * t + 4 * g + j;
+            if (row < rows_here) orow[row] = s[t][j];
+          }
+      }
+      return;
+    }
+  }
+
+  // ---- weights of the value product -------------------------------------------------------------------
+  float m = 0.0f, l = 0.0f;
+  uint32_t pa[2][4];
+  if (MODE == kFlash) {
+    m = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) m = fmaxf(m, s[t][j]);
+    m = fmaxf(m, shfl_xor_f(m, 16));
+    m = fmaxf(m, shfl_xor_f(m, 32));
+  }
+  const float msafe = (m == -INFINITY) ? 0.0f : m;
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    float p[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      p[j] = (MODE == kFlash) ? __expf(s[t][j] - msafe) : wgt[t][j];
+      l += p[j];
+      p[j] *= vn[t][j];
+    }
+    pa[t >> 1][2 * (t & 1)] = pack_h2(p[0], p[1]);
+    pa[t >> 1][2 * (t & 1) + 1] = pack_h2(p[2], p[3]);
+  }
+  l += shfl_xor_f(l, 16);
+  l += shfl_xor_f(l, 32);
+
+  // ---- values ------------------------------------------------------------------------------------------
+  f4 accS[8];
+#pragma unroll
+  for (int et = 0; et < 8; ++et) accS[et] = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int kb2 = 0; kb2 < 2; ++kb2) {
+    const u4 A = {pa[kb2][0], pa[kb2][1], pa[kb2][2], pa[kb2][3]};
+#pragma unroll
+    for (int et = 0; et < 8; ++et) {
+      u4 B;
+#pragma unroll
+      for (int qd = 0; qd < 4; ++qd) {
+        const uint32_t src = (et & 1) ? Y[kb2][qd] : X[kb2][qd];
+        B[qd] = lutv_s[(src >> (6 * (et >> 1))) & 63u];
+      }
+      accS[et] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, A), __builtin_bit_cast(h8, B),
+                                                        accS[et], 0, 0, 0);
+    }
+  }
+
+  // ---- merge the eight waves (one barrier per round of 8 heads), as in the dense-key kernel ------------
+  float (*S_all)[8][kD] = reinterpret_cast<float (*)[8][kD]>(big_s);
+  const int64_t grp = (int64_t)seq * a.n_kv + kvh;
+  float* pS = a.ws_S + (grp * a.n_tiles_max + tile) * (int64_t)(n_rep * kD);
+  float* pml = a.ws_ml + (grp * a.n_tiles_max + tile) * (int64_t)(n_rep * 2);
+  if (g == 0) {
+    m_s[wave][n16] = m;
+    l_s[wave][n16] = l;
+  }
+  if (lane == 0) t_s[wave] = inv_tscale * a.v_unscale;
+  for (int h0 = 0; h0 < n_rep; h0 += 8) {
+    __syncthreads();
+    if ((g >> 1) == (h0 >> 3)) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float4* dst = reinterpret_cast<float4*>(&S_all[wave][(4 * g + j) & 7][8 * n16]);
+        dst[0] = make_float4(accS[0][j], accS[1][j], accS[2][j], accS[3][j]);
+        dst[1] = make_float4(accS[4][j], accS[5][j], accS[6][j], accS[7][j]);
+      }
+    }
+    __syncthreads();
+    const int rows = min(8, n_rep - h0);
+    for (int i = tid; i < rows * kD; i += kMfmaThreads) {
+      const int hl = i >> 7, e = i & 127, h = h0 + hl;
+      float M = m_s[0][h];
+#pragma unroll
+      for (int w = 1; w < kWaves; ++w) M = fmaxf(M, m_s[w][h]);
+      float sum = 0.0f;
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) {
+        const float mw = m_s[w][h];
+        const float f = (mw == -INFINITY) ? 0.0f : __expf(mw - M) * t_s[w];
+        sum += f * S_all[w][hl][e];
+      }
+      pS[h * kD + e] = sum;
+    }
+  }
+  if (tid < n_rep) {
+    const int h = tid;
+    float M = m_s[0][h];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) M = fmaxf(M, m_s[w][h]);
+    float L = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) L += (m_s[w][h] == -INFINITY) ? 0.0f : __expf(m_s[w][h] - M) * l_s[w][h];
+    pml[2 * h] = M;
+    pml[2 * h + 1] = L;
+  }
+}
+
+}  // namespace tqm

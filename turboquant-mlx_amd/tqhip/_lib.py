@@ -34,7 +34,7 @@ class DecodeShape(C.Structure):
         ("v_seq_stride", C.c_int64), ("v_head_stride", C.c_int64),
         ("vn_seq_stride", C.c_int64), ("vn_head_stride", C.c_int64),
         ("mask", C.c_void_p), ("mask_seq_stride", C.c_int64), ("mask_head_stride", C.c_int64),
-        ("attn_scale", C.c_float), ("out_dtype", C.c_int32),
+        ("attn_scale", C.c_float), ("out_dtype", C.c_int32), ("allow_mma", C.c_int32),
     ]
 
 
@@ -46,11 +46,11 @@ PROTOTYPES = {
     "tq_encode": (_i, [_p, _i, _p, _fp, _p, _p, _l, _l, _l, _l, _i, _i, _i, _p]),
     "tq_dequant": (_i, [_p, _p, _fp, _p, _p, _i, _l, _l, _l, _l, _l, _i, _i, _p]),
     "tq_prerotate_query": (_i, [_p, _i, _p, _p, _l, _i, _p]),
-    "tq_prerot_qk_scores": (_i, [_p, _p, _p, _fp, _p, _i, _i, _l, _l, _l, _i, _i, _p]),
+    "tq_prerot_qk_scores": (_i, [_p, _p, _p, _fp, _p, _i, _i, _l, _l, _l, _i, _i, _i, _p]),
     "tq_packed_qk_scores": (_i, [_p, _p, _p, _fp, _p, _p, _i, _l, _l, _l, _i, _i, _p]),
     "tq_dense_qk_scores": (_i, [_p, _i, _p, _p, _i, _i, _l, _l, _i, _f, _p]),
     "tq_softmax_rows": (_i, [_p, _p, _l, _p, _l, _l, _f, _p]),
-    "tq_sparse_v_matvec": (_i, [_p, _p, _p, _fp, _p, _p, _p, _z, _i, _i, _l, _l, _l, _i, _i, _f, _p]),
+    "tq_sparse_v_matvec": (_i, [_p, _p, _p, _fp, _p, _p, _p, _z, _i, _i, _l, _l, _l, _i, _i, _f, _i, _p]),
     "tq_flash_decode": (_i, [_p, _p, _p, _p, _p, _fp, _fp, _p, _p, _p, _z, C.POINTER(DecodeShape), _p]),
     "tq_vonly_decode_attn": (_i, [_p, _i, _p, _p, _p, _fp, _p, _p, _p, _z, C.POINTER(DecodeShape), _p]),
     "tq_vonly_decode_attn_phases": (_i, [_p, _i, _p, _p, _p, _fp, _p, _p, _p, _z, C.POINTER(DecodeShape), _i, _p]),

@@ -1,0 +1,144 @@
+"""Per-kernel micro-benchmarks at the shapes of the reference's configurations.
+
+Methodology of the reference's scripts/bench_sparse_v.py:49-57 (warm-up, then a timed loop with a
+sync at the end), adapted to a GPU with large caches: HIP events on the launch stream, many
+back-to-back launches, and rotation over several independent input sets so that the 256 MB
+Infinity Cache cannot serve the reads.  Prints one line per case: us per call, GB/s of algorithmic
+bytes and the fraction of 8 TB/s.
+
+    python -m tqhip.bench_kernels [--iters 200] [--cases encode,scores,flash,sparse_v,vonly]
+"""
+from __future__ import annotations
+
+import argparse
+import math
+
+import torch
+
+import tqhip
+from tqhip.quantizer import gaussian_boundaries, gaussian_codebook
+
+PEAK = 8000.0
+
+
+def timeit(fns, iters, warmup=10):
+    """fns: list of zero-arg callables (one per input set), called round-robin."""
+    for i in range(warmup):
+        fns[i % len(fns)]()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(iters):
+        fns[i % len(fns)]()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / iters
+
+
+def report(name, us, nbytes):
+    gbs = nbytes / us / 1e3
+    print(f"{name:58s} {us:10.2f} us  {gbs:8.1f} GB/s  {100 * gbs / PEAK:5.1f} % of 8 TB/s", flush=True)
+
+
+def n_sets_for(nbytes):
+    return max(2, min(16, int(math.ceil(420e6 / max(nbytes, 1)))))
+
+
+def bench_encode(iters, dev):
+    cb = gaussian_codebook(3)
+    bd = gaussian_boundaries(cb)
+    signs = tqhip.random_diagonal_sign(128, 43, device=dev)
+    for n_vecs, label in ((4096, "config 1: 4096 vectors"), (131072 * 8, "config 5: 1 048 576 vectors")):
+        nbytes = n_vecs * (256 + 56)
+        xs = [torch.randn((n_vecs, 128), device=dev, dtype=torch.float16) for _ in range(n_sets_for(nbytes))]
+        if "config 5" in label:
+            for x in xs:
+                x[:, 17] *= 20                          # 1 % outlier channels scaled x20
+        fns = [(lambda x=x: tqhip.fused_quantize(x, signs, bd, 128, 3)) for x in xs]
+        report(f"encode d=128 3-bit, {label}", timeit(fns, iters), nbytes)
+        p, n = tqhip.fused_quantize(xs[0], signs, bd, 128, 3)
+        fns = [(lambda: tqhip.dequant_fp16(p, n, cb, signs, 128, 3))]
+        report(f"dequant_fp16 d=128 3-bit, {n_vecs} vectors (cache-warm)", timeit(fns, iters), n_vecs * (56 + 256))
+
+
+def packed_sets(n_kv, T, dev, n_sets, seed):
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    sets = []
+    for _ in range(n_sets):
+        p = torch.randint(0, 2 ** 30, (n_kv, T, 13), generator=g, device=dev, dtype=torch.int32).view(torch.uint32)
+        n = torch.rand((n_kv, T), generator=g, device=dev) + 0.1
+        sets.append((p, n))
+    return sets
+
+
+def bench_scores(iters, dev):
+    cb = gaussian_codebook(3)
+    for T in (4096, 16384, 65536):
+        nbytes = 224 * T + 112 * T + 14336
+        sets = packed_sets(4, T, dev, n_sets_for(nbytes), 3)
+        q_rot = torch.randn((28, 128), device=dev)
+        fns = [(lambda p=p, n=n: tqhip.prerot_fused_qk_scores(q_rot, p, n, cb, 128, 3, n_rep=7)) for p, n in sets]
+        report(f"config 3: prerot scores 28/4 heads, T={T}", timeit(fns, iters), nbytes)
+
+
+def bench_sparse_v(iters, dev):
+    cb = gaussian_codebook(3)
+    signs = tqhip.random_diagonal_sign(128, 43, device=dev)
+    for T in (8192, 32768):
+        nbytes = 28 * T * 4 + 4 * T * 56 + 28 * 128 * 4
+        sets = packed_sets(4, T, dev, n_sets_for(nbytes), 4)
+        w = torch.softmax(torch.randn((28, T), device=dev) * 5, dim=-1)
+        for thr in (0.0, 1e-5):
+            fns = [(lambda p=p, n=n: tqhip.sparse_v_matvec(w, p, n, cb, signs, 128, 3, threshold=thr, n_rep=7))
+                   for p, n in sets]
+            report(f"sparse_v_matvec 28/4 heads, T={T}, thr={thr:g}", timeit(fns, iters), nbytes)
+
+
+def bench_flash(iters, dev):
+    cb = gaussian_codebook(3)
+    signs = tqhip.random_diagonal_sign(128, 43, device=dev)
+    g = torch.Generator()
+    g.manual_seed(4)
+    lens = torch.randint(4096, 32769, (16,), generator=g)
+    offs = torch.cat([torch.zeros(1, dtype=torch.int64), lens.cumsum(0)]).to(torch.int32).to(dev)
+    total = int(lens.sum())
+    nbytes = 896 * total + 262144
+    k = packed_sets(8, total, dev, 2, 5)
+    v = packed_sets(8, total, dev, 2, 6)
+    q_rot = torch.randn((16, 32, 128), device=dev)
+    fns = [(lambda i=i: tqhip.flash_decode(q_rot, k[i][0], k[i][1], v[i][0], v[i][1], cb, cb, signs, 128, 3,
+                                           1 / math.sqrt(128), n_rep=4, seq_offsets=offs,
+                                           max_seq_len=int(lens.max()), out_dtype=torch.float16)) for i in range(2)]
+    report(f"config 4: flash decode 32/8 heads, 16 seqs, sum L={total}", timeit(fns, max(20, iters // 10)), nbytes)
+
+
+def bench_vonly(iters, dev):
+    cb = gaussian_codebook(3)
+    signs = tqhip.random_diagonal_sign(128, 43, device=dev)
+    for T in (4096, 32768, 131072):
+        nbytes = 4 * T * 312 + 28 * 256 * 2
+        sets = packed_sets(4, T, dev, n_sets_for(nbytes), 7)
+        ks = [torch.randn((4, T, 128), device=dev, dtype=torch.float16) for _ in sets]
+        q = torch.randn((1, 28, 128), device=dev, dtype=torch.float16)
+        fns = [(lambda k=k, p=p, n=n: tqhip.vonly_decode(q, k, p, n, cb, signs, 128, 3, 1 / math.sqrt(128), n_rep=7))
+               for k, (p, n) in zip(ks, sets)]
+        report(f"config 2 shape: V-only decode 28/4 heads, T={T} (python-call launch)", timeit(fns, iters), nbytes)
+
+
+CASES = {"encode": bench_encode, "scores": bench_scores, "sparse_v": bench_sparse_v, "flash": bench_flash,
+         "vonly": bench_vonly}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--iters", type=int, default=200)
+    ap.add_argument("--cases", default=",".join(CASES))
+    args = ap.parse_args()
+    dev = torch.device("cuda:0")
+    for c in args.cases.split(","):
+        CASES[c](args.iters, dev)
+
+
+if __name__ == "__main__":
+    main()

@@ -253,11 +253,20 @@ def _check_gqa(n_q: int, n_kv: int, n_rep: int):
         raise ValueError(f"n_q_heads ({n_q}) must equal n_kv_heads ({n_kv}) * n_rep ({n_rep})")
 
 
+def _mma_flag(precision: str) -> int:
+    if precision not in ("fp32", "fp16"):
+        raise ValueError(f"precision must be 'fp32' or 'fp16', got {precision!r}")
+    return 1 if precision == "fp16" else 0
+
+
 def prerot_fused_qk_scores(q_rot: torch.Tensor, k_packed: torch.Tensor, k_norms: torch.Tensor,
-                           centroids, dim: int, bits: int, n_rep: int = 1) -> torch.Tensor:
+                           centroids, dim: int, bits: int, n_rep: int = 1,
+                           precision: str = "fp32") -> torch.Tensor:
     """metal_kernels_v4.py:153-221.  Scores of pre-rotated queries against packed K, GQA-aware.
 
     q_rot (n_q, dim); k_packed (n_kv, seq, pdim); k_norms (n_kv, seq) -> (n_q, seq) float32.
+    precision="fp32" keeps the reference's float32 arithmetic; "fp16" rounds q_rot and the
+    centroids to half and runs on the matrix cores (float32 accumulation, ~3e-4 relative).
     """
     _need_gpu(q_rot, k_packed, k_norms)
     n_q = q_rot.shape[0]
@@ -270,7 +279,7 @@ def prerot_fused_qk_scores(q_rot: torch.Tensor, k_packed: torch.Tensor, k_norms:
     out = torch.empty((n_q, seq_len), dtype=torch.float32, device=q_rot.device)
     _lib.check(_lib.load().tq_prerot_qk_scores(
         _ptr(q_rot), _ptr(k_packed), _ptr(k_norms), _host_table(centroids), _ptr(out),
-        n_kv, n_rep, seq_len, phs, nhs, dim, bits, _stream(q_rot)))
+        n_kv, n_rep, seq_len, phs, nhs, dim, bits, _mma_flag(precision), _stream(q_rot)))
     return out
 
 
@@ -333,11 +342,13 @@ def softmax_rows(scores: torch.Tensor, scale: float = 1.0, mask: torch.Tensor | 
 # ------------------------------------------------------------------ sparse V
 
 def sparse_v_matvec(weights: torch.Tensor, v_packed: torch.Tensor, v_norms: torch.Tensor, centroids,
-                    signs, dim: int, bits: int, threshold: float = 1e-5, n_rep: int = 1) -> torch.Tensor:
+                    signs, dim: int, bits: int, threshold: float = 1e-5, n_rep: int = 1,
+                    precision: str = "fp32") -> torch.Tensor:
     """sparse_v.py:94-186.  Weighted sum of dequantised V rows with the butterfly pulled out of
     the position loop; positions with weight < threshold are skipped; threshold <= 0 is dense.
 
     weights (n_q, seq); v_packed (n_kv, seq, pdim); v_norms (n_kv, seq) -> (n_q, dim) float32.
+    precision as in prerot_fused_qk_scores ("fp16": weights * norm and centroids rounded to half).
     """
     if dim & (dim - 1):
         raise ValueError(f"dim must be a power of 2, got {dim}")
@@ -359,7 +370,8 @@ def sparse_v_matvec(weights: torch.Tensor, v_packed: torch.Tensor, v_norms: torc
     ws = _workspace(weights.device, stream.value or 0, need)
     _lib.check(lib.tq_sparse_v_matvec(
         _ptr(weights), _ptr(v_packed), _ptr(v_norms), _host_table(centroids), _ptr(signs), _ptr(out),
-        _ptr(ws), ws.numel(), n_kv, n_rep, seq_len, phs, nhs, dim, bits, float(max(threshold, 0.0)), stream))
+        _ptr(ws), ws.numel(), n_kv, n_rep, seq_len, phs, nhs, dim, bits, float(max(threshold, 0.0)),
+        _mma_flag(precision), stream))
     return out
 
 
@@ -371,7 +383,8 @@ def count_active_positions(weights: torch.Tensor, threshold: float = 1e-5) -> in
 # ------------------------------------------------------------------ fused decode attention
 
 def _decode_shape(*, n_seq, n_kv, n_rep, dim, bits, block_size, seq_len, seq_offsets, k_strides, kn_strides,
-                  v_strides, vn_strides, mask, mask_strides, attn_scale, out_dtype) -> DecodeShape:
+                  v_strides, vn_strides, mask, mask_strides, attn_scale, out_dtype,
+                  allow_mma: bool = True) -> DecodeShape:
     sh = DecodeShape()
     sh.n_seq, sh.n_kv_heads, sh.n_rep, sh.dim, sh.bits, sh.block_size = n_seq, n_kv, n_rep, dim, bits, block_size
     sh.seq_len = seq_len
@@ -384,6 +397,7 @@ def _decode_shape(*, n_seq, n_kv, n_rep, dim, bits, block_size, seq_len, seq_off
     sh.mask_seq_stride, sh.mask_head_stride = mask_strides
     sh.attn_scale = float(attn_scale)
     sh.out_dtype = _DTYPES[out_dtype]
+    sh.allow_mma = 1 if allow_mma else 0
     return sh
 
 
@@ -429,8 +443,12 @@ def _mask_layout(mask, n_seq: int, n_q: int, seq_len: int, device):
 def flash_decode(q_rot: torch.Tensor, k_packed, k_norms, v_packed, v_norms, k_centroids, v_centroids,
                  v_signs, dim: int, bits: int, attn_scale: float, *, n_rep: int = 1, block_size: int = 16,
                  seq_len: int | None = None, seq_offsets: torch.Tensor | None = None,
-                 max_seq_len: int | None = None, mask=None, out_dtype=torch.float32) -> torch.Tensor:
+                 max_seq_len: int | None = None, mask=None, out_dtype=torch.float32,
+                 precision: str = "fp16") -> torch.Tensor:
     """Batched form of flash_attention_turboquant (tq_flash_decode).
+
+    precision="fp16" (default): matrix-core kernels where the shape allows (d = 128, 3-bit,
+    n_rep <= 16), operands rounded to half, float32 accumulation; "fp32": float32 kernels.
 
     q_rot (n_seq, n_q, dim) float32.  K/V either cache layout [n_seq, n_kv, T_alloc, *] with the
     uniform valid length `seq_len`, or ragged [n_kv, sum(L), *] with int32 `seq_offsets`
@@ -464,7 +482,8 @@ def flash_decode(q_rot: torch.Tensor, k_packed, k_norms, v_packed, v_norms, k_ce
     out = torch.empty((n_seq, n_q, dim), dtype=out_dtype, device=q_rot.device)
     sh = _decode_shape(n_seq=n_seq, n_kv=n_kv, n_rep=n_rep, dim=dim, bits=bits, block_size=block_size,
                        seq_len=T, seq_offsets=seq_offsets, k_strides=ks, kn_strides=kns, v_strides=vs,
-                       vn_strides=vns, mask=mask, mask_strides=ms, attn_scale=attn_scale, out_dtype=out_dtype)
+                       vn_strides=vns, mask=mask, mask_strides=ms, attn_scale=attn_scale, out_dtype=out_dtype,
+                       allow_mma=bool(_mma_flag(precision)))
     lib = _lib.load()
     need = lib.tq_workspace_bytes(_lib.TQ_OP_FLASH_DECODE, n_seq, n_q, T, dim)
     stream = _stream(q_rot)
@@ -478,19 +497,20 @@ def flash_decode(q_rot: torch.Tensor, k_packed, k_norms, v_packed, v_norms, k_ce
 
 def flash_attention_turboquant(q_rot, k_packed, k_norms, v_packed, v_norms, k_centroids, v_centroids,
                                v_signs, dim: int, bits: int, attn_scale: float, block_size: int = 16,
-                               n_rep: int = 1) -> torch.Tensor:
+                               n_rep: int = 1, precision: str = "fp16") -> torch.Tensor:
     """flash_attention.py:168-274.  One sequence: q_rot (n_q, dim); K/V (n_kv, seq, pdim) + (n_kv, seq)
     -> (n_q, dim) float32 = softmax(QK * scale) @ V over the packed cache."""
     out = flash_decode(q_rot.unsqueeze(0), k_packed, k_norms, v_packed, v_norms, k_centroids, v_centroids,
-                       v_signs, dim, bits, attn_scale, n_rep=n_rep, block_size=block_size)
+                       v_signs, dim, bits, attn_scale, n_rep=n_rep, block_size=block_size, precision=precision)
     return out[0]
 
 
 def vonly_decode(q: torch.Tensor, k: torch.Tensor, v_packed, v_norms, v_centroids, v_signs, dim: int,
                  bits: int, attn_scale: float, *, n_rep: int = 1, seq_len: int | None = None,
                  seq_offsets: torch.Tensor | None = None, max_seq_len: int | None = None, mask=None,
-                 out_dtype=torch.float32) -> torch.Tensor:
+                 out_dtype=torch.float32, precision: str = "fp16") -> torch.Tensor:
     """Dense-softmax decode attention over fp16 keys and packed values (tq_vonly_decode_attn).
+    precision as in flash_decode (the matrix-core path also needs fp16 queries).
 
     q (n_seq, n_q, dim) fp16/bf16/fp32; k [n_seq, n_kv, T_alloc, dim] or ragged [n_kv, sum(L), dim] fp16;
     V as in flash_decode.  Returns (n_seq, n_q, dim) `out_dtype`.
@@ -520,7 +540,8 @@ def vonly_decode(q: torch.Tensor, k: torch.Tensor, v_packed, v_norms, v_centroid
     out = torch.empty((n_seq, n_q, dim), dtype=out_dtype, device=q.device)
     sh = _decode_shape(n_seq=n_seq, n_kv=n_kv, n_rep=n_rep, dim=dim, bits=bits, block_size=16, seq_len=T,
                        seq_offsets=seq_offsets, k_strides=ks, kn_strides=(0, 0), v_strides=vs, vn_strides=vns,
-                       mask=mask, mask_strides=ms, attn_scale=attn_scale, out_dtype=out_dtype)
+                       mask=mask, mask_strides=ms, attn_scale=attn_scale, out_dtype=out_dtype,
+                       allow_mma=bool(_mma_flag(precision)))
     lib = _lib.load()
     need = lib.tq_workspace_bytes(_lib.TQ_OP_VONLY_DECODE, n_seq, n_q, T, dim)
     stream = _stream(q)
