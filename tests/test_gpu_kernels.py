@@ -145,6 +145,98 @@ def test_config1_roundtrip(tq):
     assert np.array_equal(host(gn.to(torch.float16)), wn.astype(np.float16))
 
 
+def _special_rows(rng, n, b):
+    """n x 128 float32 rows: random scales, a zero row, one-hot rows, and rows whose butterfly
+    outputs sit within a few ulp of a decision boundary."""
+    x = (rng.standard_normal((n, 128)) * rng.choice([1e-3, 1.0, 300.0], size=(n, 1))).astype(F32)
+    x[5] = 0.0
+    x[6] = 0.0
+    x[6, 127] = -2.5
+    x[7] = 0.0
+    x[7, 64] = 1e-3
+    H = np.array([[1.0 if bin(j & k).count("1") % 2 == 0 else -1.0 for k in range(128)] for j in range(128)])
+    for r in range(32, 232):
+        z = rng.standard_normal(128)
+        z[rng.integers(0, 128)] = float(b[rng.integers(0, 7)]) * (1 + rng.integers(-3, 4) * 2.0 ** -23)
+        z *= math.sqrt(128) / np.linalg.norm(z)
+        x[r] = (H @ z) / 128.0
+    return x
+
+
+@pytest.mark.parametrize("variant", ["mlx", "metal"])
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+def test_encode_streaming_kernel(tq, dtype, variant):
+    """At d = 128 / 3-bit a row count that is a multiple of 16 takes the streaming encoder (four
+    lanes per vector, reciprocal + fma division, guessed level + one compare): its bits must be the
+    oracle's, for every input type and both threshold rules, special rows included."""
+    rng = np.random.default_rng(31)
+    c, b = tables(3)
+    s = o.random_diagonal_sign(128, 43)
+    n = 16 * 261
+    x = _special_rows(rng, n, b)
+    if dtype == "f32":
+        xt = torch.from_numpy(x)
+    elif dtype == "f16":
+        xt = torch.from_numpy(x).to(torch.float16)
+    else:
+        xt = torch.from_numpy(x).to(torch.bfloat16)
+    xt[100] = float("nan")
+    xt[101, 3] = float("nan")
+    ref_in = xt.float().numpy()
+    ok = ~np.isnan(ref_in).any(axis=1)
+    wp, wn = o.fused_quantize(ref_in[ok], s, b, 128, 3, variant)
+    gp, gn = tq.fused_quantize(xt.cuda(), dev(s), b, 128, 3, variant=variant)
+    gp, gn = host(gp), host(gn)
+    assert np.array_equal(gp[ok], wp) and np.array_equal(gn[ok], wn)
+    assert (gp[~ok] == 0).all() and np.isnan(gn[~ok]).all()          # NaN compares false with every threshold
+    # the generic one-wavefront-per-vector kernel (ragged count) gives the same words
+    gp2, gn2 = tq.fused_quantize(xt[: n - 3].cuda(), dev(s), b, 128, 3, variant=variant)
+    assert np.array_equal(host(gp2), gp[: n - 3])
+    assert np.array_equal(host(gn2)[ok[: n - 3]], gn[: n - 3][ok[: n - 3]])
+
+
+def test_encode_and_dequant_into_strided_groups(tq):
+    """Cache layout: groups (batch x head) of rows with a stride larger than the rows written, at a
+    row offset; both streaming kernels must place every row where the generic ones do."""
+    rng = np.random.default_rng(32)
+    c, b = tables(3)
+    s = o.random_diagonal_sign(128, 42)
+    G, R, alloc, off = 3, 48, 256, 32
+    x = rng.standard_normal((G, R, 128)).astype(np.float16)
+    packed = torch.zeros((G, alloc, 13), dtype=torch.int32, device="cuda").view(torch.uint32)
+    norms = torch.zeros((G, alloc), dtype=torch.float32, device="cuda")
+    tq.encode_into(dev(x), dev(s), b, packed, norms, n_groups=G, rows_per_group=R, packed_group_stride=alloc,
+                   norms_group_stride=alloc, dim=128, bits=3, packed_row_offset=off, norms_row_offset=off)
+    wp, wn = o.fused_quantize(x.reshape(-1, 128), s, b, 128, 3)
+    hp, hn = host(packed), host(norms)
+    assert np.array_equal(hp[:, off:off + R], wp.reshape(G, R, 13)) and np.array_equal(hn[:, off:off + R], wn.reshape(G, R))
+    assert (hp[:, :off] == 0).all() and (hp[:, off + R:] == 0).all() and (hn[:, off + R:] == 0).all()
+    for dt in (torch.float32, torch.float16, torch.bfloat16):
+        out = torch.zeros((G, alloc, 128), dtype=dt, device="cuda")
+        tq.dequant_into(packed, norms, c, dev(s), out, n_groups=G, rows_per_group=R, packed_group_stride=alloc,
+                        norms_group_stride=alloc, out_group_stride=alloc, dim=128, bits=3, packed_row_offset=off,
+                        norms_row_offset=off, out_row_offset=off)
+        want = torch.from_numpy(o.packed_dequantize(wp, wn, c, s, 128, 3)).to(dt).reshape(G, R, 128)
+        assert torch.equal(out[:, off:off + R].cpu(), want)
+        assert (out[:, :off] == 0).all() and (out[:, off + R:] == 0).all()
+
+
+@pytest.mark.parametrize("dt", [torch.float32, torch.float16, torch.bfloat16])
+def test_dequant_streaming_kernel(tq, dt):
+    rng = np.random.default_rng(33)
+    c, b = tables(3)
+    s = o.random_diagonal_sign(128, 43)
+    n = 16 * 70
+    p = o.pack_indices(rng.integers(0, 8, size=(n, 128)).astype(np.uint8), 3)
+    nr = (rng.random(n) * rng.choice([1e-3, 1.0, 500.0], size=n)).astype(F32)
+    nr[3] = 0.0
+    want = torch.from_numpy(o.packed_dequantize(p, nr, c, s, 128, 3)).to(dt)
+    out = torch.empty((n, 128), dtype=dt, device="cuda")
+    tq.dequant_into(dev(p), dev(nr), c, dev(s), out, n_groups=1, rows_per_group=n, packed_group_stride=n,
+                    norms_group_stride=n, out_group_stride=n, dim=128, bits=3)
+    assert torch.equal(out.cpu(), want)
+
+
 # ------------------------------------------------------------------ dequant / prerotate
 
 @pytest.mark.parametrize("dim,bits", [(128, 3), (64, 4), (32, 2), (256, 3), (128, 1)])

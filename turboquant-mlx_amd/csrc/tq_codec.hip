@@ -4,7 +4,9 @@
 #include "tq_common.h"
 
 #include <math.h>
+#include <cmath>
 #include <string.h>
+#include <mutex>
 
 namespace {
 
@@ -88,6 +90,214 @@ __global__ __launch_bounds__(kBlock) void encode_kernel(const T* __restrict__ x,
   }
 }
 
+// ---------------------------------------------------------------- encode, d = 128, 3-bit
+// The streaming encoder for the cache's own shape.  Four lanes own one vector, so a wavefront
+// encodes 16 vectors per pass: lane ls = lane % 4 of a vector holds the four 8-element chunks
+// c = ls + 4k (k = 0..3), element e = 32k + 8ls + j.  Each load instruction therefore reads 64
+// contiguous bytes per vector; butterfly stages 1, 2, 4, 32 and 64 and five of the seven levels of
+// the sum-of-squares tree stay inside a lane, and stages 8 and 16 are quad-permute lane exchanges
+// folded into the add.  Results are bit-identical to encode_kernel:
+//  * the sum of squares is added in the same stride-halving tree order;
+//  * x / n is computed as q = x*r, q += r * fma(-n, q, x) with r = 1/n correctly rounded, which
+//    yields the correctly rounded quotient (checked against IEEE division on 3e10 operand pairs
+//    with |x| <= n), at 3 operations per element instead of a full division;
+//  * the count of thresholds exceeded is g + (w > t[g]) with g = clamp(floor(alpha*w + beta), 0, 6),
+//    where the host has verified that g is the count or one less for every w.
+// Packed words leave through LDS so that a wavefront stores 208 contiguous words per pass.
+constexpr int kEncVecs = 16;      // vectors per wavefront pass
+constexpr int kEncPasses = 4;     // passes per wavefront once there are rows enough to fill the chip
+
+struct EncodeGuess { float alpha, beta; };
+
+__device__ __forceinline__ float quad_xor1(float v) {
+  return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true));   // lanes 1,0,3,2
+}
+__device__ __forceinline__ float quad_xor2(float v) {
+  return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xF, 0xF, true));   // lanes 2,3,0,1
+}
+
+// Raw butterfly of a 128-vector spread over four lanes (element e = 32k + 8*ls + j in xs[k][j] of
+// lane ls), stages in the order of strides 1, 2, ..., 64.  flip1 / flip2 are 0x80000000 in the
+// lanes whose ls has bit 0 / bit 1 set (the upper element of a pair computes partner - own).
+__device__ __forceinline__ void butterfly_4lane(float (&xs)[4][8], uint32_t flip1, uint32_t flip2) {
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+#pragma unroll
+    for (int h = 1; h < 8; h <<= 1)
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (!(j & h)) {
+          const float a = xs[k][j], b = xs[k][j + h];
+          xs[k][j] = a + b;
+          xs[k][j + h] = a - b;
+        }
+  }
+#pragma unroll
+  for (int k = 0; k < 4; ++k)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float a = xs[k][j];
+      xs[k][j] = quad_xor1(a) + __uint_as_float(__float_as_uint(a) ^ flip1);
+    }
+#pragma unroll
+  for (int k = 0; k < 4; ++k)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float a = xs[k][j];
+      xs[k][j] = quad_xor2(a) + __uint_as_float(__float_as_uint(a) ^ flip2);
+    }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const float a0 = xs[0][j] + xs[1][j], a1 = xs[0][j] - xs[1][j];
+    const float a2 = xs[2][j] + xs[3][j], a3 = xs[2][j] - xs[3][j];
+    xs[0][j] = a0 + a2; xs[2][j] = a0 - a2;
+    xs[1][j] = a1 + a3; xs[3][j] = a1 - a3;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void encode128x3_kernel(const T* __restrict__ x,
+                                                             const float* __restrict__ signs, Thresholds thr,
+                                                             EncodeGuess gs, uint32_t* __restrict__ packed,
+                                                             float* __restrict__ norms, RowMap rm, int passes) {
+  constexpr bool kHalfWidth = sizeof(T) == 2;
+  constexpr int NM = kHalfWidth ? 4 : 8;                       // sign masks per chunk
+  __shared__ float thr_s[8];
+  __shared__ __align__(16) float sg_s[128];
+  __shared__ uint32_t chunk_s[kWavesPerBlock][kEncVecs * 16 + 4];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ls = lane & 3, v = lane >> 2;
+  if (tid < 8) {
+    float t = INFINITY;
+#pragma unroll
+    for (int i = 0; i < 7; ++i) t = (tid == i) ? thr.t[i] : t;
+    thr_s[tid] = t;
+  }
+  if (tid < 128) sg_s[tid] = signs[tid];
+  __syncthreads();
+
+  // sign flips as xor masks on the raw input bits
+  uint32_t sm[4][NM];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const float4 a = *reinterpret_cast<const float4*>(&sg_s[32 * k + 8 * ls]);
+    const float4 b = *reinterpret_cast<const float4*>(&sg_s[32 * k + 8 * ls + 4]);
+    const float sv[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    if (kHalfWidth) {
+#pragma unroll
+      for (int jp = 0; jp < 4; ++jp)
+        sm[k][jp] = ((__float_as_uint(sv[2 * jp]) >> 16) & 0x8000u) | (__float_as_uint(sv[2 * jp + 1]) & 0x80000000u);
+    } else {
+#pragma unroll
+      for (int j = 0; j < NM; ++j) sm[k][j] = __float_as_uint(sv[j & 7]) & 0x80000000u;
+    }
+  }
+  const uint32_t flip1 = (ls & 1) ? 0x80000000u : 0u;          // upper lane of a pair computes partner - own
+  const uint32_t flip2 = (ls & 2) ? 0x80000000u : 0u;
+  uint32_t* chunks = chunk_s[wave];
+
+  // first batch of 16 rows of this wavefront and its place in the (group, row) map
+  const uint32_t batch0 = ((uint32_t)blockIdx.x * kWavesPerBlock + wave) * (uint32_t)passes;
+  uint32_t row0 = batch0 * kEncVecs;
+  uint32_t grp = row0 / (uint32_t)rm.rows_per_group;
+  uint32_t rin = row0 - grp * (uint32_t)rm.rows_per_group;
+
+  for (int pass = 0; pass < passes; ++pass) {
+    if (row0 >= (uint32_t)rm.n_rows) break;                    // uniform over the wavefront
+    // ---- load, flip signs, widen
+    float xs[4][8];
+    const T* xr = x + ((int64_t)row0 + v) * 128 + 8 * ls;
+    if (kHalfWidth) {
+      uint4 raw[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) raw[k] = *reinterpret_cast<const uint4*>(xr + 32 * k);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const uint32_t w[4] = {raw[k].x ^ sm[k][0], raw[k].y ^ sm[k][1], raw[k].z ^ sm[k][2], raw[k].w ^ sm[k][3]};
+#pragma unroll
+        for (int jp = 0; jp < 4; ++jp) {
+          if (sizeof(T) == 2 && __is_same(T, __half)) {
+            xs[k][2 * jp] = __half2float(__ushort_as_half((unsigned short)(w[jp] & 0xFFFFu)));
+            xs[k][2 * jp + 1] = __half2float(__ushort_as_half((unsigned short)(w[jp] >> 16)));
+          } else {
+            xs[k][2 * jp] = __uint_as_float(w[jp] << 16);
+            xs[k][2 * jp + 1] = __uint_as_float(w[jp] & 0xFFFF0000u);
+          }
+        }
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const uint4 a = *reinterpret_cast<const uint4*>(xr + 32 * k);
+        const uint4 b = *reinterpret_cast<const uint4*>(xr + 32 * k + 4);
+        const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+        for (int j = 0; j < 8; ++j) xs[k][j] = __uint_as_float(w[j] ^ sm[k][j & (NM - 1)]);
+      }
+    }
+    // ---- sum of squares: strides 64, 32 (k), 16, 8 (lanes), 4, 2, 1 (j)
+    float t8[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float s0 = xs[0][j] * xs[0][j], s1 = xs[1][j] * xs[1][j];
+      const float s2 = xs[2][j] * xs[2][j], s3 = xs[3][j] * xs[3][j];
+      t8[j] = (s0 + s2) + (s1 + s3);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) t8[j] = t8[j] + quad_xor2(t8[j]);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) t8[j] = t8[j] + quad_xor1(t8[j]);
+    const float ss = ((t8[0] + t8[4]) + (t8[2] + t8[6])) + ((t8[1] + t8[5]) + (t8[3] + t8[7]));
+    const float nrm = sqrtf(ss);
+    const float safe = fmaxf(nrm, 1e-8f);
+    const float rinv = 1.0f / safe;
+    // ---- unit vector
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float q0 = xs[k][j] * rinv;
+        const float rem = __fmaf_rn(-safe, q0, xs[k][j]);
+        xs[k][j] = __fmaf_rn(rem, rinv, q0);
+      }
+    butterfly_4lane(xs, flip1, flip2);
+    // ---- levels, 24 bits per chunk
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      uint32_t bits24 = 0;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float w = xs[k][j];
+        const float h = __builtin_amdgcn_fmed3f(__fmaf_rn(w, gs.alpha, gs.beta), 0.0f, 6.0f);
+        const int g = (int)h;
+        const uint32_t idx = (uint32_t)g + ((w > thr_s[g]) ? 1u : 0u);
+        bits24 |= idx << (3 * j);
+      }
+      chunks[v * 16 + ls + 4 * k] = bits24;
+    }
+    // ---- words: word wd of a row holds elements 10wd .. 10wd+9 = chunks (5wd)/4 and the next
+    uint32_t* prow = packed + ((int64_t)grp * rm.packed_group_stride + rin) * 13;
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const int id = it * 64 + lane;
+      if (id < kEncVecs * 13) {
+        const int vv = id / 13, wd = id - 13 * vv;
+        const int a = (5 * wd) >> 2, sh = 3 * ((10 * wd) & 7);
+        const uint32_t lo = chunks[vv * 16 + a], hi = chunks[vv * 16 + a + 1];
+        const uint32_t word = ((lo >> sh) | (hi << (24 - sh))) & (wd == 12 ? 0xFFFFFFu : 0x3FFFFFFFu);
+        prow[id] = word;
+      }
+    }
+    if (ls == 0) norms[(int64_t)grp * rm.norms_group_stride + rin + v] = nrm;
+    row0 += kEncVecs;
+    rin += kEncVecs;
+    if (rin >= (uint32_t)rm.rows_per_group) { rin = 0; ++grp; }
+  }
+}
+
 // ---------------------------------------------------------------- dequant
 template <int D, int BITS>
 __device__ __forceinline__ void load_centroid_values(const uint32_t* __restrict__ prow, const float* cb,
@@ -140,6 +350,128 @@ __global__ __launch_bounds__(kBlock) void dequant_kernel(const uint32_t* __restr
       int e = lane + 64 * i;
       if (e < D) store_from_float<TO>(orow + e, ((v[i] * s) * sg[i]) * nrm);
     }
+  }
+}
+
+// ---------------------------------------------------------------- dequant, d = 128, 3-bit
+// Same four-lanes-per-vector layout as encode128x3_kernel.  The 208 packed words of a pass are
+// read with coalesced loads into LDS; a lane cuts the 24 bits of each of its chunks out of two
+// words and looks centroid pairs up in a 64-entry table of (c[a]*s, c[b]*s).  Arithmetic per
+// element, in this order, as in dequant_kernel: butterfly, * s, * sign, * norm, round to TO.
+template <typename TO>
+__global__ __launch_bounds__(kBlock) void dequant128x3_kernel(const uint32_t* __restrict__ packed,
+                                                              const float* __restrict__ norms, Codebook cbk,
+                                                              const float* __restrict__ signs, float s,
+                                                              TO* __restrict__ out, RowMap rm, int passes) {
+  __shared__ __align__(16) float sg_s[128];
+  __shared__ __align__(8) float2 pair_s[64];
+  __shared__ uint32_t words_s[kWavesPerBlock][kEncVecs * 13 + 3];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ls = lane & 3, v = lane >> 2;
+  if (tid < 64) {
+    float clo = 0.0f, chi = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      clo = ((tid & 7) == i) ? cbk.c[i] : clo;
+      chi = ((tid >> 3) == i) ? cbk.c[i] : chi;
+    }
+    pair_s[tid] = make_float2(clo * s, chi * s);
+  }
+  if (tid >= 128) sg_s[tid - 128] = signs[tid - 128];
+  __syncthreads();
+
+  uint32_t sm[4][8];                                           // sign bit of each element of this lane
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const float4 a = *reinterpret_cast<const float4*>(&sg_s[32 * k + 8 * ls]);
+    const float4 b = *reinterpret_cast<const float4*>(&sg_s[32 * k + 8 * ls + 4]);
+    const float sv[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+    for (int j = 0; j < 8; ++j) sm[k][j] = __float_as_uint(sv[j]) & 0x80000000u;
+  }
+  const uint32_t flip1 = (ls & 1) ? 0x80000000u : 0u;
+  const uint32_t flip2 = (ls & 2) ? 0x80000000u : 0u;
+  uint32_t* words = words_s[wave];
+  // words / shifts of the 24 bits of chunk c = ls + 4k: elements 8c .. 8c+7 start in word 8c/10
+  // (chunk 15, the last 8 elements, is all of word 12: taken as word 11 >> 30, which is 0, | word 12)
+  int cw[4], csl[4], csh[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int c = ls + 4 * k;
+    cw[k] = (c == 15) ? 11 : (8 * c) / 10;
+    const int s0 = (c == 15) ? 10 : (8 * c) % 10;
+    csl[k] = 3 * s0;
+    csh[k] = 30 - 3 * s0;
+  }
+
+  const uint32_t batch0 = ((uint32_t)blockIdx.x * kWavesPerBlock + wave) * (uint32_t)passes;
+  uint32_t row0 = batch0 * kEncVecs;
+  uint32_t grp = row0 / (uint32_t)rm.rows_per_group;
+  uint32_t rin = row0 - grp * (uint32_t)rm.rows_per_group;
+
+  for (int pass = 0; pass < passes; ++pass) {
+    if (row0 >= (uint32_t)rm.n_rows) break;                    // uniform over the wavefront
+    const uint32_t* prow = packed + ((int64_t)grp * rm.packed_group_stride + rin) * 13;
+    const float nrm = norms[(int64_t)grp * rm.norms_group_stride + rin + v];
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const int id = it * 64 + lane;
+      if (id < kEncVecs * 13) words[id] = prow[id];
+    }
+    float xs[4][8];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t* rw = words + v * 13 + cw[k];
+      const uint32_t f = ((rw[0] >> csl[k]) | (rw[1] << csh[k])) & 0xFFFFFFu;
+#pragma unroll
+      for (int jp = 0; jp < 4; ++jp) {
+        const float2 c2 = pair_s[(f >> (6 * jp)) & 63u];
+        xs[k][2 * jp] = c2.x;
+        xs[k][2 * jp + 1] = c2.y;
+      }
+    }
+    butterfly_4lane(xs, flip1, flip2);
+    TO* orow = out + ((int64_t)grp * rm.out_group_stride + rin + v) * 128 + 8 * ls;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      float r[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        float t = (xs[k][j] * s) * nrm;
+        asm volatile("" : "+v"(t));                            // keep the multiply out of the narrowing convert
+        r[j] = t;
+      }
+      if (sizeof(TO) == 4) {
+        uint4 a, b;
+        a.x = __float_as_uint(r[0]) ^ sm[k][0]; a.y = __float_as_uint(r[1]) ^ sm[k][1];
+        a.z = __float_as_uint(r[2]) ^ sm[k][2]; a.w = __float_as_uint(r[3]) ^ sm[k][3];
+        b.x = __float_as_uint(r[4]) ^ sm[k][4]; b.y = __float_as_uint(r[5]) ^ sm[k][5];
+        b.z = __float_as_uint(r[6]) ^ sm[k][6]; b.w = __float_as_uint(r[7]) ^ sm[k][7];
+        *reinterpret_cast<uint4*>(orow + 32 * k) = a;
+        *reinterpret_cast<uint4*>(orow + 32 * k + 4) = b;
+      } else {
+        uint32_t w[4];
+#pragma unroll
+        for (int jp = 0; jp < 4; ++jp) {
+          uint32_t lo, hi;
+          if (__is_same(TO, __half)) {
+            lo = __half_as_ushort(__float2half_rn(r[2 * jp]));
+            hi = __half_as_ushort(__float2half_rn(r[2 * jp + 1]));
+          } else {
+            lo = __bfloat16_as_ushort(__float2bfloat16(r[2 * jp]));
+            hi = __bfloat16_as_ushort(__float2bfloat16(r[2 * jp + 1]));
+          }
+          w[jp] = (lo | (hi << 16)) ^ ((sm[k][2 * jp] >> 16) | sm[k][2 * jp + 1]);
+        }
+        *reinterpret_cast<uint4*>(orow + 32 * k) = make_uint4(w[0], w[1], w[2], w[3]);
+      }
+    }
+    row0 += kEncVecs;
+    rin += kEncVecs;
+    if (rin >= (uint32_t)rm.rows_per_group) { rin = 0; ++grp; }
   }
 }
 
@@ -241,6 +573,56 @@ float double_rounding_threshold(float b, float s) {
   return ord2f(lo);
 }
 
+// Finds alpha, beta with  j <= alpha * t[j] + beta < j + 1  for every threshold j (with margin), so
+// that floor(alpha * w + beta), clamped to 0..nb-1, is the count of thresholds below w or one
+// less.  False when no such line exists (then the generic kernel counts them one by one).
+bool level_guess_search(const float* t, int nb, EncodeGuess& out);
+
+// The search result is kept for the last threshold set seen.
+bool level_guess(const float* t, int nb, EncodeGuess& out) {
+  static std::mutex mu;
+  static float last_t[15];
+  static int last_nb = 0;
+  static bool last_ok = false;
+  static EncodeGuess last_out;
+  std::lock_guard<std::mutex> lock(mu);
+  if (last_nb != nb || memcmp(last_t, t, nb * sizeof(float)) != 0) {
+    last_ok = level_guess_search(t, nb, last_out);
+    memcpy(last_t, t, nb * sizeof(float));
+    last_nb = nb;
+  }
+  out = last_out;
+  return last_ok;
+}
+
+bool level_guess_search(const float* t, int nb, EncodeGuess& out) {
+  for (int i = 0; i < nb; ++i)
+    if (!std::isfinite(t[i]) || (i > 0 && !(t[i] > t[i - 1]))) return false;
+  const double span = (double)t[nb - 1] - (double)t[0];
+  if (!(span > 0)) return false;
+  double best_w = 0.0, best_a = 0.0, best_b = 0.0;
+  for (int s = 1; s <= 4000; ++s) {
+    const double a = (double)(nb + 1) * s / (1000.0 * span);       // up to 4x the mean level density
+    double lo = -1e300, hi = 1e300;
+    for (int j = 0; j < nb; ++j) {
+      lo = std::fmax(lo, j - a * (double)t[j]);
+      hi = std::fmin(hi, j + 1 - a * (double)t[j]);
+    }
+    if (hi - lo > best_w) { best_w = hi - lo; best_a = a; best_b = 0.5 * (lo + hi); }
+  }
+  if (best_w < 0.1) return false;
+  out.alpha = (float)best_a;
+  out.beta = (float)best_b;
+  return true;
+}
+
+// Passes per wavefront of the four-lanes-per-vector kernels: several, to spread the set-up cost,
+// once every CU has a few workgroups anyway.
+int fast_passes(int64_t n_rows) {
+  const int64_t rows_per_block_pass = (int64_t)kEncVecs * kWavesPerBlock;
+  return (n_rows >= rows_per_block_pass * kEncPasses * 256 * 4) ? kEncPasses : 1;
+}
+
 int grid_for_rows(int64_t rows) {
   int64_t blocks = (rows + kWavesPerBlock - 1) / kWavesPerBlock;
   const int64_t cap = 256 * 16;  // 16 blocks of 4 waves per CU keeps every SIMD supplied
@@ -298,6 +680,22 @@ extern "C" int tq_encode(const void* x, int x_dtype, const float* signs, const f
   RowMap rm{n_rows, rows_per_group, packed_group_stride, norms_group_stride, 0};
   hipStream_t stream = (hipStream_t)stream_;
   const int grid = grid_for_rows(n_rows);
+  EncodeGuess gs{};
+  if (dim == 128 && bits == 3 && rows_per_group % kEncVecs == 0 && n_rows < (int64_t)1 << 31 &&
+      tq::aligned(x, 16) && level_guess(thr.t, nb, gs)) {
+    const int passes = fast_passes(n_rows);
+    const int64_t rows_per_block = (int64_t)kEncVecs * passes * kWavesPerBlock;
+    const int fgrid = (int)((n_rows + rows_per_block - 1) / rows_per_block);
+    if (x_dtype == TQ_F32)
+      encode128x3_kernel<float><<<fgrid, kBlock, 0, stream>>>((const float*)x, signs, thr, gs, packed, norms, rm, passes);
+    else if (x_dtype == TQ_F16)
+      encode128x3_kernel<__half><<<fgrid, kBlock, 0, stream>>>((const __half*)x, signs, thr, gs, packed, norms, rm, passes);
+    else
+      encode128x3_kernel<__hip_bfloat16><<<fgrid, kBlock, 0, stream>>>((const __hip_bfloat16*)x, signs, thr, gs,
+                                                                      packed, norms, rm, passes);
+    TQ_CHECK_LAUNCH("tq_encode launch");
+    return TQ_OK;
+  }
 #define LAUNCH_ENC(T)                                                                               \
   TQ_DISPATCH_DIM(dim, TQ_DISPATCH_BITS(bits, (encode_kernel<D_, B_, T><<<grid, kBlock, 0, stream>>>( \
                                                   (const T*)x, signs, thr, packed, norms, rm))))
@@ -328,6 +726,21 @@ extern "C" int tq_dequant(const uint32_t* packed, const float* norms, const floa
   RowMap rm{n_rows, rows_per_group, packed_group_stride, norms_group_stride, out_group_stride};
   hipStream_t stream = (hipStream_t)stream_;
   const int grid = grid_for_rows(n_rows);
+  if (dim == 128 && bits == 3 && rows_per_group % kEncVecs == 0 && n_rows < (int64_t)1 << 31 &&
+      tq::aligned(out, 16) && (out_group_stride * 128 * (int64_t)tq::dtype_size(out_dtype)) % 16 == 0) {
+    const int passes = fast_passes(n_rows);
+    const int64_t rows_per_block = (int64_t)kEncVecs * passes * kWavesPerBlock;
+    const int fgrid = (int)((n_rows + rows_per_block - 1) / rows_per_block);
+    if (out_dtype == TQ_F32)
+      dequant128x3_kernel<float><<<fgrid, kBlock, 0, stream>>>(packed, norms, cb, signs, s, (float*)out, rm, passes);
+    else if (out_dtype == TQ_F16)
+      dequant128x3_kernel<__half><<<fgrid, kBlock, 0, stream>>>(packed, norms, cb, signs, s, (__half*)out, rm, passes);
+    else
+      dequant128x3_kernel<__hip_bfloat16><<<fgrid, kBlock, 0, stream>>>(packed, norms, cb, signs, s,
+                                                                       (__hip_bfloat16*)out, rm, passes);
+    TQ_CHECK_LAUNCH("tq_dequant launch");
+    return TQ_OK;
+  }
 #define LAUNCH_DEQ(T)                                                                                 \
   TQ_DISPATCH_DIM(dim, TQ_DISPATCH_BITS(bits, (dequant_kernel<D_, B_, T><<<grid, kBlock, 0, stream>>>( \
                                                   packed, norms, cb, signs, s, (T*)out, rm))))

@@ -10,6 +10,8 @@ from .adaptive import make_adaptive_cache
 from .quantizer import PolarQuantizer
 from .ops import (
     fused_quantize,
+    encode_into,
+    dequant_into,
     dequant_fp16,
     packed_dequantize,
     packed_fused_qk_scores,
