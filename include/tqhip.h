@@ -245,6 +245,33 @@ int tq_vonly_decode_attn_phases(const void* q, int q_dtype, const void* k_f16,
  */
 size_t tq_workspace_bytes(int op, int n_seq, int n_q_heads, int64_t max_seq_len, int dim);
 
+/*
+ * Chunked-prefill attention: n_rows query rows per q head (positions q_pos0 .. q_pos0 + n_rows - 1)
+ * against kv_len cached positions held PACKED (K and V), causal when `causal` != 0 (row i sees
+ * positions <= q_pos0 + i).  No kernel of the reference does this: its prefill dequantises the
+ * whole cache to fp16 and runs stock SDPA over it (cache.py:125-129, 209-210 feeding
+ * mlx-lm's scaled_dot_product_attention); the arithmetic here is flash_attention.py:79-162
+ * (rotated-domain scores and value sum, one butterfly per output row) applied to many rows.
+ *   q   [n_kv*n_rep, n_rows, dim] q_dtype, contiguous, NOT pre-rotated (k_signs are applied here)
+ *   k_packed / v_packed [n_kv, *_head_stride rows, pdim], k_norms / v_norms [n_kv, *_head_stride]
+ *   out [n_kv*n_rep, n_rows, dim] out_dtype, contiguous
+ * Matrix-core kernel: q_rot, the centroids and softmax weights * value norm are fp16 operands,
+ * accumulation is float32.  dim 128 / 3-bit only (TQ_ERR_UNSUPPORTED otherwise).  The workspace
+ * (tq_prefill_workspace_bytes, 256-byte aligned) is scratch as for the decode ops.
+ */
+int tq_prefill_attn(const void* q, int q_dtype,
+                    const uint32_t* k_packed, const float* k_norms,
+                    const uint32_t* v_packed, const float* v_norms,
+                    const float* k_centroids /* host */, const float* v_centroids /* host */,
+                    const float* k_signs, const float* v_signs,
+                    void* out, int out_dtype, void* workspace, size_t workspace_bytes,
+                    int n_kv_heads, int n_rep, int64_t n_rows, int64_t kv_len, int64_t q_pos0,
+                    int64_t k_head_stride, int64_t kn_head_stride,
+                    int64_t v_head_stride, int64_t vn_head_stride,
+                    int dim, int bits, float attn_scale, int causal, tq_stream_t stream);
+
+size_t tq_prefill_workspace_bytes(int n_q_heads, int64_t n_rows, int64_t kv_len, int dim);
+
 #ifdef __cplusplus
 }
 #endif

@@ -419,3 +419,32 @@ def dense_attention(q, k, v, attn_scale: float, mask=None) -> np.ndarray:
             if np.asarray(mask).ndim == 3 else s + np.asarray(mask, dtype=np.float64)
     w = _softmax64(s)
     return np.einsum("grqt,gtd->grqd", w, v).reshape(n_q, S_q, v.shape[-1])
+
+
+def prefill_attention(q, k_packed, k_norms, v_packed, v_norms, k_centroids, v_centroids, k_signs,
+                      v_signs, dim: int, bits: int, attn_scale: float, q_pos0: int, n_rep: int = 1,
+                      causal: bool = True) -> np.ndarray:
+    """Chunk of query rows against a packed cache, as the reference's prefill computes it:
+    dequantise K and V (cache.py:125-129, 209-210 -> quantizer.py:108-132) and run plain
+    softmax attention with the causal rule "row i sees positions <= q_pos0 + i"
+    (cache.py:314-334 builds that mask with mlx-lm's create_causal_mask(N, offset)).
+
+    q: (n_q, n_rows, dim); k_packed/v_packed: (n_kv, T, pdim); norms (n_kv, T).  float64 result
+    (n_q, n_rows, dim)."""
+    q = np.asarray(q)
+    n_q, n_rows, _ = q.shape
+    n_kv, T = np.asarray(k_norms).shape
+    if n_q != n_kv * n_rep:
+        raise ValueError(
+            f"n_q_heads ({n_q}) must equal n_kv_heads ({n_kv}) * n_rep ({n_rep})")
+    pd = packed_dim(dim, bits)
+    k = packed_dequantize(np.asarray(k_packed).reshape(-1, pd), np.asarray(k_norms).reshape(-1),
+                          k_centroids, k_signs, dim, bits).reshape(n_kv, T, dim)
+    v = packed_dequantize(np.asarray(v_packed).reshape(-1, pd), np.asarray(v_norms).reshape(-1),
+                          v_centroids, v_signs, dim, bits).reshape(n_kv, T, dim)
+    mask = None
+    if causal:
+        pos = np.arange(T)[None, :]
+        row = np.arange(n_rows)[:, None] + int(q_pos0)
+        mask = np.where(pos <= row, 0.0, -np.inf)                      # (n_rows, T), broadcast over heads
+    return dense_attention(q.astype(np.float64), k, v, attn_scale, mask)

@@ -664,3 +664,81 @@ def test_config4_flash_ragged_full_heads(tq):
         want = o.flash_attention_turboquant(o.prerotate_query(q[i], ks), kp[:, a:e], kn[:, a:e], vp[:, a:e],
                                             vn[:, a:e], c, c, vs, D, bits, sc, 16, n_rep)
         close(got[i], want)
+
+
+# ------------------------------------------------------------------ chunked prefill over packed K/V
+
+def _prefill_case(rng, n_kv, n_rep, T, n_rows, outliers=False):
+    c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, n_kv, T, 128, 3, outliers=outliers)
+    q = rng.standard_normal((n_kv * n_rep, n_rows, 128)).astype(np.float16)
+    if outliers:
+        q[..., 7] *= 20
+    return c, ks, vs, kp, kn, vp, vn, q
+
+
+@pytest.mark.parametrize("n_kv,n_rep,T,n_rows,pos0", [
+    (2, 2, 300, 300, 0),        # whole prompt in one chunk, ragged everywhere
+    (2, 4, 1000, 256, 744),     # tail chunk of exactly one workgroup of rows
+    (1, 1, 777, 130, 500),      # chunk in the middle of a longer cache (positions past it are ignored)
+    (2, 2, 2500, 513, 1987),    # three row blocks, several splits
+])
+def test_prefill_attention_matches_oracle(tq, n_kv, n_rep, T, n_rows, pos0):
+    rng = np.random.default_rng(51)
+    c, ks, vs, kp, kn, vp, vn, q = _prefill_case(rng, n_kv, n_rep, T, n_rows)
+    sc = 1 / math.sqrt(128)
+    want = o.prefill_attention(q, kp, kn, vp, vn, c, c, ks, vs, 128, 3, sc, pos0, n_rep)
+    got = tq.prefill_attention(dev(q), dev(kp), dev(kn), dev(vp), dev(vn), c, c, dev(ks), dev(vs), 128, 3, sc,
+                               n_rep=n_rep, q_pos0=pos0, out_dtype=torch.float32)
+    assert got.shape == (n_kv * n_rep, n_rows, 128)
+    close(host(got).reshape(-1, 128), want.reshape(-1, 128), row_scale=True)
+    rel = np.abs(host(got) - want).max() / np.abs(want).max()
+    assert rel < 1e-3, rel
+
+
+def test_prefill_attention_noncausal_fp16_out_and_outliers(tq):
+    """1 % outlier channels (x20) in K, V and q as in BASELINE config 5; fp16 output; and the
+    non-causal form, where every row sees every position."""
+    rng = np.random.default_rng(52)
+    n_kv, n_rep, T, n_rows = 2, 4, 1500, 200
+    c, ks, vs, kp, kn, vp, vn, q = _prefill_case(rng, n_kv, n_rep, T, n_rows, outliers=True)
+    sc = 1 / math.sqrt(128)
+    for causal in (True, False):
+        want = o.prefill_attention(q, kp, kn, vp, vn, c, c, ks, vs, 128, 3, sc, T - n_rows, n_rep, causal=causal)
+        got = tq.prefill_attention(dev(q), dev(kp), dev(kn), dev(vp), dev(vn), c, c, dev(ks), dev(vs), 128, 3, sc,
+                                   n_rep=n_rep, causal=causal)
+        assert got.dtype == torch.float16
+        err = np.abs(host(got).astype(np.float64) - want)
+        scale = np.abs(want).max(axis=-1, keepdims=True)
+        assert (err <= 1e-3 + 3e-3 * scale).all(), (err / scale).max()     # + fp16 rounding of the output
+
+
+def test_prefill_attention_equals_decode_rows(tq):
+    """Each row of a prefill chunk is one decode step over its prefix: compare with the
+    float32 flash decode kernel of this library (independent code path)."""
+    rng = np.random.default_rng(53)
+    n_kv, n_rep, T, n_rows = 2, 2, 640, 64
+    c, ks, vs, kp, kn, vp, vn, q = _prefill_case(rng, n_kv, n_rep, T, n_rows)
+    sc = 1 / math.sqrt(128)
+    got = host(tq.prefill_attention(dev(q), dev(kp), dev(kn), dev(vp), dev(vn), c, c, dev(ks), dev(vs), 128, 3, sc,
+                                    n_rep=n_rep, out_dtype=torch.float32))
+    for i in (0, 17, 63):
+        L = T - n_rows + i + 1
+        q_rot = tq.prerotate_query(dev(q[:, i]), dev(ks))
+        ref = host(tq.flash_attention_turboquant(q_rot, dev(kp[:, :L]), dev(kn[:, :L]), dev(vp[:, :L]), dev(vn[:, :L]),
+                                                 c, c, dev(vs), 128, 3, sc, n_rep=n_rep, precision="fp32"))
+        close(got[:, i], ref, row_scale=True)
+
+
+def test_prefill_attention_argument_errors(tq):
+    rng = np.random.default_rng(54)
+    c, ks, vs, kp, kn, vp, vn, q = _prefill_case(rng, 2, 2, 128, 16)
+    args = (dev(kp), dev(kn), dev(vp), dev(vn), c, c, dev(ks), dev(vs))
+    with pytest.raises(ValueError):
+        tq.prefill_attention(dev(q), *args, 128, 3, 0.1, n_rep=3)                 # 4 q heads != 2 * 3
+    with pytest.raises(ValueError):
+        tq.prefill_attention(dev(q), *args, 128, 3, 0.1, n_rep=2, q_pos0=500)     # chunk starts past the cache
+    with pytest.raises(RuntimeError):
+        tq.prefill_attention(dev(q[..., :64]), dev(kp), dev(kn), dev(vp), dev(vn), c, c, dev(ks[:64]), dev(vs[:64]),
+                             64, 3, 0.1, n_rep=2)                                 # no kernel for d = 64
+    empty = tq.prefill_attention(dev(q[:, :0]), *args, 128, 3, 0.1, n_rep=2, q_pos0=0)
+    assert empty.shape == (4, 0, 128)

@@ -409,3 +409,32 @@ def test_vonly_decode_equals_dense_attention():
     full = o.dense_attention(q.astype(np.float64)[:, None, :], K, V, sc)[:, 0, :]
     cosv = (got * full).sum() / np.linalg.norm(got) / np.linalg.norm(full)
     assert cosv > 0.95
+
+
+def test_prefill_attention_rows_are_prefix_flash_decodes():
+    """Pins the causal indexing of prefill_attention: row i of a chunk that starts at q_pos0 must be
+    the single-token flash attention (rotated-domain formula, pinned above) over positions
+    0 .. q_pos0 + i; and without the causal rule every row sees all positions."""
+    rng = np.random.default_rng(77)
+    n_kv, n_rep, T, D, bits, n_rows, pos0 = 2, 2, 50, 128, 3, 7, 43
+    c = o.gaussian_codebook(bits)
+    b = o.gaussian_boundaries(c)
+    ks, vs = o.random_diagonal_sign(D, 42), o.random_diagonal_sign(D, 43)
+    K = rng.standard_normal((n_kv * T, D)).astype(np.float16)
+    V = rng.standard_normal((n_kv * T, D)).astype(np.float16)
+    kp, kn = o.fused_quantize(K, ks, b, D, bits)
+    vp, vn = o.fused_quantize(V, vs, b, D, bits)
+    kp, vp = kp.reshape(n_kv, T, -1), vp.reshape(n_kv, T, -1)
+    kn, vn = kn.reshape(n_kv, T), vn.reshape(n_kv, T)
+    q = rng.standard_normal((n_kv * n_rep, n_rows, D)).astype(np.float32)
+    sc = 1 / np.sqrt(D)
+    got = o.prefill_attention(q, kp, kn, vp, vn, c, c, ks, vs, D, bits, sc, pos0, n_rep)
+    assert got.shape == (n_kv * n_rep, n_rows, D)
+    for i in (0, 3, n_rows - 1):
+        L = pos0 + i + 1
+        want = o.flash_attention_turboquant(o.prerotate_query(q[:, i], ks), kp[:, :L], kn[:, :L], vp[:, :L],
+                                            vn[:, :L], c, c, vs, D, bits, sc, 16, n_rep)
+        assert np.allclose(got[:, i], want, rtol=1e-5, atol=1e-6)
+    full = o.prefill_attention(q, kp, kn, vp, vn, c, c, ks, vs, D, bits, sc, pos0, n_rep, causal=False)
+    want = o.flash_attention_turboquant(o.prerotate_query(q[:, 2], ks), kp, kn, vp, vn, c, c, vs, D, bits, sc, 16, n_rep)
+    assert np.allclose(full[:, 2], want, rtol=1e-5, atol=1e-6)

@@ -463,44 +463,6 @@ void fill_codebook(Codebook& cb, const float* c, int bits) {
   for (int i = 0; i < 16; ++i) cb.c[i] = (c && i < (1 << bits)) ? c[i] : 0.0f;
 }
 
-// The matrix-core kernels hold the codebook as fp16.  Rounding the 2^bits levels to fp16 is a
-// systematic error (the same few values at every position, so it does not average out over a
-// sequence); multiplying the table by a scale a in [1, 2) first and dividing the result by a
-// afterwards (in float32) leaves the mathematics alone, and a can be chosen so that every a*c[i]
-// lies within a few 2^-16 of an fp16 value.  Returns 1/a; the search result is kept for the last
-// table seen.
-float fill_codebook_fp16(Codebook& cb, const float* c, int bits) {
-  static std::mutex mu;
-  static float last_c[16], last_scale = 0.0f;
-  static int last_n = 0;
-  const int n = 1 << bits;
-  float scale = 1.0f;
-  {
-    std::lock_guard<std::mutex> lock(mu);
-    if (last_n == n && last_scale != 0.0f && std::memcmp(last_c, c, n * sizeof(float)) == 0) {
-      scale = last_scale;
-    } else {
-      double best = 1e30;
-      for (int j = 0; j < 65536; ++j) {
-        const float a = 1.0f + (float)j * (1.0f / 65536.0f);
-        double worst = 0.0;
-        for (int i = 0; i < n && worst < best; ++i) {
-          const float v = a * c[i];
-          if (v == 0.0f) continue;
-          const float r = (float)(_Float16)v;
-          worst = std::fmax(worst, std::fabs(((double)r - (double)v) / (double)v));
-        }
-        if (worst < best) { best = worst; scale = a; }
-      }
-      std::memcpy(last_c, c, n * sizeof(float));
-      last_n = n;
-      last_scale = scale;
-    }
-  }
-  for (int i = 0; i < 16; ++i) cb.c[i] = (i < n) ? scale * c[i] : 0.0f;
-  return 1.0f / scale;
-}
-
 int check_heads(int n_kv, int n_rep, const char* who) {
   if (n_kv < 1) return tq::fail(TQ_ERR_ARG, "%s: n_kv_heads must be >= 1, got %d", who, n_kv);
   if (n_rep < 1) return tq::fail(TQ_ERR_NREP, "%s: n_rep must be >= 1, got %d", who, n_rep);
@@ -599,7 +561,7 @@ int launch_vonly_mfma(const void* q, const void* k_f16, const uint32_t* v_packed
   }
 #endif
   Codebook vcb;
-  a.v_unscale = fill_codebook_fp16(vcb, v_centroids, sh.bits);
+  a.v_unscale = tq::fill_codebook_fp16(vcb, v_centroids, sh.bits);
   if (phases & 1) {
     dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
     tqm::vonly_tile_mfma_kernel<<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb);
@@ -650,8 +612,8 @@ int launch_packed_mfma(const float* q_rot_or_weights, const uint32_t* k_packed, 
   a.threshold = threshold;
   Codebook kcb, vcb;
   fill_codebook(kcb, nullptr, sh.bits);
-  if (MODE != tqm::kWeights) a.score_scale *= fill_codebook_fp16(kcb, k_centroids, sh.bits);
-  a.v_unscale = fill_codebook_fp16(vcb, v_centroids, sh.bits);
+  if (MODE != tqm::kWeights) a.score_scale *= tq::fill_codebook_fp16(kcb, k_centroids, sh.bits);
+  a.v_unscale = tq::fill_codebook_fp16(vcb, v_centroids, sh.bits);
   dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
   tqm::packed_tile_mfma_kernel<MODE><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, kcb, vcb);
   TQ_CHECK_LAUNCH(who);
@@ -716,7 +678,7 @@ extern "C" int tq_prerot_qk_scores(const float* q_rot, const uint32_t* k_packed,
     a.seq_len = seq_len; a.k_head_stride = packed_head_stride; a.kn_head_stride = norms_head_stride;
     a.n_kv = n_kv_heads; a.n_rep = n_rep; a.n_tiles_max = 1;
     Codebook cbh;
-    a.score_scale = fill_codebook_fp16(cbh, centroids, bits) / (float)dim;
+    a.score_scale = tq::fill_codebook_fp16(cbh, centroids, bits) / (float)dim;
     dim3 grid((unsigned)((seq_len + tqm::kTilePos - 1) / tqm::kTilePos), n_kv_heads, 1);
     tqm::packed_tile_mfma_kernel<tqm::kScores><<<grid, tqm::kMfmaThreads, 0, (hipStream_t)stream_>>>(a, cbh, cbh);
     TQ_CHECK_LAUNCH("tq_prerot_qk_scores launch");

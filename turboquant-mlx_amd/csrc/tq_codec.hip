@@ -109,52 +109,6 @@ constexpr int kEncPasses = 4;     // passes per wavefront once there are rows en
 
 struct EncodeGuess { float alpha, beta; };
 
-__device__ __forceinline__ float quad_xor1(float v) {
-  return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true));   // lanes 1,0,3,2
-}
-__device__ __forceinline__ float quad_xor2(float v) {
-  return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xF, 0xF, true));   // lanes 2,3,0,1
-}
-
-// Raw butterfly of a 128-vector spread over four lanes (element e = 32k + 8*ls + j in xs[k][j] of
-// lane ls), stages in the order of strides 1, 2, ..., 64.  flip1 / flip2 are 0x80000000 in the
-// lanes whose ls has bit 0 / bit 1 set (the upper element of a pair computes partner - own).
-__device__ __forceinline__ void butterfly_4lane(float (&xs)[4][8], uint32_t flip1, uint32_t flip2) {
-#pragma unroll
-  for (int k = 0; k < 4; ++k) {
-#pragma unroll
-    for (int h = 1; h < 8; h <<= 1)
-#pragma unroll
-      for (int j = 0; j < 8; ++j)
-        if (!(j & h)) {
-          const float a = xs[k][j], b = xs[k][j + h];
-          xs[k][j] = a + b;
-          xs[k][j + h] = a - b;
-        }
-  }
-#pragma unroll
-  for (int k = 0; k < 4; ++k)
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const float a = xs[k][j];
-      xs[k][j] = quad_xor1(a) + __uint_as_float(__float_as_uint(a) ^ flip1);
-    }
-#pragma unroll
-  for (int k = 0; k < 4; ++k)
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const float a = xs[k][j];
-      xs[k][j] = quad_xor2(a) + __uint_as_float(__float_as_uint(a) ^ flip2);
-    }
-#pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const float a0 = xs[0][j] + xs[1][j], a1 = xs[0][j] - xs[1][j];
-    const float a2 = xs[2][j] + xs[3][j], a3 = xs[2][j] - xs[3][j];
-    xs[0][j] = a0 + a2; xs[2][j] = a0 - a2;
-    xs[1][j] = a1 + a3; xs[3][j] = a1 - a3;
-  }
-}
-
 template <typename T>
 __global__ __launch_bounds__(kBlock) void encode128x3_kernel(const T* __restrict__ x,
                                                              const float* __restrict__ signs, Thresholds thr,

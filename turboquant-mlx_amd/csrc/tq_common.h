@@ -7,6 +7,9 @@
 #include <stdint.h>
 #include <stdio.h>
 #include <stdarg.h>
+#include <cmath>
+#include <cstring>
+#include <mutex>
 
 #include "../../include/tqhip.h"
 
@@ -169,6 +172,52 @@ template <> __device__ __forceinline__ void store_from_float<__hip_bfloat16>(__h
   *p = __float2bfloat16(v);
 }
 
+__device__ __forceinline__ float quad_xor1(float v) {
+  return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true));   // lanes 1,0,3,2
+}
+__device__ __forceinline__ float quad_xor2(float v) {
+  return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xF, 0xF, true));   // lanes 2,3,0,1
+}
+
+// Raw butterfly of a 128-vector spread over four lanes (element e = 32k + 8*ls + j in xs[k][j] of
+// lane ls), stages in the order of strides 1, 2, ..., 64.  flip1 / flip2 are 0x80000000 in the
+// lanes whose ls has bit 0 / bit 1 set (the upper element of a pair computes partner - own).
+__device__ __forceinline__ void butterfly_4lane(float (&xs)[4][8], uint32_t flip1, uint32_t flip2) {
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+#pragma unroll
+    for (int h = 1; h < 8; h <<= 1)
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (!(j & h)) {
+          const float a = xs[k][j], b = xs[k][j + h];
+          xs[k][j] = a + b;
+          xs[k][j + h] = a - b;
+        }
+  }
+#pragma unroll
+  for (int k = 0; k < 4; ++k)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float a = xs[k][j];
+      xs[k][j] = quad_xor1(a) + __uint_as_float(__float_as_uint(a) ^ flip1);
+    }
+#pragma unroll
+  for (int k = 0; k < 4; ++k)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float a = xs[k][j];
+      xs[k][j] = quad_xor2(a) + __uint_as_float(__float_as_uint(a) ^ flip2);
+    }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const float a0 = xs[0][j] + xs[1][j], a1 = xs[0][j] - xs[1][j];
+    const float a2 = xs[2][j] + xs[3][j], a3 = xs[2][j] - xs[3][j];
+    xs[0][j] = a0 + a2; xs[2][j] = a0 - a2;
+    xs[1][j] = a1 + a3; xs[3][j] = a1 - a3;
+  }
+}
+
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
   for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, shfl_xor_f(v, m));
@@ -182,3 +231,45 @@ __device__ __forceinline__ float wave_sum(float v) {
 }
 
 }  // namespace tqd
+
+namespace tq {
+
+// The matrix-core kernels hold the codebook as fp16.  Rounding the 2^bits levels to fp16 is a
+// systematic error (the same few values at every position, so it does not average out over a
+// sequence); multiplying the table by a scale a in [1, 2) first and dividing the result by a
+// afterwards (in float32) leaves the mathematics alone, and a can be chosen so that every a*c[i]
+// lies within a few 2^-16 of an fp16 value.  Returns 1/a; the search result is kept for the last
+// table seen.
+inline float fill_codebook_fp16(tqd::Codebook& cb, const float* c, int bits) {
+  static std::mutex mu;
+  static float last_c[16], last_scale = 0.0f;
+  static int last_n = 0;
+  const int n = 1 << bits;
+  float scale = 1.0f;
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    if (last_n == n && last_scale != 0.0f && std::memcmp(last_c, c, n * sizeof(float)) == 0) {
+      scale = last_scale;
+    } else {
+      double best = 1e30;
+      for (int j = 0; j < 65536; ++j) {
+        const float a = 1.0f + (float)j * (1.0f / 65536.0f);
+        double worst = 0.0;
+        for (int i = 0; i < n && worst < best; ++i) {
+          const float v = a * c[i];
+          if (v == 0.0f) continue;
+          const float r = (float)(_Float16)v;
+          worst = std::fmax(worst, std::fabs(((double)r - (double)v) / (double)v));
+        }
+        if (worst < best) { best = worst; scale = a; }
+      }
+      std::memcpy(last_c, c, n * sizeof(float));
+      last_n = n;
+      last_scale = scale;
+    }
+  }
+  for (int i = 0; i < 16; ++i) cb.c[i] = (i < n) ? scale * c[i] : 0.0f;
+  return 1.0f / scale;
+}
+
+}  // namespace tq

@@ -22,6 +22,7 @@ from .ops import (
     count_active_positions,
     flash_attention_turboquant,
     flash_decode,
+    prefill_attention,
     vonly_decode,
     dense_qk_scores,
     softmax_rows,

@@ -6,7 +6,7 @@ back-to-back launches, and rotation over several independent input sets so that 
 Infinity Cache cannot serve the reads.  Prints one line per case: us per call, GB/s of algorithmic
 bytes and the fraction of 8 TB/s.
 
-    python -m tqhip.bench_kernels [--iters 200] [--cases encode,scores,flash,sparse_v,vonly]
+    python -m tqhip.bench_kernels [--iters 200] [--cases encode,scores,flash,sparse_v,vonly,prefill]
 """
 from __future__ import annotations
 
@@ -126,7 +126,28 @@ def bench_vonly(iters, dev):
         report(f"config 2 shape: V-only decode 28/4 heads, T={T} (python-call launch)", timeit(fns, iters), nbytes)
 
 
-CASES = {"encode": bench_encode, "scores": bench_scores, "sparse_v": bench_sparse_v, "flash": bench_flash,
+def bench_prefill(iters, dev):
+    """BASELINE config 5, attention half: a chunk of 512 query rows x 32 heads at the end of a
+    131072-position packed cache (8 kv heads), causal.  Matrix-core bound: reported in TFLOP/s of
+    the 4 * rows * heads * d * visible-positions useful flops against the 2.5 PFLOP/s fp16 peak."""
+    cb = gaussian_codebook(3)
+    ks = tqhip.random_diagonal_sign(128, 42, device=dev)
+    vs = tqhip.random_diagonal_sign(128, 43, device=dev)
+    n_rows = 512
+    for T in (8192, 32768, 131072):
+        (kp, kn), (vp, vn) = packed_sets(8, T, dev, 1, 8)[0], packed_sets(8, T, dev, 1, 9)[0]
+        q = torch.randn((32, n_rows, 128), device=dev, dtype=torch.float16)
+        fn = lambda: tqhip.prefill_attention(q, kp, kn, vp, vn, cb, cb, ks, vs, 128, 3, 1 / math.sqrt(128), n_rep=4)
+        us = timeit([fn], max(5, iters // 20), warmup=2)
+        visible = sum(T - n_rows + i + 1 for i in range(n_rows))
+        flops = 4.0 * 32 * 128 * visible
+        nbytes = 8 * T * 112 + 2 * 32 * n_rows * 256
+        print(f"config 5: prefill chunk 512 rows x 32/8 heads, T={T:<7d} {us:10.1f} us  {flops / us / 1e6:8.1f} TFLOP/s  "
+              f"{100 * flops / us / 1e6 / 2500:5.1f} % of 2.5 PFLOP/s  ({nbytes / us / 1e3:6.1f} GB/s of packed cache)",
+              flush=True)
+
+
+CASES = {"prefill": bench_prefill, "encode": bench_encode, "scores": bench_scores, "sparse_v": bench_sparse_v, "flash": bench_flash,
          "vonly": bench_vonly}
 
 

@@ -550,3 +550,54 @@ def vonly_decode(q: torch.Tensor, k: torch.Tensor, v_packed, v_norms, v_centroid
         _ptr(q), _dt(q), _ptr(k), _ptr(v_packed), _ptr(v_norms), _host_table(v_centroids), _ptr(v_signs),
         _ptr(out), _ptr(ws), ws.numel(), C.byref(sh), stream))
     return out
+
+
+def prefill_attention(q: torch.Tensor, k_packed, k_norms, v_packed, v_norms, k_centroids, v_centroids,
+                      k_signs, v_signs, dim: int, bits: int, attn_scale: float, *, n_rep: int = 1,
+                      kv_len: int | None = None, q_pos0: int | None = None, causal: bool = True,
+                      out_dtype=None) -> torch.Tensor:
+    """Chunked-prefill attention over packed K and V on the matrix cores (tq_prefill_attn).
+
+    The reference dequantises the whole cache and calls stock SDPA for this step (cache.py:125-129,
+    209-210); here the packed rows are decoded tile by tile in LDS and never written back.
+
+    q (n_q, n_rows, dim) fp16/bf16/fp32, not pre-rotated; k_packed / v_packed (n_kv, T_alloc, pdim) uint32,
+    k_norms / v_norms (n_kv, T_alloc) fp32; the first kv_len positions are attended (default T_alloc).
+    q_pos0 is the cache position of query row 0 (default kv_len - n_rows: the chunk is the cache's
+    tail).  Returns (n_q, n_rows, dim) in out_dtype (default q.dtype).
+    """
+    _need_gpu(q, k_packed, k_norms, v_packed, v_norms)
+    n_q, n_rows, _ = q.shape
+    n_kv = k_norms.shape[0]
+    _check_gqa(n_q, n_kv, n_rep)
+    pd = packed_dim(dim, bits)
+    if q.dtype not in _DTYPES:
+        q = q.float()
+    q = q.contiguous()
+    k_packed = _u32(k_packed)
+    v_packed = _u32(v_packed)
+    if k_packed.stride(-1) != 1 or k_packed.stride(-2) != pd or v_packed.stride(-1) != 1 or v_packed.stride(-2) != pd:
+        k_packed, v_packed = k_packed.contiguous(), v_packed.contiguous()
+    k_norms = k_norms.to(torch.float32)
+    v_norms = v_norms.to(torch.float32)
+    if k_norms.stride(-1) != 1 or v_norms.stride(-1) != 1:
+        k_norms, v_norms = k_norms.contiguous(), v_norms.contiguous()
+    T = int(kv_len if kv_len is not None else k_norms.shape[-1])
+    pos0 = int(q_pos0 if q_pos0 is not None else T - n_rows)
+    out_dtype = out_dtype or q.dtype
+    out = torch.empty((n_q, n_rows, dim), dtype=out_dtype, device=q.device)
+    if n_rows == 0:
+        return out
+    k_signs = _as_f32_dev(k_signs, q)
+    v_signs = _as_f32_dev(v_signs, q)
+    lib = _lib.load()
+    need = lib.tq_prefill_workspace_bytes(n_q, n_rows, T, dim)
+    stream = _stream(q)
+    ws = _workspace(q.device, stream.value or 0, max(need, 256))
+    _lib.check(lib.tq_prefill_attn(
+        _ptr(q), _dt(q), _ptr(k_packed), _ptr(k_norms), _ptr(v_packed), _ptr(v_norms),
+        _host_table(k_centroids), _host_table(v_centroids), _ptr(k_signs), _ptr(v_signs),
+        _ptr(out), _dt(out), _ptr(ws), ws.numel(), n_kv, n_rep, n_rows, T, pos0,
+        k_packed.stride(0) // pd, k_norms.stride(0), v_packed.stride(0) // pd, v_norms.stride(0),
+        dim, bits, float(attn_scale), 1 if causal else 0, stream))
+    return out
