@@ -86,10 +86,11 @@ __device__ __forceinline__ uint32_t chunk_field(const uint32_t* row, int w0, int
 // fetched while the current one is computed.
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void prefill_tile_kernel(PrefillArgs a, Codebook kcb, Codebook vcb) {
-  __shared__ __align__(16) _Float16 Ks[kBlkPos * kKStride];
-  __shared__ __align__(16) _Float16 Vt[kD * kVStride];
-  __shared__ uint32_t stK[kStageWords + 4], stV[kStageWords + 4];
-  __shared__ __align__(16) float kn_s[kBlkPos], vn_s[kBlkPos];
+  __shared__ __align__(16) _Float16 Ks2[2][kBlkPos * kKStride];
+  __shared__ __align__(16) _Float16 Vt2[2][kD * kVStride];
+  __shared__ uint32_t stK2[2][kStageWords + 4], stV2[2][kStageWords + 4];
+  __shared__ float stN2[2][2 * kBlkPos];                       // raw key norms, then raw value norms
+  __shared__ __align__(16) float kn_s2[2][kBlkPos], vn_s2[2][kBlkPos];
   __shared__ uint32_t lutk_s[64], lutv_s[64];
   __shared__ __align__(16) float alpha_s[kWaves][kWaveRows];
 
@@ -182,19 +183,24 @@ void prefill_tile_kernel(PrefillArgs a, Codebook kcb, Codebook vcb) {
     else if (tid < 128) pn = (pb + tid - 64 < a.kv_len) ? vnbase[pb + tid - 64] : 0.0f;
   };
 
-  if (p_lo < p_hi) prefetch(p_lo);
-  for (int64_t pb = p_lo; pb < p_hi; pb += kBlkPos) {
-    // ---- stage the fetched words
+  // Pipeline over blocks with ONE barrier per block: block b+1 is decoded into the other LDS
+  // buffer in the same stretch of code that computes block b, so decode arithmetic and LDS
+  // traffic can be scheduled between the matrix instructions.
+  auto stage = [&](int sb) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int id = tid + kThreads * i;
-      if (id < kStageWords) { stK[id] = pk[i]; stV[id] = pv[i]; }
+      if (id < kStageWords) { stK2[sb][id] = pk[i]; stV2[sb][id] = pv[i]; }
     }
-    if (tid < 64) kn_s[tid] = pn * a.score_scale;
-    else if (tid < 128) vn_s[tid - 64] = pn * kVnScale;
-    __syncthreads();                       // staged words visible; everyone has left the previous block's Ks / Vt
-    if (pb + kBlkPos < p_hi) prefetch(pb + kBlkPos);
-
+    if (tid < 128) stN2[sb][tid] = pn;
+  };
+  auto decode = [&](int sb) {
+    const uint32_t* stK = stK2[sb];
+    const uint32_t* stV = stV2[sb];
+    _Float16* Ks = Ks2[sb];
+    _Float16* Vt = Vt2[sb];
+    if (tid < 64) kn_s2[sb][tid] = stN2[sb][tid] * a.score_scale;
+    else if (tid < 128) vn_s2[sb][tid - 64] = stN2[sb][tid] * kVnScale;
     // ---- decode keys: 16 elements of one position
     {
       const uint32_t* row = stK + kpos * kPdim;
@@ -221,110 +227,152 @@ void prefill_tile_kernel(PrefillArgs a, Codebook kcb, Codebook vcb) {
         *reinterpret_cast<uint32_t*>(&Vt[(8 * vc + 2 * i + 1) * kVStride + vslot]) = lutv_s[(Y >> (6 * i)) & 63u];
       }
     }
-    __syncthreads();
-
-    // ---- S^T = K Q^T : accumulator (pt, ct) holds positions 16pt + 4g + j of row 16ct + n16
-    f4 sacc[4][kRowTiles];
+  };
+  auto compute = [&](int sb, int64_t pb) {
+    const _Float16* Ks = Ks2[sb];
+    const _Float16* Vt = Vt2[sb];
+    const float* kn_s = kn_s2[sb];
+    const float* vn_s = vn_s2[sb];
+    // Two sub-blocks of 32 positions, each with its own online-softmax step, so that only 32
+    // positions of scores are live at a time; the registers this frees hold operands that are
+    // read from LDS two (keys) or three (values) matrix instructions ahead of their use.
+    const int64_t first_lim = a.causal ? min(a.kv_len, a.q_pos0 + wrow0 + 1) : a.kv_len;
+    const _Float16* kop = Ks + n16 * kKStride + 8 * g;               // + (16 pt) * kKStride + 32 kb
+    const _Float16* vop = Vt + n16 * kVStride + 8 * g;               // + (16 et) * kVStride + 32 kb2
+#pragma nounroll
+    for (int h = 0; h < 2; ++h) {
+      // ---- S^T = K Q^T : accumulator (t, ct) holds positions 32h + 16t + 4g + j of row 16ct + n16
+      f4 sacc[2][kRowTiles];
 #pragma unroll
-    for (int pt = 0; pt < 4; ++pt) {
+      for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int ct = 0; ct < kRowTiles; ++ct) sacc[pt][ct] = f4{0.f, 0.f, 0.f, 0.f};
+        for (int ct = 0; ct < kRowTiles; ++ct) sacc[t][ct] = f4{0.f, 0.f, 0.f, 0.f};
+      u4 kreg[3];
+      kreg[0] = *reinterpret_cast<const u4*>(kop + (32 * h) * kKStride);
+      kreg[1] = *reinterpret_cast<const u4*>(kop + (32 * h) * kKStride + 32);
 #pragma unroll
-      for (int kb = 0; kb < 4; ++kb) {
-        const u4 A = *reinterpret_cast<const u4*>(&Ks[(16 * pt + n16) * kKStride + 32 * kb + 8 * g]);
+      for (int i = 0; i < 8; ++i) {                                   // i = 4t + kb
+        if (i + 2 < 8)
+          kreg[(i + 2) % 3] = *reinterpret_cast<const u4*>(kop + (32 * h + 16 * ((i + 2) >> 2)) * kKStride +
+                                                           32 * ((i + 2) & 3));
+        const u4 A = kreg[i % 3];
 #pragma unroll
         for (int ct = 0; ct < kRowTiles; ++ct) {
-          sacc[pt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, A),
-                                                                __builtin_bit_cast(h8, qlo[ct][kb]),
-                                                                sacc[pt][ct], 0, 0, 0);
-          sacc[pt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, A),
-                                                                __builtin_bit_cast(h8, qhi[ct][kb]),
-                                                                sacc[pt][ct], 0, 0, 0);
+          sacc[i >> 2][ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, A),
+                                                                    __builtin_bit_cast(h8, qlo[ct][i & 3]),
+                                                                    sacc[i >> 2][ct], 0, 0, 0);
+          sacc[i >> 2][ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, A),
+                                                                    __builtin_bit_cast(h8, qhi[ct][i & 3]),
+                                                                    sacc[i >> 2][ct], 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      // first value operands: in flight during the softmax arithmetic
+      u4 vreg[4];
+#pragma unroll
+      for (int i = 0; i < 3; ++i) vreg[i] = *reinterpret_cast<const u4*>(vop + (16 * i) * kVStride + 32 * h);
+      __builtin_amdgcn_sched_barrier(0);
+
+      // ---- scale by key norm (log2 units), mask
+      const bool need_mask = pb + 32 * (h + 1) > first_lim;              // uniform over the wavefront
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const float4 kn4 = *reinterpret_cast<const float4*>(&kn_s[32 * h + 16 * t + 4 * g]);
+        const float knv[4] = {kn4.x, kn4.y, kn4.z, kn4.w};
+#pragma unroll
+        for (int ct = 0; ct < kRowTiles; ++ct)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) sacc[t][ct][j] *= knv[j];
+      }
+      if (need_mask) {
+#pragma unroll
+        for (int ct = 0; ct < kRowTiles; ++ct) {
+          const int64_t r = wrow0 + 16 * ct + n16;
+          const int64_t lim = a.causal ? min(a.kv_len, a.q_pos0 + r + 1) : a.kv_len;
+          // own positions 32h + 16t + 4g + j are visible while 16t + j < rel
+          const int rel = (int)min((int64_t)kBlkPos, max((int64_t)0, lim - pb)) - 4 * g - 32 * h;
+#pragma unroll
+          for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) sacc[t][ct][j] = (16 * t + j >= rel) ? -INFINITY : sacc[t][ct][j];
         }
       }
-    }
-    // ---- scale by key norm (log2 units), mask
-    const int64_t first_lim = a.causal ? min(a.kv_len, a.q_pos0 + wrow0 + 1) : a.kv_len;
-    const bool need_mask = pb + kBlkPos > first_lim;                     // uniform over the wavefront
-#pragma unroll
-    for (int pt = 0; pt < 4; ++pt) {
-      const float4 kn4 = *reinterpret_cast<const float4*>(&kn_s[16 * pt + 4 * g]);
-      const float knv[4] = {kn4.x, kn4.y, kn4.z, kn4.w};
-#pragma unroll
-      for (int ct = 0; ct < kRowTiles; ++ct)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) sacc[pt][ct][j] *= knv[j];
-    }
-    if (need_mask) {
+      // ---- online softmax per row (a row lives in the four lanes n16 + 16g)
+      uint32_t pa[kRowTiles][4];
+      bool rescale = false;
 #pragma unroll
       for (int ct = 0; ct < kRowTiles; ++ct) {
-        const int64_t r = wrow0 + 16 * ct + n16;
-        const int64_t lim = a.causal ? min(a.kv_len, a.q_pos0 + r + 1) : a.kv_len;
-        const int rel = (int)min((int64_t)kBlkPos, max((int64_t)0, lim - pb)) - 4 * g;   // own positions < rel are visible
+        float mx = -INFINITY;
 #pragma unroll
-        for (int pt = 0; pt < 4; ++pt)
+        for (int t = 0; t < 2; ++t)
 #pragma unroll
-          for (int j = 0; j < 4; ++j) sacc[pt][ct][j] = (16 * pt + j >= rel) ? -INFINITY : sacc[pt][ct][j];
-      }
-    }
-    // ---- online softmax per row (a row lives in the four lanes n16 + 16g)
-    uint32_t pa[kRowTiles][2][4];
-    bool rescale = false;
+          for (int j = 0; j < 4; ++j) mx = fmaxf(mx, sacc[t][ct][j]);
+        mx = fmaxf(mx, shfl_xor_f(mx, 16));
+        mx = fmaxf(mx, shfl_xor_f(mx, 32));
+        const float m_new = fmaxf(m_run[ct], mx);
+        const float msafe = (m_new == -INFINITY) ? 0.0f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f(m_run[ct] - msafe);   // v_exp_f32: 2^-inf = 0, tiny results flush to 0
+        rescale = rescale || (alpha != 1.0f);
+        m_run[ct] = m_new;
+        float lsum = 0.0f;
 #pragma unroll
-    for (int ct = 0; ct < kRowTiles; ++ct) {
-      float mx = -INFINITY;
+        for (int t = 0; t < 2; ++t) {
+          const float4 vn4 = *reinterpret_cast<const float4*>(&vn_s[32 * h + 16 * t + 4 * g]);
+          float p[4];
 #pragma unroll
-      for (int pt = 0; pt < 4; ++pt)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) mx = fmaxf(mx, sacc[pt][ct][j]);
-      mx = fmaxf(mx, shfl_xor_f(mx, 16));
-      mx = fmaxf(mx, shfl_xor_f(mx, 32));
-      const float m_new = fmaxf(m_run[ct], mx);
-      const float msafe = (m_new == -INFINITY) ? 0.0f : m_new;
-      const float alpha = __builtin_amdgcn_exp2f(m_run[ct] - msafe);   // v_exp_f32: 2^-inf = 0, tiny results flush to 0
-      rescale = rescale || (alpha != 1.0f);
-      m_run[ct] = m_new;
-      float lsum = 0.0f;
-#pragma unroll
-      for (int pt = 0; pt < 4; ++pt) {
-        const float4 vn4 = *reinterpret_cast<const float4*>(&vn_s[16 * pt + 4 * g]);
-        float p[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          p[j] = __builtin_amdgcn_exp2f(sacc[pt][ct][j] - msafe);
-          lsum += p[j];
+          for (int j = 0; j < 4; ++j) {
+            p[j] = __builtin_amdgcn_exp2f(sacc[t][ct][j] - msafe);
+            lsum += p[j];
+          }
+          pa[ct][2 * t] = pack_h2(p[0] * vn4.x, p[1] * vn4.y);
+          pa[ct][2 * t + 1] = pack_h2(p[2] * vn4.z, p[3] * vn4.w);
         }
-        pa[ct][pt >> 1][2 * (pt & 1)] = pack_h2(p[0] * vn4.x, p[1] * vn4.y);
-        pa[ct][pt >> 1][2 * (pt & 1) + 1] = pack_h2(p[2] * vn4.z, p[3] * vn4.w);
+        l_run[ct] = l_run[ct] * alpha + lsum;
+        if (g == 0) alpha_s[wave][16 * ct + n16] = alpha;
       }
-      l_run[ct] = l_run[ct] * alpha + lsum;
-      if (g == 0) alpha_s[wave][16 * ct + n16] = alpha;
-    }
-    // ---- rescale the output accumulators (rows 16ct + 4g + j) when some running maximum moved
-    if (__any(rescale)) {
+      // ---- rescale the output accumulators (rows 16ct + 4g + j) when some running maximum moved
+      if (__any(rescale)) {
 #pragma unroll
-      for (int ct = 0; ct < kRowTiles; ++ct) {
-        const float4 a4 = *reinterpret_cast<const float4*>(&alpha_s[wave][16 * ct + 4 * g]);
-        const float av[4] = {a4.x, a4.y, a4.z, a4.w};
+        for (int ct = 0; ct < kRowTiles; ++ct) {
+          const float4 a4 = *reinterpret_cast<const float4*>(&alpha_s[wave][16 * ct + 4 * g]);
+          const float av[4] = {a4.x, a4.y, a4.z, a4.w};
 #pragma unroll
-        for (int et = 0; et < 8; ++et)
+          for (int et = 0; et < 8; ++et)
 #pragma unroll
-          for (int j = 0; j < 4; ++j) oacc[ct][et][j] *= av[j];
+            for (int j = 0; j < 4; ++j) oacc[ct][et][j] *= av[j];
+        }
       }
-    }
-    // ---- O += P V
-#pragma unroll
-    for (int kb2 = 0; kb2 < 2; ++kb2)
+      // ---- O += P V over the 32 positions of this sub-block
 #pragma unroll
       for (int et = 0; et < 8; ++et) {
-        const u4 B = *reinterpret_cast<const u4*>(&Vt[(16 * et + n16) * kVStride + 32 * kb2 + 8 * g]);
+        if (et + 3 < 8) vreg[(et + 3) & 3] = *reinterpret_cast<const u4*>(vop + (16 * (et + 3)) * kVStride + 32 * h);
+        const u4 B = vreg[et & 3];
 #pragma unroll
         for (int ct = 0; ct < kRowTiles; ++ct) {
-          const u4 A = {pa[ct][kb2][0], pa[ct][kb2][1], pa[ct][kb2][2], pa[ct][kb2][3]};
+          const u4 A = {pa[ct][0], pa[ct][1], pa[ct][2], pa[ct][3]};
           oacc[ct][et] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, A), __builtin_bit_cast(h8, B),
                                                                 oacc[ct][et], 0, 0, 0);
         }
+        __builtin_amdgcn_sched_barrier(0);
       }
+    }
+  };
+
+  if (p_lo < p_hi) {
+    prefetch(p_lo);
+    stage(0);
+    __syncthreads();
+    if (p_lo + kBlkPos < p_hi) prefetch(p_lo + kBlkPos);
+    decode(0);
+  }
+  int sb = 0;
+  for (int64_t pb = p_lo; pb < p_hi; pb += kBlkPos, sb ^= 1) {
+    const bool more = pb + kBlkPos < p_hi;
+    if (more) stage(sb ^ 1);               // words of block b+1 (fetched during block b-1)
+    __syncthreads();                       // block b decoded by all; block b-1 computed by all; stage of b+1 visible
+    if (pb + 2 * kBlkPos < p_hi) prefetch(pb + 2 * kBlkPos);
+    if (more) decode(sb ^ 1);
+    compute(sb, pb);
   }
 
   // ---- partial results of this split
