@@ -314,3 +314,84 @@ def test_vonly_decode_attention_on_cache(tq, thr):
     ko, vo = cache._k_cache.keys[..., :S, :], cache._v_tq._v_deq_buf[..., :S, :]
     ref = o.dense_attention(host(q)[0], host(ko)[0], host(vo)[0], sc)
     assert cos(host(out)[0], ref) > 0.999
+
+
+# ------------------------------------------------------------------ prefill off the packed cache, dispatcher
+
+def test_prefill_attention_on_cache_two_chunks(tq):
+    """A prompt fed in two chunks through a fused cache: each chunk's attention comes from the packed
+    storage and must equal the oracle's dense attention over the dequantised cache with the offset
+    causal mask (what the reference's non-fused prefill computes, cache.py:209-218 + SDPA)."""
+    B, n_q, n_kv, D = 2, 8, 4, 128
+    sc = 1 / math.sqrt(D)
+    chunks = (320, 200)
+    cache = tq.TurboQuantKVCache(bits=3, fused=True)
+    c = o.gaussian_codebook(3)
+    ks, vs = o.random_diagonal_sign(D, 42), o.random_diagonal_sign(D, 43)
+    seed = 60
+    for S in chunks:
+        k, v, q = rand((B, n_kv, S, D), seed), rand((B, n_kv, S, D), seed + 1), rand((B, n_q, S, D), seed + 2)
+        seed += 3
+        cache.update_and_fetch(k, v)
+        out = tq.turboquant_prefill_attention(q, cache, sc)
+        assert out.shape == (B, n_q, S, D) and out.dtype == q.dtype
+        kp, kn, vp, vn = [t.cpu().numpy() for t in cache.state]
+        for b in range(B):
+            want = o.prefill_attention(host(q)[b], kp[b], kn[b], vp[b], vn[b], c, c, ks, vs, D, 3, sc,
+                                       cache.offset - S, n_q // n_kv)
+            err = np.abs(host(out)[b] - want)
+            scale = np.abs(want).max(axis=-1, keepdims=True)
+            assert (err <= 1e-3 + 3e-3 * scale).all(), (err / scale).max()      # fp16 output rounding included
+
+
+def test_sdpa_dispatcher_routes_by_cache(tq):
+    """patch.py:14-41: the dispatcher sends a fused cache's decode step to turboquant_attention, its
+    multi-token step to the packed prefill, a V-only cache's decode step to the fused V-only kernel,
+    and everything else to stock SDPA; apply_patch / remove_patch install and restore it."""
+    import types
+    from tqhip import patch
+    B, n_q, n_kv, S, D = 1, 8, 4, 256, 128
+    sc = 1 / math.sqrt(D)
+    k, v = rand((B, n_kv, S, D), 70), rand((B, n_kv, S, D), 71)
+    qs, q1 = rand((B, n_q, S, D), 72), rand((B, n_q, 1, D), 73)
+    k1, v1 = rand((B, n_kv, 1, D), 74), rand((B, n_kv, 1, D), 75)
+
+    fused = tq.TurboQuantKVCache(bits=3, fused=True)
+    kk, vv = fused.update_and_fetch(k, v)
+    out = patch.scaled_dot_product_attention(qs, kk, vv, fused, sc, fused.make_mask(S))
+    assert torch.equal(out, tq.turboquant_prefill_attention(qs, fused, sc))
+    kk, vv = fused.update_and_fetch(k1, v1)
+    out = patch.scaled_dot_product_attention(q1, kk, vv, fused, sc, fused.make_mask(1))
+    assert torch.equal(out, tq.turboquant_attention(q1, fused, sc, fused=True))
+    with pytest.raises(ValueError):
+        patch.scaled_dot_product_attention(qs, kk, vv, fused, sc, torch.ones((S, S + 1), dtype=torch.bool, device="cuda"))
+
+    plain = tq.TurboQuantKVCache(bits=3)
+    kd, vd = plain.update_and_fetch(k, v)
+    out = patch.scaled_dot_product_attention(qs, kd, vd, plain, sc, plain.make_mask(S))
+    ref = o.dense_attention(host(qs)[0], host(kd)[0], host(vd)[0], sc,
+                            np.where(np.tril(np.ones((S, S))) > 0, 0.0, -np.inf))
+    assert np.abs(host(out)[0] - ref).max() < 5e-3
+    # the packed prefill and stock SDPA over the dequantised cache agree (same quantised K/V)
+    assert cos(host(tq.turboquant_prefill_attention(qs, fused_like(tq, k, v), sc))[0], ref) > 0.9995
+
+    vo = tq.VOnlyTurboQuantCache(bits=3)
+    vo.update_and_fetch(k, v)
+    kk, vv = vo.update_and_fetch(k1, v1)
+    out = patch.scaled_dot_product_attention(q1, kk, vv, vo, sc, None)
+    assert torch.equal(out, tq.vonly_decode_attention(q1, vo, sc))
+
+    mod = types.SimpleNamespace(scaled_dot_product_attention="original")
+    bare = types.SimpleNamespace()
+    tq.apply_patch(mod, bare)
+    tq.apply_patch(mod)                                    # idempotent
+    assert mod.scaled_dot_product_attention is patch.scaled_dot_product_attention
+    assert bare.scaled_dot_product_attention is patch.scaled_dot_product_attention
+    tq.remove_patch()
+    assert mod.scaled_dot_product_attention == "original" and not hasattr(bare, "scaled_dot_product_attention")
+
+
+def fused_like(tq, k, v):
+    cache = tq.TurboQuantKVCache(bits=3, fused=True)
+    cache.update_and_fetch(k, v)
+    return cache

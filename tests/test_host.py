@@ -120,3 +120,20 @@ def test_cache_meta_state_and_masks_on_host():
     assert kv.make_mask(1) is None and kv.make_mask(2) == "causal"
     r = tqhip.KVCache.from_state(kv.state)
     assert r.offset == 295 and torch.equal(r.keys, k[..., :295, :])
+
+
+def test_patch_install_and_restore_on_host():
+    """patch.py:44-90: apply_patch replaces the attribute on every module given, once; remove_patch
+    puts back what was there (or removes the attribute when there was none)."""
+    import types
+    import tqhip
+    from tqhip import patch
+    a = types.SimpleNamespace(scaled_dot_product_attention=len)
+    b = types.SimpleNamespace()
+    tqhip.apply_patch(a, b)
+    tqhip.apply_patch(a)
+    assert a.scaled_dot_product_attention is patch.scaled_dot_product_attention
+    assert b.scaled_dot_product_attention is patch.scaled_dot_product_attention
+    tqhip.remove_patch()
+    assert a.scaled_dot_product_attention is len and not hasattr(b, "scaled_dot_product_attention")
+    tqhip.remove_patch()                                   # nothing left to undo

@@ -30,7 +30,8 @@ from .ops import (
     unpack_indices,
     packed_dim,
 )
-from .attention import turboquant_attention, vonly_decode_attention
+from .attention import turboquant_attention, turboquant_prefill_attention, vonly_decode_attention
+from .patch import apply_patch, remove_patch, scaled_dot_product_attention
 from .rotation import (
     walsh_hadamard_transform,
     randomized_hadamard_transform,

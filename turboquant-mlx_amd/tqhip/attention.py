@@ -117,3 +117,27 @@ def vonly_decode_attention(queries: torch.Tensor, cache, attn_scale: float, mask
                                  vq.centroids, vq.signs, tq._v_dim, bits, threshold=thr, n_rep=n_rep)
         outputs.append(mv[:, None, :].to(queries.dtype))
     return torch.stack(outputs, dim=0)
+
+
+def turboquant_prefill_attention(queries: torch.Tensor, cache, attn_scale: float, causal: bool = True) -> torch.Tensor:
+    """Multi-token forward (prompt chunk) straight off the packed K and V of a TurboQuantKVCache,
+    after `cache.update_and_fetch` has encoded the chunk: the last S of the cache's `offset`
+    positions are the chunk's own, and query row i attends positions <= offset - S + i.
+
+    The reference has no such path: its prefill dequantises the whole cache (cache.py:209-218) and
+    hands fp16 K/V to stock SDPA, and with fused=True it returns zero placeholders (cache.py:162-165)
+    that only a decode step knows how to bypass.  queries (B, n_heads, S, dim) -> same shape and dtype.
+    """
+    B, n_q, S, dim = queries.shape
+    total = cache.offset
+    if S > total:
+        raise ValueError(f"the cache holds {total} positions, fewer than the {S} query rows")
+    n_kv = cache.k_packed.shape[1]
+    n_rep = n_q // n_kv
+    kq, vq = cache._k_q, cache._v_q
+    outs = [ops.prefill_attention(queries[b], cache.k_packed[b], cache.k_norms[b], cache.v_packed[b],
+                                  cache.v_norms[b], kq.centroids, vq.centroids, kq.signs, vq.signs, dim,
+                                  cache.quant_bits, attn_scale, n_rep=n_rep, kv_len=total, q_pos0=total - S,
+                                  causal=causal)
+            for b in range(B)]
+    return torch.stack(outs, dim=0)
