@@ -78,8 +78,10 @@ def bench_scores(iters, dev):
         nbytes = 224 * T + 112 * T + 14336
         sets = packed_sets(4, T, dev, n_sets_for(nbytes), 3)
         q_rot = torch.randn((28, 128), device=dev)
-        fns = [(lambda p=p, n=n: tqhip.prerot_fused_qk_scores(q_rot, p, n, cb, 128, 3, n_rep=7)) for p, n in sets]
-        report(f"config 3: prerot scores 28/4 heads, T={T}", timeit(fns, iters), nbytes)
+        for prec in ("fp32", "fp16"):
+            fns = [(lambda p=p, n=n: tqhip.prerot_fused_qk_scores(q_rot, p, n, cb, 128, 3, n_rep=7, precision=prec))
+                   for p, n in sets]
+            report(f"config 3: prerot scores 28/4 heads, T={T}, {prec} operands", timeit(fns, iters), nbytes)
 
 
 def bench_sparse_v(iters, dev):
@@ -89,10 +91,10 @@ def bench_sparse_v(iters, dev):
         nbytes = 28 * T * 4 + 4 * T * 56 + 28 * 128 * 4
         sets = packed_sets(4, T, dev, n_sets_for(nbytes), 4)
         w = torch.softmax(torch.randn((28, T), device=dev) * 5, dim=-1)
-        for thr in (0.0, 1e-5):
-            fns = [(lambda p=p, n=n: tqhip.sparse_v_matvec(w, p, n, cb, signs, 128, 3, threshold=thr, n_rep=7))
-                   for p, n in sets]
-            report(f"sparse_v_matvec 28/4 heads, T={T}, thr={thr:g}", timeit(fns, iters), nbytes)
+        for thr, prec in ((0.0, "fp32"), (1e-5, "fp32"), (1e-5, "fp16")):
+            fns = [(lambda p=p, n=n: tqhip.sparse_v_matvec(w, p, n, cb, signs, 128, 3, threshold=thr, n_rep=7,
+                                                           precision=prec)) for p, n in sets]
+            report(f"sparse_v_matvec 28/4 heads, T={T}, thr={thr:g}, {prec} operands", timeit(fns, iters), nbytes)
 
 
 def bench_flash(iters, dev):
