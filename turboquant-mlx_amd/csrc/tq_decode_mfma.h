@@ -83,8 +83,19 @@ struct MfmaArgs {
       a.trace[((blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 16 + (slot)] =     \
           __builtin_amdgcn_s_memrealtime();                                                         \
   } while (0)
+// per-wave variant: lane 0 of wave w > 0 writes slot `base_slot_of[w]` (spare slots of the record)
+#define TQ_STAMP_WAVE()                                                                             \
+  do {                                                                                              \
+    const int w_ = threadIdx.x >> 6;                                                                \
+    if (a.trace && (threadIdx.x & 63) == 0 && w_ > 0) {                                             \
+      const int slot_ = (w_ <= 3) ? 3 + w_ : 7 + w_;          /* waves 1..3 -> 4..6, 4..7 -> 11..14 */ \
+      a.trace[((blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 16 + slot_] =      \
+          __builtin_amdgcn_s_memrealtime();                                                         \
+    }                                                                                               \
+  } while (0)
 #else
 #define TQ_STAMP(slot) do {} while (0)
+#define TQ_STAMP_WAVE() do {} while (0)
 #endif
 
 __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
@@ -101,7 +112,8 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
   __shared__ uint32_t lut_s[64];                       // half2(c[i & 7], c[i >> 3])
   __shared__ __align__(16) uint32_t q_s[kHeadsMax][kD / 2];   // fp16 pairs, rows >= n_rep are zero
   __shared__ __align__(16) float nrm_s[kWaves][kWavePos];
-  __shared__ float m_s[kWaves][kHeadsMax], l_s[kWaves][kHeadsMax], t_s[kWaves];
+  __shared__ float m_s[kWaves][kHeadsMax], l_s[kWaves][kHeadsMax], M_s[kHeadsMax];
+  __shared__ __align__(16) float f_s[kWaves][kHeadsMax];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -166,6 +178,13 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
   // ALU / LDS work) placed between them; scheduling barriers keep the compiler from regrouping.
   const u4* kbase = reinterpret_cast<const u4*>(
       a.k + ((int64_t)seq * a.k_seq_stride + (int64_t)kvh * a.k_head_stride + first + tile_p0) * kD);
+  // Every wave issues its V block (needed first) before any wave issues K: the CU's memory
+  // pipeline takes requests in issue order, and without this the last wave's V block queues
+  // behind the first waves' K loads and that wave reaches the merge a microsecond late.
+  // A bare barrier: it orders the issue, it does not wait for any data.
+  __builtin_amdgcn_sched_barrier(0);
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_sched_barrier(0);
   u4 kreg[16];
   auto issue_k = [&](int i) {
     const int r = 4 * i + (lane >> 4);
@@ -341,10 +360,13 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
                                                         accS[et], 0, 0, 0);
   }
   TQ_STAMP(3);
+  TQ_STAMP_WAVE();
 
-  // ---- merge the eight waves: one barrier ------------------------------------------------------------
-  // Every wave deposits its unscaled accumulator rows together with (m, l, 2^k scale); the
-  // cooperative sum below rescales while it adds.  Eight query heads fit the 32 KB buffer per round.
+  // ---- merge the eight waves ----------------------------------------------------------------------------
+  // (1) every wave publishes (m, l) per head; (2) 128 threads turn them into one factor
+  // e^(m_w - M_h) per (wave, head); (3) every wave scales its own accumulator rows by its factors
+  // and deposits them; (4) a float4 sum over the eight deposits goes to the workspace.  The
+  // exponentials are evaluated once per (wave, head), not once per element.
   float (*S_all)[8][kD] = reinterpret_cast<float (*)[8][kD]>(big_s);    // [wave][head in round][128]
   const int64_t grp = (int64_t)seq * a.n_kv + kvh;
   float* pS = a.ws_S + (grp * a.n_tiles_max + tile) * (int64_t)(n_rep * kD);
@@ -353,45 +375,52 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
     m_s[wave][n16] = m;
     l_s[wave][n16] = l;
   }
-  if (lane == 0) t_s[wave] = inv_tscale * a.v_unscale;
+  __syncthreads();                                       // (m, l) visible; the staging area is free
+  if (tid < kWaves * kHeadsMax) {
+    const int w = tid >> 4, h = tid & 15;
+    float M = m_s[0][h];
+#pragma unroll
+    for (int ww = 1; ww < kWaves; ++ww) M = fmaxf(M, m_s[ww][h]);
+    const float mw = m_s[w][h];
+    f_s[w][h] = (mw == -INFINITY) ? 0.0f : __expf(mw - M);
+    if (w == 0) M_s[h] = M;
+  }
+  __syncthreads();
+  TQ_STAMP(8);
+  const float4 f4own = *reinterpret_cast<const float4*>(&f_s[wave][4 * g]);   // heads 4g .. 4g+3 of this lane's rows
+  const float wscale = inv_tscale * a.v_unscale;
+  const float fown[4] = {f4own.x * wscale, f4own.y * wscale, f4own.z * wscale, f4own.w * wscale};
   for (int h0 = 0; h0 < n_rep; h0 += 8) {
-    __syncthreads();                                     // staging area (or the previous round) is free
+    if (h0) __syncthreads();                             // the previous round has been summed
     if ((g >> 1) == (h0 >> 3)) {                         // lanes whose rows 4g+j fall in this round
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         float4* dst = reinterpret_cast<float4*>(&S_all[wave][(4 * g + j) & 7][8 * n16]);
-        dst[0] = make_float4(accS[0][j], accS[1][j], accS[2][j], accS[3][j]);
-        dst[1] = make_float4(accS[4][j], accS[5][j], accS[6][j], accS[7][j]);
+        const float f = fown[j];
+        dst[0] = make_float4(accS[0][j] * f, accS[1][j] * f, accS[2][j] * f, accS[3][j] * f);
+        dst[1] = make_float4(accS[4][j] * f, accS[5][j] * f, accS[6][j] * f, accS[7][j] * f);
       }
     }
     __syncthreads();
-    TQ_STAMP(8);
     const int rows = min(8, n_rep - h0);
-    for (int i = tid; i < rows * kD; i += kMfmaThreads) {
-      const int hl = i >> 7, e = i & 127, h = h0 + hl;
-      float M = m_s[0][h];
+    if (tid < rows * (kD / 4)) {                         // one float4 of one head per thread
+      const int hl = tid >> 5, e4 = tid & 31;
+      float4 sum = *reinterpret_cast<const float4*>(&S_all[0][hl][4 * e4]);
 #pragma unroll
-      for (int w = 1; w < kWaves; ++w) M = fmaxf(M, m_s[w][h]);
-      float sum = 0.0f;
-#pragma unroll
-      for (int w = 0; w < kWaves; ++w) {
-        const float mw = m_s[w][h];
-        const float f = (mw == -INFINITY) ? 0.0f : __expf(mw - M) * t_s[w];
-        sum += f * S_all[w][hl][e];
+      for (int w = 1; w < kWaves; ++w) {
+        const float4 x = *reinterpret_cast<const float4*>(&S_all[w][hl][4 * e4]);
+        sum.x += x.x; sum.y += x.y; sum.z += x.z; sum.w += x.w;
       }
-      pS[h * kD + e] = sum;
+      *reinterpret_cast<float4*>(pS + (h0 + hl) * kD + 4 * e4) = sum;
     }
   }
   TQ_STAMP(9);
   if (tid < n_rep) {
     const int h = tid;
-    float M = m_s[0][h];
-#pragma unroll
-    for (int w = 1; w < kWaves; ++w) M = fmaxf(M, m_s[w][h]);
     float L = 0.0f;
 #pragma unroll
-    for (int w = 0; w < kWaves; ++w) L += (m_s[w][h] == -INFINITY) ? 0.0f : __expf(m_s[w][h] - M) * l_s[w][h];
-    pml[2 * h] = M;
+    for (int w = 0; w < kWaves; ++w) L += f_s[w][h] * l_s[w][h];
+    pml[2 * h] = M_s[h];
     pml[2 * h + 1] = L;
   }
   TQ_STAMP(10);

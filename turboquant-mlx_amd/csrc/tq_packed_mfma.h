@@ -113,7 +113,8 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
   __shared__ __align__(16) uint32_t q_s[kHeadsMax][kD / 2];      // rotated queries as half2: rounded value ...
   __shared__ __align__(16) uint32_t ql_s[kHeadsMax][kD / 2];     // ... and what the rounding lost
   __shared__ __align__(16) float kn_s[kWaves][kWavePos], vn_s[kWaves][kWavePos];
-  __shared__ float m_s[kWaves][kHeadsMax], l_s[kWaves][kHeadsMax], t_s[kWaves];
+  __shared__ float m_s[kWaves][kHeadsMax], l_s[kWaves][kHeadsMax], M_s[kHeadsMax];
+  __shared__ __align__(16) float f_s[kWaves][kHeadsMax];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -331,7 +332,8 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
     }
   }
 
-  // ---- merge the eight waves (one barrier per round of 8 heads), as in the dense-key kernel ------------
+  // ---- merge the eight waves, as in the dense-key kernel: one factor per (wave, head), scaled deposits,
+  // float4 sum -------------------------------------------------------------------------------------------
   float (*S_all)[8][kD] = reinterpret_cast<float (*)[8][kD]>(big_s);
   const int64_t grp = (int64_t)seq * a.n_kv + kvh;
   float* pS = a.ws_S + (grp * a.n_tiles_max + tile) * (int64_t)(n_rep * kD);
@@ -340,43 +342,50 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
     m_s[wave][n16] = m;
     l_s[wave][n16] = l;
   }
-  if (lane == 0) t_s[wave] = inv_tscale * a.v_unscale;
+  __syncthreads();
+  if (tid < kWaves * kHeadsMax) {
+    const int w = tid >> 4, h = tid & 15;
+    float M = m_s[0][h];
+#pragma unroll
+    for (int ww = 1; ww < kWaves; ++ww) M = fmaxf(M, m_s[ww][h]);
+    const float mw = m_s[w][h];
+    f_s[w][h] = (mw == -INFINITY) ? 0.0f : __expf(mw - M);
+    if (w == 0) M_s[h] = M;
+  }
+  __syncthreads();
+  const float4 f4own = *reinterpret_cast<const float4*>(&f_s[wave][4 * g]);
+  const float wscale = inv_tscale * a.v_unscale;
+  const float fown[4] = {f4own.x * wscale, f4own.y * wscale, f4own.z * wscale, f4own.w * wscale};
   for (int h0 = 0; h0 < n_rep; h0 += 8) {
-    __syncthreads();
+    if (h0) __syncthreads();
     if ((g >> 1) == (h0 >> 3)) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         float4* dst = reinterpret_cast<float4*>(&S_all[wave][(4 * g + j) & 7][8 * n16]);
-        dst[0] = make_float4(accS[0][j], accS[1][j], accS[2][j], accS[3][j]);
-        dst[1] = make_float4(accS[4][j], accS[5][j], accS[6][j], accS[7][j]);
+        const float f = fown[j];
+        dst[0] = make_float4(accS[0][j] * f, accS[1][j] * f, accS[2][j] * f, accS[3][j] * f);
+        dst[1] = make_float4(accS[4][j] * f, accS[5][j] * f, accS[6][j] * f, accS[7][j] * f);
       }
     }
     __syncthreads();
     const int rows = min(8, n_rep - h0);
-    for (int i = tid; i < rows * kD; i += kMfmaThreads) {
-      const int hl = i >> 7, e = i & 127, h = h0 + hl;
-      float M = m_s[0][h];
+    if (tid < rows * (kD / 4)) {
+      const int hl = tid >> 5, e4 = tid & 31;
+      float4 sum = *reinterpret_cast<const float4*>(&S_all[0][hl][4 * e4]);
 #pragma unroll
-      for (int w = 1; w < kWaves; ++w) M = fmaxf(M, m_s[w][h]);
-      float sum = 0.0f;
-#pragma unroll
-      for (int w = 0; w < kWaves; ++w) {
-        const float mw = m_s[w][h];
-        const float f = (mw == -INFINITY) ? 0.0f : __expf(mw - M) * t_s[w];
-        sum += f * S_all[w][hl][e];
+      for (int w = 1; w < kWaves; ++w) {
+        const float4 x = *reinterpret_cast<const float4*>(&S_all[w][hl][4 * e4]);
+        sum.x += x.x; sum.y += x.y; sum.z += x.z; sum.w += x.w;
       }
-      pS[h * kD + e] = sum;
+      *reinterpret_cast<float4*>(pS + (h0 + hl) * kD + 4 * e4) = sum;
     }
   }
   if (tid < n_rep) {
     const int h = tid;
-    float M = m_s[0][h];
-#pragma unroll
-    for (int w = 1; w < kWaves; ++w) M = fmaxf(M, m_s[w][h]);
     float L = 0.0f;
 #pragma unroll
-    for (int w = 0; w < kWaves; ++w) L += (m_s[w][h] == -INFINITY) ? 0.0f : __expf(m_s[w][h] - M) * l_s[w][h];
-    pml[2 * h] = M;
+    for (int w = 0; w < kWaves; ++w) L += f_s[w][h] * l_s[w][h];
+    pml[2 * h] = M_s[h];
     pml[2 * h + 1] = L;
   }
 }
