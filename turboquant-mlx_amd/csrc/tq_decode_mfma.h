@@ -104,6 +104,10 @@ __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
 }
 
 // grid = (n_tiles_max, n_kv, n_seq), 512 threads.
+// PLAIN = no mask, no ragged offsets, seq_len a multiple of the tile, 16-byte aligned V rows (checked
+// by the host): every tile is full, so the row clamps, the validity selects, the mask reads and the
+// narrow V path drop out, and K / V addresses are a uniform base plus a lane-constant offset.
+template <bool PLAIN>
 __global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
   // 32 KB used three ways: per-wave staging (8 x 4 KB) first for the packed V block, then for K
@@ -124,14 +128,14 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
   const int64_t q_row0 = (int64_t)seq * n_q + (int64_t)kvh * n_rep;
 
   int64_t first = 0, len = a.seq_len;
-  if (a.seq_offsets) {
+  if (!PLAIN && a.seq_offsets) {
     first = a.seq_offsets[seq];
     len = (int64_t)a.seq_offsets[seq + 1] - first;
   }
   const int64_t tile_p0 = (int64_t)tile * kTilePos;
   TQ_STAMP(0);
   if (tile_p0 >= len) return;                          // the merge pass never reads this tile
-  const int rows_here = (int)min((int64_t)kTilePos, len - tile_p0);   // valid rows of this tile
+  const int rows_here = PLAIN ? kTilePos : (int)min((int64_t)kTilePos, len - tile_p0);   // valid rows of this tile
   const int last_row = rows_here - 1;
   const int wrow0 = wave * kWavePos;                                  // wave's first row inside the tile
 
@@ -146,7 +150,7 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
   {
     const float* nb = a.v_norms + (int64_t)seq * a.vn_seq_stride + (int64_t)kvh * a.vn_head_stride + first + tile_p0;
     int row = wrow0 + lane;
-    row = row < last_row ? row : last_row;
+    if (!PLAIN) row = row < last_row ? row : last_row;
     my_norm = nb[(unsigned)row];
   }
   // packed V of the wave: 64 rows x 52 bytes, contiguous.  Full, 16-byte aligned blocks take four
@@ -154,14 +158,14 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
   // clamped to the last valid word.  Either way the LDS image is the plain copy of the block.
   const uint32_t* vblock = a.v_packed +
       ((int64_t)seq * a.v_seq_stride + (int64_t)kvh * a.v_head_stride + first + tile_p0 + wrow0) * kPdim;
-  const bool v_wide = (wrow0 + kWavePos <= rows_here) && ((reinterpret_cast<uintptr_t>(vblock) & 15) == 0);
+  const bool v_wide = PLAIN || ((wrow0 + kWavePos <= rows_here) && ((reinterpret_cast<uintptr_t>(vblock) & 15) == 0));
   u4 vq[4];
   uint32_t vd[13];
   if (v_wide) {
-    const u4* vb4 = reinterpret_cast<const u4*>(vblock);
+    const char* vb = reinterpret_cast<const char*>(vblock);
 #pragma unroll
-    for (int i = 0; i < 3; ++i) vq[i] = vb4[i * 64 + lane];
-    vq[3] = vb4[192 + (lane & 15)];                      // 208 pieces in all; lanes >= 16 repeat
+    for (int i = 0; i < 3; ++i) vq[i] = *reinterpret_cast<const u4*>(vb + i * 1024 + (uint32_t)(lane * 16));
+    vq[3] = *reinterpret_cast<const u4*>(vb + 3072 + (uint32_t)((lane & 15) * 16));   // 208 pieces in all; lanes >= 16 repeat
   } else {
     const int valid_words = max(0, rows_here - wrow0) * kPdim;       // words of the block inside the sequence
     const uint32_t* tile_base = vblock - (int64_t)wrow0 * kPdim;     // row 0 of the tile: always valid
@@ -186,12 +190,20 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
   __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_sched_barrier(0);
   u4 kreg[16];
+  // byte offsets of this lane's piece for even / odd instruction numbers (r & 7 depends on i & 1 only)
+  const uint32_t koff_even = (uint32_t)(((wrow0 + (lane >> 4)) * 16 + ((lane & 15) ^ ((lane >> 4) & 7))) * 16);
+  const uint32_t koff_odd = (uint32_t)(((wrow0 + 4 + (lane >> 4)) * 16 + ((lane & 15) ^ ((4 + (lane >> 4)) & 7))) * 16);
   auto issue_k = [&](int i) {
-    const int r = 4 * i + (lane >> 4);
-    const int piece = (lane & 15) ^ (r & 7);
-    int row = wrow0 + r;
-    row = row < last_row ? row : last_row;
-    kreg[i] = kbase[(unsigned)(row * 16 + piece)];
+    if (PLAIN) {
+      const char* kb = reinterpret_cast<const char*>(kbase) + (i >> 1) * 2048;      // 8 rows of 256 bytes per pair
+      kreg[i] = *reinterpret_cast<const u4*>(kb + ((i & 1) ? koff_odd : koff_even));
+    } else {
+      const int r = 4 * i + (lane >> 4);
+      const int piece = (lane & 15) ^ (r & 7);
+      int row = wrow0 + r;
+      row = row < last_row ? row : last_row;
+      kreg[i] = *reinterpret_cast<const u4*>(reinterpret_cast<const char*>(kbase) + (uint32_t)((row * 16 + piece) * 16));
+    }
   };
 #pragma unroll
   for (int i = 0; i < 8; ++i) issue_k(i);
@@ -294,10 +306,14 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
     for (int j = 0; j < 4; ++j) {
       const int row = wrow0 + 16 * t + 4 * g + j;                      // accumulator row 4g + j of tile t
       float v = acc[j] * a.attn_scale;
-      if (a.mask && row < rows_here && n16 < n_rep)
-        v += a.mask[(int64_t)seq * a.mask_seq_stride + ((int64_t)kvh * n_rep + n16) * a.mask_head_stride +
-                    tile_p0 + row];
-      s[t][j] = (row < rows_here) ? v : -INFINITY;
+      if (PLAIN) {
+        s[t][j] = v;
+      } else {
+        if (a.mask && row < rows_here && n16 < n_rep)
+          v += a.mask[(int64_t)seq * a.mask_seq_stride + ((int64_t)kvh * n_rep + n16) * a.mask_head_stride +
+                      tile_p0 + row];
+        s[t][j] = (row < rows_here) ? v : -INFINITY;
+      }
     }
   };
   // schedule: look-ups (ALU + LDS) alternate with K instalments and score tiles, so the memory
