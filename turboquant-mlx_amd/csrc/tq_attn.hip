@@ -564,7 +564,8 @@ int launch_vonly_mfma(const void* q, const void* k_f16, const uint32_t* v_packed
   a.v_unscale = tq::fill_codebook_fp16(vcb, v_centroids, sh.bits);
   if (phases & 1) {
     dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
-    const bool plain = !sh.mask && !sh.seq_offsets && sh.seq_len % tqm::kTilePos == 0 && tq::aligned(v_packed, 16) &&
+    const bool plain = !sh.mask && !sh.seq_offsets && sh.attn_scale > 0.0f && sh.seq_len % tqm::kTilePos == 0 &&
+                       tq::aligned(v_packed, 16) &&
                        sh.v_seq_stride % 4 == 0 && sh.v_head_stride % 4 == 0;
     if (plain) tqm::vonly_tile_mfma_kernel<true><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb);
     else tqm::vonly_tile_mfma_kernel<false><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb);

@@ -51,6 +51,7 @@ constexpr int kWavePos = 64;
 constexpr int kTilePos = kWaves * kWavePos;      // 512 positions per workgroup
 constexpr int kMfmaThreads = kWaves * 64;
 constexpr int kHeadsMax = 16;
+constexpr float kLog2e = 1.44269504088896340736f;
 constexpr int kMergeThreads = 256;
 
 struct MfmaArgs {
@@ -238,15 +239,13 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
   }
   nmax = fmaxf(nmax, shfl_xor_f(nmax, 16));
   nmax = fmaxf(nmax, shfl_xor_f(nmax, 32));
-  // power-of-two scale 2^-floor(log2 nmax): keeps P * norm inside half range whatever the norms are
+  // power-of-two scale 2^kexp, kexp = -floor(log2 nmax) (clamped to +-100): keeps P * norm inside half
+  // range whatever the norms are.  It enters through the exponent of the weights (exact), not as
+  // a multiplication of the norms.
   int ex = (int)((__float_as_uint(nmax) >> 23) & 0xFF);
-  ex = ex < 1 ? 127 : (ex > 253 ? 253 : ex);
-  const float tscale = __uint_as_float((uint32_t)(254 - ex) << 23);
+  ex = ex < 27 ? (ex < 1 ? 127 : 27) : (ex > 227 ? 227 : ex);
+  const float kexp = (float)(127 - ex);
   const float inv_tscale = __uint_as_float((uint32_t)ex << 23);
-#pragma unroll
-  for (int t = 0; t < 4; ++t)
-#pragma unroll
-    for (int j = 0; j < 4; ++j) vn[t][j] *= tscale;
 
   // ---- packed V -> table indices (registers), then look-ups interleaved with the score tiles -----------
   uint32_t* stage = reinterpret_cast<uint32_t*>(big_s) + wave * 1024;   // this wave's 4 KB
@@ -291,6 +290,7 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
   };
   // one 16-position score tile: K pieces through the wave's staging area, 4 matrix instructions
   float s[4][4];
+  const float cs = a.attn_scale * kLog2e;                // scores are kept in log2 units: e^x = 2^(x log2 e)
   u4* kst = reinterpret_cast<u4*>(stage);                             // 256 pieces of 16 bytes
   auto qk_tile = [&](int t) {
 #pragma unroll
@@ -305,13 +305,13 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int row = wrow0 + 16 * t + 4 * g + j;                      // accumulator row 4g + j of tile t
-      float v = acc[j] * a.attn_scale;
       if (PLAIN) {
-        s[t][j] = v;
+        s[t][j] = acc[j];                                              // raw: the scale joins the exponent's fma
       } else {
+        float v = acc[j] * cs;                                         // log2 units
         if (a.mask && row < rows_here && n16 < n_rep)
-          v += a.mask[(int64_t)seq * a.mask_seq_stride + ((int64_t)kvh * n_rep + n16) * a.mask_head_stride +
-                      tile_p0 + row];
+          v += kLog2e * a.mask[(int64_t)seq * a.mask_seq_stride + ((int64_t)kvh * n_rep + n16) * a.mask_head_stride +
+                               tile_p0 + row];
         s[t][j] = (row < rows_here) ? v : -INFINITY;
       }
     }
@@ -345,7 +345,11 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
     for (int j = 0; j < 4; ++j) m = fmaxf(m, s[t][j]);
   m = fmaxf(m, shfl_xor_f(m, 16));
   m = fmaxf(m, shfl_xor_f(m, 32));
-  const float msafe = (m == -INFINITY) ? 0.0f : m;
+  // PLAIN: s is the raw product and attn_scale > 0 (host check), so the maximum commutes with the
+  // scaling; weights = 2^(s * cs - m * cs + kexp) in one fma + v_exp_f32.
+  const float arg_scale = PLAIN ? cs : 1.0f;
+  m = m * arg_scale;                                     // log2 units from here on (-inf stays -inf)
+  const float bias = kexp - ((m == -INFINITY) ? 0.0f : m);
   float l = 0.0f;
   uint32_t pa[2][4];                                     // A operands of the value product
 #pragma unroll
@@ -353,7 +357,7 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
     float p[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      p[j] = __expf(s[t][j] - msafe);
+      p[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][j], arg_scale, bias));   // weight * 2^kexp
       l += p[j];
       p[j] *= vn[t][j];
     }
@@ -362,6 +366,7 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
   }
   l += shfl_xor_f(l, 16);
   l += shfl_xor_f(l, 32);
+  l *= inv_tscale;
 
   // ---- values ------------------------------------------------------------------------------------------
   f4 accS[8];
@@ -398,7 +403,7 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
 #pragma unroll
     for (int ww = 1; ww < kWaves; ++ww) M = fmaxf(M, m_s[ww][h]);
     const float mw = m_s[w][h];
-    f_s[w][h] = (mw == -INFINITY) ? 0.0f : __expf(mw - M);
+    f_s[w][h] = (mw == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(mw - M);
     if (w == 0) M_s[h] = M;
   }
   __syncthreads();
@@ -477,8 +482,8 @@ __global__ __launch_bounds__(kMergeThreads) void decode_merge_rows_kernel(
     for (int u = 0; u < 8; ++u) {
       if (t0 + 8 * u < n_tiles && ml[u].x != -INFINITY) {
         const float Mn = fmaxf(M, ml[u].x);
-        const float fo = (M == -INFINITY) ? 0.0f : __expf(M - Mn);
-        const float fc = __expf(ml[u].x - Mn);
+        const float fo = (M == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(M - Mn);
+        const float fc = __builtin_amdgcn_exp2f(ml[u].x - Mn);
         acc = acc * fo + x[u] * fc;
         L = L * fo + ml[u].y * fc;
         M = Mn;
@@ -496,7 +501,7 @@ __global__ __launch_bounds__(kMergeThreads) void decode_merge_rows_kernel(
   float v[2] = {0.0f, 0.0f};
 #pragma unroll
   for (int p = 0; p < 8; ++p) {
-    const float f = (ml_s[p][0] == -INFINITY) ? 0.0f : __expf(ml_s[p][0] - Mt);
+    const float f = (ml_s[p][0] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(ml_s[p][0] - Mt);
     Lt += f * ml_s[p][1];
     v[0] += f * acc_s[p][lane];
     v[1] += f * acc_s[p][lane + 64];

@@ -104,7 +104,7 @@ __device__ __forceinline__ void fill_lut(uint32_t* lut, const Codebook& cb, int 
 
 // grid = (n_tiles_max, n_kv, n_seq), 512 threads.
 template <int MODE>
-__global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(2, 4)))
+__global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(4, 4)))
 void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
   constexpr bool HAS_K = MODE != kWeights;
   constexpr bool HAS_V = MODE != kScores;
@@ -182,7 +182,8 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
       (&q_s[0][0])[tid + i * kMfmaThreads] = *reinterpret_cast<const uint32_t*>(&h);
       (&ql_s[0][0])[tid + i * kMfmaThreads] = pack_h2(my_q[i].x - back.x, my_q[i].y - back.y);
     }
-    kn_s[wave][lane] = my_kn;
+    // the score scale rides on the key norm: log2 units for the softmax, plain units for kScores
+    kn_s[wave][lane] = my_kn * (MODE == kFlash ? a.score_scale * kLog2e : a.score_scale);
   }
   if (HAS_V) vn_s[wave][lane] = my_vn;
   __syncthreads();
@@ -191,7 +192,7 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
 
   // ---- V: norms, table indices --------------------------------------------------------------------------
   float vn[4][4];
-  float inv_tscale = 1.0f;
+  float inv_tscale = 1.0f, kexp = 0.0f;
   uint32_t X[2][4], Y[2][4];
   if (HAS_V) {
     float nmax = 0.0f;
@@ -204,13 +205,16 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
     nmax = fmaxf(nmax, shfl_xor_f(nmax, 16));
     nmax = fmaxf(nmax, shfl_xor_f(nmax, 32));
     int ex = (int)((__float_as_uint(nmax) >> 23) & 0xFF);
-    ex = ex < 1 ? 127 : (ex > 253 ? 253 : ex);
-    const float tscale = __uint_as_float((uint32_t)(254 - ex) << 23);
+    ex = ex < 27 ? (ex < 1 ? 127 : 27) : (ex > 227 ? 227 : ex);
+    kexp = (float)(127 - ex);                            // weights carry 2^kexp: through the exponent (kFlash) ...
     inv_tscale = __uint_as_float((uint32_t)ex << 23);
+    if (MODE == kWeights) {                              // ... or, for given weights, on the norms
+      const float tscale = __uint_as_float((uint32_t)(254 - ex) << 23);
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
+      for (int t = 0; t < 4; ++t)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) vn[t][j] *= tscale;
+        for (int j = 0; j < 4; ++j) vn[t][j] *= tscale;
+    }
 
     stage_block(vb_, stage, lane);
     int w0, sh_lo, sh_hi;
@@ -262,9 +266,9 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int row = wrow0 + 16 * t + 4 * g + j;
-        float v = (acc[j] * knv[j]) * a.score_scale;
+        float v = acc[j] * knv[j];
         if (MODE == kFlash && a.mask && row < rows_here && n16 < n_rep)
-          v += a.mask[(int64_t)seq * a.mask_seq_stride + ((int64_t)kvh * n_rep + n16) * a.mask_head_stride +
+          v += kLog2e * a.mask[(int64_t)seq * a.mask_seq_stride + ((int64_t)kvh * n_rep + n16) * a.mask_head_stride +
                       tile_p0 + row];
         s[t][j] = (row < rows_here) ? v : -INFINITY;
       }
@@ -296,13 +300,13 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
     m = fmaxf(m, shfl_xor_f(m, 16));
     m = fmaxf(m, shfl_xor_f(m, 32));
   }
-  const float msafe = (m == -INFINITY) ? 0.0f : m;
+  const float bias = kexp - ((m == -INFINITY) ? 0.0f : m);
 #pragma unroll
   for (int t = 0; t < 4; ++t) {
     float p[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      p[j] = (MODE == kFlash) ? __expf(s[t][j] - msafe) : wgt[t][j];
+      p[j] = (MODE == kFlash) ? __builtin_amdgcn_exp2f(s[t][j] + bias) : wgt[t][j];   // kFlash: weight * 2^kexp
       l += p[j];
       p[j] *= vn[t][j];
     }
@@ -311,6 +315,7 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
   }
   l += shfl_xor_f(l, 16);
   l += shfl_xor_f(l, 32);
+  if (MODE == kFlash) l *= inv_tscale;
 
   // ---- values ------------------------------------------------------------------------------------------
   f4 accS[8];
@@ -349,7 +354,7 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
 #pragma unroll
     for (int ww = 1; ww < kWaves; ++ww) M = fmaxf(M, m_s[ww][h]);
     const float mw = m_s[w][h];
-    f_s[w][h] = (mw == -INFINITY) ? 0.0f : __expf(mw - M);
+    f_s[w][h] = (mw == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(mw - M);
     if (w == 0) M_s[h] = M;
   }
   __syncthreads();
