@@ -467,6 +467,8 @@ __global__ __launch_bounds__(kMergeThreads) void decode_merge_rows_kernel(
   const int64_t grp = (int64_t)seq * n_kv + kvh;
   const float* gS = ws_S + grp * n_tiles_max * (int64_t)(n_rep * kD) + r * kD + 4 * eq;
   const float* gml = ws_ml + grp * n_tiles_max * (int64_t)(n_rep * 2) + r * 2;
+  // issued first: the signs are only needed at the very end, their latency hides behind everything else
+  const float sign0 = signs[lane], sign1 = signs[lane + 64];
   float M = -INFINITY, L = 0.0f;
   f4 acc = {0.f, 0.f, 0.f, 0.f};
   for (int t0 = ph; t0 < n_tiles; t0 += 64) {            // 8 tiles per lane group and round
@@ -478,16 +480,22 @@ __global__ __launch_bounds__(kMergeThreads) void decode_merge_rows_kernel(
       x[u] = *reinterpret_cast<const f4*>(gS + (int64_t)t * (n_rep * kD));
       ml[u] = *reinterpret_cast<const float2*>(gml + (int64_t)t * (n_rep * 2));
     }
+    // maximum of the round first, then one independent 2^(m - M) per tile
+    float Mr = M;
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      if (t0 + 8 * u < n_tiles && ml[u].x != -INFINITY) {
-        const float Mn = fmaxf(M, ml[u].x);
-        const float fo = (M == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(M - Mn);
-        const float fc = __builtin_amdgcn_exp2f(ml[u].x - Mn);
-        acc = acc * fo + x[u] * fc;
-        L = L * fo + ml[u].y * fc;
-        M = Mn;
+    for (int u = 0; u < 8; ++u)
+      if (t0 + 8 * u < n_tiles) Mr = fmaxf(Mr, ml[u].x);
+    if (Mr != -INFINITY) {
+      const float fo = (M == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(M - Mr);
+      acc = acc * fo;
+      L = L * fo;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const float fc = (t0 + 8 * u < n_tiles && ml[u].x != -INFINITY) ? __builtin_amdgcn_exp2f(ml[u].x - Mr) : 0.0f;
+        acc = acc + x[u] * fc;
+        L = L + ml[u].y * fc;
       }
+      M = Mr;
     }
   }
   *reinterpret_cast<f4*>(&acc_s[ph][4 * eq]) = acc;
@@ -511,7 +519,7 @@ __global__ __launch_bounds__(kMergeThreads) void decode_merge_rows_kernel(
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int e = lane + 64 * i;
-    float val = (v[i] * signs[e]) * inv_dim;
+    float val = (v[i] * (i ? sign1 : sign0)) * inv_dim;
     if (NORM) val = (Lt > 0.0f) ? val / Lt : 0.0f;
     store_from_float<TO>(o + e, val);
   }
