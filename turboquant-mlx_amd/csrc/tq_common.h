@@ -105,6 +105,30 @@ template <int D> struct Lay { static constexpr int EPL = (D >= 64) ? D / 64 : 1;
 
 __device__ __forceinline__ float shfl_xor_f(float v, int m) { return __shfl_xor(v, m, TQ_WAVE); }
 
+// Value of lane (own ^ H): lanes 1 and 2 apart through a quad permute folded into the consuming
+// instruction, 4 to 16 apart through ds_swizzle (no address register), 32 apart through a permute.
+template <int H>
+__device__ __forceinline__ float lane_xor(float v) {
+  if constexpr (H == 1) {
+    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true));
+  } else if constexpr (H == 2) {
+    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xF, 0xF, true));
+  } else if constexpr (H <= 16) {
+    return __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), (H << 10) | 0x1F));   // xor mask, and mask 31
+  } else {
+    return __shfl_xor(v, H, TQ_WAVE);
+  }
+}
+
+// One lane-exchange stage: the element whose lane has bit H clear receives own + partner, the
+// other partner - own (= partner + (-own): the same single rounding).
+template <int H, int EPL>
+__device__ __forceinline__ void butterfly_lane_stage(float (&v)[EPL], int lane) {
+  const uint32_t flip = (lane & H) ? 0x80000000u : 0u;
+#pragma unroll
+  for (int i = 0; i < EPL; ++i) v[i] = lane_xor<H>(v[i]) + __uint_as_float(__float_as_uint(v[i]) ^ flip);
+}
+
 // Raw (un-normalised) Walsh-Hadamard butterfly, stages h = 1, 2, ..., D/2; the element whose
 // index has bit h clear receives a+b, its partner a-b.  Stages below 64 exchange lanes, stages
 // from 64 up are register-to-register.  Float adds only, so the result is the same expression
@@ -112,15 +136,12 @@ __device__ __forceinline__ float shfl_xor_f(float v, int m) { return __shfl_xor(
 template <int D>
 __device__ __forceinline__ void raw_butterfly(float (&v)[Lay<D>::EPL], int lane) {
   constexpr int EPL = Lay<D>::EPL;
-#pragma unroll
-  for (int h = 1; h < 64 && h < D; h <<= 1) {
-    const bool upper = (lane & h) != 0;
-#pragma unroll
-    for (int i = 0; i < EPL; ++i) {
-      float p = shfl_xor_f(v[i], h);
-      v[i] = upper ? (p - v[i]) : (v[i] + p);
-    }
-  }
+  if constexpr (D > 1) butterfly_lane_stage<1, EPL>(v, lane);
+  if constexpr (D > 2) butterfly_lane_stage<2, EPL>(v, lane);
+  if constexpr (D > 4) butterfly_lane_stage<4, EPL>(v, lane);
+  if constexpr (D > 8) butterfly_lane_stage<8, EPL>(v, lane);
+  if constexpr (D > 16) butterfly_lane_stage<16, EPL>(v, lane);
+  if constexpr (D > 32) butterfly_lane_stage<32, EPL>(v, lane);
 #pragma unroll
   for (int h = 64; h < D; h <<= 1) {
     const int hs = h / 64;
