@@ -395,3 +395,33 @@ def fused_like(tq, k, v):
     cache = tq.TurboQuantKVCache(bits=3, fused=True)
     cache.update_and_fetch(k, v)
     return cache
+
+
+def test_vonly_cache_fused_mode(tq):
+    """fused=True on a V-only cache: values are only encoded (placeholder returned), the packed state
+    is the unfused cache's, decode attention is identical, and a multi-token step through the
+    dispatcher dequantises on demand."""
+    from tqhip import patch
+    B, n_q, n_kv, S, D = 1, 8, 4, 300, 128
+    sc = 1 / math.sqrt(D)
+    k, v = rand((B, n_kv, S, D), 80), rand((B, n_kv, S, D), 81)
+    k1, v1 = rand((B, n_kv, 1, D), 82), rand((B, n_kv, 1, D), 83)
+    q1, qs = rand((B, n_q, 1, D), 84), rand((B, n_q, S, D), 85)
+    plain, fused = tq.VOnlyTurboQuantCache(bits=3), tq.VOnlyTurboQuantCache(bits=3, fused=True)
+    kp_, vp_ = plain.update_and_fetch(k, v)
+    kf_, vf_ = fused.update_and_fetch(k, v)
+    assert torch.equal(kp_, kf_) and vf_.shape == vp_.shape and float(vf_.abs().max()) == 0.0
+    assert vf_.untyped_storage().nbytes() == vf_.element_size()          # one element, expanded
+    assert torch.equal(fused.dequantized_values(torch.float16), vp_)
+    # multi-token step: stock SDPA over K and the on-demand dequantised V
+    a = patch.scaled_dot_product_attention(qs, kf_, vf_, fused, sc, "causal")
+    b = patch.scaled_dot_product_attention(qs, kp_, vp_, plain, sc, "causal")
+    assert torch.equal(a, b)
+    plain.update_and_fetch(k1, v1)
+    kf_, vf_ = fused.update_and_fetch(k1, v1)
+    assert fused.offset == S + 1 and vf_.shape == (B, n_kv, S + 1, D)
+    for x, y in zip(plain.state, fused.state):
+        assert torch.equal(x, y)
+    assert torch.equal(tq.vonly_decode_attention(q1, fused, sc), tq.vonly_decode_attention(q1, plain, sc))
+    assert torch.equal(patch.scaled_dot_product_attention(q1, kf_, vf_, fused, sc, None),
+                       tq.vonly_decode_attention(q1, plain, sc))

@@ -53,10 +53,12 @@ def turboquant_attention(queries: torch.Tensor, cache, attn_scale: float, mask=N
         m = None
         if mask is not None:
             m = torch.stack([_mask_rows(mask, b, n_q, total).expand(n_q, total) for b in range(B)])
+        od = queries.dtype if queries.dtype in (torch.float16, torch.bfloat16, torch.float32) else torch.float32
         out = ops.flash_decode(q_rot, cache.k_packed, cache.k_norms, cache.v_packed, cache.v_norms,
                                kq.centroids, vq.centroids, vq.signs, dim, bits, attn_scale, n_rep=n_rep,
-                               seq_len=total, mask=m)
-        return out[:, :, None, :].to(queries.dtype)
+                               seq_len=total, mask=m, out_dtype=od)
+        out = out[:, :, None, :]
+        return out if out.dtype == queries.dtype else out.to(queries.dtype)
 
     outputs = []
     for b in range(B):
@@ -105,9 +107,11 @@ def vonly_decode_attention(queries: torch.Tensor, cache, attn_scale: float, mask
         m = None
         if mask is not None:
             m = torch.stack([_mask_rows(mask, b, n_q, total).expand(n_q, total) for b in range(B)])
+        od = queries.dtype if queries.dtype in (torch.float16, torch.bfloat16, torch.float32) else torch.float32
         out = ops.vonly_decode(queries[:, :, 0, :], kc.keys, tq.v_packed, tq.v_norms, vq.centroids, vq.signs,
-                               dim, bits, attn_scale, n_rep=n_rep, seq_len=total, mask=m)
-        return out[:, :, None, :].to(queries.dtype)
+                               dim, bits, attn_scale, n_rep=n_rep, seq_len=total, mask=m, out_dtype=od)
+        out = out[:, :, None, :]                           # written in the query dtype by the merge pass
+        return out if out.dtype == queries.dtype else out.to(queries.dtype)
     outputs = []
     for b in range(B):
         scores = ops.dense_qk_scores(queries[b, :, 0, :], kc.keys[b, :, :total, :], 1.0, n_rep=n_rep)

@@ -39,7 +39,14 @@ def _need_gpu(*tensors):
                 f"{t.device}; there is no CPU fallback")
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(t: torch.Tensor):
+    """Raw hipStream_t of torch's current stream on the tensor's device."""
+    if _raw_stream is not None:                       # avoids building a torch.cuda.Stream object per call
+        idx = t.device.index
+        return C.c_void_p(_raw_stream(torch.cuda.current_device() if idx is None else idx))
     return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
 
 
@@ -57,7 +64,7 @@ def _dt(t: torch.Tensor) -> int:
 def _host_table(x):
     """Small table (boundaries / centroids) as a ctypes float array.  Accepts tensors, lists."""
     if isinstance(x, torch.Tensor):
-        key = (x.data_ptr(), x._version, x.numel(), str(x.device))
+        key = (x.data_ptr(), x._version, x.numel())
         hit = _host_table.cache.get(key)
         if hit is None:
             hit = _lib.host_floats(x.detach().float().cpu().tolist())
@@ -72,6 +79,8 @@ _host_table.cache = {}
 
 
 def _as_f32_dev(x, like: torch.Tensor) -> torch.Tensor:
+    if isinstance(x, torch.Tensor) and x.dtype == torch.float32 and x.device == like.device and x.is_contiguous():
+        return x
     if not isinstance(x, torch.Tensor):
         x = torch.tensor(list(x), dtype=torch.float32)
     return x.to(device=like.device, dtype=torch.float32).contiguous()
@@ -467,8 +476,8 @@ def flash_decode(q_rot: torch.Tensor, k_packed, k_norms, v_packed, v_norms, k_ce
     q_rot = q_rot.to(torch.float32).contiguous()
     k_packed, ks = _kv_layout(_u32(k_packed), pd, ragged)
     v_packed, vs = _kv_layout(_u32(v_packed), pd, ragged)
-    k_norms, kns = _norm_layout(k_norms.to(torch.float32))
-    v_norms, vns = _norm_layout(v_norms.to(torch.float32))
+    k_norms, kns = _norm_layout(k_norms if k_norms.dtype == torch.float32 else k_norms.to(torch.float32))
+    v_norms, vns = _norm_layout(v_norms if v_norms.dtype == torch.float32 else v_norms.to(torch.float32))
     if ragged:
         if max_seq_len is None:
             raise ValueError("max_seq_len is required with seq_offsets")
@@ -528,7 +537,7 @@ def vonly_decode(q: torch.Tensor, k: torch.Tensor, v_packed, v_norms, v_centroid
     q = q.contiguous()
     k, ks = _kv_layout(k, dim, ragged)
     v_packed, vs = _kv_layout(_u32(v_packed), pd, ragged)
-    v_norms, vns = _norm_layout(v_norms.to(torch.float32))
+    v_norms, vns = _norm_layout(v_norms if v_norms.dtype == torch.float32 else v_norms.to(torch.float32))
     if ragged:
         if max_seq_len is None:
             raise ValueError("max_seq_len is required with seq_offsets")

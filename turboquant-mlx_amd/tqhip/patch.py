@@ -50,9 +50,12 @@ def scaled_dot_product_attention(queries, keys, values, cache, scale, mask=None,
             return turboquant_prefill_attention(queries, cache, scale, causal=mask is not None)
         raise ValueError("a fused TurboQuantKVCache holds no dequantised K/V: a multi-token step takes "
                          "mask=None or mask='causal' (cache.make_mask(N)), not an explicit array")
-    if isinstance(cache, VOnlyTurboQuantCache) and is_decode and cache.offset > 0:
-        return vonly_decode_attention(queries, cache, scale, mask,
-                                      sparse_v_threshold=getattr(cache, "sparse_v_threshold", None))
+    if isinstance(cache, VOnlyTurboQuantCache) and cache.offset > 0:
+        if is_decode:
+            return vonly_decode_attention(queries, cache, scale, mask,
+                                          sparse_v_threshold=getattr(cache, "sparse_v_threshold", None))
+        if cache.fused:                    # the values handed in are a placeholder
+            values = cache.dequantized_values(queries.dtype)
     return _stock_sdpa(queries, keys, values, scale, mask)
 
 

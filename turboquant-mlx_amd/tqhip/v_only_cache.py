@@ -11,16 +11,46 @@ from .kvcache import KVCache
 class VOnlyTurboQuantCache:
     """update_and_fetch stores K in fp16, compresses V and returns (K_fp16, V_dequantised).
     With no_v_buffer=True the fp16 V buffer is not kept: V is re-dequantised from the packed
-    storage on every call (v_only_cache.py:41-49)."""
+    storage on every call (v_only_cache.py:41-49).
 
-    def __init__(self, bits: int = 3, seed: int = 42, no_v_buffer: bool = False):
+    fused=True (not in the reference, which relies on MLX never evaluating an unused dequant; same
+    meaning as TurboQuantKVCache(fused=True), cache.py:162-165): V is only encoded, and the second
+    return value is a stride-0 all-zero placeholder of the right shape.  For callers that read the
+    packed values directly (vonly_decode_attention, tqhip.patch); `dequantized_values()` gives the
+    fp16 values when a multi-token step needs them."""
+
+    def __init__(self, bits: int = 3, seed: int = 42, no_v_buffer: bool = False, fused: bool = False):
         self._k_cache = KVCache()
         self._v_tq = TurboQuantKVCache(bits=bits, seed=seed, v_only=True)
         self._v_bits = bits
         self._no_v_buffer = no_v_buffer
+        self.fused = fused
+        self._zero, self._zero_key = None, None
+
+    def _encode_only(self, keys, values):
+        tq = self._v_tq
+        B, H, S, v_dim = values.shape
+        tq._dtype = keys.dtype
+        tq._ensure_quantizer(keys.shape[-1], v_dim, values.device)
+        tq._ensure_storage(B, H, S, values.device)
+        tq._encode(values, tq._v_q, tq.v_packed, tq.v_norms, B, H, S, v_dim, tq.offset)
+        tq.offset += S
+
+    def dequantized_values(self, dtype=None) -> torch.Tensor:
+        """All cached values, dequantised: [B, H, offset, D]."""
+        tq = self._v_tq
+        B, H = tq.v_packed.shape[0], tq.v_packed.shape[1]
+        return tq._full_dequant(tq.v_packed, tq.v_norms, tq._v_q, tq._v_dim, B, H, tq.offset, dtype or tq._dtype)
 
     def update_and_fetch(self, keys: torch.Tensor, values: torch.Tensor):
         k_out, _ = self._k_cache.update_and_fetch(keys, values)
+        if self.fused:
+            self._encode_only(keys, values)
+            B, H, _, v_dim = values.shape
+            key = (values.dtype, values.device)
+            if self._zero is None or self._zero_key != key:          # one element, made once
+                self._zero, self._zero_key = torch.zeros((1, 1, 1, 1), dtype=values.dtype, device=values.device), key
+            return k_out, self._zero.expand(B, H, self._v_tq.offset, v_dim)
         if self._no_v_buffer:                                    # v_only_cache.py:54-75
             tq = self._v_tq
             B, H, S, v_dim = values.shape
