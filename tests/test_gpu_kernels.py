@@ -742,3 +742,45 @@ def test_prefill_attention_argument_errors(tq):
                              64, 3, 0.1, n_rep=2)                                 # no kernel for d = 64
     empty = tq.prefill_attention(dev(q[:, :0]), *args, 128, 3, 0.1, n_rep=2, q_pos0=0)
     assert empty.shape == (4, 0, 128)
+
+
+# ------------------------------------------------------------------ HIP graph capture
+
+def test_decode_ops_replay_under_hip_graph(tq):
+    """The ops only launch kernels on torch's current stream (no allocation once the workspace exists,
+    no memset nodes), so a decode step can be captured once and replayed.  Every replay - with the
+    inputs rewritten in place and eager work in between - must reproduce the eager result."""
+    rng = np.random.default_rng(90)
+    n_kv, n_rep, T, D, bits = 4, 7, 2048, 128, 3
+    c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, n_kv, T, D, bits)
+    sc = 1 / math.sqrt(D)
+    q = dev(rng.standard_normal((1, n_kv * n_rep, D)).astype(np.float16))
+    Kd, vpd, vnd, kpd, knd = dev(K), dev(vp), dev(vn), dev(kp), dev(kn)
+    vsd, ksd = dev(vs), dev(ks)
+
+    def step():
+        a = tq.vonly_decode(q, Kd, vpd, vnd, c, vsd, D, bits, sc, n_rep=n_rep)
+        q_rot = tq.prerotate_query(q[0], ksd)
+        b = tq.flash_attention_turboquant(q_rot, kpd, knd, vpd, vnd, c, c, vsd, D, bits, sc, n_rep=n_rep)
+        return a, b
+
+    step()                                                    # warm-up: workspace, tables
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        step()
+        with torch.cuda.graph(graph, stream=side):
+            ga, gb = step()
+    torch.cuda.current_stream().wait_stream(side)
+    for it in range(4):
+        q.copy_(dev(rng.standard_normal((1, n_kv * n_rep, D)).astype(np.float16)))
+        if it == 2:
+            Kd.mul_(0.5)                                       # the graph reads the buffers, not a snapshot
+        graph.replay()
+        torch.cuda.synchronize()
+        ra, rb = ga.clone(), gb.clone()
+        ea, eb = step()                                        # eager work between the replays
+        torch.cuda.synchronize()
+        assert torch.equal(ra, ea) and torch.equal(rb, eb), it
