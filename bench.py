@@ -107,7 +107,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the hot path shards by kv head "
-              "with no communication; see DESIGN.md). Run with --gpus 1.", file=sys.stderr)
+              "with no communication). Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
 
     import numpy as np

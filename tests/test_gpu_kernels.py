@@ -127,7 +127,7 @@ def test_encode_near_boundary_values(tq):
 
 
 def test_config1_roundtrip(tq):
-    """BASELINE config 1: [1,4,1024,128] fp16 N(0,1): indices bit-exact, reconstruction MSE equal."""
+    """benchmark configuration 1: [1,4,1024,128] fp16 N(0,1): indices bit-exact, reconstruction MSE equal."""
     rng = np.random.default_rng(0)
     x = rng.standard_normal((1, 4, 1024, 128)).astype(np.float16)
     s = o.random_diagonal_sign(128, 43)
@@ -474,7 +474,7 @@ def test_flash_argument_errors(tq):
 
 
 def test_flash_ragged_batch(tq):
-    """A batch of sequences of different lengths in one launch (BASELINE config 4 shape, scaled down):
+    """A batch of sequences of different lengths in one launch (benchmark configuration 4 shape, scaled down):
     32 q heads, 8 kv heads, lengths drawn from the seed, fp16 output."""
     rng = np.random.default_rng(17)
     n_kv, n_rep, D, bits, n_seq = 8, 4, 128, 3, 5
@@ -548,7 +548,7 @@ def test_vonly_decode_ragged_and_mask(tq):
 
 
 def test_config2_full_size(tq):
-    """BASELINE config 2 at full size: 28 q / 4 kv heads, d=128, 32768 positions; V encoded on the
+    """benchmark configuration 2 at full size: 28 q / 4 kv heads, d=128, 32768 positions; V encoded on the
     GPU (bit-exact against the oracle), then the fused V-only decode step against the oracle."""
     rng = np.random.default_rng(2)
     n_kv, n_rep, T, D, bits = 4, 7, 32768, 128, 3
@@ -580,7 +580,7 @@ def test_config2_full_size(tq):
 
 @pytest.mark.parametrize("T", [4096, 16384, 65536])
 def test_config3_scores(tq, T):
-    """BASELINE config 3: pre-rotated-Q scoring over packed K, 28/4 heads, d=128."""
+    """benchmark configuration 3: pre-rotated-Q scoring over packed K, 28/4 heads, d=128."""
     rng = np.random.default_rng(3)
     n_kv, n_rep, D, bits = 4, 7, 128, 3
     c, b = tables(bits)
@@ -646,7 +646,7 @@ def test_flash_and_vonly_both_precisions(tq, precision):
 
 
 def test_config4_flash_ragged_full_heads(tq):
-    """BASELINE config 4 shape (scaled in length): 32 q / 8 kv heads, 16 sequences of ragged length,
+    """benchmark configuration 4 shape (scaled in length): 32 q / 8 kv heads, 16 sequences of ragged length,
     fp16 output, packed K and V."""
     rng = np.random.default_rng(4)
     n_kv, n_rep, D, bits, n_seq = 8, 4, 128, 3, 16
@@ -696,7 +696,7 @@ def test_prefill_attention_matches_oracle(tq, n_kv, n_rep, T, n_rows, pos0):
 
 
 def test_prefill_attention_noncausal_fp16_out_and_outliers(tq):
-    """1 % outlier channels (x20) in K, V and q as in BASELINE config 5; fp16 output; and the
+    """1 % outlier channels (x20) in K, V and q as in benchmark configuration 5; fp16 output; and the
     non-causal form, where every row sees every position."""
     rng = np.random.default_rng(52)
     n_kv, n_rep, T, n_rows = 2, 4, 1500, 200

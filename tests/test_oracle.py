@@ -218,7 +218,7 @@ def test_quantize_variants_differ_only_in_double_rounding():
 
 
 def test_config1_statistics():
-    # BASELINE config 1: [1,4,1024,128] fp16 N(0,1); textbook 8-level Lloyd-Max distortion
+    # benchmark configuration 1: [1,4,1024,128] fp16 N(0,1); textbook 8-level Lloyd-Max distortion
     rng = np.random.default_rng(0)
     x = rng.standard_normal((1, 4, 1024, 128)).astype(np.float16)
     s = o.random_diagonal_sign(128, 43)

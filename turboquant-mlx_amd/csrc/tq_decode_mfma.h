@@ -4,7 +4,7 @@
 // Tile pass.  A workgroup of 8 wavefronts owns 512 consecutive KV positions of one kv head; a
 // wavefront owns 64 of them and serves all n_rep query heads that share the kv head.  A CU can only
 // start one wave-wide load instruction every ~24 clocks, so the pass is built to need few of them
-// (22 per wave) and to have all of them in flight before any arithmetic starts:
+// (Q, norm, 4 for V, 16 for K per wave), issued as early as the schedule below allows:
 //
 //   K rows   16 x 16-byte loads per lane, fully coalesced (an instruction reads 4 whole rows), then
 //            turned into matrix-operand layout (one row per lane) through a 4 KB per-wave LDS buffer
@@ -25,7 +25,7 @@
 //
 // Merge pass.  One workgroup per query head folds the tile partials (running-maximum rescale),
 // applies the ONE Walsh-Hadamard butterfly per output row, signs, 1/dim and 1/l.  As a dependent
-// launch it costs about 1.3 us plus its own ~1 us; merging inside the tile pass instead (last
+// launch it costs a launch gap plus one memory round trip; merging inside the tile pass instead (last
 // workgroup to arrive) was measured slower, because a single CU cannot pull the ~230 KB of partials
 // of a kv head quickly and the counter/visibility round trips sit on the critical path.
 //

@@ -129,7 +129,7 @@ def bench_vonly(iters, dev):
 
 
 def bench_prefill(iters, dev):
-    """BASELINE config 5, attention half: a chunk of 512 query rows x 32 heads at the end of a
+    """benchmark configuration 5, attention half: a chunk of 512 query rows x 32 heads at the end of a
     131072-position packed cache (8 kv heads), causal.  Matrix-core bound: reported in TFLOP/s of
     the 4 * rows * heads * d * visible-positions useful flops against the 2.5 PFLOP/s fp16 peak."""
     cb = gaussian_codebook(3)
