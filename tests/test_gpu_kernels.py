@@ -784,3 +784,33 @@ def test_decode_ops_replay_under_hip_graph(tq):
         ea, eb = step()                                        # eager work between the replays
         torch.cuda.synchronize()
         assert torch.equal(ra, ea) and torch.equal(rb, eb), it
+
+
+# ------------------------------------------------------------------ streaming V-only kernel (several blocks per workgroup)
+
+@pytest.mark.parametrize("n_seq,n_kv,n_rep,T,blocks", [(8, 8, 2, 4096, 2), (8, 8, 2, 6144, 3), (4, 8, 4, 16384, 4)])
+def test_vonly_decode_streaming_blocks(tq, n_seq, n_kv, n_rep, T, blocks):
+    """Unmasked caches with more than 256 tiles of 512 positions take the streaming kernel, in which a
+    workgroup runs through `blocks` consecutive tiles with an online softmax.  Value norms jump by
+    factors of 2^+-6 between tiles and the largest scores sit in different tiles per head, so both the
+    running-maximum rescale and the change of the power-of-two norm scale are exercised."""
+    assert (T // 512) * n_kv * n_seq // 256 == blocks
+    rng = np.random.default_rng(95)
+    D, bits = 128, 3
+    c, b = tables(bits)
+    vs = o.random_diagonal_sign(D, 43)
+    sc = 1 / math.sqrt(D)
+    K = rng.standard_normal((n_seq, n_kv, T, D)).astype(np.float16)
+    V = rng.standard_normal((n_seq, n_kv, T, D)).astype(np.float32)
+    V *= (2.0 ** rng.integers(-6, 7, size=(n_seq, n_kv, T // 512, 1, 1))).repeat(512, axis=2).reshape(n_seq, n_kv, T, 1, 1)[..., 0]
+    q = rng.standard_normal((n_seq, n_kv * n_rep, D)).astype(np.float16)
+    Kd, qd = dev(K), dev(q)
+    vp, vn = tq.fused_quantize(dev(V.astype(np.float16)).reshape(-1, D), dev(vs), b, D, bits)
+    vp, vn = vp.reshape(n_seq, n_kv, T, -1), vn.reshape(n_seq, n_kv, T)
+    got = host(tq.vonly_decode(qd, Kd, vp, vn, c, dev(vs), D, bits, sc, n_rep=n_rep))
+    ref32 = host(tq.vonly_decode(qd, Kd, vp, vn, c, dev(vs), D, bits, sc, n_rep=n_rep, precision="fp32"))
+    hp, hn = host(vp), host(vn)
+    for sidx in range(0, n_seq, max(1, n_seq // 2)):             # oracle on a subset of the sequences
+        want = o.vonly_decode_attention(q[sidx], K[sidx], hp[sidx], hn[sidx], c, vs, D, bits, sc)
+        close(got[sidx], want, row_scale=True)
+    close(got.reshape(-1, D), ref32.reshape(-1, D), row_scale=True)   # every sequence against the float32 kernels

@@ -535,7 +535,18 @@ int launch_vonly_mfma(const void* q, const void* k_f16, const uint32_t* v_packed
                       size_t workspace_bytes, const tq_decode_shape& sh, hipStream_t stream, int phases) {
   const char* who = "tq_vonly_decode_attn";
   const int n_q = sh.n_kv_heads * sh.n_rep;
-  const int n_tiles = (int)((sh.seq_len + tqm::kTilePos - 1) / tqm::kTilePos);
+  const bool plain = !sh.mask && !sh.seq_offsets && sh.attn_scale > 0.0f && sh.seq_len % tqm::kTilePos == 0 &&
+                     tq::aligned(v_packed, 16) && sh.v_seq_stride % 4 == 0 && sh.v_head_stride % 4 == 0;
+  // Long unmasked caches: several consecutive 512-position blocks per workgroup, as many as still leave
+  // one workgroup per CU (256) and divide the length.
+  int n_blocks = 1;
+  if (plain) {
+    const int64_t wgs = (sh.seq_len / tqm::kTilePos) * sh.n_kv_heads * sh.n_seq;
+    for (int nb = (int)(wgs / 256 < 8 ? wgs / 256 : 8); nb > 1; --nb)
+      if ((sh.seq_len / tqm::kTilePos) % nb == 0) { n_blocks = nb; break; }
+  }
+  const int tile_pos = tqm::kTilePos * n_blocks;
+  const int n_tiles = (int)((sh.seq_len + tile_pos - 1) / tile_pos);
   const size_t need = (size_t)sh.n_seq * n_q * n_tiles * (tqm::kD + 2) * sizeof(float);
   if (!workspace || workspace_bytes < need)
     return tq::fail(TQ_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, need, workspace_bytes);
@@ -564,10 +575,8 @@ int launch_vonly_mfma(const void* q, const void* k_f16, const uint32_t* v_packed
   a.v_unscale = tq::fill_codebook_fp16(vcb, v_centroids, sh.bits);
   if (phases & 1) {
     dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
-    const bool plain = !sh.mask && !sh.seq_offsets && sh.attn_scale > 0.0f && sh.seq_len % tqm::kTilePos == 0 &&
-                       tq::aligned(v_packed, 16) &&
-                       sh.v_seq_stride % 4 == 0 && sh.v_head_stride % 4 == 0;
-    if (plain) tqm::vonly_tile_mfma_kernel<true><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb);
+    if (n_blocks > 1) tqm::vonly_stream_kernel<<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb, n_blocks);
+    else     if (plain) tqm::vonly_tile_mfma_kernel<true><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb);
     else tqm::vonly_tile_mfma_kernel<false><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb);
     TQ_CHECK_LAUNCH(who);
   }
@@ -576,7 +585,7 @@ int launch_vonly_mfma(const void* q, const void* k_f16, const uint32_t* v_packed
   const float inv_dim = 1.0f / (float)sh.dim;
 #define LAUNCH_MERGE_M(TO)                                                                                \
   tqm::decode_merge_rows_kernel<TO, true><<<mgrid, tqm::kMergeThreads, 0, stream>>>(                        \
-      a.ws_S, a.ws_ml, sh.seq_offsets, sh.seq_len, n_tiles, sh.n_kv_heads, sh.n_rep, v_signs, inv_dim, (TO*)out)
+      a.ws_S, a.ws_ml, sh.seq_offsets, sh.seq_len, n_tiles, sh.n_kv_heads, sh.n_rep, v_signs, inv_dim, (TO*)out, tile_pos)
   if (sh.out_dtype == TQ_F16) { LAUNCH_MERGE_M(__half); }
   else if (sh.out_dtype == TQ_BF16) { LAUNCH_MERGE_M(__hip_bfloat16); }
   else { LAUNCH_MERGE_M(float); }
@@ -625,7 +634,7 @@ int launch_packed_mfma(const float* q_rot_or_weights, const uint32_t* k_packed, 
   const float inv_dim = 1.0f / (float)sh.dim;
 #define LAUNCH_MERGE_P(TO)                                                                                    \
   tqm::decode_merge_rows_kernel<TO, MODE == tqm::kFlash><<<mgrid, tqm::kMergeThreads, 0, stream>>>(            \
-      a.ws_S, a.ws_ml, sh.seq_offsets, sh.seq_len, n_tiles, sh.n_kv_heads, sh.n_rep, v_signs, inv_dim, (TO*)out)
+      a.ws_S, a.ws_ml, sh.seq_offsets, sh.seq_len, n_tiles, sh.n_kv_heads, sh.n_rep, v_signs, inv_dim, (TO*)out, tqm::kTilePos)
   if (sh.out_dtype == TQ_F16) { LAUNCH_MERGE_P(__half); }
   else if (sh.out_dtype == TQ_BF16) { LAUNCH_MERGE_P(__hip_bfloat16); }
   else { LAUNCH_MERGE_P(float); }

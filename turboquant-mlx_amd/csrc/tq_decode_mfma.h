@@ -447,6 +447,302 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
   TQ_STAMP(10);
 }
 
+// Streaming variant for long unmasked caches: one workgroup runs through n_blocks CONSECUTIVE
+// 512-position blocks with an online softmax in registers (the flash recurrence: running maximum,
+// rescale of the accumulators when it moves), and only then merges its eight waves and stores
+// one partial.  The fixed work of a tile - address set-up, Q / table staging, cross-wave merge,
+// partial store, about 40 % of a wave's instructions - is paid once per n_blocks blocks, the loads
+// of block b+1 are in flight while block b is computed, and the merge pass folds n_blocks times
+// fewer partials.  With one block it would do exactly what vonly_tile_mfma_kernel<true> does.
+// The partial of a workgroup is taken relative to R = m - kexp (running maximum in log2 units minus
+// the exponent of the power-of-two norm scale of the block that set it): weights are
+// 2^(s*cs - R), and moving from R_old to R_new multiplies accumulators and weight sum by 2^(R_old - R_new).
+// grid = (seq_len / (512 * n_blocks), n_kv, n_seq), 512 threads.
+__global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
+  __shared__ __align__(16) unsigned char big_s[32768];
+  __shared__ uint32_t lut_s[64];
+  __shared__ __align__(16) uint32_t q_s[kHeadsMax][kD / 2];
+  __shared__ __align__(16) float nrm_s[kWaves][kWavePos];
+  __shared__ __align__(16) float alpha_s[kWaves][kHeadsMax];
+  __shared__ float m_s[kWaves][kHeadsMax], l_s[kWaves][kHeadsMax], M_s[kHeadsMax];
+  __shared__ __align__(16) float f_s[kWaves][kHeadsMax];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int n16 = lane & 15, g = lane >> 4;
+  const int tile = blockIdx.x, kvh = blockIdx.y, seq = blockIdx.z;
+  const int n_rep = a.n_rep;
+  const int n_q = a.n_kv * n_rep;
+  const int64_t q_row0 = (int64_t)seq * n_q + (int64_t)kvh * n_rep;
+  const int64_t tile_p0 = (int64_t)tile * kTilePos * n_blocks;
+  const int wrow0 = wave * kWavePos;
+
+  // per-block strides: 512 rows of norms (4 B), packed V (52 B), K (256 B)
+  const float* nb = a.v_norms + (int64_t)seq * a.vn_seq_stride + (int64_t)kvh * a.vn_head_stride + tile_p0 + wrow0 + lane;
+  const char* vb = reinterpret_cast<const char*>(
+      a.v_packed + ((int64_t)seq * a.v_seq_stride + (int64_t)kvh * a.v_head_stride + tile_p0 + wrow0) * kPdim);
+  const char* kbase = reinterpret_cast<const char*>(
+      a.k + ((int64_t)seq * a.k_seq_stride + (int64_t)kvh * a.k_head_stride + tile_p0) * kD);
+  const uint32_t voff = (uint32_t)(lane * 16), voff3 = (uint32_t)(3072 + (lane & 15) * 16);
+  const uint32_t koff_even = (uint32_t)(((wrow0 + (lane >> 4)) * 16 + ((lane & 15) ^ ((lane >> 4) & 7))) * 16);
+  const uint32_t koff_odd = (uint32_t)(((wrow0 + 4 + (lane >> 4)) * 16 + ((lane & 15) ^ ((4 + (lane >> 4)) & 7))) * 16);
+
+  uint32_t my_q[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int w = tid + i * kMfmaThreads;
+    my_q[i] = (w < n_rep * (kD / 2)) ? reinterpret_cast<const uint32_t*>(a.q + q_row0 * kD)[w] : 0u;
+  }
+  float my_norm = nb[0];
+  u4 vq[4];
+#pragma unroll
+  for (int i = 0; i < 3; ++i) vq[i] = *reinterpret_cast<const u4*>(vb + i * 1024 + voff);
+  vq[3] = *reinterpret_cast<const u4*>(vb + voff3);
+  __builtin_amdgcn_sched_barrier(0);
+  __builtin_amdgcn_s_barrier();                          // orders the issue: all V blocks ahead of all K
+  __builtin_amdgcn_sched_barrier(0);
+  u4 kreg[16];
+  auto issue_k = [&](const char* kb0, int i) {
+    kreg[i] = *reinterpret_cast<const u4*>(kb0 + (i >> 1) * 2048 + ((i & 1) ? koff_odd : koff_even));
+  };
+#pragma unroll
+  for (int i = 0; i < 8; ++i) issue_k(kbase, i);
+  __builtin_amdgcn_sched_barrier(0);
+
+  if (tid < 64) {
+    float clo = 0.0f, chi = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      clo = ((tid & 7) == i) ? vcb.c[i] : clo;
+      chi = ((tid >> 3) == i) ? vcb.c[i] : chi;
+    }
+    lut_s[tid] = pack_h2(clo, chi);
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) (&q_s[0][0])[tid + i * kMfmaThreads] = my_q[i];
+  __syncthreads();
+
+  u4 qreg[4];
+#pragma unroll
+  for (int kb = 0; kb < 4; ++kb) qreg[kb] = *reinterpret_cast<const u4*>(&q_s[n16][(4 * kb + g) * 4]);
+  const float cs = a.attn_scale * kLog2e;
+  uint32_t* stage = reinterpret_cast<uint32_t*>(big_s) + wave * 1024;   // this wave's 4 KB
+  u4* kst = reinterpret_cast<u4*>(stage);
+  const int w0 = (n16 == 15) ? 11 : (8 * n16) / 10;
+  const int s0 = (n16 == 15) ? 10 : (8 * n16) % 10;
+  const int sh_lo = 3 * s0, sh_hi = 30 - 3 * s0;
+  constexpr uint32_t kEven = 0x1C71C7u;
+
+  f4 accS[8];
+#pragma unroll
+  for (int et = 0; et < 8; ++et) accS[et] = f4{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, R_run = -INFINITY, l_run = 0.0f, inv_tscale = 1.0f;
+
+  for (int b = 0; b < n_blocks; ++b) {
+    const char* kb_cur = kbase + (int64_t)b * (kTilePos * kD * 2);
+    // ---- norms of the block (wave-local through LDS), power-of-two scale
+    nrm_s[wave][lane] = my_norm;
+    float vn[4][4];
+    float nmax = 0.0f;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const float4 n4 = *reinterpret_cast<const float4*>(&nrm_s[wave][16 * t + 4 * g]);
+      vn[t][0] = n4.x; vn[t][1] = n4.y; vn[t][2] = n4.z; vn[t][3] = n4.w;
+      nmax = fmaxf(nmax, fmaxf(fmaxf(n4.x, n4.y), fmaxf(n4.z, n4.w)));
+    }
+    nmax = fmaxf(nmax, shfl_xor_f(nmax, 16));
+    nmax = fmaxf(nmax, shfl_xor_f(nmax, 32));
+    int ex = (int)((__float_as_uint(nmax) >> 23) & 0xFF);
+    ex = ex < 27 ? (ex < 1 ? 127 : 27) : (ex > 227 ? 227 : ex);
+    const float kexp = (float)(127 - ex);
+    inv_tscale = __uint_as_float((uint32_t)ex << 23);
+
+    // ---- packed V -> table indices
+    {
+      u4* st4 = reinterpret_cast<u4*>(stage);
+#pragma unroll
+      for (int i = 0; i < 3; ++i) st4[i * 64 + lane] = vq[i];
+      if (lane < 16) st4[192 + lane] = vq[3];
+    }
+    uint32_t X[2][4], Y[2][4];
+#pragma unroll
+    for (int kb2 = 0; kb2 < 2; ++kb2)
+#pragma unroll
+      for (int qd = 0; qd < 4; ++qd) {
+        const int t = 2 * kb2 + (qd >> 1), jp = qd & 1;
+        const uint32_t* ra = stage + (16 * t + 4 * g + 2 * jp) * kPdim + w0;
+        const uint32_t fa = ((ra[0] >> sh_lo) | (ra[1] << sh_hi)) & 0xFFFFFFu;
+        const uint32_t fb = ((ra[kPdim] >> sh_lo) | (ra[kPdim + 1] << sh_hi)) & 0xFFFFFFu;
+        X[kb2][qd] = (fa & kEven) | ((fb & kEven) << 3);
+        Y[kb2][qd] = ((fa >> 3) & kEven) | (fb & (kEven << 3));
+      }
+    u4 breg[2][8];
+    auto lookups = [&](int kb2) {
+#pragma unroll
+      for (int et = 0; et < 8; ++et)
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) {
+          const uint32_t src = (et & 1) ? Y[kb2][qd] : X[kb2][qd];
+          breg[kb2][et][qd] = lut_s[(src >> (6 * (et >> 1))) & 63u];
+        }
+    };
+    float s[4][4];
+    auto qk_tile = [&](int t) {
+#pragma unroll
+      for (int ii = 0; ii < 4; ++ii) kst[ii * 64 + lane] = kreg[4 * t + ii];
+      f4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb) {
+        const u4 ka = kst[n16 * 16 + ((4 * kb + g) ^ (n16 & 7))];
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, ka), __builtin_bit_cast(h8, qreg[kb]),
+                                                     acc, 0, 0, 0);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) s[t][j] = acc[j];
+    };
+    __builtin_amdgcn_sched_barrier(0);
+    lookups(0);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 8; i < 12; ++i) issue_k(kb_cur, i);
+    __builtin_amdgcn_sched_barrier(0);
+    qk_tile(0);
+    __builtin_amdgcn_sched_barrier(0);
+    lookups(1);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 12; i < 16; ++i) issue_k(kb_cur, i);
+    __builtin_amdgcn_sched_barrier(0);
+    qk_tile(1);
+    qk_tile(2);
+    qk_tile(3);
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- norms and V block of the next block: in flight during the softmax and the value product of this one
+    if (b + 1 < n_blocks) {
+      my_norm = nb[(b + 1) * kTilePos];
+      const char* vbn = vb + (int64_t)(b + 1) * (kTilePos * kPdim * 4);
+#pragma unroll
+      for (int i = 0; i < 3; ++i) vq[i] = *reinterpret_cast<const u4*>(vbn + i * 1024 + voff);
+      vq[3] = *reinterpret_cast<const u4*>(vbn + voff3);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- online softmax over the wave's 64 positions of this block
+    float mb = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) mb = fmaxf(mb, s[t][j]);
+    mb = fmaxf(mb, shfl_xor_f(mb, 16));
+    mb = fmaxf(mb, shfl_xor_f(mb, 32));
+    const float m_new = fmaxf(m_run, mb * cs);            // log2 units; attn_scale > 0 (host check)
+    const float R_new = m_new - kexp;
+    const float factor = __builtin_amdgcn_exp2f(R_run - R_new);      // 0 on the first block
+    m_run = m_new;
+    R_run = R_new;
+    float lsum = 0.0f;
+    uint32_t pa[2][4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      float p[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        p[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][j], cs, -R_new));   // weight * 2^kexp
+        lsum += p[j];
+        p[j] *= vn[t][j];
+      }
+      pa[t >> 1][2 * (t & 1)] = pack_h2(p[0], p[1]);
+      pa[t >> 1][2 * (t & 1) + 1] = pack_h2(p[2], p[3]);
+    }
+    l_run = l_run * factor + lsum;                         // per-lane part; the four lanes of a head share `factor`
+    if (b > 0 && __any(factor != 1.0f)) {                  // accumulator rows are heads 4g + j: factors through LDS
+      if (g == 0) alpha_s[wave][n16] = factor;
+      const float4 a4 = *reinterpret_cast<const float4*>(&alpha_s[wave][4 * g]);
+      const float av[4] = {a4.x, a4.y, a4.z, a4.w};
+#pragma unroll
+      for (int et = 0; et < 8; ++et)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) accS[et][j] *= av[j];
+    }
+#pragma unroll
+    for (int kb2 = 0; kb2 < 2; ++kb2) {
+      const u4 A = {pa[kb2][0], pa[kb2][1], pa[kb2][2], pa[kb2][3]};
+#pragma unroll
+      for (int et = 0; et < 8; ++et)
+        accS[et] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, A), __builtin_bit_cast(h8, breg[kb2][et]),
+                                                          accS[et], 0, 0, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (b + 1 < n_blocks) {                                // first K instalment of the next block (operand registers are free now)
+      const char* kbn = kb_cur + kTilePos * kD * 2;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) issue_k(kbn, i);
+    }
+  }
+
+  // ---- merge the eight waves (as in vonly_tile_mfma_kernel): m is the running maximum, the weight sum
+  // and the accumulators carry 2^kexp of the last block
+  float l = l_run;
+  l += shfl_xor_f(l, 16);
+  l += shfl_xor_f(l, 32);
+  l *= inv_tscale;
+  const float m = m_run;
+  float (*S_all)[8][kD] = reinterpret_cast<float (*)[8][kD]>(big_s);
+  const int64_t grp = (int64_t)seq * a.n_kv + kvh;
+  float* pS = a.ws_S + (grp * a.n_tiles_max + tile) * (int64_t)(n_rep * kD);
+  float* pml = a.ws_ml + (grp * a.n_tiles_max + tile) * (int64_t)(n_rep * 2);
+  if (g == 0) {
+    m_s[wave][n16] = m;
+    l_s[wave][n16] = l;
+  }
+  __syncthreads();
+  if (tid < kWaves * kHeadsMax) {
+    const int w = tid >> 4, h = tid & 15;
+    float M = m_s[0][h];
+#pragma unroll
+    for (int ww = 1; ww < kWaves; ++ww) M = fmaxf(M, m_s[ww][h]);
+    f_s[w][h] = __builtin_amdgcn_exp2f(m_s[w][h] - M);
+    if (w == 0) M_s[h] = M;
+  }
+  __syncthreads();
+  const float4 f4own = *reinterpret_cast<const float4*>(&f_s[wave][4 * g]);
+  const float wscale = inv_tscale * a.v_unscale;
+  const float fown[4] = {f4own.x * wscale, f4own.y * wscale, f4own.z * wscale, f4own.w * wscale};
+  for (int h0 = 0; h0 < n_rep; h0 += 8) {
+    if (h0) __syncthreads();
+    if ((g >> 1) == (h0 >> 3)) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float4* dst = reinterpret_cast<float4*>(&S_all[wave][(4 * g + j) & 7][8 * n16]);
+        const float f = fown[j];
+        dst[0] = make_float4(accS[0][j] * f, accS[1][j] * f, accS[2][j] * f, accS[3][j] * f);
+        dst[1] = make_float4(accS[4][j] * f, accS[5][j] * f, accS[6][j] * f, accS[7][j] * f);
+      }
+    }
+    __syncthreads();
+    const int rows = min(8, n_rep - h0);
+    if (tid < rows * (kD / 4)) {
+      const int hl = tid >> 5, e4 = tid & 31;
+      float4 sum = *reinterpret_cast<const float4*>(&S_all[0][hl][4 * e4]);
+#pragma unroll
+      for (int w = 1; w < kWaves; ++w) {
+        const float4 x = *reinterpret_cast<const float4*>(&S_all[w][hl][4 * e4]);
+        sum.x += x.x; sum.y += x.y; sum.z += x.z; sum.w += x.w;
+      }
+      *reinterpret_cast<float4*>(pS + (h0 + hl) * kD + 4 * e4) = sum;
+    }
+  }
+  if (tid < n_rep) {
+    const int h = tid;
+    float L = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) L += f_s[w][h] * l_s[w][h];
+    pml[2 * h] = M_s[h];
+    pml[2 * h + 1] = L;
+  }
+}
+
 // Merge pass: grid = (n_q, n_seq), 256 threads.  Lane group ph = tid / 32 folds tiles ph, ph + 8, ...
 // (4 elements per lane) with a running maximum; the 8 groups are then combined through LDS and wave 0
 // finishes the row.  NORM = false (given weights, all maxima zero) skips the division by l.
@@ -454,7 +750,7 @@ template <typename TO, bool NORM>
 __global__ __launch_bounds__(kMergeThreads) void decode_merge_rows_kernel(
     const float* __restrict__ ws_S, const float* __restrict__ ws_ml, const int32_t* __restrict__ seq_offsets,
     int64_t seq_len, int n_tiles_max, int n_kv, int n_rep, const float* __restrict__ signs, float inv_dim,
-    TO* __restrict__ out) {
+    TO* __restrict__ out, int tile_pos) {
   __shared__ __align__(16) float acc_s[8][kD];
   __shared__ float ml_s[8][2];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -463,7 +759,7 @@ __global__ __launch_bounds__(kMergeThreads) void decode_merge_rows_kernel(
   const int kvh = head / n_rep, r = head - kvh * n_rep;
   int64_t len = seq_len;
   if (seq_offsets) len = (int64_t)seq_offsets[seq + 1] - seq_offsets[seq];
-  const int n_tiles = (int)((len + kTilePos - 1) / kTilePos);
+  const int n_tiles = (int)((len + tile_pos - 1) / tile_pos);
   const int64_t grp = (int64_t)seq * n_kv + kvh;
   const float* gS = ws_S + grp * n_tiles_max * (int64_t)(n_rep * kD) + r * kD + 4 * eq;
   const float* gml = ws_ml + grp * n_tiles_max * (int64_t)(n_rep * 2) + r * 2;
