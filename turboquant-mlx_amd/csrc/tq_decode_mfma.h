@@ -447,23 +447,26 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
   TQ_STAMP(10);
 }
 
-// Streaming variant for long unmasked caches: one workgroup runs through n_blocks CONSECUTIVE
-// 512-position blocks with an online softmax in registers (the flash recurrence: running maximum,
-// rescale of the accumulators when it moves), and only then merges its eight waves and stores
-// one partial.  The fixed work of a tile - address set-up, Q / table staging, cross-wave merge,
-// partial store, about 40 % of a wave's instructions - is paid once per n_blocks blocks, the loads
-// of block b+1 are in flight while block b is computed, and the merge pass folds n_blocks times
-// fewer partials.  With one block it would do exactly what vonly_tile_mfma_kernel<true> does.
+// Streaming variant for unmasked full tiles: one workgroup runs through n_blocks CONSECUTIVE
+// 512-position blocks; a wave walks its 64 rows of every block in STEPS of 32 positions with an
+// online softmax in registers (the flash recurrence: running maximum, rescale of the accumulators
+// when it moves).  Loads are double-buffered: the norm, packed-V and K loads of step s+1 are
+// issued in three instalments between the phases of step s, so memory streams while the ALUs and
+// matrix cores work, and the value product of the first 32 rows does not wait for the K rows of
+// the last 32.  The fixed work of a tile (address set-up, Q / table staging, cross-wave merge,
+// partial store) is paid once per workgroup.
 // The partial of a workgroup is taken relative to R = m - kexp (running maximum in log2 units minus
-// the exponent of the power-of-two norm scale of the block that set it): weights are
+// the exponent of the power-of-two norm scale of the step that set it): weights are
 // 2^(s*cs - R), and moving from R_old to R_new multiplies accumulators and weight sum by 2^(R_old - R_new).
 // grid = (seq_len / (512 * n_blocks), n_kv, n_seq), 512 threads.
+constexpr int kStepPos = 32;
+
 __global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
   __shared__ __align__(16) unsigned char big_s[32768];
   __shared__ uint32_t lut_s[64];
   __shared__ __align__(16) uint32_t q_s[kHeadsMax][kD / 2];
-  __shared__ __align__(16) float nrm_s[kWaves][kWavePos];
+  __shared__ __align__(16) float nrm_s[kWaves][kStepPos];
   __shared__ __align__(16) float alpha_s[kWaves][kHeadsMax];
   __shared__ float m_s[kWaves][kHeadsMax], l_s[kWaves][kHeadsMax], M_s[kHeadsMax];
   __shared__ __align__(16) float f_s[kWaves][kHeadsMax];
@@ -476,17 +479,32 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
   const int n_q = a.n_kv * n_rep;
   const int64_t q_row0 = (int64_t)seq * n_q + (int64_t)kvh * n_rep;
   const int64_t tile_p0 = (int64_t)tile * kTilePos * n_blocks;
-  const int wrow0 = wave * kWavePos;
+  const int n_steps = 2 * n_blocks;
 
-  // per-block strides: 512 rows of norms (4 B), packed V (52 B), K (256 B)
-  const float* nb = a.v_norms + (int64_t)seq * a.vn_seq_stride + (int64_t)kvh * a.vn_head_stride + tile_p0 + wrow0 + lane;
-  const char* vb = reinterpret_cast<const char*>(
-      a.v_packed + ((int64_t)seq * a.v_seq_stride + (int64_t)kvh * a.v_head_stride + tile_p0 + wrow0) * kPdim);
+  // row of step s inside the workgroup's range: block s/2, this wave's 64 rows, half s%2
+  auto step_row = [&](int s) { return (s >> 1) * kTilePos + wave * kWavePos + (s & 1) * kStepPos; };
+  const float* nbase = a.v_norms + (int64_t)seq * a.vn_seq_stride + (int64_t)kvh * a.vn_head_stride + tile_p0 + (lane & 31);
+  const char* vbase = reinterpret_cast<const char*>(
+      a.v_packed + ((int64_t)seq * a.v_seq_stride + (int64_t)kvh * a.v_head_stride + tile_p0) * kPdim);
   const char* kbase = reinterpret_cast<const char*>(
       a.k + ((int64_t)seq * a.k_seq_stride + (int64_t)kvh * a.k_head_stride + tile_p0) * kD);
-  const uint32_t voff = (uint32_t)(lane * 16), voff3 = (uint32_t)(3072 + (lane & 15) * 16);
-  const uint32_t koff_even = (uint32_t)(((wrow0 + (lane >> 4)) * 16 + ((lane & 15) ^ ((lane >> 4) & 7))) * 16);
-  const uint32_t koff_odd = (uint32_t)(((wrow0 + 4 + (lane >> 4)) * 16 + ((lane & 15) ^ ((4 + (lane >> 4)) & 7))) * 16);
+  const uint32_t voff0 = (uint32_t)(lane * 16), voff1 = (uint32_t)((lane < 40 ? 64 + lane : 103) * 16);   // 104 pieces
+  const uint32_t koff_even = (uint32_t)(((lane >> 4) * 16 + ((lane & 15) ^ ((lane >> 4) & 7))) * 16);
+  const uint32_t koff_odd = (uint32_t)(((4 + (lane >> 4)) * 16 + ((lane & 15) ^ ((4 + (lane >> 4)) & 7))) * 16);
+  auto issue_nv = [&](int s, float& nrm, u4 (&vqx)[2]) {
+    const int r = step_row(s);
+    nrm = nbase[r];
+    const char* vb = vbase + (int64_t)r * (kPdim * 4);
+    vqx[0] = *reinterpret_cast<const u4*>(vb + voff0);
+    vqx[1] = *reinterpret_cast<const u4*>(vb + voff1);
+  };
+  auto issue_k4 = [&](int s, u4 (&kx)[8], int part) {     // instructions 4*part .. 4*part+3: rows 16*part .. +15 of the step
+    const char* kb = kbase + (int64_t)step_row(s) * (kD * 2) + part * 4096;
+    kx[4 * part + 0] = *reinterpret_cast<const u4*>(kb + koff_even);
+    kx[4 * part + 1] = *reinterpret_cast<const u4*>(kb + koff_odd);
+    kx[4 * part + 2] = *reinterpret_cast<const u4*>(kb + 2048 + koff_even);
+    kx[4 * part + 3] = *reinterpret_cast<const u4*>(kb + 2048 + koff_odd);
+  };
 
   uint32_t my_q[2];
 #pragma unroll
@@ -494,20 +512,14 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
     const int w = tid + i * kMfmaThreads;
     my_q[i] = (w < n_rep * (kD / 2)) ? reinterpret_cast<const uint32_t*>(a.q + q_row0 * kD)[w] : 0u;
   }
-  float my_norm = nb[0];
-  u4 vq[4];
-#pragma unroll
-  for (int i = 0; i < 3; ++i) vq[i] = *reinterpret_cast<const u4*>(vb + i * 1024 + voff);
-  vq[3] = *reinterpret_cast<const u4*>(vb + voff3);
+  float nrmA, nrmB = 0.0f;
+  u4 vqA[2], vqB[2], kA[8], kB[8];
+  issue_nv(0, nrmA, vqA);
   __builtin_amdgcn_sched_barrier(0);
-  __builtin_amdgcn_s_barrier();                          // orders the issue: all V blocks ahead of all K
+  __builtin_amdgcn_s_barrier();                          // orders the issue: every wave's first V block ahead of all K
   __builtin_amdgcn_sched_barrier(0);
-  u4 kreg[16];
-  auto issue_k = [&](const char* kb0, int i) {
-    kreg[i] = *reinterpret_cast<const u4*>(kb0 + (i >> 1) * 2048 + ((i & 1) ? koff_odd : koff_even));
-  };
-#pragma unroll
-  for (int i = 0; i < 8; ++i) issue_k(kbase, i);
+  issue_k4(0, kA, 0);
+  issue_k4(0, kA, 1);
   __builtin_amdgcn_sched_barrier(0);
 
   if (tid < 64) {
@@ -539,14 +551,14 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
   for (int et = 0; et < 8; ++et) accS[et] = f4{0.f, 0.f, 0.f, 0.f};
   float m_run = -INFINITY, R_run = -INFINITY, l_run = 0.0f, inv_tscale = 1.0f;
 
-  for (int b = 0; b < n_blocks; ++b) {
-    const char* kb_cur = kbase + (int64_t)b * (kTilePos * kD * 2);
-    // ---- norms of the block (wave-local through LDS), power-of-two scale
-    nrm_s[wave][lane] = my_norm;
-    float vn[4][4];
+  // one step on the buffers (nrm, vqx, kx); `next(i)` issues instalment i (0: norm + V, 1 and 2: K) of the following step
+  auto step = [&](int sidx, float nrm, u4 (&vqx)[2], u4 (&kx)[8], auto&& next) {
+    // ---- norms (wave-local through LDS), power-of-two scale
+    if (lane < kStepPos) nrm_s[wave][lane] = nrm;
+    float vn[2][4];
     float nmax = 0.0f;
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
+    for (int t = 0; t < 2; ++t) {
       const float4 n4 = *reinterpret_cast<const float4*>(&nrm_s[wave][16 * t + 4 * g]);
       vn[t][0] = n4.x; vn[t][1] = n4.y; vn[t][2] = n4.z; vn[t][3] = n4.w;
       nmax = fmaxf(nmax, fmaxf(fmaxf(n4.x, n4.y), fmaxf(n4.z, n4.w)));
@@ -557,40 +569,42 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
     ex = ex < 27 ? (ex < 1 ? 127 : 27) : (ex > 227 ? 227 : ex);
     const float kexp = (float)(127 - ex);
     inv_tscale = __uint_as_float((uint32_t)ex << 23);
-
-    // ---- packed V -> table indices
+    // ---- packed V -> table indices -> centroid pairs
     {
       u4* st4 = reinterpret_cast<u4*>(stage);
-#pragma unroll
-      for (int i = 0; i < 3; ++i) st4[i * 64 + lane] = vq[i];
-      if (lane < 16) st4[192 + lane] = vq[3];
+      st4[lane] = vqx[0];
+      if (lane < 40) st4[64 + lane] = vqx[1];
     }
-    uint32_t X[2][4], Y[2][4];
+    __builtin_amdgcn_sched_barrier(0);
+    next(0);
+    __builtin_amdgcn_sched_barrier(0);
+    uint32_t X[4], Y[4];
 #pragma unroll
-    for (int kb2 = 0; kb2 < 2; ++kb2)
+    for (int qd = 0; qd < 4; ++qd) {
+      const int t = qd >> 1, jp = qd & 1;
+      const uint32_t* ra = stage + (16 * t + 4 * g + 2 * jp) * kPdim + w0;
+      const uint32_t fa = ((ra[0] >> sh_lo) | (ra[1] << sh_hi)) & 0xFFFFFFu;
+      const uint32_t fb = ((ra[kPdim] >> sh_lo) | (ra[kPdim + 1] << sh_hi)) & 0xFFFFFFu;
+      X[qd] = (fa & kEven) | ((fb & kEven) << 3);
+      Y[qd] = ((fa >> 3) & kEven) | (fb & (kEven << 3));
+    }
+    u4 breg[8];
+#pragma unroll
+    for (int et = 0; et < 8; ++et)
 #pragma unroll
       for (int qd = 0; qd < 4; ++qd) {
-        const int t = 2 * kb2 + (qd >> 1), jp = qd & 1;
-        const uint32_t* ra = stage + (16 * t + 4 * g + 2 * jp) * kPdim + w0;
-        const uint32_t fa = ((ra[0] >> sh_lo) | (ra[1] << sh_hi)) & 0xFFFFFFu;
-        const uint32_t fb = ((ra[kPdim] >> sh_lo) | (ra[kPdim + 1] << sh_hi)) & 0xFFFFFFu;
-        X[kb2][qd] = (fa & kEven) | ((fb & kEven) << 3);
-        Y[kb2][qd] = ((fa >> 3) & kEven) | (fb & (kEven << 3));
+        const uint32_t src = (et & 1) ? Y[qd] : X[qd];
+        breg[et][qd] = lut_s[(src >> (6 * (et >> 1))) & 63u];
       }
-    u4 breg[2][8];
-    auto lookups = [&](int kb2) {
+    __builtin_amdgcn_sched_barrier(0);
+    next(1);
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- scores of the 32 rows
+    float s[2][4];
 #pragma unroll
-      for (int et = 0; et < 8; ++et)
+    for (int t = 0; t < 2; ++t) {
 #pragma unroll
-        for (int qd = 0; qd < 4; ++qd) {
-          const uint32_t src = (et & 1) ? Y[kb2][qd] : X[kb2][qd];
-          breg[kb2][et][qd] = lut_s[(src >> (6 * (et >> 1))) & 63u];
-        }
-    };
-    float s[4][4];
-    auto qk_tile = [&](int t) {
-#pragma unroll
-      for (int ii = 0; ii < 4; ++ii) kst[ii * 64 + lane] = kreg[4 * t + ii];
+      for (int ii = 0; ii < 4; ++ii) kst[ii * 64 + lane] = kx[4 * t + ii];
       f4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int kb = 0; kb < 4; ++kb) {
@@ -600,51 +614,26 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
       }
 #pragma unroll
       for (int j = 0; j < 4; ++j) s[t][j] = acc[j];
-    };
-    __builtin_amdgcn_sched_barrier(0);
-    lookups(0);
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int i = 8; i < 12; ++i) issue_k(kb_cur, i);
-    __builtin_amdgcn_sched_barrier(0);
-    qk_tile(0);
-    __builtin_amdgcn_sched_barrier(0);
-    lookups(1);
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int i = 12; i < 16; ++i) issue_k(kb_cur, i);
-    __builtin_amdgcn_sched_barrier(0);
-    qk_tile(1);
-    qk_tile(2);
-    qk_tile(3);
-    __builtin_amdgcn_sched_barrier(0);
-    // ---- norms and V block of the next block: in flight during the softmax and the value product of this one
-    if (b + 1 < n_blocks) {
-      my_norm = nb[(b + 1) * kTilePos];
-      const char* vbn = vb + (int64_t)(b + 1) * (kTilePos * kPdim * 4);
-#pragma unroll
-      for (int i = 0; i < 3; ++i) vq[i] = *reinterpret_cast<const u4*>(vbn + i * 1024 + voff);
-      vq[3] = *reinterpret_cast<const u4*>(vbn + voff3);
+      if (t == 0) {
+        __builtin_amdgcn_sched_barrier(0);
+        next(2);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
-    __builtin_amdgcn_sched_barrier(0);
-
-    // ---- online softmax over the wave's 64 positions of this block
-    float mb = -INFINITY;
-#pragma unroll
-    for (int t = 0; t < 4; ++t)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) mb = fmaxf(mb, s[t][j]);
+    // ---- online softmax
+    float mb = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
+                     fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3])));
     mb = fmaxf(mb, shfl_xor_f(mb, 16));
     mb = fmaxf(mb, shfl_xor_f(mb, 32));
     const float m_new = fmaxf(m_run, mb * cs);            // log2 units; attn_scale > 0 (host check)
     const float R_new = m_new - kexp;
-    const float factor = __builtin_amdgcn_exp2f(R_run - R_new);      // 0 on the first block
+    const float factor = __builtin_amdgcn_exp2f(R_run - R_new);      // 0 on the first step
     m_run = m_new;
     R_run = R_new;
     float lsum = 0.0f;
-    uint32_t pa[2][4];
+    uint32_t pa[4];
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
+    for (int t = 0; t < 2; ++t) {
       float p[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
@@ -652,11 +641,11 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
         lsum += p[j];
         p[j] *= vn[t][j];
       }
-      pa[t >> 1][2 * (t & 1)] = pack_h2(p[0], p[1]);
-      pa[t >> 1][2 * (t & 1) + 1] = pack_h2(p[2], p[3]);
+      pa[2 * t] = pack_h2(p[0], p[1]);
+      pa[2 * t + 1] = pack_h2(p[2], p[3]);
     }
     l_run = l_run * factor + lsum;                         // per-lane part; the four lanes of a head share `factor`
-    if (b > 0 && __any(factor != 1.0f)) {                  // accumulator rows are heads 4g + j: factors through LDS
+    if (sidx > 0 && __any(factor != 1.0f)) {               // accumulator rows are heads 4g + j: factors through LDS
       if (g == 0) alpha_s[wave][n16] = factor;
       const float4 a4 = *reinterpret_cast<const float4*>(&alpha_s[wave][4 * g]);
       const float av[4] = {a4.x, a4.y, a4.z, a4.w};
@@ -665,24 +654,25 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) accS[et][j] *= av[j];
     }
+    const u4 A = {pa[0], pa[1], pa[2], pa[3]};
 #pragma unroll
-    for (int kb2 = 0; kb2 < 2; ++kb2) {
-      const u4 A = {pa[kb2][0], pa[kb2][1], pa[kb2][2], pa[kb2][3]};
-#pragma unroll
-      for (int et = 0; et < 8; ++et)
-        accS[et] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, A), __builtin_bit_cast(h8, breg[kb2][et]),
-                                                          accS[et], 0, 0, 0);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    if (b + 1 < n_blocks) {                                // first K instalment of the next block (operand registers are free now)
-      const char* kbn = kb_cur + kTilePos * kD * 2;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) issue_k(kbn, i);
-    }
+    for (int et = 0; et < 8; ++et)
+      accS[et] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, A), __builtin_bit_cast(h8, breg[et]),
+                                                        accS[et], 0, 0, 0);
+  };
+
+  for (int sidx = 0; sidx < n_steps; sidx += 2) {         // steps come in pairs: buffers A and B stay in fixed registers
+    step(sidx, nrmA, vqA, kA, [&](int i) {
+      if (i == 0) issue_nv(sidx + 1, nrmB, vqB); else issue_k4(sidx + 1, kB, i - 1);
+    });
+    const bool more = sidx + 2 < n_steps;                  // uniform
+    step(sidx + 1, nrmB, vqB, kB, [&](int i) {
+      if (more) { if (i == 0) issue_nv(sidx + 2, nrmA, vqA); else issue_k4(sidx + 2, kA, i - 1); }
+    });
   }
 
   // ---- merge the eight waves (as in vonly_tile_mfma_kernel): m is the running maximum, the weight sum
-  // and the accumulators carry 2^kexp of the last block
+  // and the accumulators carry 2^kexp of the last step
   float l = l_run;
   l += shfl_xor_f(l, 16);
   l += shfl_xor_f(l, 32);
