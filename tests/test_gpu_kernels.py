@@ -814,3 +814,157 @@ def test_vonly_decode_streaming_blocks(tq, n_seq, n_kv, n_rep, T, blocks):
         want = o.vonly_decode_attention(q[sidx], K[sidx], hp[sidx], hn[sidx], c, vs, D, bits, sc)
         close(got[sidx], want, row_scale=True)
     close(got.reshape(-1, D), ref32.reshape(-1, D), row_scale=True)   # every sequence against the float32 kernels
+
+
+# ------------------------------------------------------------------ seeded sweep over decode shapes
+
+def _draw_decode_case(seed):
+    """One decode-attention case drawn from the seed: head counts (including group sizes that do not
+    divide the 16-row matrix tile evenly), a ragged batch or a cache-layout batch, lengths from 1
+    to a few thousand (log-uniform, so tile boundaries, single positions and multi-tile sequences
+    all occur), an optional additive mask per sequence or per head, and the query dtype."""
+    rng = np.random.default_rng(1000 + seed)
+    n_kv = int(rng.choice([1, 2, 3, 4, 5, 8]))
+    n_rep = int(rng.choice([1, 2, 3, 4, 5, 7, 8, 12, 16]))
+    ragged = bool(rng.integers(0, 2))
+    n_seq = int(rng.integers(1, 5))
+    hi = 3000 if n_kv * n_rep <= 32 else 1200
+    lens = np.exp(rng.uniform(0.0, math.log(hi), size=n_seq)).astype(np.int64).clip(1, hi)
+    if not ragged:
+        lens[:] = lens[0]
+    mask_kind = ["none", "seq", "head"][int(rng.integers(0, 3))] if not ragged else "none"
+    qdt = [np.float16, np.float32][int(rng.integers(0, 2))]
+    return rng, n_kv, n_rep, ragged, n_seq, lens, mask_kind, qdt
+
+
+def _draw_mask(rng, kind, n_seq, n_q, T):
+    if kind == "none":
+        return None
+    shape = (n_seq, 1, T) if kind == "seq" else (n_seq, n_q, T)
+    m = np.where(rng.random(shape) < 0.3, -np.inf, 0.0).astype(F32)
+    m[..., int(rng.integers(0, T))] = 0.0          # no row fully masked
+    return m + (rng.standard_normal(shape) * 0.5).astype(F32) * np.isfinite(m)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_decode_sweep_vonly_and_flash(tq, seed):
+    """vonly_decode and flash_decode (both precisions) on shapes drawn from the seed, each sequence
+    checked against the oracle's single-sequence functions."""
+    rng, n_kv, n_rep, ragged, n_seq, lens, mask_kind, qdt = _draw_decode_case(seed)
+    D, bits, sc = 128, 3, 1 / math.sqrt(128)
+    n_q = n_kv * n_rep
+    print(f"seed {seed}: n_kv {n_kv} n_rep {n_rep} ragged {ragged} lens {lens.tolist()} mask {mask_kind} "
+          f"q {np.dtype(qdt).name}", flush=True)
+    q = rng.standard_normal((n_seq, n_q, D)).astype(qdt)
+    if ragged:
+        offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, n_kv, int(offs[-1]), D, bits)
+        kw = dict(seq_offsets=dev(offs), max_seq_len=int(lens.max()))
+        per_seq = [tuple(a[:, offs[i]:offs[i + 1]] for a in (K, kp, kn, vp, vn)) for i in range(n_seq)]
+        dK, dkp, dkn, dvp, dvn = (dev(a) for a in (K, kp, kn, vp, vn))
+        mask = None
+    else:
+        T = int(lens[0])
+        T_alloc = T + int(rng.integers(0, 70))
+        c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, n_seq * n_kv, T_alloc, D, bits)
+        K, kp, kn, vp, vn = (a.reshape(n_seq, n_kv, *a.shape[1:]) for a in (K, kp, kn, vp, vn))
+        kw = dict(seq_len=T)
+        per_seq = [tuple(a[i, :, :T] for a in (K, kp, kn, vp, vn)) for i in range(n_seq)]
+        dK, dkp, dkn, dvp, dvn = (dev(a) for a in (K, kp, kn, vp, vn))
+        mask = _draw_mask(rng, mask_kind, n_seq, n_q, T)
+        if mask is not None:
+            kw["mask"] = dev(mask)
+    q_rot = tq.prerotate_query(dev(q.reshape(-1, D)), dev(ks)).reshape(n_seq, n_q, D)
+    for precision in ("fp16", "fp32"):
+        gv = host(tq.vonly_decode(dev(q), dK, dvp, dvn, c, dev(vs), D, bits, sc, n_rep=n_rep,
+                                  precision=precision, **kw))
+        gf = host(tq.flash_decode(q_rot, dkp, dkn, dvp, dvn, c, c, dev(vs), D, bits, sc, n_rep=n_rep,
+                                  precision=precision, **kw))
+        for i in range(n_seq):
+            Ki, kpi, kni, vpi, vni = per_seq[i]
+            mi = None if mask is None else np.broadcast_to(mask[i], (n_q, mask.shape[-1]))
+            close(gv[i], o.vonly_decode_attention(q[i], Ki, vpi, vni, c, vs, D, bits, sc, mask=mi))
+            close(gf[i], o.turboquant_attention_single(q[i].astype(F32), kpi, kni, vpi, vni, c, ks, c, vs,
+                                                       D, bits, sc, mask=mi))
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_decode_sweep_scores_and_sparse_v(tq, seed):
+    """The two unfused kernels on drawn shapes: scores of packed K (float32 kernel held to float32
+    rounding, matrix-core kernel to 1e-3 of the row scale) and the thresholded V sum."""
+    rng, n_kv, n_rep, _, _, lens, _, _ = _draw_decode_case(100 + seed)
+    D, bits, T = 128, 3, int(lens[0])
+    n_q = n_kv * n_rep
+    print(f"seed {seed}: n_kv {n_kv} n_rep {n_rep} T {T}", flush=True)
+    c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, n_kv, T, D, bits)
+    q_rot = o.prerotate_query(rng.standard_normal((n_q, D)).astype(F32), ks)
+    want = o.prerot_fused_qk_scores(q_rot, kp, kn, c, D, bits, n_rep)
+    got32 = host(tq.prerot_fused_qk_scores(dev(q_rot), dev(kp), dev(kn), c, D, bits, n_rep))
+    close(got32, want, rel=1e-5, abs_=1e-5)
+    got16 = host(tq.prerot_fused_qk_scores(dev(q_rot), dev(kp), dev(kn), c, D, bits, n_rep, precision="fp16"))
+    close(got16, want, rel=1e-3, abs_=1e-3 * float(np.abs(want).max()))
+    w = rng.random((n_q, T)).astype(F32) ** 8
+    w /= w.sum(axis=-1, keepdims=True)
+    thr = float(rng.choice([0.0, 1e-5, 1e-3]))
+    wantv = o.sparse_v_matvec(w, vp, vn, c, vs, D, bits, threshold=thr, n_rep=n_rep)
+    for precision in ("fp32", "fp16"):
+        gotv = host(tq.sparse_v_matvec(dev(w), dev(vp), dev(vn), c, dev(vs), D, bits, threshold=thr,
+                                       n_rep=n_rep, precision=precision))
+        close(gotv, wantv)
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_prefill_sweep(tq, seed):
+    """Prefill attention on drawn shapes: chunk length, chunk position inside the cache (tail, middle,
+    start), cache allocation longer than the attended length, group size, causal or not."""
+    rng = np.random.default_rng(2000 + seed)
+    n_kv = int(rng.choice([1, 2, 3]))
+    n_rep = int(rng.choice([1, 2, 4, 7]))
+    kv_len = int(np.exp(rng.uniform(math.log(2), math.log(2600))))
+    n_rows = int(rng.integers(1, min(kv_len, 600) + 1))
+    causal = bool(rng.integers(0, 4))
+    where = int(rng.integers(0, 3))
+    pos0 = [kv_len - n_rows, int(rng.integers(0, kv_len - n_rows + 1)), 0][where]
+    T_alloc = kv_len + int(rng.integers(0, 100))
+    print(f"seed {seed}: n_kv {n_kv} n_rep {n_rep} kv_len {kv_len} alloc {T_alloc} rows {n_rows} pos0 {pos0} "
+          f"causal {causal}", flush=True)
+    c, ks, vs, kp, kn, vp, vn, q = _prefill_case(rng, n_kv, n_rep, T_alloc, n_rows)
+    sc = 1 / math.sqrt(128)
+    want = o.prefill_attention(q, kp[:, :kv_len], kn[:, :kv_len], vp[:, :kv_len], vn[:, :kv_len], c, c, ks, vs,
+                               128, 3, sc, pos0, n_rep, causal=causal)
+    got = tq.prefill_attention(dev(q), dev(kp), dev(kn), dev(vp), dev(vn), c, c, dev(ks), dev(vs), 128, 3, sc,
+                               n_rep=n_rep, kv_len=kv_len, q_pos0=pos0, causal=causal, out_dtype=torch.float32)
+    close(host(got).reshape(-1, 128), want.reshape(-1, 128), row_scale=True)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_encode_sweep(tq, seed):
+    """encode_into / dequant_into on drawn group layouts (row counts that do and do not meet the
+    streaming kernel's 16-row granularity, strides, offsets) and input scales: bit-exact."""
+    rng = np.random.default_rng(3000 + seed)
+    c, b = tables(3)
+    s = o.random_diagonal_sign(128, 42 + seed)
+    G = int(rng.integers(1, 6))
+    R = int(rng.choice([1, 5, 16, 17, 48, 64, 250, 1024]))
+    off = int(rng.integers(0, 40))
+    alloc = off + R + int(rng.integers(0, 40))
+    dt = [np.float16, np.float32][int(rng.integers(0, 2))]
+    variant = ["mlx", "metal"][int(rng.integers(0, 2))]
+    print(f"seed {seed}: G {G} R {R} off {off} alloc {alloc} {np.dtype(dt).name} {variant}", flush=True)
+    x = (rng.standard_normal((G, R, 128)) * np.exp(rng.uniform(-6, 6, size=(G, R, 1)))).astype(dt)
+    packed = torch.zeros((G, alloc, 13), dtype=torch.int32, device="cuda").view(torch.uint32)
+    norms = torch.zeros((G, alloc), dtype=torch.float32, device="cuda")
+    tq.encode_into(dev(x), dev(s), b, packed, norms, n_groups=G, rows_per_group=R, packed_group_stride=alloc,
+                   norms_group_stride=alloc, dim=128, bits=3, packed_row_offset=off, norms_row_offset=off,
+                   variant=variant)
+    wp, wn = o.fused_quantize(x.reshape(-1, 128), s, b, 128, 3, variant)
+    hp, hn = host(packed), host(norms)
+    assert np.array_equal(hp[:, off:off + R], wp.reshape(G, R, 13))
+    assert np.array_equal(hn[:, off:off + R], wn.reshape(G, R))
+    assert (hp[:, :off] == 0).all() and (hp[:, off + R:] == 0).all()
+    out = torch.zeros((G, alloc, 128), dtype=torch.float16, device="cuda")
+    tq.dequant_into(packed, norms, c, dev(s), out, n_groups=G, rows_per_group=R, packed_group_stride=alloc,
+                    norms_group_stride=alloc, out_group_stride=alloc, dim=128, bits=3, packed_row_offset=off,
+                    norms_row_offset=off, out_row_offset=off)
+    want = torch.from_numpy(o.packed_dequantize(wp, wn, c, s, 128, 3)).to(torch.float16).reshape(G, R, 128)
+    assert torch.equal(out[:, off:off + R].cpu(), want)
