@@ -213,6 +213,15 @@ int tq_flash_decode(const float* q_rot,
                     const tq_decode_shape* shape /* host */, tq_stream_t stream);
 
 /*
+ * Which tile pass tq_flash_decode takes on the matrix-core path for a batch of this shape:
+ * 0 = one workgroup per 512-position tile; n >= 2 = the streaming pass, one workgroup per
+ * n * 256 consecutive positions (large unmasked batches).  Informational: lets a caller or a test
+ * know which kernel a shape exercises.  No counterpart in the reference (one kernel per call,
+ * flash_attention.py:168-274).
+ */
+int tq_flash_decode_plan(int n_seq, int n_kv_heads, int64_t max_seq_len, int ragged, int masked);
+
+/*
  * Decode attention for a V-only cache: fp16 keys, packed values, dense softmax (threshold 0):
  *   out = butterfly(sum_p softmax_p(<q,K_p>*attn_scale + mask) * v_norm * c_v[idx_v]) * v_signs / dim.
  * The composition dense-K scores -> softmax -> sparse_v_matvec of hybrid_attention.py:52-88 /

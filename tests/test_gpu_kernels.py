@@ -968,3 +968,68 @@ def test_encode_sweep(tq, seed):
                     norms_row_offset=off, out_row_offset=off)
     want = torch.from_numpy(o.packed_dequantize(wp, wn, c, s, 128, 3)).to(torch.float16).reshape(G, R, 128)
     assert torch.equal(out[:, off:off + R].cpu(), want)
+
+
+# ------------------------------------------------------------------ streaming flash pass
+
+def _flash_plan(tq, n_seq, n_kv, max_len, ragged, masked=False):
+    from tqhip import _lib
+    return _lib.load().tq_flash_decode_plan(n_seq, n_kv, max_len, int(ragged), int(masked))
+
+
+def test_flash_streaming_pass_ragged(tq):
+    """A ragged batch large enough for the streaming pass (several 256-position steps per workgroup):
+    sequences start at arbitrary rows (every misalignment of the 52-byte rows against 16 bytes),
+    lengths end inside a step, inside a wave's 64 rows and one row past a step."""
+    rng = np.random.default_rng(61)
+    n_kv, n_rep, D, bits = 8, 4, 128, 3
+    lens = np.array([4097, 2561, 1025, 7000, 1, 3333, 5121, 6143])
+    n_seq = len(lens)
+    assert _flash_plan(tq, n_seq, n_kv, int(lens.max()), True) >= 2
+    offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    assert len({int(o) % 4 for o in offs[:-1]}) == 4          # all four row misalignments occur
+    c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, n_kv, int(offs[-1]), D, bits)
+    q = rng.standard_normal((n_seq, n_kv * n_rep, D)).astype(F32)
+    sc = 1 / math.sqrt(D)
+    q_rot = tq.prerotate_query(dev(q.reshape(-1, D)), dev(ks)).reshape(n_seq, n_kv * n_rep, D)
+    got = host(tq.flash_decode(q_rot, dev(kp), dev(kn), dev(vp), dev(vn), c, c, dev(vs), D, bits, sc, n_rep=n_rep,
+                               seq_offsets=dev(offs), max_seq_len=int(lens.max())))
+    for i in range(n_seq):
+        a, e = offs[i], offs[i + 1]
+        want = o.flash_attention_turboquant(o.prerotate_query(q[i], ks), kp[:, a:e], kn[:, a:e], vp[:, a:e],
+                                            vn[:, a:e], c, c, vs, D, bits, sc, 16, n_rep)
+        close(got[i], want)
+
+
+@pytest.mark.parametrize("n_seq,n_kv,n_rep,T,outliers", [(2, 8, 2, 16500, False), (1, 4, 7, 70000, False),
+                                                          (3, 8, 1, 12289, True)])
+def test_flash_streaming_pass_cache_layout(tq, n_seq, n_kv, n_rep, T, outliers):
+    """Cache layout [n_seq, n_kv, T_alloc, *] with a valid length that is not a multiple of anything;
+    value norms spread over six decades so that the running power-of-two scale moves between steps."""
+    rng = np.random.default_rng(62)
+    D, bits, T_alloc = 128, 3, T + 37
+    assert _flash_plan(tq, n_seq, n_kv, T, False) >= 2
+    c, b = tables(bits)
+    ks, vs = o.random_diagonal_sign(D, 42), o.random_diagonal_sign(D, 43)
+    kp = o.pack_indices(rng.integers(0, 8, size=(n_seq, n_kv, T_alloc, D)).astype(np.uint8), bits)
+    vp = o.pack_indices(rng.integers(0, 8, size=(n_seq, n_kv, T_alloc, D)).astype(np.uint8), bits)
+    kn = (rng.random((n_seq, n_kv, T_alloc)) * 12 + 6).astype(F32)
+    vn = (rng.random((n_seq, n_kv, T_alloc)) + 0.5).astype(F32)
+    if outliers:
+        vn *= np.exp(rng.uniform(-7, 7, size=vn.shape)).astype(F32)
+    q = rng.standard_normal((n_seq, n_kv * n_rep, D)).astype(F32)
+    sc = 1 / math.sqrt(D)
+    q_rot = tq.prerotate_query(dev(q.reshape(-1, D)), dev(ks)).reshape(n_seq, -1, D)
+    got = host(tq.flash_decode(q_rot, dev(kp), dev(kn), dev(vp), dev(vn), c, c, dev(vs), D, bits, sc,
+                               n_rep=n_rep, seq_len=T))
+    for i in range(n_seq):
+        want = o.turboquant_attention_single(q[i], kp[i, :, :T], kn[i, :, :T], vp[i, :, :T], vn[i, :, :T],
+                                             c, ks, c, vs, D, bits, sc)
+        close(got[i], want, row_scale=outliers)
+
+
+def test_flash_plan_masked_and_small_batches_take_the_tile_pass(tq):
+    assert _flash_plan(tq, 1, 4, 4096, False) == 0
+    assert _flash_plan(tq, 16, 8, 32768, True, masked=True) == 0
+    assert _flash_plan(tq, 16, 8, 32768, True) == 4
+    assert _flash_plan(tq, 1, 8, 131072, False) == 8

@@ -594,6 +594,17 @@ int launch_vonly_mfma(const void* q, const void* k_f16, const uint32_t* v_packed
   return TQ_OK;
 }
 
+// Steps of 256 positions that one workgroup of the streaming flash pass runs through, or 0 for the
+// single-tile pass.  The streaming pass wants at least two workgroups per CU (512 on this part) so
+// that the set-up of one overlaps the arithmetic of another: the largest step count up to 8 that
+// leaves that many; ragged batches (true lengths unknown on the host, max_seq_len is an upper bound)
+// stop at 4, which keeps the tail of the launch short.
+int flash_stream_steps(int n_seq, int n_kv, int64_t max_seq_len, bool ragged) {
+  const int64_t units = (int64_t)n_seq * n_kv * ((max_seq_len + tqm::kSStepPos - 1) / tqm::kSStepPos);
+  int n = (int)std::min<int64_t>(ragged ? 4 : 8, units / 512);
+  return n >= 2 ? n : 0;
+}
+
 // Matrix-core path over packed keys/values: MODE = tqm::kFlash (tq_flash_decode) or tqm::kWeights
 // (tq_sparse_v_matvec): tile pass + merge pass.
 template <int MODE>
@@ -627,14 +638,25 @@ int launch_packed_mfma(const float* q_rot_or_weights, const uint32_t* k_packed, 
   fill_codebook(kcb, nullptr, sh.bits);
   if (MODE != tqm::kWeights) a.score_scale *= tq::fill_codebook_fp16(kcb, k_centroids, sh.bits);
   a.v_unscale = tq::fill_codebook_fp16(vcb, v_centroids, sh.bits);
-  dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
-  tqm::packed_tile_mfma_kernel<MODE><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, kcb, vcb);
+  int tile_pos = tqm::kTilePos;
+  const int n_steps = (MODE == tqm::kFlash && !sh.mask)
+                          ? flash_stream_steps(sh.n_seq, sh.n_kv_heads, sh.seq_len, sh.seq_offsets != nullptr) : 0;
+  if (n_steps >= 2) {
+    tile_pos = tqm::kSStepPos * n_steps;
+    a.n_tiles_max = (int)((sh.seq_len + tile_pos - 1) / tile_pos);
+    dim3 grid(a.n_tiles_max, sh.n_kv_heads, sh.n_seq);
+    tqm::packed_stream_kernel<<<grid, tqm::kSThreads, 0, stream>>>(a, kcb, vcb, n_steps);
+  } else {
+    dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
+    tqm::packed_tile_mfma_kernel<MODE><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, kcb, vcb);
+  }
   TQ_CHECK_LAUNCH(who);
   dim3 mgrid(n_q, sh.n_seq);
   const float inv_dim = 1.0f / (float)sh.dim;
+  const int n_parts = a.n_tiles_max;
 #define LAUNCH_MERGE_P(TO)                                                                                    \
   tqm::decode_merge_rows_kernel<TO, MODE == tqm::kFlash><<<mgrid, tqm::kMergeThreads, 0, stream>>>(            \
-      a.ws_S, a.ws_ml, sh.seq_offsets, sh.seq_len, n_tiles, sh.n_kv_heads, sh.n_rep, v_signs, inv_dim, (TO*)out, tqm::kTilePos)
+      a.ws_S, a.ws_ml, sh.seq_offsets, sh.seq_len, n_parts, sh.n_kv_heads, sh.n_rep, v_signs, inv_dim, (TO*)out, tile_pos)
   if (sh.out_dtype == TQ_F16) { LAUNCH_MERGE_P(__half); }
   else if (sh.out_dtype == TQ_BF16) { LAUNCH_MERGE_P(__hip_bfloat16); }
   else { LAUNCH_MERGE_P(float); }
@@ -770,6 +792,11 @@ extern "C" int tq_sparse_v_matvec(const float* weights, const uint32_t* v_packed
   return launch_decode<kWeights>(weights, TQ_F32, nullptr, nullptr, nullptr, v_packed, v_norms, nullptr,
                                  centroids, signs, out, workspace, workspace_bytes, sh, thr,
                                  (hipStream_t)stream_, "tq_sparse_v_matvec");
+}
+
+extern "C" int tq_flash_decode_plan(int n_seq, int n_kv_heads, int64_t max_seq_len, int ragged, int masked) {
+  if (n_seq < 1 || n_kv_heads < 1 || max_seq_len < 0) return 0;
+  return masked ? 0 : flash_stream_steps(n_seq, n_kv_heads, max_seq_len, ragged != 0);
 }
 
 extern "C" int tq_flash_decode(const float* q_rot, const uint32_t* k_packed, const float* k_norms,

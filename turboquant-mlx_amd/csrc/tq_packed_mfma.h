@@ -91,7 +91,7 @@ __device__ __forceinline__ void piece_bits(int pc, int& w0, int& sh_lo, int& sh_
 }
 
 __device__ __forceinline__ void fill_lut(uint32_t* lut, const Codebook& cb, int tid) {
-  if (tid < 64) {
+  if ((unsigned)tid < 64u) {
     float clo = 0.0f, chi = 0.0f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -390,6 +390,320 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
     float L = 0.0f;
 #pragma unroll
     for (int w = 0; w < kWaves; ++w) L += f_s[w][h] * l_s[w][h];
+    pml[2 * h] = M_s[h];
+    pml[2 * h + 1] = L;
+  }
+}
+
+// Streaming flash-decode pass (packed K and V, no mask): a workgroup of FOUR waves runs through
+// n_steps consecutive 256-position steps of one (sequence, kv head), a wave 64 positions per step,
+// with the online-softmax recurrence in registers, and writes one partial at the end.  Two such
+// workgroups share a CU, so the set-up and the cross-wave merge of one overlap the arithmetic of
+// the other; the packed rows and norms of step s+1 are fetched into registers before step s is
+// computed.  The fixed work of a tile (query staging, tables, merge, partial store) is paid once
+// per n_steps * 256 positions and the merge pass sees that many fewer partials.
+//
+// Loads: a wave's 64 rows of 52 bytes start at an arbitrary multiple of 4 bytes (ragged batches
+// start a sequence at any row).  They are fetched as ALIGNED 16-byte pieces from the 16-byte
+// boundary at or below the first row (at most 209 pieces) into the wave's LDS image, and rows are
+// read from the image at the misalignment offset.  An aligned 16-byte piece never crosses a page,
+// so a piece that holds at least one valid byte is readable in full; pieces with no valid byte
+// (rows past the end of the sequence) are not fetched and read as zero, and their positions get
+// -inf scores.
+constexpr int kSWaves = 4;
+constexpr int kSThreads = kSWaves * 64;
+constexpr int kSStepPos = kSWaves * kWavePos;     // 256 positions per workgroup step
+constexpr int kSImageBytes = 4096;                // 209 pieces of 16 bytes, rounded up
+
+__global__ __launch_bounds__(kSThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps) {
+  __shared__ __align__(16) unsigned char big_s[kSWaves * 2 * kSImageBytes];   // per wave: K image, V image; later S_all[4][8][128]
+  __shared__ uint32_t lutk_s[64], lutv_s[64];
+  __shared__ __align__(16) uint32_t q_s[kHeadsMax][kD / 2];
+  __shared__ __align__(16) uint32_t ql_s[kHeadsMax][kD / 2];
+  __shared__ __align__(16) float kn_s[kSWaves][kWavePos], vn_s[kSWaves][kWavePos];
+  __shared__ __align__(16) float alpha_s[kSWaves][kHeadsMax];
+  __shared__ float m_s[kSWaves][kHeadsMax], l_s[kSWaves][kHeadsMax], M_s[kHeadsMax];
+  __shared__ __align__(16) float f_s[kSWaves][kHeadsMax];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int n16 = lane & 15, g = lane >> 4;
+  const int wg = blockIdx.x, kvh = blockIdx.y, seq = blockIdx.z;
+  const int n_rep = a.n_rep;
+  const int n_q = a.n_kv * n_rep;
+  const int64_t q_row0 = (int64_t)seq * n_q + (int64_t)kvh * n_rep;
+
+  int64_t first = 0, len = a.seq_len;
+  if (a.seq_offsets) {
+    first = a.seq_offsets[seq];
+    len = (int64_t)a.seq_offsets[seq + 1] - first;
+  }
+  const int64_t wg_p0 = (int64_t)wg * kSStepPos * n_steps;
+  if (wg_p0 >= len) return;
+
+  // ---- addresses: row 0 of the sequence for this kv head, misalignment of the wave's blocks
+  const char* krow0 = reinterpret_cast<const char*>(
+      a.k_packed + ((int64_t)seq * a.k_seq_stride + (int64_t)kvh * a.k_head_stride + first) * kPdim);
+  const char* vrow0 = reinterpret_cast<const char*>(
+      a.v_packed + ((int64_t)seq * a.v_seq_stride + (int64_t)kvh * a.v_head_stride + first) * kPdim);
+  // every block of this workgroup starts a multiple of 64 rows = 208 pieces after row wg_p0: one misalignment
+  const int kmis = (int)((reinterpret_cast<uintptr_t>(krow0) + (uint64_t)wg_p0 * (kPdim * 4)) & 15);
+  const int vmis = (int)((reinterpret_cast<uintptr_t>(vrow0) + (uint64_t)wg_p0 * (kPdim * 4)) & 15);
+  const float* knrow0 = a.k_norms + (int64_t)seq * a.kn_seq_stride + (int64_t)kvh * a.kn_head_stride + first;
+  const float* vnrow0 = a.v_norms + (int64_t)seq * a.vn_seq_stride + (int64_t)kvh * a.vn_head_stride + first;
+
+  auto rows_left_of = [&](int s) {
+    const int64_t p0w = wg_p0 + (int64_t)s * kSStepPos + wave * kWavePos;
+    const int64_t left = len - p0w;
+    return (int)(left < 0 ? 0 : (left > kWavePos ? kWavePos : left));
+  };
+  auto issue = [&](int s, u4 (&kq)[4], u4 (&vq)[4], float& kn, float& vn) {
+    const int64_t p0w = wg_p0 + (int64_t)s * kSStepPos + wave * kWavePos;
+    const int rows = rows_left_of(s);
+    const int kbytes = rows ? kmis + rows * (kPdim * 4) : 0;
+    const int vbytes = rows ? vmis + rows * (kPdim * 4) : 0;
+    const char* kb = krow0 + p0w * (kPdim * 4) - kmis;
+    const char* vb = vrow0 + p0w * (kPdim * 4) - vmis;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int off = (i * 64 + lane) * 16;
+      kq[i] = (off < kbytes) ? *reinterpret_cast<const u4*>(kb + off) : u4{0u, 0u, 0u, 0u};
+      vq[i] = (off < vbytes) ? *reinterpret_cast<const u4*>(vb + off) : u4{0u, 0u, 0u, 0u};
+    }
+    kn = (lane < rows) ? knrow0[p0w + lane] : 0.0f;
+    vn = (lane < rows) ? vnrow0[p0w + lane] : 0.0f;
+  };
+
+  float2 my_q[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int w = tid + i * kSThreads;                                  // word = 2 consecutive elements
+    my_q[i] = (w < n_rep * (kD / 2)) ? reinterpret_cast<const float2*>(a.q_rot + q_row0 * kD)[w] : make_float2(0.f, 0.f);
+  }
+  u4 kqA[4], vqA[4], kqB[4], vqB[4];
+  float knA, vnA, knB = 0.0f, vnB = 0.0f;
+  issue(0, kqA, vqA, knA, vnA);
+
+  fill_lut(lutk_s, kcb, tid);
+  fill_lut(lutv_s, vcb, tid - 64);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const __half2 h = __floats2half2_rn(my_q[i].x, my_q[i].y);
+    const float2 back = __half22float2(h);
+    (&q_s[0][0])[tid + i * kSThreads] = *reinterpret_cast<const uint32_t*>(&h);
+    (&ql_s[0][0])[tid + i * kSThreads] = pack_h2(my_q[i].x - back.x, my_q[i].y - back.y);
+  }
+  __syncthreads();
+
+  u4 qreg[4], qlow[4];
+#pragma unroll
+  for (int kb = 0; kb < 4; ++kb) {
+    qreg[kb] = *reinterpret_cast<const u4*>(&q_s[n16][(4 * kb + g) * 4]);
+    qlow[kb] = *reinterpret_cast<const u4*>(&ql_s[n16][(4 * kb + g) * 4]);
+  }
+  unsigned char* image = big_s + wave * (2 * kSImageBytes);
+  const uint32_t* kimg = reinterpret_cast<const uint32_t*>(image + kmis);
+  const uint32_t* vimg = reinterpret_cast<const uint32_t*>(image + kSImageBytes + vmis);
+  int kw0[4], ksl[4], ksh[4];
+#pragma unroll
+  for (int kb = 0; kb < 4; ++kb) piece_bits(4 * kb + g, kw0[kb], ksl[kb], ksh[kb]);
+  int vw0, vsl, vsh;
+  piece_bits(n16, vw0, vsl, vsh);
+  constexpr uint32_t kEven = 0x1C71C7u;
+  const float kscale = a.score_scale * kLog2e;           // scores in log2 units
+
+  f4 accS[8];
+#pragma unroll
+  for (int et = 0; et < 8; ++et) accS[et] = f4{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, R_run = -INFINITY, l_run = 0.0f, inv_tscale = 1.0f;
+
+  // one step on the buffers (kq, vq, kn, vn); `next()` issues the loads of the following step
+  auto step = [&](int sidx, u4 (&kq)[4], u4 (&vq)[4], float kn, float vn_, auto&& next) {
+    const int rows = rows_left_of(sidx);                 // uniform over the wave
+    if (rows <= 0) return;                               // steps only run out at the end: nothing follows
+    // ---- images and norms into the wave's LDS area
+    {
+      u4* k4 = reinterpret_cast<u4*>(image);
+      u4* v4 = reinterpret_cast<u4*>(image + kSImageBytes);
+#pragma unroll
+      for (int i = 0; i < 3; ++i) { k4[i * 64 + lane] = kq[i]; v4[i * 64 + lane] = vq[i]; }
+      if (lane < 17) { k4[192 + lane] = kq[3]; v4[192 + lane] = vq[3]; }
+      kn_s[wave][lane] = kn * kscale;
+      vn_s[wave][lane] = vn_;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    next();
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- scores of the 64 rows (log2 units)
+    float s[4][4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      f4 acc = {0.f, 0.f, 0.f, 0.f};
+      const uint32_t* krow = kimg + (16 * t + n16) * kPdim;
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb) {
+        const uint32_t f = ((krow[kw0[kb]] >> ksl[kb]) | (krow[kw0[kb] + 1] << ksh[kb])) & 0xFFFFFFu;
+        u4 ka;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) ka[k] = lutk_s[(f >> (6 * k)) & 63u];
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, ka), __builtin_bit_cast(h8, qreg[kb]),
+                                                     acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, ka), __builtin_bit_cast(h8, qlow[kb]),
+                                                     acc, 0, 0, 0);
+      }
+      const float4 kn4 = *reinterpret_cast<const float4*>(&kn_s[wave][16 * t + 4 * g]);
+      const float knv[4] = {kn4.x, kn4.y, kn4.z, kn4.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) s[t][j] = (16 * t + 4 * g + j < rows) ? acc[j] * knv[j] : -INFINITY;
+    }
+    // ---- value norms, their power-of-two scale
+    float vn[4][4];
+    float nmax = 0.0f;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const float4 n4 = *reinterpret_cast<const float4*>(&vn_s[wave][16 * t + 4 * g]);
+      vn[t][0] = n4.x; vn[t][1] = n4.y; vn[t][2] = n4.z; vn[t][3] = n4.w;
+      nmax = fmaxf(nmax, fmaxf(fmaxf(n4.x, n4.y), fmaxf(n4.z, n4.w)));
+    }
+    nmax = fmaxf(nmax, shfl_xor_f(nmax, 16));
+    nmax = fmaxf(nmax, shfl_xor_f(nmax, 32));
+    int ex = (int)((__float_as_uint(nmax) >> 23) & 0xFF);
+    ex = ex < 27 ? (ex < 1 ? 127 : 27) : (ex > 227 ? 227 : ex);
+    const float kexp = (float)(127 - ex);
+    inv_tscale = __uint_as_float((uint32_t)ex << 23);
+    // ---- online softmax: rows >= 1, so the maximum of the step is finite
+    float mb = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) mb = fmaxf(mb, s[t][j]);
+    mb = fmaxf(mb, shfl_xor_f(mb, 16));
+    mb = fmaxf(mb, shfl_xor_f(mb, 32));
+    const float m_new = fmaxf(m_run, mb);
+    const float R_new = m_new - kexp;
+    const float factor = __builtin_amdgcn_exp2f(R_run - R_new);      // 0 on the wave's first step
+    m_run = m_new;
+    R_run = R_new;
+    float lsum = 0.0f;
+    uint32_t pa[2][4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      float p[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        p[j] = __builtin_amdgcn_exp2f(s[t][j] - R_new);              // weight * 2^kexp
+        lsum += p[j];
+        p[j] *= vn[t][j];
+      }
+      pa[t >> 1][2 * (t & 1)] = pack_h2(p[0], p[1]);
+      pa[t >> 1][2 * (t & 1) + 1] = pack_h2(p[2], p[3]);
+    }
+    l_run = l_run * factor + lsum;
+    if (sidx > 0 && __any(factor != 1.0f)) {               // accumulator rows are heads 4g + j: factors through LDS
+      if (g == 0) alpha_s[wave][n16] = factor;
+      const float4 a4 = *reinterpret_cast<const float4*>(&alpha_s[wave][4 * g]);
+      const float av[4] = {a4.x, a4.y, a4.z, a4.w};
+#pragma unroll
+      for (int et = 0; et < 8; ++et)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) accS[et][j] *= av[j];
+    }
+    // ---- values: packed V -> interleaved table indices -> centroid pairs, 32 positions at a time
+#pragma unroll
+    for (int kb2 = 0; kb2 < 2; ++kb2) {
+      uint32_t X[4], Y[4];
+#pragma unroll
+      for (int qd = 0; qd < 4; ++qd) {
+        const int t = 2 * kb2 + (qd >> 1), jp = qd & 1;
+        const uint32_t* ra = vimg + (16 * t + 4 * g + 2 * jp) * kPdim + vw0;
+        const uint32_t fa = ((ra[0] >> vsl) | (ra[1] << vsh)) & 0xFFFFFFu;
+        const uint32_t fb = ((ra[kPdim] >> vsl) | (ra[kPdim + 1] << vsh)) & 0xFFFFFFu;
+        X[qd] = (fa & kEven) | ((fb & kEven) << 3);
+        Y[qd] = ((fa >> 3) & kEven) | (fb & (kEven << 3));
+      }
+      const u4 A = {pa[kb2][0], pa[kb2][1], pa[kb2][2], pa[kb2][3]};
+#pragma unroll
+      for (int et = 0; et < 8; ++et) {
+        u4 B;
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) {
+          const uint32_t src = (et & 1) ? Y[qd] : X[qd];
+          B[qd] = lutv_s[(src >> (6 * (et >> 1))) & 63u];
+        }
+        accS[et] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, A), __builtin_bit_cast(h8, B),
+                                                          accS[et], 0, 0, 0);
+      }
+    }
+  };
+
+  for (int sidx = 0; sidx < n_steps; sidx += 2) {          // steps come in pairs: buffers A and B stay in fixed registers
+    step(sidx, kqA, vqA, knA, vnA, [&]() {
+      if (sidx + 1 < n_steps) issue(sidx + 1, kqB, vqB, knB, vnB);
+    });
+    if (sidx + 1 < n_steps)
+      step(sidx + 1, kqB, vqB, knB, vnB, [&]() {
+        if (sidx + 2 < n_steps) issue(sidx + 2, kqA, vqA, knA, vnA);
+      });
+  }
+
+  // ---- merge the four waves: one factor per (wave, head), scaled deposits, float4 sum.  A wave that saw
+  // no valid row has m = -inf, l = 0 and zero accumulators.
+  float l = l_run;
+  l += shfl_xor_f(l, 16);
+  l += shfl_xor_f(l, 32);
+  l *= inv_tscale;
+  float (*S_all)[8][kD] = reinterpret_cast<float (*)[8][kD]>(big_s);
+  const int64_t grp = (int64_t)seq * a.n_kv + kvh;
+  float* pS = a.ws_S + (grp * a.n_tiles_max + wg) * (int64_t)(n_rep * kD);
+  float* pml = a.ws_ml + (grp * a.n_tiles_max + wg) * (int64_t)(n_rep * 2);
+  if (g == 0) {
+    m_s[wave][n16] = m_run;
+    l_s[wave][n16] = l;
+  }
+  __syncthreads();                                         // also: every wave is done with its images
+  if (tid < kSWaves * kHeadsMax) {
+    const int w = tid >> 4, h = tid & 15;
+    float M = m_s[0][h];
+#pragma unroll
+    for (int ww = 1; ww < kSWaves; ++ww) M = fmaxf(M, m_s[ww][h]);
+    const float mw = m_s[w][h];
+    f_s[w][h] = (mw == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(mw - M);
+    if (w == 0) M_s[h] = M;
+  }
+  __syncthreads();
+  const float4 f4own = *reinterpret_cast<const float4*>(&f_s[wave][4 * g]);
+  const float wscale = inv_tscale * a.v_unscale;
+  const float fown[4] = {f4own.x * wscale, f4own.y * wscale, f4own.z * wscale, f4own.w * wscale};
+  for (int h0 = 0; h0 < n_rep; h0 += 8) {
+    if (h0) __syncthreads();
+    if ((g >> 1) == (h0 >> 3)) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float4* dst = reinterpret_cast<float4*>(&S_all[wave][(4 * g + j) & 7][8 * n16]);
+        const float f = fown[j];
+        dst[0] = make_float4(accS[0][j] * f, accS[1][j] * f, accS[2][j] * f, accS[3][j] * f);
+        dst[1] = make_float4(accS[4][j] * f, accS[5][j] * f, accS[6][j] * f, accS[7][j] * f);
+      }
+    }
+    __syncthreads();
+    const int rows = min(8, n_rep - h0);
+    if (tid < rows * (kD / 4)) {
+      const int hl = tid >> 5, e4 = tid & 31;
+      float4 sum = *reinterpret_cast<const float4*>(&S_all[0][hl][4 * e4]);
+#pragma unroll
+      for (int w = 1; w < kSWaves; ++w) {
+        const float4 x = *reinterpret_cast<const float4*>(&S_all[w][hl][4 * e4]);
+        sum.x += x.x; sum.y += x.y; sum.z += x.z; sum.w += x.w;
+      }
+      *reinterpret_cast<float4*>(pS + (h0 + hl) * kD + 4 * e4) = sum;
+    }
+  }
+  if (tid < n_rep) {
+    const int h = tid;
+    float L = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kSWaves; ++w) L += f_s[w][h] * l_s[w][h];
     pml[2 * h] = M_s[h];
     pml[2 * h + 1] = L;
   }

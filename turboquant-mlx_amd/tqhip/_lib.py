@@ -52,6 +52,7 @@ PROTOTYPES = {
     "tq_softmax_rows": (_i, [_p, _p, _l, _p, _l, _l, _f, _p]),
     "tq_sparse_v_matvec": (_i, [_p, _p, _p, _fp, _p, _p, _p, _z, _i, _i, _l, _l, _l, _i, _i, _f, _i, _p]),
     "tq_flash_decode": (_i, [_p, _p, _p, _p, _p, _fp, _fp, _p, _p, _p, _z, C.POINTER(DecodeShape), _p]),
+    "tq_flash_decode_plan": (_i, [_i, _i, _l, _i, _i]),
     "tq_vonly_decode_attn": (_i, [_p, _i, _p, _p, _p, _fp, _p, _p, _p, _z, C.POINTER(DecodeShape), _p]),
     "tq_vonly_decode_attn_phases": (_i, [_p, _i, _p, _p, _p, _fp, _p, _p, _p, _z, C.POINTER(DecodeShape), _i, _p]),
     "tq_workspace_bytes": (_z, [_i, _i, _i, _l, _i]),
