@@ -366,15 +366,30 @@ __global__ __launch_bounds__(kBlock) void dequant128x3_kernel(const uint32_t* __
   uint32_t grp = row0 / (uint32_t)rm.rows_per_group;
   uint32_t rin = row0 - grp * (uint32_t)rm.rows_per_group;
 
-  for (int pass = 0; pass < passes; ++pass) {
-    if (row0 >= (uint32_t)rm.n_rows) break;                    // uniform over the wavefront
-    const uint32_t* prow = packed + ((int64_t)grp * rm.packed_group_stride + rin) * 13;
-    const float nrm = norms[(int64_t)grp * rm.norms_group_stride + rin + v];
+  // the packed words and the norm of the next pass are fetched while the current one is computed
+  uint32_t pw[4];
+  float pn = 0.0f;
+  auto fetch = [&](uint32_t g_, uint32_t r_) {
+    const uint32_t* prow = packed + ((int64_t)g_ * rm.packed_group_stride + r_) * 13;
+    pn = norms[(int64_t)g_ * rm.norms_group_stride + r_ + v];
 #pragma unroll
     for (int it = 0; it < 4; ++it) {
       const int id = it * 64 + lane;
-      if (id < kEncVecs * 13) words[id] = prow[id];
+      pw[it] = (id < kEncVecs * 13) ? prow[id] : 0u;
     }
+  };
+  if (row0 < (uint32_t)rm.n_rows) fetch(grp, rin);
+  for (int pass = 0; pass < passes; ++pass) {
+    if (row0 >= (uint32_t)rm.n_rows) break;                    // uniform over the wavefront
+    const float nrm = pn;
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const int id = it * 64 + lane;
+      if (id < kEncVecs * 13) words[id] = pw[it];
+    }
+    uint32_t nrin = rin + kEncVecs, ngrp = grp;
+    if (nrin >= (uint32_t)rm.rows_per_group) { nrin = 0; ++ngrp; }
+    if (pass + 1 < passes && row0 + kEncVecs < (uint32_t)rm.n_rows) fetch(ngrp, nrin);
     float xs[4][8];
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
@@ -424,8 +439,8 @@ __global__ __launch_bounds__(kBlock) void dequant128x3_kernel(const uint32_t* __
       }
     }
     row0 += kEncVecs;
-    rin += kEncVecs;
-    if (rin >= (uint32_t)rm.rows_per_group) { rin = 0; ++grp; }
+    rin = nrin;
+    grp = ngrp;
   }
 }
 
