@@ -6,7 +6,7 @@ back-to-back launches, and rotation over several independent input sets so that 
 Infinity Cache cannot serve the reads.  Prints one line per case: us per call, GB/s of algorithmic
 bytes and the fraction of 8 TB/s.
 
-    python -m tqhip.bench_kernels [--iters 200] [--cases encode,scores,flash,sparse_v,vonly,prefill]
+    python -m tqhip.bench_kernels [--iters 200] [--cases encode,scores,flash,flash_long,sparse_v,vonly,prefill]
 """
 from __future__ import annotations
 
@@ -115,6 +115,22 @@ def bench_flash(iters, dev):
     report(f"config 4: flash decode 32/8 heads, 16 seqs, sum L={total}", timeit(fns, max(20, iters // 10)), nbytes)
 
 
+def bench_flash_long(iters, dev):
+    """Flash decode of ONE long sequence (cache layout), packed K and V: the streaming pass at its
+    longest step count."""
+    cb = gaussian_codebook(3)
+    signs = tqhip.random_diagonal_sign(128, 43, device=dev)
+    for n_q, n_kv, T in ((32, 8, 32768), (32, 8, 131072), (28, 4, 131072)):
+        nbytes = n_kv * T * 112 + 2 * n_q * 512
+        n_sets = max(2, n_sets_for(nbytes))
+        ks, vs = packed_sets(n_kv, T, dev, n_sets, 5), packed_sets(n_kv, T, dev, n_sets, 6)
+        q_rot = torch.randn((1, n_q, 128), device=dev)
+        fns = [(lambda i=i: tqhip.flash_decode(q_rot, ks[i][0], ks[i][1], vs[i][0], vs[i][1], cb, cb, signs, 128, 3,
+                                               1 / math.sqrt(128), n_rep=n_q // n_kv, out_dtype=torch.float16))
+               for i in range(n_sets)]
+        report(f"flash decode, one sequence, {n_q}/{n_kv} heads, T={T}", timeit(fns, max(20, iters // 4)), nbytes)
+
+
 def bench_vonly(iters, dev):
     cb = gaussian_codebook(3)
     signs = tqhip.random_diagonal_sign(128, 43, device=dev)
@@ -150,7 +166,7 @@ def bench_prefill(iters, dev):
 
 
 CASES = {"prefill": bench_prefill, "encode": bench_encode, "scores": bench_scores, "sparse_v": bench_sparse_v, "flash": bench_flash,
-         "vonly": bench_vonly}
+         "flash_long": bench_flash_long, "vonly": bench_vonly}
 
 
 def main():
