@@ -101,8 +101,12 @@ __global__ __launch_bounds__(kBlock) void encode_kernel(const T* __restrict__ x,
 //  * x / n is computed as q = x*r, q += r * fma(-n, q, x) with r = 1/n correctly rounded, which
 //    yields the correctly rounded quotient (checked against IEEE division on 3e10 operand pairs
 //    with |x| <= n), at 3 operations per element instead of a full division;
-//  * the count of thresholds exceeded is g + (w > t[g]) with g = clamp(floor(alpha*w + beta), 0, 6),
-//    where the host has verified that g is the count or one less for every w.
+//  * the count of thresholds exceeded is g + (w > t[g]) where g is a guess that the host has verified to be
+//    the count or one less for every w: v = fma(w, alpha, beta + 2^20 + 32) lies in [2^20, 2^21), where
+//    floats are 1/8 apart, so bits 3..8 of v are 32 + floor(alpha*w + beta) (to within the rounding to
+//    1/8) and, masked, are the byte offset into a 64-entry LDS table of (t[g], g) pairs whose entries
+//    below / above the seven levels hold (+inf, 0) / (-inf, 6): no clamp, no float-to-int convert, no
+//    address shift.  A NaN norm forces all indices of the vector to 0 (as comparisons with NaN do).
 // Packed words leave through LDS so that a wavefront stores 208 contiguous words per pass.
 constexpr int kEncVecs = 16;      // vectors per wavefront pass
 constexpr int kEncPasses = 4;     // passes per wavefront once there are rows enough to fill the chip
@@ -116,7 +120,7 @@ __global__ __launch_bounds__(kBlock) void encode128x3_kernel(const T* __restrict
                                                              float* __restrict__ norms, RowMap rm, int passes) {
   constexpr bool kHalfWidth = sizeof(T) == 2;
   constexpr int NM = kHalfWidth ? 4 : 8;                       // sign masks per chunk
-  __shared__ float thr_s[8];
+  __shared__ __align__(8) uint2 lvl_s[64];                     // (threshold bits, guess) by 32 + floor(alpha*w + beta)
   __shared__ __align__(16) float sg_s[128];
   __shared__ uint32_t chunk_s[kWavesPerBlock][kEncVecs * 16 + 4];
 
@@ -124,11 +128,12 @@ __global__ __launch_bounds__(kBlock) void encode128x3_kernel(const T* __restrict
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ls = lane & 3, v = lane >> 2;
-  if (tid < 8) {
-    float t = INFINITY;
+  if (tid < 64) {
+    const int gq = tid - 32;
+    float t = gq < 0 ? INFINITY : -INFINITY;
 #pragma unroll
-    for (int i = 0; i < 7; ++i) t = (tid == i) ? thr.t[i] : t;
-    thr_s[tid] = t;
+    for (int i = 0; i < 7; ++i) t = (gq == i) ? thr.t[i] : t;
+    lvl_s[tid] = make_uint2(__float_as_uint(t), (uint32_t)(gq < 0 ? 0 : (gq > 6 ? 6 : gq)));
   }
   if (tid < 128) sg_s[tid] = signs[tid];
   __syncthreads();
@@ -159,6 +164,13 @@ __global__ __launch_bounds__(kBlock) void encode128x3_kernel(const T* __restrict
   uint32_t grp = row0 / (uint32_t)rm.rows_per_group;
   uint32_t rin = row0 - grp * (uint32_t)rm.rows_per_group;
 
+  // 16-bit inputs: the rows of the next pass are fetched while the current one is computed
+  uint4 nraw[4] = {};
+  if (kHalfWidth && row0 < (uint32_t)rm.n_rows) {
+    const T* xr = x + ((int64_t)row0 + v) * 128 + 8 * ls;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) nraw[k] = *reinterpret_cast<const uint4*>(xr + 32 * k);
+  }
   for (int pass = 0; pass < passes; ++pass) {
     if (row0 >= (uint32_t)rm.n_rows) break;                    // uniform over the wavefront
     // ---- load, flip signs, widen
@@ -167,7 +179,11 @@ __global__ __launch_bounds__(kBlock) void encode128x3_kernel(const T* __restrict
     if (kHalfWidth) {
       uint4 raw[4];
 #pragma unroll
-      for (int k = 0; k < 4; ++k) raw[k] = *reinterpret_cast<const uint4*>(xr + 32 * k);
+      for (int k = 0; k < 4; ++k) raw[k] = nraw[k];
+      if (pass + 1 < passes && row0 + kEncVecs < (uint32_t)rm.n_rows) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) nraw[k] = *reinterpret_cast<const uint4*>(xr + kEncVecs * 128 + 32 * k);
+      }
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         const uint32_t w[4] = {raw[k].x ^ sm[k][0], raw[k].y ^ sm[k][1], raw[k].z ^ sm[k][2], raw[k].w ^ sm[k][3]};
@@ -225,12 +241,12 @@ __global__ __launch_bounds__(kBlock) void encode128x3_kernel(const T* __restrict
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const float w = xs[k][j];
-        const float h = __builtin_amdgcn_fmed3f(__fmaf_rn(w, gs.alpha, gs.beta), 0.0f, 6.0f);
-        const int g = (int)h;
-        const uint32_t idx = (uint32_t)g + ((w > thr_s[g]) ? 1u : 0u);
+        const uint32_t off = __float_as_uint(__fmaf_rn(w, gs.alpha, gs.beta)) & 0x1F8u;
+        const uint2 lv = *reinterpret_cast<const uint2*>(reinterpret_cast<const unsigned char*>(lvl_s) + off);
+        const uint32_t idx = lv.y + ((w > __uint_as_float(lv.x)) ? 1u : 0u);
         bits24 |= idx << (3 * j);
       }
-      chunks[v * 16 + ls + 4 * k] = bits24;
+      chunks[v * 16 + ls + 4 * k] = (nrm != nrm) ? 0u : bits24;
     }
     // ---- words: word wd of a row holds elements 10wd .. 10wd+9 = chunks (5wd)/4 and the next
     uint32_t* prow = packed + ((int64_t)grp * rm.packed_group_stride + rin) * 13;
@@ -542,9 +558,12 @@ float double_rounding_threshold(float b, float s) {
   return ord2f(lo);
 }
 
-// Finds alpha, beta with  j <= alpha * t[j] + beta < j + 1  for every threshold j (with margin), so
-// that floor(alpha * w + beta), clamped to 0..nb-1, is the count of thresholds below w or one
-// less.  False when no such line exists (then the generic kernel counts them one by one).
+// Finds alpha, beta with  j + 1/16 < alpha * t[j] + beta < j + 1 - 1/16  for every threshold j (and a
+// further margin of 0.01), beta a multiple of 1/8.  The kernel evaluates v = fma(w, alpha, beta + 2^20 + 32)
+// in float: one rounding, to a multiple of 1/8, i.e. at most 1/16 away from alpha*w + beta, so
+// floor(v) - 2^20 - 32 is the count of thresholds below w or one less for every w.  |w| <= sqrt(128)
+// (raw butterfly of a unit vector), so the guess must stay within +-32 of zero for the 64-entry table.
+// False when no such line exists (then the generic kernel counts the thresholds one by one).
 bool level_guess_search(const float* t, int nb, EncodeGuess& out);
 
 // The search result is kept for the last threshold set seen.
@@ -579,9 +598,19 @@ bool level_guess_search(const float* t, int nb, EncodeGuess& out) {
     }
     if (hi - lo > best_w) { best_w = hi - lo; best_a = a; best_b = 0.5 * (lo + hi); }
   }
-  if (best_w < 0.1) return false;
+  if (best_w < 0.2) return false;
   out.alpha = (float)best_a;
-  out.beta = (float)best_b;
+  const double a = (double)out.alpha;
+  double lo = -1e300, hi = 1e300;
+  for (int j = 0; j < nb; ++j) {
+    lo = std::fmax(lo, j - a * (double)t[j]);
+    hi = std::fmin(hi, j + 1 - a * (double)t[j]);
+  }
+  const double b = std::floor(0.5 * (lo + hi) * 8.0 + 0.5) / 8.0;
+  const double margin = 1.0 / 16.0 + 0.01;
+  if (!(b - lo >= margin && hi - b >= margin)) return false;
+  if (!(a * 11.4 + std::fabs(b) < 31.0)) return false;
+  out.beta = (float)(b + 1048576.0 + 32.0);                  // exact: a multiple of 1/8 below 2^21
   return true;
 }
 
