@@ -1033,3 +1033,20 @@ def test_flash_plan_masked_and_small_batches_take_the_tile_pass(tq):
     assert _flash_plan(tq, 16, 8, 32768, True, masked=True) == 0
     assert _flash_plan(tq, 16, 8, 32768, True) == 4
     assert _flash_plan(tq, 1, 8, 131072, False) == 8
+
+
+def test_encode_fp16_denormal_and_tiny_inputs(tq):
+    """fp16 inputs whose elements are mostly subnormal halves (scale 1e-5) or exactly representable tiny
+    values: the streaming encoder widens them inside mixed-precision multiplies and must still be
+    bit-exact, norms included."""
+    rng = np.random.default_rng(71)
+    c, b = tables(3)
+    s = o.random_diagonal_sign(128, 43)
+    x = (rng.standard_normal((640, 128)) * np.repeat([1e-5, 3e-5, 1e-4, 6e-8], 160)[:, None]).astype(np.float16)
+    x[5] = 0
+    x[6, 3] = np.float16(6e-8)          # one subnormal element, everything else zero
+    x[6, :3] = 0; x[6, 4:] = 0
+    assert (np.abs(x[x != 0]).astype(np.float32) < 6.1e-5).mean() > 0.5
+    wp, wn = o.fused_quantize(x, s, b, 128, 3)
+    gp, gn = tq.fused_quantize(dev(x), dev(s), b, 128, 3)
+    assert np.array_equal(host(gp), wp) and np.array_equal(host(gn), wn)

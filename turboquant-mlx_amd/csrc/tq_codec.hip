@@ -108,6 +108,32 @@ __global__ __launch_bounds__(kBlock) void encode_kernel(const T* __restrict__ x,
 //    below / above the seven levels hold (+inf, 0) / (-inf, 6): no clamp, no float-to-int convert, no
 //    address shift.  A NaN norm forces all indices of the vector to 0 (as comparisons with NaN do).
 // Packed words leave through LDS so that a wavefront stores 208 contiguous words per pass.
+// Mixed-precision FMA on one half of a packed fp16 pair (HI = 0: low half, 1: high half), so that fp16
+// inputs need no separate widening instruction.  A product is taken as fma(a, b, -0): adding -0 changes
+// no value, not even the sign of a zero, so it rounds exactly like the float32 multiply of the widened
+// operands.
+template <int HI>
+__device__ __forceinline__ float mix_sq(uint32_t h2, float negzero) {           // widen(h) * widen(h)
+  float d;
+  if (HI) asm("v_fma_mix_f32 %0, %1, %1, %2 op_sel:[1,1,0] op_sel_hi:[1,1,0]" : "=v"(d) : "v"(h2), "v"(negzero));
+  else    asm("v_fma_mix_f32 %0, %1, %1, %2 op_sel:[0,0,0] op_sel_hi:[1,1,0]" : "=v"(d) : "v"(h2), "v"(negzero));
+  return d;
+}
+template <int HI>
+__device__ __forceinline__ float mix_mul(uint32_t h2, float b, float negzero) { // widen(h) * b
+  float d;
+  if (HI) asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(d) : "v"(h2), "v"(b), "v"(negzero));
+  else    asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel:[0,0,0] op_sel_hi:[1,0,0]" : "=v"(d) : "v"(h2), "v"(b), "v"(negzero));
+  return d;
+}
+template <int HI>
+__device__ __forceinline__ float mix_fma_addend(float a, float b, uint32_t h2) { // fma(a, b, widen(h))
+  float d;
+  if (HI) asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel:[0,0,1] op_sel_hi:[0,0,1]" : "=v"(d) : "v"(a), "v"(b), "v"(h2));
+  else    asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel:[0,0,0] op_sel_hi:[0,0,1]" : "=v"(d) : "v"(a), "v"(b), "v"(h2));
+  return d;
+}
+
 constexpr int kEncVecs = 16;      // vectors per wavefront pass
 constexpr int kEncPasses = 4;     // passes per wavefront once there are rows enough to fill the chip
 
@@ -173,8 +199,11 @@ __global__ __launch_bounds__(kBlock) void encode128x3_kernel(const T* __restrict
   }
   for (int pass = 0; pass < passes; ++pass) {
     if (row0 >= (uint32_t)rm.n_rows) break;                    // uniform over the wavefront
-    // ---- load, flip signs, widen
+    // ---- load, flip signs, widen (fp16: the packed pairs stay as they are and are widened inside the
+    // mixed-precision multiplies below)
+    constexpr bool kMix = __is_same(T, __half);
     float xs[4][8];
+    uint32_t hw[4][4];
     const T* xr = x + ((int64_t)row0 + v) * 128 + 8 * ls;
     if (kHalfWidth) {
       uint4 raw[4];
@@ -189,10 +218,8 @@ __global__ __launch_bounds__(kBlock) void encode128x3_kernel(const T* __restrict
         const uint32_t w[4] = {raw[k].x ^ sm[k][0], raw[k].y ^ sm[k][1], raw[k].z ^ sm[k][2], raw[k].w ^ sm[k][3]};
 #pragma unroll
         for (int jp = 0; jp < 4; ++jp) {
-          if (sizeof(T) == 2 && __is_same(T, __half)) {
-            xs[k][2 * jp] = __half2float(__ushort_as_half((unsigned short)(w[jp] & 0xFFFFu)));
-            xs[k][2 * jp + 1] = __half2float(__ushort_as_half((unsigned short)(w[jp] >> 16)));
-          } else {
+          hw[k][jp] = w[jp];
+          if (!kMix) {
             xs[k][2 * jp] = __uint_as_float(w[jp] << 16);
             xs[k][2 * jp + 1] = __uint_as_float(w[jp] & 0xFFFF0000u);
           }
@@ -208,13 +235,18 @@ __global__ __launch_bounds__(kBlock) void encode128x3_kernel(const T* __restrict
         for (int j = 0; j < 8; ++j) xs[k][j] = __uint_as_float(w[j] ^ sm[k][j & (NM - 1)]);
       }
     }
+    const float negzero = -0.0f;
     // ---- sum of squares: strides 64, 32 (k), 16, 8 (lanes), 4, 2, 1 (j)
     float t8[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const float s0 = xs[0][j] * xs[0][j], s1 = xs[1][j] * xs[1][j];
-      const float s2 = xs[2][j] * xs[2][j], s3 = xs[3][j] * xs[3][j];
-      t8[j] = (s0 + s2) + (s1 + s3);
+      float sq[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        if (kMix) sq[k] = (j & 1) ? mix_sq<1>(hw[k][j >> 1], negzero) : mix_sq<0>(hw[k][j >> 1], negzero);
+        else sq[k] = xs[k][j] * xs[k][j];
+      }
+      t8[j] = (sq[0] + sq[2]) + (sq[1] + sq[3]);
     }
 #pragma unroll
     for (int j = 0; j < 8; ++j) t8[j] = t8[j] + quad_xor2(t8[j]);
@@ -224,14 +256,22 @@ __global__ __launch_bounds__(kBlock) void encode128x3_kernel(const T* __restrict
     const float nrm = sqrtf(ss);
     const float safe = fmaxf(nrm, 1e-8f);
     const float rinv = 1.0f / safe;
+    const float nsafe = -safe;
     // ---- unit vector
 #pragma unroll
     for (int k = 0; k < 4; ++k)
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        const float q0 = xs[k][j] * rinv;
-        const float rem = __fmaf_rn(-safe, q0, xs[k][j]);
-        xs[k][j] = __fmaf_rn(rem, rinv, q0);
+        if (kMix) {
+          const uint32_t h2 = hw[k][j >> 1];
+          const float q0 = (j & 1) ? mix_mul<1>(h2, rinv, negzero) : mix_mul<0>(h2, rinv, negzero);
+          const float rem = (j & 1) ? mix_fma_addend<1>(nsafe, q0, h2) : mix_fma_addend<0>(nsafe, q0, h2);
+          xs[k][j] = __fmaf_rn(rem, rinv, q0);
+        } else {
+          const float q0 = xs[k][j] * rinv;
+          const float rem = __fmaf_rn(nsafe, q0, xs[k][j]);
+          xs[k][j] = __fmaf_rn(rem, rinv, q0);
+        }
       }
     butterfly_4lane(xs, flip1, flip2);
     // ---- levels, 24 bits per chunk
