@@ -1050,3 +1050,40 @@ def test_encode_fp16_denormal_and_tiny_inputs(tq):
     wp, wn = o.fused_quantize(x, s, b, 128, 3)
     gp, gn = tq.fused_quantize(dev(x), dev(s), b, 128, 3)
     assert np.array_equal(host(gp), wp) and np.array_equal(host(gn), wn)
+
+
+# ------------------------------------------------------------------ committed closed-form vectors
+
+def _golden_cases():
+    import json
+    import os
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "kat_vectors.json")
+    with open(path) as f:
+        return json.load(f)["cases"]
+
+
+@pytest.mark.parametrize("case", _golden_cases(), ids=lambda c: c["name"])
+def test_kernels_reproduce_closed_form_vectors(tq, case):
+    """The committed known answers (exact rational arithmetic on the Hadamard closed form) through the
+    C ABI: encode bit-exact in both threshold variants and from fp16 and fp32 inputs, alone (generic
+    kernel) and as 48 repeated rows (streaming kernel for d = 128 / 3-bit); dequant to float32 rounding."""
+    d, bits = case["dim"], case["bits"]
+    x = np.array(case["x"], np.float32)
+    s = np.array(case["signs"], np.float32)
+    c, b = tables(bits)
+    want_words = np.array([int(w, 16) for w in case["packed_hex"]], np.uint32)
+    for variant in ("mlx", "metal"):
+        for dt in (np.float32, np.float16):
+            for reps in (1, 48):
+                xs = np.repeat(x[None, :], reps, axis=0).astype(dt)
+                gp, gn = tq.fused_quantize(dev(xs), dev(s), b, d, bits, variant=variant)
+                gp, gn = host(gp), host(gn)
+                assert (gp == want_words[None, :]).all(), (variant, dt, reps)
+                assert (gn == np.float32(case["norm"])).all()
+    p = dev(np.repeat(want_words[None, :], 48, axis=0))
+    n = dev(np.full(48, case["norm"], np.float32))
+    want = np.array(case["dequant"])
+    tol = 2e-6 * max(1.0, np.abs(want).max())
+    for reps in (1, 48):
+        deq = host(tq.packed_dequantize(p[:reps], n[:reps], c, dev(s), d, bits)).astype(np.float64)
+        assert np.abs(deq - want[None, :]).max() <= tol

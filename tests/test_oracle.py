@@ -438,3 +438,36 @@ def test_prefill_attention_rows_are_prefix_flash_decodes():
     full = o.prefill_attention(q, kp, kn, vp, vn, c, c, ks, vs, D, bits, sc, pos0, n_rep, causal=False)
     want = o.flash_attention_turboquant(o.prerotate_query(q[:, 2], ks), kp, kn, vp, vn, c, c, vs, D, bits, sc, 16, n_rep)
     assert np.allclose(full[:, 2], want, rtol=1e-5, atol=1e-6)
+
+
+# ------------------------------------------------------------------ committed closed-form vectors
+
+def _golden_cases():
+    import json
+    import os
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "kat_vectors.json")
+    with open(path) as f:
+        return json.load(f)["cases"]
+
+
+@pytest.mark.parametrize("case", _golden_cases(), ids=lambda c: c["name"])
+@pytest.mark.parametrize("variant", ["mlx", "metal"])
+def test_oracle_reproduces_closed_form_vectors(case, variant):
+    """tests/golden/kat_vectors.json is derived in exact rational arithmetic from the Hadamard closed
+    form (tests/golden/make_kat_vectors.py, no oracle code involved): indices, packed words and norms
+    must match bit for bit, the dequantised vector to float32 rounding."""
+    d, bits = case["dim"], case["bits"]
+    x = np.array(case["x"], np.float32)[None, :]
+    s = np.array(case["signs"], np.float32)
+    c = o.gaussian_codebook(bits)
+    b = o.gaussian_boundaries(c)
+    idx, nrm = o.quantize(x, s, b, variant)
+    assert idx[0].tolist() == case["idx"]
+    assert float(nrm.reshape(-1)[0]) == case["norm"]
+    want_words = np.array([int(w, 16) for w in case["packed_hex"]], np.uint32)
+    assert np.array_equal(o.pack_indices(idx, bits)[0], want_words)
+    p, n = o.fused_quantize(x, s, b, d, bits, variant)
+    assert np.array_equal(p[0], want_words) and float(n[0]) == case["norm"]
+    deq = o.packed_dequantize(p, n, c, s, d, bits)[0].astype(np.float64)
+    want = np.array(case["dequant"])
+    assert np.abs(deq - want).max() <= 2e-6 * max(1.0, np.abs(want).max())
