@@ -1087,3 +1087,26 @@ def test_kernels_reproduce_closed_form_vectors(tq, case):
     for reps in (1, 48):
         deq = host(tq.packed_dequantize(p[:reps], n[:reps], c, dev(s), d, bits)).astype(np.float64)
         assert np.abs(deq - want[None, :]).max() <= tol
+
+
+@pytest.mark.parametrize("n_kv,n_rep", [(8, 1), (4, 5), (2, 16)])
+def test_flash_streaming_pass_group_sizes_and_leading_offset(tq, n_kv, n_rep):
+    """Streaming pass with 1, 5 and 16 query heads per kv head, and a batch whose first sequence does not
+    start at row 0 (every block misaligned against 16 bytes by the same amount)."""
+    rng = np.random.default_rng(63 + n_rep)
+    D, bits = 128, 3
+    n_seq = 64 // n_kv                                 # 64 (sequence, kv head) pairs x 17 steps of 256 positions
+    lens = rng.integers(4000, 4600, size=n_seq)
+    offs = (3 + np.concatenate([[0], np.cumsum(lens)])).astype(np.int32)
+    assert _flash_plan(tq, n_seq, n_kv, int(lens.max()), True) >= 2
+    c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, n_kv, int(offs[-1]), D, bits)
+    q = rng.standard_normal((n_seq, n_kv * n_rep, D)).astype(F32)
+    sc = 1 / math.sqrt(D)
+    q_rot = tq.prerotate_query(dev(q.reshape(-1, D)), dev(ks)).reshape(n_seq, n_kv * n_rep, D)
+    got = host(tq.flash_decode(q_rot, dev(kp), dev(kn), dev(vp), dev(vn), c, c, dev(vs), D, bits, sc, n_rep=n_rep,
+                               seq_offsets=dev(offs), max_seq_len=int(lens.max())))
+    for i in range(0, n_seq, max(1, n_seq // 6)):
+        a, e = offs[i], offs[i + 1]
+        want = o.flash_attention_turboquant(o.prerotate_query(q[i], ks), kp[:, a:e], kn[:, a:e], vp[:, a:e],
+                                            vn[:, a:e], c, c, vs, D, bits, sc, 16, n_rep)
+        close(got[i], want)
