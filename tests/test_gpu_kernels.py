@@ -1110,3 +1110,43 @@ def test_flash_streaming_pass_group_sizes_and_leading_offset(tq, n_kv, n_rep):
         want = o.flash_attention_turboquant(o.prerotate_query(q[i], ks), kp[:, a:e], kn[:, a:e], vp[:, a:e],
                                             vn[:, a:e], c, c, vs, D, bits, sc, 16, n_rep)
         close(got[i], want)
+
+
+def test_config4_full_size_paths_agree(tq):
+    """benchmark configuration 4 at full size (16 sequences of 4096..32768 positions, 32 q / 8 kv heads, fp16
+    out): the streaming pass, the one-tile-per-workgroup pass (forced by an all-zero mask) and the float32
+    kernels are three separate code paths and must agree; the two shortest sequences are also checked
+    against the oracle."""
+    rng = np.random.default_rng(4)
+    n_kv, n_rep, D, bits, n_seq = 8, 4, 128, 3, 16
+    lens = rng.integers(4096, 32769, size=n_seq)
+    offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    total, max_len = int(offs[-1]), int(lens.max())
+    assert _flash_plan(tq, n_seq, n_kv, max_len, True) >= 2
+    c, b = tables(bits)
+    ks, vs = o.random_diagonal_sign(D, 42), o.random_diagonal_sign(D, 43)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(4)
+    kp = torch.randint(0, 2 ** 30, (n_kv, total, 13), generator=g, device="cuda", dtype=torch.int32).view(torch.uint32)
+    vp = torch.randint(0, 2 ** 30, (n_kv, total, 13), generator=g, device="cuda", dtype=torch.int32).view(torch.uint32)
+    kn = torch.rand((n_kv, total), generator=g, device="cuda") * 8 + 7
+    vn = torch.rand((n_kv, total), generator=g, device="cuda") + 0.5
+    q = rng.standard_normal((n_seq, n_kv * n_rep, D)).astype(F32)
+    sc = 1 / math.sqrt(D)
+    q_rot = tq.prerotate_query(dev(q.reshape(-1, D)), dev(ks)).reshape(n_seq, n_kv * n_rep, D)
+    kw = dict(n_rep=n_rep, seq_offsets=dev(offs), max_seq_len=max_len)
+    a = tq.flash_decode(q_rot, kp, kn, vp, vn, c, c, dev(vs), D, bits, sc, out_dtype=torch.float16, **kw)
+    zero_mask = torch.zeros((n_seq, 1, max_len), device="cuda")
+    t = tq.flash_decode(q_rot, kp, kn, vp, vn, c, c, dev(vs), D, bits, sc, out_dtype=torch.float16, mask=zero_mask, **kw)
+    f = tq.flash_decode(q_rot, kp, kn, vp, vn, c, c, dev(vs), D, bits, sc, precision="fp32", **kw)
+    assert a.dtype == torch.float16
+    a, t, f = host(a).astype(F32), host(t).astype(F32), host(f)
+    close(a.reshape(-1, D), f.reshape(-1, D), rel=3e-3, row_scale=True)     # + fp16 rounding of the output
+    close(t.reshape(-1, D), f.reshape(-1, D), rel=3e-3, row_scale=True)
+    close(a.reshape(-1, D), t.reshape(-1, D), rel=2e-3, row_scale=True)
+    hk, hkn, hv, hvn = host(kp), host(kn), host(vp), host(vn)
+    for i in np.argsort(lens)[:2]:
+        s0, s1 = offs[i], offs[i + 1]
+        want = o.flash_attention_turboquant(o.prerotate_query(q[i], ks), hk[:, s0:s1], hkn[:, s0:s1], hv[:, s0:s1],
+                                            hvn[:, s0:s1], c, c, vs, D, bits, sc, 16, n_rep)
+        close(a[i], want, rel=3e-3, row_scale=True)
