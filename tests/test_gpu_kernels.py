@@ -1150,3 +1150,64 @@ def test_config4_full_size_paths_agree(tq):
         want = o.flash_attention_turboquant(o.prerotate_query(q[i], ks), hk[:, s0:s1], hkn[:, s0:s1], hv[:, s0:s1],
                                             hvn[:, s0:s1], c, c, vs, D, bits, sc, 16, n_rep)
         close(a[i], want, rel=3e-3, row_scale=True)
+
+
+def test_config5_full_size_encode_paths_agree(tq):
+    """benchmark configuration 5, encode half, at full size: 1 048 576 fp16 vectors with one channel scaled
+    x20.  The streaming encoder (rows in multiples of 16) and the generic one-wavefront-per-vector encoder
+    (taken for a row count that is not a multiple of 16) must produce identical words and norms over the
+    whole tensor; 32 768 vectors spread over it are also compared with the oracle bit for bit."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(5)
+    n = 131072 * 8
+    x = torch.randn((n, 128), generator=g, device="cuda", dtype=torch.float16)
+    x[:, 17] *= 20
+    c, b = tables(3)
+    s = o.random_diagonal_sign(128, 42)
+    fp, fn = tq.fused_quantize(x, dev(s), b, 128, 3)                    # streaming kernel
+    gp, gn = tq.fused_quantize(x[: n - 1], dev(s), b, 128, 3)           # generic kernel: n - 1 rows
+    assert torch.equal(fp[: n - 1].view(torch.int32), gp.view(torch.int32)) and torch.equal(fn[: n - 1], gn)
+    pick = torch.arange(0, n, 32, device="cuda")
+    wp, wn = o.fused_quantize(host(x[pick]), s, b, 128, 3)
+    assert np.array_equal(host(fp.view(torch.int32)[pick]).view(np.uint32), wp) and np.array_equal(host(fn[pick]), wn)
+
+
+def test_config5_full_size_prefill_rows_are_decode_steps(tq):
+    """benchmark configuration 5, attention half, at full size: a 512-row causal chunk at the end of a 131 072-position
+    packed cache, 32 q / 8 kv heads.  Row i of the chunk is one decode step over positions 0 .. T-512+i: three
+    rows are compared with the float32 flash-decode kernels (a separate code path) over those prefixes."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(55)
+    n_kv, n_rep, T, n_rows, D, bits = 8, 4, 131072, 512, 128, 3
+    c, b = tables(bits)
+    ks, vs = dev(o.random_diagonal_sign(D, 42)), dev(o.random_diagonal_sign(D, 43))
+    kp = torch.randint(0, 2 ** 30, (n_kv, T, 13), generator=g, device="cuda", dtype=torch.int32).view(torch.uint32)
+    vp = torch.randint(0, 2 ** 30, (n_kv, T, 13), generator=g, device="cuda", dtype=torch.int32).view(torch.uint32)
+    kn = torch.rand((n_kv, T), generator=g, device="cuda") * 8 + 7
+    vn = torch.rand((n_kv, T), generator=g, device="cuda") + 0.5
+    q = torch.randn((n_kv * n_rep, n_rows, D), generator=g, device="cuda", dtype=torch.float16)
+    sc = 1 / math.sqrt(D)
+    got = tq.prefill_attention(q, kp, kn, vp, vn, c, c, ks, vs, D, bits, sc, n_rep=n_rep, out_dtype=torch.float32)
+    for i in (0, 255, 511):
+        L = T - n_rows + i + 1
+        q_rot = tq.prerotate_query(q[:, i].float(), ks)
+        ref = tq.flash_attention_turboquant(q_rot, kp[:, :L], kn[:, :L], vp[:, :L], vn[:, :L], c, c, vs, D, bits, sc,
+                                            n_rep=n_rep, precision="fp32")
+        close(host(got[:, i]), host(ref), row_scale=True)
+
+
+def test_config3_full_size_scores(tq):
+    """benchmark configuration 3 at its largest size: 28 q / 4 kv heads against 65 536 packed keys; the float32
+    kernel to float32 rounding and the matrix-core kernel to 1e-3 of the row scale, both against the oracle."""
+    rng = np.random.default_rng(3)
+    n_kv, n_rep, T, D, bits = 4, 7, 65536, 128, 3
+    c, b = tables(bits)
+    ks = o.random_diagonal_sign(D, 42)
+    kp = o.pack_indices(rng.integers(0, 8, size=(n_kv, T, D)).astype(np.uint8), bits)
+    kn = (rng.random((n_kv, T)) * 8 + 7).astype(F32)
+    q_rot = o.prerotate_query(rng.standard_normal((n_kv * n_rep, D)).astype(F32), ks)
+    want = o.prerot_fused_qk_scores(q_rot, kp, kn, c, D, bits, n_rep)
+    got32 = host(tq.prerot_fused_qk_scores(dev(q_rot), dev(kp), dev(kn), c, D, bits, n_rep))
+    close(got32, want, rel=1e-5, abs_=1e-4)
+    got16 = host(tq.prerot_fused_qk_scores(dev(q_rot), dev(kp), dev(kn), c, D, bits, n_rep, precision="fp16"))
+    close(got16, want, rel=1e-3, abs_=1e-3 * float(np.abs(want).max()))
