@@ -1211,3 +1211,22 @@ def test_config3_full_size_scores(tq):
     close(got32, want, rel=1e-5, abs_=1e-4)
     got16 = host(tq.prerot_fused_qk_scores(dev(q_rot), dev(kp), dev(kn), c, D, bits, n_rep, precision="fp16"))
     close(got16, want, rel=1e-3, abs_=1e-3 * float(np.abs(want).max()))
+
+
+def test_vonly_decode_bf16_queries_take_the_matrix_core_path(tq):
+    """bf16 queries (a bf16 model over an fp16 key cache): converted to fp16 on load, which is exact for
+    query-sized values, so the result must match the oracle evaluated on the bf16 values, for the tile
+    pass (T = 2048) and the streaming pass (T = 16384, 4 kv heads x 8 heads each)."""
+    rng = np.random.default_rng(81)
+    D, bits, sc = 128, 3, 1 / math.sqrt(128)
+    for n_kv, n_rep, T in ((4, 7, 2048), (4, 8, 16384)):
+        c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, n_kv, T, D, bits)
+        qt = torch.from_numpy(rng.standard_normal((1, n_kv * n_rep, D)).astype(F32)).to(torch.bfloat16)
+        got = tq.vonly_decode(qt.cuda(), dev(K), dev(vp), dev(vn), c, dev(vs), D, bits, sc, n_rep=n_rep,
+                              out_dtype=torch.bfloat16)
+        assert got.dtype == torch.bfloat16
+        want = o.vonly_decode_attention(qt[0].float().numpy(), K, vp, vn, c, vs, D, bits, sc)
+        err = np.abs(got[0].float().cpu().numpy().astype(np.float64) - want)
+        assert (err <= 1e-3 + 6e-3 * np.abs(want)).all(), err.max()       # bf16 rounding of the output: 2^-8
+        got32 = host(tq.vonly_decode(qt.cuda(), dev(K), dev(vp), dev(vn), c, dev(vs), D, bits, sc, n_rep=n_rep))
+        close(got32[0], want)

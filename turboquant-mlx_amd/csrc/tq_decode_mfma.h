@@ -55,7 +55,8 @@ constexpr float kLog2e = 1.44269504088896340736f;
 constexpr int kMergeThreads = 256;
 
 struct MfmaArgs {
-  const __half* q;            // [n_seq, n_q, 128] fp16
+  const __half* q;            // [n_seq, n_q, 128] fp16, or bf16 when q_bf16 is set (converted to fp16 on load: exact
+                              // for values inside the fp16 range, which queries are)
   const __half* k;            // dense keys, rows of 128 halfs
   const uint32_t* v_packed;
   const float* v_norms;
@@ -70,6 +71,7 @@ struct MfmaArgs {
   int32_t n_kv, n_rep, n_tiles_max;
   float attn_scale;
   float v_unscale;            // 1 / the scale the value table was multiplied by on the host
+  int32_t q_bf16;
 #ifdef TQ_TRACE
   unsigned long long* trace;
 #endif
@@ -146,6 +148,7 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
   for (int i = 0; i < 2; ++i) {
     const int w = tid + i * kMfmaThreads;
     my_q[i] = (w < n_rep * (kD / 2)) ? reinterpret_cast<const uint32_t*>(a.q + q_row0 * kD)[w] : 0u;
+    if (a.q_bf16) my_q[i] = pack_h2(__uint_as_float(my_q[i] << 16), __uint_as_float(my_q[i] & 0xFFFF0000u));
   }
   float my_norm;
   {
@@ -511,6 +514,7 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
   for (int i = 0; i < 2; ++i) {
     const int w = tid + i * kMfmaThreads;
     my_q[i] = (w < n_rep * (kD / 2)) ? reinterpret_cast<const uint32_t*>(a.q + q_row0 * kD)[w] : 0u;
+    if (a.q_bf16) my_q[i] = pack_h2(__uint_as_float(my_q[i] << 16), __uint_as_float(my_q[i] & 0xFFFF0000u));
   }
   float nrmA, nrmB = 0.0f;
   u4 vqA[2], vqB[2], kA[8], kB[8];
