@@ -425,3 +425,29 @@ def test_vonly_cache_fused_mode(tq):
     assert torch.equal(tq.vonly_decode_attention(q1, fused, sc), tq.vonly_decode_attention(q1, plain, sc))
     assert torch.equal(patch.scaled_dot_product_attention(q1, kf_, vf_, fused, sc, None),
                        tq.vonly_decode_attention(q1, plain, sc))
+
+
+def test_vonly_cache_with_a_bf16_model(tq):
+    """bf16 keys, values and queries: keys are stored as float16 (exactly), values are dequantised in bf16,
+    a decode step runs on the matrix-core path and matches the oracle on the bf16 inputs, and a multi-token
+    step through the dispatcher works on mixed dtypes."""
+    from tqhip import patch
+    B, n_q, n_kv, S, D = 1, 8, 4, 600, 128
+    sc = 1 / math.sqrt(D)
+    bf = lambda shape, seed: rand(shape, seed).to(torch.bfloat16)
+    k, v, q1, qs = bf((B, n_kv, S, D), 90), bf((B, n_kv, S, D), 91), bf((B, n_q, 1, D), 92), bf((B, n_q, 16, D), 93)
+    cache = tq.VOnlyTurboQuantCache(bits=3, fused=True)
+    k_out, v_out = cache.update_and_fetch(k, v)
+    assert k_out.dtype == torch.float16 and torch.equal(k_out.float(), k.float())       # bf16 -> fp16 is exact here
+    assert v_out.dtype == torch.bfloat16
+    got = patch.scaled_dot_product_attention(q1, k_out, v_out, cache, sc, None)
+    assert got.dtype == torch.bfloat16 and got.shape == (B, n_q, 1, D)
+    vq = cache._v_tq._v_q
+    want = o.vonly_decode_attention(q1[0, :, 0].float().cpu().numpy(), k[0].float().cpu().numpy().astype(np.float16),
+                                    cache._v_tq.v_packed[0, :, :S].cpu().numpy().view(np.uint32),
+                                    cache._v_tq.v_norms[0, :, :S].cpu().numpy(), np.asarray(vq.centroids.cpu()),
+                                    vq.signs.cpu().numpy(), D, 3, sc)
+    err = np.abs(got[0, :, 0].float().cpu().numpy().astype(np.float64) - want)
+    assert (err <= 1e-3 + 6e-3 * np.abs(want)).all(), err.max()
+    multi = patch.scaled_dot_product_attention(qs, k_out, v_out, cache, sc, None)
+    assert multi.dtype == torch.bfloat16 and multi.shape == (B, n_q, 16, D) and bool(torch.isfinite(multi.float()).all())

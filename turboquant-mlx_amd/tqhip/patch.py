@@ -24,6 +24,10 @@ _MISSING = object()
 
 
 def _stock_sdpa(queries, keys, values, scale, mask):
+    if keys.dtype != queries.dtype:            # a V-only cache hands out float16 keys whatever the model's dtype
+        keys = keys.to(queries.dtype)
+    if values.dtype != queries.dtype:
+        values = values.to(queries.dtype)
     n_rep = queries.shape[1] // keys.shape[1]
     if n_rep > 1:
         keys = keys.repeat_interleave(n_rep, dim=1)

@@ -43,7 +43,11 @@ class VOnlyTurboQuantCache:
         return tq._full_dequant(tq.v_packed, tq.v_norms, tq._v_q, tq._v_dim, B, H, tq.offset, dtype or tq._dtype)
 
     def update_and_fetch(self, keys: torch.Tensor, values: torch.Tensor):
-        k_out, _ = self._k_cache.update_and_fetch(keys, values)
+        # The decode kernels read float16 keys: bf16 / float32 keys are stored as float16 (exact for bf16
+        # values inside the float16 range, which keys are); the reference keeps whatever dtype it is
+        # given (v_only_cache.py:41-47), so `state` then differs in the dtype of its first entry.
+        k16 = keys if keys.dtype == torch.float16 else keys.to(torch.float16)
+        k_out, _ = self._k_cache.update_and_fetch(k16, values)
         if self.fused:
             self._encode_only(keys, values)
             B, H, _, v_dim = values.shape
