@@ -451,3 +451,30 @@ def test_vonly_cache_with_a_bf16_model(tq):
     assert (err <= 1e-3 + 6e-3 * np.abs(want)).all(), err.max()
     multi = patch.scaled_dot_product_attention(qs, k_out, v_out, cache, sc, None)
     assert multi.dtype == torch.bfloat16 and multi.shape == (B, n_q, 16, D) and bool(torch.isfinite(multi.float()).all())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_packed_cache_with_bf16_and_float32_models(tq, dtype):
+    """A fused TurboQuantKVCache under a bf16 / float32 model: the prompt chunk and a decode step through the
+    dispatcher return the model's dtype and agree with stock SDPA over the dequantised cache of an unfused
+    twin (same packed state)."""
+    from tqhip import patch
+    B, n_q, n_kv, S, D = 1, 8, 4, 200, 128
+    sc = 1 / math.sqrt(D)
+    mk = lambda shape, seed: rand(shape, seed).to(dtype)
+    k, v, qs = mk((B, n_kv, S, D), 95), mk((B, n_kv, S, D), 96), mk((B, n_q, S, D), 97)
+    k1, v1, q1 = mk((B, n_kv, 1, D), 98), mk((B, n_kv, 1, D), 99), mk((B, n_q, 1, D), 100)
+    fused, plain = tq.TurboQuantKVCache(bits=3, fused=True), tq.TurboQuantKVCache(bits=3)
+    kk, vv = fused.update_and_fetch(k, v)
+    kd, vd = plain.update_and_fetch(k, v)
+    assert torch.equal(fused.k_packed.view(torch.int32), plain.k_packed.view(torch.int32))
+    a = patch.scaled_dot_product_attention(qs, kk, vv, fused, sc, "causal")
+    b = patch.scaled_dot_product_attention(qs, kd, vd, plain, sc, "causal")
+    assert a.dtype == dtype and b.dtype == dtype
+    assert cos(host(a), host(b)) > 0.9995
+    kk, vv = fused.update_and_fetch(k1, v1)
+    kd, vd = plain.update_and_fetch(k1, v1)
+    a = patch.scaled_dot_product_attention(q1, kk, vv, fused, sc, None)
+    b = patch.scaled_dot_product_attention(q1, kd, vd, plain, sc, None)
+    assert a.dtype == dtype and a.shape == (B, n_q, 1, D)
+    assert cos(host(a), host(b)) > 0.9995
