@@ -1230,3 +1230,25 @@ def test_vonly_decode_bf16_queries_take_the_matrix_core_path(tq):
         assert (err <= 1e-3 + 6e-3 * np.abs(want)).all(), err.max()       # bf16 rounding of the output: 2^-8
         got32 = host(tq.vonly_decode(qt.cuda(), dev(K), dev(vp), dev(vn), c, dev(vs), D, bits, sc, n_rep=n_rep))
         close(got32[0], want)
+
+
+def test_vonly_decode_float32_queries_keep_their_precision(tq):
+    """float32 queries on the matrix-core path enter as fp16 value + fp16 remainder.  On data with x20 outlier
+    channels in K (peaked softmax, logits in the hundreds) rounding the query to one fp16 shows; the
+    two-term form must stay close to the float32 kernels."""
+    rng = np.random.default_rng(91)
+    n_kv, n_rep, T, D, bits = 4, 7, 4096, 128, 3
+    c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, n_kv, T, D, bits, outliers=True)
+    q = rng.standard_normal((1, n_kv * n_rep, D)).astype(F32)
+    q[..., 7] *= 3
+    sc = 1 / math.sqrt(D)
+    args = (dev(K), dev(vp), dev(vn), c, dev(vs), D, bits, sc)
+    ref = host(tq.vonly_decode(dev(q), *args, n_rep=n_rep, precision="fp32"))[0]
+    two = host(tq.vonly_decode(dev(q), *args, n_rep=n_rep))[0]
+    one = host(tq.vonly_decode(dev(q.astype(np.float16)), *args, n_rep=n_rep))[0]
+    scale = np.abs(ref).max(axis=-1, keepdims=True)
+    e_two, e_one = (np.abs(two - ref) / scale).max(), (np.abs(one - ref) / scale).max()
+    print(f"max error / row scale: two-term {e_two:.2e}, one fp16 {e_one:.2e}")
+    assert e_two < 1e-3 and e_two < 0.5 * e_one
+    want = o.vonly_decode_attention(q[0], K, vp, vn, c, vs, D, bits, sc)
+    close(two, want, row_scale=True)

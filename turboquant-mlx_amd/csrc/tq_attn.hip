@@ -530,7 +530,7 @@ int launch_decode(const void* q, int q_dtype, const uint32_t* k_packed, const fl
 }
 
 // Matrix-core path: tile pass (partials of 512-position tiles) + merge pass.
-int launch_vonly_mfma(const void* q, bool q_bf16, const void* k_f16, const uint32_t* v_packed, const float* v_norms,
+int launch_vonly_mfma(const void* q, int q_dtype, const void* k_f16, const uint32_t* v_packed, const float* v_norms,
                       const float* v_centroids, const float* v_signs, void* out, void* workspace,
                       size_t workspace_bytes, const tq_decode_shape& sh, hipStream_t stream, int phases) {
   const char* who = "tq_vonly_decode_attn";
@@ -552,7 +552,8 @@ int launch_vonly_mfma(const void* q, bool q_bf16, const void* k_f16, const uint3
     return tq::fail(TQ_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, need, workspace_bytes);
   if (!tq::aligned(workspace, 16)) return tq::fail(TQ_ERR_ALIGN, "%s: workspace must be 16-byte aligned", who);
   tqm::MfmaArgs a{};
-  a.q = (const __half*)q; a.k = (const __half*)k_f16; a.q_bf16 = q_bf16 ? 1 : 0;
+  a.q = (const __half*)q; a.k = (const __half*)k_f16; a.q_bf16 = q_dtype == TQ_BF16 ? 1 : 0;
+  const bool q_f32 = q_dtype == TQ_F32;
   a.v_packed = v_packed; a.v_norms = v_norms;
   a.seq_offsets = sh.seq_offsets; a.mask = sh.mask;
   a.ws_S = (float*)workspace;
@@ -575,9 +576,15 @@ int launch_vonly_mfma(const void* q, bool q_bf16, const void* k_f16, const uint3
   a.v_unscale = tq::fill_codebook_fp16(vcb, v_centroids, sh.bits);
   if (phases & 1) {
     dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
-    if (n_blocks > 1) tqm::vonly_stream_kernel<<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb, n_blocks);
-    else     if (plain) tqm::vonly_tile_mfma_kernel<true><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb);
-    else tqm::vonly_tile_mfma_kernel<false><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb);
+    if (q_f32) {
+      if (n_blocks > 1) tqm::vonly_stream_kernel<true><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb, n_blocks);
+      else if (plain) tqm::vonly_tile_mfma_kernel<true, true><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb);
+      else tqm::vonly_tile_mfma_kernel<false, true><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb);
+    } else {
+      if (n_blocks > 1) tqm::vonly_stream_kernel<false><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb, n_blocks);
+      else if (plain) tqm::vonly_tile_mfma_kernel<true, false><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb);
+      else tqm::vonly_tile_mfma_kernel<false, false><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb);
+    }
     TQ_CHECK_LAUNCH(who);
   }
   if (!(phases & 2)) return TQ_OK;
@@ -828,9 +835,9 @@ extern "C" int tq_vonly_decode_attn_phases(const void* q, int q_dtype, const voi
   if (shape->seq_len > 0 && (!k_f16 || !v_packed || !v_norms))
     return tq::fail(TQ_ERR_NULL, "tq_vonly_decode_attn: null pointer");
   if (!tq::aligned(k_f16, 16)) return tq::fail(TQ_ERR_ALIGN, "tq_vonly_decode_attn: k must be 16-byte aligned");
-  // d = 128, 3-bit, fp16 or bf16 queries, at most 16 query heads per kv head: matrix-core tile pass.
-  if (mma_shape(*shape) && (q_dtype == TQ_F16 || q_dtype == TQ_BF16) && tq::aligned(q, 4))
-    return launch_vonly_mfma(q, q_dtype == TQ_BF16, k_f16, v_packed, v_norms, v_centroids, v_signs, out, workspace, workspace_bytes,
+  // d = 128, 3-bit, at most 16 query heads per kv head: matrix-core tile pass (float32 queries as fp16 value + remainder).
+  if (mma_shape(*shape) && tq::aligned(q, q_dtype == TQ_F32 ? 8 : 4))
+    return launch_vonly_mfma(q, q_dtype, k_f16, v_packed, v_norms, v_centroids, v_signs, out, workspace, workspace_bytes,
                              *shape, (hipStream_t)stream_, phases);
   return launch_decode<kDenseK>(q, q_dtype, nullptr, nullptr, k_f16, v_packed, v_norms, nullptr, v_centroids,
                                 v_signs, out, workspace, workspace_bytes, *shape, 0.0f, (hipStream_t)stream_,

@@ -110,7 +110,9 @@ __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
 // PLAIN = no mask, no ragged offsets, seq_len a multiple of the tile, 16-byte aligned V rows (checked
 // by the host): every tile is full, so the row clamps, the validity selects, the mask reads and the
 // narrow V path drop out, and K / V addresses are a uniform base plus a lane-constant offset.
-template <bool PLAIN>
+// QF32: the queries are float32 and enter as an fp16 value plus the fp16 remainder of that rounding (two
+// matrix instructions per key operand), which keeps float32-query fidelity; otherwise fp16 (or bf16) queries.
+template <bool PLAIN, bool QF32>
 __global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
   // 32 KB used three ways: per-wave staging (8 x 4 KB) first for the packed V block, then for K
@@ -118,6 +120,7 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
   __shared__ __align__(16) unsigned char big_s[32768];
   __shared__ uint32_t lut_s[64];                       // half2(c[i & 7], c[i >> 3])
   __shared__ __align__(16) uint32_t q_s[kHeadsMax][kD / 2];   // fp16 pairs, rows >= n_rep are zero
+  __shared__ __align__(16) uint32_t ql_s[QF32 ? kHeadsMax : 1][kD / 2];   // QF32: what rounding the query to fp16 lost
   __shared__ __align__(16) float nrm_s[kWaves][kWavePos];
   __shared__ float m_s[kWaves][kHeadsMax], l_s[kWaves][kHeadsMax], M_s[kHeadsMax];
   __shared__ __align__(16) float f_s[kWaves][kHeadsMax];
@@ -143,12 +146,21 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
   const int wrow0 = wave * kWavePos;                                  // wave's first row inside the tile
 
   // ---- issue every global load of this wave, small ones first -------------------------------------
-  uint32_t my_q[2];                                    // Q rows of this kv head: n_rep x 64 words, <= 1024
+  uint32_t my_q[2], my_ql[2] = {0u, 0u};               // Q rows of this kv head: n_rep x 64 words, <= 1024
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int w = tid + i * kMfmaThreads;
-    my_q[i] = (w < n_rep * (kD / 2)) ? reinterpret_cast<const uint32_t*>(a.q + q_row0 * kD)[w] : 0u;
-    if (a.q_bf16) my_q[i] = pack_h2(__uint_as_float(my_q[i] << 16), __uint_as_float(my_q[i] & 0xFFFF0000u));
+    if (QF32) {
+      const float2 f = (w < n_rep * (kD / 2)) ? reinterpret_cast<const float2*>(reinterpret_cast<const float*>(a.q) + q_row0 * kD)[w]
+                                              : make_float2(0.f, 0.f);
+      const __half2 h = __floats2half2_rn(f.x, f.y);
+      const float2 back = __half22float2(h);
+      my_q[i] = *reinterpret_cast<const uint32_t*>(&h);
+      my_ql[i] = pack_h2(f.x - back.x, f.y - back.y);
+    } else {
+      my_q[i] = (w < n_rep * (kD / 2)) ? reinterpret_cast<const uint32_t*>(a.q + q_row0 * kD)[w] : 0u;
+      if (a.q_bf16) my_q[i] = pack_h2(__uint_as_float(my_q[i] << 16), __uint_as_float(my_q[i] & 0xFFFF0000u));
+    }
   }
   float my_norm;
   {
@@ -223,15 +235,21 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
     lut_s[tid] = pack_h2(clo, chi);
   }
 #pragma unroll
-  for (int i = 0; i < 2; ++i) (&q_s[0][0])[tid + i * kMfmaThreads] = my_q[i];
+  for (int i = 0; i < 2; ++i) {
+    (&q_s[0][0])[tid + i * kMfmaThreads] = my_q[i];
+    if (QF32) (&ql_s[0][0])[tid + i * kMfmaThreads] = my_ql[i];
+  }
   nrm_s[wave][lane] = my_norm;
   __syncthreads();
   TQ_STAMP(1);
 
   // ---- Q operand and the V norms of this lane's 16 positions ----------------------------------------
-  u4 qreg[4];
+  u4 qreg[4], qlow[4];
 #pragma unroll
-  for (int kb = 0; kb < 4; ++kb) qreg[kb] = *reinterpret_cast<const u4*>(&q_s[n16][(4 * kb + g) * 4]);
+  for (int kb = 0; kb < 4; ++kb) {
+    qreg[kb] = *reinterpret_cast<const u4*>(&q_s[n16][(4 * kb + g) * 4]);
+    if (QF32) qlow[kb] = *reinterpret_cast<const u4*>(&ql_s[n16][(4 * kb + g) * 4]);
+  }
   float vn[4][4];
   float nmax = 0.0f;
 #pragma unroll
@@ -302,6 +320,8 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
 #pragma unroll
     for (int kb = 0; kb < 4; ++kb) {
       const u4 ka = kst[n16 * 16 + ((4 * kb + g) ^ (n16 & 7))];       // piece 4kb+g of row n16
+      if (QF32) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, ka), __builtin_bit_cast(h8, qlow[kb]),
+                                                             acc, 0, 0, 0);
       acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, ka), __builtin_bit_cast(h8, qreg[kb]),
                                                    acc, 0, 0, 0);
     }
@@ -464,11 +484,13 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
 // grid = (seq_len / (512 * n_blocks), n_kv, n_seq), 512 threads.
 constexpr int kStepPos = 32;
 
+template <bool QF32>
 __global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
   __shared__ __align__(16) unsigned char big_s[32768];
   __shared__ uint32_t lut_s[64];
   __shared__ __align__(16) uint32_t q_s[kHeadsMax][kD / 2];
+  __shared__ __align__(16) uint32_t ql_s[QF32 ? kHeadsMax : 1][kD / 2];
   __shared__ __align__(16) float nrm_s[kWaves][kStepPos];
   __shared__ __align__(16) float alpha_s[kWaves][kHeadsMax];
   __shared__ float m_s[kWaves][kHeadsMax], l_s[kWaves][kHeadsMax], M_s[kHeadsMax];
@@ -509,12 +531,21 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
     kx[4 * part + 3] = *reinterpret_cast<const u4*>(kb + 2048 + koff_odd);
   };
 
-  uint32_t my_q[2];
+  uint32_t my_q[2], my_ql[2] = {0u, 0u};
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int w = tid + i * kMfmaThreads;
-    my_q[i] = (w < n_rep * (kD / 2)) ? reinterpret_cast<const uint32_t*>(a.q + q_row0 * kD)[w] : 0u;
-    if (a.q_bf16) my_q[i] = pack_h2(__uint_as_float(my_q[i] << 16), __uint_as_float(my_q[i] & 0xFFFF0000u));
+    if (QF32) {
+      const float2 f = (w < n_rep * (kD / 2)) ? reinterpret_cast<const float2*>(reinterpret_cast<const float*>(a.q) + q_row0 * kD)[w]
+                                              : make_float2(0.f, 0.f);
+      const __half2 h = __floats2half2_rn(f.x, f.y);
+      const float2 back = __half22float2(h);
+      my_q[i] = *reinterpret_cast<const uint32_t*>(&h);
+      my_ql[i] = pack_h2(f.x - back.x, f.y - back.y);
+    } else {
+      my_q[i] = (w < n_rep * (kD / 2)) ? reinterpret_cast<const uint32_t*>(a.q + q_row0 * kD)[w] : 0u;
+      if (a.q_bf16) my_q[i] = pack_h2(__uint_as_float(my_q[i] << 16), __uint_as_float(my_q[i] & 0xFFFF0000u));
+    }
   }
   float nrmA, nrmB = 0.0f;
   u4 vqA[2], vqB[2], kA[8], kB[8];
@@ -536,12 +567,18 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
     lut_s[tid] = pack_h2(clo, chi);
   }
 #pragma unroll
-  for (int i = 0; i < 2; ++i) (&q_s[0][0])[tid + i * kMfmaThreads] = my_q[i];
+  for (int i = 0; i < 2; ++i) {
+    (&q_s[0][0])[tid + i * kMfmaThreads] = my_q[i];
+    if (QF32) (&ql_s[0][0])[tid + i * kMfmaThreads] = my_ql[i];
+  }
   __syncthreads();
 
-  u4 qreg[4];
+  u4 qreg[4], qlow[4];
 #pragma unroll
-  for (int kb = 0; kb < 4; ++kb) qreg[kb] = *reinterpret_cast<const u4*>(&q_s[n16][(4 * kb + g) * 4]);
+  for (int kb = 0; kb < 4; ++kb) {
+    qreg[kb] = *reinterpret_cast<const u4*>(&q_s[n16][(4 * kb + g) * 4]);
+    if (QF32) qlow[kb] = *reinterpret_cast<const u4*>(&ql_s[n16][(4 * kb + g) * 4]);
+  }
   const float cs = a.attn_scale * kLog2e;
   uint32_t* stage = reinterpret_cast<uint32_t*>(big_s) + wave * 1024;   // this wave's 4 KB
   u4* kst = reinterpret_cast<u4*>(stage);
@@ -613,6 +650,8 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
 #pragma unroll
       for (int kb = 0; kb < 4; ++kb) {
         const u4 ka = kst[n16 * 16 + ((4 * kb + g) ^ (n16 & 7))];
+        if (QF32) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, ka), __builtin_bit_cast(h8, qlow[kb]),
+                                                               acc, 0, 0, 0);
         acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, ka), __builtin_bit_cast(h8, qreg[kb]),
                                                      acc, 0, 0, 0);
       }

@@ -519,8 +519,8 @@ def vonly_decode(q: torch.Tensor, k: torch.Tensor, v_packed, v_norms, v_centroid
                  seq_offsets: torch.Tensor | None = None, max_seq_len: int | None = None, mask=None,
                  out_dtype=torch.float32, precision: str = "fp16") -> torch.Tensor:
     """Dense-softmax decode attention over fp16 keys and packed values (tq_vonly_decode_attn).
-    precision as in flash_decode (the matrix-core path also needs fp16 or bf16 queries; float32 queries take the
-    float32 kernels).
+    precision as in flash_decode (on the matrix-core path fp16 queries enter as they are, bf16 converted to
+    fp16, float32 as an fp16 value plus the fp16 remainder of that rounding).
 
     q (n_seq, n_q, dim) fp16/bf16/fp32; k [n_seq, n_kv, T_alloc, dim] or ragged [n_kv, sum(L), dim] fp16;
     V as in flash_decode.  Returns (n_seq, n_q, dim) `out_dtype`.
