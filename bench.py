@@ -39,7 +39,7 @@ N_SETS = 10
 # copy of ALGO_BYTES bytes (FETCH_SIZE reads 19986.7 for 39950 KiB -> factor 1.9988; WRITE_SIZE
 # reads 39950.0 -> factor 1.0000).  Tile pass: FETCH_SIZE 20059.3 -> 40095 KiB, WRITE_SIZE 916.0
 # -> 916 KiB.  Summary: profiles/vonly_decode_c2_pmc_traffic.md.
-MEASURED_TRAFFIC_BYTES = int((20059.3 * 39950.0 / 19986.7 + 916.0) * 1024)
+MEASURED_TRAFFIC_BYTES = 41995395           # (20059.3 * 39950.0 / 19986.7 + 916.0) KiB, unrounded inputs
 
 
 def make_sets(torch, tqhip, dev):
