@@ -1252,3 +1252,25 @@ def test_vonly_decode_float32_queries_keep_their_precision(tq):
     assert e_two < 1e-3 and e_two < 0.5 * e_one
     want = o.vonly_decode_attention(q[0], K, vp, vn, c, vs, D, bits, sc)
     close(two, want, row_scale=True)
+
+
+def test_encode_overflowing_norm_and_infinite_elements(tq):
+    """float32 vectors whose sum of squares overflows (norm = inf: every finite element divides to 0, index 3)
+    and vectors with an infinite element (inf / inf = NaN spreads to every output, index 0): the streaming
+    and the generic encoder must both follow the oracle."""
+    rng = np.random.default_rng(92)
+    c, b = tables(3)
+    s = o.random_diagonal_sign(128, 42)
+    x = rng.standard_normal((48, 128)).astype(F32)
+    x[3] *= 1e25
+    x[7, 11] = np.inf
+    x[20, 5] = -np.inf
+    x[21] *= 3e19
+    with np.errstate(all="ignore"):
+        wp, wn = o.fused_quantize(x, s, b, 128, 3)
+    for rows in (48, 47):                                              # streaming / generic kernel
+        gp, gn = tq.fused_quantize(dev(x[:rows]), dev(s), b, 128, 3)
+        assert np.array_equal(host(gp), wp[:rows])
+        assert np.array_equal(host(gn), wn[:rows], equal_nan=True)
+    assert np.isinf(wn[3]) and (o.unpack_indices(wp[3:4], 3, 128) == 3).all()
+    assert (o.unpack_indices(wp[7:8], 3, 128) == 0).all()

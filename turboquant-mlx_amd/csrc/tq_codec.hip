@@ -256,7 +256,9 @@ __global__ __launch_bounds__(kBlock) void encode128x3_kernel(const T* __restrict
     const float nrm = sqrtf(ss);
     const float safe = fmaxf(nrm, 1e-8f);
     const float rinv = 1.0f / safe;
-    const float nsafe = -safe;
+    // a norm that overflowed to infinity: x / inf is 0 for every finite x, which q = x * 0 already is; the
+    // correction term must then not multiply infinity by that zero
+    const float nsafe = (safe == INFINITY) ? 0.0f : -safe;
     // ---- unit vector
 #pragma unroll
     for (int k = 0; k < 4; ++k)
