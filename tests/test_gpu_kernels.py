@@ -1274,3 +1274,17 @@ def test_encode_overflowing_norm_and_infinite_elements(tq):
         assert np.array_equal(host(gn), wn[:rows], equal_nan=True)
     assert np.isinf(wn[3]) and (o.unpack_indices(wp[3:4], 3, 128) == 3).all()
     assert (o.unpack_indices(wp[7:8], 3, 128) == 0).all()
+
+
+@pytest.mark.parametrize("scale", [1e-19, 1e-21, 1e-22, 1e-23, 1e-30, 1e-42])
+def test_encode_tiny_float32_inputs(tq, scale):
+    """float32 inputs whose squares are subnormal or underflow (norm subnormal or 0, clamped to 1e-8 by the
+    quantiser): both encoders must follow the oracle bit for bit, subnormal arithmetic included."""
+    rng = np.random.default_rng(93)
+    c, b = tables(3)
+    s = o.random_diagonal_sign(128, 42)
+    x = (rng.standard_normal((48, 128)) * scale).astype(F32)
+    wp, wn = o.fused_quantize(x, s, b, 128, 3)
+    for rows in (48, 47):                                              # streaming / generic kernel
+        gp, gn = tq.fused_quantize(dev(x[:rows]), dev(s), b, 128, 3)
+        assert np.array_equal(host(gp), wp[:rows]) and np.array_equal(host(gn), wn[:rows])
