@@ -1288,3 +1288,29 @@ def test_encode_tiny_float32_inputs(tq, scale):
     for rows in (48, 47):                                              # streaming / generic kernel
         gp, gn = tq.fused_quantize(dev(x[:rows]), dev(s), b, 128, 3)
         assert np.array_equal(host(gp), wp[:rows]) and np.array_equal(host(gn), wn[:rows])
+
+
+def test_fully_masked_rows_yield_zeros(tq):
+    """A query head whose every position is masked: the kernels return zeros for it (softmax over an empty set;
+    the reference's mx.softmax would give NaN there) and leave the other heads untouched, on the matrix-core
+    and the float32 paths of both fused decode ops."""
+    rng = np.random.default_rng(94)
+    n_kv, n_rep, T, D, bits = 2, 4, 700, 128, 3
+    c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, n_kv, T, D, bits)
+    q = rng.standard_normal((1, n_kv * n_rep, D)).astype(np.float16)
+    sc = 1 / math.sqrt(D)
+    mask = np.zeros((1, n_kv * n_rep, T), F32)
+    mask[0, 0, :] = -np.inf                       # head 0 sees nothing
+    mask[0, 5, 100:] = -np.inf                    # head 5 sees the first 100 positions
+    q_rot = tq.prerotate_query(dev(q.reshape(-1, D).astype(F32)), dev(ks)).reshape(1, -1, D)
+    for precision in ("fp16", "fp32"):
+        a = host(tq.vonly_decode(dev(q), dev(K), dev(vp), dev(vn), c, dev(vs), D, bits, sc, n_rep=n_rep,
+                                 mask=dev(mask), precision=precision))[0]
+        f = host(tq.flash_decode(q_rot, dev(kp), dev(kn), dev(vp), dev(vn), c, c, dev(vs), D, bits, sc, n_rep=n_rep,
+                                 mask=dev(mask), precision=precision))[0]
+        assert (a[0] == 0).all() and (f[0] == 0).all(), precision
+        want_v = o.vonly_decode_attention(q[0, 4:8], K[1:], vp[1:], vn[1:], c, vs, D, bits, sc, mask=mask[0, 4:8])
+        close(a[4:8], want_v)
+        want_f = o.turboquant_attention_single(q[0, 4:8].astype(F32), kp[1:], kn[1:], vp[1:], vn[1:], c, ks, c, vs,
+                                               D, bits, sc, mask=mask[0, 4:8])
+        close(f[4:8], want_f)
