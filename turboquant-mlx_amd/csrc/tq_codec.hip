@@ -378,6 +378,9 @@ __global__ __launch_bounds__(kBlock) void dequant128x3_kernel(const uint32_t* __
   __shared__ __align__(16) float sg_s[128];
   __shared__ __align__(8) float2 pair_s[64];
   __shared__ uint32_t words_s[kWavesPerBlock][kEncVecs * 13 + 3];
+  // 16-bit outputs leave through LDS: 16 rows of 256 bytes at a pitch of 320 (conflict-free 16-byte writes per
+  // lane and reads per row segment), so that every store instruction writes 1 KB of contiguous memory
+  __shared__ __align__(16) unsigned char orow_s[sizeof(TO) == 2 ? kWavesPerBlock : 1][sizeof(TO) == 2 ? kEncVecs * 320 : 16];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -493,8 +496,15 @@ __global__ __launch_bounds__(kBlock) void dequant128x3_kernel(const uint32_t* __
           }
           w[jp] = (lo | (hi << 16)) ^ ((sm[k][2 * jp] >> 16) | sm[k][2 * jp + 1]);
         }
-        *reinterpret_cast<uint4*>(orow + 32 * k) = make_uint4(w[0], w[1], w[2], w[3]);
+        *reinterpret_cast<uint4*>(&orow_s[wave][v * 320 + 64 * k + 16 * ls]) = make_uint4(w[0], w[1], w[2], w[3]);
       }
+    }
+    if (sizeof(TO) == 2) {
+      unsigned char* oblock = reinterpret_cast<unsigned char*>(out + ((int64_t)grp * rm.out_group_stride + rin) * 128);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        *reinterpret_cast<uint4*>(oblock + (i * 64 + lane) * 16) =
+            *reinterpret_cast<const uint4*>(&orow_s[wave][(4 * i + (lane >> 4)) * 320 + (lane & 15) * 16]);
     }
     row0 += kEncVecs;
     rin = nrin;
