@@ -274,15 +274,29 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
       }
     }
     if (MODE == kScores) {
-      if (n16 < n_rep) {
-        float* orow = a.scores + ((int64_t)kvh * n_rep + n16) * len + tile_p0;
+      // The wave's 64 x n_rep scores leave through its LDS area (the key image has been consumed), so that a
+      // store instruction writes whole 256-byte runs of a head's row instead of 64 separate floats: the
+      // area is [16 heads][16 units of 4 positions], the unit index xor-ed with the head (conflict-free
+      // 16-byte accesses both ways).
+      f4* sc = reinterpret_cast<f4*>(stage);
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
+      for (int t = 0; t < 4; ++t) sc[n16 * 16 + ((4 * t + g) ^ n16)] = f4{s[t][0], s[t][1], s[t][2], s[t][3]};
+      const bool vec_ok = ((len & 3) == 0) && ((reinterpret_cast<uintptr_t>(a.scores) & 15) == 0);   // uniform
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const int row = wrow0 + 16 * t + 4 * g + j;
-            if (row < rows_here) orow[row] = s[t][j];
+      for (int i = 0; i < 4; ++i) {
+        const int h = 4 * i + g, unit = n16;                          // lane -> head 4i + lane / 16, positions 4 * (lane % 16) ..
+        if (h < n_rep) {
+          const f4 v = sc[h * 16 + (unit ^ h)];
+          const int row0 = wrow0 + 4 * unit;
+          float* dst = a.scores + ((int64_t)kvh * n_rep + h) * len + tile_p0 + row0;
+          if (vec_ok && row0 + 4 <= rows_here) {
+            *reinterpret_cast<f4*>(dst) = v;
+          } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              if (row0 + j < rows_here) dst[j] = v[j];
           }
+        }
       }
       return;
     }
