@@ -162,15 +162,26 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
   // given weights: lane (head n16, group g) takes positions 16t + 4g + j
   float wgt[4][4];
   if (MODE == kWeights) {
+    // four consecutive positions per (lane, t): one 16-byte load where the row is aligned and inside the tile
+    const bool vec_ok = ((len & 3) == 0) && ((reinterpret_cast<uintptr_t>(a.weights) & 15) == 0);   // uniform
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
+    for (int t = 0; t < 4; ++t) {
+      const int row0 = wrow0 + 16 * t + 4 * g;
+      const float* src = a.weights + ((int64_t)kvh * n_rep + n16) * len + tile_p0 + row0;
+      float w[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+      if (n16 < n_rep) {
+        if (vec_ok && row0 + 4 <= rows_here) {
+          const f4 v = *reinterpret_cast<const f4*>(src);
+          w[0] = v[0]; w[1] = v[1]; w[2] = v[2]; w[3] = v[3];
+        } else {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int row = wrow0 + 16 * t + 4 * g + j;
-        float w = 0.0f;
-        if (row < rows_here && n16 < n_rep) w = a.weights[((int64_t)kvh * n_rep + n16) * len + tile_p0 + row];
-        wgt[t][j] = (w < a.threshold) ? 0.0f : w;
+          for (int j = 0; j < 4; ++j)
+            if (row0 + j < rows_here) w[j] = src[j];
+        }
       }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) wgt[t][j] = (w[j] < a.threshold) ? 0.0f : w[j];
+    }
   }
   if (HAS_K) fill_lut(lutk_s, kcb, tid);
   if (HAS_V) fill_lut(lutv_s, vcb, tid);
