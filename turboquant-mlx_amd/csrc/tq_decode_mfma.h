@@ -101,6 +101,20 @@ struct MfmaArgs {
 #define TQ_STAMP_WAVE() do {} while (0)
 #endif
 
+// additive mask of four consecutive positions row0 .. row0 + 3 of one head: one 16-byte load where the row is
+// aligned and the positions are inside the tile, else element by element; positions past the tile read as 0
+__device__ __forceinline__ void load_mask4(const float* src, int row0, int rows_here, bool vec_ok, float (&m)[4]) {
+  m[0] = m[1] = m[2] = m[3] = 0.0f;
+  if (vec_ok && row0 + 4 <= rows_here) {
+    const f4 v = *reinterpret_cast<const f4*>(src);
+    m[0] = v[0]; m[1] = v[1]; m[2] = v[2]; m[3] = v[3];
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (row0 + j < rows_here) m[j] = src[j];
+  }
+}
+
 __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
   __half2 h = __floats2half2_rn(a, b);
   return *reinterpret_cast<uint32_t*>(&h);
@@ -313,6 +327,8 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
   float s[4][4];
   const float cs = a.attn_scale * kLog2e;                // scores are kept in log2 units: e^x = 2^(x log2 e)
   u4* kst = reinterpret_cast<u4*>(stage);                             // 256 pieces of 16 bytes
+  const bool mask_vec = a.mask && ((reinterpret_cast<uintptr_t>(a.mask) & 15) == 0) && ((a.mask_seq_stride & 3) == 0) &&
+                        ((a.mask_head_stride & 3) == 0);      // uniform
   auto qk_tile = [&](int t) {
 #pragma unroll
     for (int ii = 0; ii < 4; ++ii) kst[ii * 64 + lane] = kreg[4 * t + ii];
@@ -325,16 +341,17 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
       acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, ka), __builtin_bit_cast(h8, qreg[kb]),
                                                    acc, 0, 0, 0);
     }
+    float mk[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (!PLAIN && a.mask && n16 < n_rep)
+      load_mask4(a.mask + (int64_t)seq * a.mask_seq_stride + ((int64_t)kvh * n_rep + n16) * a.mask_head_stride + tile_p0 +
+                     wrow0 + 16 * t + 4 * g, wrow0 + 16 * t + 4 * g, rows_here, mask_vec, mk);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int row = wrow0 + 16 * t + 4 * g + j;                      // accumulator row 4g + j of tile t
       if (PLAIN) {
         s[t][j] = acc[j];                                              // raw: the scale joins the exponent's fma
       } else {
-        float v = acc[j] * cs;                                         // log2 units
-        if (a.mask && row < rows_here && n16 < n_rep)
-          v += kLog2e * a.mask[(int64_t)seq * a.mask_seq_stride + ((int64_t)kvh * n_rep + n16) * a.mask_head_stride +
-                               tile_p0 + row];
+        const float v = __builtin_fmaf(mk[j], kLog2e, acc[j] * cs);    // log2 units
         s[t][j] = (row < rows_here) ? v : -INFINITY;
       }
     }

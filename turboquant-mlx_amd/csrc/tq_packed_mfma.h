@@ -246,6 +246,8 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
 
   // ---- K: scores ----------------------------------------------------------------------------------------
   float s[4][4];
+  const bool mask_vec = a.mask && ((reinterpret_cast<uintptr_t>(a.mask) & 15) == 0) && ((a.mask_seq_stride & 3) == 0) &&
+                        ((a.mask_head_stride & 3) == 0);      // uniform
   if (HAS_K) {
     u4 qreg[4], qlow[4];
 #pragma unroll
@@ -274,13 +276,14 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
       }
       const float4 kn4 = *reinterpret_cast<const float4*>(&kn_s[wave][16 * t + 4 * g]);
       const float knv[4] = {kn4.x, kn4.y, kn4.z, kn4.w};
+      float mk[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+      if (MODE == kFlash && a.mask && n16 < n_rep)
+        load_mask4(a.mask + (int64_t)seq * a.mask_seq_stride + ((int64_t)kvh * n_rep + n16) * a.mask_head_stride + tile_p0 +
+                       wrow0 + 16 * t + 4 * g, wrow0 + 16 * t + 4 * g, rows_here, mask_vec, mk);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int row = wrow0 + 16 * t + 4 * g + j;
-        float v = acc[j] * knv[j];
-        if (MODE == kFlash && a.mask && row < rows_here && n16 < n_rep)
-          v += kLog2e * a.mask[(int64_t)seq * a.mask_seq_stride + ((int64_t)kvh * n_rep + n16) * a.mask_head_stride +
-                      tile_p0 + row];
+        const float v = (MODE == kFlash) ? __builtin_fmaf(mk[j], kLog2e, acc[j] * knv[j]) : acc[j] * knv[j];
         s[t][j] = (row < rows_here) ? v : -INFINITY;
       }
     }
