@@ -378,9 +378,11 @@ __global__ __launch_bounds__(kBlock) void dequant128x3_kernel(const uint32_t* __
   __shared__ __align__(16) float sg_s[128];
   __shared__ __align__(8) float2 pair_s[64];
   __shared__ uint32_t words_s[kWavesPerBlock][kEncVecs * 13 + 3];
-  // 16-bit outputs leave through LDS: 16 rows of 256 bytes at a pitch of 320 (conflict-free 16-byte writes per
-  // lane and reads per row segment), so that every store instruction writes 1 KB of contiguous memory
-  __shared__ __align__(16) unsigned char orow_s[sizeof(TO) == 2 ? kWavesPerBlock : 1][sizeof(TO) == 2 ? kEncVecs * 320 : 16];
+  // Outputs leave through LDS: 16 rows of 256 (16-bit) or 512 (float32) bytes at a padded pitch (conflict-free
+  // 16-byte writes per lane and reads per row segment), so that every store instruction writes 1 KB of
+  // contiguous memory
+  constexpr int kPitch = sizeof(TO) == 2 ? 320 : 528;          // row of 256 / 512 bytes plus padding
+  __shared__ __align__(16) unsigned char orow_s[kWavesPerBlock][kEncVecs * kPitch];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -464,7 +466,6 @@ __global__ __launch_bounds__(kBlock) void dequant128x3_kernel(const uint32_t* __
       }
     }
     butterfly_4lane(xs, flip1, flip2);
-    TO* orow = out + ((int64_t)grp * rm.out_group_stride + rin + v) * 128 + 8 * ls;
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       float r[8];
@@ -480,8 +481,8 @@ __global__ __launch_bounds__(kBlock) void dequant128x3_kernel(const uint32_t* __
         a.z = __float_as_uint(r[2]) ^ sm[k][2]; a.w = __float_as_uint(r[3]) ^ sm[k][3];
         b.x = __float_as_uint(r[4]) ^ sm[k][4]; b.y = __float_as_uint(r[5]) ^ sm[k][5];
         b.z = __float_as_uint(r[6]) ^ sm[k][6]; b.w = __float_as_uint(r[7]) ^ sm[k][7];
-        *reinterpret_cast<uint4*>(orow + 32 * k) = a;
-        *reinterpret_cast<uint4*>(orow + 32 * k + 4) = b;
+        *reinterpret_cast<uint4*>(&orow_s[wave][v * kPitch + 128 * k + 32 * ls]) = a;
+        *reinterpret_cast<uint4*>(&orow_s[wave][v * kPitch + 128 * k + 32 * ls + 16]) = b;
       } else {
         uint32_t w[4];
 #pragma unroll
@@ -496,15 +497,18 @@ __global__ __launch_bounds__(kBlock) void dequant128x3_kernel(const uint32_t* __
           }
           w[jp] = (lo | (hi << 16)) ^ ((sm[k][2 * jp] >> 16) | sm[k][2 * jp + 1]);
         }
-        *reinterpret_cast<uint4*>(&orow_s[wave][v * 320 + 64 * k + 16 * ls]) = make_uint4(w[0], w[1], w[2], w[3]);
+        *reinterpret_cast<uint4*>(&orow_s[wave][v * kPitch + 64 * k + 16 * ls]) = make_uint4(w[0], w[1], w[2], w[3]);
       }
     }
-    if (sizeof(TO) == 2) {
+    {
       unsigned char* oblock = reinterpret_cast<unsigned char*>(out + ((int64_t)grp * rm.out_group_stride + rin) * 128);
+      constexpr int kPiecesPerRow = 8 * (int)sizeof(TO);           // 16-byte pieces in a row: 16 or 32
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        *reinterpret_cast<uint4*>(oblock + (i * 64 + lane) * 16) =
-            *reinterpret_cast<const uint4*>(&orow_s[wave][(4 * i + (lane >> 4)) * 320 + (lane & 15) * 16]);
+      for (int i = 0; i < (int)(2 * sizeof(TO)); ++i) {            // 4 or 8 KB per pass
+        const int piece = i * 64 + lane;
+        *reinterpret_cast<uint4*>(oblock + piece * 16) =
+            *reinterpret_cast<const uint4*>(&orow_s[wave][(piece / kPiecesPerRow) * kPitch + (piece % kPiecesPerRow) * 16]);
+      }
     }
     row0 += kEncVecs;
     rin = nrin;

@@ -59,6 +59,8 @@ def bench_encode(iters, dev):
         p, n = tqhip.fused_quantize(xs[0], signs, bd, 128, 3)
         fns = [(lambda: tqhip.dequant_fp16(p, n, cb, signs, 128, 3))]
         report(f"dequant_fp16 d=128 3-bit, {n_vecs} vectors (cache-warm)", timeit(fns, iters), n_vecs * (56 + 256))
+        fns = [(lambda: tqhip.packed_dequantize(p, n, cb, signs, 128, 3))]
+        report(f"packed_dequantize (float32 out), {n_vecs} vectors", timeit(fns, iters), n_vecs * (56 + 512))
 
 
 def packed_sets(n_kv, T, dev, n_sets, seed):
