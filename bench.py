@@ -37,9 +37,9 @@ N_SETS = 10
 # `python bench.py --steps 60 --warmup 6 --no-cpu --no-graph` (FETCH_SIZE, then WRITE_SIZE), each
 # scaled by what the same counter reads for `python bench.py --calibrate-copy --steps 40`, a plain
 # copy of ALGO_BYTES bytes (FETCH_SIZE reads 19986.7 for 39950 KiB -> factor 1.9988; WRITE_SIZE
-# reads 39950.0 -> factor 1.0000).  Tile pass: FETCH_SIZE 20059.3 -> 40095 KiB, WRITE_SIZE 916.0
+# reads 39950.0 -> factor 1.0000).  Tile pass: FETCH_SIZE 20059.2 -> 40095 KiB, WRITE_SIZE 916.0
 # -> 916 KiB.  Summary: profiles/vonly_decode_c2_pmc_traffic.md.
-MEASURED_TRAFFIC_BYTES = 41995395           # (20059.3 * 39950.0 / 19986.7 + 916.0) KiB, unrounded inputs
+MEASURED_TRAFFIC_BYTES = 41995386           # (20059.2 * 39950.0 / 19986.7 + 916.0) KiB, unrounded inputs
 
 
 def make_sets(torch, tqhip, dev):
