@@ -172,22 +172,46 @@ __global__ __launch_bounds__(kThreads) void dense_scores_kernel(const QT* __rest
 }
 
 // ---------------------------------------------------------------- row softmax
+// grid = (n_rows, n_chunks).  Every workgroup takes the maximum and the sum of exponentials over the WHOLE row
+// (two sweeps; with several chunks per row the row comes from L2 for all but the first reader) and then
+// writes the weights of its own chunk, so a few long rows still fill the chip with one launch and without
+// scratch memory.  16-byte accesses where the row is aligned.
 __global__ __launch_bounds__(kThreads) void softmax_rows_kernel(const float* __restrict__ scores,
                                                                 const float* __restrict__ mask,
                                                                 int64_t mask_row_stride,
                                                                 float* __restrict__ weights, int64_t seq_len,
-                                                                float scale) {
+                                                                float scale, int64_t chunk_len) {
   __shared__ float red[kWaves];
   const int64_t row = blockIdx.x;
   const float* s = scores + row * seq_len;
   const float* mk = mask ? mask + row * mask_row_stride : nullptr;
   float* w = weights + row * seq_len;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  float m = -INFINITY;
-  for (int64_t p = threadIdx.x; p < seq_len; p += kThreads) {
+  const bool vec = ((seq_len & 3) == 0) && ((reinterpret_cast<uintptr_t>(scores) & 15) == 0) &&
+                   ((reinterpret_cast<uintptr_t>(weights) & 15) == 0) && ((chunk_len & 3) == 0) &&
+                   (!mask || (((reinterpret_cast<uintptr_t>(mask) & 15) == 0) && ((mask_row_stride & 3) == 0)));
+  auto logits4 = [&](int64_t p, float (&v)[4]) {                      // four consecutive logits (vec only)
+    const float4 x = *reinterpret_cast<const float4*>(s + p);
+    v[0] = x.x * scale; v[1] = x.y * scale; v[2] = x.z * scale; v[3] = x.w * scale;
+    if (mk) {
+      const float4 m4 = *reinterpret_cast<const float4*>(mk + p);
+      v[0] += m4.x; v[1] += m4.y; v[2] += m4.z; v[3] += m4.w;
+    }
+  };
+  auto logit = [&](int64_t p) {
     float v = s[p] * scale;
     if (mk) v += mk[p];
-    m = fmaxf(m, v);
+    return v;
+  };
+  float m = -INFINITY;
+  if (vec) {
+    for (int64_t p = 4 * (int64_t)threadIdx.x; p < seq_len; p += 4 * kThreads) {
+      float v[4];
+      logits4(p, v);
+      m = fmaxf(m, fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])));
+    }
+  } else {
+    for (int64_t p = threadIdx.x; p < seq_len; p += kThreads) m = fmaxf(m, logit(p));
   }
   m = wave_max(m);
   if (lane == 0) red[wave] = m;
@@ -196,19 +220,30 @@ __global__ __launch_bounds__(kThreads) void softmax_rows_kernel(const float* __r
   __syncthreads();
   if (m == -INFINITY) m = 0.0f;
   float l = 0.0f;
-  for (int64_t p = threadIdx.x; p < seq_len; p += kThreads) {
-    float v = s[p] * scale;
-    if (mk) v += mk[p];
-    l += expf(v - m);
+  if (vec) {
+    for (int64_t p = 4 * (int64_t)threadIdx.x; p < seq_len; p += 4 * kThreads) {
+      float v[4];
+      logits4(p, v);
+      l += (expf(v[0] - m) + expf(v[1] - m)) + (expf(v[2] - m) + expf(v[3] - m));
+    }
+  } else {
+    for (int64_t p = threadIdx.x; p < seq_len; p += kThreads) l += expf(logit(p) - m);
   }
   l = wave_sum(l);
   if (lane == 0) red[wave] = l;
   __syncthreads();
   l = (red[0] + red[1]) + (red[2] + red[3]);
-  for (int64_t p = threadIdx.x; p < seq_len; p += kThreads) {
-    float v = s[p] * scale;
-    if (mk) v += mk[p];
-    w[p] = expf(v - m) / l;
+  const int64_t p_lo = (int64_t)blockIdx.y * chunk_len;
+  const int64_t p_hi = p_lo + chunk_len < seq_len ? p_lo + chunk_len : seq_len;
+  if (vec) {
+    for (int64_t p = p_lo + 4 * (int64_t)threadIdx.x; p < p_hi; p += 4 * kThreads) {
+      float v[4];
+      logits4(p, v);
+      *reinterpret_cast<float4*>(w + p) = make_float4(expf(v[0] - m) / l, expf(v[1] - m) / l, expf(v[2] - m) / l,
+                                                      expf(v[3] - m) / l);
+    }
+  } else {
+    for (int64_t p = p_lo + threadIdx.x; p < p_hi; p += kThreads) w[p] = expf(logit(p) - m) / l;
   }
 }
 
@@ -768,8 +803,15 @@ extern "C" int tq_softmax_rows(const float* scores, const float* mask, int64_t m
   if (n_rows == 0 || seq_len == 0) return TQ_OK;
   if (!scores || !weights) return tq::fail(TQ_ERR_NULL, "tq_softmax_rows: null pointer");
   if (n_rows > 0x7FFFFFFF) return tq::fail(TQ_ERR_ARG, "tq_softmax_rows: too many rows");
-  softmax_rows_kernel<<<(int)n_rows, kThreads, 0, (hipStream_t)stream_>>>(scores, mask, mask_row_stride, weights,
-                                                                         seq_len, scale);
+  // chunks per row: enough workgroups to fill the chip when the rows are few and long (at least 4096 positions each)
+  int64_t n_chunks = 512 / n_rows;
+  if (n_chunks > seq_len / 4096) n_chunks = seq_len / 4096;
+  if (n_chunks < 1) n_chunks = 1;
+  int64_t chunk_len = (seq_len + n_chunks - 1) / n_chunks;
+  chunk_len = (chunk_len + 3) & ~(int64_t)3;
+  n_chunks = (seq_len + chunk_len - 1) / chunk_len;
+  softmax_rows_kernel<<<dim3((unsigned)n_rows, (unsigned)n_chunks), kThreads, 0, (hipStream_t)stream_>>>(
+      scores, mask, mask_row_stride, weights, seq_len, scale, chunk_len);
   TQ_CHECK_LAUNCH("tq_softmax_rows launch");
   return TQ_OK;
 }
