@@ -1314,3 +1314,25 @@ def test_fully_masked_rows_yield_zeros(tq):
         want_f = o.turboquant_attention_single(q[0, 4:8].astype(F32), kp[1:], kn[1:], vp[1:], vn[1:], c, ks, c, vs,
                                                D, bits, sc, mask=mask[0, 4:8])
         close(f[4:8], want_f)
+
+
+@pytest.mark.parametrize("n_rows,T,mask_kind", [(1, 1, "none"), (3, 7, "row"), (28, 4096, "shared"), (28, 32770, "none"),
+                                                (2, 65536, "row"), (7, 16384, "shared"), (300, 513, "row"), (28, 32768, "none")])
+def test_softmax_rows_shapes(tq, n_rows, T, mask_kind):
+    """softmax_rows (fused_attention.py:78-94) on few long rows (several workgroups per row), many short rows,
+    lengths that are not a multiple of 4, with a shared or a per-row additive mask: against float64 numpy."""
+    rng = np.random.default_rng(n_rows * 1000 + T)
+    x = (rng.standard_normal((n_rows, T)) * 3).astype(F32)
+    scale = 0.37
+    mask = None
+    if mask_kind != "none":
+        shape = (T,) if mask_kind == "shared" else (n_rows, T)
+        mask = np.where(rng.random(shape) < 0.3, -np.inf, 0.0).astype(F32)
+        mask[..., 0] = 0.0
+    got = host(tq.softmax_rows(dev(x), scale, None if mask is None else dev(mask)))
+    z = x.astype(np.float64) * np.float64(F32(scale)) + (0.0 if mask is None else mask.astype(np.float64))
+    z = z - z.max(axis=-1, keepdims=True)
+    want = np.exp(z) / np.exp(z).sum(axis=-1, keepdims=True)
+    assert got.shape == want.shape
+    assert np.abs(got - want).max() <= 1e-7 + 2e-6 * want.max()
+    assert np.abs(got.sum(axis=-1) - 1.0).max() < 1e-5
