@@ -247,6 +247,26 @@ int tq_vonly_decode_attn_phases(const void* q, int q_dtype, const void* k_f16,
                                 const tq_decode_shape* shape /* host */, int phases, tq_stream_t stream);
 
 /*
+ * Decode attention for a V-only cache with the sparse-V threshold: weights of the softmax over the whole
+ * sequence that are below `threshold` contribute nothing,
+ *   w_p = softmax_p(<q,K_p>*attn_scale + mask);   out = butterfly(sum_{p: !(w_p < threshold)} w_p * v_norm * c_v[idx_v]) * v_signs / dim,
+ * i.e. dense-K scores -> softmax -> sparse_v_matvec(threshold) of hybrid_attention.py:52-88 (threshold rule of
+ * sparse_v.py:59-65, 163-164; the call with sparse_v_threshold of fused_attention.py:109-121) in one call:
+ * a scores pass, a weights-and-values pass and the merge pass, with the scores of the step held in `workspace`
+ * (tq_vonly_sparse_workspace_bytes) instead of three tensors of the caller.  Arguments as tq_vonly_decode_attn;
+ * threshold >= 0 (0 = dense: every position contributes).  Rows whose positions are all masked out yield zeros.
+ * Matrix-core shape only: dim 128, 3-bit values, n_rep <= 16, non-empty cache (TQ_ERR_UNSUPPORTED otherwise:
+ * compose tq_dense_qk_scores, tq_softmax_rows and tq_sparse_v_matvec for those).
+ */
+int tq_vonly_sparse_decode_attn(const void* q, int q_dtype, const void* k_f16,
+                                const uint32_t* v_packed, const float* v_norms,
+                                const float* v_centroids, const float* v_signs, float threshold,
+                                void* out, void* workspace, size_t workspace_bytes,
+                                const tq_decode_shape* shape /* host */, tq_stream_t stream);
+
+size_t tq_vonly_sparse_workspace_bytes(int n_seq, int n_q_heads, int64_t max_seq_len);
+
+/*
  * Bytes of workspace the op needs for this shape (host computation, no GPU call).  The workspace
  * holds per-tile partial results between the two passes of a call; its contents need not be
  * preserved or cleared between calls.  Calls that share a workspace must be ordered (same stream);

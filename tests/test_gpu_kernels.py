@@ -1336,3 +1336,121 @@ def test_softmax_rows_shapes(tq, n_rows, T, mask_kind):
     assert got.shape == want.shape
     assert np.abs(got - want).max() <= 1e-7 + 2e-6 * want.max()
     assert np.abs(got.sum(axis=-1) - 1.0).max() < 1e-5
+
+
+# ------------------------------------------------------------------ thresholded V-only decode in one call
+
+@pytest.mark.parametrize("n_seq,n_kv,n_rep,T,thr,qdt,mask_kind", [
+    (1, 4, 7, 1500, 1e-5, np.float16, "none"), (2, 2, 4, 513, 1e-3, np.float32, "seq"),
+    (1, 8, 1, 2048, 1e-4, np.float16, "head"), (3, 1, 16, 77, 1e-2, np.float16, "none"),
+    (1, 4, 7, 4099, 1e-5, np.float32, "head"), (2, 3, 5, 1, 1e-5, np.float16, "none")])
+def test_vonly_sparse_decode_matches_oracle(tq, n_seq, n_kv, n_rep, T, thr, qdt, mask_kind):
+    """tq_vonly_sparse_decode_attn (scores pass, weights-and-values pass, merge) against the oracle's
+    dense scores -> softmax -> thresholded value sum, cache layout with an allocation longer than the
+    valid length."""
+    rng = np.random.default_rng(7 * T + n_rep)
+    D, bits, sc = 128, 3, 1 / math.sqrt(128)
+    n_q = n_kv * n_rep
+    T_alloc = T + 37
+    c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, n_seq * n_kv, T_alloc, D, bits)
+    K, vp, vn = (a.reshape(n_seq, n_kv, *a.shape[1:]) for a in (K, vp, vn))
+    q = rng.standard_normal((n_seq, n_q, D)).astype(qdt)
+    mask = _draw_mask(rng, mask_kind, n_seq, n_q, T)
+    kw = {} if mask is None else dict(mask=dev(mask))
+    got = host(tq.vonly_decode(dev(q), dev(K), dev(vp), dev(vn), c, dev(vs), D, bits, sc, n_rep=n_rep, seq_len=T,
+                               sparse_v_threshold=thr, **kw))
+    dropped = 0
+    for i in range(n_seq):
+        mi = None if mask is None else np.broadcast_to(mask[i], (n_q, T))
+        want = o.vonly_decode_attention(q[i], K[i, :, :T], vp[i, :, :T], vn[i, :, :T], c, vs, D, bits, sc,
+                                        threshold=thr, mask=mi)
+        dense = o.vonly_decode_attention(q[i], K[i, :, :T], vp[i, :, :T], vn[i, :, :T], c, vs, D, bits, sc, mask=mi)
+        dropped += int(np.abs(want - dense).max() > 0)
+        close(got[i], want)
+    if T >= 500:
+        assert dropped > 0                         # the threshold did remove something in these cases
+
+
+def test_vonly_sparse_decode_ragged_batch_and_dtypes(tq):
+    """Ragged batch (sequence offsets into [n_kv, sum(L), *] tensors, lengths that end inside a tile and inside
+    a wave's rows), bf16 queries and fp16 output."""
+    rng = np.random.default_rng(401)
+    n_kv, n_rep, D, bits, sc, thr = 4, 7, 128, 3, 1 / math.sqrt(128), 1e-4
+    lens = np.array([1300, 1, 512, 65, 2049])
+    offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, n_kv, int(offs[-1]), D, bits)
+    qt = torch.from_numpy(rng.standard_normal((len(lens), n_kv * n_rep, D)).astype(F32)).to(torch.bfloat16)
+    got = tq.vonly_decode(qt.cuda(), dev(K), dev(vp), dev(vn), c, dev(vs), D, bits, sc, n_rep=n_rep,
+                          seq_offsets=dev(offs), max_seq_len=int(lens.max()), out_dtype=torch.float16,
+                          sparse_v_threshold=thr)
+    assert got.dtype == torch.float16
+    got = host(got.float())
+    for i in range(len(lens)):
+        a, e = offs[i], offs[i + 1]
+        want = o.vonly_decode_attention(qt[i].float().numpy(), K[:, a:e], vp[:, a:e], vn[:, a:e], c, vs, D, bits, sc,
+                                        threshold=thr)
+        close(got[i], want, rel=3e-3, abs_=2e-3)           # + fp16 rounding of the output
+
+
+def test_vonly_sparse_decode_threshold_limits(tq):
+    """A threshold above every weight drops every position (exact zeros, sparse_v.py:59-65); a threshold below
+    every representable weight changes nothing against the dense fused step; a fully masked head yields zeros."""
+    rng = np.random.default_rng(402)
+    n_kv, n_rep, T, D, bits, sc = 2, 4, 900, 128, 3, 1 / math.sqrt(128)
+    c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, n_kv, T, D, bits)
+    q = rng.standard_normal((1, n_kv * n_rep, D)).astype(np.float16)
+    args = (dev(q), dev(K), dev(vp), dev(vn), c, dev(vs), D, bits, sc)
+    none_left = host(tq.vonly_decode(*args, n_rep=n_rep, sparse_v_threshold=2.0))
+    assert (none_left == 0).all()
+    all_kept = host(tq.vonly_decode(*args, n_rep=n_rep, sparse_v_threshold=1e-37))
+    dense = host(tq.vonly_decode(*args, n_rep=n_rep))
+    close(all_kept, dense, rel=1e-3, abs_=2e-4)
+    close(all_kept[0], o.vonly_decode_attention(q[0], K, vp, vn, c, vs, D, bits, sc))
+    mask = np.zeros((1, n_kv * n_rep, T), F32)
+    mask[0, 2, :] = -np.inf
+    masked = host(tq.vonly_decode(*args, n_rep=n_rep, mask=dev(mask), sparse_v_threshold=1e-5))[0]
+    assert (masked[2] == 0).all()
+    close(masked[4:], o.vonly_decode_attention(q[0, 4:], K[1:], vp[1:], vn[1:], c, vs, D, bits, sc, threshold=1e-5))
+
+
+def test_vonly_sparse_decode_rejects_other_shapes(tq):
+    """dim 64 / 4-bit caches have no one-call thresholded step: the wrapper says which ops to compose."""
+    rng = np.random.default_rng(403)
+    c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, 2, 64, 64, 4)
+    q = rng.standard_normal((1, 2, 64)).astype(np.float16)
+    with pytest.raises(ValueError, match="compose dense_qk_scores"):
+        tq.vonly_decode(dev(q), dev(K), dev(vp), dev(vn), c, dev(vs), 64, 4, 0.125, n_rep=1, sparse_v_threshold=1e-5)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_decode_sweep_vonly_sparse(tq, seed):
+    """The thresholded step on the drawn decode shapes (ragged and cache-layout batches, masks, query dtypes)."""
+    rng, n_kv, n_rep, ragged, n_seq, lens, mask_kind, qdt = _draw_decode_case(500 + seed)
+    D, bits, sc = 128, 3, 1 / math.sqrt(128)
+    n_q = n_kv * n_rep
+    thr = float(rng.choice([1e-5, 1e-4, 1e-3]))
+    print(f"seed {seed}: n_kv {n_kv} n_rep {n_rep} ragged {ragged} lens {lens.tolist()} mask {mask_kind} "
+          f"q {np.dtype(qdt).name} thr {thr:g}", flush=True)
+    q = rng.standard_normal((n_seq, n_q, D)).astype(qdt)
+    if ragged:
+        offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, n_kv, int(offs[-1]), D, bits)
+        kw = dict(seq_offsets=dev(offs), max_seq_len=int(lens.max()))
+        per_seq = [tuple(a[:, offs[i]:offs[i + 1]] for a in (K, vp, vn)) for i in range(n_seq)]
+        mask = None
+    else:
+        T = int(lens[0])
+        T_alloc = T + int(rng.integers(0, 70))
+        c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, n_seq * n_kv, T_alloc, D, bits)
+        K, vp, vn = (a.reshape(n_seq, n_kv, *a.shape[1:]) for a in (K, vp, vn))
+        kw = dict(seq_len=T)
+        per_seq = [tuple(a[i, :, :T] for a in (K, vp, vn)) for i in range(n_seq)]
+        mask = _draw_mask(rng, mask_kind, n_seq, n_q, T)
+        if mask is not None:
+            kw["mask"] = dev(mask)
+    got = host(tq.vonly_decode(dev(q), dev(K), dev(vp), dev(vn), c, dev(vs), D, bits, sc, n_rep=n_rep,
+                               sparse_v_threshold=thr, **kw))
+    for i in range(n_seq):
+        Ki, vpi, vni = per_seq[i]
+        mi = None if mask is None else np.broadcast_to(mask[i], (n_q, mask.shape[-1]))
+        close(got[i], o.vonly_decode_attention(q[i], Ki, vpi, vni, c, vs, D, bits, sc, threshold=thr, mask=mi))

@@ -676,6 +676,7 @@ int launch_packed_mfma(const float* q_rot_or_weights, const uint32_t* k_packed, 
   a.n_kv = sh.n_kv_heads; a.n_rep = sh.n_rep; a.n_tiles_max = n_tiles;
   a.score_scale = sh.attn_scale / (float)sh.dim;
   a.threshold = threshold;
+  a.w_stride = sh.seq_len;                               // given weights: one sequence, rows of seq_len floats
   Codebook kcb, vcb;
   fill_codebook(kcb, nullptr, sh.bits);
   if (MODE != tqm::kWeights) a.score_scale *= tq::fill_codebook_fp16(kcb, k_centroids, sh.bits);
@@ -703,6 +704,74 @@ int launch_packed_mfma(const float* q_rot_or_weights, const uint32_t* k_packed, 
   else if (sh.out_dtype == TQ_BF16) { LAUNCH_MERGE_P(__hip_bfloat16); }
   else { LAUNCH_MERGE_P(float); }
 #undef LAUNCH_MERGE_P
+  TQ_CHECK_LAUNCH(who);
+  return TQ_OK;
+}
+
+// Thresholded V-only decode on the matrix cores: scores pass (fp16 keys -> scores in log2 units + per-tile
+// softmax statistics), weights pass (2^(s - M) / L, weights below the threshold dropped, value sums per tile),
+// merge pass.  Workspace: scores | statistics | partial sums | their (0, l) pairs.
+size_t vonly_sparse_ws_bytes(int n_seq, int n_q, int64_t seq_len) {
+  const int64_t t_pad = (seq_len + 3) & ~(int64_t)3;
+  const int64_t n_tiles = (seq_len + tqm::kTilePos - 1) / tqm::kTilePos;
+  return ((size_t)n_seq * n_q * t_pad + (size_t)n_seq * n_q * n_tiles * (tqm::kD + 4)) * sizeof(float);
+}
+
+int launch_vonly_sparse(const void* q, int q_dtype, const void* k_f16, const uint32_t* v_packed, const float* v_norms,
+                        const float* v_centroids, const float* v_signs, float threshold, void* out, void* workspace,
+                        size_t workspace_bytes, const tq_decode_shape& sh, hipStream_t stream) {
+  const char* who = "tq_vonly_sparse_decode_attn";
+  const int n_q = sh.n_kv_heads * sh.n_rep;
+  const int64_t t_pad = (sh.seq_len + 3) & ~(int64_t)3;
+  const int n_tiles = (int)((sh.seq_len + tqm::kTilePos - 1) / tqm::kTilePos);
+  const size_t need = vonly_sparse_ws_bytes(sh.n_seq, n_q, sh.seq_len);
+  if (!workspace || workspace_bytes < need)
+    return tq::fail(TQ_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, need, workspace_bytes);
+  if (!tq::aligned(workspace, 16)) return tq::fail(TQ_ERR_ALIGN, "%s: workspace must be 16-byte aligned", who);
+  float* scores = (float*)workspace;                                    // [n_seq * n_q, t_pad]
+  float* stats = scores + (size_t)sh.n_seq * n_q * t_pad;               // [n_seq * n_kv, n_tiles, n_rep, 2]
+  float* ws_S = stats + (size_t)sh.n_seq * n_q * n_tiles * 2;           // [n_seq * n_kv, n_tiles, n_rep, 128]
+  float* ws_ml = ws_S + (size_t)sh.n_seq * n_q * n_tiles * tqm::kD;
+
+  tqm::MfmaArgs m{};
+  m.q = (const __half*)q; m.k = (const __half*)k_f16; m.q_bf16 = q_dtype == TQ_BF16 ? 1 : 0;
+  m.seq_offsets = sh.seq_offsets; m.mask = sh.mask;
+  m.ws_ml = stats; m.scores = scores; m.scores_stride = t_pad;
+  m.seq_len = sh.seq_len;
+  m.k_seq_stride = sh.k_seq_stride; m.k_head_stride = sh.k_head_stride;
+  m.mask_seq_stride = sh.mask_seq_stride; m.mask_head_stride = sh.mask_head_stride;
+  m.n_kv = sh.n_kv_heads; m.n_rep = sh.n_rep; m.n_tiles_max = n_tiles;
+  m.attn_scale = sh.attn_scale;
+  dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
+  if (q_dtype == TQ_F32) tqm::vonly_scores_kernel<true><<<grid, tqm::kMfmaThreads, 0, stream>>>(m);
+  else tqm::vonly_scores_kernel<false><<<grid, tqm::kMfmaThreads, 0, stream>>>(m);
+  TQ_CHECK_LAUNCH(who);
+
+  tqm::PackedArgs a{};
+  a.weights = scores; a.stats = stats; a.w_stride = t_pad;
+  a.v_packed = v_packed; a.v_norms = v_norms;
+  a.seq_offsets = sh.seq_offsets;
+  a.ws_S = ws_S; a.ws_ml = ws_ml;
+  a.seq_len = sh.seq_len;
+  a.v_seq_stride = sh.v_seq_stride; a.v_head_stride = sh.v_head_stride;
+  a.vn_seq_stride = sh.vn_seq_stride; a.vn_head_stride = sh.vn_head_stride;
+  a.n_kv = sh.n_kv_heads; a.n_rep = sh.n_rep; a.n_tiles_max = n_tiles;
+  a.threshold = threshold;
+  Codebook kcb, vcb;
+  fill_codebook(kcb, nullptr, sh.bits);
+  a.v_unscale = tq::fill_codebook_fp16(vcb, v_centroids, sh.bits);
+  tqm::packed_tile_mfma_kernel<tqm::kSoftWeights><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, kcb, vcb);
+  TQ_CHECK_LAUNCH(who);
+
+  dim3 mgrid(n_q, sh.n_seq);
+  const float inv_dim = 1.0f / (float)sh.dim;
+#define LAUNCH_MERGE_S(TO)                                                                                  \
+  tqm::decode_merge_rows_kernel<TO, false><<<mgrid, tqm::kMergeThreads, 0, stream>>>(                         \
+      ws_S, ws_ml, sh.seq_offsets, sh.seq_len, n_tiles, sh.n_kv_heads, sh.n_rep, v_signs, inv_dim, (TO*)out, tqm::kTilePos)
+  if (sh.out_dtype == TQ_F16) { LAUNCH_MERGE_S(__half); }
+  else if (sh.out_dtype == TQ_BF16) { LAUNCH_MERGE_S(__hip_bfloat16); }
+  else { LAUNCH_MERGE_S(float); }
+#undef LAUNCH_MERGE_S
   TQ_CHECK_LAUNCH(who);
   return TQ_OK;
 }
@@ -892,4 +961,28 @@ extern "C" int tq_vonly_decode_attn(const void* q, int q_dtype, const void* k_f1
                                     const tq_decode_shape* shape, tq_stream_t stream_) {
   return tq_vonly_decode_attn_phases(q, q_dtype, k_f16, v_packed, v_norms, v_centroids, v_signs, out, workspace,
                                      workspace_bytes, shape, 3, stream_);
+}
+
+extern "C" size_t tq_vonly_sparse_workspace_bytes(int n_seq, int n_q_heads, int64_t max_seq_len) {
+  if (n_seq < 1 || n_q_heads < 1 || max_seq_len < 0) return 0;
+  return vonly_sparse_ws_bytes(n_seq, n_q_heads, max_seq_len);
+}
+
+extern "C" int tq_vonly_sparse_decode_attn(const void* q, int q_dtype, const void* k_f16, const uint32_t* v_packed,
+                                           const float* v_norms, const float* v_centroids, const float* v_signs,
+                                           float threshold, void* out, void* workspace, size_t workspace_bytes,
+                                           const tq_decode_shape* shape, tq_stream_t stream_) {
+  const char* who = "tq_vonly_sparse_decode_attn";
+  if (int rc = check_shape(shape, who, 256)) return rc;
+  if (tq::check_dtype(q_dtype)) return tq::fail(TQ_ERR_DTYPE, "%s: unknown q_dtype %d", who, q_dtype);
+  if (!q || !v_centroids || !v_signs || !out) return tq::fail(TQ_ERR_NULL, "%s: null pointer", who);
+  if (shape->seq_len > 0 && (!k_f16 || !v_packed || !v_norms)) return tq::fail(TQ_ERR_NULL, "%s: null pointer", who);
+  if (!tq::aligned(k_f16, 16)) return tq::fail(TQ_ERR_ALIGN, "%s: k must be 16-byte aligned", who);
+  if (!(threshold >= 0.0f)) return tq::fail(TQ_ERR_ARG, "%s: threshold must be >= 0", who);
+  if (!(shape->dim == 128 && shape->bits == 3 && shape->n_rep <= tqm::kHeadsMax && shape->seq_len > 0 &&
+        tq::aligned(q, q_dtype == TQ_F32 ? 8 : 4)))
+    return tq::fail(TQ_ERR_UNSUPPORTED, "%s: dim 128, 3-bit values, n_rep <= 16 and a non-empty cache only "
+                                        "(compose tq_dense_qk_scores, tq_softmax_rows and tq_sparse_v_matvec otherwise)", who);
+  return launch_vonly_sparse(q, q_dtype, k_f16, v_packed, v_norms, v_centroids, v_signs, threshold, out, workspace,
+                             workspace_bytes, *shape, (hipStream_t)stream_);
 }

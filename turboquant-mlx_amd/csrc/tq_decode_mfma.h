@@ -72,6 +72,8 @@ struct MfmaArgs {
   float attn_scale;
   float v_unscale;            // 1 / the scale the value table was multiplied by on the host
   int32_t q_bf16;
+  float* scores;              // vonly_scores_kernel: [n_seq * n_q, scores_stride] f32, log2 units
+  int64_t scores_stride;      // floats per score row (a multiple of 4)
 #ifdef TQ_TRACE
   unsigned long long* trace;
 #endif
@@ -485,6 +487,170 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
     pml[2 * h + 1] = L;
   }
   TQ_STAMP(10);
+}
+
+// Scores pass of the thresholded decode step (weights below a threshold are dropped, and the threshold
+// applies to the FINAL softmax weights, so the scores of the whole sequence must exist before any value
+// is summed).  Same tiling and K path as the kernel above, no V work: a workgroup writes the scaled
+// (and masked) scores of its 512 positions in log2 units, s = (q . k) * attn_scale * log2 e + mask * log2 e,
+// to a.scores and one (maximum, sum of 2^(s - maximum)) pair per query head to a.ws_ml, from which the
+// second pass derives the softmax denominator of the sequence.
+// grid = (n_tiles_max, n_kv, n_seq), 512 threads.
+template <bool QF32>
+__global__ __launch_bounds__(kMfmaThreads) void vonly_scores_kernel(MfmaArgs a) {
+  __shared__ __align__(16) unsigned char big_s[32768];        // per-wave 4 KB: K tiles, then the score block
+  __shared__ __align__(16) uint32_t q_s[kHeadsMax][kD / 2];
+  __shared__ __align__(16) uint32_t ql_s[QF32 ? kHeadsMax : 1][kD / 2];
+  __shared__ float m_s[kWaves][kHeadsMax], l_s[kWaves][kHeadsMax];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int n16 = lane & 15, g = lane >> 4;
+  const int tile = blockIdx.x, kvh = blockIdx.y, seq = blockIdx.z;
+  const int n_rep = a.n_rep;
+  const int n_q = a.n_kv * n_rep;
+  const int64_t q_row0 = (int64_t)seq * n_q + (int64_t)kvh * n_rep;
+
+  int64_t first = 0, len = a.seq_len;
+  if (a.seq_offsets) {
+    first = a.seq_offsets[seq];
+    len = (int64_t)a.seq_offsets[seq + 1] - first;
+  }
+  const int64_t tile_p0 = (int64_t)tile * kTilePos;
+  if (tile_p0 >= len) return;                          // the second pass never reads this tile
+  const int rows_here = (int)min((int64_t)kTilePos, len - tile_p0);
+  const int last_row = rows_here - 1;
+  const int wrow0 = wave * kWavePos;
+
+  uint32_t my_q[2], my_ql[2] = {0u, 0u};
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int w = tid + i * kMfmaThreads;
+    if (QF32) {
+      const float2 f = (w < n_rep * (kD / 2)) ? reinterpret_cast<const float2*>(reinterpret_cast<const float*>(a.q) + q_row0 * kD)[w]
+                                              : make_float2(0.f, 0.f);
+      const __half2 h = __floats2half2_rn(f.x, f.y);
+      const float2 back = __half22float2(h);
+      my_q[i] = *reinterpret_cast<const uint32_t*>(&h);
+      my_ql[i] = pack_h2(f.x - back.x, f.y - back.y);
+    } else {
+      my_q[i] = (w < n_rep * (kD / 2)) ? reinterpret_cast<const uint32_t*>(a.q + q_row0 * kD)[w] : 0u;
+      if (a.q_bf16) my_q[i] = pack_h2(__uint_as_float(my_q[i] << 16), __uint_as_float(my_q[i] & 0xFFFF0000u));
+    }
+  }
+  // K: instruction i reads rows 4i .. 4i+3 of the wave (1 KB contiguous); lane L takes 16-byte piece
+  // (L & 15) ^ (row & 7) of row 4i + (L >> 4); rows past the end of the sequence repeat the last valid row
+  const char* kbase = reinterpret_cast<const char*>(
+      a.k + ((int64_t)seq * a.k_seq_stride + (int64_t)kvh * a.k_head_stride + first + tile_p0) * kD);
+  u4 kreg[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int r = 4 * i + (lane >> 4);
+    const int piece = (lane & 15) ^ (r & 7);
+    int row = wrow0 + r;
+    row = row < last_row ? row : last_row;
+    kreg[i] = *reinterpret_cast<const u4*>(kbase + (uint32_t)((row * 16 + piece) * 16));
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    (&q_s[0][0])[tid + i * kMfmaThreads] = my_q[i];
+    if (QF32) (&ql_s[0][0])[tid + i * kMfmaThreads] = my_ql[i];
+  }
+  __syncthreads();
+
+  u4 qreg[4], qlow[4];
+#pragma unroll
+  for (int kb = 0; kb < 4; ++kb) {
+    qreg[kb] = *reinterpret_cast<const u4*>(&q_s[n16][(4 * kb + g) * 4]);
+    if (QF32) qlow[kb] = *reinterpret_cast<const u4*>(&ql_s[n16][(4 * kb + g) * 4]);
+  }
+  u4* kst = reinterpret_cast<u4*>(big_s) + wave * 256;          // this wave's 256 pieces of 16 bytes
+  const float cs = a.attn_scale * kLog2e;
+  const bool mask_vec = a.mask && ((reinterpret_cast<uintptr_t>(a.mask) & 15) == 0) && ((a.mask_seq_stride & 3) == 0) &&
+                        ((a.mask_head_stride & 3) == 0);      // uniform
+  float s[4][4];                                               // positions 16t + 4g + j of head n16
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+#pragma unroll
+    for (int ii = 0; ii < 4; ++ii) kst[ii * 64 + lane] = kreg[4 * t + ii];
+    f4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+      const u4 ka = kst[n16 * 16 + ((4 * kb + g) ^ (n16 & 7))];
+      if (QF32) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, ka), __builtin_bit_cast(h8, qlow[kb]),
+                                                             acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, ka), __builtin_bit_cast(h8, qreg[kb]),
+                                                   acc, 0, 0, 0);
+    }
+    float mk[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (a.mask && n16 < n_rep)
+      load_mask4(a.mask + (int64_t)seq * a.mask_seq_stride + ((int64_t)kvh * n_rep + n16) * a.mask_head_stride + tile_p0 +
+                     wrow0 + 16 * t + 4 * g, wrow0 + 16 * t + 4 * g, rows_here, mask_vec, mk);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int row = wrow0 + 16 * t + 4 * g + j;
+      const float v = __builtin_fmaf(mk[j], kLog2e, acc[j] * cs);
+      s[t][j] = (row < rows_here) ? v : -INFINITY;
+    }
+  }
+  // statistics of head n16 over the wave's 64 positions
+  float m = -INFINITY;
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) m = fmaxf(m, s[t][j]);
+  m = fmaxf(m, shfl_xor_f(m, 16));
+  m = fmaxf(m, shfl_xor_f(m, 32));
+  const float msafe = (m == -INFINITY) ? 0.0f : m;
+  float l = 0.0f;
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) l += __builtin_amdgcn_exp2f(s[t][j] - msafe);
+  l += shfl_xor_f(l, 16);
+  l += shfl_xor_f(l, 32);
+  if (g == 0) {
+    m_s[wave][n16] = m;
+    l_s[wave][n16] = l;
+  }
+  // The wave's 64 x n_rep scores leave through its LDS area (the last K tile has been consumed; LDS
+  // operations of one wave complete in order): [16 heads][16 units of 4 positions], the unit index
+  // xor-ed with the head, so that a store instruction writes 256-byte runs of a head's row.
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+    kst[n16 * 16 + ((4 * t + g) ^ n16)] = __builtin_bit_cast(u4, f4{s[t][0], s[t][1], s[t][2], s[t][3]});
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int h = 4 * i + g;
+    if (h < n_rep) {
+      const f4 v = __builtin_bit_cast(f4, kst[h * 16 + (n16 ^ h)]);
+      const int row0 = wrow0 + 4 * n16;
+      float* dst = a.scores + (q_row0 + h) * a.scores_stride + tile_p0 + row0;
+      if (row0 + 4 <= rows_here) {
+        *reinterpret_cast<f4*>(dst) = v;                     // rows are 16-byte aligned (host check)
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (row0 + j < rows_here) dst[j] = v[j];
+      }
+    }
+  }
+  __syncthreads();
+  if (tid < n_rep) {
+    float M = m_s[0][tid];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) M = fmaxf(M, m_s[w][tid]);
+    float L = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      const float mw = m_s[w][tid];
+      L += (mw == -INFINITY) ? 0.0f : l_s[w][tid] * __builtin_amdgcn_exp2f(mw - M);
+    }
+    const int64_t grp = (int64_t)seq * a.n_kv + kvh;
+    float* pml = a.ws_ml + (grp * a.n_tiles_max + tile) * (int64_t)(n_rep * 2);
+    pml[2 * tid] = M;
+    pml[2 * tid + 1] = L;
+  }
 }
 
 // Streaming variant for unmasked full tiles: one workgroup runs through n_blocks CONSECUTIVE

@@ -21,11 +21,13 @@
 
 namespace tqm {
 
-enum PackedMode { kFlash = 0, kScores = 1, kWeights = 2 };
+enum PackedMode { kFlash = 0, kScores = 1, kWeights = 2, kSoftWeights = 3 };
 
 struct PackedArgs {
   const float* q_rot;         // kFlash / kScores: [n_seq, n_q, 128] f32
-  const float* weights;       // kWeights: [n_q, T] f32 (one sequence)
+  const float* weights;       // kWeights: [n_seq * n_q, w_stride] f32 weights; kSoftWeights: scores in log2 units
+  const float* stats;         // kSoftWeights: [n_seq * n_kv, n_tiles_max, n_rep, 2] (maximum, sum of 2^(s - maximum)) per tile
+  int64_t w_stride;           // floats per row of `weights`
   const uint32_t* k_packed;
   const float* k_norms;
   const uint32_t* v_packed;
@@ -106,7 +108,8 @@ __device__ __forceinline__ void fill_lut(uint32_t* lut, const Codebook& cb, int 
 template <int MODE>
 __global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(4, 4)))
 void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
-  constexpr bool HAS_K = MODE != kWeights;
+  constexpr bool GIVEN = MODE == kWeights || MODE == kSoftWeights;   // weights come from memory, no keys
+  constexpr bool HAS_K = !GIVEN;
   constexpr bool HAS_V = MODE != kScores;
   __shared__ __align__(16) unsigned char big_s[32768];      // per-wave 4 KB areas, later S_all[8][8][128]
   __shared__ uint32_t lutk_s[64], lutv_s[64];
@@ -115,6 +118,7 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
   __shared__ __align__(16) float kn_s[kWaves][kWavePos], vn_s[kWaves][kWavePos];
   __shared__ float m_s[kWaves][kHeadsMax], l_s[kWaves][kHeadsMax], M_s[kHeadsMax];
   __shared__ __align__(16) float f_s[kWaves][kHeadsMax];
+  __shared__ float iL_s[kHeadsMax];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -161,27 +165,76 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
   }
   // given weights: lane (head n16, group g) takes positions 16t + 4g + j
   float wgt[4][4];
-  if (MODE == kWeights) {
-    // four consecutive positions per (lane, t): one 16-byte load where the row is aligned and inside the tile
-    const bool vec_ok = ((len & 3) == 0) && ((reinterpret_cast<uintptr_t>(a.weights) & 15) == 0);   // uniform
+  if (GIVEN) {
+    // four consecutive positions per (lane, t): one 16-byte load where the row is aligned and inside the tile.
+    // kSoftWeights: the rows hold scores s in log2 units (absent positions count as -inf); they are fetched
+    // first, so that their latency overlaps the fold of the statistics below.
+    const bool vec_ok = ((a.w_stride & 3) == 0) && ((reinterpret_cast<uintptr_t>(a.weights) & 15) == 0);   // uniform
+    const float absent = (MODE == kSoftWeights) ? -INFINITY : 0.0f;     // positions outside the tile / heads past n_rep
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       const int row0 = wrow0 + 16 * t + 4 * g;
-      const float* src = a.weights + ((int64_t)kvh * n_rep + n16) * len + tile_p0 + row0;
-      float w[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+      const float* src = a.weights + (q_row0 + n16) * a.w_stride + tile_p0 + row0;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) wgt[t][j] = absent;
       if (n16 < n_rep) {
         if (vec_ok && row0 + 4 <= rows_here) {
           const f4 v = *reinterpret_cast<const f4*>(src);
-          w[0] = v[0]; w[1] = v[1]; w[2] = v[2]; w[3] = v[3];
+          wgt[t][0] = v[0]; wgt[t][1] = v[1]; wgt[t][2] = v[2]; wgt[t][3] = v[3];
         } else {
 #pragma unroll
           for (int j = 0; j < 4; ++j)
-            if (row0 + j < rows_here) w[j] = src[j];
+            if (row0 + j < rows_here) wgt[t][j] = src[j];
         }
       }
-#pragma unroll
-      for (int j = 0; j < 4; ++j) wgt[t][j] = (w[j] < a.threshold) ? 0.0f : w[j];
     }
+    // kSoftWeights: the weight is 2^(s - M) / L with (M, L) of the whole sequence, folded here from the per-tile
+    // pairs the scores pass left (every workgroup folds them itself: a few KB from L2).  Rows that are masked
+    // out entirely (L = 0) get weight 0.
+    float Mh = 0.0f, iL = 1.0f;
+    if (MODE == kSoftWeights) {
+      float* part_m = reinterpret_cast<float*>(big_s);                  // [32 parts][16 heads]
+      float* part_l = part_m + 32 * kHeadsMax;
+      const int h = tid & 15, part = tid >> 4;
+      const int n_t = (int)((len + kTilePos - 1) / kTilePos);
+      const float* st = a.stats + (((int64_t)seq * a.n_kv + kvh) * a.n_tiles_max) * (int64_t)(n_rep * 2);
+      float M = -INFINITY, L = 0.0f;
+      if (h < n_rep) {
+        for (int t = part; t < n_t; t += 32) {
+          const float2 ml = *reinterpret_cast<const float2*>(st + (int64_t)t * (n_rep * 2) + 2 * h);
+          const float Mn = fmaxf(M, ml.x);
+          if (Mn != -INFINITY) {
+            L = L * __builtin_amdgcn_exp2f(M - Mn) + ml.y * __builtin_amdgcn_exp2f(ml.x - Mn);
+            M = Mn;
+          }
+        }
+      }
+      part_m[part * kHeadsMax + h] = M;
+      part_l[part * kHeadsMax + h] = L;
+      __syncthreads();
+      if (tid < kHeadsMax) {
+        float Mt = -INFINITY;
+        for (int p = 0; p < 32; ++p) Mt = fmaxf(Mt, part_m[p * kHeadsMax + tid]);
+        float Lt = 0.0f;
+        for (int p = 0; p < 32; ++p) {
+          const float pm = part_m[p * kHeadsMax + tid];
+          Lt += (pm == -INFINITY) ? 0.0f : part_l[p * kHeadsMax + tid] * __builtin_amdgcn_exp2f(pm - Mt);
+        }
+        M_s[tid] = (Mt == -INFINITY) ? 0.0f : Mt;
+        iL_s[tid] = (Lt > 0.0f) ? 1.0f / Lt : 0.0f;
+      }
+      __syncthreads();
+      Mh = M_s[n16];
+      iL = iL_s[n16];
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float w = wgt[t][j];
+        if (MODE == kSoftWeights) w = __builtin_amdgcn_exp2f(w - Mh) * iL;
+        wgt[t][j] = (w < a.threshold) ? 0.0f : w;
+      }
   }
   if (HAS_K) fill_lut(lutk_s, kcb, tid);
   if (HAS_V) fill_lut(lutv_s, vcb, tid);
@@ -219,7 +272,7 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
     ex = ex < 27 ? (ex < 1 ? 127 : 27) : (ex > 227 ? 227 : ex);
     kexp = (float)(127 - ex);                            // weights carry 2^kexp: through the exponent (kFlash) ...
     inv_tscale = __uint_as_float((uint32_t)ex << 23);
-    if (MODE == kWeights) {                              // ... or, for given weights, on the norms
+    if (GIVEN) {                                         // ... or, for given weights, on the norms
       const float tscale = __uint_as_float((uint32_t)(254 - ex) << 23);
 #pragma unroll
       for (int t = 0; t < 4; ++t)

@@ -4,7 +4,8 @@
 query, score it against the packed keys, scale, mask, softmax, then the butterfly-pulled-out
 weighted sum over packed values.  `vonly_decode_attention` is the same for a V-only cache, whose
 keys are fp16.  Both can run as ONE fused launch per step when no positive sparse-V threshold is
-asked for (the threshold is defined on final softmax weights, so it needs the unfused passes).
+asked for; the threshold is defined on final softmax weights, so with one the scores of the whole
+sequence are produced first (for a V-only cache inside one library call, otherwise as separate ops).
 """
 from __future__ import annotations
 
@@ -90,8 +91,9 @@ def vonly_decode_attention(queries: torch.Tensor, cache, attn_scale: float, mask
     (the dense-K-scores -> softmax -> sparse_v_matvec shape of hybrid_attention.py:52-88).
 
     queries (B, n_heads, 1, dim) -> (B, n_heads, 1, dim) in queries.dtype.  With no positive
-    threshold the step is one fused launch; otherwise scores, softmax and sparse-V run separately
-    so that the threshold applies to the final weights (sparse_v.py:60-61).
+    threshold the step is one fused launch; with one it is one call of three passes (scores, weights
+    and values, merge) so that the threshold applies to the final weights (sparse_v.py:60-61); shapes
+    outside the matrix-core kernels (dim != 128, bits != 3) run scores, softmax and sparse-V separately.
     """
     B, n_q, S_q, dim = queries.shape
     if S_q != 1:
@@ -103,13 +105,14 @@ def vonly_decode_attention(queries: torch.Tensor, cache, attn_scale: float, mask
     vq = tq._v_q
     bits = tq.quant_bits
     thr = sparse_v_threshold if (sparse_v_threshold is not None and sparse_v_threshold >= 0.0) else 0.0
-    if thr == 0.0:
+    if thr == 0.0 or (ops.vonly_sparse_supported(dim, bits, n_rep) and total > 0):
         m = None
         if mask is not None:
             m = torch.stack([_mask_rows(mask, b, n_q, total).expand(n_q, total) for b in range(B)])
         od = queries.dtype if queries.dtype in (torch.float16, torch.bfloat16, torch.float32) else torch.float32
         out = ops.vonly_decode(queries[:, :, 0, :], kc.keys, tq.v_packed, tq.v_norms, vq.centroids, vq.signs,
-                               dim, bits, attn_scale, n_rep=n_rep, seq_len=total, mask=m, out_dtype=od)
+                               dim, bits, attn_scale, n_rep=n_rep, seq_len=total, mask=m, out_dtype=od,
+                               sparse_v_threshold=thr)
         out = out[:, :, None, :]                           # written in the query dtype by the merge pass
         return out if out.dtype == queries.dtype else out.to(queries.dtype)
     outputs = []

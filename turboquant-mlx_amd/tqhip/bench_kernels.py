@@ -144,6 +144,20 @@ def bench_vonly(iters, dev):
         fns = [(lambda k=k, p=p, n=n: tqhip.vonly_decode(q, k, p, n, cb, signs, 128, 3, 1 / math.sqrt(128), n_rep=7))
                for k, (p, n) in zip(ks, sets)]
         report(f"config 2 shape: V-only decode 28/4 heads, T={T} (python-call launch)", timeit(fns, iters), nbytes)
+        if T == 32768:
+            # sparse-V threshold 1e-5 on the final weights: one call (scores pass, weights-and-values pass, merge) ...
+            fns = [(lambda k=k, p=p, n=n: tqhip.vonly_decode(q, k, p, n, cb, signs, 128, 3, 1 / math.sqrt(128), n_rep=7,
+                                                             sparse_v_threshold=1e-5)) for k, (p, n) in zip(ks, sets)]
+            report(f"config 2 shape, threshold 1e-5: thresholded V-only decode, T={T}, one call", timeit(fns, iters), nbytes)
+
+            # ... against the composition of the three separate ops it replaces
+            def composed(k, p, n):
+                sc = tqhip.dense_qk_scores(q[0], k, 1.0, n_rep=7)
+                w = tqhip.softmax_rows(sc, 1 / math.sqrt(128))
+                return tqhip.sparse_v_matvec(w, p, n, cb, signs, 128, 3, threshold=1e-5, n_rep=7, precision="fp16")
+            fns = [(lambda k=k, p=p, n=n: composed(k, p, n)) for k, (p, n) in zip(ks, sets)]
+            report(f"config 2 shape, threshold 1e-5: dense scores + softmax + sparse-V as three ops, T={T}",
+                   timeit(fns, iters), nbytes)
 
 
 def bench_prefill(iters, dev):

@@ -514,13 +514,22 @@ def flash_attention_turboquant(q_rot, k_packed, k_norms, v_packed, v_norms, k_ce
     return out[0]
 
 
+def vonly_sparse_supported(dim: int, bits: int, n_rep: int) -> bool:
+    """Shapes the thresholded one-call V-only decode step covers (the matrix-core kernels)."""
+    return dim == 128 and bits == 3 and 1 <= n_rep <= 16
+
+
 def vonly_decode(q: torch.Tensor, k: torch.Tensor, v_packed, v_norms, v_centroids, v_signs, dim: int,
                  bits: int, attn_scale: float, *, n_rep: int = 1, seq_len: int | None = None,
                  seq_offsets: torch.Tensor | None = None, max_seq_len: int | None = None, mask=None,
-                 out_dtype=torch.float32, precision: str = "fp16") -> torch.Tensor:
+                 out_dtype=torch.float32, precision: str = "fp16", sparse_v_threshold: float = 0.0) -> torch.Tensor:
     """Dense-softmax decode attention over fp16 keys and packed values (tq_vonly_decode_attn).
     precision as in flash_decode (on the matrix-core path fp16 queries enter as they are, bf16 converted to
     fp16, float32 as an fp16 value plus the fp16 remainder of that rounding).
+
+    sparse_v_threshold > 0: softmax weights below it are dropped from the value sum (threshold rule of
+    sparse_v.py:59-65 on the final weights, as in hybrid_attention.py:52-88) -- tq_vonly_sparse_decode_attn,
+    matrix-core shape only (see vonly_sparse_supported).
 
     q (n_seq, n_q, dim) fp16/bf16/fp32; k [n_seq, n_kv, T_alloc, dim] or ragged [n_kv, sum(L), dim] fp16;
     V as in flash_decode.  Returns (n_seq, n_q, dim) `out_dtype`.
@@ -553,8 +562,18 @@ def vonly_decode(q: torch.Tensor, k: torch.Tensor, v_packed, v_norms, v_centroid
                        mask=mask, mask_strides=ms, attn_scale=attn_scale, out_dtype=out_dtype,
                        allow_mma=bool(_mma_flag(precision)))
     lib = _lib.load()
-    need = lib.tq_workspace_bytes(_lib.TQ_OP_VONLY_DECODE, n_seq, n_q, T, dim)
     stream = _stream(q)
+    if sparse_v_threshold and sparse_v_threshold > 0.0:
+        if not (vonly_sparse_supported(dim, bits, n_rep) and T > 0):
+            raise ValueError("thresholded V-only decode needs dim 128, 3-bit values, n_rep <= 16 and a non-empty cache; "
+                             "compose dense_qk_scores, softmax_rows and sparse_v_matvec for other shapes")
+        need = lib.tq_vonly_sparse_workspace_bytes(n_seq, n_q, T)
+        ws = _workspace(q.device, stream.value or 0, need)
+        _lib.check(lib.tq_vonly_sparse_decode_attn(
+            _ptr(q), _dt(q), _ptr(k), _ptr(v_packed), _ptr(v_norms), _host_table(v_centroids), _ptr(v_signs),
+            float(sparse_v_threshold), _ptr(out), _ptr(ws), ws.numel(), C.byref(sh), stream))
+        return out
+    need = lib.tq_workspace_bytes(_lib.TQ_OP_VONLY_DECODE, n_seq, n_q, T, dim)
     ws = _workspace(q.device, stream.value or 0, need)
     _lib.check(lib.tq_vonly_decode_attn(
         _ptr(q), _dt(q), _ptr(k), _ptr(v_packed), _ptr(v_norms), _host_table(v_centroids), _ptr(v_signs),
