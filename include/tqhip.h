@@ -267,6 +267,21 @@ int tq_vonly_sparse_decode_attn(const void* q, int q_dtype, const void* k_f16,
 size_t tq_vonly_sparse_workspace_bytes(int n_seq, int n_q_heads, int64_t max_seq_len);
 
 /*
+ * The thresholded decode step over packed keys AND packed values: turboquant_attention with
+ * sparse_v_threshold > 0 (fused_attention.py:70-121: prerot_fused_qk_scores -> * attn_scale + mask -> softmax
+ * -> sparse_v_matvec(threshold)) in one call of three passes, for batches and ragged lengths as
+ * tq_flash_decode.  q_rot is the pre-rotated query (tq_prerotate_query).  Workspace:
+ * tq_vonly_sparse_workspace_bytes (same layout).  Same shape limits and error as tq_vonly_sparse_decode_attn
+ * (compose tq_prerot_qk_scores, tq_softmax_rows and tq_sparse_v_matvec for other shapes).
+ */
+int tq_flash_sparse_decode(const float* q_rot,
+                           const uint32_t* k_packed, const float* k_norms,
+                           const uint32_t* v_packed, const float* v_norms,
+                           const float* k_centroids, const float* v_centroids, const float* v_signs,
+                           float threshold, void* out, void* workspace, size_t workspace_bytes,
+                           const tq_decode_shape* shape /* host */, tq_stream_t stream);
+
+/*
  * Bytes of workspace the op needs for this shape (host computation, no GPU call).  The workspace
  * holds per-tile partial results between the two passes of a call; its contents need not be
  * preserved or cleared between calls.  Calls that share a workspace must be ordered (same stream);

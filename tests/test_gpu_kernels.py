@@ -39,15 +39,29 @@ def tables(bits):
     return c, o.gaussian_boundaries(c)
 
 
-def close(got, want, rel=REL, abs_=ABS, row_scale=False):
+def close(got, want, rel=REL, abs_=ABS, row_scale=False, extra=0.0):
     """|err| <= abs + rel * |want| elementwise; with row_scale the relative part is taken against the
     largest magnitude of the output row (the reference's own measure, tests/test_flash_attention.py:
     max_abs / max_ref), which is the meaningful one when an outlier channel dominates a row: the
     Hadamard mixing spreads any operand rounding over all elements of the row."""
     err = np.abs(got.astype(np.float64) - want.astype(np.float64))
     ref = np.abs(want).max(axis=-1, keepdims=True) if row_scale else np.abs(want)
-    ok = err <= abs_ + rel * ref
+    ok = err <= abs_ + rel * ref + extra
     assert ok.all(), f"max err {err.max():.3e} (want scale {np.abs(want).max():.3e}), {(~ok).sum()} bad"
+
+
+def threshold_slack(w, thr, vp, vn, c, vs, n_rep, band):
+    """Extra tolerance for a thresholded value sum: a weight within `band` (relative) of the threshold may fall on
+    either side when the scores behind it differ in the last places (fp16 operands, summation order); such a
+    position moves the output by its whole contribution w * |dequantised V row|.  Returns (n_q, dim): the sum of
+    those contributions over the ambiguous positions of each head (zero when there are none)."""
+    amb = np.abs(w.astype(np.float64) - thr) <= band * thr                      # (n_q, T)
+    if not amb.any():
+        return np.zeros((w.shape[0], 128))
+    n_kv, T = vn.shape
+    vhat = np.abs(o.packed_dequantize(vp.reshape(-1, vp.shape[-1]), vn.reshape(-1), c, vs, 128, 3)).reshape(n_kv, T, 128)
+    wa = (w * amb).reshape(n_kv, n_rep, T).astype(np.float64)
+    return np.matmul(wa, vhat.astype(np.float64)).reshape(-1, 128)
 
 
 # ------------------------------------------------------------------ encode
@@ -1454,3 +1468,103 @@ def test_decode_sweep_vonly_sparse(tq, seed):
         Ki, vpi, vni = per_seq[i]
         mi = None if mask is None else np.broadcast_to(mask[i], (n_q, mask.shape[-1]))
         close(got[i], o.vonly_decode_attention(q[i], Ki, vpi, vni, c, vs, D, bits, sc, threshold=thr, mask=mi))
+
+
+# ------------------------------------------------------------------ thresholded decode over packed keys in one call
+
+def _packed_weights(q, kp, kn, c, ks, sc, n_rep, mask):
+    """Final softmax weights of one sequence over packed keys, as the oracle's turboquant_attention forms them."""
+    s = o.prerot_fused_qk_scores(o.prerotate_query(q, ks), kp, kn, c, 128, 3, n_rep) * F32(sc)
+    if mask is not None:
+        s = s + np.asarray(mask, dtype=F32)
+    return o._softmax64(s).astype(F32)
+
+
+@pytest.mark.parametrize("n_seq,n_kv,n_rep,T,thr,mask_kind", [
+    (1, 8, 4, 1500, 1e-5, "none"), (2, 2, 7, 513, 1e-3, "seq"), (1, 4, 1, 2048, 1e-4, "head"),
+    (3, 1, 16, 77, 1e-2, "none"), (2, 3, 5, 1, 1e-5, "none")])
+def test_flash_sparse_decode_matches_oracle(tq, n_seq, n_kv, n_rep, T, thr, mask_kind):
+    """tq_flash_sparse_decode against the oracle's turboquant_attention with a sparse-V threshold
+    (scores of packed K -> scale, mask, softmax -> thresholded value sum)."""
+    rng = np.random.default_rng(11 * T + n_rep)
+    D, bits, sc = 128, 3, 1 / math.sqrt(128)
+    n_q = n_kv * n_rep
+    T_alloc = T + 21
+    c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, n_seq * n_kv, T_alloc, D, bits)
+    kp, kn, vp, vn = (a.reshape(n_seq, n_kv, *a.shape[1:]) for a in (kp, kn, vp, vn))
+    q = rng.standard_normal((n_seq, n_q, D)).astype(F32)
+    mask = _draw_mask(rng, mask_kind, n_seq, n_q, T)
+    kw = {} if mask is None else dict(mask=dev(mask))
+    q_rot = tq.prerotate_query(dev(q.reshape(-1, D)), dev(ks)).reshape(n_seq, n_q, D)
+    got = host(tq.flash_decode(q_rot, dev(kp), dev(kn), dev(vp), dev(vn), c, c, dev(vs), D, bits, sc, n_rep=n_rep,
+                               seq_len=T, sparse_v_threshold=thr, **kw))
+    for i in range(n_seq):
+        mi = None if mask is None else np.broadcast_to(mask[i], (n_q, T))
+        want = o.turboquant_attention_single(q[i], kp[i, :, :T], kn[i, :, :T], vp[i, :, :T], vn[i, :, :T], c, ks, c, vs,
+                                             D, bits, sc, sparse_v_threshold=thr, mask=mi)
+        w = _packed_weights(q[i], kp[i, :, :T], kn[i, :, :T], c, ks, sc, n_rep, mi)
+        close(got[i], want, extra=threshold_slack(w, thr, vp[i, :, :T], vn[i, :, :T], c, vs, n_rep, 1e-2))
+
+
+def test_flash_sparse_decode_ragged_and_limits(tq):
+    """Ragged batch; a threshold above every weight gives exact zeros; a vanishing one equals the dense fused step."""
+    rng = np.random.default_rng(411)
+    n_kv, n_rep, D, bits, sc = 8, 4, 128, 3, 1 / math.sqrt(128)
+    lens = np.array([1300, 1, 512, 65, 2049])
+    offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, n_kv, int(offs[-1]), D, bits)
+    q = rng.standard_normal((len(lens), n_kv * n_rep, D)).astype(F32)
+    q_rot = tq.prerotate_query(dev(q.reshape(-1, D)), dev(ks)).reshape(len(lens), -1, D)
+    args = (q_rot, dev(kp), dev(kn), dev(vp), dev(vn), c, c, dev(vs), D, bits, sc)
+    kw = dict(n_rep=n_rep, seq_offsets=dev(offs), max_seq_len=int(lens.max()))
+    got = host(tq.flash_decode(*args, sparse_v_threshold=1e-4, **kw))
+    for i in range(len(lens)):
+        a, e = offs[i], offs[i + 1]
+        want = o.turboquant_attention_single(q[i], kp[:, a:e], kn[:, a:e], vp[:, a:e], vn[:, a:e], c, ks, c, vs,
+                                             D, bits, sc, sparse_v_threshold=1e-4)
+        w = _packed_weights(q[i], kp[:, a:e], kn[:, a:e], c, ks, sc, n_rep, None)
+        close(got[i], want, extra=threshold_slack(w, 1e-4, vp[:, a:e], vn[:, a:e], c, vs, n_rep, 1e-2))
+    assert (host(tq.flash_decode(*args, sparse_v_threshold=2.0, **kw)) == 0).all()
+    close(host(tq.flash_decode(*args, sparse_v_threshold=1e-37, **kw)), host(tq.flash_decode(*args, **kw)),
+          rel=1e-3, abs_=2e-4)
+    with pytest.raises(ValueError, match="compose prerot_fused_qk_scores"):
+        c4, ks4, vs4, K4, V4, kp4, kn4, vp4, vn4 = kv_fixture(rng, 2, 64, 64, 4)
+        tq.flash_decode(torch.zeros((1, 2, 64), device="cuda"), dev(kp4), dev(kn4), dev(vp4), dev(vn4), c4, c4, dev(vs4),
+                        64, 4, 0.125, n_rep=1, sparse_v_threshold=1e-5)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_decode_sweep_flash_sparse(tq, seed):
+    """The thresholded packed-key step on the drawn decode shapes."""
+    rng, n_kv, n_rep, ragged, n_seq, lens, mask_kind, qdt = _draw_decode_case(600 + seed)
+    D, bits, sc = 128, 3, 1 / math.sqrt(128)
+    n_q = n_kv * n_rep
+    thr = float(rng.choice([1e-5, 1e-4, 1e-3]))
+    print(f"seed {seed}: n_kv {n_kv} n_rep {n_rep} ragged {ragged} lens {lens.tolist()} mask {mask_kind} thr {thr:g}", flush=True)
+    q = rng.standard_normal((n_seq, n_q, D)).astype(F32)
+    if ragged:
+        offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, n_kv, int(offs[-1]), D, bits)
+        kw = dict(seq_offsets=dev(offs), max_seq_len=int(lens.max()))
+        per_seq = [tuple(a[:, offs[i]:offs[i + 1]] for a in (kp, kn, vp, vn)) for i in range(n_seq)]
+        mask = None
+    else:
+        T = int(lens[0])
+        T_alloc = T + int(rng.integers(0, 70))
+        c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, n_seq * n_kv, T_alloc, D, bits)
+        kp, kn, vp, vn = (a.reshape(n_seq, n_kv, *a.shape[1:]) for a in (kp, kn, vp, vn))
+        kw = dict(seq_len=T)
+        per_seq = [tuple(a[i, :, :T] for a in (kp, kn, vp, vn)) for i in range(n_seq)]
+        mask = _draw_mask(rng, mask_kind, n_seq, n_q, T)
+        if mask is not None:
+            kw["mask"] = dev(mask)
+    q_rot = tq.prerotate_query(dev(q.reshape(-1, D)), dev(ks)).reshape(n_seq, n_q, D)
+    got = host(tq.flash_decode(q_rot, dev(kp), dev(kn), dev(vp), dev(vn), c, c, dev(vs), D, bits, sc, n_rep=n_rep,
+                               sparse_v_threshold=thr, **kw))
+    for i in range(n_seq):
+        kpi, kni, vpi, vni = per_seq[i]
+        mi = None if mask is None else np.broadcast_to(mask[i], (n_q, mask.shape[-1]))
+        w = _packed_weights(q[i], kpi, kni, c, ks, sc, n_rep, mi)
+        close(got[i], o.turboquant_attention_single(q[i], kpi, kni, vpi, vni, c, ks, c, vs, D, bits, sc,
+                                                    sparse_v_threshold=thr, mask=mi),
+              extra=threshold_slack(w, thr, vpi, vni, c, vs, n_rep, 1e-2))

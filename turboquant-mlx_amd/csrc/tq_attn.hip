@@ -708,6 +708,42 @@ int launch_packed_mfma(const float* q_rot_or_weights, const uint32_t* k_packed, 
   return TQ_OK;
 }
 
+// Second and third pass of the thresholded decode steps: weights 2^(s - M) / L from the scores and per-tile
+// statistics, weights below the threshold dropped, value sums per tile; then the merge pass.
+int launch_soft_weights(const float* scores, const float* stats, float* ws_S, float* ws_ml, int64_t t_pad, int n_tiles,
+                        const uint32_t* v_packed, const float* v_norms, const float* v_centroids, const float* v_signs,
+                        float threshold, void* out, const tq_decode_shape& sh, hipStream_t stream, const char* who) {
+  const int n_q = sh.n_kv_heads * sh.n_rep;
+  dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
+  tqm::PackedArgs a{};
+  a.weights = scores; a.stats = stats; a.w_stride = t_pad;
+  a.v_packed = v_packed; a.v_norms = v_norms;
+  a.seq_offsets = sh.seq_offsets;
+  a.ws_S = ws_S; a.ws_ml = ws_ml;
+  a.seq_len = sh.seq_len;
+  a.v_seq_stride = sh.v_seq_stride; a.v_head_stride = sh.v_head_stride;
+  a.vn_seq_stride = sh.vn_seq_stride; a.vn_head_stride = sh.vn_head_stride;
+  a.n_kv = sh.n_kv_heads; a.n_rep = sh.n_rep; a.n_tiles_max = n_tiles;
+  a.threshold = threshold;
+  Codebook kcb, vcb;
+  fill_codebook(kcb, nullptr, sh.bits);
+  a.v_unscale = tq::fill_codebook_fp16(vcb, v_centroids, sh.bits);
+  tqm::packed_tile_mfma_kernel<tqm::kSoftWeights><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, kcb, vcb);
+  TQ_CHECK_LAUNCH(who);
+
+  dim3 mgrid(n_q, sh.n_seq);
+  const float inv_dim = 1.0f / (float)sh.dim;
+#define LAUNCH_MERGE_S(TO)                                                                                  \
+  tqm::decode_merge_rows_kernel<TO, false><<<mgrid, tqm::kMergeThreads, 0, stream>>>(                         \
+      ws_S, ws_ml, sh.seq_offsets, sh.seq_len, n_tiles, sh.n_kv_heads, sh.n_rep, v_signs, inv_dim, (TO*)out, tqm::kTilePos)
+  if (sh.out_dtype == TQ_F16) { LAUNCH_MERGE_S(__half); }
+  else if (sh.out_dtype == TQ_BF16) { LAUNCH_MERGE_S(__hip_bfloat16); }
+  else { LAUNCH_MERGE_S(float); }
+#undef LAUNCH_MERGE_S
+  TQ_CHECK_LAUNCH(who);
+  return TQ_OK;
+}
+
 // Thresholded V-only decode on the matrix cores: scores pass (fp16 keys -> scores in log2 units + per-tile
 // softmax statistics), weights pass (2^(s - M) / L, weights below the threshold dropped, value sums per tile),
 // merge pass.  Workspace: scores | statistics | partial sums | their (0, l) pairs.
@@ -747,33 +783,45 @@ int launch_vonly_sparse(const void* q, int q_dtype, const void* k_f16, const uin
   else tqm::vonly_scores_kernel<false><<<grid, tqm::kMfmaThreads, 0, stream>>>(m);
   TQ_CHECK_LAUNCH(who);
 
-  tqm::PackedArgs a{};
-  a.weights = scores; a.stats = stats; a.w_stride = t_pad;
-  a.v_packed = v_packed; a.v_norms = v_norms;
-  a.seq_offsets = sh.seq_offsets;
-  a.ws_S = ws_S; a.ws_ml = ws_ml;
-  a.seq_len = sh.seq_len;
-  a.v_seq_stride = sh.v_seq_stride; a.v_head_stride = sh.v_head_stride;
-  a.vn_seq_stride = sh.vn_seq_stride; a.vn_head_stride = sh.vn_head_stride;
-  a.n_kv = sh.n_kv_heads; a.n_rep = sh.n_rep; a.n_tiles_max = n_tiles;
-  a.threshold = threshold;
-  Codebook kcb, vcb;
-  fill_codebook(kcb, nullptr, sh.bits);
-  a.v_unscale = tq::fill_codebook_fp16(vcb, v_centroids, sh.bits);
-  tqm::packed_tile_mfma_kernel<tqm::kSoftWeights><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, kcb, vcb);
-  TQ_CHECK_LAUNCH(who);
+  return launch_soft_weights(scores, stats, ws_S, ws_ml, t_pad, n_tiles, v_packed, v_norms, v_centroids, v_signs,
+                             threshold, out, sh, stream, who);
+}
 
-  dim3 mgrid(n_q, sh.n_seq);
-  const float inv_dim = 1.0f / (float)sh.dim;
-#define LAUNCH_MERGE_S(TO)                                                                                  \
-  tqm::decode_merge_rows_kernel<TO, false><<<mgrid, tqm::kMergeThreads, 0, stream>>>(                         \
-      ws_S, ws_ml, sh.seq_offsets, sh.seq_len, n_tiles, sh.n_kv_heads, sh.n_rep, v_signs, inv_dim, (TO*)out, tqm::kTilePos)
-  if (sh.out_dtype == TQ_F16) { LAUNCH_MERGE_S(__half); }
-  else if (sh.out_dtype == TQ_BF16) { LAUNCH_MERGE_S(__hip_bfloat16); }
-  else { LAUNCH_MERGE_S(float); }
-#undef LAUNCH_MERGE_S
+// The same over packed keys: scores pass = the packed-key score kernel with the attention scale, the mask and
+// the per-tile statistics (tq_flash_sparse_decode).
+int launch_flash_sparse(const float* q_rot, const uint32_t* k_packed, const float* k_norms, const uint32_t* v_packed,
+                        const float* v_norms, const float* k_centroids, const float* v_centroids, const float* v_signs,
+                        float threshold, void* out, void* workspace, size_t workspace_bytes, const tq_decode_shape& sh,
+                        hipStream_t stream) {
+  const char* who = "tq_flash_sparse_decode";
+  const int n_q = sh.n_kv_heads * sh.n_rep;
+  const int64_t t_pad = (sh.seq_len + 3) & ~(int64_t)3;
+  const int n_tiles = (int)((sh.seq_len + tqm::kTilePos - 1) / tqm::kTilePos);
+  const size_t need = vonly_sparse_ws_bytes(sh.n_seq, n_q, sh.seq_len);
+  if (!workspace || workspace_bytes < need)
+    return tq::fail(TQ_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, need, workspace_bytes);
+  if (!tq::aligned(workspace, 16)) return tq::fail(TQ_ERR_ALIGN, "%s: workspace must be 16-byte aligned", who);
+  float* scores = (float*)workspace;
+  float* stats = scores + (size_t)sh.n_seq * n_q * t_pad;
+  float* ws_S = stats + (size_t)sh.n_seq * n_q * n_tiles * 2;
+  float* ws_ml = ws_S + (size_t)sh.n_seq * n_q * n_tiles * tqm::kD;
+
+  tqm::PackedArgs a{};
+  a.q_rot = q_rot; a.k_packed = k_packed; a.k_norms = k_norms;
+  a.seq_offsets = sh.seq_offsets; a.mask = sh.mask;
+  a.scores = scores; a.stats_out = stats; a.w_stride = t_pad;
+  a.seq_len = sh.seq_len;
+  a.k_seq_stride = sh.k_seq_stride; a.k_head_stride = sh.k_head_stride;
+  a.kn_seq_stride = sh.kn_seq_stride; a.kn_head_stride = sh.kn_head_stride;
+  a.mask_seq_stride = sh.mask_seq_stride; a.mask_head_stride = sh.mask_head_stride;
+  a.n_kv = sh.n_kv_heads; a.n_rep = sh.n_rep; a.n_tiles_max = n_tiles;
+  Codebook kcb;
+  a.score_scale = sh.attn_scale / (float)sh.dim * tq::fill_codebook_fp16(kcb, k_centroids, sh.bits);
+  dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
+  tqm::packed_tile_mfma_kernel<tqm::kSoftScores><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, kcb, kcb);
   TQ_CHECK_LAUNCH(who);
-  return TQ_OK;
+  return launch_soft_weights(scores, stats, ws_S, ws_ml, t_pad, n_tiles, v_packed, v_norms, v_centroids, v_signs,
+                             threshold, out, sh, stream, who);
 }
 
 bool mma_shape(const tq_decode_shape& sh) {
@@ -985,4 +1033,23 @@ extern "C" int tq_vonly_sparse_decode_attn(const void* q, int q_dtype, const voi
                                         "(compose tq_dense_qk_scores, tq_softmax_rows and tq_sparse_v_matvec otherwise)", who);
   return launch_vonly_sparse(q, q_dtype, k_f16, v_packed, v_norms, v_centroids, v_signs, threshold, out, workspace,
                              workspace_bytes, *shape, (hipStream_t)stream_);
+}
+
+extern "C" int tq_flash_sparse_decode(const float* q_rot, const uint32_t* k_packed, const float* k_norms,
+                                      const uint32_t* v_packed, const float* v_norms, const float* k_centroids,
+                                      const float* v_centroids, const float* v_signs, float threshold, void* out,
+                                      void* workspace, size_t workspace_bytes, const tq_decode_shape* shape,
+                                      tq_stream_t stream_) {
+  const char* who = "tq_flash_sparse_decode";
+  if (int rc = check_shape(shape, who, 128)) return rc;
+  if (!q_rot || !k_centroids || !v_centroids || !v_signs || !out) return tq::fail(TQ_ERR_NULL, "%s: null pointer", who);
+  if (shape->seq_len > 0 && (!k_packed || !k_norms || !v_packed || !v_norms))
+    return tq::fail(TQ_ERR_NULL, "%s: null pointer", who);
+  if (!(threshold >= 0.0f)) return tq::fail(TQ_ERR_ARG, "%s: threshold must be >= 0", who);
+  if (!(shape->dim == 128 && shape->bits == 3 && shape->n_rep <= tqm::kHeadsMax && shape->seq_len > 0 &&
+        tq::aligned(q_rot, 8)))
+    return tq::fail(TQ_ERR_UNSUPPORTED, "%s: dim 128, 3-bit, n_rep <= 16 and a non-empty cache only "
+                                        "(compose tq_prerot_qk_scores, tq_softmax_rows and tq_sparse_v_matvec otherwise)", who);
+  return launch_flash_sparse(q_rot, k_packed, k_norms, v_packed, v_norms, k_centroids, v_centroids, v_signs, threshold,
+                             out, workspace, workspace_bytes, *shape, (hipStream_t)stream_);
 }

@@ -21,7 +21,7 @@
 
 namespace tqm {
 
-enum PackedMode { kFlash = 0, kScores = 1, kWeights = 2, kSoftWeights = 3 };
+enum PackedMode { kFlash = 0, kScores = 1, kWeights = 2, kSoftWeights = 3, kSoftScores = 4 };
 
 struct PackedArgs {
   const float* q_rot;         // kFlash / kScores: [n_seq, n_q, 128] f32
@@ -34,7 +34,8 @@ struct PackedArgs {
   const float* v_norms;
   const int32_t* seq_offsets;
   const float* mask;
-  float* scores;              // kScores: [n_q, T] f32
+  float* scores;              // kScores: [n_q, T] f32; kSoftScores: [n_seq * n_q, w_stride] f32, log2 units
+  float* stats_out;           // kSoftScores: [n_seq * n_kv, n_tiles_max, n_rep, 2] (maximum, sum of 2^(s - maximum)) per tile
   float* ws_S;
   float* ws_ml;
   int64_t seq_len;
@@ -110,7 +111,8 @@ __global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(4,
 void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
   constexpr bool GIVEN = MODE == kWeights || MODE == kSoftWeights;   // weights come from memory, no keys
   constexpr bool HAS_K = !GIVEN;
-  constexpr bool HAS_V = MODE != kScores;
+  constexpr bool HAS_V = MODE != kScores && MODE != kSoftScores;
+  constexpr bool SOFT = MODE == kFlash || MODE == kSoftScores;        // scores carry attn_scale * log2 e and the mask
   __shared__ __align__(16) unsigned char big_s[32768];      // per-wave 4 KB areas, later S_all[8][8][128]
   __shared__ uint32_t lutk_s[64], lutv_s[64];
   __shared__ __align__(16) uint32_t q_s[kHeadsMax][kD / 2];      // rotated queries as half2: rounded value ...
@@ -247,7 +249,7 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
       (&ql_s[0][0])[tid + i * kMfmaThreads] = pack_h2(my_q[i].x - back.x, my_q[i].y - back.y);
     }
     // the score scale rides on the key norm: log2 units for the softmax, plain units for kScores
-    kn_s[wave][lane] = my_kn * (MODE == kFlash ? a.score_scale * kLog2e : a.score_scale);
+    kn_s[wave][lane] = my_kn * (SOFT ? a.score_scale * kLog2e : a.score_scale);
   }
   if (HAS_V) vn_s[wave][lane] = my_vn;
   __syncthreads();
@@ -330,17 +332,39 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
       const float4 kn4 = *reinterpret_cast<const float4*>(&kn_s[wave][16 * t + 4 * g]);
       const float knv[4] = {kn4.x, kn4.y, kn4.z, kn4.w};
       float mk[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-      if (MODE == kFlash && a.mask && n16 < n_rep)
+      if (SOFT && a.mask && n16 < n_rep)
         load_mask4(a.mask + (int64_t)seq * a.mask_seq_stride + ((int64_t)kvh * n_rep + n16) * a.mask_head_stride + tile_p0 +
                        wrow0 + 16 * t + 4 * g, wrow0 + 16 * t + 4 * g, rows_here, mask_vec, mk);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int row = wrow0 + 16 * t + 4 * g + j;
-        const float v = (MODE == kFlash) ? __builtin_fmaf(mk[j], kLog2e, acc[j] * knv[j]) : acc[j] * knv[j];
+        const float v = SOFT ? __builtin_fmaf(mk[j], kLog2e, acc[j] * knv[j]) : acc[j] * knv[j];
         s[t][j] = (row < rows_here) ? v : -INFINITY;
       }
     }
-    if (MODE == kScores) {
+    if (MODE == kScores || MODE == kSoftScores) {
+      // kSoftScores: softmax statistics of head n16 over the wave's 64 positions, combined over the waves below
+      if (MODE == kSoftScores) {
+        float m = -INFINITY;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) m = fmaxf(m, s[t][j]);
+        m = fmaxf(m, shfl_xor_f(m, 16));
+        m = fmaxf(m, shfl_xor_f(m, 32));
+        const float msafe = (m == -INFINITY) ? 0.0f : m;
+        float l = 0.0f;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) l += __builtin_amdgcn_exp2f(s[t][j] - msafe);
+        l += shfl_xor_f(l, 16);
+        l += shfl_xor_f(l, 32);
+        if (g == 0) {
+          m_s[wave][n16] = m;
+          l_s[wave][n16] = l;
+        }
+      }
       // The wave's 64 x n_rep scores leave through its LDS area (the key image has been consumed), so that a
       // store instruction writes whole 256-byte runs of a head's row instead of 64 separate floats: the
       // area is [16 heads][16 units of 4 positions], the unit index xor-ed with the head (conflict-free
@@ -348,14 +372,15 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
       f4* sc = reinterpret_cast<f4*>(stage);
 #pragma unroll
       for (int t = 0; t < 4; ++t) sc[n16 * 16 + ((4 * t + g) ^ n16)] = f4{s[t][0], s[t][1], s[t][2], s[t][3]};
-      const bool vec_ok = ((len & 3) == 0) && ((reinterpret_cast<uintptr_t>(a.scores) & 15) == 0);   // uniform
+      const int64_t row_len = (MODE == kSoftScores) ? a.w_stride : len;
+      const bool vec_ok = ((row_len & 3) == 0) && ((reinterpret_cast<uintptr_t>(a.scores) & 15) == 0);   // uniform
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int h = 4 * i + g, unit = n16;                          // lane -> head 4i + lane / 16, positions 4 * (lane % 16) ..
         if (h < n_rep) {
           const f4 v = sc[h * 16 + (unit ^ h)];
           const int row0 = wrow0 + 4 * unit;
-          float* dst = a.scores + ((int64_t)kvh * n_rep + h) * len + tile_p0 + row0;
+          float* dst = a.scores + ((MODE == kSoftScores ? q_row0 : (int64_t)kvh * n_rep) + h) * row_len + tile_p0 + row0;
           if (vec_ok && row0 + 4 <= rows_here) {
             *reinterpret_cast<f4*>(dst) = v;
           } else {
@@ -363,6 +388,23 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
             for (int j = 0; j < 4; ++j)
               if (row0 + j < rows_here) dst[j] = v[j];
           }
+        }
+      }
+      if (MODE == kSoftScores) {
+        __syncthreads();
+        if (tid < n_rep) {
+          float M = m_s[0][tid];
+#pragma unroll
+          for (int w = 1; w < kWaves; ++w) M = fmaxf(M, m_s[w][tid]);
+          float L = 0.0f;
+#pragma unroll
+          for (int w = 0; w < kWaves; ++w) {
+            const float mw = m_s[w][tid];
+            L += (mw == -INFINITY) ? 0.0f : l_s[w][tid] * __builtin_amdgcn_exp2f(mw - M);
+          }
+          float* pst = a.stats_out + ((((int64_t)seq * a.n_kv + kvh) * a.n_tiles_max) + tile) * (int64_t)(n_rep * 2);
+          pst[2 * tid] = M;
+          pst[2 * tid + 1] = L;
         }
       }
       return;

@@ -36,8 +36,9 @@ def turboquant_attention(queries: torch.Tensor, cache, attn_scale: float, mask=N
     """fused_attention.py:20-125.  queries (B, n_heads, 1, dim) against a TurboQuantKVCache holding
     packed K and V; returns (B, n_heads, 1, dim) in queries.dtype.
 
-    fused=True runs the whole step as one launch (pre-rotation aside) when neither a v_buffer nor a
-    positive sparse-V threshold is requested; the result is the same up to float32 summation order.
+    fused=True runs the whole step as one library call (pre-rotation aside) when no v_buffer is given: one
+    launch + merge without a sparse-V threshold, three passes with one (d = 128 / 3-bit / n_rep <= 16; other
+    shapes compose the separate ops); the result is the same up to summation order and operand rounding.
     """
     B, n_q, S_q, dim = queries.shape
     if S_q != 1:
@@ -49,7 +50,8 @@ def turboquant_attention(queries: torch.Tensor, cache, attn_scale: float, mask=N
     kq, vq = cache._k_q, cache._v_q
     thr = sparse_v_threshold if (sparse_v_threshold is not None and sparse_v_threshold >= 0.0) else 0.0
 
-    if fused and v_buffer is None and thr == 0.0:
+    one_call_thr = thr > 0.0 and ops.vonly_sparse_supported(dim, bits, n_rep) and total > 0 and dim == cache._v_dim
+    if fused and v_buffer is None and (thr == 0.0 or one_call_thr):
         q_rot = ops.prerotate_query(queries.reshape(B * n_q, dim), kq.signs).reshape(B, n_q, dim)
         m = None
         if mask is not None:
@@ -57,7 +59,7 @@ def turboquant_attention(queries: torch.Tensor, cache, attn_scale: float, mask=N
         od = queries.dtype if queries.dtype in (torch.float16, torch.bfloat16, torch.float32) else torch.float32
         out = ops.flash_decode(q_rot, cache.k_packed, cache.k_norms, cache.v_packed, cache.v_norms,
                                kq.centroids, vq.centroids, vq.signs, dim, bits, attn_scale, n_rep=n_rep,
-                               seq_len=total, mask=m, out_dtype=od)
+                               seq_len=total, mask=m, out_dtype=od, sparse_v_threshold=thr)
         out = out[:, :, None, :]
         return out if out.dtype == queries.dtype else out.to(queries.dtype)
 

@@ -115,6 +115,12 @@ def bench_flash(iters, dev):
                                            1 / math.sqrt(128), n_rep=4, seq_offsets=offs,
                                            max_seq_len=int(lens.max()), out_dtype=torch.float16)) for i in range(2)]
     report(f"config 4: flash decode 32/8 heads, 16 seqs, sum L={total}", timeit(fns, max(20, iters // 10)), nbytes)
+    fns = [(lambda i=i: tqhip.flash_decode(q_rot, k[i][0], k[i][1], v[i][0], v[i][1], cb, cb, signs, 128, 3,
+                                           1 / math.sqrt(128), n_rep=4, seq_offsets=offs,
+                                           max_seq_len=int(lens.max()), out_dtype=torch.float16,
+                                           sparse_v_threshold=1e-5)) for i in range(2)]
+    report(f"config 4, threshold 1e-5: thresholded flash decode (scores, weights + values, merge), one call",
+           timeit(fns, max(20, iters // 10)), nbytes)
 
 
 def bench_flash_long(iters, dev):

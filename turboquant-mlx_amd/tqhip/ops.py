@@ -453,8 +453,12 @@ def flash_decode(q_rot: torch.Tensor, k_packed, k_norms, v_packed, v_norms, k_ce
                  v_signs, dim: int, bits: int, attn_scale: float, *, n_rep: int = 1, block_size: int = 16,
                  seq_len: int | None = None, seq_offsets: torch.Tensor | None = None,
                  max_seq_len: int | None = None, mask=None, out_dtype=torch.float32,
-                 precision: str = "fp16") -> torch.Tensor:
+                 precision: str = "fp16", sparse_v_threshold: float = 0.0) -> torch.Tensor:
     """Batched form of flash_attention_turboquant (tq_flash_decode).
+
+    sparse_v_threshold > 0: softmax weights below it are dropped from the value sum (the threshold of
+    sparse_v.py:59-65 on the final weights, as turboquant_attention applies it, fused_attention.py:109-121)
+    -- tq_flash_sparse_decode, matrix-core shape only (see vonly_sparse_supported).
 
     precision="fp16" (default): matrix-core kernels where the shape allows (d = 128, 3-bit,
     n_rep <= 16), operands rounded to half, float32 accumulation; "fp32": float32 kernels.
@@ -494,8 +498,19 @@ def flash_decode(q_rot: torch.Tensor, k_packed, k_norms, v_packed, v_norms, k_ce
                        vn_strides=vns, mask=mask, mask_strides=ms, attn_scale=attn_scale, out_dtype=out_dtype,
                        allow_mma=bool(_mma_flag(precision)))
     lib = _lib.load()
-    need = lib.tq_workspace_bytes(_lib.TQ_OP_FLASH_DECODE, n_seq, n_q, T, dim)
     stream = _stream(q_rot)
+    if sparse_v_threshold and sparse_v_threshold > 0.0:
+        if not (vonly_sparse_supported(dim, bits, n_rep) and T > 0):
+            raise ValueError("thresholded flash decode needs dim 128, 3-bit, n_rep <= 16 and a non-empty cache; "
+                             "compose prerot_fused_qk_scores, softmax_rows and sparse_v_matvec for other shapes")
+        need = lib.tq_vonly_sparse_workspace_bytes(n_seq, n_q, T)
+        ws = _workspace(q_rot.device, stream.value or 0, need)
+        _lib.check(lib.tq_flash_sparse_decode(
+            _ptr(q_rot), _ptr(k_packed), _ptr(k_norms), _ptr(v_packed), _ptr(v_norms),
+            _host_table(k_centroids), _host_table(v_centroids), _ptr(v_signs), float(sparse_v_threshold), _ptr(out),
+            _ptr(ws), ws.numel(), C.byref(sh), stream))
+        return out
+    need = lib.tq_workspace_bytes(_lib.TQ_OP_FLASH_DECODE, n_seq, n_q, T, dim)
     ws = _workspace(q_rot.device, stream.value or 0, need)
     _lib.check(lib.tq_flash_decode(
         _ptr(q_rot), _ptr(k_packed), _ptr(k_norms), _ptr(v_packed), _ptr(v_norms),

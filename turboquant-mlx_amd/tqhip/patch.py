@@ -48,8 +48,9 @@ def scaled_dot_product_attention(queries, keys, values, cache, scale, mask=None,
     is_decode = queries.shape[2] == 1
     if isinstance(cache, TurboQuantKVCache) and not cache.v_only and cache.offset > 0 and cache.fused:
         if is_decode:
+            # one library call either way; with a threshold, shapes outside the matrix-core kernels compose the ops
             return turboquant_attention(queries, cache, scale, mask, sparse_v_threshold=cache.sparse_v_threshold,
-                                        fused=not cache.sparse_v_threshold)
+                                        fused=True)
         if mask is None or (isinstance(mask, str) and mask == "causal"):
             return turboquant_prefill_attention(queries, cache, scale, causal=mask is not None)
         raise ValueError("a fused TurboQuantKVCache holds no dequantised K/V: a multi-token step takes "
