@@ -710,13 +710,15 @@ int launch_packed_mfma(const float* q_rot_or_weights, const uint32_t* k_packed, 
 
 // Second and third pass of the thresholded decode steps: weights 2^(s - M) / L from the scores and per-tile
 // statistics, weights below the threshold dropped, value sums per tile; then the merge pass.
-int launch_soft_weights(const float* scores, const float* stats, float* ws_S, float* ws_ml, int64_t t_pad, int n_tiles,
+int launch_soft_weights(const float* scores, const float* stats, int stats_tile_pos, float* ws_S, float* ws_ml, int64_t t_pad, int n_tiles,
                         const uint32_t* v_packed, const float* v_norms, const float* v_centroids, const float* v_signs,
                         float threshold, void* out, const tq_decode_shape& sh, hipStream_t stream, const char* who) {
   const int n_q = sh.n_kv_heads * sh.n_rep;
   dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
   tqm::PackedArgs a{};
   a.weights = scores; a.stats = stats; a.w_stride = t_pad;
+  a.stats_tile_pos = stats_tile_pos;
+  a.n_stats_max = (int)((sh.seq_len + stats_tile_pos - 1) / stats_tile_pos);
   a.v_packed = v_packed; a.v_norms = v_norms;
   a.seq_offsets = sh.seq_offsets;
   a.ws_S = ws_S; a.ws_ml = ws_ml;
@@ -747,10 +749,15 @@ int launch_soft_weights(const float* scores, const float* stats, float* ws_S, fl
 // Thresholded V-only decode on the matrix cores: scores pass (fp16 keys -> scores in log2 units + per-tile
 // softmax statistics), weights pass (2^(s - M) / L, weights below the threshold dropped, value sums per tile),
 // merge pass.  Workspace: scores | statistics | partial sums | their (0, l) pairs.
+constexpr int kSparseStatsPos = 256;     // finest granularity of the per-tile statistics (scores pass of the fp16-key step)
+
 size_t vonly_sparse_ws_bytes(int n_seq, int n_q, int64_t seq_len) {
   const int64_t t_pad = (seq_len + 3) & ~(int64_t)3;
   const int64_t n_tiles = (seq_len + tqm::kTilePos - 1) / tqm::kTilePos;
-  return ((size_t)n_seq * n_q * t_pad + (size_t)n_seq * n_q * n_tiles * (tqm::kD + 4)) * sizeof(float);
+  const int64_t n_stats = (seq_len + kSparseStatsPos - 1) / kSparseStatsPos;
+  // every section starts 16-byte aligned: the statistics are padded to a multiple of four floats
+  return ((size_t)n_seq * n_q * t_pad + (((size_t)n_seq * n_q * n_stats * 2 + 3) & ~(size_t)3) +
+          (size_t)n_seq * n_q * n_tiles * (tqm::kD + 2)) * sizeof(float);
 }
 
 int launch_vonly_sparse(const void* q, int q_dtype, const void* k_f16, const uint32_t* v_packed, const float* v_norms,
@@ -764,9 +771,10 @@ int launch_vonly_sparse(const void* q, int q_dtype, const void* k_f16, const uin
   if (!workspace || workspace_bytes < need)
     return tq::fail(TQ_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, need, workspace_bytes);
   if (!tq::aligned(workspace, 16)) return tq::fail(TQ_ERR_ALIGN, "%s: workspace must be 16-byte aligned", who);
+  const int n_stats = (int)((sh.seq_len + kSparseStatsPos - 1) / kSparseStatsPos);
   float* scores = (float*)workspace;                                    // [n_seq * n_q, t_pad]
-  float* stats = scores + (size_t)sh.n_seq * n_q * t_pad;               // [n_seq * n_kv, n_tiles, n_rep, 2]
-  float* ws_S = stats + (size_t)sh.n_seq * n_q * n_tiles * 2;           // [n_seq * n_kv, n_tiles, n_rep, 128]
+  float* stats = scores + (size_t)sh.n_seq * n_q * t_pad;               // [n_seq * n_kv, n_stats, n_rep, 2]
+  float* ws_S = stats + (((size_t)sh.n_seq * n_q * n_stats * 2 + 3) & ~(size_t)3);   // [n_seq * n_kv, n_tiles, n_rep, 128]
   float* ws_ml = ws_S + (size_t)sh.n_seq * n_q * n_tiles * tqm::kD;
 
   tqm::MfmaArgs m{};
@@ -776,15 +784,16 @@ int launch_vonly_sparse(const void* q, int q_dtype, const void* k_f16, const uin
   m.seq_len = sh.seq_len;
   m.k_seq_stride = sh.k_seq_stride; m.k_head_stride = sh.k_head_stride;
   m.mask_seq_stride = sh.mask_seq_stride; m.mask_head_stride = sh.mask_head_stride;
-  m.n_kv = sh.n_kv_heads; m.n_rep = sh.n_rep; m.n_tiles_max = n_tiles;
+  m.n_kv = sh.n_kv_heads; m.n_rep = sh.n_rep; m.n_tiles_max = n_stats;
   m.attn_scale = sh.attn_scale;
-  dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
-  if (q_dtype == TQ_F32) tqm::vonly_scores_kernel<true><<<grid, tqm::kMfmaThreads, 0, stream>>>(m);
-  else tqm::vonly_scores_kernel<false><<<grid, tqm::kMfmaThreads, 0, stream>>>(m);
+  // workgroups of four waves (256 positions), several per CU: the loads of one overlap the arithmetic and stores of another
+  dim3 sgrid(n_stats, sh.n_kv_heads, sh.n_seq);
+  if (q_dtype == TQ_F32) tqm::vonly_scores_kernel<true, 4><<<sgrid, 256, 0, stream>>>(m);
+  else tqm::vonly_scores_kernel<false, 4><<<sgrid, 256, 0, stream>>>(m);
   TQ_CHECK_LAUNCH(who);
 
-  return launch_soft_weights(scores, stats, ws_S, ws_ml, t_pad, n_tiles, v_packed, v_norms, v_centroids, v_signs,
-                             threshold, out, sh, stream, who);
+  return launch_soft_weights(scores, stats, kSparseStatsPos, ws_S, ws_ml, t_pad, n_tiles, v_packed, v_norms, v_centroids,
+                             v_signs, threshold, out, sh, stream, who);
 }
 
 // The same over packed keys: scores pass = the packed-key score kernel with the attention scale, the mask and
@@ -803,7 +812,7 @@ int launch_flash_sparse(const float* q_rot, const uint32_t* k_packed, const floa
   if (!tq::aligned(workspace, 16)) return tq::fail(TQ_ERR_ALIGN, "%s: workspace must be 16-byte aligned", who);
   float* scores = (float*)workspace;
   float* stats = scores + (size_t)sh.n_seq * n_q * t_pad;
-  float* ws_S = stats + (size_t)sh.n_seq * n_q * n_tiles * 2;
+  float* ws_S = stats + (((size_t)sh.n_seq * n_q * n_tiles * 2 + 3) & ~(size_t)3);
   float* ws_ml = ws_S + (size_t)sh.n_seq * n_q * n_tiles * tqm::kD;
 
   tqm::PackedArgs a{};
@@ -820,8 +829,8 @@ int launch_flash_sparse(const float* q_rot, const uint32_t* k_packed, const floa
   dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
   tqm::packed_tile_mfma_kernel<tqm::kSoftScores><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, kcb, kcb);
   TQ_CHECK_LAUNCH(who);
-  return launch_soft_weights(scores, stats, ws_S, ws_ml, t_pad, n_tiles, v_packed, v_norms, v_centroids, v_signs,
-                             threshold, out, sh, stream, who);
+  return launch_soft_weights(scores, stats, tqm::kTilePos, ws_S, ws_ml, t_pad, n_tiles, v_packed, v_norms, v_centroids,
+                             v_signs, threshold, out, sh, stream, who);
 }
 
 bool mma_shape(const tq_decode_shape& sh) {

@@ -496,12 +496,14 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
 // to a.scores and one (maximum, sum of 2^(s - maximum)) pair per query head to a.ws_ml, from which the
 // second pass derives the softmax denominator of the sequence.
 // grid = (n_tiles_max, n_kv, n_seq), 512 threads.
-template <bool QF32>
-__global__ __launch_bounds__(kMfmaThreads) void vonly_scores_kernel(MfmaArgs a) {
-  __shared__ __align__(16) unsigned char big_s[32768];        // per-wave 4 KB: K tiles, then the score block
+template <bool QF32, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void vonly_scores_kernel(MfmaArgs a) {
+  constexpr int kPos = WAVES * kWavePos;             // positions per workgroup
+  constexpr int kThr = WAVES * 64;
+  __shared__ __align__(16) unsigned char big_s[WAVES * 4096]; // per-wave 4 KB: K tiles, then the score block
   __shared__ __align__(16) uint32_t q_s[kHeadsMax][kD / 2];
   __shared__ __align__(16) uint32_t ql_s[QF32 ? kHeadsMax : 1][kD / 2];
-  __shared__ float m_s[kWaves][kHeadsMax], l_s[kWaves][kHeadsMax];
+  __shared__ float m_s[WAVES][kHeadsMax], l_s[WAVES][kHeadsMax];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -516,16 +518,18 @@ __global__ __launch_bounds__(kMfmaThreads) void vonly_scores_kernel(MfmaArgs a) 
     first = a.seq_offsets[seq];
     len = (int64_t)a.seq_offsets[seq + 1] - first;
   }
-  const int64_t tile_p0 = (int64_t)tile * kTilePos;
+  const int64_t tile_p0 = (int64_t)tile * kPos;
   if (tile_p0 >= len) return;                          // the second pass never reads this tile
-  const int rows_here = (int)min((int64_t)kTilePos, len - tile_p0);
+  const int rows_here = (int)min((int64_t)kPos, len - tile_p0);
   const int last_row = rows_here - 1;
   const int wrow0 = wave * kWavePos;
 
-  uint32_t my_q[2], my_ql[2] = {0u, 0u};
+  constexpr int kQIt = kHeadsMax * (kD / 2) / kThr;
+  uint32_t my_q[kQIt], my_ql[kQIt];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int w = tid + i * kMfmaThreads;
+  for (int i = 0; i < kQIt; ++i) {
+    my_ql[i] = 0u;
+    const int w = tid + i * kThr;
     if (QF32) {
       const float2 f = (w < n_rep * (kD / 2)) ? reinterpret_cast<const float2*>(reinterpret_cast<const float*>(a.q) + q_row0 * kD)[w]
                                               : make_float2(0.f, 0.f);
@@ -552,9 +556,9 @@ __global__ __launch_bounds__(kMfmaThreads) void vonly_scores_kernel(MfmaArgs a) 
     kreg[i] = *reinterpret_cast<const u4*>(kbase + (uint32_t)((row * 16 + piece) * 16));
   }
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    (&q_s[0][0])[tid + i * kMfmaThreads] = my_q[i];
-    if (QF32) (&ql_s[0][0])[tid + i * kMfmaThreads] = my_ql[i];
+  for (int i = 0; i < kQIt; ++i) {
+    (&q_s[0][0])[tid + i * kThr] = my_q[i];
+    if (QF32) (&ql_s[0][0])[tid + i * kThr] = my_ql[i];
   }
   __syncthreads();
 
@@ -639,10 +643,10 @@ __global__ __launch_bounds__(kMfmaThreads) void vonly_scores_kernel(MfmaArgs a) 
   if (tid < n_rep) {
     float M = m_s[0][tid];
 #pragma unroll
-    for (int w = 1; w < kWaves; ++w) M = fmaxf(M, m_s[w][tid]);
+    for (int w = 1; w < WAVES; ++w) M = fmaxf(M, m_s[w][tid]);
     float L = 0.0f;
 #pragma unroll
-    for (int w = 0; w < kWaves; ++w) {
+    for (int w = 0; w < WAVES; ++w) {
       const float mw = m_s[w][tid];
       L += (mw == -INFINITY) ? 0.0f : l_s[w][tid] * __builtin_amdgcn_exp2f(mw - M);
     }

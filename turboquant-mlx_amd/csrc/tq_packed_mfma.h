@@ -28,6 +28,8 @@ struct PackedArgs {
   const float* weights;       // kWeights: [n_seq * n_q, w_stride] f32 weights; kSoftWeights: scores in log2 units
   const float* stats;         // kSoftWeights: [n_seq * n_kv, n_tiles_max, n_rep, 2] (maximum, sum of 2^(s - maximum)) per tile
   int64_t w_stride;           // floats per row of `weights`
+  int32_t stats_tile_pos;     // kSoftWeights: positions per entry of `stats`
+  int32_t n_stats_max;        //               entries of `stats` per (sequence, kv head)
   const uint32_t* k_packed;
   const float* k_norms;
   const uint32_t* v_packed;
@@ -198,8 +200,8 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
       float* part_m = reinterpret_cast<float*>(big_s);                  // [32 parts][16 heads]
       float* part_l = part_m + 32 * kHeadsMax;
       const int h = tid & 15, part = tid >> 4;
-      const int n_t = (int)((len + kTilePos - 1) / kTilePos);
-      const float* st = a.stats + (((int64_t)seq * a.n_kv + kvh) * a.n_tiles_max) * (int64_t)(n_rep * 2);
+      const int n_t = (int)((len + a.stats_tile_pos - 1) / a.stats_tile_pos);
+      const float* st = a.stats + (((int64_t)seq * a.n_kv + kvh) * a.n_stats_max) * (int64_t)(n_rep * 2);
       float M = -INFINITY, L = 0.0f;
       if (h < n_rep) {
         for (int t = part; t < n_t; t += 32) {
