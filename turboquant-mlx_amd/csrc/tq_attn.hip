@@ -121,6 +121,82 @@ __device__ __forceinline__ void load_q_tile(const QT* __restrict__ q, int64_t q_
 }
 
 // ---------------------------------------------------------------- stand-alone score kernels
+// Packed rows of a wave's 64 consecutive positions, fetched with coalesced loads (instruction i reads words
+// 64 i .. 64 i + 63 of the contiguous block) into LDS at an odd row pitch, so that every lane then reads its own
+// row without bank conflicts.  Rows at or past rows_here are not fetched.
+template <int PDIM>
+__device__ __forceinline__ void stage_rows(const uint32_t* __restrict__ block, int rows_here, uint32_t* dst, int lane) {
+  constexpr int PSTR = PDIM | 1;
+  const int valid = rows_here * PDIM;
+#pragma unroll
+  for (int i = 0; i < PDIM; ++i) {
+    const int idx = i * 64 + lane;
+    if (idx < valid) {
+      const int row = idx / PDIM;
+      dst[row * PSTR + (idx - row * PDIM)] = block[idx];
+    }
+  }
+}
+
+// acc[u][r] = sum_e c[idx_e(row u)] * q[r][e] over NP packed rows in LDS (rows `pitch` words apart), element order
+// e = 0, 1, ...: one fused multiply-add per (row, head, element).  The query rows are read at wave-uniform
+// addresses, which the compiler turns into scalar loads: the vector ALU sees them as scalar-register operands and
+// no LDS bandwidth goes into re-reading the query for every position; NP rows per lane share each of them.
+// qrow[r] points at row min(r, n_local - 1).
+template <int D, int BITS, int NP>
+__device__ __forceinline__ void score_packed_uniform_q(const uint32_t* row, int pitch, const float* cb,
+                                                       const float* const (&qrow)[kRMax], float (&acc)[NP][kRMax]) {
+  constexpr int VPW = Pk<BITS>::VPW;
+  constexpr int PDIM = Pk<BITS>::pdim(D);
+#pragma unroll
+  for (int u = 0; u < NP; ++u)
+#pragma unroll
+    for (int r = 0; r < kRMax; ++r) acc[u][r] = 0.0f;
+  // Full words in a rolled loop (few live registers, so many waves per SIMD hide the scalar-load latency),
+  // the last, partly filled word unrolled with its element count known at compile time.
+  constexpr int FULL = D / VPW;
+#pragma unroll 1
+  for (int w = 0; w < FULL; ++w) {
+    uint32_t word[NP];
+#pragma unroll
+    for (int u = 0; u < NP; ++u) word[u] = row[u * pitch + w];
+#pragma unroll
+    for (int i = 0; i < VPW; ++i) {
+      float c[NP];
+#pragma unroll
+      for (int u = 0; u < NP; ++u) c[u] = cb[(word[u] >> (i * BITS)) & Pk<BITS>::MASK];
+#pragma unroll
+      for (int r = 0; r < kRMax; ++r) {
+        const float qv = qrow[r][w * VPW + i];
+#pragma unroll
+        for (int u = 0; u < NP; ++u) acc[u][r] = __builtin_fmaf(c[u], qv, acc[u][r]);
+      }
+    }
+  }
+  if (FULL < PDIM) {
+    uint32_t word[NP];
+#pragma unroll
+    for (int u = 0; u < NP; ++u) word[u] = row[u * pitch + FULL];
+#pragma unroll
+    for (int i = 0; i < D - FULL * VPW; ++i) {
+      float c[NP];
+#pragma unroll
+      for (int u = 0; u < NP; ++u) c[u] = cb[(word[u] >> (i * BITS)) & Pk<BITS>::MASK];
+#pragma unroll
+      for (int r = 0; r < kRMax; ++r) {
+        const float qv = qrow[r][FULL * VPW + i];
+#pragma unroll
+        for (int u = 0; u < NP; ++u) acc[u][r] = __builtin_fmaf(c[u], qv, acc[u][r]);
+      }
+    }
+  }
+}
+
+// grid = (ceil(seq_len / kScoreTile), n_kv * n_rgroups): a wave takes 128 consecutive positions, a lane the
+// positions lane and lane + 64 of them.
+constexpr int kScoreNP = 1;
+constexpr int kScoreTile = kThreads * kScoreNP;
+
 template <int D, int BITS>
 __global__ __launch_bounds__(kThreads) void prerot_scores_kernel(const float* __restrict__ q_rot,
                                                                  const uint32_t* __restrict__ k_packed,
@@ -130,23 +206,38 @@ __global__ __launch_bounds__(kThreads) void prerot_scores_kernel(const float* __
                                                                  int64_t p_head_stride, int64_t n_head_stride,
                                                                  float inv_dim) {
   constexpr int PDIM = Pk<BITS>::pdim(D);
+  constexpr int PSTR = PDIM | 1;
   __shared__ float cb[16];
-  __shared__ __align__(16) float q_s[D][kRMax];
+  __shared__ uint32_t rows_s[kWaves][kScoreNP * 64 * PSTR];
   const int kvh = blockIdx.y / n_rgroups;
   const int r0 = (blockIdx.y % n_rgroups) * kRMax;
   const int n_local = min(kRMax, n_rep - r0);
   const int64_t q_row0 = (int64_t)kvh * n_rep + r0;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   if (threadIdx.x < 16) cb[threadIdx.x] = cbk.c[threadIdx.x];
-  load_q_tile<float, D>(q_rot, q_row0, n_local, q_s);
-  __syncthreads();
-  const int64_t p = (int64_t)blockIdx.x * kTile + threadIdx.x;
-  if (p >= seq_len) return;
-  float acc[kRMax];
-  score_packed<D, BITS>(k_packed + ((int64_t)kvh * p_head_stride + p) * PDIM, cb, q_s, acc);
-  const float nrm = k_norms[(int64_t)kvh * n_head_stride + p];
+  const int64_t wp0 = (int64_t)blockIdx.x * kScoreTile + wave * (64 * kScoreNP);    // first position of this wave
+  const int rows_here = (int)max((int64_t)0, min((int64_t)(64 * kScoreNP), seq_len - wp0));
 #pragma unroll
-  for (int r = 0; r < kRMax; ++r)
-    if (r < n_local) scores[(q_row0 + r) * seq_len + p] = (acc[r] * nrm) * inv_dim;
+  for (int u = 0; u < kScoreNP; ++u)
+    stage_rows<PDIM>(k_packed + ((int64_t)kvh * p_head_stride + wp0 + 64 * u) * PDIM, rows_here - 64 * u,
+                     rows_s[wave] + u * 64 * PSTR, lane);
+  __syncthreads();
+  if (lane >= rows_here) return;
+  const float* qrow[kRMax];
+#pragma unroll
+  for (int r = 0; r < kRMax; ++r) qrow[r] = q_rot + (q_row0 + min(r, n_local - 1)) * D;
+  float acc[kScoreNP][kRMax];
+  score_packed_uniform_q<D, BITS, kScoreNP>(&rows_s[wave][lane * PSTR], 64 * PSTR, cb, qrow, acc);
+#pragma unroll
+  for (int u = 0; u < kScoreNP; ++u) {
+    const int64_t p = wp0 + 64 * u + lane;
+    if (p < seq_len) {
+      const float nrm = k_norms[(int64_t)kvh * n_head_stride + p];
+#pragma unroll
+      for (int r = 0; r < kRMax; ++r)
+        if (r < n_local) scores[(q_row0 + r) * seq_len + p] = (acc[u][r] * nrm) * inv_dim;
+    }
+  }
 }
 
 template <int D, typename QT>
@@ -888,7 +979,7 @@ extern "C" int tq_prerot_qk_scores(const float* q_rot, const uint32_t* k_packed,
     return TQ_OK;
   }
   const int n_rgroups = (n_rep + kRMax - 1) / kRMax;
-  dim3 grid(n_tiles_for(seq_len), n_kv_heads * n_rgroups);
+  dim3 grid((unsigned)((seq_len + kScoreTile - 1) / kScoreTile), n_kv_heads * n_rgroups);
   hipStream_t stream = (hipStream_t)stream_;
   TQ_DISPATCH_DIM(dim, TQ_DISPATCH_BITS(bits, (prerot_scores_kernel<D_, B_><<<grid, kThreads, 0, stream>>>(
                                                   q_rot, k_packed, k_norms, cb, scores, n_rep, n_rgroups,
