@@ -59,33 +59,8 @@ __device__ __forceinline__ void seq_range(const int32_t* seq_offsets, int64_t se
   }
 }
 
-// ---- score of one position against up to kRMax query heads, packed keys:
-//      acc[r] = sum_e c[idx_e] * q_rot[r][e]           (q_s is [D][kRMax] in LDS)
-template <int D, int BITS>
-__device__ __forceinline__ void score_packed(const uint32_t* __restrict__ krow, const float* cb,
-                                             const float (*q_s)[kRMax], float (&acc)[kRMax]) {
-  constexpr int VPW = Pk<BITS>::VPW;
-  constexpr int PDIM = Pk<BITS>::pdim(D);
-#pragma unroll
-  for (int r = 0; r < kRMax; ++r) acc[r] = 0.0f;
-#pragma unroll 1
-  for (int w = 0; w < PDIM; ++w) {
-    const uint32_t word = krow[w];
-#pragma unroll
-    for (int i = 0; i < VPW; ++i) {
-      const int e = w * VPW + i;
-      if (e < D) {
-        const float c = cb[(word >> (i * BITS)) & Pk<BITS>::MASK];
-        const float4 qa = *reinterpret_cast<const float4*>(&q_s[e][0]);
-        const float4 qb = *reinterpret_cast<const float4*>(&q_s[e][4]);
-        acc[0] += c * qa.x; acc[1] += c * qa.y; acc[2] += c * qa.z; acc[3] += c * qa.w;
-        acc[4] += c * qb.x; acc[5] += c * qb.y; acc[6] += c * qb.z; acc[7] += c * qb.w;
-      }
-    }
-  }
-}
-
-// ---- same for fp16 keys: acc[r] = sum_e K[e] * q[r][e]
+// ---- score of one position against up to kRMax query heads, fp16 keys: acc[r] = sum_e K[e] * q[r][e]
+//      (q_s is [D][kRMax] in LDS)
 template <int D>
 __device__ __forceinline__ void score_dense(const __half* __restrict__ krow, const float (*q_s)[kRMax],
                                             float (&acc)[kRMax]) {
@@ -346,8 +321,8 @@ __global__ __launch_bounds__(kThreads) void decode_tile_kernel(DecodeArgs a, Cod
   constexpr int VPW = Pk<BITS>::VPW;
   constexpr int PDIM = Pk<BITS>::pdim(D);
   __shared__ float cbk_s[16], cbv_s[16];
-  __shared__ __align__(16) float q_s[KMODE == kWeights ? 1 : D][kRMax];
-  __shared__ float p_s[kRMax][kTile];
+  __shared__ __align__(16) float q_s[KMODE == kDenseK ? D : 1][kRMax];
+  __shared__ uint32_t vrows_s[kWaves][66 * (PDIM | 1)];      // 64 rows + two that the pipelined loop reads ahead
   __shared__ float red_s[kWaves][kRMax];
   __shared__ float acc_s[kWaves][kRMax][D >= 64 ? D : 64];
 
@@ -368,13 +343,23 @@ __global__ __launch_bounds__(kThreads) void decode_tile_kernel(DecodeArgs a, Cod
     cbk_s[threadIdx.x] = kcb.c[threadIdx.x];
     cbv_s[threadIdx.x] = vcb.c[threadIdx.x];
   }
-  if (KMODE != kWeights) load_q_tile<QT, D>(reinterpret_cast<const QT*>(a.q), q_row0, n_local, q_s);
+  if (KMODE == kDenseK) load_q_tile<QT, D>(reinterpret_cast<const QT*>(a.q), q_row0, n_local, q_s);
+  const float* qrow[kRMax];                                // kPackedK: rows of the pre-rotated query, wave-uniform
+  if (KMODE == kPackedK) {
+#pragma unroll
+    for (int r = 0; r < kRMax; ++r) qrow[r] = reinterpret_cast<const float*>(a.q) + (q_row0 + min(r, n_local - 1)) * D;
+    // packed key rows of this wave's 64 positions (thread t of the workgroup owns position p0 + t)
+    const int k_here = (int)max((int64_t)0, min((int64_t)TQ_WAVE, len - p0 - wave * TQ_WAVE));
+    stage_rows<PDIM>(a.k_packed + ((int64_t)seq * a.k_seq_stride + (int64_t)kvh * a.k_head_stride + first + p0 +
+                                  wave * TQ_WAVE) * PDIM, k_here, vrows_s[wave], lane);
+  }
   __syncthreads();
 
   // ---- phase 1: one position per thread -> up to kRMax scores / weights
   const int64_t p = p0 + threadIdx.x;
   const bool live = p < len;
   float sc[kRMax];
+  float pw[kRMax];                    // weight of this thread's position for each head (0 past the end)
   if (KMODE == kWeights) {
     const float* wts = reinterpret_cast<const float*>(a.q);
 #pragma unroll
@@ -384,13 +369,15 @@ __global__ __launch_bounds__(kThreads) void decode_tile_kernel(DecodeArgs a, Cod
         w = wts[(q_row0 + r) * len + p];
         if (w < a.threshold) w = 0.0f;
       }
-      p_s[r][threadIdx.x] = w;
+      pw[r] = w;
     }
   } else {
     if (live) {
       if (KMODE == kPackedK) {
-        const int64_t row = (int64_t)seq * a.k_seq_stride + (int64_t)kvh * a.k_head_stride + first + p;
-        score_packed<D, BITS>(a.k_packed + row * PDIM, cbk_s, q_s, sc);
+        float acc1[1][kRMax];
+        score_packed_uniform_q<D, BITS, 1>(&vrows_s[wave][lane * (PDIM | 1)], 0, cbk_s, qrow, acc1);
+#pragma unroll
+        for (int r = 0; r < kRMax; ++r) sc[r] = acc1[0][r];
         const float nrm = a.k_norms[(int64_t)seq * a.kn_seq_stride + (int64_t)kvh * a.kn_head_stride + first + p];
 #pragma unroll
         for (int r = 0; r < kRMax; ++r) sc[r] = ((sc[r] * nrm) * a.inv_dim) * a.attn_scale;
@@ -427,7 +414,7 @@ __global__ __launch_bounds__(kThreads) void decode_tile_kernel(DecodeArgs a, Cod
 #pragma unroll
     for (int r = 0; r < kRMax; ++r) {
       const float e = (mx[r] == -INFINITY) ? 0.0f : expf(sc[r] - mx[r]);
-      p_s[r][threadIdx.x] = e;
+      pw[r] = e;
       ls[r] = wave_sum(e);
       if (lane == 0) red_s[wave][r] = ls[r];
     }
@@ -442,7 +429,10 @@ __global__ __launch_bounds__(kThreads) void decode_tile_kernel(DecodeArgs a, Cod
   }
   __syncthreads();
 
-  // ---- phase 3: V accumulation in the rotated domain; wave w walks positions [64w, 64w+64)
+  // ---- phase 3: V accumulation in the rotated domain; wave w walks positions [64w, 64w+64).
+  // The wave's packed rows come in with coalesced loads and are read back from LDS; the weight of position
+  // 64w + j (held by lane j of this same wave) and its norm reach the arithmetic as scalar operands through
+  // v_readlane, so the loop has no global load and no LDS read of weights.
   float acc[kRMax][EPL];
 #pragma unroll
   for (int r = 0; r < kRMax; ++r)
@@ -456,20 +446,35 @@ __global__ __launch_bounds__(kThreads) void decode_tile_kernel(DecodeArgs a, Cod
     wsh[i] = (e % VPW) * BITS;
   }
   const int t_begin = wave * TQ_WAVE;
-  const int t_end = (int)min((int64_t)(t_begin + TQ_WAVE), len - p0);
+  const int n_here = (int)max((int64_t)0, min((int64_t)TQ_WAVE, len - p0 - t_begin));       // uniform over the wave
   const int64_t vrow0 = (int64_t)seq * a.v_seq_stride + (int64_t)kvh * a.v_head_stride + first + p0;
   const int64_t vnrow0 = (int64_t)seq * a.vn_seq_stride + (int64_t)kvh * a.vn_head_stride + first + p0;
-  for (int t = t_begin; t < t_end; ++t) {
-    const uint32_t* vrow = a.v_packed + (vrow0 + t) * PDIM;
-    const float nrm = a.v_norms[vnrow0 + t];
-    float c[EPL];
+  stage_rows<PDIM>(a.v_packed + (vrow0 + t_begin) * PDIM, n_here, vrows_s[wave], lane);
+  const float my_nrm = (lane < n_here) ? a.v_norms[vnrow0 + t_begin + lane] : 0.0f;
+  __builtin_amdgcn_wave_barrier();                      // the rows are read back by this wave only; LDS operations of a wave complete in order
+  // software pipeline: the packed words of position j + 2 and the centroids of position j + 1 are fetched from
+  // LDS while the multiply-adds of position j run (rows 64 and 65 of the wave's area exist and are never used)
+  const uint32_t* vrows = vrows_s[wave];
+  uint32_t wnext[EPL];
+  float cnext[EPL];
 #pragma unroll
-    for (int i = 0; i < EPL; ++i) c[i] = cbv_s[(vrow[widx[i]] >> wsh[i]) & Pk<BITS>::MASK];
+  for (int i = 0; i < EPL; ++i) cnext[i] = cbv_s[(vrows[widx[i]] >> wsh[i]) & Pk<BITS>::MASK];
+#pragma unroll
+  for (int i = 0; i < EPL; ++i) wnext[i] = vrows[(PDIM | 1) + widx[i]];
+  for (int j = 0; j < n_here; ++j) {
+    float cn[EPL];
+    const float nrm = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_nrm), j));
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) cn[i] = cnext[i] * nrm;
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) cnext[i] = cbv_s[(wnext[i] >> wsh[i]) & Pk<BITS>::MASK];
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) wnext[i] = vrows[(j + 2) * (PDIM | 1) + widx[i]];
 #pragma unroll
     for (int r = 0; r < kRMax; ++r) {
-      const float wn = p_s[r][t] * nrm;
+      const float w = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, pw[r]), j));
 #pragma unroll
-      for (int i = 0; i < EPL; ++i) acc[r][i] += wn * c[i];
+      for (int i = 0; i < EPL; ++i) acc[r][i] = __builtin_fmaf(w, cn[i], acc[r][i]);
     }
   }
 #pragma unroll
