@@ -484,19 +484,27 @@ __global__ __launch_bounds__(256) void prefill_merge_kernel(const float* __restr
 
 struct SplitPlan { int n_splits, cap; int64_t split_len; };
 
-// Enough workgroups to fill 256 CUs a few times over, at least 8 blocks of positions per split.
-// cap bounds n_splits for every shorter kv_len too (n_splits itself is not monotone in kv_len),
-// so a workspace sized with cap(kv_len) serves the causal launch, which may see fewer positions.
+// Splits of the key positions: a workgroup fills a CU (LDS), so the launch runs in rounds of 256 workgroups and
+// its duration goes as rounds * split length, i.e. as ceil(columns * n / 256) / n for n splits of
+// columns = row blocks * query heads.  The smallest n within 3 % of the best such figure is taken (fewer splits =
+// less merge traffic: 4 at benchmark configuration 5, one workgroup per CU), with at least 8 blocks of positions
+// per split and at most 32 splits.  cap bounds n_splits for every shorter kv_len too (the causal launch may see
+// fewer positions than the workspace was sized for).
 SplitPlan plan_splits(int n_q, int64_t n_rows, int64_t kv_len) {
   const int64_t row_blocks = (n_rows + kWgRows - 1) / kWgRows;
   const int64_t blocks = (kv_len + kBlkPos - 1) / kBlkPos;
-  int64_t want = (1024 + row_blocks * n_q - 1) / (row_blocks * n_q);
-  const int64_t most = blocks / 8 > 0 ? blocks / 8 : 1;
-  if (want > most) want = most;
-  if (want < 1) want = 1;
+  const int64_t cols = row_blocks * n_q;
+  int64_t most = blocks / 8 > 0 ? blocks / 8 : 1;
+  if (most > 32) most = 32;
+  int64_t want = 1;
+  double best = 1e30;
+  for (int64_t n = 1; n <= most; ++n) {
+    const double cost = (double)((cols * n + 255) / 256) / (double)n;
+    if (cost < best * 0.97) { best = cost; want = n; }
+  }
   const int64_t per = (blocks + want - 1) / want;
   SplitPlan p;
-  p.cap = (int)want;
+  p.cap = (int)want;      // the scan is a prefix of itself for any shorter kv_len, so its choice there is <= want
   p.split_len = per * kBlkPos;
   p.n_splits = (int)((blocks + per - 1) / per);
   if (p.n_splits < 1) p.n_splits = 1;
