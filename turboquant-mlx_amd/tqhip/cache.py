@@ -183,6 +183,15 @@ class TurboQuantKVCache:
         return buf, alloc
 
     # ---------------------------------------------------------------- cache.py:131-218
+    def _zero_like(self, t: torch.Tensor) -> torch.Tensor:
+        """A zero scalar of t's dtype on t's device, made once: the source of the stride-0 placeholders
+        (a fresh one per step would cost a fill launch each)."""
+        key = (t.dtype, t.device)
+        z = self.__dict__.setdefault("_zero_scalars", {}).get(key)
+        if z is None:
+            z = self._zero_scalars[key] = t.new_zeros(())
+        return z
+
     def update_and_fetch(self, keys: torch.Tensor, values: torch.Tensor):
         B, H, S, k_dim = keys.shape
         v_dim = values.shape[3]
@@ -201,8 +210,8 @@ class TurboQuantKVCache:
 
         if self.fused:
             # zero placeholders of the right shape that own no memory (stride-0 views)
-            return (keys.new_zeros(()).expand(B, H, total, k_dim),
-                    values.new_zeros(()).expand(B, H, total, v_dim))
+            return (self._zero_like(keys).expand(B, H, total, k_dim),
+                    self._zero_like(values).expand(B, H, total, v_dim))
 
         incremental = S <= 4 and self._v_deq_buf is not None and self._deq_offset == prev
 
@@ -215,7 +224,7 @@ class TurboQuantKVCache:
                 self._v_deq_buf, self._deq_alloc = self._prefill_buffer(
                     self.v_packed, self.v_norms, self._v_q, v_dim, B, H, total, values.dtype)
             self._deq_offset = total
-            return keys.new_zeros(()).expand(B, H, total, k_dim), self._v_deq_buf[..., :total, :]
+            return self._zero_like(keys).expand(B, H, total, k_dim), self._v_deq_buf[..., :total, :]
 
         if incremental:
             self._k_deq_buf = self._incremental(self.k_packed, self.k_norms, self._k_q, k_dim,
