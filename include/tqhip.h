@@ -282,6 +282,23 @@ int tq_flash_sparse_decode(const float* q_rot,
                            const tq_decode_shape* shape /* host */, tq_stream_t stream);
 
 /*
+ * turboquant_attention in one call, from the query itself (fused_attention.py:56-121: prerotate_query ->
+ * prerot_fused_qk_scores -> * attn_scale + mask -> softmax -> sparse_v_matvec): tq_flash_decode
+ * (threshold == 0) or tq_flash_sparse_decode (threshold > 0) with the pre-rotation q_rot = butterfly(q * k_signs)
+ * of tq_prerotate_query done inside the kernels (same bits), which saves the separate launch and the q_rot
+ * tensor.  q [n_seq, n_kv*n_rep, dim] of q_dtype; k_signs [dim] f32 on the device.  Workspace:
+ * tq_workspace_bytes(TQ_OP_FLASH_DECODE, ...) for threshold == 0, tq_vonly_sparse_workspace_bytes otherwise.
+ * Matrix-core shape only (dim 128, 3-bit, n_rep <= 16, non-empty cache; TQ_ERR_UNSUPPORTED otherwise: call
+ * tq_prerotate_query and tq_flash_decode).
+ */
+int tq_flash_decode_from_q(const void* q, int q_dtype, const float* k_signs,
+                           const uint32_t* k_packed, const float* k_norms,
+                           const uint32_t* v_packed, const float* v_norms,
+                           const float* k_centroids, const float* v_centroids, const float* v_signs,
+                           float threshold, void* out, void* workspace, size_t workspace_bytes,
+                           const tq_decode_shape* shape /* host */, tq_stream_t stream);
+
+/*
  * Bytes of workspace the op needs for this shape (host computation, no GPU call).  The workspace
  * holds per-tile partial results between the two passes of a call; its contents need not be
  * preserved or cleared between calls.  Calls that share a workspace must be ordered (same stream);

@@ -1568,3 +1568,58 @@ def test_decode_sweep_flash_sparse(tq, seed):
         close(got[i], o.turboquant_attention_single(q[i], kpi, kni, vpi, vni, c, ks, c, vs, D, bits, sc,
                                                     sparse_v_threshold=thr, mask=mi),
               extra=threshold_slack(w, thr, vpi, vni, c, vs, n_rep, 1e-2))
+
+
+# ------------------------------------------------------------------ decode step from the query itself (rotation in-kernel)
+
+@pytest.mark.parametrize("qdt", ["float32", "float16", "bfloat16"])
+@pytest.mark.parametrize("case", ["tile", "stream_ragged", "masked", "threshold"])
+def test_flash_decode_from_q_equals_prerotate_then_flash(tq, qdt, case):
+    """tq_flash_decode_from_q rotates the query inside the attention kernels with the stage order of
+    tq_prerotate_query: the result must be IDENTICAL to prerotate_query followed by flash_decode, for every
+    query dtype, on the tile pass, the streaming pass (ragged batch), with a mask and with a threshold."""
+    rng = np.random.default_rng(sum(map(ord, qdt + case)))
+    D, bits, sc = 128, 3, 1 / math.sqrt(128)
+    n_kv, n_rep = (8, 4) if case == "stream_ragged" else (4, 7)
+    n_q = n_kv * n_rep
+    c, b = tables(bits)
+    ks, vs = o.random_diagonal_sign(D, 42), o.random_diagonal_sign(D, 43)
+    kw = {}
+    if case == "stream_ragged":
+        lens = np.array([4097, 2561, 1025, 7000, 1, 3333, 5121, 6143])
+        offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        assert _flash_plan(tq, len(lens), n_kv, int(lens.max()), True) >= 2
+        shape, n_seq = (n_kv, int(offs[-1])), len(lens)
+        kw = dict(seq_offsets=dev(offs), max_seq_len=int(lens.max()))
+    else:
+        n_seq, T = 2, 1111
+        shape = (n_seq, n_kv, T + 13)
+        kw = dict(seq_len=T)
+        if case == "masked":
+            kw["mask"] = dev(_draw_mask(rng, "head", n_seq, n_q, T))
+        if case == "threshold":
+            kw["sparse_v_threshold"] = 1e-4
+    kp = o.pack_indices(rng.integers(0, 8, size=shape + (D,)).astype(np.uint8), bits)
+    vp = o.pack_indices(rng.integers(0, 8, size=shape + (D,)).astype(np.uint8), bits)
+    kn = (rng.random(shape) * 12 + 6).astype(F32)
+    vn = (rng.random(shape) + 0.5).astype(F32)
+    q = torch.from_numpy(rng.standard_normal((n_seq, n_q, D)).astype(F32)).to(getattr(torch, qdt)).cuda()
+    q_rot = tq.prerotate_query(q.reshape(-1, D), dev(ks)).reshape(n_seq, n_q, D)
+    two = tq.flash_decode(q_rot, dev(kp), dev(kn), dev(vp), dev(vn), c, c, dev(vs), D, bits, sc, n_rep=n_rep, **kw)
+    one = tq.flash_decode_from_q(q, dev(ks), dev(kp), dev(kn), dev(vp), dev(vn), c, c, dev(vs), D, bits, sc, n_rep=n_rep, **kw)
+    assert torch.equal(one, two)
+    assert torch.isfinite(one).all()
+
+
+def test_flash_decode_from_q_against_oracle_and_shape_limits(tq):
+    rng = np.random.default_rng(77)
+    n_kv, n_rep, T, D, bits, sc = 2, 16, 700, 128, 3, 1 / math.sqrt(128)
+    c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, n_kv, T, D, bits)
+    q = rng.standard_normal((1, n_kv * n_rep, D)).astype(np.float16)
+    got = host(tq.flash_decode_from_q(dev(q), dev(ks), dev(kp[None]), dev(kn[None]), dev(vp[None]), dev(vn[None]), c, c,
+                                      dev(vs), D, bits, sc, n_rep=n_rep))
+    close(got[0], o.turboquant_attention_single(q[0].astype(F32), kp, kn, vp, vn, c, ks, c, vs, D, bits, sc))
+    c4, ks4, vs4, K4, V4, kp4, kn4, vp4, vn4 = kv_fixture(rng, 2, 64, 64, 4)
+    with pytest.raises(ValueError, match="prerotate_query"):
+        tq.flash_decode_from_q(torch.zeros((1, 2, 64), device="cuda"), dev(ks4), dev(kp4[None]), dev(kn4[None]),
+                               dev(vp4[None]), dev(vn4[None]), c4, c4, dev(vs4), 64, 4, 0.125, n_rep=1)

@@ -750,7 +750,8 @@ int launch_packed_mfma(const float* q_rot_or_weights, const uint32_t* k_packed, 
                        const uint32_t* v_packed, const float* v_norms, const float* k_centroids,
                        const float* v_centroids, const float* v_signs, void* out, void* workspace,
                        size_t workspace_bytes, const tq_decode_shape& sh, float threshold, hipStream_t stream,
-                       const char* who) {
+                       const char* who, const void* q_raw = nullptr, int q_dtype = TQ_F32,
+                       const float* k_signs = nullptr) {
   const int n_q = sh.n_kv_heads * sh.n_rep;
   const int n_tiles = (int)((sh.seq_len + tqm::kTilePos - 1) / tqm::kTilePos);
   const size_t need = (size_t)sh.n_seq * n_q * n_tiles * (tqm::kD + 2) * sizeof(float);
@@ -759,6 +760,7 @@ int launch_packed_mfma(const float* q_rot_or_weights, const uint32_t* k_packed, 
   if (!tq::aligned(workspace, 16)) return tq::fail(TQ_ERR_ALIGN, "%s: workspace must be 16-byte aligned", who);
   tqm::PackedArgs a{};
   if (MODE == tqm::kWeights) a.weights = q_rot_or_weights; else a.q_rot = q_rot_or_weights;
+  a.q_raw = q_raw; a.q_dtype = q_dtype; a.k_signs = k_signs;      // set: the kernel rotates the query itself
   a.k_packed = k_packed; a.k_norms = k_norms; a.v_packed = v_packed; a.v_norms = v_norms;
   a.seq_offsets = sh.seq_offsets; a.mask = sh.mask;
   a.ws_S = (float*)workspace;
@@ -897,7 +899,8 @@ int launch_vonly_sparse(const void* q, int q_dtype, const void* k_f16, const uin
 int launch_flash_sparse(const float* q_rot, const uint32_t* k_packed, const float* k_norms, const uint32_t* v_packed,
                         const float* v_norms, const float* k_centroids, const float* v_centroids, const float* v_signs,
                         float threshold, void* out, void* workspace, size_t workspace_bytes, const tq_decode_shape& sh,
-                        hipStream_t stream) {
+                        hipStream_t stream, const void* q_raw = nullptr, int q_dtype = TQ_F32,
+                        const float* k_signs = nullptr) {
   const char* who = "tq_flash_sparse_decode";
   const int n_q = sh.n_kv_heads * sh.n_rep;
   const int64_t t_pad = (sh.seq_len + 3) & ~(int64_t)3;
@@ -913,6 +916,7 @@ int launch_flash_sparse(const float* q_rot, const uint32_t* k_packed, const floa
 
   tqm::PackedArgs a{};
   a.q_rot = q_rot; a.k_packed = k_packed; a.k_norms = k_norms;
+  a.q_raw = q_raw; a.q_dtype = q_dtype; a.k_signs = k_signs;
   a.seq_offsets = sh.seq_offsets; a.mask = sh.mask;
   a.scores = scores; a.stats_out = stats; a.w_stride = t_pad;
   a.seq_len = sh.seq_len;
@@ -1157,4 +1161,30 @@ extern "C" int tq_flash_sparse_decode(const float* q_rot, const uint32_t* k_pack
                                         "(compose tq_prerot_qk_scores, tq_softmax_rows and tq_sparse_v_matvec otherwise)", who);
   return launch_flash_sparse(q_rot, k_packed, k_norms, v_packed, v_norms, k_centroids, v_centroids, v_signs, threshold,
                              out, workspace, workspace_bytes, *shape, (hipStream_t)stream_);
+}
+
+extern "C" int tq_flash_decode_from_q(const void* q, int q_dtype, const float* k_signs, const uint32_t* k_packed,
+                                      const float* k_norms, const uint32_t* v_packed, const float* v_norms,
+                                      const float* k_centroids, const float* v_centroids, const float* v_signs,
+                                      float threshold, void* out, void* workspace, size_t workspace_bytes,
+                                      const tq_decode_shape* shape, tq_stream_t stream_) {
+  const char* who = "tq_flash_decode_from_q";
+  if (int rc = check_shape(shape, who, 128)) return rc;
+  if (tq::check_dtype(q_dtype)) return tq::fail(TQ_ERR_DTYPE, "%s: unknown q_dtype %d", who, q_dtype);
+  if (!q || !k_signs || !k_centroids || !v_centroids || !v_signs || !out) return tq::fail(TQ_ERR_NULL, "%s: null pointer", who);
+  if (shape->seq_len > 0 && (!k_packed || !k_norms || !v_packed || !v_norms))
+    return tq::fail(TQ_ERR_NULL, "%s: null pointer", who);
+  if (!(threshold >= 0.0f)) return tq::fail(TQ_ERR_ARG, "%s: threshold must be >= 0", who);
+  if (!(shape->dim == 128 && shape->bits == 3 && shape->n_rep <= tqm::kHeadsMax && shape->seq_len > 0 &&
+        tq::aligned(q, (int)tq::dtype_size(q_dtype))))
+    return tq::fail(TQ_ERR_UNSUPPORTED, "%s: dim 128, 3-bit, n_rep <= 16 and a non-empty cache only "
+                                        "(call tq_prerotate_query and tq_flash_decode otherwise)", who);
+  hipStream_t stream = (hipStream_t)stream_;
+  if (threshold > 0.0f)
+    return launch_flash_sparse(nullptr, k_packed, k_norms, v_packed, v_norms, k_centroids, v_centroids, v_signs, threshold,
+                               out, workspace, workspace_bytes, *shape, stream, q, q_dtype, k_signs);
+  tq_decode_shape sh = *shape;
+  sh.allow_mma = 1;
+  return launch_packed_mfma<tqm::kFlash>(nullptr, k_packed, k_norms, v_packed, v_norms, k_centroids, v_centroids, v_signs,
+                                         out, workspace, workspace_bytes, sh, 0.0f, stream, who, q, q_dtype, k_signs);
 }

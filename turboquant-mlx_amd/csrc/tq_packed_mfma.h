@@ -24,7 +24,10 @@ namespace tqm {
 enum PackedMode { kFlash = 0, kScores = 1, kWeights = 2, kSoftWeights = 3, kSoftScores = 4 };
 
 struct PackedArgs {
-  const float* q_rot;         // kFlash / kScores: [n_seq, n_q, 128] f32
+  const float* q_rot;         // kFlash / kScores: [n_seq, n_q, 128] f32, pre-rotated; or NULL with q_raw set
+  const void* q_raw;          // the query itself, [n_seq, n_q, 128] of q_dtype: rotated inside the kernel
+  const float* k_signs;       //   (q * k_signs, raw butterfly: the bits of tq_prerotate_query)
+  int32_t q_dtype;
   const float* weights;       // kWeights: [n_seq * n_q, w_stride] f32 weights; kSoftWeights: scores in log2 units
   const float* stats;         // kSoftWeights: [n_seq * n_kv, n_tiles_max, n_rep, 2] (maximum, sum of 2^(s - maximum)) per tile
   int64_t w_stride;           // floats per row of `weights`
@@ -107,6 +110,46 @@ __device__ __forceinline__ void fill_lut(uint32_t* lut, const Codebook& cb, int 
   }
 }
 
+// Query rows of one kv head, rotated in place of a separate pre-rotation launch: wave w takes rows w, w + N_WAVES, ...
+// of the 16 (rows at or past n_rep are zeros), lane l the elements l and l + 64; q * signs, the raw butterfly of
+// tq_prerotate_query (same stage order, hence the same bits), then the fp16 value and the fp16 remainder of that
+// rounding into q_s / ql_s.  Runs while the key/value loads are in flight.
+template <int N_WAVES>
+__device__ __forceinline__ void rotate_query_rows(const void* q_raw, int q_dtype, const float* k_signs, int64_t q_row0,
+                                                  int n_rep, int wave, int lane, uint32_t (*q_s)[kD / 2],
+                                                  uint32_t (*ql_s)[kD / 2]) {
+  const float s0 = k_signs[lane], s1 = k_signs[lane + 64];
+#pragma unroll
+  for (int it = 0; it < kHeadsMax / N_WAVES; ++it) {
+    const int r = wave + it * N_WAVES;
+    float v[2] = {0.0f, 0.0f};
+    if (r < n_rep) {
+      const int64_t base = (q_row0 + r) * kD;
+      if (q_dtype == TQ_F32) {
+        v[0] = reinterpret_cast<const float*>(q_raw)[base + lane];
+        v[1] = reinterpret_cast<const float*>(q_raw)[base + lane + 64];
+      } else if (q_dtype == TQ_F16) {
+        v[0] = __half2float(reinterpret_cast<const __half*>(q_raw)[base + lane]);
+        v[1] = __half2float(reinterpret_cast<const __half*>(q_raw)[base + lane + 64]);
+      } else {
+        v[0] = __uint_as_float((uint32_t)reinterpret_cast<const uint16_t*>(q_raw)[base + lane] << 16);
+        v[1] = __uint_as_float((uint32_t)reinterpret_cast<const uint16_t*>(q_raw)[base + lane + 64] << 16);
+      }
+      v[0] *= s0;
+      v[1] *= s1;
+    }
+    raw_butterfly<kD>(v, lane);
+    __half* hi = reinterpret_cast<__half*>(&q_s[r][0]);
+    __half* lo = reinterpret_cast<__half*>(&ql_s[r][0]);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const __half h = __float2half_rn(v[i]);
+      hi[lane + 64 * i] = h;
+      lo[lane + 64 * i] = __float2half_rn(v[i] - __half2float(h));
+    }
+  }
+}
+
 // grid = (n_tiles_max, n_kv, n_seq), 512 threads.
 template <int MODE>
 __global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(4, 4)))
@@ -147,7 +190,7 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
 
   // ---- loads ----------------------------------------------------------------------------------------
   float2 my_q[2];
-  if (HAS_K) {
+  if (HAS_K && !a.q_raw) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int w = tid + i * kMfmaThreads;                           // word = 2 consecutive elements
@@ -243,12 +286,16 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
   if (HAS_K) fill_lut(lutk_s, kcb, tid);
   if (HAS_V) fill_lut(lutv_s, vcb, tid);
   if (HAS_K) {
+    if (a.q_raw) {
+      rotate_query_rows<kWaves>(a.q_raw, a.q_dtype, a.k_signs, q_row0, n_rep, wave, lane, q_s, ql_s);
+    } else {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const __half2 h = __floats2half2_rn(my_q[i].x, my_q[i].y);
-      const float2 back = __half22float2(h);
-      (&q_s[0][0])[tid + i * kMfmaThreads] = *reinterpret_cast<const uint32_t*>(&h);
-      (&ql_s[0][0])[tid + i * kMfmaThreads] = pack_h2(my_q[i].x - back.x, my_q[i].y - back.y);
+      for (int i = 0; i < 2; ++i) {
+        const __half2 h = __floats2half2_rn(my_q[i].x, my_q[i].y);
+        const float2 back = __half22float2(h);
+        (&q_s[0][0])[tid + i * kMfmaThreads] = *reinterpret_cast<const uint32_t*>(&h);
+        (&ql_s[0][0])[tid + i * kMfmaThreads] = pack_h2(my_q[i].x - back.x, my_q[i].y - back.y);
+      }
     }
     // the score scale rides on the key norm: log2 units for the softmax, plain units for kScores
     kn_s[wave][lane] = my_kn * (SOFT ? a.score_scale * kLog2e : a.score_scale);
@@ -601,10 +648,12 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
   };
 
   float2 my_q[4];
+  if (!a.q_raw) {
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int w = tid + i * kSThreads;                                  // word = 2 consecutive elements
-    my_q[i] = (w < n_rep * (kD / 2)) ? reinterpret_cast<const float2*>(a.q_rot + q_row0 * kD)[w] : make_float2(0.f, 0.f);
+    for (int i = 0; i < 4; ++i) {
+      const int w = tid + i * kSThreads;                                  // word = 2 consecutive elements
+      my_q[i] = (w < n_rep * (kD / 2)) ? reinterpret_cast<const float2*>(a.q_rot + q_row0 * kD)[w] : make_float2(0.f, 0.f);
+    }
   }
   u4 kqA[4], vqA[4], kqB[4], vqB[4];
   float knA, vnA, knB = 0.0f, vnB = 0.0f;
@@ -612,12 +661,16 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
 
   fill_lut(lutk_s, kcb, tid);
   fill_lut(lutv_s, vcb, tid - 64);
+  if (a.q_raw) {
+    rotate_query_rows<kSWaves>(a.q_raw, a.q_dtype, a.k_signs, q_row0, n_rep, wave, lane, q_s, ql_s);
+  } else {
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const __half2 h = __floats2half2_rn(my_q[i].x, my_q[i].y);
-    const float2 back = __half22float2(h);
-    (&q_s[0][0])[tid + i * kSThreads] = *reinterpret_cast<const uint32_t*>(&h);
-    (&ql_s[0][0])[tid + i * kSThreads] = pack_h2(my_q[i].x - back.x, my_q[i].y - back.y);
+    for (int i = 0; i < 4; ++i) {
+      const __half2 h = __floats2half2_rn(my_q[i].x, my_q[i].y);
+      const float2 back = __half22float2(h);
+      (&q_s[0][0])[tid + i * kSThreads] = *reinterpret_cast<const uint32_t*>(&h);
+      (&ql_s[0][0])[tid + i * kSThreads] = pack_h2(my_q[i].x - back.x, my_q[i].y - back.y);
+    }
   }
   __syncthreads();
 

@@ -22,6 +22,7 @@ from .ops import (
     count_active_positions,
     flash_attention_turboquant,
     flash_decode,
+    flash_decode_from_q,
     prefill_attention,
     vonly_decode,
     dense_qk_scores,

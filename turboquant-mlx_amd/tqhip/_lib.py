@@ -57,6 +57,7 @@ PROTOTYPES = {
     "tq_vonly_decode_attn_phases": (_i, [_p, _i, _p, _p, _p, _fp, _p, _p, _p, _z, C.POINTER(DecodeShape), _i, _p]),
     "tq_vonly_sparse_decode_attn": (_i, [_p, _i, _p, _p, _p, _fp, _p, _f, _p, _p, _z, C.POINTER(DecodeShape), _p]),
     "tq_vonly_sparse_workspace_bytes": (_z, [_i, _i, _l]),
+    "tq_flash_decode_from_q": (_i, [_p, _i, _p, _p, _p, _p, _p, _fp, _fp, _p, _f, _p, _p, _z, C.POINTER(DecodeShape), _p]),
     "tq_flash_sparse_decode": (_i, [_p, _p, _p, _p, _p, _fp, _fp, _p, _f, _p, _p, _z, C.POINTER(DecodeShape), _p]),
     "tq_workspace_bytes": (_z, [_i, _i, _i, _l, _i]),
     "tq_prefill_attn": (_i, [_p, _i, _p, _p, _p, _p, _fp, _fp, _p, _p, _p, _i, _p, _z, _i, _i, _l, _l, _l,

@@ -52,14 +52,20 @@ def turboquant_attention(queries: torch.Tensor, cache, attn_scale: float, mask=N
 
     one_call_thr = thr > 0.0 and ops.vonly_sparse_supported(dim, bits, n_rep) and total > 0 and dim == cache._v_dim
     if fused and v_buffer is None and (thr == 0.0 or one_call_thr):
-        q_rot = ops.prerotate_query(queries.reshape(B * n_q, dim), kq.signs).reshape(B, n_q, dim)
         m = None
         if mask is not None:
             m = torch.stack([_mask_rows(mask, b, n_q, total).expand(n_q, total) for b in range(B)])
         od = queries.dtype if queries.dtype in (torch.float16, torch.bfloat16, torch.float32) else torch.float32
-        out = ops.flash_decode(q_rot, cache.k_packed, cache.k_norms, cache.v_packed, cache.v_norms,
-                               kq.centroids, vq.centroids, vq.signs, dim, bits, attn_scale, n_rep=n_rep,
-                               seq_len=total, mask=m, out_dtype=od, sparse_v_threshold=thr)
+        if ops.vonly_sparse_supported(dim, bits, n_rep) and total > 0 and dim == cache._v_dim:
+            # one call: the kernels rotate the query themselves
+            out = ops.flash_decode_from_q(queries[:, :, 0, :], kq.signs, cache.k_packed, cache.k_norms, cache.v_packed,
+                                          cache.v_norms, kq.centroids, vq.centroids, vq.signs, dim, bits, attn_scale,
+                                          n_rep=n_rep, seq_len=total, mask=m, out_dtype=od, sparse_v_threshold=thr)
+        else:
+            q_rot = ops.prerotate_query(queries.reshape(B * n_q, dim), kq.signs).reshape(B, n_q, dim)
+            out = ops.flash_decode(q_rot, cache.k_packed, cache.k_norms, cache.v_packed, cache.v_norms,
+                                   kq.centroids, vq.centroids, vq.signs, dim, bits, attn_scale, n_rep=n_rep,
+                                   seq_len=total, mask=m, out_dtype=od, sparse_v_threshold=thr)
         out = out[:, :, None, :]
         return out if out.dtype == queries.dtype else out.to(queries.dtype)
 

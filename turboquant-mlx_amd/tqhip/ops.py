@@ -519,6 +519,61 @@ def flash_decode(q_rot: torch.Tensor, k_packed, k_norms, v_packed, v_norms, k_ce
     return out
 
 
+def flash_decode_from_q(q: torch.Tensor, k_signs, k_packed, k_norms, v_packed, v_norms, k_centroids, v_centroids,
+                        v_signs, dim: int, bits: int, attn_scale: float, *, n_rep: int = 1,
+                        seq_len: int | None = None, seq_offsets: torch.Tensor | None = None,
+                        max_seq_len: int | None = None, mask=None, out_dtype=torch.float32,
+                        sparse_v_threshold: float = 0.0) -> torch.Tensor:
+    """The decode step of turboquant_attention (fused_attention.py:56-121) in ONE library call from the query
+    itself: the pre-rotation of prerotate_query happens inside the attention kernels (tq_flash_decode_from_q).
+    q (n_seq, n_q, dim) fp16 / bf16 / float32; other arguments as flash_decode.  Matrix-core shapes only
+    (vonly_sparse_supported); callers fall back to prerotate_query + flash_decode otherwise."""
+    _need_gpu(q, k_packed, k_norms, v_packed, v_norms, seq_offsets)
+    n_seq, n_q, _ = q.shape
+    ragged = seq_offsets is not None
+    n_kv = k_norms.shape[-2]
+    _check_gqa(n_q, n_kv, n_rep)
+    if not vonly_sparse_supported(dim, bits, n_rep):
+        raise ValueError("flash_decode_from_q needs dim 128, 3-bit, n_rep <= 16; use prerotate_query + flash_decode")
+    pd = packed_dim(dim, bits)
+    if q.dtype not in _DTYPES:
+        q = q.float()
+    q = q.contiguous()
+    k_packed, ks = _kv_layout(_u32(k_packed), pd, ragged)
+    v_packed, vs = _kv_layout(_u32(v_packed), pd, ragged)
+    k_norms, kns = _norm_layout(k_norms if k_norms.dtype == torch.float32 else k_norms.to(torch.float32))
+    v_norms, vns = _norm_layout(v_norms if v_norms.dtype == torch.float32 else v_norms.to(torch.float32))
+    if ragged:
+        if max_seq_len is None:
+            raise ValueError("max_seq_len is required with seq_offsets")
+        if seq_offsets.dtype != torch.int32 or seq_offsets.numel() != n_seq + 1:
+            raise ValueError("seq_offsets must be int32 with n_seq + 1 entries")
+        T = int(max_seq_len)
+    else:
+        T = int(seq_len if seq_len is not None else k_norms.shape[-1])
+    if T <= 0:
+        raise ValueError("flash_decode_from_q needs a non-empty cache")
+    k_signs = _as_f32_dev(k_signs, q)
+    v_signs = _as_f32_dev(v_signs, q)
+    mask, ms = _mask_layout(mask, n_seq, n_q, T, q.device)
+    out = torch.empty((n_seq, n_q, dim), dtype=out_dtype, device=q.device)
+    sh = _decode_shape(n_seq=n_seq, n_kv=n_kv, n_rep=n_rep, dim=dim, bits=bits, block_size=16,
+                       seq_len=T, seq_offsets=seq_offsets, k_strides=ks, kn_strides=kns, v_strides=vs,
+                       vn_strides=vns, mask=mask, mask_strides=ms, attn_scale=attn_scale, out_dtype=out_dtype,
+                       allow_mma=True)
+    lib = _lib.load()
+    stream = _stream(q)
+    thr = float(sparse_v_threshold) if sparse_v_threshold and sparse_v_threshold > 0.0 else 0.0
+    need = (lib.tq_vonly_sparse_workspace_bytes(n_seq, n_q, T) if thr > 0.0
+            else lib.tq_workspace_bytes(_lib.TQ_OP_FLASH_DECODE, n_seq, n_q, T, dim))
+    ws = _workspace(q.device, stream.value or 0, need)
+    _lib.check(lib.tq_flash_decode_from_q(
+        _ptr(q), _dt(q), _ptr(k_signs), _ptr(k_packed), _ptr(k_norms), _ptr(v_packed), _ptr(v_norms),
+        _host_table(k_centroids), _host_table(v_centroids), _ptr(v_signs), thr, _ptr(out),
+        _ptr(ws), ws.numel(), C.byref(sh), stream))
+    return out
+
+
 def flash_attention_turboquant(q_rot, k_packed, k_norms, v_packed, v_norms, k_centroids, v_centroids,
                                v_signs, dim: int, bits: int, attn_scale: float, block_size: int = 16,
                                n_rep: int = 1, precision: str = "fp16") -> torch.Tensor:
