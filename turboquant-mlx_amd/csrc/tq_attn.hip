@@ -238,16 +238,23 @@ __global__ __launch_bounds__(kThreads) void dense_scores_kernel(const QT* __rest
 }
 
 // ---------------------------------------------------------------- row softmax
-// grid = (n_rows, n_chunks).  Every workgroup takes the maximum and the sum of exponentials over the WHOLE row
-// (two sweeps; with several chunks per row the row comes from L2 for all but the first reader) and then
-// writes the weights of its own chunk, so a few long rows still fill the chip with one launch and without
-// scratch memory.  16-byte accesses where the row is aligned.
-__global__ __launch_bounds__(kThreads) void softmax_rows_kernel(const float* __restrict__ scores,
+// grid = (n_rows, n_chunks).  Every workgroup takes the maximum and the sum of exponentials over the WHOLE row in
+// ONE sweep (online: a running maximum per thread, the sum rescaled when it moves) and then writes the weights of
+// its own chunk, so a few long rows still fill the chip with one launch and without scratch memory.  With
+// several chunks per row the row is read n_chunks times (from L2 for all but the first reader): the host keeps
+// n_chunks at about one workgroup per CU, since that re-reading is what bounds the launch.  Logits are kept in
+// log2 units (scale and mask times log2 e) so that e^x is one v_exp_f32.  16-byte accesses where the row is aligned.
+constexpr int kSmThreads = 256;
+constexpr int kSmWaves = kSmThreads / 64;
+
+__global__ __launch_bounds__(kSmThreads) void softmax_rows_kernel(const float* __restrict__ scores,
                                                                 const float* __restrict__ mask,
                                                                 int64_t mask_row_stride,
                                                                 float* __restrict__ weights, int64_t seq_len,
                                                                 float scale, int64_t chunk_len) {
-  __shared__ float red[kWaves];
+  __shared__ float red_m[kSmWaves], red_l[kSmWaves];
+  constexpr float kLog2eF = 1.44269504088896340736f;
+  const float scale2 = scale * kLog2eF;
   const int64_t row = blockIdx.x;
   const float* s = scores + row * seq_len;
   const float* mk = mask ? mask + row * mask_row_stride : nullptr;
@@ -258,58 +265,109 @@ __global__ __launch_bounds__(kThreads) void softmax_rows_kernel(const float* __r
                    (!mask || (((reinterpret_cast<uintptr_t>(mask) & 15) == 0) && ((mask_row_stride & 3) == 0)));
   auto logits4 = [&](int64_t p, float (&v)[4]) {                      // four consecutive logits (vec only)
     const float4 x = *reinterpret_cast<const float4*>(s + p);
-    v[0] = x.x * scale; v[1] = x.y * scale; v[2] = x.z * scale; v[3] = x.w * scale;
+    v[0] = x.x * scale2; v[1] = x.y * scale2; v[2] = x.z * scale2; v[3] = x.w * scale2;
     if (mk) {
       const float4 m4 = *reinterpret_cast<const float4*>(mk + p);
-      v[0] += m4.x; v[1] += m4.y; v[2] += m4.z; v[3] += m4.w;
+      v[0] = __builtin_fmaf(m4.x, kLog2eF, v[0]); v[1] = __builtin_fmaf(m4.y, kLog2eF, v[1]);
+      v[2] = __builtin_fmaf(m4.z, kLog2eF, v[2]); v[3] = __builtin_fmaf(m4.w, kLog2eF, v[3]);
     }
   };
   auto logit = [&](int64_t p) {
-    float v = s[p] * scale;
-    if (mk) v += mk[p];
+    float v = s[p] * scale2;
+    if (mk) v = __builtin_fmaf(mk[p], kLog2eF, v);
     return v;
   };
-  float m = -INFINITY;
+  // ---- one sweep: per-thread running maximum m and sum l of 2^(x - m); kSweep 16-byte pieces per step, all
+  // loads of a step issued before any is used
+  constexpr int kSweep = 8;
+  float m = -INFINITY, l = 0.0f;
   if (vec) {
-    for (int64_t p = 4 * (int64_t)threadIdx.x; p < seq_len; p += 4 * kThreads) {
-      float v[4];
-      logits4(p, v);
-      m = fmaxf(m, fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])));
+    // the pieces of step i + 1 are requested before those of step i are reduced
+    float4 nx[kSweep], nm[kSweep];
+    auto fetch = [&](int64_t p) {
+#pragma unroll
+      for (int u = 0; u < kSweep; ++u) {
+        const int64_t pu = p + (int64_t)u * 4 * kSmThreads;
+        const bool ok = pu < seq_len;
+        nx[u] = ok ? *reinterpret_cast<const float4*>(s + pu) : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+        if (mk) nm[u] = ok ? *reinterpret_cast<const float4*>(mk + pu) : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+    };
+    const int64_t step = 4 * (int64_t)kSmThreads * kSweep;
+    int64_t p = 4 * (int64_t)threadIdx.x;
+    if (p < seq_len) fetch(p);
+    for (; p < seq_len; p += step) {
+      float v[kSweep][4];
+#pragma unroll
+      for (int u = 0; u < kSweep; ++u) {
+        v[u][0] = nx[u].x * scale2; v[u][1] = nx[u].y * scale2; v[u][2] = nx[u].z * scale2; v[u][3] = nx[u].w * scale2;
+        if (mk) {
+          v[u][0] = __builtin_fmaf(nm[u].x, kLog2eF, v[u][0]); v[u][1] = __builtin_fmaf(nm[u].y, kLog2eF, v[u][1]);
+          v[u][2] = __builtin_fmaf(nm[u].z, kLog2eF, v[u][2]); v[u][3] = __builtin_fmaf(nm[u].w, kLog2eF, v[u][3]);
+        }
+      }
+      if (p + step < seq_len) fetch(p + step);
+      float mb = m;
+#pragma unroll
+      for (int u = 0; u < kSweep; ++u) mb = fmaxf(mb, fmaxf(fmaxf(v[u][0], v[u][1]), fmaxf(v[u][2], v[u][3])));
+      if (mb != -INFINITY) {
+        float add = 0.0f;
+#pragma unroll
+        for (int u = 0; u < kSweep; ++u)
+          add += (__builtin_amdgcn_exp2f(v[u][0] - mb) + __builtin_amdgcn_exp2f(v[u][1] - mb)) +
+                 (__builtin_amdgcn_exp2f(v[u][2] - mb) + __builtin_amdgcn_exp2f(v[u][3] - mb));
+        l = l * __builtin_amdgcn_exp2f(m - mb) + add;          // m = -inf: l is 0 and 2^-inf = 0
+        m = mb;
+      }
     }
   } else {
-    for (int64_t p = threadIdx.x; p < seq_len; p += kThreads) m = fmaxf(m, logit(p));
-  }
-  m = wave_max(m);
-  if (lane == 0) red[wave] = m;
-  __syncthreads();
-  m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-  __syncthreads();
-  if (m == -INFINITY) m = 0.0f;
-  float l = 0.0f;
-  if (vec) {
-    for (int64_t p = 4 * (int64_t)threadIdx.x; p < seq_len; p += 4 * kThreads) {
-      float v[4];
-      logits4(p, v);
-      l += (expf(v[0] - m) + expf(v[1] - m)) + (expf(v[2] - m) + expf(v[3] - m));
+    for (int64_t p = threadIdx.x; p < seq_len; p += kSmThreads) {
+      const float v = logit(p);
+      const float mb = fmaxf(m, v);
+      if (mb != -INFINITY) {
+        l = l * __builtin_amdgcn_exp2f(m - mb) + __builtin_amdgcn_exp2f(v - mb);
+        m = mb;
+      }
     }
-  } else {
-    for (int64_t p = threadIdx.x; p < seq_len; p += kThreads) l += expf(logit(p) - m);
   }
+  // ---- combine the threads: maximum first, then the sums rescaled to it
+  float M = wave_max(m);
+  if (lane == 0) red_m[wave] = M;
+  __syncthreads();
+  M = red_m[0];
+#pragma unroll
+  for (int i = 1; i < kSmWaves; ++i) M = fmaxf(M, red_m[i]);
+  if (M == -INFINITY) M = 0.0f;                                  // a fully masked row: l = 0 and every weight is 0 * inf = NaN, as a softmax over nothing is
+  l = (m == -INFINITY) ? 0.0f : l * __builtin_amdgcn_exp2f(m - M);
   l = wave_sum(l);
-  if (lane == 0) red[wave] = l;
+  if (lane == 0) red_l[wave] = l;
   __syncthreads();
-  l = (red[0] + red[1]) + (red[2] + red[3]);
+  l = 0.0f;
+#pragma unroll
+  for (int i = 0; i < kSmWaves; ++i) l += red_l[i];
+  const float inv_l = 1.0f / l;
   const int64_t p_lo = (int64_t)blockIdx.y * chunk_len;
   const int64_t p_hi = p_lo + chunk_len < seq_len ? p_lo + chunk_len : seq_len;
   if (vec) {
-    for (int64_t p = p_lo + 4 * (int64_t)threadIdx.x; p < p_hi; p += 4 * kThreads) {
-      float v[4];
-      logits4(p, v);
-      *reinterpret_cast<float4*>(w + p) = make_float4(expf(v[0] - m) / l, expf(v[1] - m) / l, expf(v[2] - m) / l,
-                                                      expf(v[3] - m) / l);
+    constexpr int kWr = 4;                               // pieces per thread and step, loaded before any is used
+    for (int64_t p = p_lo + 4 * (int64_t)threadIdx.x; p < p_hi; p += 4 * kSmThreads * kWr) {
+      float v[kWr][4];
+#pragma unroll
+      for (int u = 0; u < kWr; ++u) {
+        const int64_t pu = p + (int64_t)u * 4 * kSmThreads;
+        if (pu < p_hi) logits4(pu, v[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < kWr; ++u) {
+        const int64_t pu = p + (int64_t)u * 4 * kSmThreads;
+        if (pu < p_hi)
+          *reinterpret_cast<float4*>(w + pu) =
+              make_float4(__builtin_amdgcn_exp2f(v[u][0] - M) * inv_l, __builtin_amdgcn_exp2f(v[u][1] - M) * inv_l,
+                          __builtin_amdgcn_exp2f(v[u][2] - M) * inv_l, __builtin_amdgcn_exp2f(v[u][3] - M) * inv_l);
+      }
     }
   } else {
-    for (int64_t p = p_lo + threadIdx.x; p < p_hi; p += kThreads) w[p] = expf(logit(p) - m) / l;
+    for (int64_t p = p_lo + threadIdx.x; p < p_hi; p += kSmThreads) w[p] = __builtin_amdgcn_exp2f(logit(p) - M) * inv_l;
   }
 }
 
@@ -1030,13 +1088,13 @@ extern "C" int tq_softmax_rows(const float* scores, const float* mask, int64_t m
   if (!scores || !weights) return tq::fail(TQ_ERR_NULL, "tq_softmax_rows: null pointer");
   if (n_rows > 0x7FFFFFFF) return tq::fail(TQ_ERR_ARG, "tq_softmax_rows: too many rows");
   // chunks per row: enough workgroups to fill the chip when the rows are few and long (at least 4096 positions each)
-  int64_t n_chunks = 512 / n_rows;
+  int64_t n_chunks = (256 + n_rows - 1) / n_rows;      // about one workgroup per CU: every chunk re-reads its whole row
   if (n_chunks > seq_len / 4096) n_chunks = seq_len / 4096;
   if (n_chunks < 1) n_chunks = 1;
   int64_t chunk_len = (seq_len + n_chunks - 1) / n_chunks;
   chunk_len = (chunk_len + 3) & ~(int64_t)3;
   n_chunks = (seq_len + chunk_len - 1) / chunk_len;
-  softmax_rows_kernel<<<dim3((unsigned)n_rows, (unsigned)n_chunks), kThreads, 0, (hipStream_t)stream_>>>(
+  softmax_rows_kernel<<<dim3((unsigned)n_rows, (unsigned)n_chunks), kSmThreads, 0, (hipStream_t)stream_>>>(
       scores, mask, mask_row_stride, weights, seq_len, scale, chunk_len);
   TQ_CHECK_LAUNCH("tq_softmax_rows launch");
   return TQ_OK;
