@@ -1625,3 +1625,62 @@ def test_flash_decode_from_q_against_oracle_and_shape_limits(tq):
     with pytest.raises(ValueError, match="prerotate_query"):
         tq.flash_decode_from_q(torch.zeros((1, 2, 64), device="cuda"), dev(ks4), dev(kp4[None]), dev(kn4[None]),
                                dev(vp4[None]), dev(vn4[None]), c4, c4, dev(vs4), 64, 4, 0.125, n_rep=1)
+
+
+# ------------------------------------------------------------------ tensors with more than 2^31 elements / words
+
+def test_addressing_past_2g_elements(tq):
+    """Tensors whose element (encode input, dequant output, fp16 keys) or word (packed rows) count exceeds 2^31:
+    every address in the kernels must be formed in 64 bits.  Data are generated on the GPU; rows at the start,
+    in the middle and at the very end are checked against the oracle (encode / dequant bit for bit), and a short
+    sequence stored BEHIND a very long one in a ragged batch is attended through both fused decode steps."""
+    D, bits, sc = 128, 3, 1 / math.sqrt(128)
+    c, b = tables(bits)
+    ks, vs = o.random_diagonal_sign(D, 42), o.random_diagonal_sign(D, 43)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(5)
+
+    # ---- encode / dequant: 16 793 216 vectors = 2.15e9 elements
+    N = (1 << 24) + 16000
+    x = torch.randn((N, D), generator=g, device="cuda", dtype=torch.float16)
+    packed, norms = tq.fused_quantize(x, dev(vs), b, D, bits)
+    deq = tq.dequant_fp16(packed, norms, c, dev(vs), D, bits)
+    for lo in (0, N // 2 - 8, N - 64):
+        wp, wn = o.fused_quantize(host(x[lo:lo + 64]), vs, b, D, bits)
+        assert np.array_equal(host(packed[lo:lo + 64]), wp), lo
+        assert np.array_equal(host(norms[lo:lo + 64]), wn), lo
+        want = torch.from_numpy(o.packed_dequantize(wp, wn, c, vs, D, bits)).to(torch.float16)
+        assert torch.equal(deq[lo:lo + 64].cpu(), want), lo
+    del deq
+
+    # ---- V-only decode: fp16 keys of the same 2.15e9 elements (one kv head), a 2000-position sequence at the end
+    n_rep, tail = 2, 2000
+    offs = torch.tensor([0, N - tail, N], dtype=torch.int32, device="cuda")
+    q = torch.randn((2, n_rep, D), generator=g, device="cuda", dtype=torch.float16)
+    got = tq.vonly_decode(q, x[None], packed[None], norms[None], c, dev(vs), D, bits, sc, n_rep=n_rep,
+                          seq_offsets=offs, max_seq_len=N - tail)
+    assert torch.isfinite(got).all()
+    want = o.vonly_decode_attention(host(q[1]), host(x[None, N - tail:]), host(packed[None, N - tail:]),
+                                    host(norms[None, N - tail:]), c, vs, D, bits, sc)
+    close(host(got[1]), want)
+    del x, packed, norms
+
+    # ---- flash decode: 165 300 000 packed rows = 2.149e9 words per tensor, a 3000-position sequence at the end
+    R, tail = 165_300_000, 3000
+    def rand_packed():
+        p = torch.randint(0, 1 << 30, (R, 13), generator=g, device="cuda", dtype=torch.int32)
+        p[:, 12] &= 0x00FFFFFF                         # the last word holds 8 fields
+        return p.view(torch.uint32)
+    kp, vp = rand_packed(), rand_packed()
+    kn = torch.rand(R, generator=g, device="cuda") * 12 + 6
+    vn = torch.rand(R, generator=g, device="cuda") + 0.5
+    offs = torch.tensor([0, R - tail, R], dtype=torch.int32, device="cuda")
+    qf = torch.randn((2, n_rep, D), generator=g, device="cuda")
+    q_rot = tq.prerotate_query(qf.reshape(-1, D), dev(ks)).reshape(2, n_rep, D)
+    got = tq.flash_decode(q_rot, kp[None], kn[None], vp[None], vn[None], c, c, dev(vs), D, bits, sc, n_rep=n_rep,
+                          seq_offsets=offs, max_seq_len=R - tail)
+    assert torch.isfinite(got).all()
+    sl = slice(R - tail, R)
+    want = o.turboquant_attention_single(host(qf[1]), host(kp[None, sl]), host(kn[None, sl]), host(vp[None, sl]),
+                                         host(vn[None, sl]), c, ks, c, vs, D, bits, sc)
+    close(host(got[1]), want)
