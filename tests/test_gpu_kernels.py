@@ -485,6 +485,11 @@ def test_flash_argument_errors(tq):
         tq.flash_attention_turboquant(q, *a, 256, 3, 0.1)
     with pytest.raises(ValueError, match="must equal n_kv_heads"):
         tq.flash_attention_turboquant(q, *a, 128, 3, 0.1, n_rep=2)
+    # sequences are a grid dimension: more than 65535 per call is refused before any launch
+    n_seq = 65536
+    offs = torch.zeros(n_seq + 1, dtype=torch.int32, device="cuda")
+    with pytest.raises(ValueError, match="at most 65535 sequences"):
+        tq.flash_decode(torch.zeros((n_seq, 2, 128), device="cuda"), *a, 128, 3, 0.1, seq_offsets=offs, max_seq_len=1)
 
 
 def test_flash_ragged_batch(tq):

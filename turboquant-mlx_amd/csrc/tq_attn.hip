@@ -1002,6 +1002,9 @@ int check_shape(const tq_decode_shape* sh, const char* who, int max_dim) {
     return tq::fail(TQ_ERR_DIM, "dim must be a power of 2 and <= %d, got %d", max_dim, sh->dim);
   if (int rc = check_heads(sh->n_kv_heads, sh->n_rep, who)) return rc;
   if (sh->n_seq < 1) return tq::fail(TQ_ERR_ARG, "%s: n_seq must be >= 1, got %d", who, sh->n_seq);
+  if (sh->n_seq > 65535 || sh->n_kv_heads > 65535)         // sequences and kv heads are grid dimensions z and y
+    return tq::fail(TQ_ERR_ARG, "%s: at most 65535 sequences and 65535 kv heads per call, got %d and %d", who,
+                    sh->n_seq, sh->n_kv_heads);
   if (sh->seq_len < 0) return tq::fail(TQ_ERR_ARG, "%s: negative seq_len", who);
   if (sh->block_size < 1 || sh->block_size > 32)
     return tq::fail(TQ_ERR_BLOCK, "block_size must be in 1..32, got %d", sh->block_size);
