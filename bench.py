@@ -77,7 +77,7 @@ def cpu_baseline(torch, sets, cb, signs, budget_s=12.0):
         run()
         n += 1
         el = time.perf_counter() - t0
-        if el > budget_s or n >= 20:
+        if el > budget_s or n >= 120:
             break
     per = el / n
     try:
