@@ -724,17 +724,26 @@ int launch_vonly_mfma(const void* q, int q_dtype, const void* k_f16, const uint3
                       size_t workspace_bytes, const tq_decode_shape& sh, hipStream_t stream, int phases) {
   const char* who = "tq_vonly_decode_attn";
   const int n_q = sh.n_kv_heads * sh.n_rep;
-  const bool plain = !sh.mask && !sh.seq_offsets && sh.attn_scale > 0.0f && sh.seq_len % tqm::kTilePos == 0 &&
-                     tq::aligned(v_packed, 16) && sh.v_seq_stride % 4 == 0 && sh.v_head_stride % 4 == 0;
+  // no mask, no ragged offsets, 16-byte aligned V rows of every tile: with full tiles on top, the PLAIN variants apply
+  const bool plain_base = !sh.mask && !sh.seq_offsets && sh.attn_scale > 0.0f && tq::aligned(v_packed, 16) &&
+                          sh.v_seq_stride % 4 == 0 && sh.v_head_stride % 4 == 0;
+  const bool plain = plain_base && sh.seq_len % tqm::kTilePos == 0;
   // Long unmasked caches: several consecutive 512-position blocks per workgroup, as many as still leave
   // one workgroup per CU (256) and divide the length.
   int n_blocks = 1;
+  const int64_t wgs8 = ((sh.seq_len + tqm::kTilePos - 1) / tqm::kTilePos) * sh.n_kv_heads * sh.n_seq;
   if (plain) {
-    const int64_t wgs = (sh.seq_len / tqm::kTilePos) * sh.n_kv_heads * sh.n_seq;
-    for (int nb = (int)(wgs / 256 < 8 ? wgs / 256 : 8); nb > 1; --nb)
+    for (int nb = (int)(wgs8 / 256 < 8 ? wgs8 / 256 : 8); nb > 1; --nb)
       if ((sh.seq_len / tqm::kTilePos) % nb == 0) { n_blocks = nb; break; }
   }
-  const int tile_pos = tqm::kTilePos * n_blocks;
+  // One tile per workgroup, as measured over lengths from 4 096 to 65 537 (28/4 heads): eight-wave workgroups
+  // (512 positions, one per CU) are the faster shape when they fill between half and all of the CUs in one round;
+  // four-wave workgroups (256 positions, up to three per CU) fill more CUs on short caches and, from 257 to 768
+  // of them, avoid the nearly empty second round of the eight-wave shape; beyond that the eight-wave shape again.
+  const int64_t wgs4 = ((sh.seq_len + 255) / 256) * sh.n_kv_heads * sh.n_seq;
+  int nw = 8;
+  if (n_blocks == 1 && (wgs8 <= 128 || (wgs8 > 256 && wgs4 <= 768))) nw = 4;
+  const int tile_pos = nw * tqm::kWavePos * n_blocks;
   const int n_tiles = (int)((sh.seq_len + tile_pos - 1) / tile_pos);
   const size_t need = (size_t)sh.n_seq * n_q * n_tiles * (tqm::kD + 2) * sizeof(float);
   if (!workspace || workspace_bytes < need)
@@ -765,27 +774,35 @@ int launch_vonly_mfma(const void* q, int q_dtype, const void* k_f16, const uint3
   a.v_unscale = tq::fill_codebook_fp16(vcb, v_centroids, sh.bits);
   if (phases & 1) {
     dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
-    if (q_f32) {
-      if (n_blocks > 1) tqm::vonly_stream_kernel<true><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb, n_blocks);
-      else if (plain) tqm::vonly_tile_mfma_kernel<true, true><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb);
-      else tqm::vonly_tile_mfma_kernel<false, true><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb);
-    } else {
-      if (n_blocks > 1) tqm::vonly_stream_kernel<false><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb, n_blocks);
-      else if (plain) tqm::vonly_tile_mfma_kernel<true, false><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb);
-      else tqm::vonly_tile_mfma_kernel<false, false><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb);
-    }
+    const bool plain4 = plain_base && sh.seq_len % 256 == 0;           // full 256-position tiles
+#define LAUNCH_TILE(QF)                                                                                          \
+    if (n_blocks > 1) tqm::vonly_stream_kernel<QF><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb, n_blocks);       \
+    else if (nw == 8 && plain) tqm::vonly_tile_mfma_kernel<true, QF, 8><<<grid, 512, 0, stream>>>(a, vcb);           \
+    else if (nw == 8) tqm::vonly_tile_mfma_kernel<false, QF, 8><<<grid, 512, 0, stream>>>(a, vcb);                   \
+    else if (plain4) tqm::vonly_tile_mfma_kernel<true, QF, 4><<<grid, 256, 0, stream>>>(a, vcb);                     \
+    else tqm::vonly_tile_mfma_kernel<false, QF, 4><<<grid, 256, 0, stream>>>(a, vcb)
+    if (q_f32) { LAUNCH_TILE(true); } else { LAUNCH_TILE(false); }
+#undef LAUNCH_TILE
     TQ_CHECK_LAUNCH(who);
   }
   if (!(phases & 2)) return TQ_OK;
   dim3 mgrid(n_q, sh.n_seq);
   const float inv_dim = 1.0f / (float)sh.dim;
-#define LAUNCH_MERGE_M(TO)                                                                                \
-  tqm::decode_merge_rows_kernel<TO, true><<<mgrid, tqm::kMergeThreads, 0, stream>>>(                        \
+#define LAUNCH_MERGE_U(TO, U_)                                                                            \
+  tqm::decode_merge_rows_kernel<TO, true, U_><<<mgrid, tqm::kMergeThreads, 0, stream>>>(                    \
       a.ws_S, a.ws_ml, sh.seq_offsets, sh.seq_len, n_tiles, sh.n_kv_heads, sh.n_rep, v_signs, inv_dim, (TO*)out, tile_pos)
+  // tiles per lane group and round: one round of loads where 64, 128 or 256 tiles cover the sequence
+#define LAUNCH_MERGE_M(TO)                                                                                \
+  do {                                                                                                    \
+    if (n_tiles <= 64) LAUNCH_MERGE_U(TO, 8);                                                             \
+    else if (n_tiles <= 128) LAUNCH_MERGE_U(TO, 16);                                                      \
+    else LAUNCH_MERGE_U(TO, 32);                                                                          \
+  } while (0)
   if (sh.out_dtype == TQ_F16) { LAUNCH_MERGE_M(__half); }
   else if (sh.out_dtype == TQ_BF16) { LAUNCH_MERGE_M(__hip_bfloat16); }
   else { LAUNCH_MERGE_M(float); }
 #undef LAUNCH_MERGE_M
+#undef LAUNCH_MERGE_U
   TQ_CHECK_LAUNCH(who);
   return TQ_OK;
 }

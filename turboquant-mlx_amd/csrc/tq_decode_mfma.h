@@ -122,24 +122,29 @@ __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
   return *reinterpret_cast<uint32_t*>(&h);
 }
 
-// grid = (n_tiles_max, n_kv, n_seq), 512 threads.
+// grid = (n_tiles_max, n_kv, n_seq), NW * 64 threads: a workgroup of NW waves owns NW * 64 consecutive positions.
+// NW = 8 (one workgroup per CU) is the faster shape when the tiles of a launch fill the CUs exactly once; NW = 4
+// lets two or three workgroups share a CU, so a launch whose tile count is not a multiple of the CU count does
+// not pay a second, nearly empty round of workgroups.
 // PLAIN = no mask, no ragged offsets, seq_len a multiple of the tile, 16-byte aligned V rows (checked
 // by the host): every tile is full, so the row clamps, the validity selects, the mask reads and the
 // narrow V path drop out, and K / V addresses are a uniform base plus a lane-constant offset.
 // QF32: the queries are float32 and enter as an fp16 value plus the fp16 remainder of that rounding (two
 // matrix instructions per key operand), which keeps float32-query fidelity; otherwise fp16 (or bf16) queries.
-template <bool PLAIN, bool QF32>
-__global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
+template <bool PLAIN, bool QF32, int NW>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 8 ? 2 : 3, NW == 8 ? 2 : 3)))
 void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
-  // 32 KB used three ways: per-wave staging (8 x 4 KB) first for the packed V block, then for K
-  // tiles; finally the cross-wave merge buffer S_all[8][8][128].
-  __shared__ __align__(16) unsigned char big_s[32768];
+  constexpr int kTPos = NW * kWavePos;                 // positions per workgroup
+  constexpr int kThr = NW * 64;
+  // 4 KB per wave used three ways: per-wave staging first for the packed V block, then for K
+  // tiles; finally the cross-wave merge buffer S_all[NW][8][128].
+  __shared__ __align__(16) unsigned char big_s[NW * 4096];
   __shared__ uint32_t lut_s[64];                       // half2(c[i & 7], c[i >> 3])
   __shared__ __align__(16) uint32_t q_s[kHeadsMax][kD / 2];   // fp16 pairs, rows >= n_rep are zero
   __shared__ __align__(16) uint32_t ql_s[QF32 ? kHeadsMax : 1][kD / 2];   // QF32: what rounding the query to fp16 lost
-  __shared__ __align__(16) float nrm_s[kWaves][kWavePos];
-  __shared__ float m_s[kWaves][kHeadsMax], l_s[kWaves][kHeadsMax], M_s[kHeadsMax];
-  __shared__ __align__(16) float f_s[kWaves][kHeadsMax];
+  __shared__ __align__(16) float nrm_s[NW][kWavePos];
+  __shared__ float m_s[NW][kHeadsMax], l_s[NW][kHeadsMax], M_s[kHeadsMax];
+  __shared__ __align__(16) float f_s[NW][kHeadsMax];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -154,18 +159,20 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
     first = a.seq_offsets[seq];
     len = (int64_t)a.seq_offsets[seq + 1] - first;
   }
-  const int64_t tile_p0 = (int64_t)tile * kTilePos;
+  const int64_t tile_p0 = (int64_t)tile * kTPos;
   TQ_STAMP(0);
   if (tile_p0 >= len) return;                          // the merge pass never reads this tile
-  const int rows_here = PLAIN ? kTilePos : (int)min((int64_t)kTilePos, len - tile_p0);   // valid rows of this tile
+  const int rows_here = PLAIN ? kTPos : (int)min((int64_t)kTPos, len - tile_p0);   // valid rows of this tile
   const int last_row = rows_here - 1;
   const int wrow0 = wave * kWavePos;                                  // wave's first row inside the tile
 
   // ---- issue every global load of this wave, small ones first -------------------------------------
-  uint32_t my_q[2], my_ql[2] = {0u, 0u};               // Q rows of this kv head: n_rep x 64 words, <= 1024
+  constexpr int kQIt = kHeadsMax * (kD / 2) / kThr;
+  uint32_t my_q[kQIt], my_ql[kQIt];                    // Q rows of this kv head: n_rep x 64 words, <= 1024
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int w = tid + i * kMfmaThreads;
+  for (int i = 0; i < kQIt; ++i) {
+    my_ql[i] = 0u;
+    const int w = tid + i * kThr;
     if (QF32) {
       const float2 f = (w < n_rep * (kD / 2)) ? reinterpret_cast<const float2*>(reinterpret_cast<const float*>(a.q) + q_row0 * kD)[w]
                                               : make_float2(0.f, 0.f);
@@ -251,9 +258,9 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
     lut_s[tid] = pack_h2(clo, chi);
   }
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    (&q_s[0][0])[tid + i * kMfmaThreads] = my_q[i];
-    if (QF32) (&ql_s[0][0])[tid + i * kMfmaThreads] = my_ql[i];
+  for (int i = 0; i < kQIt; ++i) {
+    (&q_s[0][0])[tid + i * kThr] = my_q[i];
+    if (QF32) (&ql_s[0][0])[tid + i * kThr] = my_ql[i];
   }
   nrm_s[wave][lane] = my_norm;
   __syncthreads();
@@ -430,7 +437,7 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
   // e^(m_w - M_h) per (wave, head); (3) every wave scales its own accumulator rows by its factors
   // and deposits them; (4) a float4 sum over the eight deposits goes to the workspace.  The
   // exponentials are evaluated once per (wave, head), not once per element.
-  float (*S_all)[8][kD] = reinterpret_cast<float (*)[8][kD]>(big_s);    // [wave][head in round][128]
+  float (*S_all)[8][kD] = reinterpret_cast<float (*)[8][kD]>(big_s);    // [wave][head in round][128]: NW x 4 KB
   const int64_t grp = (int64_t)seq * a.n_kv + kvh;
   float* pS = a.ws_S + (grp * a.n_tiles_max + tile) * (int64_t)(n_rep * kD);
   float* pml = a.ws_ml + (grp * a.n_tiles_max + tile) * (int64_t)(n_rep * 2);
@@ -439,11 +446,11 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
     l_s[wave][n16] = l;
   }
   __syncthreads();                                       // (m, l) visible; the staging area is free
-  if (tid < kWaves * kHeadsMax) {
+  if (tid < NW * kHeadsMax) {
     const int w = tid >> 4, h = tid & 15;
     float M = m_s[0][h];
 #pragma unroll
-    for (int ww = 1; ww < kWaves; ++ww) M = fmaxf(M, m_s[ww][h]);
+    for (int ww = 1; ww < NW; ++ww) M = fmaxf(M, m_s[ww][h]);
     const float mw = m_s[w][h];
     f_s[w][h] = (mw == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(mw - M);
     if (w == 0) M_s[h] = M;
@@ -470,7 +477,7 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
       const int hl = tid >> 5, e4 = tid & 31;
       float4 sum = *reinterpret_cast<const float4*>(&S_all[0][hl][4 * e4]);
 #pragma unroll
-      for (int w = 1; w < kWaves; ++w) {
+      for (int w = 1; w < NW; ++w) {
         const float4 x = *reinterpret_cast<const float4*>(&S_all[w][hl][4 * e4]);
         sum.x += x.x; sum.y += x.y; sum.z += x.z; sum.w += x.w;
       }
@@ -482,7 +489,7 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
     const int h = tid;
     float L = 0.0f;
 #pragma unroll
-    for (int w = 0; w < kWaves; ++w) L += f_s[w][h] * l_s[w][h];
+    for (int w = 0; w < NW; ++w) L += f_s[w][h] * l_s[w][h];
     pml[2 * h] = M_s[h];
     pml[2 * h + 1] = L;
   }
@@ -964,9 +971,11 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
 }
 
 // Merge pass: grid = (n_q, n_seq), 256 threads.  Lane group ph = tid / 32 folds tiles ph, ph + 8, ...
-// (4 elements per lane) with a running maximum; the 8 groups are then combined through LDS and wave 0
-// finishes the row.  NORM = false (given weights, all maxima zero) skips the division by l.
-template <typename TO, bool NORM>
+// (4 elements per lane) with a running maximum, U tiles per round with all loads of a round issued together (a
+// round costs one memory round trip, so the host picks U to cover the tiles in one round where it can: 8, 16
+// or 32); the 8 groups are then combined through LDS and wave 0 finishes the row.  NORM = false (given weights,
+// all maxima zero) skips the division by l.
+template <typename TO, bool NORM, int U = 8>
 __global__ __launch_bounds__(kMergeThreads) void decode_merge_rows_kernel(
     const float* __restrict__ ws_S, const float* __restrict__ ws_ml, const int32_t* __restrict__ seq_offsets,
     int64_t seq_len, int n_tiles_max, int n_kv, int n_rep, const float* __restrict__ signs, float inv_dim,
@@ -987,11 +996,11 @@ __global__ __launch_bounds__(kMergeThreads) void decode_merge_rows_kernel(
   const float sign0 = signs[lane], sign1 = signs[lane + 64];
   float M = -INFINITY, L = 0.0f;
   f4 acc = {0.f, 0.f, 0.f, 0.f};
-  for (int t0 = ph; t0 < n_tiles; t0 += 64) {            // 8 tiles per lane group and round
-    f4 x[8];
-    float2 ml[8];
+  for (int t0 = ph; t0 < n_tiles; t0 += 8 * U) {         // U tiles per lane group and round
+    f4 x[U];
+    float2 ml[U];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
+    for (int u = 0; u < U; ++u) {
       const int t = min(t0 + 8 * u, n_tiles - 1);
       x[u] = *reinterpret_cast<const f4*>(gS + (int64_t)t * (n_rep * kD));
       ml[u] = *reinterpret_cast<const float2*>(gml + (int64_t)t * (n_rep * 2));
@@ -999,14 +1008,14 @@ __global__ __launch_bounds__(kMergeThreads) void decode_merge_rows_kernel(
     // maximum of the round first, then one independent 2^(m - M) per tile
     float Mr = M;
 #pragma unroll
-    for (int u = 0; u < 8; ++u)
+    for (int u = 0; u < U; ++u)
       if (t0 + 8 * u < n_tiles) Mr = fmaxf(Mr, ml[u].x);
     if (Mr != -INFINITY) {
       const float fo = (M == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(M - Mr);
       acc = acc * fo;
       L = L * fo;
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
+      for (int u = 0; u < U; ++u) {
         const float fc = (t0 + 8 * u < n_tiles && ml[u].x != -INFINITY) ? __builtin_amdgcn_exp2f(ml[u].x - Mr) : 0.0f;
         acc = acc + x[u] * fc;
         L = L + ml[u].y * fc;
