@@ -1689,3 +1689,43 @@ def test_addressing_past_2g_elements(tq):
     want = o.turboquant_attention_single(host(qf[1]), host(kp[None, sl]), host(kn[None, sl]), host(vp[None, sl]),
                                          host(vn[None, sl]), c, ks, c, vs, D, bits, sc)
     close(host(got[1]), want)
+
+
+@pytest.mark.parametrize("n_seq,n_kv,n_rep,T,qdt", [(1, 4, 7, 50001, "float16"), (1, 4, 7, 65537, "float32"),
+                                                     (2, 2, 4, 98305, "bfloat16"), (1, 8, 1, 26113, "float16")])
+def test_vonly_streaming_pass_with_a_ragged_end(tq, n_seq, n_kv, n_rep, T, qdt):
+    """Unmasked caches too long for one round of tile workgroups and of a length that is no multiple of the
+    streaming pass's range: the last workgroup of a kv head runs through fewer blocks, whole waves (and, at
+    T = k * 512 * blocks + 1, whole steps) see no valid row.  Random packed values; against the oracle."""
+    rng = np.random.default_rng(T)
+    D, bits, sc = 128, 3, 1 / math.sqrt(128)
+    c, b = tables(bits)
+    vs = o.random_diagonal_sign(D, 43)
+    K = rng.standard_normal((n_seq, n_kv, T, D)).astype(np.float16)          # exactly T rows: nothing to read past the end
+    vp = o.pack_indices(rng.integers(0, 8, size=(n_seq, n_kv, T, D)).astype(np.uint8), bits)
+    vn = ((rng.random((n_seq, n_kv, T)) + 0.5) * np.exp(rng.uniform(-3, 3, size=(n_seq, n_kv, T)))).astype(F32)
+    q = torch.from_numpy(rng.standard_normal((n_seq, n_kv * n_rep, D)).astype(F32)).to(getattr(torch, qdt))
+    got = host(tq.vonly_decode(q.cuda(), dev(K), dev(vp), dev(vn), c, dev(vs), D, bits, sc, n_rep=n_rep).float())
+    for i in range(n_seq):
+        want = o.vonly_decode_attention(q[i].float().numpy(), K[i], vp[i], vn[i], c, vs, D, bits, sc)
+        close(got[i], want, rel=(1e-2 if qdt == "bfloat16" else REL), abs_=(4e-3 if qdt == "bfloat16" else ABS), row_scale=True)
+
+
+def test_attended_length_beyond_the_tensors_is_refused(tq):
+    """The kernels trust seq_len / kv_len: the wrappers refuse a length that the K/V tensors do not hold."""
+    rng = np.random.default_rng(12)
+    c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, 2, 100, 128, 3)
+    q = dev(rng.standard_normal((1, 2, 128)).astype(np.float16))
+    with pytest.raises(ValueError, match="exceeds the 100 rows"):
+        tq.vonly_decode(q, dev(K[None]), dev(vp[None]), dev(vn[None]), c, dev(vs), 128, 3, 0.1, seq_len=101)
+    with pytest.raises(ValueError, match="exceeds the 100 rows"):
+        tq.flash_decode(q.float(), dev(kp[None]), dev(kn[None]), dev(vp[None]), dev(vn[None]), c, c, dev(vs), 128, 3, 0.1,
+                        seq_len=4096)
+    with pytest.raises(ValueError, match="exceeds the 100 rows"):
+        tq.flash_decode_from_q(q, dev(ks), dev(kp[None]), dev(kn[None]), dev(vp[None]), dev(vn[None]), c, c, dev(vs), 128, 3,
+                               0.1, seq_len=101)
+    with pytest.raises(ValueError, match="exceeds the 100 rows"):
+        tq.prefill_attention(dev(rng.standard_normal((2, 4, 128)).astype(np.float16)), dev(kp), dev(kn), dev(vp), dev(vn),
+                             c, c, dev(ks), dev(vs), 128, 3, 0.1, n_rep=1, kv_len=101)
+    with pytest.raises(ValueError, match="holds 1 sequences"):
+        tq.vonly_decode(torch.cat([q, q]), dev(K[None]), dev(vp[None]), dev(vn[None]), c, dev(vs), 128, 3, 0.1)

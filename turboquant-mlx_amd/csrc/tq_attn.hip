@@ -732,15 +732,28 @@ int launch_vonly_mfma(const void* q, int q_dtype, const void* k_f16, const uint3
   // one workgroup per CU (256) and divide the length.
   int n_blocks = 1;
   const int64_t wgs8 = ((sh.seq_len + tqm::kTilePos - 1) / tqm::kTilePos) * sh.n_kv_heads * sh.n_seq;
+  bool ragged_stream = false;
   if (plain) {
     for (int nb = (int)(wgs8 / 256 < 8 ? wgs8 / 256 : 8); nb > 1; --nb)
       if ((sh.seq_len / tqm::kTilePos) % nb == 0) { n_blocks = nb; break; }
+  }
+  const int64_t wgs4 = ((sh.seq_len + 255) / 256) * sh.n_kv_heads * sh.n_seq;
+  if (n_blocks == 1 && plain_base && wgs4 > 768) {
+    // Long caches of any length: the streaming pass with a ragged end.  Blocks per workgroup: the count that
+    // minimises rounds of 256 workgroups times blocks per workgroup (ties: fewer blocks, more workgroups).
+    const int64_t blocks = (sh.seq_len + tqm::kTilePos - 1) / tqm::kTilePos;
+    int64_t best_cost = INT64_MAX;
+    for (int nb = 2; nb <= 8; ++nb) {
+      const int64_t wgs = ((blocks + nb - 1) / nb) * sh.n_kv_heads * sh.n_seq;
+      const int64_t cost = ((wgs + 255) / 256) * nb;
+      if (cost < best_cost) { best_cost = cost; n_blocks = nb; }
+    }
+    ragged_stream = true;
   }
   // One tile per workgroup, as measured over lengths from 4 096 to 65 537 (28/4 heads): eight-wave workgroups
   // (512 positions, one per CU) are the faster shape when they fill between half and all of the CUs in one round;
   // four-wave workgroups (256 positions, up to three per CU) fill more CUs on short caches and, from 257 to 768
   // of them, avoid the nearly empty second round of the eight-wave shape; beyond that the eight-wave shape again.
-  const int64_t wgs4 = ((sh.seq_len + 255) / 256) * sh.n_kv_heads * sh.n_seq;
   int nw = 8;
   if (n_blocks == 1 && (wgs8 <= 128 || (wgs8 > 256 && wgs4 <= 768))) nw = 4;
   const int tile_pos = nw * tqm::kWavePos * n_blocks;
@@ -776,7 +789,8 @@ int launch_vonly_mfma(const void* q, int q_dtype, const void* k_f16, const uint3
     dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
     const bool plain4 = plain_base && sh.seq_len % 256 == 0;           // full 256-position tiles
 #define LAUNCH_TILE(QF)                                                                                          \
-    if (n_blocks > 1) tqm::vonly_stream_kernel<QF><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb, n_blocks);       \
+    if (n_blocks > 1 && ragged_stream) tqm::vonly_stream_kernel<QF, true><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb, n_blocks); \
+    else if (n_blocks > 1) tqm::vonly_stream_kernel<QF, false><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb, n_blocks); \
     else if (nw == 8 && plain) tqm::vonly_tile_mfma_kernel<true, QF, 8><<<grid, 512, 0, stream>>>(a, vcb);           \
     else if (nw == 8) tqm::vonly_tile_mfma_kernel<false, QF, 8><<<grid, 512, 0, stream>>>(a, vcb);                   \
     else if (plain4) tqm::vonly_tile_mfma_kernel<true, QF, 4><<<grid, 256, 0, stream>>>(a, vcb);                     \

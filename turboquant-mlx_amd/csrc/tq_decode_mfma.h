@@ -675,10 +675,14 @@ __global__ __launch_bounds__(WAVES * 64) void vonly_scores_kernel(MfmaArgs a) {
 // The partial of a workgroup is taken relative to R = m - kexp (running maximum in log2 units minus
 // the exponent of the power-of-two norm scale of the step that set it): weights are
 // 2^(s*cs - R), and moving from R_old to R_new multiplies accumulators and weight sum by 2^(R_old - R_new).
-// grid = (seq_len / (512 * n_blocks), n_kv, n_seq), 512 threads.
+// grid = (ceil(seq_len / (512 * n_blocks)), n_kv, n_seq), 512 threads.
+// RAGGED = the length is not a multiple of 512 * n_blocks: the last workgroup of a (sequence, kv head) runs
+// through fewer blocks, loads of rows past the end are redirected to valid rows (norms and K rows to the last
+// valid row, packed-V pieces with no valid byte to the first piece of the last partly valid step; an aligned
+// 16-byte piece that holds a valid byte never crosses a page) and the scores of those rows are set to -inf.
 constexpr int kStepPos = 32;
 
-template <bool QF32>
+template <bool QF32, bool RAGGED>
 __global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
   __shared__ __align__(16) unsigned char big_s[32768];
@@ -698,11 +702,16 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
   const int n_q = a.n_kv * n_rep;
   const int64_t q_row0 = (int64_t)seq * n_q + (int64_t)kvh * n_rep;
   const int64_t tile_p0 = (int64_t)tile * kTilePos * n_blocks;
-  const int n_steps = 2 * n_blocks;
+  // positions of this workgroup's range that exist (RAGGED: the last workgroup has fewer)
+  const int valid = RAGGED ? (int)min((int64_t)kTilePos * n_blocks, a.seq_len - tile_p0) : kTilePos * n_blocks;
+  const int n_steps = RAGGED ? 2 * ((valid + kTilePos - 1) / kTilePos) : 2 * n_blocks;
+  const int last_valid = valid - 1;
+  const int last_step_row = last_valid & ~(kStepPos - 1);               // first row of the last partly valid step
 
   // row of step s inside the workgroup's range: block s/2, this wave's 64 rows, half s%2
   auto step_row = [&](int s) { return (s >> 1) * kTilePos + wave * kWavePos + (s & 1) * kStepPos; };
-  const float* nbase = a.v_norms + (int64_t)seq * a.vn_seq_stride + (int64_t)kvh * a.vn_head_stride + tile_p0 + (lane & 31);
+  const float* nbase = a.v_norms + (int64_t)seq * a.vn_seq_stride + (int64_t)kvh * a.vn_head_stride + tile_p0 +
+                       (RAGGED ? 0 : (lane & 31));
   const char* vbase = reinterpret_cast<const char*>(
       a.v_packed + ((int64_t)seq * a.v_seq_stride + (int64_t)kvh * a.v_head_stride + tile_p0) * kPdim);
   const char* kbase = reinterpret_cast<const char*>(
@@ -712,17 +721,36 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
   const uint32_t koff_odd = (uint32_t)(((4 + (lane >> 4)) * 16 + ((lane & 15) ^ ((4 + (lane >> 4)) & 7))) * 16);
   auto issue_nv = [&](int s, float& nrm, u4 (&vqx)[2]) {
     const int r = step_row(s);
-    nrm = nbase[r];
-    const char* vb = vbase + (int64_t)r * (kPdim * 4);
-    vqx[0] = *reinterpret_cast<const u4*>(vb + voff0);
-    vqx[1] = *reinterpret_cast<const u4*>(vb + voff1);
+    if (RAGGED) {
+      nrm = nbase[min(r + (lane & 31), last_valid)];
+      const int rc = min(r, last_step_row);                             // a step with no valid row re-reads the last one that has
+      const uint32_t limit = (uint32_t)((valid - rc) * (kPdim * 4));     // bytes of valid rows from rc on (> 0)
+      const char* vb = vbase + (int64_t)rc * (kPdim * 4);
+      vqx[0] = *reinterpret_cast<const u4*>(vb + (voff0 < limit ? voff0 : 0u));
+      vqx[1] = *reinterpret_cast<const u4*>(vb + (voff1 < limit ? voff1 : 0u));
+    } else {
+      nrm = nbase[r];
+      const char* vb = vbase + (int64_t)r * (kPdim * 4);
+      vqx[0] = *reinterpret_cast<const u4*>(vb + voff0);
+      vqx[1] = *reinterpret_cast<const u4*>(vb + voff1);
+    }
   };
   auto issue_k4 = [&](int s, u4 (&kx)[8], int part) {     // instructions 4*part .. 4*part+3: rows 16*part .. +15 of the step
-    const char* kb = kbase + (int64_t)step_row(s) * (kD * 2) + part * 4096;
-    kx[4 * part + 0] = *reinterpret_cast<const u4*>(kb + koff_even);
-    kx[4 * part + 1] = *reinterpret_cast<const u4*>(kb + koff_odd);
-    kx[4 * part + 2] = *reinterpret_cast<const u4*>(kb + 2048 + koff_even);
-    kx[4 * part + 3] = *reinterpret_cast<const u4*>(kb + 2048 + koff_odd);
+    if (RAGGED) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int rin = 16 * part + 4 * i + (lane >> 4);                  // row inside the step
+        const int piece = (lane & 15) ^ (rin & 7);
+        const int row = min(step_row(s) + rin, last_valid);
+        kx[4 * part + i] = *reinterpret_cast<const u4*>(kbase + (int64_t)row * (kD * 2) + piece * 16);
+      }
+    } else {
+      const char* kb = kbase + (int64_t)step_row(s) * (kD * 2) + part * 4096;
+      kx[4 * part + 0] = *reinterpret_cast<const u4*>(kb + koff_even);
+      kx[4 * part + 1] = *reinterpret_cast<const u4*>(kb + koff_odd);
+      kx[4 * part + 2] = *reinterpret_cast<const u4*>(kb + 2048 + koff_even);
+      kx[4 * part + 3] = *reinterpret_cast<const u4*>(kb + 2048 + koff_odd);
+    }
   };
 
   uint32_t my_q[2], my_ql[2] = {0u, 0u};
@@ -850,7 +878,10 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
                                                      acc, 0, 0, 0);
       }
 #pragma unroll
-      for (int j = 0; j < 4; ++j) s[t][j] = acc[j];
+      for (int j = 0; j < 4; ++j) {
+        s[t][j] = acc[j];
+        if (RAGGED && step_row(sidx) + 16 * t + 4 * g + j > last_valid) s[t][j] = -INFINITY;
+      }
       if (t == 0) {
         __builtin_amdgcn_sched_barrier(0);
         next(2);
@@ -863,10 +894,13 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
     mb = fmaxf(mb, shfl_xor_f(mb, 16));
     mb = fmaxf(mb, shfl_xor_f(mb, 32));
     const float m_new = fmaxf(m_run, mb * cs);            // log2 units; attn_scale > 0 (host check)
-    const float R_new = m_new - kexp;
-    const float factor = __builtin_amdgcn_exp2f(R_run - R_new);      // 0 on the first step
+    // RAGGED: a wave whose rows so far all lie past the end has seen nothing yet (m_new = -inf): it keeps its
+    // empty state (weights 2^-inf = 0, no rescale) instead of forming -inf - -inf
+    const bool empty = RAGGED && m_new == -INFINITY;
+    const float R_new = empty ? 0.0f : m_new - kexp;
+    const float factor = empty ? 1.0f : __builtin_amdgcn_exp2f(R_run - R_new);      // 0 on the first step
     m_run = m_new;
-    R_run = R_new;
+    R_run = empty ? R_run : R_new;
     float lsum = 0.0f;
     uint32_t pa[4];
 #pragma unroll

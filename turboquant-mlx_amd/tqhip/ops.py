@@ -410,6 +410,17 @@ def _decode_shape(*, n_seq, n_kv, n_rep, dim, bits, block_size, seq_len, seq_off
     return sh
 
 
+def _check_rows(T: int, ragged: bool, n_seq: int, **tensors):
+    """The kernels trust the attended length: refuse one that exceeds what the tensors hold (cache layout: rows
+    per (sequence, head); ragged batch: the rows of all sequences together) before anything is launched."""
+    for name, t in tensors.items():
+        rows = t.shape[-2] if name in ("k", "k_packed", "v_packed") else t.shape[-1]
+        if T > rows:
+            raise ValueError(f"attended length {T} exceeds the {rows} rows of {name}")
+        if not ragged and t.dim() >= 3 + (name in ("k", "k_packed", "v_packed")) and t.shape[0] != n_seq:
+            raise ValueError(f"{name} holds {t.shape[0]} sequences, the query {n_seq}")
+
+
 def _kv_layout(t: torch.Tensor, inner: int, ragged: bool):
     """Strides in rows for KV addressing.  Accepts [H, T, inner] (one sequence or ragged batch) or
     [B, H, T, inner] (cache layout); the last two axes must be row-contiguous."""
@@ -490,6 +501,7 @@ def flash_decode(q_rot: torch.Tensor, k_packed, k_norms, v_packed, v_norms, k_ce
         T = int(max_seq_len)
     else:
         T = int(seq_len if seq_len is not None else k_norms.shape[-1])
+    _check_rows(T, ragged, n_seq, k_packed=k_packed, k_norms=k_norms, v_packed=v_packed, v_norms=v_norms)
     v_signs = _as_f32_dev(v_signs, q_rot)
     mask, ms = _mask_layout(mask, n_seq, n_q, T, q_rot.device)
     out = torch.empty((n_seq, n_q, dim), dtype=out_dtype, device=q_rot.device)
@@ -553,6 +565,7 @@ def flash_decode_from_q(q: torch.Tensor, k_signs, k_packed, k_norms, v_packed, v
         T = int(seq_len if seq_len is not None else k_norms.shape[-1])
     if T <= 0:
         raise ValueError("flash_decode_from_q needs a non-empty cache")
+    _check_rows(T, ragged, n_seq, k_packed=k_packed, k_norms=k_norms, v_packed=v_packed, v_norms=v_norms)
     k_signs = _as_f32_dev(k_signs, q)
     v_signs = _as_f32_dev(v_signs, q)
     mask, ms = _mask_layout(mask, n_seq, n_q, T, q.device)
@@ -624,6 +637,7 @@ def vonly_decode(q: torch.Tensor, k: torch.Tensor, v_packed, v_norms, v_centroid
         T = int(max_seq_len)
     else:
         T = int(seq_len if seq_len is not None else v_norms.shape[-1])
+    _check_rows(T, ragged, n_seq, k=k, v_packed=v_packed, v_norms=v_norms)
     v_signs = _as_f32_dev(v_signs, q)
     mask, ms = _mask_layout(mask, n_seq, n_q, T, q.device)
     out = torch.empty((n_seq, n_q, dim), dtype=out_dtype, device=q.device)
@@ -682,6 +696,7 @@ def prefill_attention(q: torch.Tensor, k_packed, k_norms, v_packed, v_norms, k_c
     if k_norms.stride(-1) != 1 or v_norms.stride(-1) != 1:
         k_norms, v_norms = k_norms.contiguous(), v_norms.contiguous()
     T = int(kv_len if kv_len is not None else k_norms.shape[-1])
+    _check_rows(T, True, 1, k_packed=k_packed, k_norms=k_norms, v_packed=v_packed, v_norms=v_norms)
     pos0 = int(q_pos0 if q_pos0 is not None else T - n_rows)
     out_dtype = out_dtype or q.dtype
     out = torch.empty((n_q, n_rows, dim), dtype=out_dtype, device=q.device)
