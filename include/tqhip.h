@@ -94,6 +94,29 @@ int tq_encode(const void* x, int x_dtype, const float* signs, const float* bound
               int dim, int bits, int variant, tq_stream_t stream);
 
 /*
+ * Append new tokens to a cache that keeps float16 keys beside PolarQuant values, in ONE launch:
+ * every new value row is encoded exactly as tq_encode does (bit-identical words and norms), and
+ * the wavefront that encodes row (g, i) also stores the key row, converted to float16 with
+ * round-to-nearest-even, and (when v_raw is not null) the value row unchanged.
+ * Replaces the insert of VOnlyTurboQuantCache.update_and_fetch (reference
+ * turboquant_mlx/v_only_cache.py:52-53,74: KVCache.update_and_fetch(keys, values) followed by the
+ * encode on insert of TurboQuantKVCache, cache.py:141-160), which is three slice assignments and
+ * one kernel there.
+ *   k_new, v_new  [n_groups*rows_per_group, dim] contiguous, dtypes k_dtype / v_dtype
+ *   k_f16         row (g, i) at k_f16 + (g*k_group_stride + i) * dim halves
+ *   v_raw         row (g, i) at v_raw + (g*v_raw_group_stride + i) * dim elements of v_dtype, or NULL
+ *   v_packed, v_norms, strides, boundaries (HOST), variant: as in tq_encode
+ * The destination pointers already point at the first free position of group 0.
+ */
+int tq_vonly_append(const void* k_new, int k_dtype, const void* v_new, int v_dtype,
+                    const float* v_signs, const float* boundaries,
+                    void* k_f16, void* v_raw, uint32_t* v_packed, float* v_norms,
+                    int64_t n_groups, int64_t rows_per_group,
+                    int64_t k_group_stride, int64_t v_raw_group_stride,
+                    int64_t packed_group_stride, int64_t norms_group_stride,
+                    int dim, int bits, int variant, tq_stream_t stream);
+
+/*
  * Dequantise packed rows: out = ((butterfly(c[idx]*s) * s) * signs) * norm, s = 1/sqrt(dim).
  * Replaces packed_dequantize (kernels.py:123-155, kernel 14-55; out_dtype TQ_F32) and
  * dequant_fp16 (metal.py:199-232, kernel 104-141; out_dtype TQ_F16).  TQ_BF16 also accepted.
@@ -233,6 +256,40 @@ int tq_vonly_decode_attn(const void* q, int q_dtype, const void* k_f16,
                          const float* v_centroids, const float* v_signs,
                          void* out, void* workspace, size_t workspace_bytes,
                          const tq_decode_shape* shape /* host */, tq_stream_t stream);
+
+/*
+ * A V-only cache as the library sees it between two growths of its storage: what a caller fills in
+ * once and reuses for every decode step (all four tensors share n_seq, n_kv_heads and t_alloc).
+ */
+typedef struct tq_vonly_cache_desc {
+  void* k_f16;               /* [n_seq, n_kv_heads, t_alloc, dim] float16, device */
+  void* v_raw;               /* [n_seq, n_kv_heads, t_alloc, dim] in the dtype of the new values, or NULL */
+  uint32_t* v_packed;        /* [n_seq, n_kv_heads, t_alloc, pdim] */
+  float* v_norms;            /* [n_seq, n_kv_heads, t_alloc] */
+  const float* v_signs;      /* [dim], device */
+  float boundaries[15];      /* 2^bits - 1 used */
+  float centroids[16];       /* 2^bits used */
+  void* workspace;           /* device, tq_workspace_bytes(TQ_OP_VONLY_DECODE, n_seq, n_q, t_alloc, dim) */
+  size_t workspace_bytes;
+  int64_t t_alloc;
+  int32_t n_seq, n_kv_heads, n_rep, dim, bits;
+  int32_t variant;           /* TQ_ENCODE_MLX / TQ_ENCODE_METAL */
+  int32_t allow_mma;         /* as in tq_decode_shape */
+} tq_vonly_cache_desc;
+
+/*
+ * One decode step of a V-only cache in one library call: tq_vonly_append of ONE new token per
+ * sequence at time index `position`, then tq_vonly_decode_attn of the query token over positions
+ * 0 .. position (both on `stream`, three launches, results identical to the two calls).
+ * Replaces, for a single-token step, VOnlyTurboQuantCache.update_and_fetch followed by the
+ * attention of hybrid_attention.py:52-88 / fused_attention.py:50-121 (v_only_cache.py:52-78).
+ *   k_new, v_new [n_seq, n_kv_heads, dim];  q [n_seq, n_kv_heads*n_rep, dim];  out likewise, out_dtype
+ * Fails with TQ_ERR_ARG when position is outside 0 .. t_alloc - 1.
+ */
+int tq_vonly_decode_step(const tq_vonly_cache_desc* cache /* host */,
+                         const void* k_new, int k_dtype, const void* v_new, int v_dtype,
+                         const void* q, int q_dtype, void* out, int out_dtype,
+                         int64_t position, float attn_scale, tq_stream_t stream);
 
 /*
  * The same call with its two passes selectable: phases = 1 runs only the tile pass (per-tile

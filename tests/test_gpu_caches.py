@@ -478,3 +478,112 @@ def test_packed_cache_with_bf16_and_float32_models(tq, dtype):
     b = patch.scaled_dot_product_attention(q1, kd, vd, plain, sc, None)
     assert a.dtype == dtype and a.shape == (B, n_q, 1, D)
     assert cos(host(a), host(b)) > 0.9995
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_vonly_cache_single_launch_append(tq, dtype):
+    """Decode-sized inserts of a fused V-only cache go through tq_vonly_append (one launch): across a
+    growth boundary and for 1, 3 and 16 tokens per step the stored keys, raw values, packed words and
+    norms equal those of the unfused cache (slice assignments + encoder) bit for bit, and the packed
+    words and norms equal the oracle's."""
+    B, n_kv, D = 2, 4, 128
+    plain, fused = tq.VOnlyTurboQuantCache(bits=3), tq.VOnlyTurboQuantCache(bits=3, fused=True)
+    ks, vs = [], []
+    for i, S in enumerate([250, 1, 3, 1, 1, 16, 1, 5]):             # 250 -> 278: grows at 256
+        k, v = rand((B, n_kv, S, D), 500 + 2 * i, dtype), rand((B, n_kv, S, D), 501 + 2 * i, dtype)
+        ks.append(k), vs.append(v)
+        plain.update_and_fetch(k, v)
+        k_out, v_out = fused.update_and_fetch(k, v)
+        assert fused.offset == plain.offset and k_out.shape[2] == fused.offset and v_out.shape[2] == fused.offset
+    assert fused._k_cache.keys.shape[2] == 512 and fused._v_tq.v_packed.shape[2] == 512
+    for x, y in zip(plain.state, fused.state):
+        assert x.dtype == y.dtype and torch.equal(x, y)
+    v_all = torch.cat(vs, dim=2)
+    want_p, want_n = oracle_pack(host(v_all), 43)
+    st = fused.state
+    assert np.array_equal(st[2].cpu().numpy().view(np.uint32), want_p)
+    assert np.array_equal(st[3].cpu().numpy(), want_n)
+    assert torch.equal(st[0], torch.cat(ks, dim=2).to(torch.float16))
+    assert torch.equal(st[1], v_all)
+
+
+def test_vonly_append_c_abi_other_shapes(tq):
+    """tq_vonly_append through ops.vonly_append_into at d = 64 / 2-bit and d = 256 / 4-bit, without the
+    raw value copy, at a position inside the storage: rows outside the inserted range stay untouched."""
+    from tqhip import ops
+    for D, bits, seed in ((64, 2, 7), (256, 4, 8)):
+        B, H, T, S, pos = 1, 3, 40, 5, 17
+        pd = ops.packed_dim(D, bits)
+        k, v = rand((B, H, S, D), 600 + D), rand((B, H, S, D), 601 + D, torch.float32)
+        signs = torch.from_numpy(o.random_diagonal_sign(D, seed)).cuda()
+        c = o.gaussian_codebook(bits)
+        bnd = o.gaussian_boundaries(c)
+        k16 = torch.full((B, H, T, D), 7.0, dtype=torch.float16, device="cuda")
+        vp = torch.full((B, H, T, pd), 123, dtype=torch.int32, device="cuda").view(torch.uint32)
+        vn = torch.full((B, H, T), -1.0, dtype=torch.float32, device="cuda")
+        ops.vonly_append_into(k, v, signs, bnd, k16, None, vp, vn, position=pos, bits=bits)
+        want_p, want_n = o.fused_quantize(host(v).reshape(-1, D), o.random_diagonal_sign(D, seed), bnd, D, bits, "mlx")
+        got_p = vp.cpu().numpy().view(np.uint32)
+        assert np.array_equal(got_p[:, :, pos:pos + S], want_p.reshape(B, H, S, pd))
+        assert np.array_equal(vn.cpu().numpy()[:, :, pos:pos + S], want_n.reshape(B, H, S))
+        assert torch.equal(k16[:, :, pos:pos + S], k)
+        keep = np.ones(T, bool); keep[pos:pos + S] = False
+        assert (got_p[:, :, keep] == 123).all() and (vn.cpu().numpy()[:, :, keep] == -1.0).all()
+        assert bool((k16[:, :, torch.from_numpy(keep).cuda()] == 7.0).all())
+    with pytest.raises(ValueError):
+        ops.vonly_append_into(k, v, signs, bnd, k16, None, vp, vn, position=T - 2, bits=bits)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_vonly_cache_decode_step_is_update_plus_attention(tq, dtype):
+    """decode_step (tq_vonly_decode_step: append + attention in one library call) gives, step after step
+    and across a growth of the storage, the very bits of update_and_fetch + vonly_decode_attention on a
+    twin cache, leaves the same state behind, and its output matches the float64 oracle."""
+    B, n_q, n_kv, D, S0 = 2, 28, 4, 128, 250
+    sc = 1 / math.sqrt(D)
+    k0, v0 = rand((B, n_kv, S0, D), 700, dtype), rand((B, n_kv, S0, D), 701, dtype)
+    a, b = tq.VOnlyTurboQuantCache(bits=3, fused=True), tq.VOnlyTurboQuantCache(bits=3, fused=True)
+    a.update_and_fetch(k0, v0), b.update_and_fetch(k0, v0)
+    for i in range(9):                                              # 250 -> 259: grows at 256
+        k1, v1, q1 = rand((B, n_kv, 1, D), 710 + 3 * i, dtype), rand((B, n_kv, 1, D), 711 + 3 * i, dtype), rand((B, n_q, 1, D), 712 + 3 * i, dtype)
+        got = a.decode_step(q1, k1, v1, sc)
+        b.update_and_fetch(k1, v1)
+        want = tq.vonly_decode_attention(q1, b, sc)
+        assert got.shape == (B, n_q, 1, D) and got.dtype == dtype and torch.equal(got, want), i
+    assert a.offset == b.offset == S0 + 9 and a._k_cache.keys.shape[2] == 512
+    for x, y in zip(a.state, b.state):
+        assert torch.equal(x, y)
+    st = a.state
+    vq = a._v_tq._v_q
+    for s in range(B):
+        ref = o.vonly_decode_attention(host(q1[s, :, 0]), st[0][s].cpu().numpy(), st[2][s].cpu().numpy().view(np.uint32),
+                                       st[3][s].cpu().numpy(), np.asarray(vq.centroids.cpu()), vq.signs.cpu().numpy(), D, 3, sc)
+        err = np.abs(host(got[s, :, 0]).astype(np.float64) - ref)
+        tol = 1e-3 + (2e-3 if dtype == torch.float16 else 6e-3) * np.abs(ref)
+        assert (err <= tol).all(), err.max()
+    # a step that the single call does not cover (two new tokens) falls back to the two calls
+    with pytest.raises(ValueError):
+        a.decode_step(rand((B, n_q, 2, D), 1), rand((B, n_kv, 2, D), 2, dtype), rand((B, n_kv, 2, D), 3, dtype), sc)
+
+
+def test_vonly_decode_step_refuses_bad_positions(tq):
+    from tqhip import ops
+    B, H, T, D = 1, 2, 256, 128
+    sg = o.random_diagonal_sign(D, 43)
+    signs = torch.from_numpy(sg).cuda()
+    c = o.gaussian_codebook(3)
+    bnd = o.gaussian_boundaries(c)
+    step = ops.VOnlyStep(torch.zeros((B, H, T, D), dtype=torch.float16, device="cuda"), None,
+                         torch.zeros((B, H, T, 13), dtype=torch.int32, device="cuda").view(torch.uint32),
+                         torch.zeros((B, H, T), device="cuda"), signs, bnd, c, n_rep=2, bits=3)
+    k, v, qq = rand((B, H, D), 1), rand((B, H, D), 2), rand((B, 4, D), 3)
+    with pytest.raises(ValueError):
+        ops.vonly_decode_step(step, k, v, qq, T, 0.1)
+    with pytest.raises(ValueError):
+        ops.vonly_decode_step(step, k, v, rand((B, 5, D), 3), 0, 0.1)
+    out = ops.vonly_decode_step(step, k, v, qq, 0, 0.1)             # one position: weight 1 -> out = dequant(v)
+    p, n = o.fused_quantize(host(v).reshape(-1, D), sg, bnd, D, 3, "mlx")
+    want = o.packed_dequantize(p, n, c, sg, D, 3)
+    assert out.shape == (B, 4, D)
+    for h in range(4):
+        assert np.allclose(host(out[0, h]), want[h // 2], rtol=2e-3, atol=1e-3)

@@ -1212,6 +1212,38 @@ extern "C" int tq_vonly_decode_attn(const void* q, int q_dtype, const void* k_f1
                                      workspace_bytes, shape, 3, stream_);
 }
 
+extern "C" int tq_vonly_decode_step(const tq_vonly_cache_desc* c, const void* k_new, int k_dtype, const void* v_new,
+                                    int v_dtype, const void* q, int q_dtype, void* out, int out_dtype,
+                                    int64_t position, float attn_scale, tq_stream_t stream_) {
+  const char* who = "tq_vonly_decode_step";
+  if (!c) return tq::fail(TQ_ERR_NULL, "%s: null cache descriptor", who);
+  if (int rc = tq::check_dim_bits(c->dim, c->bits)) return rc;
+  if (c->n_seq < 1 || c->n_kv_heads < 1 || c->t_alloc < 1)
+    return tq::fail(TQ_ERR_ARG, "%s: empty cache descriptor (n_seq %d, n_kv_heads %d, t_alloc %lld)", who, c->n_seq,
+                    c->n_kv_heads, (long long)c->t_alloc);
+  if (position < 0 || position >= c->t_alloc)
+    return tq::fail(TQ_ERR_ARG, "%s: position %lld outside the storage of %lld positions", who, (long long)position,
+                    (long long)c->t_alloc);
+  if (!c->k_f16 || !c->v_packed || !c->v_norms) return tq::fail(TQ_ERR_NULL, "%s: null pointer", who);
+  const int pdim = tq::packed_dim(c->dim, c->bits);
+  const int64_t groups = (int64_t)c->n_seq * c->n_kv_heads;
+  if (int rc = tq_vonly_append(
+          k_new, k_dtype, v_new, v_dtype, c->v_signs, c->boundaries, (__half*)c->k_f16 + position * c->dim,
+          c->v_raw ? (char*)c->v_raw + position * c->dim * (int64_t)tq::dtype_size(v_dtype) : nullptr,
+          c->v_packed + position * pdim, c->v_norms + position, groups, 1, c->t_alloc, c->t_alloc, c->t_alloc,
+          c->t_alloc, c->dim, c->bits, c->variant, stream_))
+    return rc;
+  tq_decode_shape sh{};
+  sh.n_seq = c->n_seq; sh.n_kv_heads = c->n_kv_heads; sh.n_rep = c->n_rep; sh.dim = c->dim; sh.bits = c->bits;
+  sh.block_size = 16;
+  sh.seq_len = position + 1;
+  sh.k_head_stride = sh.v_head_stride = sh.vn_head_stride = c->t_alloc;
+  sh.k_seq_stride = sh.v_seq_stride = sh.vn_seq_stride = c->t_alloc * c->n_kv_heads;
+  sh.attn_scale = attn_scale; sh.out_dtype = out_dtype; sh.allow_mma = c->allow_mma;
+  return tq_vonly_decode_attn(q, q_dtype, c->k_f16, c->v_packed, c->v_norms, c->centroids, c->v_signs, out,
+                              c->workspace, c->workspace_bytes, &sh, stream_);
+}
+
 extern "C" size_t tq_vonly_sparse_workspace_bytes(int n_seq, int n_q_heads, int64_t max_seq_len) {
   if (n_seq < 1 || n_q_heads < 1 || max_seq_len < 0) return 0;
   return vonly_sparse_ws_bytes(n_seq, n_q_heads, max_seq_len);

@@ -21,6 +21,18 @@ struct RowMap {
   int64_t n_rows, rows_per_group, packed_group_stride, norms_group_stride, out_group_stride;
 };
 
+// Optional row copies done by the wavefront that encodes a row (the append of a cache that keeps
+// float16 keys beside its packed values): key row `row` of k_src (dtype k_dtype) goes, converted to
+// float16, to k_dst + (g * k_group_stride + r) * D, and the value row itself, unchanged, to
+// v_dst + (g * v_group_stride + r) * D.  Null destinations switch a copy off.
+struct RowCopy {
+  const void* k_src;
+  __half* k_dst;
+  void* v_dst;
+  int64_t k_group_stride, v_group_stride;
+  int k_dtype;
+};
+
 // ---------------------------------------------------------------- encode
 // Per vector: sum of squares in stride-halving tree order, sqrt, divide by max(n, 1e-8), sign
 // flip, raw butterfly, count of thresholds exceeded (strict >), pack.  `thr` holds the decision
@@ -29,7 +41,7 @@ template <int D, int BITS, typename T>
 __global__ __launch_bounds__(kBlock) void encode_kernel(const T* __restrict__ x,
                                                         const float* __restrict__ signs,
                                                         Thresholds thr, uint32_t* __restrict__ packed,
-                                                        float* __restrict__ norms, RowMap rm) {
+                                                        float* __restrict__ norms, RowMap rm, RowCopy rc) {
   constexpr int EPL = Lay<D>::EPL;
   constexpr int VPW = Pk<BITS>::VPW;
   constexpr int PDIM = Pk<BITS>::pdim(D);
@@ -85,6 +97,27 @@ __global__ __launch_bounds__(kBlock) void encode_kernel(const T* __restrict__ x,
         packed[(g * rm.packed_group_stride + r) * PDIM + lane] = word;
       }
       if (lane == 0) norms[g * rm.norms_group_stride + r] = nrm;
+      if (rc.v_dst) {
+        T* vd = (T*)rc.v_dst + (g * rc.v_group_stride + r) * D;
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) {
+          const int e = lane + 64 * i;
+          if (e < D) vd[e] = x[row * D + e];
+        }
+      }
+      if (rc.k_dst) {
+        __half* kd = rc.k_dst + (g * rc.k_group_stride + r) * D;
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) {
+          const int e = lane + 64 * i;
+          if (e < D) {
+            const int64_t at = row * D + e;
+            if (rc.k_dtype == TQ_F16) kd[e] = ((const __half*)rc.k_src)[at];
+            else if (rc.k_dtype == TQ_F32) kd[e] = __float2half_rn(((const float*)rc.k_src)[at]);
+            else kd[e] = __float2half_rn(__bfloat162float(((const __hip_bfloat16*)rc.k_src)[at]));
+          }
+        }
+      }
     }
     __syncthreads();
   }
@@ -752,12 +785,52 @@ extern "C" int tq_encode(const void* x, int x_dtype, const float* signs, const f
   }
 #define LAUNCH_ENC(T)                                                                               \
   TQ_DISPATCH_DIM(dim, TQ_DISPATCH_BITS(bits, (encode_kernel<D_, B_, T><<<grid, kBlock, 0, stream>>>( \
-                                                  (const T*)x, signs, thr, packed, norms, rm))))
+                                                  (const T*)x, signs, thr, packed, norms, rm, RowCopy{}))))
   if (x_dtype == TQ_F32) { LAUNCH_ENC(float); }
   else if (x_dtype == TQ_F16) { LAUNCH_ENC(__half); }
   else { LAUNCH_ENC(__hip_bfloat16); }
 #undef LAUNCH_ENC
   TQ_CHECK_LAUNCH("tq_encode launch");
+  return TQ_OK;
+}
+
+extern "C" int tq_vonly_append(const void* k_new, int k_dtype, const void* v_new, int v_dtype,
+                               const float* v_signs, const float* boundaries, void* k_f16, void* v_raw,
+                               uint32_t* v_packed, float* v_norms, int64_t n_groups, int64_t rows_per_group,
+                               int64_t k_group_stride, int64_t v_raw_group_stride, int64_t packed_group_stride,
+                               int64_t norms_group_stride, int dim, int bits, int variant, tq_stream_t stream_) {
+  if (int rc = tq::check_dim_bits(dim, bits)) return rc;
+  if (tq::check_dtype(k_dtype) || tq::check_dtype(v_dtype))
+    return tq::fail(TQ_ERR_DTYPE, "tq_vonly_append: unknown dtype %d / %d", k_dtype, v_dtype);
+  if (variant != TQ_ENCODE_MLX && variant != TQ_ENCODE_METAL)
+    return tq::fail(TQ_ERR_ARG, "tq_vonly_append: unknown variant %d", variant);
+  if (n_groups < 0 || rows_per_group < 0) return tq::fail(TQ_ERR_ARG, "tq_vonly_append: negative row count");
+  const int64_t n_rows = n_groups * rows_per_group;
+  if (n_rows == 0) return TQ_OK;
+  if (!k_new || !v_new || !v_signs || !boundaries || !k_f16 || !v_packed || !v_norms)
+    return tq::fail(TQ_ERR_NULL, "tq_vonly_append: null pointer");
+  if (!tq::aligned(k_new, tq::dtype_size(k_dtype)) || !tq::aligned(v_new, tq::dtype_size(v_dtype)) ||
+      !tq::aligned(v_signs, 4) || !tq::aligned(k_f16, 2) || !tq::aligned(v_packed, 4) || !tq::aligned(v_norms, 4) ||
+      (v_raw && !tq::aligned(v_raw, tq::dtype_size(v_dtype))))
+    return tq::fail(TQ_ERR_ALIGN, "tq_vonly_append: misaligned pointer");
+  const int nb = (1 << bits) - 1;
+  Thresholds thr;
+  const float s = (float)(1.0 / sqrt((double)dim));
+  for (int i = 0; i < 15; ++i) thr.t[i] = INFINITY;
+  for (int i = 0; i < nb; ++i)
+    thr.t[i] = (variant == TQ_ENCODE_MLX) ? double_rounding_threshold(boundaries[i], s) : boundaries[i];
+  RowMap rm{n_rows, rows_per_group, packed_group_stride, norms_group_stride, 0};
+  RowCopy rc{k_new, (__half*)k_f16, v_raw, k_group_stride, v_raw_group_stride, k_dtype};
+  hipStream_t stream = (hipStream_t)stream_;
+  const int grid = grid_for_rows(n_rows);
+#define LAUNCH_APP(T)                                                                               \
+  TQ_DISPATCH_DIM(dim, TQ_DISPATCH_BITS(bits, (encode_kernel<D_, B_, T><<<grid, kBlock, 0, stream>>>( \
+                                                  (const T*)v_new, v_signs, thr, v_packed, v_norms, rm, rc))))
+  if (v_dtype == TQ_F32) { LAUNCH_APP(float); }
+  else if (v_dtype == TQ_F16) { LAUNCH_APP(__half); }
+  else { LAUNCH_APP(__hip_bfloat16); }
+#undef LAUNCH_APP
+  TQ_CHECK_LAUNCH("tq_vonly_append launch");
   return TQ_OK;
 }
 

@@ -25,6 +25,9 @@ from .ops import (
     flash_decode_from_q,
     prefill_attention,
     vonly_decode,
+    vonly_append_into,
+    vonly_decode_step,
+    VOnlyStep,
     dense_qk_scores,
     softmax_rows,
     pack_indices,

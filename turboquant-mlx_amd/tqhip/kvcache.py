@@ -42,14 +42,13 @@ class KVCache:
         self.values = None
         self.offset = 0
 
-    def update_and_fetch(self, keys: torch.Tensor, values: torch.Tensor):
+    def reserve(self, B, H, S, k_dim, v_dim, k_dtype, v_dtype, device):
+        """Make room for S more positions (growth in steps of 256, zero-filled) without inserting."""
         prev = self.offset
-        B, H, S, k_dim = keys.shape
-        v_dim = values.shape[3]
         if self.keys is None or prev + S > self.keys.shape[2]:
             n_steps = (self.step + S - 1) // self.step
-            new_k = torch.zeros((B, H, n_steps * self.step, k_dim), dtype=keys.dtype, device=keys.device)
-            new_v = torch.zeros((B, H, n_steps * self.step, v_dim), dtype=values.dtype, device=values.device)
+            new_k = torch.zeros((B, H, n_steps * self.step, k_dim), dtype=k_dtype, device=device)
+            new_v = torch.zeros((B, H, n_steps * self.step, v_dim), dtype=v_dtype, device=device)
             if self.keys is not None:
                 if prev % self.step != 0:
                     self.keys = self.keys[..., :prev, :]
@@ -58,6 +57,11 @@ class KVCache:
                 self.values = torch.cat([self.values, new_v], dim=2)
             else:
                 self.keys, self.values = new_k, new_v
+
+    def update_and_fetch(self, keys: torch.Tensor, values: torch.Tensor):
+        prev = self.offset
+        B, H, S, k_dim = keys.shape
+        self.reserve(B, H, S, k_dim, values.shape[3], keys.dtype, values.dtype, keys.device)
         self.offset += S
         self.keys[..., prev:self.offset, :] = keys
         self.values[..., prev:self.offset, :] = values

@@ -177,6 +177,38 @@ def encode_into(x: torch.Tensor, signs: torch.Tensor, boundaries, packed: torch.
         dim, bits, var, _stream(x)))
 
 
+def vonly_append_into(keys: torch.Tensor, values: torch.Tensor, signs: torch.Tensor, boundaries,
+                      k_f16: torch.Tensor, v_raw, v_packed: torch.Tensor, v_norms: torch.Tensor, *,
+                      position: int, bits: int, variant: str = "mlx") -> None:
+    """Insert the S new tokens `keys`, `values` [B, H, S, D] at time index `position` of a cache with
+    float16 keys `k_f16` [B, H, T_alloc, D], optional unencoded values `v_raw` (same dtype as
+    `values`, or None) and packed values `v_packed` [B, H, T_alloc, pdim] / `v_norms` [B, H, T_alloc]
+    in one launch (tq_vonly_append).  Same result as the slice assignments + encode_into of
+    VOnlyTurboQuantCache.update_and_fetch (v_only_cache.py:52-53)."""
+    _need_gpu(keys, values, signs, k_f16, v_packed, v_norms)
+    B, H, S, D = values.shape
+    if keys.shape != values.shape:
+        raise ValueError(f"keys {tuple(keys.shape)} and values {tuple(values.shape)} must have one shape")
+    if k_f16.dtype != torch.float16 or not k_f16.is_contiguous():
+        raise ValueError("k_f16 must be a contiguous float16 tensor")
+    for name, t in (("k_f16", k_f16), ("v_packed", v_packed), ("v_norms", v_norms)) + ((("v_raw", v_raw),) if v_raw is not None else ()):
+        if tuple(t.shape[:2]) != (B, H) or t.shape[2] < position + S:
+            raise ValueError(f"{name} {tuple(t.shape)} cannot hold positions {position}..{position + S} of {B} x {H} groups")
+    if v_raw is not None and (v_raw.dtype != values.dtype or not v_raw.is_contiguous()):
+        raise ValueError("v_raw must be contiguous and of the dtype of values")
+    keys, values = keys.contiguous(), values.contiguous()
+    pd = packed_dim(D, bits)
+    var = {"mlx": _lib.TQ_ENCODE_MLX, "metal": _lib.TQ_ENCODE_METAL}[variant]
+    lib = _lib.load()
+    _lib.check(lib.tq_vonly_append(
+        _ptr(keys), _dt(keys), _ptr(values), _dt(values), _ptr(signs), _host_table(boundaries),
+        C.c_void_p(k_f16.data_ptr() + position * D * 2),
+        None if v_raw is None else C.c_void_p(v_raw.data_ptr() + position * D * v_raw.element_size()),
+        C.c_void_p(v_packed.data_ptr() + position * pd * 4), C.c_void_p(v_norms.data_ptr() + position * 4),
+        B * H, S, k_f16.shape[2], 0 if v_raw is None else v_raw.shape[2], v_packed.shape[2], v_norms.shape[2],
+        D, bits, var, _stream(values)))
+
+
 def fused_quantize(vectors: torch.Tensor, signs: torch.Tensor, boundaries, dim: int, bits: int,
                    variant: str = "mlx"):
     """metal.py:147-196.  (n_vecs, dim) fp16/bf16/fp32 -> packed (n_vecs, pdim) uint32, norms (n_vecs,) f32.
@@ -662,6 +694,78 @@ def vonly_decode(q: torch.Tensor, k: torch.Tensor, v_packed, v_norms, v_centroid
     _lib.check(lib.tq_vonly_decode_attn(
         _ptr(q), _dt(q), _ptr(k), _ptr(v_packed), _ptr(v_norms), _host_table(v_centroids), _ptr(v_signs),
         _ptr(out), _ptr(ws), ws.numel(), C.byref(sh), stream))
+    return out
+
+
+class VOnlyStep:
+    """The storage of a V-only cache as tq_vonly_decode_step takes it (struct tq_vonly_cache_desc), filled in
+    once and reused until the storage is reallocated.  Keeps the tensors it points into alive."""
+
+    def __init__(self, k_f16: torch.Tensor, v_raw, v_packed: torch.Tensor, v_norms: torch.Tensor, signs: torch.Tensor,
+                 boundaries, centroids, *, n_rep: int, bits: int, variant: str = "mlx", precision: str = "fp16"):
+        _need_gpu(k_f16, v_raw, v_packed, v_norms, signs)
+        B, H, T, D = k_f16.shape
+        pd = packed_dim(D, bits)
+        if k_f16.dtype != torch.float16:
+            raise ValueError("k_f16 must be float16")
+        shapes = [("k_f16", k_f16, (B, H, T, D)), ("v_packed", v_packed, (B, H, T, pd)), ("v_norms", v_norms, (B, H, T))]
+        if v_raw is not None:
+            shapes.append(("v_raw", v_raw, (B, H, T, D)))
+        for name, t, want in shapes:
+            if tuple(t.shape) != want or not t.is_contiguous():
+                raise ValueError(f"{name} must be a contiguous {want} tensor, got {tuple(t.shape)}")
+        if v_norms.dtype != torch.float32:
+            raise ValueError("v_norms must be float32")
+        if n_rep < 1:
+            raise ValueError(f"n_rep must be >= 1, got {n_rep}")
+        self._keep = (k_f16, v_raw, v_packed, v_norms, signs)
+        self.v_dtype = None if v_raw is None else v_raw.dtype
+        self.shape = (B, H, T, D)
+        self.n_rep = n_rep
+        d = _lib.VOnlyCacheDesc()
+        d.k_f16, d.v_packed, d.v_norms, d.v_signs = k_f16.data_ptr(), _u32(v_packed).data_ptr(), v_norms.data_ptr(), signs.data_ptr()
+        d.v_raw = None if v_raw is None else v_raw.data_ptr()
+        b = [float(x) for x in (boundaries.tolist() if isinstance(boundaries, torch.Tensor) else boundaries)]
+        c = [float(x) for x in (centroids.tolist() if isinstance(centroids, torch.Tensor) else centroids)]
+        if len(b) != (1 << bits) - 1 or len(c) != 1 << bits:
+            raise ValueError(f"{bits}-bit tables need {(1 << bits) - 1} boundaries and {1 << bits} centroids")
+        for i, x in enumerate(b):
+            d.boundaries[i] = x
+        for i, x in enumerate(c):
+            d.centroids[i] = x
+        d.t_alloc, d.n_seq, d.n_kv_heads, d.n_rep, d.dim, d.bits = T, B, H, n_rep, D, bits
+        d.variant = {"mlx": _lib.TQ_ENCODE_MLX, "metal": _lib.TQ_ENCODE_METAL}[variant]
+        d.allow_mma = _mma_flag(precision)
+        self.desc = d
+        self._ref = C.byref(d)
+        self._need = _lib.load().tq_workspace_bytes(_lib.TQ_OP_VONLY_DECODE, B, H * n_rep, T, D)
+
+
+def vonly_decode_step(step: VOnlyStep, keys: torch.Tensor, values: torch.Tensor, q: torch.Tensor, position: int,
+                      attn_scale: float, out_dtype=None) -> torch.Tensor:
+    """One decode step of a V-only cache in one library call (tq_vonly_decode_step): insert the new token
+    keys / values (B, n_kv, dim) at time index `position`, then attend with q (B, n_kv * n_rep, dim) over
+    positions 0 .. position.  Same result as vonly_append_into followed by vonly_decode.  Returns
+    (B, n_q, dim) in out_dtype (default q.dtype)."""
+    _need_gpu(keys, values, q)
+    B, H, T, D = step.shape
+    n_q = H * step.n_rep
+    if tuple(keys.shape) != (B, H, D) or tuple(values.shape) != (B, H, D) or tuple(q.shape) != (B, n_q, D):
+        raise ValueError(f"expected keys / values {(B, H, D)} and q {(B, n_q, D)}, got {tuple(keys.shape)}, "
+                         f"{tuple(values.shape)}, {tuple(q.shape)}")
+    if step.v_dtype is not None and values.dtype != step.v_dtype:
+        raise ValueError(f"values are {values.dtype}, the cache keeps {step.v_dtype}")
+    if not 0 <= position < T:
+        raise ValueError(f"position {position} outside the storage of {T} positions")
+    keys, values, q = keys.contiguous(), values.contiguous(), q.contiguous()
+    out = torch.empty((B, n_q, D), dtype=out_dtype or q.dtype, device=q.device)
+    stream = _stream(q)
+    ws = _workspace(q.device, stream.value or 0, step._need)
+    d = step.desc
+    d.workspace, d.workspace_bytes = ws.data_ptr(), ws.numel()
+    _lib.check(_lib.load().tq_vonly_decode_step(
+        step._ref, _ptr(keys), _dt(keys), _ptr(values), _dt(values), _ptr(q), _dt(q), _ptr(out), _dt(out),
+        position, attn_scale, stream))
     return out
 
 

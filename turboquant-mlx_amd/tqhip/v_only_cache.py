@@ -26,6 +26,7 @@ class VOnlyTurboQuantCache:
         self._no_v_buffer = no_v_buffer
         self.fused = fused
         self._zero, self._zero_key = None, None
+        self._step, self._step_key = None, None
 
     def _encode_only(self, keys, values):
         tq = self._v_tq
@@ -35,6 +36,70 @@ class VOnlyTurboQuantCache:
         tq._ensure_storage(B, H, S, values.device)
         tq._encode(values, tq._v_q, tq.v_packed, tq.v_norms, B, H, S, v_dim, tq.offset)
         tq.offset += S
+
+    # Decode-sized inserts of a fused cache go through one launch (key rows to float16, value rows
+    # raw and encoded) instead of two slice assignments, a cast and the encoder.
+    _FUSED_APPEND_MAX_TOKENS = 16
+
+    def _append_fused(self, keys, values) -> bool:
+        from . import ops
+        kc, tq = self._k_cache, self._v_tq
+        B, H, S, v_dim = values.shape
+        if (S > self._FUSED_APPEND_MAX_TOKENS or keys.shape != values.shape or not values.is_cuda
+                or (kc.values is not None and kc.values.dtype != values.dtype)
+                or (kc.keys is not None and kc.keys.dtype != torch.float16)
+                or kc.offset != tq.offset):
+            return False
+        kc.reserve(B, H, S, keys.shape[3], v_dim, torch.float16, values.dtype, values.device)
+        tq._dtype = keys.dtype
+        tq._ensure_quantizer(keys.shape[-1], v_dim, values.device)
+        tq._ensure_storage(B, H, S, values.device)
+        if not (kc.keys.is_contiguous() and kc.values.is_contiguous() and tq.v_packed.is_contiguous()
+                and tq.v_norms.is_contiguous()):
+            return False                  # storage handed in through `state` as slices: the general path copes
+        ops.vonly_append_into(keys, values, tq._v_q.signs, tq._v_q.boundaries, kc.keys, kc.values,
+                              tq.v_packed, tq.v_norms, position=kc.offset, bits=tq.quant_bits,
+                              variant=tq.encode_variant)
+        kc.offset += S
+        tq.offset += S
+        return True
+
+    def decode_step(self, queries: torch.Tensor, keys: torch.Tensor, values: torch.Tensor, attn_scale: float):
+        """Insert one token and attend in one library call: the result of `update_and_fetch(keys, values)`
+        followed by `vonly_decode_attention(queries, self, attn_scale)` (no mask, no sparse-V threshold).
+        queries (B, n_heads, 1, dim), keys / values (B, n_kv, 1, dim) -> (B, n_heads, 1, dim) in queries.dtype.
+        Not in the reference, where the two halves are separate calls of the model's attention layer
+        (v_only_cache.py:52-78, then SDPA)."""
+        from . import attention, ops
+        kc, tq = self._k_cache, self._v_tq
+        B, n_q, S_q, dim = queries.shape
+        H = values.shape[1]
+        if (S_q != 1 or values.shape[2] != 1 or keys.shape != values.shape or n_q % H or not values.is_cuda
+                or queries.dtype not in (torch.float16, torch.bfloat16, torch.float32)
+                or (kc.values is not None and kc.values.dtype != values.dtype)
+                or (kc.keys is not None and kc.keys.dtype != torch.float16) or kc.offset != tq.offset):
+            self.update_and_fetch(keys, values)
+            return attention.vonly_decode_attention(queries, self, attn_scale)
+        kc.reserve(B, H, 1, dim, dim, torch.float16, values.dtype, values.device)
+        tq._dtype = keys.dtype
+        tq._ensure_quantizer(dim, dim, values.device)
+        tq._ensure_storage(B, H, 1, values.device)
+        key = (kc.keys.data_ptr(), kc.values.data_ptr(), tq.v_packed.data_ptr(), tq.v_norms.data_ptr(),
+               kc.keys.shape[2], n_q)
+        if self._step_key != key:
+            try:
+                self._step = ops.VOnlyStep(kc.keys, kc.values, tq.v_packed, tq.v_norms, tq._v_q.signs,
+                                           tq._v_q.boundaries, tq._v_q.centroids, n_rep=n_q // H,
+                                           bits=tq.quant_bits, variant=tq.encode_variant)
+            except ValueError:                     # storage handed in through `state` as slices
+                self.update_and_fetch(keys, values)
+                return attention.vonly_decode_attention(queries, self, attn_scale)
+            self._step_key = key
+        out = ops.vonly_decode_step(self._step, keys[:, :, 0, :], values[:, :, 0, :], queries[:, :, 0, :],
+                                    kc.offset, attn_scale)
+        kc.offset += 1
+        tq.offset += 1
+        return out[:, :, None, :]
 
     def dequantized_values(self, dtype=None) -> torch.Tensor:
         """All cached values, dequantised: [B, H, offset, D]."""
@@ -46,10 +111,14 @@ class VOnlyTurboQuantCache:
         # The decode kernels read float16 keys: bf16 / float32 keys are stored as float16 (exact for bf16
         # values inside the float16 range, which keys are); the reference keeps whatever dtype it is
         # given (v_only_cache.py:41-47), so `state` then differs in the dtype of its first entry.
-        k16 = keys if keys.dtype == torch.float16 else keys.to(torch.float16)
-        k_out, _ = self._k_cache.update_and_fetch(k16, values)
+        if self.fused and self._append_fused(keys, values):
+            k_out = self._k_cache.keys[..., :self._k_cache.offset, :]
+        else:
+            k16 = keys if keys.dtype == torch.float16 else keys.to(torch.float16)
+            k_out, _ = self._k_cache.update_and_fetch(k16, values)
+            if self.fused:
+                self._encode_only(keys, values)
         if self.fused:
-            self._encode_only(keys, values)
             B, H, _, v_dim = values.shape
             key = (values.dtype, values.device)
             if self._zero is None or self._zero_key != key:          # one element, made once
