@@ -146,8 +146,8 @@ def main():
                 C.c_void_p(vn.data_ptr()), cb_host, C.c_void_p(signs.data_ptr()), C.c_void_p(outs[i].data_ptr()),
                 C.c_void_p(ws.data_ptr()), ws.numel(), C.byref(shape), C.c_void_p(stream))
 
-    def step(i, argsets, phases=3):
-        a = argsets[i % N_SETS]
+    def step(i, argsets, phases=3, rot=N_SETS):
+        a = argsets[i % rot]
         rc = lib.tq_vonly_decode_attn_phases(*a[:-1], phases, a[-1])
         if rc != 0:
             _lib.check(rc)
@@ -157,6 +157,7 @@ def main():
     eager_args = [bound(i, cur.cuda_stream) for i in range(N_SETS)]
     step(0, eager_args)
     torch.cuda.synchronize()
+    checked = outs[0].clone()
     cpu = None
     if not args.no_cpu:
         ref, cpu = cpu_baseline(torch, sets, cb, signs)
@@ -167,19 +168,19 @@ def main():
 
     side = torch.cuda.Stream(device=dev)
 
-    def timed(phases):
+    def timed(phases, rot=N_SETS):
         """ms per launch of `args.steps` back-to-back calls (HIP graph replay unless --no-graph),
-        bracketed by HIP events on the launch stream."""
+        bracketed by HIP events on the launch stream, rotating over the first `rot` buffer sets."""
         ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         with torch.cuda.stream(side):
             s_args = [bound(i, side.cuda_stream) for i in range(N_SETS)]
             for i in range(args.warmup):
-                step(i, s_args, phases)
+                step(i, s_args, phases, rot)
             side.synchronize()
             if args.no_graph:
                 ev0.record(side)
                 for i in range(args.steps):
-                    step(i, s_args, phases)
+                    step(i, s_args, phases, rot)
                 ev1.record(side)
                 side.synchronize()
             else:
@@ -188,7 +189,7 @@ def main():
                     g_stream = torch.cuda.current_stream(dev)
                     g_args = [bound(i, g_stream.cuda_stream) for i in range(N_SETS)]
                     for i in range(args.steps):
-                        step(i, g_args, phases)
+                        step(i, g_args, phases, rot)
                 graph.replay()                  # one untimed replay: instantiation, page-in
                 torch.cuda.synchronize()
                 ev0.record(side)
@@ -201,14 +202,15 @@ def main():
     mode = "eager" if args.no_graph else "hipgraph"
     ms_per_step = timed(3)                      # whole step: tile pass + merge pass
     ms_tile = timed(1)                          # dominant kernel alone, same launch pattern
+    ms_warm = timed(3, rot=1)                   # one buffer set over and over: its 41 MB stay in the 256 MB Infinity Cache
     gbs = ALGO_BYTES / (ms_per_step * 1e-3) / 1e9
     gbs_tile = ALGO_BYTES / (ms_tile * 1e-3) / 1e9
     step(0, eager_args)                         # leave outs[0] = the full result of set 0
     torch.cuda.synchronize()
 
     # the timed steps must have produced the same result as the checked eager step
-    if not torch.equal(outs[0], outs[0]) or torch.isnan(outs[0]).any():
-        print("bench: NaN in timed output", file=sys.stderr)
+    if not torch.equal(outs[0], checked):
+        print("bench: the timed steps left a result that differs from the checked one", file=sys.stderr)
         sys.exit(1)
 
     line = {
@@ -227,6 +229,9 @@ def main():
                      "note": "algorithmic bytes / event-timed launch period of the tile pass alone; "
                              "`value` covers the whole step (tile pass + merge pass)"},
         "cpu_baseline": cpu,
+        "warm_cache": {"us_per_layer": round(ms_warm * 1e3, 3), "value": round(ALGO_BYTES / (ms_warm * 1e-3) / 1e9, 1),
+                       "unit": "GB/s", "note": "same step on ONE buffer set (inputs served from the Infinity Cache); "
+                                               "reported beside `value`, never as it"},
     }
     print(json.dumps(line))
 

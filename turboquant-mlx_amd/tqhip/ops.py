@@ -196,6 +196,10 @@ def vonly_append_into(keys: torch.Tensor, values: torch.Tensor, signs: torch.Ten
             raise ValueError(f"{name} {tuple(t.shape)} cannot hold positions {position}..{position + S} of {B} x {H} groups")
     if v_raw is not None and (v_raw.dtype != values.dtype or not v_raw.is_contiguous()):
         raise ValueError("v_raw must be contiguous and of the dtype of values")
+    if (v_packed.dtype not in (torch.uint32, torch.int32) or v_norms.dtype != torch.float32
+            or not v_packed.is_contiguous() or not v_norms.is_contiguous()):
+        raise ValueError("v_packed must be contiguous uint32 and v_norms contiguous float32")
+    signs = _as_f32_dev(signs, values)
     keys, values = keys.contiguous(), values.contiguous()
     pd = packed_dim(D, bits)
     var = {"mlx": _lib.TQ_ENCODE_MLX, "metal": _lib.TQ_ENCODE_METAL}[variant]
@@ -716,6 +720,8 @@ class VOnlyStep:
                 raise ValueError(f"{name} must be a contiguous {want} tensor, got {tuple(t.shape)}")
         if v_norms.dtype != torch.float32:
             raise ValueError("v_norms must be float32")
+        if v_packed.dtype not in (torch.uint32, torch.int32):
+            raise ValueError("v_packed must be uint32 (or its int32 view)")
         if n_rep < 1:
             raise ValueError(f"n_rep must be >= 1, got {n_rep}")
         self._keep = (k_f16, v_raw, v_packed, v_norms, signs)
@@ -723,7 +729,7 @@ class VOnlyStep:
         self.shape = (B, H, T, D)
         self.n_rep = n_rep
         d = _lib.VOnlyCacheDesc()
-        d.k_f16, d.v_packed, d.v_norms, d.v_signs = k_f16.data_ptr(), _u32(v_packed).data_ptr(), v_norms.data_ptr(), signs.data_ptr()
+        d.k_f16, d.v_packed, d.v_norms, d.v_signs = k_f16.data_ptr(), v_packed.data_ptr(), v_norms.data_ptr(), signs.data_ptr()
         d.v_raw = None if v_raw is None else v_raw.data_ptr()
         b = [float(x) for x in (boundaries.tolist() if isinstance(boundaries, torch.Tensor) else boundaries)]
         c = [float(x) for x in (centroids.tolist() if isinstance(centroids, torch.Tensor) else centroids)]
