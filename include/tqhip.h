@@ -292,6 +292,40 @@ int tq_vonly_decode_step(const tq_vonly_cache_desc* cache /* host */,
                          int64_t position, float attn_scale, tq_stream_t stream);
 
 /*
+ * A cache with packed keys AND values as the library sees it between two growths of its storage
+ * (all four tensors share n_seq, n_kv_heads and t_alloc; keys and values share dim and bits, hence
+ * the tables, and differ in their sign vectors: seeds s and s + 1 of cache.py:92,96).
+ */
+typedef struct tq_packed_cache_desc {
+  uint32_t* k_packed;        /* [n_seq, n_kv_heads, t_alloc, pdim] */
+  float* k_norms;            /* [n_seq, n_kv_heads, t_alloc] */
+  uint32_t* v_packed;
+  float* v_norms;
+  const float* k_signs;      /* [dim], device */
+  const float* v_signs;
+  float boundaries[15];      /* 2^bits - 1 used */
+  float centroids[16];       /* 2^bits used */
+  void* workspace;           /* device, tq_workspace_bytes(TQ_OP_FLASH_DECODE, n_seq, n_q, t_alloc, dim) */
+  size_t workspace_bytes;
+  int64_t t_alloc;
+  int32_t n_seq, n_kv_heads, n_rep, dim, bits;
+  int32_t variant;           /* TQ_ENCODE_MLX / TQ_ENCODE_METAL */
+} tq_packed_cache_desc;
+
+/*
+ * One decode step of a packed cache in one library call: tq_encode of ONE new key and value row
+ * per sequence and kv head at time index `position`, then tq_flash_decode_from_q (no mask, no
+ * threshold) of the query token over positions 0 .. position; results identical to the three calls.
+ * Replaces, for a single-token step, TurboQuantKVCache.update_and_fetch (cache.py:131-165) followed
+ * by turboquant_attention (fused_attention.py:20-125).  Shapes and errors as tq_vonly_decode_step;
+ * TQ_ERR_UNSUPPORTED where tq_flash_decode_from_q has no kernel (it needs dim 128, 3 bits, n_rep <= 16).
+ */
+int tq_packed_decode_step(const tq_packed_cache_desc* cache /* host */,
+                          const void* k_new, int k_dtype, const void* v_new, int v_dtype,
+                          const void* q, int q_dtype, void* out, int out_dtype,
+                          int64_t position, float attn_scale, tq_stream_t stream);
+
+/*
  * The same call with its two passes selectable: phases = 1 runs only the tile pass (per-tile
  * partial sums and softmax statistics into `workspace`), phases = 2 only the merge pass (workspace
  * -> out), phases = 3 both (= tq_vonly_decode_attn).  For callers that time or overlap the passes;

@@ -587,3 +587,39 @@ def test_vonly_decode_step_refuses_bad_positions(tq):
     assert out.shape == (B, 4, D)
     for h in range(4):
         assert np.allclose(host(out[0, h]), want[h // 2], rtol=2e-3, atol=1e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_packed_cache_decode_step_is_update_plus_attention(tq, dtype):
+    """TurboQuantKVCache.decode_step (tq_packed_decode_step: two encodes + attention from the unrotated query
+    in one library call) gives, step after step and across a growth of the storage, the very bits of
+    update_and_fetch + turboquant_attention(fused=True) on a twin cache, leaves the same state behind, and
+    its output matches the float64 oracle; a 4-bit cache takes the two-call route and agrees as well."""
+    B, n_q, n_kv, D, S0 = 2, 32, 8, 128, 250
+    sc = 1 / math.sqrt(D)
+    k0, v0 = rand((B, n_kv, S0, D), 800, dtype), rand((B, n_kv, S0, D), 801, dtype)
+    a, b = tq.TurboQuantKVCache(bits=3, fused=True), tq.TurboQuantKVCache(bits=3, fused=True)
+    a.update_and_fetch(k0, v0), b.update_and_fetch(k0, v0)
+    for i in range(9):                                              # 250 -> 259: grows at 256
+        k1, v1, q1 = rand((B, n_kv, 1, D), 810 + 3 * i, dtype), rand((B, n_kv, 1, D), 811 + 3 * i, dtype), rand((B, n_q, 1, D), 812 + 3 * i, dtype)
+        got = a.decode_step(q1, k1, v1, sc)
+        b.update_and_fetch(k1, v1)
+        want = tq.turboquant_attention(q1, b, sc, fused=True)
+        assert got.shape == (B, n_q, 1, D) and got.dtype == dtype and torch.equal(got, want), i
+    assert a.offset == b.offset == S0 + 9 and a.v_packed.shape[2] == 512
+    for x, y in zip(a.state, b.state):
+        assert torch.equal(x, y)
+    kp, kn, vp, vn = [t.cpu().numpy() for t in a.state]
+    kq, vq = a._k_q, a._v_q
+    for s in range(B):
+        ref = o.turboquant_attention_single(host(q1[s, :, 0]), kp[s].view(np.uint32), kn[s], vp[s].view(np.uint32), vn[s],
+                                            np.asarray(kq.centroids.cpu()), kq.signs.cpu().numpy(),
+                                            np.asarray(vq.centroids.cpu()), vq.signs.cpu().numpy(), D, 3, sc)
+        err = np.abs(host(got[s, :, 0]).astype(np.float64) - ref)
+        tol = 1e-3 + (2e-3 if dtype == torch.float16 else 6e-3) * np.abs(ref)
+        assert (err <= tol).all(), err.max()
+    c4, d4 = tq.TurboQuantKVCache(bits=4, fused=True), tq.TurboQuantKVCache(bits=4, fused=True)
+    c4.update_and_fetch(k0, v0), d4.update_and_fetch(k0, v0)
+    got = c4.decode_step(q1, k1, v1, sc)
+    d4.update_and_fetch(k1, v1)
+    assert torch.equal(got, tq.turboquant_attention(q1, d4, sc, fused=True)) and c4.offset == d4.offset

@@ -1312,3 +1312,38 @@ extern "C" int tq_flash_decode_from_q(const void* q, int q_dtype, const float* k
   return launch_packed_mfma<tqm::kFlash>(nullptr, k_packed, k_norms, v_packed, v_norms, k_centroids, v_centroids, v_signs,
                                          out, workspace, workspace_bytes, sh, 0.0f, stream, who, q, q_dtype, k_signs);
 }
+
+extern "C" int tq_packed_decode_step(const tq_packed_cache_desc* c, const void* k_new, int k_dtype, const void* v_new,
+                                     int v_dtype, const void* q, int q_dtype, void* out, int out_dtype,
+                                     int64_t position, float attn_scale, tq_stream_t stream_) {
+  const char* who = "tq_packed_decode_step";
+  if (!c) return tq::fail(TQ_ERR_NULL, "%s: null cache descriptor", who);
+  if (int rc = tq::check_dim_bits(c->dim, c->bits)) return rc;
+  if (c->n_seq < 1 || c->n_kv_heads < 1 || c->t_alloc < 1)
+    return tq::fail(TQ_ERR_ARG, "%s: empty cache descriptor (n_seq %d, n_kv_heads %d, t_alloc %lld)", who, c->n_seq,
+                    c->n_kv_heads, (long long)c->t_alloc);
+  if (position < 0 || position >= c->t_alloc)
+    return tq::fail(TQ_ERR_ARG, "%s: position %lld outside the storage of %lld positions", who, (long long)position,
+                    (long long)c->t_alloc);
+  if (!c->k_packed || !c->k_norms || !c->v_packed || !c->v_norms) return tq::fail(TQ_ERR_NULL, "%s: null pointer", who);
+  if (!(c->dim == 128 && c->bits == 3 && c->n_rep >= 1 && c->n_rep <= tqm::kHeadsMax))
+    return tq::fail(TQ_ERR_UNSUPPORTED, "%s: dim 128, 3-bit and n_rep <= 16 only (call tq_encode, "
+                                        "tq_prerotate_query and tq_flash_decode otherwise)", who);
+  const int pdim = tq::packed_dim(c->dim, c->bits);
+  const int64_t groups = (int64_t)c->n_seq * c->n_kv_heads;
+  if (int rc = tq_encode(k_new, k_dtype, c->k_signs, c->boundaries, c->k_packed + position * pdim, c->k_norms + position,
+                         groups, 1, c->t_alloc, c->t_alloc, c->dim, c->bits, c->variant, stream_))
+    return rc;
+  if (int rc = tq_encode(v_new, v_dtype, c->v_signs, c->boundaries, c->v_packed + position * pdim, c->v_norms + position,
+                         groups, 1, c->t_alloc, c->t_alloc, c->dim, c->bits, c->variant, stream_))
+    return rc;
+  tq_decode_shape sh{};
+  sh.n_seq = c->n_seq; sh.n_kv_heads = c->n_kv_heads; sh.n_rep = c->n_rep; sh.dim = c->dim; sh.bits = c->bits;
+  sh.block_size = 16;
+  sh.seq_len = position + 1;
+  sh.k_head_stride = sh.kn_head_stride = sh.v_head_stride = sh.vn_head_stride = c->t_alloc;
+  sh.k_seq_stride = sh.kn_seq_stride = sh.v_seq_stride = sh.vn_seq_stride = c->t_alloc * c->n_kv_heads;
+  sh.attn_scale = attn_scale; sh.out_dtype = out_dtype; sh.allow_mma = 1;
+  return tq_flash_decode_from_q(q, q_dtype, c->k_signs, c->k_packed, c->k_norms, c->v_packed, c->v_norms, c->centroids,
+                                c->centroids, c->v_signs, 0.0f, out, c->workspace, c->workspace_bytes, &sh, stream_);
+}

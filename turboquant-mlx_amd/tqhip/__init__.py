@@ -28,6 +28,8 @@ from .ops import (
     vonly_append_into,
     vonly_decode_step,
     VOnlyStep,
+    packed_decode_step,
+    PackedStep,
     dense_qk_scores,
     softmax_rows,
     pack_indices,

@@ -49,6 +49,17 @@ class VOnlyCacheDesc(C.Structure):
     ]
 
 
+class PackedCacheDesc(C.Structure):
+    """Mirror of struct tq_packed_cache_desc."""
+    _fields_ = [
+        ("k_packed", C.c_void_p), ("k_norms", C.c_void_p), ("v_packed", C.c_void_p), ("v_norms", C.c_void_p),
+        ("k_signs", C.c_void_p), ("v_signs", C.c_void_p), ("boundaries", C.c_float * 15), ("centroids", C.c_float * 16),
+        ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t), ("t_alloc", C.c_int64),
+        ("n_seq", C.c_int32), ("n_kv_heads", C.c_int32), ("n_rep", C.c_int32), ("dim", C.c_int32),
+        ("bits", C.c_int32), ("variant", C.c_int32),
+    ]
+
+
 # name -> (restype, argtypes); the authoritative list of exported symbols
 PROTOTYPES = {
     "tq_version": (_i, []),
@@ -67,6 +78,7 @@ PROTOTYPES = {
     "tq_flash_decode_plan": (_i, [_i, _i, _l, _i, _i]),
     "tq_vonly_decode_attn": (_i, [_p, _i, _p, _p, _p, _fp, _p, _p, _p, _z, C.POINTER(DecodeShape), _p]),
     "tq_vonly_decode_step": (_i, [C.POINTER(VOnlyCacheDesc), _p, _i, _p, _i, _p, _i, _p, _i, _l, _f, _p]),
+    "tq_packed_decode_step": (_i, [C.POINTER(PackedCacheDesc), _p, _i, _p, _i, _p, _i, _p, _i, _l, _f, _p]),
     "tq_vonly_decode_attn_phases": (_i, [_p, _i, _p, _p, _p, _fp, _p, _p, _p, _z, C.POINTER(DecodeShape), _i, _p]),
     "tq_vonly_sparse_decode_attn": (_i, [_p, _i, _p, _p, _p, _fp, _p, _f, _p, _p, _z, C.POINTER(DecodeShape), _p]),
     "tq_vonly_sparse_workspace_bytes": (_z, [_i, _i, _l]),

@@ -89,6 +89,7 @@ class TurboQuantKVCache:
         self._k_pdim = None
         self._v_pdim = None
         self._dtype = None
+        self._step, self._step_key = None, None
 
     # ---------------------------------------------------------------- setup (cache.py:90-123)
     def _device(self):
@@ -191,6 +192,42 @@ class TurboQuantKVCache:
         if z is None:
             z = self._zero_scalars[key] = t.new_zeros(())
         return z
+
+    def decode_step(self, queries: torch.Tensor, keys: torch.Tensor, values: torch.Tensor, attn_scale: float):
+        """Encode one token and attend in one library call: the result of `update_and_fetch(keys, values)`
+        followed by `turboquant_attention(queries, self, attn_scale, fused=True)` (no mask, no threshold) on
+        a cache with packed keys and values.  queries (B, n_heads, 1, dim), keys / values (B, n_kv, 1, dim)
+        -> (B, n_heads, 1, dim) in queries.dtype.  Not in the reference, where the two halves are separate
+        calls of the model's attention layer (cache.py:131-165, fused_attention.py:20-125)."""
+        from . import attention
+        B, n_q, S_q, dim = queries.shape
+        H = values.shape[1]
+        ok = (not self.v_only and S_q == 1 and values.shape[2] == 1 and keys.shape == values.shape
+              and keys.shape[3] == dim and n_q % H == 0 and values.is_cuda
+              and queries.dtype in (torch.float16, torch.bfloat16, torch.float32)
+              and ops.vonly_sparse_supported(dim, self.quant_bits, n_q // H))
+        if ok:
+            self._dtype = keys.dtype
+            self._ensure_quantizer(dim, dim, values.device)
+            self._ensure_storage(B, H, 1, values.device)
+            key = (self.k_packed.data_ptr(), self.k_norms.data_ptr(), self.v_packed.data_ptr(),
+                   self.v_norms.data_ptr(), self.v_packed.shape[2], n_q)
+            if self._step_key != key:
+                try:
+                    self._step = ops.PackedStep(self.k_packed, self.k_norms, self.v_packed, self.v_norms,
+                                                self._k_q.signs, self._v_q.signs, self._v_q.boundaries,
+                                                self._v_q.centroids, dim=dim, n_rep=n_q // H, bits=self.quant_bits,
+                                                variant=self.encode_variant)
+                    self._step_key = key
+                except ValueError:                 # storage handed in through `state` as slices
+                    ok = False
+        if not ok:
+            self.update_and_fetch(keys, values)
+            return attention.turboquant_attention(queries, self, attn_scale, fused=True)
+        out = ops.packed_decode_step(self._step, keys[:, :, 0, :], values[:, :, 0, :], queries[:, :, 0, :],
+                                     self.offset, attn_scale)
+        self.offset += 1          # _deq_offset stays behind: the next unfused fetch dequantises the whole cache
+        return out[:, :, None, :]
 
     def update_and_fetch(self, keys: torch.Tensor, values: torch.Tensor):
         B, H, S, k_dim = keys.shape

@@ -775,6 +775,77 @@ def vonly_decode_step(step: VOnlyStep, keys: torch.Tensor, values: torch.Tensor,
     return out
 
 
+def _fill_table(dst, values, n, what):
+    vals = [float(x) for x in (values.tolist() if isinstance(values, torch.Tensor) else values)]
+    if len(vals) != n:
+        raise ValueError(f"expected {n} {what}, got {len(vals)}")
+    for i, x in enumerate(vals):
+        dst[i] = x
+
+
+class PackedStep:
+    """The storage of a cache with packed keys and values as tq_packed_decode_step takes it (struct
+    tq_packed_cache_desc), filled in once and reused until the storage is reallocated.  Keeps the tensors
+    it points into alive."""
+
+    def __init__(self, k_packed: torch.Tensor, k_norms: torch.Tensor, v_packed: torch.Tensor, v_norms: torch.Tensor,
+                 k_signs: torch.Tensor, v_signs: torch.Tensor, boundaries, centroids, *, dim: int, n_rep: int,
+                 bits: int, variant: str = "mlx"):
+        _need_gpu(k_packed, k_norms, v_packed, v_norms, k_signs, v_signs)
+        B, H, T = k_norms.shape
+        pd = packed_dim(dim, bits)
+        for name, t, want, dts in (("k_packed", k_packed, (B, H, T, pd), (torch.uint32, torch.int32)),
+                                   ("v_packed", v_packed, (B, H, T, pd), (torch.uint32, torch.int32)),
+                                   ("k_norms", k_norms, (B, H, T), (torch.float32,)),
+                                   ("v_norms", v_norms, (B, H, T), (torch.float32,))):
+            if tuple(t.shape) != want or not t.is_contiguous() or t.dtype not in dts:
+                raise ValueError(f"{name} must be a contiguous {want} tensor of {dts[0]}, got {tuple(t.shape)} {t.dtype}")
+        for name, t in (("k_signs", k_signs), ("v_signs", v_signs)):
+            if t.dtype != torch.float32 or t.numel() != dim or not t.is_contiguous():
+                raise ValueError(f"{name} must be {dim} contiguous float32 values")
+        if n_rep < 1:
+            raise ValueError(f"n_rep must be >= 1, got {n_rep}")
+        self._keep = (k_packed, k_norms, v_packed, v_norms, k_signs, v_signs)
+        self.shape = (B, H, T, dim)
+        self.n_rep = n_rep
+        d = _lib.PackedCacheDesc()
+        d.k_packed, d.k_norms, d.v_packed, d.v_norms = k_packed.data_ptr(), k_norms.data_ptr(), v_packed.data_ptr(), v_norms.data_ptr()
+        d.k_signs, d.v_signs = k_signs.data_ptr(), v_signs.data_ptr()
+        _fill_table(d.boundaries, boundaries, (1 << bits) - 1, "boundaries")
+        _fill_table(d.centroids, centroids, 1 << bits, "centroids")
+        d.t_alloc, d.n_seq, d.n_kv_heads, d.n_rep, d.dim, d.bits = T, B, H, n_rep, dim, bits
+        d.variant = {"mlx": _lib.TQ_ENCODE_MLX, "metal": _lib.TQ_ENCODE_METAL}[variant]
+        self.desc = d
+        self._ref = C.byref(d)
+        self._need = _lib.load().tq_workspace_bytes(_lib.TQ_OP_FLASH_DECODE, B, H * n_rep, T, dim)
+
+
+def packed_decode_step(step: PackedStep, keys: torch.Tensor, values: torch.Tensor, q: torch.Tensor, position: int,
+                       attn_scale: float, out_dtype=None) -> torch.Tensor:
+    """One decode step of a packed cache in one library call (tq_packed_decode_step): encode the new token
+    keys / values (B, n_kv, dim) at time index `position`, then attend with q (B, n_kv * n_rep, dim; not
+    pre-rotated) over positions 0 .. position.  Same result as two encode_into calls followed by
+    flash_decode_from_q.  Returns (B, n_q, dim) in out_dtype (default q.dtype)."""
+    _need_gpu(keys, values, q)
+    B, H, T, D = step.shape
+    n_q = H * step.n_rep
+    if tuple(keys.shape) != (B, H, D) or tuple(values.shape) != (B, H, D) or tuple(q.shape) != (B, n_q, D):
+        raise ValueError(f"expected keys / values {(B, H, D)} and q {(B, n_q, D)}, got {tuple(keys.shape)}, "
+                         f"{tuple(values.shape)}, {tuple(q.shape)}")
+    if not 0 <= position < T:
+        raise ValueError(f"position {position} outside the storage of {T} positions")
+    keys, values, q = keys.contiguous(), values.contiguous(), q.contiguous()
+    out = torch.empty((B, n_q, D), dtype=out_dtype or q.dtype, device=q.device)
+    stream = _stream(q)
+    ws = _workspace(q.device, stream.value or 0, step._need)
+    d = step.desc
+    d.workspace, d.workspace_bytes = ws.data_ptr(), ws.numel()
+    _lib.check(_lib.load().tq_packed_decode_step(
+        step._ref, _ptr(keys), _dt(keys), _ptr(values), _dt(values), _ptr(q), _dt(q), _ptr(out), _dt(out),
+        position, attn_scale, stream))
+    return out
+
+
 def prefill_attention(q: torch.Tensor, k_packed, k_norms, v_packed, v_norms, k_centroids, v_centroids,
                       k_signs, v_signs, dim: int, bits: int, attn_scale: float, *, n_rep: int = 1,
                       kv_len: int | None = None, q_pos0: int | None = None, causal: bool = True,
