@@ -292,6 +292,31 @@ int tq_vonly_decode_step(const tq_vonly_cache_desc* cache /* host */,
                          int64_t position, float attn_scale, tq_stream_t stream);
 
 /*
+ * tq_vonly_append with the insert position read from DEVICE memory when the kernel runs: row (g, i)
+ * goes to time index *position_dev + i of group g, the destination pointers point at time index 0
+ * and all four tensors hold t_alloc positions per group; rows that would land outside 0 .. t_alloc - 1
+ * are dropped.  For a decode step recorded once in a HIP graph and replayed while a device counter
+ * advances; the reference's insert position is a host integer (cache.offset, v_only_cache.py:80-82).
+ */
+int tq_vonly_append_at(const void* k_new, int k_dtype, const void* v_new, int v_dtype,
+                       const float* v_signs, const float* boundaries,
+                       void* k_f16, void* v_raw, uint32_t* v_packed, float* v_norms,
+                       int64_t n_groups, int64_t rows_per_group, int64_t t_alloc,
+                       int dim, int bits, int variant, const int64_t* position_dev, tq_stream_t stream);
+
+/*
+ * tq_vonly_decode_step with the position read from device memory: inserts ONE token per sequence at
+ * *position_dev and attends over positions 0 .. *position_dev (clamped to the storage).  Grids and the
+ * workspace are sized for t_alloc positions, so the same recorded launches serve every step until the
+ * storage is reallocated; the caller advances the counter between steps (on the same stream).
+ * dim 128, 3-bit values, n_rep <= 16 only (TQ_ERR_UNSUPPORTED otherwise).
+ */
+int tq_vonly_decode_step_at(const tq_vonly_cache_desc* cache /* host */,
+                            const void* k_new, int k_dtype, const void* v_new, int v_dtype,
+                            const void* q, int q_dtype, void* out, int out_dtype,
+                            const int64_t* position_dev /* device */, float attn_scale, tq_stream_t stream);
+
+/*
  * A cache with packed keys AND values as the library sees it between two growths of its storage
  * (all four tensors share n_seq, n_kv_heads and t_alloc; keys and values share dim and bits, hence
  * the tables, and differ in their sign vectors: seeds s and s + 1 of cache.py:92,96).

@@ -623,3 +623,62 @@ def test_packed_cache_decode_step_is_update_plus_attention(tq, dtype):
     got = c4.decode_step(q1, k1, v1, sc)
     d4.update_and_fetch(k1, v1)
     assert torch.equal(got, tq.turboquant_attention(q1, d4, sc, fused=True)) and c4.offset == d4.offset
+
+
+def test_vonly_decode_step_replayed_from_a_hip_graph(tq):
+    """A decode step recorded ONCE in a HIP graph with the position held in device memory
+    (tq_vonly_decode_step_at) and replayed for ten tokens, with eager work and synchronisations between the
+    replays: every replay matches the eager step on a twin cache and the float64 oracle, and the two caches
+    end in the same state bit for bit.  An insert past the storage is dropped."""
+    B, n_q, n_kv, D, S0, N = 1, 28, 4, 128, 300, 10
+    sc = 1 / math.sqrt(D)
+    k0, v0 = rand((B, n_kv, S0, D), 900), rand((B, n_kv, S0, D), 901)
+    cg, ce = tq.VOnlyTurboQuantCache(bits=3, fused=True), tq.VOnlyTurboQuantCache(bits=3, fused=True)
+    cg.reserve(B, n_kv, 1024, D)
+    cg.update_and_fetch(k0, v0), ce.update_and_fetch(k0, v0)
+    t_alloc = cg._k_cache.keys.shape[2]
+    assert t_alloc == 1024 and cg._v_tq.v_packed.shape[2] == 1024
+    pos = torch.tensor([S0], dtype=torch.int64, device="cuda")
+    qs, ks, vs = rand((B, n_q, 1, D), 902), rand((B, n_kv, 1, D), 903), rand((B, n_kv, 1, D), 904)
+    out_s = torch.empty((B, n_q, D), dtype=torch.float16, device="cuda")
+
+    def check(step_no, q, k, v):
+        want = ce.decode_step(q, k, v, sc)
+        got = out_s.clone()
+        err = (got.float() - want[:, :, 0].float()).abs()
+        assert bool((err <= 1e-3 + 2e-3 * want[:, :, 0].float().abs()).all()), (step_no, float(err.max()))
+        return got
+
+    cg.decode_step(qs, ks, vs, sc, position=pos, out=out_s)          # eager once: workspace, descriptor
+    pos.add_(1)
+    check(-1, qs, ks, vs)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        cg.decode_step(qs, ks, vs, sc, position=pos, out=out_s)
+        pos.add_(1)
+    for i in range(N):
+        q, k, v = rand((B, n_q, 1, D), 910 + 3 * i), rand((B, n_kv, 1, D), 911 + 3 * i), rand((B, n_kv, 1, D), 912 + 3 * i)
+        qs.copy_(q), ks.copy_(k), vs.copy_(v)
+        graph.replay()
+        got = check(i, q, k, v)
+        torch.cuda.synchronize()
+        assert int(pos.item()) == S0 + 2 + i
+    cg.set_offset(S0 + 1 + N)
+    assert cg.offset == ce.offset == S0 + 1 + N
+    for x, y in zip(cg.state, ce.state):
+        assert torch.equal(x, y)
+    st = cg.state
+    vq = cg._v_tq._v_q
+    ref = o.vonly_decode_attention(host(q[0, :, 0]), st[0][0].cpu().numpy(), st[2][0].cpu().numpy().view(np.uint32),
+                                   st[3][0].cpu().numpy(), np.asarray(vq.centroids.cpu()), vq.signs.cpu().numpy(), D, 3, sc)
+    err = np.abs(host(got[0]).astype(np.float64) - ref)
+    assert (err <= 1e-3 + 2e-3 * np.abs(ref)).all(), err.max()
+    # past the storage: nothing is written, the step still runs
+    before = [t.clone() for t in (cg._k_cache.keys, cg._v_tq.v_packed, cg._v_tq.v_norms)]
+    pos.fill_(t_alloc)
+    graph.replay()
+    torch.cuda.synchronize()
+    for x, y in zip(before, (cg._k_cache.keys, cg._v_tq.v_packed, cg._v_tq.v_norms)):
+        assert torch.equal(x, y)
+    assert bool(torch.isfinite(out_s.float()).all())

@@ -721,11 +721,13 @@ int launch_decode(const void* q, int q_dtype, const uint32_t* k_packed, const fl
 // Matrix-core path: tile pass (partials of 512-position tiles) + merge pass.
 int launch_vonly_mfma(const void* q, int q_dtype, const void* k_f16, const uint32_t* v_packed, const float* v_norms,
                       const float* v_centroids, const float* v_signs, void* out, void* workspace,
-                      size_t workspace_bytes, const tq_decode_shape& sh, hipStream_t stream, int phases) {
+                      size_t workspace_bytes, const tq_decode_shape& sh, hipStream_t stream, int phases,
+                      const int64_t* len_dev = nullptr, int64_t len_bias = 0) {
   const char* who = "tq_vonly_decode_attn";
   const int n_q = sh.n_kv_heads * sh.n_rep;
   // no mask, no ragged offsets, 16-byte aligned V rows of every tile: with full tiles on top, the PLAIN variants apply
-  const bool plain_base = !sh.mask && !sh.seq_offsets && sh.attn_scale > 0.0f && tq::aligned(v_packed, 16) &&
+  // (a length read on the device rules them out as well: sh.seq_len is then only its upper bound)
+  const bool plain_base = !sh.mask && !sh.seq_offsets && !len_dev && sh.attn_scale > 0.0f && tq::aligned(v_packed, 16) &&
                           sh.v_seq_stride % 4 == 0 && sh.v_head_stride % 4 == 0;
   const bool plain = plain_base && sh.seq_len % tqm::kTilePos == 0;
   // Long unmasked caches: several consecutive 512-position blocks per workgroup, as many as still leave
@@ -767,6 +769,7 @@ int launch_vonly_mfma(const void* q, int q_dtype, const void* k_f16, const uint3
   const bool q_f32 = q_dtype == TQ_F32;
   a.v_packed = v_packed; a.v_norms = v_norms;
   a.seq_offsets = sh.seq_offsets; a.mask = sh.mask;
+  a.len_dev = len_dev; a.len_bias = len_bias;
   a.ws_S = (float*)workspace;
   a.ws_ml = a.ws_S + (size_t)sh.n_seq * n_q * n_tiles * tqm::kD;
   a.seq_len = sh.seq_len;
@@ -804,7 +807,8 @@ int launch_vonly_mfma(const void* q, int q_dtype, const void* k_f16, const uint3
   const float inv_dim = 1.0f / (float)sh.dim;
 #define LAUNCH_MERGE_U(TO, U_)                                                                            \
   tqm::decode_merge_rows_kernel<TO, true, U_><<<mgrid, tqm::kMergeThreads, 0, stream>>>(                    \
-      a.ws_S, a.ws_ml, sh.seq_offsets, sh.seq_len, n_tiles, sh.n_kv_heads, sh.n_rep, v_signs, inv_dim, (TO*)out, tile_pos)
+      a.ws_S, a.ws_ml, sh.seq_offsets, sh.seq_len, n_tiles, sh.n_kv_heads, sh.n_rep, v_signs, inv_dim, (TO*)out, tile_pos, \
+      len_dev, len_bias)
   // tiles per lane group and round: one round of loads where 64, 128 or 256 tiles cover the sequence
 #define LAUNCH_MERGE_M(TO)                                                                                \
   do {                                                                                                    \
@@ -1311,6 +1315,38 @@ extern "C" int tq_flash_decode_from_q(const void* q, int q_dtype, const float* k
   sh.allow_mma = 1;
   return launch_packed_mfma<tqm::kFlash>(nullptr, k_packed, k_norms, v_packed, v_norms, k_centroids, v_centroids, v_signs,
                                          out, workspace, workspace_bytes, sh, 0.0f, stream, who, q, q_dtype, k_signs);
+}
+
+extern "C" int tq_vonly_decode_step_at(const tq_vonly_cache_desc* c, const void* k_new, int k_dtype, const void* v_new,
+                                       int v_dtype, const void* q, int q_dtype, void* out, int out_dtype,
+                                       const int64_t* position_dev, float attn_scale, tq_stream_t stream_) {
+  const char* who = "tq_vonly_decode_step_at";
+  if (!c || !position_dev) return tq::fail(TQ_ERR_NULL, "%s: null cache descriptor or position_dev", who);
+  if (c->n_seq < 1 || c->n_kv_heads < 1 || c->t_alloc < 1)
+    return tq::fail(TQ_ERR_ARG, "%s: empty cache descriptor (n_seq %d, n_kv_heads %d, t_alloc %lld)", who, c->n_seq,
+                    c->n_kv_heads, (long long)c->t_alloc);
+  if (!c->k_f16 || !c->v_packed || !c->v_norms || !q || !out || !c->v_signs)
+    return tq::fail(TQ_ERR_NULL, "%s: null pointer", who);
+  tq_decode_shape sh{};
+  sh.n_seq = c->n_seq; sh.n_kv_heads = c->n_kv_heads; sh.n_rep = c->n_rep; sh.dim = c->dim; sh.bits = c->bits;
+  sh.block_size = 16;
+  sh.seq_len = c->t_alloc;                                 // upper bound: sizes the grid and the workspace
+  sh.k_head_stride = sh.v_head_stride = sh.vn_head_stride = c->t_alloc;
+  sh.k_seq_stride = sh.v_seq_stride = sh.vn_seq_stride = c->t_alloc * c->n_kv_heads;
+  sh.attn_scale = attn_scale; sh.out_dtype = out_dtype; sh.allow_mma = 1;
+  if (int rc = check_shape(&sh, who, 256)) return rc;
+  if (tq::check_dtype(q_dtype)) return tq::fail(TQ_ERR_DTYPE, "%s: unknown q_dtype %d", who, q_dtype);
+  if (!(mma_shape(sh) && tq::aligned(q, q_dtype == TQ_F32 ? 8 : 4) && tq::aligned(c->k_f16, 16)))
+    return tq::fail(TQ_ERR_UNSUPPORTED, "%s: dim 128, 3-bit values, n_rep <= 16 and aligned q / k only", who);
+  const int n_q = c->n_kv_heads * c->n_rep;
+  if (c->workspace_bytes < tq_workspace_bytes(TQ_OP_VONLY_DECODE, c->n_seq, n_q, c->t_alloc, c->dim))
+    return tq::fail(TQ_ERR_WORKSPACE, "%s: workspace too small for %lld positions", who, (long long)c->t_alloc);
+  if (int rc = tq_vonly_append_at(k_new, k_dtype, v_new, v_dtype, c->v_signs, c->boundaries, c->k_f16, c->v_raw,
+                                  c->v_packed, c->v_norms, (int64_t)c->n_seq * c->n_kv_heads, 1, c->t_alloc, c->dim,
+                                  c->bits, c->variant, position_dev, stream_))
+    return rc;
+  return launch_vonly_mfma(q, q_dtype, c->k_f16, c->v_packed, c->v_norms, c->centroids, c->v_signs, out, c->workspace,
+                           c->workspace_bytes, sh, (hipStream_t)stream_, 3, position_dev, 1);
 }
 
 extern "C" int tq_packed_decode_step(const tq_packed_cache_desc* c, const void* k_new, int k_dtype, const void* v_new,

@@ -25,12 +25,18 @@ struct RowMap {
 // float16 keys beside its packed values): key row `row` of k_src (dtype k_dtype) goes, converted to
 // float16, to k_dst + (g * k_group_stride + r) * D, and the value row itself, unchanged, to
 // v_dst + (g * v_group_stride + r) * D.  Null destinations switch a copy off.
+// With pos_dev set, every destination row index (packed words, norms and the two copies) is
+// shifted by the value pos_dev points to, read on the GPU when the kernel runs: a launch recorded
+// once (HIP graph) then inserts at whatever position the device counter holds.  Rows that would
+// land outside 0 .. pos_cap - 1 are not stored.
 struct RowCopy {
   const void* k_src;
   __half* k_dst;
   void* v_dst;
   int64_t k_group_stride, v_group_stride;
   int k_dtype;
+  const int64_t* pos_dev;
+  int64_t pos_cap;
 };
 
 // ---------------------------------------------------------------- encode
@@ -86,7 +92,13 @@ __global__ __launch_bounds__(kBlock) void encode_kernel(const T* __restrict__ x,
     __syncthreads();
     if (valid) {
       const int64_t g = row / rm.rows_per_group;
-      const int64_t r = row - g * rm.rows_per_group;
+      int64_t r = row - g * rm.rows_per_group;
+      bool store = true;
+      if (rc.pos_dev) {
+        r += *rc.pos_dev;
+        store = r >= 0 && r < rc.pos_cap;
+      }
+      if (store) {
       if (lane < PDIM) {
         uint32_t word = 0;
 #pragma unroll
@@ -117,6 +129,7 @@ __global__ __launch_bounds__(kBlock) void encode_kernel(const T* __restrict__ x,
             else kd[e] = __float2half_rn(__bfloat162float(((const __hip_bfloat16*)rc.k_src)[at]));
           }
         }
+      }
       }
     }
     __syncthreads();
@@ -794,11 +807,13 @@ extern "C" int tq_encode(const void* x, int x_dtype, const float* signs, const f
   return TQ_OK;
 }
 
-extern "C" int tq_vonly_append(const void* k_new, int k_dtype, const void* v_new, int v_dtype,
+namespace {
+int vonly_append(const void* k_new, int k_dtype, const void* v_new, int v_dtype,
                                const float* v_signs, const float* boundaries, void* k_f16, void* v_raw,
                                uint32_t* v_packed, float* v_norms, int64_t n_groups, int64_t rows_per_group,
                                int64_t k_group_stride, int64_t v_raw_group_stride, int64_t packed_group_stride,
-                               int64_t norms_group_stride, int dim, int bits, int variant, tq_stream_t stream_) {
+                               int64_t norms_group_stride, int dim, int bits, int variant, const int64_t* pos_dev,
+                               int64_t pos_cap, tq_stream_t stream_) {
   if (int rc = tq::check_dim_bits(dim, bits)) return rc;
   if (tq::check_dtype(k_dtype) || tq::check_dtype(v_dtype))
     return tq::fail(TQ_ERR_DTYPE, "tq_vonly_append: unknown dtype %d / %d", k_dtype, v_dtype);
@@ -820,7 +835,9 @@ extern "C" int tq_vonly_append(const void* k_new, int k_dtype, const void* v_new
   for (int i = 0; i < nb; ++i)
     thr.t[i] = (variant == TQ_ENCODE_MLX) ? double_rounding_threshold(boundaries[i], s) : boundaries[i];
   RowMap rm{n_rows, rows_per_group, packed_group_stride, norms_group_stride, 0};
-  RowCopy rc{k_new, (__half*)k_f16, v_raw, k_group_stride, v_raw_group_stride, k_dtype};
+  if (pos_dev && (!tq::aligned(pos_dev, 8) || pos_cap < 1))
+    return tq::fail(TQ_ERR_ARG, "tq_vonly_append_at: position_dev must be 8-byte aligned and t_alloc >= 1");
+  RowCopy rc{k_new, (__half*)k_f16, v_raw, k_group_stride, v_raw_group_stride, k_dtype, pos_dev, pos_cap};
   hipStream_t stream = (hipStream_t)stream_;
   const int grid = grid_for_rows(n_rows);
 #define LAUNCH_APP(T)                                                                               \
@@ -832,6 +849,31 @@ extern "C" int tq_vonly_append(const void* k_new, int k_dtype, const void* v_new
 #undef LAUNCH_APP
   TQ_CHECK_LAUNCH("tq_vonly_append launch");
   return TQ_OK;
+}
+}  // namespace
+
+extern "C" int tq_vonly_append(const void* k_new, int k_dtype, const void* v_new, int v_dtype,
+                               const float* v_signs, const float* boundaries, void* k_f16, void* v_raw,
+                               uint32_t* v_packed, float* v_norms, int64_t n_groups, int64_t rows_per_group,
+                               int64_t k_group_stride, int64_t v_raw_group_stride, int64_t packed_group_stride,
+                               int64_t norms_group_stride, int dim, int bits, int variant, tq_stream_t stream_) {
+  return vonly_append(k_new, k_dtype, v_new, v_dtype, v_signs, boundaries, k_f16, v_raw, v_packed, v_norms, n_groups,
+                      rows_per_group, k_group_stride, v_raw_group_stride, packed_group_stride, norms_group_stride, dim,
+                      bits, variant, nullptr, 0, stream_);
+}
+
+extern "C" int tq_vonly_append_at(const void* k_new, int k_dtype, const void* v_new, int v_dtype,
+                                  const float* v_signs, const float* boundaries, void* k_f16, void* v_raw,
+                                  uint32_t* v_packed, float* v_norms, int64_t n_groups, int64_t rows_per_group,
+                                  int64_t t_alloc, int dim, int bits, int variant, const int64_t* position_dev,
+                                  tq_stream_t stream_) {
+  if (!position_dev) return tq::fail(TQ_ERR_NULL, "tq_vonly_append_at: null position_dev");
+  if (rows_per_group > t_alloc)
+    return tq::fail(TQ_ERR_ARG, "tq_vonly_append_at: %lld new rows per group do not fit %lld positions",
+                    (long long)rows_per_group, (long long)t_alloc);
+  return vonly_append(k_new, k_dtype, v_new, v_dtype, v_signs, boundaries, k_f16, v_raw, v_packed, v_norms, n_groups,
+                      rows_per_group, t_alloc, t_alloc, t_alloc, t_alloc, dim, bits, variant, position_dev, t_alloc,
+                      stream_);
 }
 
 extern "C" int tq_dequant(const uint32_t* packed, const float* norms, const float* centroids,

@@ -61,6 +61,8 @@ struct MfmaArgs {
   const uint32_t* v_packed;
   const float* v_norms;
   const int32_t* seq_offsets;
+  const int64_t* len_dev;     // optional (tile + merge pass of the V-only step, no seq_offsets): every sequence attends
+  int64_t len_bias;           // min(max(*len_dev + len_bias, 0), seq_len) positions, read when the kernel runs
   const float* mask;
   float* ws_S;                // [n_seq * n_kv, n_tiles_max, n_rep, 128]
   float* ws_ml;               // [n_seq * n_kv, n_tiles_max, n_rep, 2]
@@ -158,6 +160,9 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
   if (!PLAIN && a.seq_offsets) {
     first = a.seq_offsets[seq];
     len = (int64_t)a.seq_offsets[seq + 1] - first;
+  } else if (!PLAIN && a.len_dev) {
+    const int64_t want = *a.len_dev + a.len_bias;
+    len = want < 0 ? 0 : (want < len ? want : len);
   }
   const int64_t tile_p0 = (int64_t)tile * kTPos;
   TQ_STAMP(0);
@@ -1013,7 +1018,7 @@ template <typename TO, bool NORM, int U = 8>
 __global__ __launch_bounds__(kMergeThreads) void decode_merge_rows_kernel(
     const float* __restrict__ ws_S, const float* __restrict__ ws_ml, const int32_t* __restrict__ seq_offsets,
     int64_t seq_len, int n_tiles_max, int n_kv, int n_rep, const float* __restrict__ signs, float inv_dim,
-    TO* __restrict__ out, int tile_pos) {
+    TO* __restrict__ out, int tile_pos, const int64_t* __restrict__ len_dev = nullptr, int64_t len_bias = 0) {
   __shared__ __align__(16) float acc_s[8][kD];
   __shared__ float ml_s[8][2];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -1021,7 +1026,12 @@ __global__ __launch_bounds__(kMergeThreads) void decode_merge_rows_kernel(
   const int head = blockIdx.x, seq = blockIdx.y;
   const int kvh = head / n_rep, r = head - kvh * n_rep;
   int64_t len = seq_len;
-  if (seq_offsets) len = (int64_t)seq_offsets[seq + 1] - seq_offsets[seq];
+  if (seq_offsets) {
+    len = (int64_t)seq_offsets[seq + 1] - seq_offsets[seq];
+  } else if (len_dev) {                                  // as the tile pass reads it
+    const int64_t want = *len_dev + len_bias;
+    len = want < 0 ? 0 : (want < len ? want : len);
+  }
   const int n_tiles = (int)((len + tile_pos - 1) / tile_pos);
   const int64_t grp = (int64_t)seq * n_kv + kvh;
   const float* gS = ws_S + grp * n_tiles_max * (int64_t)(n_rep * kD) + r * kD + 4 * eq;

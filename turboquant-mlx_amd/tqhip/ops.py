@@ -747,13 +747,18 @@ class VOnlyStep:
         self._need = _lib.load().tq_workspace_bytes(_lib.TQ_OP_VONLY_DECODE, B, H * n_rep, T, D)
 
 
-def vonly_decode_step(step: VOnlyStep, keys: torch.Tensor, values: torch.Tensor, q: torch.Tensor, position: int,
-                      attn_scale: float, out_dtype=None) -> torch.Tensor:
+def vonly_decode_step(step: VOnlyStep, keys: torch.Tensor, values: torch.Tensor, q: torch.Tensor, position,
+                      attn_scale: float, out_dtype=None, out: torch.Tensor | None = None) -> torch.Tensor:
     """One decode step of a V-only cache in one library call (tq_vonly_decode_step): insert the new token
     keys / values (B, n_kv, dim) at time index `position`, then attend with q (B, n_kv * n_rep, dim) over
     positions 0 .. position.  Same result as vonly_append_into followed by vonly_decode.  Returns
-    (B, n_q, dim) in out_dtype (default q.dtype)."""
-    _need_gpu(keys, values, q)
+    (B, n_q, dim) in out_dtype (default q.dtype), written into `out` when one is given.
+
+    `position` may be a one-element int64 tensor on the GPU (tq_vonly_decode_step_at): the kernels then read
+    the position when they run, so the launches can be recorded once in a HIP graph and replayed while the
+    caller advances the counter (`position.add_(1)` on the same stream, after the step); the grids cover the
+    whole storage, which costs a few idle workgroups, and an insert past the storage is dropped."""
+    _need_gpu(keys, values, q, out)
     B, H, T, D = step.shape
     n_q = H * step.n_rep
     if tuple(keys.shape) != (B, H, D) or tuple(values.shape) != (B, H, D) or tuple(q.shape) != (B, n_q, D):
@@ -761,17 +766,30 @@ def vonly_decode_step(step: VOnlyStep, keys: torch.Tensor, values: torch.Tensor,
                          f"{tuple(values.shape)}, {tuple(q.shape)}")
     if step.v_dtype is not None and values.dtype != step.v_dtype:
         raise ValueError(f"values are {values.dtype}, the cache keeps {step.v_dtype}")
-    if not 0 <= position < T:
+    on_device = isinstance(position, torch.Tensor)
+    if on_device:
+        if position.dtype != torch.int64 or position.numel() != 1 or not position.is_cuda:
+            raise ValueError("a device-side position must be a one-element int64 tensor on the GPU")
+    elif not 0 <= position < T:
         raise ValueError(f"position {position} outside the storage of {T} positions")
     keys, values, q = keys.contiguous(), values.contiguous(), q.contiguous()
-    out = torch.empty((B, n_q, D), dtype=out_dtype or q.dtype, device=q.device)
+    if out is None:
+        out = torch.empty((B, n_q, D), dtype=out_dtype or q.dtype, device=q.device)
+    elif tuple(out.shape) != (B, n_q, D) or not out.is_contiguous():
+        raise ValueError(f"out must be a contiguous {(B, n_q, D)} tensor")
     stream = _stream(q)
     ws = _workspace(q.device, stream.value or 0, step._need)
     d = step.desc
     d.workspace, d.workspace_bytes = ws.data_ptr(), ws.numel()
-    _lib.check(_lib.load().tq_vonly_decode_step(
-        step._ref, _ptr(keys), _dt(keys), _ptr(values), _dt(values), _ptr(q), _dt(q), _ptr(out), _dt(out),
-        position, attn_scale, stream))
+    lib = _lib.load()
+    if on_device:
+        _lib.check(lib.tq_vonly_decode_step_at(
+            step._ref, _ptr(keys), _dt(keys), _ptr(values), _dt(values), _ptr(q), _dt(q), _ptr(out), _dt(out),
+            _ptr(position), attn_scale, stream))
+    else:
+        _lib.check(lib.tq_vonly_decode_step(
+            step._ref, _ptr(keys), _dt(keys), _ptr(values), _dt(values), _ptr(q), _dt(q), _ptr(out), _dt(out),
+            position, attn_scale, stream))
     return out
 
 

@@ -64,12 +64,40 @@ class VOnlyTurboQuantCache:
         tq.offset += S
         return True
 
-    def decode_step(self, queries: torch.Tensor, keys: torch.Tensor, values: torch.Tensor, attn_scale: float):
+    def reserve(self, B: int, H: int, n_positions: int, dim: int, dtype=torch.float16, device="cuda"):
+        """Allocate storage for `n_positions` more positions now, so that steps recorded in a HIP graph keep
+        their addresses for that long (storage otherwise grows in steps of 256, which reallocates)."""
+        kc, tq = self._k_cache, self._v_tq
+        device = torch.device(device)
+        tq._ensure_quantizer(dim, dim, device)
+        need = kc.offset + n_positions
+        have = 0 if kc.keys is None else kc.keys.shape[2]
+        if need > have:
+            kc.reserve(B, H, need - kc.offset, dim, dim, torch.float16, dtype, device)
+        if tq.v_packed is None or need > tq.v_packed.shape[2]:
+            tq._ensure_storage(B, H, need - tq.offset, device)
+
+    def set_offset(self, n: int):
+        """Set the number of valid positions (keys and values alike): for a caller that replayed recorded steps
+        with a device-side position and now tells the host-side bookkeeping how far the cache has got."""
+        if not 0 <= n <= (0 if self._k_cache.keys is None else self._k_cache.keys.shape[2]):
+            raise ValueError(f"offset {n} outside the storage")
+        self._k_cache.offset = n
+        self._v_tq.offset = n
+
+    def decode_step(self, queries: torch.Tensor, keys: torch.Tensor, values: torch.Tensor, attn_scale: float,
+                    position: torch.Tensor | None = None, out: torch.Tensor | None = None):
         """Insert one token and attend in one library call: the result of `update_and_fetch(keys, values)`
         followed by `vonly_decode_attention(queries, self, attn_scale)` (no mask, no sparse-V threshold).
         queries (B, n_heads, 1, dim), keys / values (B, n_kv, 1, dim) -> (B, n_heads, 1, dim) in queries.dtype.
         Not in the reference, where the two halves are separate calls of the model's attention layer
-        (v_only_cache.py:52-78, then SDPA)."""
+        (v_only_cache.py:52-78, then SDPA).
+
+        With `position` (one-element int64 GPU tensor holding the cache's current offset) the kernels read the
+        insert position and the attended length from it when they run: the step can be recorded in a HIP graph
+        once and replayed, the caller advancing the tensor by one after every step and calling `set_offset`
+        when it is done replaying; `reserve` keeps the storage from moving meanwhile.  `out` (B, n_heads, dim)
+        receives the result when given."""
         from . import attention, ops
         kc, tq = self._k_cache, self._v_tq
         B, n_q, S_q, dim = queries.shape
@@ -78,6 +106,9 @@ class VOnlyTurboQuantCache:
                 or queries.dtype not in (torch.float16, torch.bfloat16, torch.float32)
                 or (kc.values is not None and kc.values.dtype != values.dtype)
                 or (kc.keys is not None and kc.keys.dtype != torch.float16) or kc.offset != tq.offset):
+            if position is not None:
+                raise ValueError("a step with a device-side position needs one new token, float16/bfloat16/float32 "
+                                 "queries and a cache whose stored values have the dtype of the new ones")
             self.update_and_fetch(keys, values)
             return attention.vonly_decode_attention(queries, self, attn_scale)
         kc.reserve(B, H, 1, dim, dim, torch.float16, values.dtype, values.device)
@@ -92,11 +123,13 @@ class VOnlyTurboQuantCache:
                                            tq._v_q.boundaries, tq._v_q.centroids, n_rep=n_q // H,
                                            bits=tq.quant_bits, variant=tq.encode_variant)
             except ValueError:                     # storage handed in through `state` as slices
+                if position is not None:
+                    raise
                 self.update_and_fetch(keys, values)
                 return attention.vonly_decode_attention(queries, self, attn_scale)
             self._step_key = key
         out = ops.vonly_decode_step(self._step, keys[:, :, 0, :], values[:, :, 0, :], queries[:, :, 0, :],
-                                    kc.offset, attn_scale)
+                                    kc.offset if position is None else position, attn_scale, out=out)
         kc.offset += 1
         tq.offset += 1
         return out[:, :, None, :]
