@@ -6,7 +6,7 @@ back-to-back launches, and rotation over several independent input sets so that 
 Infinity Cache cannot serve the reads.  Prints one line per case: us per call, GB/s of algorithmic
 bytes and the fraction of 8 TB/s.
 
-    python -m tqhip.bench_kernels [--iters 200] [--cases encode,scores,flash,flash_long,sparse_v,vonly,prefill]
+    python -m tqhip.bench_kernels [--iters 200] [--cases encode,scores,flash,flash_long,sparse_v,vonly,prefill,step]
 """
 from __future__ import annotations
 
@@ -187,7 +187,74 @@ def bench_prefill(iters, dev):
               flush=True)
 
 
-CASES = {"prefill": bench_prefill, "encode": bench_encode, "scores": bench_scores, "sparse_v": bench_sparse_v, "flash": bench_flash,
+def bench_step(iters, dev):
+    """Wall time of a whole layer step (insert one token + attention) through the cache objects: the two calls
+    of the reference's surface, the single library call, and 28 layers recorded in a HIP graph with the position
+    in device memory.  Wall clock (perf_counter around a synchronised loop): host cost is the point."""
+    import time
+    D, L = 128, 28
+    sc = 1 / math.sqrt(D)
+
+    def wall(fn, n):
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n * 1e6
+
+    n = max(20, iters // 2)
+    for T in (4096, 30720):
+        for kind, n_q, n_kv in (("V-only cache", 28, 4), ("packed cache", 32, 8)):
+            mk = (lambda: tqhip.VOnlyTurboQuantCache(bits=3, fused=True)) if kind == "V-only cache" else \
+                 (lambda: tqhip.TurboQuantKVCache(bits=3, fused=True))
+            k0 = torch.randn((1, n_kv, T, D), device=dev, dtype=torch.float16)
+            v0 = torch.randn((1, n_kv, T, D), device=dev, dtype=torch.float16)
+            k1, v1 = torch.randn((1, n_kv, 1, D), device=dev, dtype=torch.float16), torch.randn((1, n_kv, 1, D), device=dev, dtype=torch.float16)
+            q = torch.randn((1, n_q, 1, D), device=dev, dtype=torch.float16)
+            c = mk()
+            c.update_and_fetch(k0, v0)
+            attend = tqhip.vonly_decode_attention if kind == "V-only cache" else \
+                (lambda qq, cc, s: tqhip.turboquant_attention(qq, cc, s, fused=True))
+
+            def two_calls():
+                c.update_and_fetch(k1, v1)
+                return attend(q, c, sc)
+            us2 = wall(two_calls, n)
+            c = mk()
+            c.update_and_fetch(k0, v0)
+            us1 = wall(lambda: c.decode_step(q, k1, v1, sc), n)
+            print(f"layer step, {kind}, {n_q}/{n_kv} heads, T~{T}: update_and_fetch + attention {us2:6.1f} us wall, "
+                  f"decode_step {us1:6.1f} us wall", flush=True)
+            del c
+        caches = [tqhip.VOnlyTurboQuantCache(bits=3, fused=True) for _ in range(L)]
+        k0 = torch.randn((1, 4, T, D), device=dev, dtype=torch.float16)
+        for c in caches:
+            c.reserve(1, 4, T + 2048, D)
+            c.update_and_fetch(k0, k0)
+        k1 = torch.randn((1, 4, 1, D), device=dev, dtype=torch.float16)
+        q = torch.randn((1, 28, 1, D), device=dev, dtype=torch.float16)
+        outs = [torch.empty((1, 28, D), device=dev, dtype=torch.float16) for _ in range(L)]
+        pos = torch.tensor([T], dtype=torch.int64, device=dev)
+
+        def token():
+            for i, c in enumerate(caches):
+                c.decode_step(q, k1, k1, sc, position=pos, out=outs[i])
+            pos.add_(1)
+        token()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            token()
+        us = wall(g.replay, n) / L
+        print(f"layer step, V-only cache, 28/4 heads, T~{T}: {L} layers recorded in a HIP graph, position in device "
+              f"memory: {us:6.1f} us per layer step", flush=True)
+        del g, caches
+
+
+CASES = {"step": bench_step, "prefill": bench_prefill, "encode": bench_encode, "scores": bench_scores, "sparse_v": bench_sparse_v, "flash": bench_flash,
          "flash_long": bench_flash_long, "vonly": bench_vonly}
 
 
