@@ -278,9 +278,13 @@ typedef struct tq_vonly_cache_desc {
 } tq_vonly_cache_desc;
 
 /*
- * One decode step of a V-only cache in one library call: tq_vonly_append of ONE new token per
- * sequence at time index `position`, then tq_vonly_decode_attn of the query token over positions
- * 0 .. position (both on `stream`, three launches, results identical to the two calls).
+ * One decode step of a V-only cache in one library call: ONE new token per sequence is inserted at
+ * time index `position` and the query token attends over positions 0 .. position.  For dim 128,
+ * 3-bit values and n_rep <= 16 that is two launches: the tile pass over positions 0 .. position - 1,
+ * and a merge pass that encodes the new value row with the encoder's own arithmetic, scores the new
+ * key, folds both in and stores the key row, the raw value row, the packed words and the norm (the
+ * stored state is bit-identical to tq_vonly_append's, the output agrees with the two calls to the
+ * rounding of one score); other shapes run tq_vonly_append followed by tq_vonly_decode_attn.
  * Replaces, for a single-token step, VOnlyTurboQuantCache.update_and_fetch followed by the
  * attention of hybrid_attention.py:52-88 / fused_attention.py:50-121 (v_only_cache.py:52-78).
  *   k_new, v_new [n_seq, n_kv_heads, dim];  q [n_seq, n_kv_heads*n_rep, dim];  out likewise, out_dtype

@@ -722,7 +722,7 @@ int launch_decode(const void* q, int q_dtype, const uint32_t* k_packed, const fl
 int launch_vonly_mfma(const void* q, int q_dtype, const void* k_f16, const uint32_t* v_packed, const float* v_norms,
                       const float* v_centroids, const float* v_signs, void* out, void* workspace,
                       size_t workspace_bytes, const tq_decode_shape& sh, hipStream_t stream, int phases,
-                      const int64_t* len_dev = nullptr, int64_t len_bias = 0) {
+                      const int64_t* len_dev = nullptr, int64_t len_bias = 0, const tqm::FreshToken* fresh = nullptr) {
   const char* who = "tq_vonly_decode_attn";
   const int n_q = sh.n_kv_heads * sh.n_rep;
   // no mask, no ragged offsets, 16-byte aligned V rows of every tile: with full tiles on top, the PLAIN variants apply
@@ -759,7 +759,8 @@ int launch_vonly_mfma(const void* q, int q_dtype, const void* k_f16, const uint3
   int nw = 8;
   if (n_blocks == 1 && (wgs8 <= 128 || (wgs8 > 256 && wgs4 <= 768))) nw = 4;
   const int tile_pos = nw * tqm::kWavePos * n_blocks;
-  const int n_tiles = (int)((sh.seq_len + tile_pos - 1) / tile_pos);
+  const int n_tiles_real = (int)((sh.seq_len + tile_pos - 1) / tile_pos);     // 0: an empty cache, merge pass only
+  const int n_tiles = n_tiles_real > 0 ? n_tiles_real : 1;
   const size_t need = (size_t)sh.n_seq * n_q * n_tiles * (tqm::kD + 2) * sizeof(float);
   if (!workspace || workspace_bytes < need)
     return tq::fail(TQ_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, need, workspace_bytes);
@@ -788,7 +789,7 @@ int launch_vonly_mfma(const void* q, int q_dtype, const void* k_f16, const uint3
 #endif
   Codebook vcb;
   a.v_unscale = tq::fill_codebook_fp16(vcb, v_centroids, sh.bits);
-  if (phases & 1) {
+  if ((phases & 1) && n_tiles_real > 0) {
     dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
     const bool plain4 = plain_base && sh.seq_len % 256 == 0;           // full 256-position tiles
 #define LAUNCH_TILE(QF)                                                                                          \
@@ -816,9 +817,24 @@ int launch_vonly_mfma(const void* q, int q_dtype, const void* k_f16, const uint3
     else if (n_tiles <= 128) LAUNCH_MERGE_U(TO, 16);                                                      \
     else LAUNCH_MERGE_U(TO, 32);                                                                          \
   } while (0)
-  if (sh.out_dtype == TQ_F16) { LAUNCH_MERGE_M(__half); }
+#define LAUNCH_FRESH_U(TO, U_)                                                                            \
+  tqm::decode_merge_fresh_kernel<TO, U_><<<mgrid, tqm::kMergeThreads + 64, 0, stream>>>(                    \
+      a.ws_S, a.ws_ml, sh.seq_len, n_tiles, sh.n_kv_heads, sh.n_rep, v_signs, inv_dim, (TO*)out, tile_pos, len_dev, *fresh)
+#define LAUNCH_FRESH_M(TO)                                                                                \
+  do {                                                                                                    \
+    if (n_tiles <= 64) LAUNCH_FRESH_U(TO, 8);                                                             \
+    else if (n_tiles <= 128) LAUNCH_FRESH_U(TO, 16);                                                      \
+    else LAUNCH_FRESH_U(TO, 32);                                                                          \
+  } while (0)
+  if (fresh) {
+    if (sh.out_dtype == TQ_F16) { LAUNCH_FRESH_M(__half); }
+    else if (sh.out_dtype == TQ_BF16) { LAUNCH_FRESH_M(__hip_bfloat16); }
+    else { LAUNCH_FRESH_M(float); }
+  } else if (sh.out_dtype == TQ_F16) { LAUNCH_MERGE_M(__half); }
   else if (sh.out_dtype == TQ_BF16) { LAUNCH_MERGE_M(__hip_bfloat16); }
   else { LAUNCH_MERGE_M(float); }
+#undef LAUNCH_FRESH_M
+#undef LAUNCH_FRESH_U
 #undef LAUNCH_MERGE_M
 #undef LAUNCH_MERGE_U
   TQ_CHECK_LAUNCH(who);
@@ -1216,6 +1232,47 @@ extern "C" int tq_vonly_decode_attn(const void* q, int q_dtype, const void* k_f1
                                      workspace_bytes, shape, 3, stream_);
 }
 
+namespace {
+constexpr int kNotFused = 1;   // not an error: the caller takes the append + attention route
+
+// A decode step as two launches: the tile pass over the positions before the new one, and a merge pass that
+// encodes and stores the new token itself (tqm::FreshToken).  dim 128, 3-bit values, n_rep <= 16.
+int vonly_step_fused(const tq_vonly_cache_desc* c, const void* k_new, int k_dtype, const void* v_new, int v_dtype,
+                     const void* q, int q_dtype, void* out, int out_dtype, int64_t position, const int64_t* position_dev,
+                     float attn_scale, tq_stream_t stream_, const char* who) {
+  if (!(c->dim == 128 && c->bits == 3 && c->n_rep >= 1 && c->n_rep <= tqm::kHeadsMax && c->allow_mma &&
+        tq::aligned(q, q_dtype == TQ_F32 ? 8 : 4) && tq::aligned(c->k_f16, 16)))
+    return kNotFused;
+  if (tq::check_dtype(k_dtype) || tq::check_dtype(v_dtype) || tq::check_dtype(q_dtype) || tq::check_dtype(out_dtype))
+    return tq::fail(TQ_ERR_DTYPE, "%s: unknown dtype", who);
+  if (c->variant != TQ_ENCODE_MLX && c->variant != TQ_ENCODE_METAL)
+    return tq::fail(TQ_ERR_ARG, "%s: unknown variant %d", who, c->variant);
+  if (!k_new || !v_new || !q || !out || !c->v_signs) return tq::fail(TQ_ERR_NULL, "%s: null pointer", who);
+  if (!tq::aligned(k_new, tq::dtype_size(k_dtype)) || !tq::aligned(v_new, tq::dtype_size(v_dtype)) ||
+      !tq::aligned(c->v_packed, 4) || !tq::aligned(c->v_norms, 4) || !tq::aligned(c->v_signs, 4) ||
+      (c->v_raw && !tq::aligned(c->v_raw, tq::dtype_size(v_dtype))))
+    return tq::fail(TQ_ERR_ALIGN, "%s: misaligned pointer", who);
+  if (c->n_seq > 65535) return tq::fail(TQ_ERR_ARG, "%s: at most 65535 sequences per call", who);
+  tqm::FreshToken f{};
+  f.k_new = k_new; f.v_new = v_new; f.q = q;
+  f.k_f16 = (__half*)c->k_f16; f.v_raw = c->v_raw; f.v_packed = c->v_packed; f.v_norms = c->v_norms;
+  f.pos_dev = position_dev; f.pos = position; f.t_alloc = c->t_alloc;
+  tq::encode_thresholds(c->boundaries, c->dim, c->bits, c->variant, f.thr);
+  for (int i = 0; i < 8; ++i) f.cent[i] = c->centroids[i];
+  f.cs = attn_scale * tqm::kLog2e;
+  f.k_dtype = k_dtype; f.v_dtype = v_dtype; f.q_dtype = q_dtype;
+  tq_decode_shape sh{};
+  sh.n_seq = c->n_seq; sh.n_kv_heads = c->n_kv_heads; sh.n_rep = c->n_rep; sh.dim = c->dim; sh.bits = c->bits;
+  sh.block_size = 16;
+  sh.seq_len = position_dev ? c->t_alloc : position;        // positions before the new one (device: upper bound)
+  sh.k_head_stride = sh.v_head_stride = sh.vn_head_stride = c->t_alloc;
+  sh.k_seq_stride = sh.v_seq_stride = sh.vn_seq_stride = c->t_alloc * c->n_kv_heads;
+  sh.attn_scale = attn_scale; sh.out_dtype = out_dtype; sh.allow_mma = 1;
+  return launch_vonly_mfma(q, q_dtype, c->k_f16, c->v_packed, c->v_norms, c->centroids, c->v_signs, out, c->workspace,
+                           c->workspace_bytes, sh, (hipStream_t)stream_, 3, position_dev, 0, &f);
+}
+}  // namespace
+
 extern "C" int tq_vonly_decode_step(const tq_vonly_cache_desc* c, const void* k_new, int k_dtype, const void* v_new,
                                     int v_dtype, const void* q, int q_dtype, void* out, int out_dtype,
                                     int64_t position, float attn_scale, tq_stream_t stream_) {
@@ -1229,6 +1286,9 @@ extern "C" int tq_vonly_decode_step(const tq_vonly_cache_desc* c, const void* k_
     return tq::fail(TQ_ERR_ARG, "%s: position %lld outside the storage of %lld positions", who, (long long)position,
                     (long long)c->t_alloc);
   if (!c->k_f16 || !c->v_packed || !c->v_norms) return tq::fail(TQ_ERR_NULL, "%s: null pointer", who);
+  if (int rc = vonly_step_fused(c, k_new, k_dtype, v_new, v_dtype, q, q_dtype, out, out_dtype, position, nullptr,
+                                attn_scale, stream_, who); rc != kNotFused)
+    return rc;
   const int pdim = tq::packed_dim(c->dim, c->bits);
   const int64_t groups = (int64_t)c->n_seq * c->n_kv_heads;
   if (int rc = tq_vonly_append(
@@ -1341,12 +1401,11 @@ extern "C" int tq_vonly_decode_step_at(const tq_vonly_cache_desc* c, const void*
   const int n_q = c->n_kv_heads * c->n_rep;
   if (c->workspace_bytes < tq_workspace_bytes(TQ_OP_VONLY_DECODE, c->n_seq, n_q, c->t_alloc, c->dim))
     return tq::fail(TQ_ERR_WORKSPACE, "%s: workspace too small for %lld positions", who, (long long)c->t_alloc);
-  if (int rc = tq_vonly_append_at(k_new, k_dtype, v_new, v_dtype, c->v_signs, c->boundaries, c->k_f16, c->v_raw,
-                                  c->v_packed, c->v_norms, (int64_t)c->n_seq * c->n_kv_heads, 1, c->t_alloc, c->dim,
-                                  c->bits, c->variant, position_dev, stream_))
+  if (!tq::aligned(position_dev, 8)) return tq::fail(TQ_ERR_ALIGN, "%s: position_dev must be 8-byte aligned", who);
+  if (int rc = vonly_step_fused(c, k_new, k_dtype, v_new, v_dtype, q, q_dtype, out, out_dtype, 0, position_dev,
+                                attn_scale, stream_, who); rc != kNotFused)
     return rc;
-  return launch_vonly_mfma(q, q_dtype, c->k_f16, c->v_packed, c->v_norms, c->centroids, c->v_signs, out, c->workspace,
-                           c->workspace_bytes, sh, (hipStream_t)stream_, 3, position_dev, 1);
+  return tq::fail(TQ_ERR_UNSUPPORTED, "%s: shape not covered", who);
 }
 
 extern "C" int tq_packed_decode_step(const tq_packed_cache_desc* c, const void* k_new, int k_dtype, const void* v_new,

@@ -733,6 +733,15 @@ int grid_for_rows(int64_t rows) {
 
 }  // namespace
 
+namespace tq {
+void encode_thresholds(const float* boundaries, int dim, int bits, int variant, float* thr_out) {
+  const float s = (float)(1.0 / sqrt((double)dim));
+  const int nb = (1 << bits) - 1;
+  for (int i = 0; i < nb; ++i)
+    thr_out[i] = (variant == TQ_ENCODE_MLX) ? double_rounding_threshold(boundaries[i], s) : boundaries[i];
+}
+}  // namespace tq
+
 // ------------------------------------------------------------------ C ABI
 
 extern "C" int tq_version(void) { return TQ_VERSION; }

@@ -54,6 +54,11 @@ inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_
 
 inline int check_dtype(int dt) { return (dt == TQ_F32 || dt == TQ_F16 || dt == TQ_BF16) ? 0 : 1; }
 
+// Decision thresholds of the encoder in the domain of the raw butterfly output for `nb` = 2^bits - 1
+// boundaries (defined beside the encoder): TQ_ENCODE_MLX reproduces the comparison of
+// fl(fl(w * s) / s) with the boundary, TQ_ENCODE_METAL compares w itself.
+void encode_thresholds(const float* boundaries, int dim, int bits, int variant, float* thr_out);
+
 inline size_t dtype_size(int dt) { return dt == TQ_F32 ? 4 : 2; }
 
 inline int check_dim_bits(int dim, int bits) {

@@ -1009,18 +1009,47 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
   }
 }
 
-// Merge pass: grid = (n_q, n_seq), 256 threads.  Lane group ph = tid / 32 folds tiles ph, ph + 8, ...
+// The token a decode step inserts, handled by the merge pass instead of a launch of its own ahead of the
+// tile pass: an extra wavefront of every merge workgroup encodes the new value row (the arithmetic of the
+// encoder, operation for operation: tree-ordered sum of squares, division by max(norm, 1e-8), signs, raw
+// butterfly, strict threshold count), takes q . k of its head against the float16-rounded new key, and hands
+// (score, 1, norm * c[idx]) to the fold as one more partial; the workgroup of the first query head of a kv
+// head also stores the key row, the raw value row, the packed words and the norm.  The tile pass then covers
+// the positions before the new one only.
+struct FreshToken {
+  const void* k_new;          // [n_seq, n_kv, 128], dtype k_dtype
+  const void* v_new;          // [n_seq, n_kv, 128], dtype v_dtype
+  const void* q;              // [n_seq, n_q, 128], dtype q_dtype
+  __half* k_f16;              // storage, time index 0 of group 0; t_alloc positions per (sequence, kv head)
+  void* v_raw;                // may be null
+  uint32_t* v_packed;
+  float* v_norms;
+  const int64_t* pos_dev;     // insert position in device memory, or null: `pos`
+  int64_t pos, t_alloc;
+  float thr[7];               // decision thresholds in the domain of the raw butterfly output
+  float cent[8];
+  float cs;                   // attn_scale * log2 e
+  int32_t k_dtype, v_dtype, q_dtype;
+};
+
+__device__ __forceinline__ float load_any(const void* p, int dtype, int64_t at) {
+  if (dtype == TQ_F16) return __half2float(((const __half*)p)[at]);
+  if (dtype == TQ_F32) return ((const float*)p)[at];
+  return __bfloat162float(((const __hip_bfloat16*)p)[at]);
+}
+
+// Merge pass: grid = (n_q, n_seq), 256 threads (320 with FRESH).  Lane group ph = tid / 32 folds tiles ph, ph + 8, ...
 // (4 elements per lane) with a running maximum, U tiles per round with all loads of a round issued together (a
 // round costs one memory round trip, so the host picks U to cover the tiles in one round where it can: 8, 16
 // or 32); the 8 groups are then combined through LDS and wave 0 finishes the row.  NORM = false (given weights,
 // all maxima zero) skips the division by l.
-template <typename TO, bool NORM, int U = 8>
-__global__ __launch_bounds__(kMergeThreads) void decode_merge_rows_kernel(
+template <typename TO, bool NORM, int U, bool FRESH>
+__device__ __forceinline__ void merge_rows_body(
     const float* __restrict__ ws_S, const float* __restrict__ ws_ml, const int32_t* __restrict__ seq_offsets,
     int64_t seq_len, int n_tiles_max, int n_kv, int n_rep, const float* __restrict__ signs, float inv_dim,
-    TO* __restrict__ out, int tile_pos, const int64_t* __restrict__ len_dev = nullptr, int64_t len_bias = 0) {
-  __shared__ __align__(16) float acc_s[8][kD];
-  __shared__ float ml_s[8][2];
+    TO* __restrict__ out, int tile_pos, const int64_t* __restrict__ len_dev, int64_t len_bias, const FreshToken* ft) {
+  __shared__ __align__(16) float acc_s[FRESH ? 9 : 8][kD];
+  __shared__ float ml_s[FRESH ? 9 : 8][2];
   const int tid = threadIdx.x, lane = tid & 63;
   const int eq = tid & 31, ph = tid >> 5;
   const int head = blockIdx.x, seq = blockIdx.y;
@@ -1038,6 +1067,73 @@ __global__ __launch_bounds__(kMergeThreads) void decode_merge_rows_kernel(
   const float* gml = ws_ml + grp * n_tiles_max * (int64_t)(n_rep * 2) + r * 2;
   // issued first: the signs are only needed at the very end, their latency hides behind everything else
   const float sign0 = signs[lane], sign1 = signs[lane + 64];
+  bool fresh_wave = false;
+  if constexpr (FRESH) fresh_wave = tid >= 256;
+  if constexpr (FRESH) { if (fresh_wave) {
+    // ---- the inserted token (one wavefront) ------------------------------------------------------------
+    const FreshToken& f = *ft;
+    const int64_t pos = f.pos_dev ? *f.pos_dev : f.pos;
+    const bool ok = pos >= 0 && pos < f.t_alloc;
+    const int64_t src = grp * kD;
+    float x[2], kx[2], qx[2], sq[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int e = lane + 64 * i;
+      x[i] = load_any(f.v_new, f.v_dtype, src + e);
+      kx[i] = __half2float(__float2half_rn(load_any(f.k_new, f.k_dtype, src + e)));
+      qx[i] = load_any(f.q, f.q_dtype, ((int64_t)seq * gridDim.x + head) * kD + e);
+      sq[i] = x[i] * x[i];
+    }
+    const float ss = tree_sum<kD>(sq);
+    const float nrm = sqrtf(ss);
+    const float safe = fmaxf(nrm, 1e-8f);
+    float v[2] = {(x[0] / safe) * sign0, (x[1] / safe) * sign1};
+    raw_butterfly<kD>(v, lane);
+    int idx[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      uint32_t n = 0;
+#pragma unroll
+      for (int b = 0; b < 7; ++b) n += (v[i] > f.thr[b]) ? 1u : 0u;
+      idx[i] = (int)n;
+      float c = f.cent[0];                               // selects, not a dynamic index into kernel arguments
+#pragma unroll
+      for (int k = 1; k < 8; ++k) c = (n == (uint32_t)k) ? f.cent[k] : c;
+      acc_s[8][lane + 64 * i] = nrm * c;
+    }
+    float d = qx[0] * kx[0] + qx[1] * kx[1];
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) d += shfl_xor_f(d, m);
+    if (lane == 0) {
+      ml_s[8][0] = ok ? d * f.cs : -INFINITY;
+      ml_s[8][1] = 1.0f;
+    }
+    // packed word `lane` holds elements 10 * lane .. 10 * lane + 9 (3-bit fields, lowest first)
+    uint32_t word = 0;
+#pragma unroll
+    for (int i = 0; i < 10; ++i) {
+      const int e = min(10 * lane + i, kD - 1);
+      const int lo = __shfl(idx[0], e & 63), hi = __shfl(idx[1], e & 63);
+      const uint32_t fld = (uint32_t)((e >> 6) ? hi : lo);
+      if (10 * lane + i < kD) word |= fld << (3 * i);
+    }
+    if (ok && r == 0) {
+      const int64_t row = grp * f.t_alloc + pos;
+      if (lane < kPdim) f.v_packed[row * kPdim + lane] = word;
+      if (lane == 0) f.v_norms[row] = nrm;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int e = lane + 64 * i;
+        f.k_f16[row * kD + e] = __float2half_rn(kx[i]);
+        if (f.v_raw) {
+          if (f.v_dtype == TQ_F32) ((float*)f.v_raw)[row * kD + e] = x[i];
+          else if (f.v_dtype == TQ_F16) ((__half*)f.v_raw)[row * kD + e] = __float2half_rn(x[i]);
+          else ((__hip_bfloat16*)f.v_raw)[row * kD + e] = __float2bfloat16(x[i]);
+        }
+      }
+    }
+  } }
+  if (!fresh_wave) {
   float M = -INFINITY, L = 0.0f;
   f4 acc = {0.f, 0.f, 0.f, 0.f};
   for (int t0 = ph; t0 < n_tiles; t0 += 8 * U) {         // U tiles per lane group and round
@@ -1069,15 +1165,17 @@ __global__ __launch_bounds__(kMergeThreads) void decode_merge_rows_kernel(
   }
   *reinterpret_cast<f4*>(&acc_s[ph][4 * eq]) = acc;
   if (eq == 0) { ml_s[ph][0] = M; ml_s[ph][1] = L; }
+  }
   __syncthreads();
   if (tid >= 64) return;
+  constexpr int NP = FRESH ? 9 : 8;
   float Mt = ml_s[0][0];
 #pragma unroll
-  for (int p = 1; p < 8; ++p) Mt = fmaxf(Mt, ml_s[p][0]);
+  for (int p = 1; p < NP; ++p) Mt = fmaxf(Mt, ml_s[p][0]);
   float Lt = 0.0f;
   float v[2] = {0.0f, 0.0f};
 #pragma unroll
-  for (int p = 0; p < 8; ++p) {
+  for (int p = 0; p < NP; ++p) {
     const float f = (ml_s[p][0] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(ml_s[p][0] - Mt);
     Lt += f * ml_s[p][1];
     v[0] += f * acc_s[p][lane];
@@ -1092,6 +1190,25 @@ __global__ __launch_bounds__(kMergeThreads) void decode_merge_rows_kernel(
     if (NORM) val = (Lt > 0.0f) ? val / Lt : 0.0f;
     store_from_float<TO>(o + e, val);
   }
+}
+
+template <typename TO, bool NORM, int U = 8>
+__global__ __launch_bounds__(kMergeThreads) void decode_merge_rows_kernel(
+    const float* __restrict__ ws_S, const float* __restrict__ ws_ml, const int32_t* __restrict__ seq_offsets,
+    int64_t seq_len, int n_tiles_max, int n_kv, int n_rep, const float* __restrict__ signs, float inv_dim,
+    TO* __restrict__ out, int tile_pos, const int64_t* __restrict__ len_dev = nullptr, int64_t len_bias = 0) {
+  merge_rows_body<TO, NORM, U, false>(ws_S, ws_ml, seq_offsets, seq_len, n_tiles_max, n_kv, n_rep, signs, inv_dim, out,
+                                      tile_pos, len_dev, len_bias, nullptr);
+}
+
+// The merge pass of a decode step that inserts its token here (see FreshToken): 320 threads.
+template <typename TO, int U>
+__global__ __launch_bounds__(kMergeThreads + 64) void decode_merge_fresh_kernel(
+    const float* __restrict__ ws_S, const float* __restrict__ ws_ml, int64_t seq_len, int n_tiles_max, int n_kv,
+    int n_rep, const float* __restrict__ signs, float inv_dim, TO* __restrict__ out, int tile_pos,
+    const int64_t* __restrict__ len_dev, FreshToken ft) {
+  merge_rows_body<TO, true, U, true>(ws_S, ws_ml, nullptr, seq_len, n_tiles_max, n_kv, n_rep, signs, inv_dim, out,
+                                     tile_pos, len_dev, 0, &ft);
 }
 
 }  // namespace tqm
