@@ -1069,13 +1069,17 @@ __device__ __forceinline__ void merge_rows_body(
   const float sign0 = signs[lane], sign1 = signs[lane + 64];
   bool fresh_wave = false;
   if constexpr (FRESH) fresh_wave = tid >= 256;
+  // what the wavefront of the inserted token keeps for its stores, which wait until the fold is under way
+  float x[2] = {0.f, 0.f}, kx[2] = {0.f, 0.f}, fresh_nrm = 0.0f;
+  int idx[2] = {0, 0};
+  int64_t fresh_row = -1;
   if constexpr (FRESH) { if (fresh_wave) {
     // ---- the inserted token (one wavefront) ------------------------------------------------------------
     const FreshToken& f = *ft;
     const int64_t pos = f.pos_dev ? *f.pos_dev : f.pos;
     const bool ok = pos >= 0 && pos < f.t_alloc;
     const int64_t src = grp * kD;
-    float x[2], kx[2], qx[2], sq[2];
+    float qx[2], sq[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int e = lane + 64 * i;
@@ -1089,7 +1093,8 @@ __device__ __forceinline__ void merge_rows_body(
     const float safe = fmaxf(nrm, 1e-8f);
     float v[2] = {(x[0] / safe) * sign0, (x[1] / safe) * sign1};
     raw_butterfly<kD>(v, lane);
-    int idx[2];
+    fresh_nrm = nrm;
+    if (ok && r == 0) fresh_row = grp * f.t_alloc + pos;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       uint32_t n = 0;
@@ -1107,30 +1112,6 @@ __device__ __forceinline__ void merge_rows_body(
     if (lane == 0) {
       ml_s[8][0] = ok ? d * f.cs : -INFINITY;
       ml_s[8][1] = 1.0f;
-    }
-    // packed word `lane` holds elements 10 * lane .. 10 * lane + 9 (3-bit fields, lowest first)
-    uint32_t word = 0;
-#pragma unroll
-    for (int i = 0; i < 10; ++i) {
-      const int e = min(10 * lane + i, kD - 1);
-      const int lo = __shfl(idx[0], e & 63), hi = __shfl(idx[1], e & 63);
-      const uint32_t fld = (uint32_t)((e >> 6) ? hi : lo);
-      if (10 * lane + i < kD) word |= fld << (3 * i);
-    }
-    if (ok && r == 0) {
-      const int64_t row = grp * f.t_alloc + pos;
-      if (lane < kPdim) f.v_packed[row * kPdim + lane] = word;
-      if (lane == 0) f.v_norms[row] = nrm;
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        const int e = lane + 64 * i;
-        f.k_f16[row * kD + e] = __float2half_rn(kx[i]);
-        if (f.v_raw) {
-          if (f.v_dtype == TQ_F32) ((float*)f.v_raw)[row * kD + e] = x[i];
-          else if (f.v_dtype == TQ_F16) ((__half*)f.v_raw)[row * kD + e] = __float2half_rn(x[i]);
-          else ((__hip_bfloat16*)f.v_raw)[row * kD + e] = __float2bfloat16(x[i]);
-        }
-      }
     }
   } }
   if (!fresh_wave) {
@@ -1167,6 +1148,33 @@ __device__ __forceinline__ void merge_rows_body(
   if (eq == 0) { ml_s[ph][0] = M; ml_s[ph][1] = L; }
   }
   __syncthreads();
+  if constexpr (FRESH) { if (fresh_wave) {
+    // packed word `lane` holds elements 10 * lane .. 10 * lane + 9 (3-bit fields, lowest first)
+    const FreshToken& f = *ft;
+    uint32_t word = 0;
+#pragma unroll
+    for (int i = 0; i < 10; ++i) {
+      const int e = min(10 * lane + i, kD - 1);
+      const int lo = __shfl(idx[0], e & 63), hi = __shfl(idx[1], e & 63);
+      const uint32_t fld = (uint32_t)((e >> 6) ? hi : lo);
+      if (10 * lane + i < kD) word |= fld << (3 * i);
+    }
+    if (fresh_row >= 0) {                                  // first query head of the kv head, position inside the storage
+      const int64_t row = fresh_row;
+      if (lane < kPdim) f.v_packed[row * kPdim + lane] = word;
+      if (lane == 0) f.v_norms[row] = fresh_nrm;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int e = lane + 64 * i;
+        f.k_f16[row * kD + e] = __float2half_rn(kx[i]);
+        if (f.v_raw) {
+          if (f.v_dtype == TQ_F32) ((float*)f.v_raw)[row * kD + e] = x[i];
+          else if (f.v_dtype == TQ_F16) ((__half*)f.v_raw)[row * kD + e] = __float2half_rn(x[i]);
+          else ((__hip_bfloat16*)f.v_raw)[row * kD + e] = __float2bfloat16(x[i]);
+        }
+      }
+    }
+  } }
   if (tid >= 64) return;
   constexpr int NP = FRESH ? 9 : 8;
   float Mt = ml_s[0][0];
