@@ -727,8 +727,9 @@ int launch_vonly_mfma(const void* q, int q_dtype, const void* k_f16, const uint3
   const int n_q = sh.n_kv_heads * sh.n_rep;
   // no mask, no ragged offsets, 16-byte aligned V rows of every tile: with full tiles on top, the PLAIN variants apply
   // (a length read on the device rules them out as well: sh.seq_len is then only its upper bound)
-  const bool plain_base = !sh.mask && !sh.seq_offsets && !len_dev && sh.attn_scale > 0.0f && tq::aligned(v_packed, 16) &&
-                          sh.v_seq_stride % 4 == 0 && sh.v_head_stride % 4 == 0;
+  const bool plain_any = !sh.mask && !sh.seq_offsets && sh.attn_scale > 0.0f && tq::aligned(v_packed, 16) &&
+                         sh.v_seq_stride % 4 == 0 && sh.v_head_stride % 4 == 0;
+  const bool plain_base = plain_any && !len_dev;
   const bool plain = plain_base && sh.seq_len % tqm::kTilePos == 0;
   // Long unmasked caches: several consecutive 512-position blocks per workgroup, as many as still leave
   // one workgroup per CU (256) and divide the length.
@@ -796,8 +797,10 @@ int launch_vonly_mfma(const void* q, int q_dtype, const void* k_f16, const uint3
     if (n_blocks > 1 && ragged_stream) tqm::vonly_stream_kernel<QF, true><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb, n_blocks); \
     else if (n_blocks > 1) tqm::vonly_stream_kernel<QF, false><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb, n_blocks); \
     else if (nw == 8 && plain) tqm::vonly_tile_mfma_kernel<true, QF, 8><<<grid, 512, 0, stream>>>(a, vcb);           \
+    else if (nw == 8 && plain_any) tqm::vonly_tile_anylen_kernel<QF, 8><<<grid, 512, 0, stream>>>(a, vcb);           \
     else if (nw == 8) tqm::vonly_tile_mfma_kernel<false, QF, 8><<<grid, 512, 0, stream>>>(a, vcb);                   \
     else if (plain4) tqm::vonly_tile_mfma_kernel<true, QF, 4><<<grid, 256, 0, stream>>>(a, vcb);                     \
+    else if (plain_any) tqm::vonly_tile_anylen_kernel<QF, 4><<<grid, 256, 0, stream>>>(a, vcb);                      \
     else tqm::vonly_tile_mfma_kernel<false, QF, 4><<<grid, 256, 0, stream>>>(a, vcb)
     if (q_f32) { LAUNCH_TILE(true); } else { LAUNCH_TILE(false); }
 #undef LAUNCH_TILE

@@ -134,8 +134,8 @@ __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
 // QF32: the queries are float32 and enter as an fp16 value plus the fp16 remainder of that rounding (two
 // matrix instructions per key operand), which keeps float32-query fidelity; otherwise fp16 (or bf16) queries.
 template <bool PLAIN, bool QF32, int NW>
-__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 8 ? 2 : 3, NW == 8 ? 2 : 3)))
-void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
+__device__ __forceinline__ void vonly_tile_body(const MfmaArgs& a, const Codebook& vcb, const int64_t first,
+                                                const int64_t len) {
   constexpr int kTPos = NW * kWavePos;                 // positions per workgroup
   constexpr int kThr = NW * 64;
   // 4 KB per wave used three ways: per-wave staging first for the packed V block, then for K
@@ -156,14 +156,6 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
   const int n_q = a.n_kv * n_rep;
   const int64_t q_row0 = (int64_t)seq * n_q + (int64_t)kvh * n_rep;
 
-  int64_t first = 0, len = a.seq_len;
-  if (!PLAIN && a.seq_offsets) {
-    first = a.seq_offsets[seq];
-    len = (int64_t)a.seq_offsets[seq + 1] - first;
-  } else if (!PLAIN && a.len_dev) {
-    const int64_t want = *a.len_dev + a.len_bias;
-    len = want < 0 ? 0 : (want < len ? want : len);
-  }
   const int64_t tile_p0 = (int64_t)tile * kTPos;
   TQ_STAMP(0);
   if (tile_p0 >= len) return;                          // the merge pass never reads this tile
@@ -499,6 +491,37 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
     pml[2 * h + 1] = L;
   }
   TQ_STAMP(10);
+}
+
+template <bool PLAIN, bool QF32, int NW>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 8 ? 2 : 3, NW == 8 ? 2 : 3)))
+void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
+  int64_t first = 0, len = a.seq_len;
+  if (!PLAIN && a.seq_offsets) {
+    first = a.seq_offsets[blockIdx.z];
+    len = (int64_t)a.seq_offsets[blockIdx.z + 1] - first;
+  } else if (!PLAIN && a.len_dev) {
+    const int64_t want = *a.len_dev + a.len_bias;
+    len = want < 0 ? 0 : (want < len ? want : len);
+  }
+  vonly_tile_body<PLAIN, QF32, NW>(a, vcb, first, len);
+}
+
+// The same pass for unmasked caches of ANY length (host-checked: no mask, no ragged offsets, positive scale,
+// 16-byte aligned value rows): a workgroup whose tile lies wholly inside the sequence runs the PLAIN body, the one
+// tile that straddles the end runs the general body, tiles past the end leave at once.  The length may live in
+// device memory (len_dev), which is what a step recorded in a HIP graph needs.
+template <bool QF32, int NW>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 8 ? 2 : 3, NW == 8 ? 2 : 3)))
+void vonly_tile_anylen_kernel(MfmaArgs a, Codebook vcb) {
+  int64_t len = a.seq_len;
+  if (a.len_dev) {
+    const int64_t want = *a.len_dev + a.len_bias;
+    len = want < 0 ? 0 : (want < len ? want : len);
+  }
+  const int64_t tile_end = ((int64_t)blockIdx.x + 1) * (NW * kWavePos);
+  if (tile_end <= len) vonly_tile_body<true, QF32, NW>(a, vcb, 0, len);
+  else vonly_tile_body<false, QF32, NW>(a, vcb, 0, len);
 }
 
 // Scores pass of the thresholded decode step (weights below a threshold are dropped, and the threshold
