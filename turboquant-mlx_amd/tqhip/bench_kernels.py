@@ -261,7 +261,8 @@ CASES = {"step": bench_step, "prefill": bench_prefill, "encode": bench_encode, "
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--iters", type=int, default=200)
-    ap.add_argument("--cases", default=",".join(CASES))
+    ap.add_argument("--cases", default=",".join(c for c in CASES if c != "step"),
+                    help="comma-separated; `step` (wall time of whole layer steps) runs only when named")
     args = ap.parse_args()
     dev = torch.device("cuda:0")
     for c in args.cases.split(","):
