@@ -1429,11 +1429,18 @@ extern "C" int tq_packed_decode_step(const tq_packed_cache_desc* c, const void* 
                                         "tq_prerotate_query and tq_flash_decode otherwise)", who);
   const int pdim = tq::packed_dim(c->dim, c->bits);
   const int64_t groups = (int64_t)c->n_seq * c->n_kv_heads;
-  if (int rc = tq_encode(k_new, k_dtype, c->k_signs, c->boundaries, c->k_packed + position * pdim, c->k_norms + position,
-                         groups, 1, c->t_alloc, c->t_alloc, c->dim, c->bits, c->variant, stream_))
-    return rc;
-  if (int rc = tq_encode(v_new, v_dtype, c->v_signs, c->boundaries, c->v_packed + position * pdim, c->v_norms + position,
-                         groups, 1, c->t_alloc, c->t_alloc, c->dim, c->bits, c->variant, stream_))
+  if (tq::check_dtype(k_dtype) || tq::check_dtype(v_dtype))
+    return tq::fail(TQ_ERR_DTYPE, "%s: unknown dtype %d / %d", who, k_dtype, v_dtype);
+  if (c->variant != TQ_ENCODE_MLX && c->variant != TQ_ENCODE_METAL)
+    return tq::fail(TQ_ERR_ARG, "%s: unknown variant %d", who, c->variant);
+  if (!k_new || !v_new || !c->k_signs || !c->v_signs) return tq::fail(TQ_ERR_NULL, "%s: null pointer", who);
+  if (!tq::aligned(k_new, tq::dtype_size(k_dtype)) || !tq::aligned(v_new, tq::dtype_size(v_dtype)) ||
+      !tq::aligned(c->k_signs, 4) || !tq::aligned(c->v_signs, 4) || !tq::aligned(c->k_packed, 4) ||
+      !tq::aligned(c->v_packed, 4) || !tq::aligned(c->k_norms, 4) || !tq::aligned(c->v_norms, 4))
+    return tq::fail(TQ_ERR_ALIGN, "%s: misaligned pointer", who);
+  if (int rc = tq::encode_pair(k_new, k_dtype, c->k_signs, c->k_packed + position * pdim, c->k_norms + position, v_new,
+                               v_dtype, c->v_signs, c->v_packed + position * pdim, c->v_norms + position, c->boundaries,
+                               groups, c->t_alloc, c->variant, stream_))
     return rc;
   tq_decode_shape sh{};
   sh.n_seq = c->n_seq; sh.n_kv_heads = c->n_kv_heads; sh.n_rep = c->n_rep; sh.dim = c->dim; sh.bits = c->bits;

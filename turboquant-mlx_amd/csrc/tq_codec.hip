@@ -733,7 +733,75 @@ int grid_for_rows(int64_t rows) {
 
 }  // namespace
 
+// Key and value rows of one decode step in one launch (d = 128, 3-bit, one wavefront per row): rows
+// 0 .. n_rows - 1 are the keys (signs, destination 0), rows n_rows .. 2 n_rows - 1 the values.  Same
+// arithmetic, operation for operation, as encode_kernel.
+struct PairSide {
+  const void* x;
+  const float* signs;
+  uint32_t* packed;
+  float* norms;
+  int dtype;
+};
+
+__global__ __launch_bounds__(kBlock) void encode_pair_kernel(PairSide k, PairSide v, Thresholds thr, int64_t n_rows,
+                                                             int64_t group_stride) {
+  constexpr int D = 128, PDIM = 13;
+  const int lane = threadIdx.x & (TQ_WAVE - 1);
+  const int wave = threadIdx.x >> 6;
+  const int64_t slot = (int64_t)blockIdx.x * kWavesPerBlock + wave;
+  if (slot >= 2 * n_rows) return;                          // no barriers below: a wavefront may leave alone
+  const bool is_v = slot >= n_rows;
+  const PairSide& s = is_v ? v : k;
+  const int64_t row = is_v ? slot - n_rows : slot;
+  float xv[2], sq[2], sg[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int64_t at = row * D + lane + 64 * i;
+    xv[i] = s.dtype == TQ_F16 ? __half2float(((const __half*)s.x)[at])
+          : s.dtype == TQ_F32 ? ((const float*)s.x)[at] : __bfloat162float(((const __hip_bfloat16*)s.x)[at]);
+    sg[i] = s.signs[lane + 64 * i];
+    sq[i] = xv[i] * xv[i];
+  }
+  const float ss = tree_sum<D>(sq);
+  const float nrm = sqrtf(ss);
+  const float safe = fmaxf(nrm, 1e-8f);
+  float w[2] = {(xv[0] / safe) * sg[0], (xv[1] / safe) * sg[1]};
+  raw_butterfly<D>(w, lane);
+  int idx[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    uint32_t n = 0;
+#pragma unroll
+    for (int b = 0; b < 7; ++b) n += (w[i] > thr.t[b]) ? 1u : 0u;
+    idx[i] = (int)n;
+  }
+  uint32_t word = 0;                                       // word `lane`: elements 10 * lane .. 10 * lane + 9
+#pragma unroll
+  for (int i = 0; i < 10; ++i) {
+    const int e = min(10 * lane + i, D - 1);
+    const int lo = __shfl(idx[0], e & 63), hi = __shfl(idx[1], e & 63);
+    const uint32_t fld = (uint32_t)((e >> 6) ? hi : lo);
+    if (10 * lane + i < D) word |= fld << (3 * i);
+  }
+  if (lane < PDIM) s.packed[row * group_stride * PDIM + lane] = word;
+  if (lane == 0) s.norms[row * group_stride] = nrm;
+}
+
 namespace tq {
+int encode_pair(const void* k_new, int k_dtype, const float* k_signs, uint32_t* k_packed, float* k_norms,
+                const void* v_new, int v_dtype, const float* v_signs, uint32_t* v_packed, float* v_norms,
+                const float* boundaries, int64_t n_rows, int64_t group_stride, int variant, tq_stream_t stream_) {
+  Thresholds thr;
+  for (int i = 0; i < 15; ++i) thr.t[i] = INFINITY;
+  encode_thresholds(boundaries, 128, 3, variant, thr.t);
+  PairSide k{k_new, k_signs, k_packed, k_norms, k_dtype}, v{v_new, v_signs, v_packed, v_norms, v_dtype};
+  const int grid = (int)((2 * n_rows + kWavesPerBlock - 1) / kWavesPerBlock);
+  encode_pair_kernel<<<grid, kBlock, 0, (hipStream_t)stream_>>>(k, v, thr, n_rows, group_stride);
+  TQ_CHECK_LAUNCH("encode_pair launch");
+  return TQ_OK;
+}
+
 void encode_thresholds(const float* boundaries, int dim, int bits, int variant, float* thr_out) {
   const float s = (float)(1.0 / sqrt((double)dim));
   const int nb = (1 << bits) - 1;

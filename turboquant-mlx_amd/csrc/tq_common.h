@@ -59,6 +59,13 @@ inline int check_dtype(int dt) { return (dt == TQ_F32 || dt == TQ_F16 || dt == T
 // fl(fl(w * s) / s) with the boundary, TQ_ENCODE_METAL compares w itself.
 void encode_thresholds(const float* boundaries, int dim, int bits, int variant, float* thr_out);
 
+// One new key row and one new value row per group (d = 128, 3-bit) encoded by ONE launch: row g of either
+// tensor goes to packed + g * group_stride * 13 words and norms + g * group_stride (defined beside the
+// encoder; the caller has validated pointers and dtypes).
+int encode_pair(const void* k_new, int k_dtype, const float* k_signs, uint32_t* k_packed, float* k_norms,
+                const void* v_new, int v_dtype, const float* v_signs, uint32_t* v_packed, float* v_norms,
+                const float* boundaries, int64_t n_rows, int64_t group_stride, int variant, tq_stream_t stream);
+
 inline size_t dtype_size(int dt) { return dt == TQ_F32 ? 4 : 2; }
 
 inline int check_dim_bits(int dim, int bits) {
