@@ -721,3 +721,23 @@ def test_vonly_decode_step_from_an_empty_cache_and_at_tile_boundaries(tq, dtype)
                 tol = 1e-3 + (8e-3 if dtype == torch.bfloat16 else 2e-3) * np.abs(ref)
                 assert (err <= tol).all(), (a.offset, err.max())
     assert a.offset == 0 + 1 + 254 + 1 + 255 + 1 + 2 + 2 + 253 + 1 + 1 + 2
+
+
+def test_vonly_decode_step_other_shapes_take_the_append_route(tq):
+    """d = 64 / 4-bit values: tq_vonly_decode_step has no two-launch form there and runs tq_vonly_append +
+    tq_vonly_decode_attn inside the one call: the very bits of the two calls of the Python surface."""
+    B, n_q, n_kv, D, S0 = 1, 6, 2, 64, 70
+    sc = 1 / math.sqrt(D)
+    a, b = tq.VOnlyTurboQuantCache(bits=4, fused=True), tq.VOnlyTurboQuantCache(bits=4, fused=True)
+    k0, v0 = rand((B, n_kv, S0, D), 1100), rand((B, n_kv, S0, D), 1101)
+    a.update_and_fetch(k0, v0), b.update_and_fetch(k0, v0)
+    for i in range(3):
+        k1, v1, q1 = rand((B, n_kv, 1, D), 1110 + 3 * i), rand((B, n_kv, 1, D), 1111 + 3 * i), rand((B, n_q, 1, D), 1112 + 3 * i)
+        got = a.decode_step(q1, k1, v1, sc)
+        b.update_and_fetch(k1, v1)
+        assert torch.equal(got, tq.vonly_decode_attention(q1, b, sc))
+    for x, y in zip(a.state, b.state):
+        assert torch.equal(x, y)
+    pos = torch.tensor([a.offset], dtype=torch.int64, device="cuda")
+    with pytest.raises((ValueError, RuntimeError)):
+        a.decode_step(q1, k1, v1, sc, position=pos)                  # the device-side position needs d = 128 / 3-bit
