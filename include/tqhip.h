@@ -355,6 +355,16 @@ int tq_packed_decode_step(const tq_packed_cache_desc* cache /* host */,
                           int64_t position, float attn_scale, tq_stream_t stream);
 
 /*
+ * tq_packed_decode_step with the position read from device memory (see tq_vonly_decode_step_at): encodes
+ * the new key and value rows at *position_dev and attends over positions 0 .. *position_dev; grids and the
+ * workspace are sized for t_alloc positions; an insert outside the storage is dropped.
+ */
+int tq_packed_decode_step_at(const tq_packed_cache_desc* cache /* host */,
+                             const void* k_new, int k_dtype, const void* v_new, int v_dtype,
+                             const void* q, int q_dtype, void* out, int out_dtype,
+                             const int64_t* position_dev /* device */, float attn_scale, tq_stream_t stream);
+
+/*
  * The same call with its two passes selectable: phases = 1 runs only the tile pass (per-tile
  * partial sums and softmax statistics into `workspace`), phases = 2 only the merge pass (workspace
  * -> out), phases = 3 both (= tq_vonly_decode_attn).  For callers that time or overlap the passes;

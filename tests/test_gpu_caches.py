@@ -741,3 +741,56 @@ def test_vonly_decode_step_other_shapes_take_the_append_route(tq):
     pos = torch.tensor([a.offset], dtype=torch.int64, device="cuda")
     with pytest.raises((ValueError, RuntimeError)):
         a.decode_step(q1, k1, v1, sc, position=pos)                  # the device-side position needs d = 128 / 3-bit
+
+
+@pytest.mark.parametrize("S0,want_alloc", [(300, 1024), (31000, 32768)])
+def test_packed_decode_step_replayed_from_a_hip_graph(tq, S0, want_alloc):
+    """The packed cache's decode step recorded once in a HIP graph with the position in device memory
+    (tq_packed_decode_step_at) and replayed for eight tokens, with eager work and synchronisations between
+    the replays: every replay matches the eager step on a twin cache, and both caches end in the same state
+    bit for bit.  An insert past the storage is dropped.  The long case runs the streaming pass (storage of
+    32768 positions x 8 kv heads), the short one the single-tile pass."""
+    B, n_q, n_kv, D, N = 1, 32, 8, 128, 8
+    sc = 1 / math.sqrt(D)
+    k0, v0 = rand((B, n_kv, S0, D), 1200), rand((B, n_kv, S0, D), 1201)
+    cg, ce = tq.TurboQuantKVCache(bits=3, fused=True), tq.TurboQuantKVCache(bits=3, fused=True)
+    cg.reserve(B, n_kv, want_alloc, D)
+    cg.update_and_fetch(k0, v0), ce.update_and_fetch(k0, v0)
+    t_alloc = cg.v_packed.shape[2]
+    assert t_alloc == want_alloc
+    from tqhip import _lib
+    assert (_lib.load().tq_flash_decode_plan(B, n_kv, t_alloc, 1, 0) >= 2) == (want_alloc == 32768)
+    pos = torch.tensor([S0], dtype=torch.int64, device="cuda")
+    qs, ks, vs = rand((B, n_q, 1, D), 1202), rand((B, n_kv, 1, D), 1203), rand((B, n_kv, 1, D), 1204)
+    out_s = torch.empty((B, n_q, D), dtype=torch.float16, device="cuda")
+
+    def check(step_no, q, k, v):
+        want = ce.decode_step(q, k, v, sc)[:, :, 0].float()
+        err = (out_s.float() - want).abs()
+        assert bool((err <= 1e-3 + 2e-3 * want.abs()).all()), (step_no, float(err.max()))
+
+    cg.decode_step(qs, ks, vs, sc, position=pos, out=out_s)
+    pos.add_(1)
+    check(-1, qs, ks, vs)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        cg.decode_step(qs, ks, vs, sc, position=pos, out=out_s)
+        pos.add_(1)
+    for i in range(N):
+        q, k, v = rand((B, n_q, 1, D), 1210 + 3 * i), rand((B, n_kv, 1, D), 1211 + 3 * i), rand((B, n_kv, 1, D), 1212 + 3 * i)
+        qs.copy_(q), ks.copy_(k), vs.copy_(v)
+        graph.replay()
+        check(i, q, k, v)
+        torch.cuda.synchronize()
+    cg.offset = int(pos.item())
+    assert cg.offset == ce.offset == S0 + 1 + N
+    for x, y in zip(cg.state, ce.state):
+        assert torch.equal(x, y)
+    before = [t.clone() for t in (cg.k_packed, cg.k_norms, cg.v_packed, cg.v_norms)]
+    pos.fill_(t_alloc)
+    graph.replay()
+    torch.cuda.synchronize()
+    for x, y in zip(before, (cg.k_packed, cg.k_norms, cg.v_packed, cg.v_norms)):
+        assert torch.equal(x, y)
+    assert bool(torch.isfinite(out_s.float()).all())

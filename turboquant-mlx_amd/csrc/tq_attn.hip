@@ -863,7 +863,7 @@ int launch_packed_mfma(const float* q_rot_or_weights, const uint32_t* k_packed, 
                        const float* v_centroids, const float* v_signs, void* out, void* workspace,
                        size_t workspace_bytes, const tq_decode_shape& sh, float threshold, hipStream_t stream,
                        const char* who, const void* q_raw = nullptr, int q_dtype = TQ_F32,
-                       const float* k_signs = nullptr) {
+                       const float* k_signs = nullptr, const int64_t* len_dev = nullptr, int64_t len_bias = 0) {
   const int n_q = sh.n_kv_heads * sh.n_rep;
   const int n_tiles = (int)((sh.seq_len + tqm::kTilePos - 1) / tqm::kTilePos);
   const size_t need = (size_t)sh.n_seq * n_q * n_tiles * (tqm::kD + 2) * sizeof(float);
@@ -892,8 +892,9 @@ int launch_packed_mfma(const float* q_rot_or_weights, const uint32_t* k_packed, 
   if (MODE != tqm::kWeights) a.score_scale *= tq::fill_codebook_fp16(kcb, k_centroids, sh.bits);
   a.v_unscale = tq::fill_codebook_fp16(vcb, v_centroids, sh.bits);
   int tile_pos = tqm::kTilePos;
+  a.len_dev = len_dev; a.len_bias = len_bias;             // a length read on the device: an upper bound on the host, like a ragged batch
   const int n_steps = (MODE == tqm::kFlash && !sh.mask)
-                          ? flash_stream_steps(sh.n_seq, sh.n_kv_heads, sh.seq_len, sh.seq_offsets != nullptr) : 0;
+                          ? flash_stream_steps(sh.n_seq, sh.n_kv_heads, sh.seq_len, sh.seq_offsets != nullptr || len_dev != nullptr) : 0;
   if (n_steps >= 2) {
     tile_pos = tqm::kSStepPos * n_steps;
     a.n_tiles_max = (int)((sh.seq_len + tile_pos - 1) / tile_pos);
@@ -909,7 +910,8 @@ int launch_packed_mfma(const float* q_rot_or_weights, const uint32_t* k_packed, 
   const int n_parts = a.n_tiles_max;
 #define LAUNCH_MERGE_P(TO)                                                                                    \
   tqm::decode_merge_rows_kernel<TO, MODE == tqm::kFlash><<<mgrid, tqm::kMergeThreads, 0, stream>>>(            \
-      a.ws_S, a.ws_ml, sh.seq_offsets, sh.seq_len, n_parts, sh.n_kv_heads, sh.n_rep, v_signs, inv_dim, (TO*)out, tile_pos)
+      a.ws_S, a.ws_ml, sh.seq_offsets, sh.seq_len, n_parts, sh.n_kv_heads, sh.n_rep, v_signs, inv_dim, (TO*)out, tile_pos, \
+      len_dev, len_bias)
   if (sh.out_dtype == TQ_F16) { LAUNCH_MERGE_P(__half); }
   else if (sh.out_dtype == TQ_BF16) { LAUNCH_MERGE_P(__hip_bfloat16); }
   else { LAUNCH_MERGE_P(float); }
@@ -1411,10 +1413,10 @@ extern "C" int tq_vonly_decode_step_at(const tq_vonly_cache_desc* c, const void*
   return tq::fail(TQ_ERR_UNSUPPORTED, "%s: shape not covered", who);
 }
 
-extern "C" int tq_packed_decode_step(const tq_packed_cache_desc* c, const void* k_new, int k_dtype, const void* v_new,
-                                     int v_dtype, const void* q, int q_dtype, void* out, int out_dtype,
-                                     int64_t position, float attn_scale, tq_stream_t stream_) {
-  const char* who = "tq_packed_decode_step";
+namespace {
+int packed_step(const tq_packed_cache_desc* c, const void* k_new, int k_dtype, const void* v_new, int v_dtype,
+                const void* q, int q_dtype, void* out, int out_dtype, int64_t position, const int64_t* position_dev,
+                float attn_scale, tq_stream_t stream_, const char* who) {
   if (!c) return tq::fail(TQ_ERR_NULL, "%s: null cache descriptor", who);
   if (int rc = tq::check_dim_bits(c->dim, c->bits)) return rc;
   if (c->n_seq < 1 || c->n_kv_heads < 1 || c->t_alloc < 1)
@@ -1440,15 +1442,43 @@ extern "C" int tq_packed_decode_step(const tq_packed_cache_desc* c, const void* 
     return tq::fail(TQ_ERR_ALIGN, "%s: misaligned pointer", who);
   if (int rc = tq::encode_pair(k_new, k_dtype, c->k_signs, c->k_packed + position * pdim, c->k_norms + position, v_new,
                                v_dtype, c->v_signs, c->v_packed + position * pdim, c->v_norms + position, c->boundaries,
-                               groups, c->t_alloc, c->variant, stream_))
+                               groups, c->t_alloc, c->variant, stream_, position_dev))
     return rc;
   tq_decode_shape sh{};
   sh.n_seq = c->n_seq; sh.n_kv_heads = c->n_kv_heads; sh.n_rep = c->n_rep; sh.dim = c->dim; sh.bits = c->bits;
   sh.block_size = 16;
-  sh.seq_len = position + 1;
+  sh.seq_len = position_dev ? c->t_alloc : position + 1;   // device position: upper bound that sizes grid and workspace
   sh.k_head_stride = sh.kn_head_stride = sh.v_head_stride = sh.vn_head_stride = c->t_alloc;
   sh.k_seq_stride = sh.kn_seq_stride = sh.v_seq_stride = sh.vn_seq_stride = c->t_alloc * c->n_kv_heads;
   sh.attn_scale = attn_scale; sh.out_dtype = out_dtype; sh.allow_mma = 1;
-  return tq_flash_decode_from_q(q, q_dtype, c->k_signs, c->k_packed, c->k_norms, c->v_packed, c->v_norms, c->centroids,
-                                c->centroids, c->v_signs, 0.0f, out, c->workspace, c->workspace_bytes, &sh, stream_);
+  if (!position_dev)
+    return tq_flash_decode_from_q(q, q_dtype, c->k_signs, c->k_packed, c->k_norms, c->v_packed, c->v_norms, c->centroids,
+                                  c->centroids, c->v_signs, 0.0f, out, c->workspace, c->workspace_bytes, &sh, stream_);
+  if (int rc = check_shape(&sh, who, 128)) return rc;
+  if (tq::check_dtype(q_dtype)) return tq::fail(TQ_ERR_DTYPE, "%s: unknown q_dtype %d", who, q_dtype);
+  if (!q || !out) return tq::fail(TQ_ERR_NULL, "%s: null pointer", who);
+  if (!tq::aligned(q, (int)tq::dtype_size(q_dtype)) || !tq::aligned(position_dev, 8))
+    return tq::fail(TQ_ERR_ALIGN, "%s: misaligned pointer", who);
+  return launch_packed_mfma<tqm::kFlash>(nullptr, c->k_packed, c->k_norms, c->v_packed, c->v_norms, c->centroids,
+                                         c->centroids, c->v_signs, out, c->workspace, c->workspace_bytes, sh, 0.0f,
+                                         (hipStream_t)stream_, who, q, q_dtype, c->k_signs, position_dev, 1);
+}
+}  // namespace
+
+extern "C" int tq_packed_decode_step(const tq_packed_cache_desc* c, const void* k_new, int k_dtype, const void* v_new,
+                                     int v_dtype, const void* q, int q_dtype, void* out, int out_dtype,
+                                     int64_t position, float attn_scale, tq_stream_t stream_) {
+  if (c && (position < 0 || position >= c->t_alloc))
+    return tq::fail(TQ_ERR_ARG, "tq_packed_decode_step: position %lld outside the storage of %lld positions",
+                    (long long)position, (long long)c->t_alloc);
+  return packed_step(c, k_new, k_dtype, v_new, v_dtype, q, q_dtype, out, out_dtype, position, nullptr, attn_scale,
+                     stream_, "tq_packed_decode_step");
+}
+
+extern "C" int tq_packed_decode_step_at(const tq_packed_cache_desc* c, const void* k_new, int k_dtype, const void* v_new,
+                                        int v_dtype, const void* q, int q_dtype, void* out, int out_dtype,
+                                        const int64_t* position_dev, float attn_scale, tq_stream_t stream_) {
+  if (!position_dev) return tq::fail(TQ_ERR_NULL, "tq_packed_decode_step_at: null position_dev");
+  return packed_step(c, k_new, k_dtype, v_new, v_dtype, q, q_dtype, out, out_dtype, 0, position_dev, attn_scale,
+                     stream_, "tq_packed_decode_step_at");
 }

@@ -744,8 +744,10 @@ struct PairSide {
   int dtype;
 };
 
+// With pos_dev set the destination row of group g is g * group_stride + *pos_dev (read when the kernel runs;
+// nothing is stored when that position is outside 0 .. group_stride - 1).
 __global__ __launch_bounds__(kBlock) void encode_pair_kernel(PairSide k, PairSide v, Thresholds thr, int64_t n_rows,
-                                                             int64_t group_stride) {
+                                                             int64_t group_stride, const int64_t* pos_dev) {
   constexpr int D = 128, PDIM = 13;
   const int lane = threadIdx.x & (TQ_WAVE - 1);
   const int wave = threadIdx.x >> 6;
@@ -784,20 +786,27 @@ __global__ __launch_bounds__(kBlock) void encode_pair_kernel(PairSide k, PairSid
     const uint32_t fld = (uint32_t)((e >> 6) ? hi : lo);
     if (10 * lane + i < D) word |= fld << (3 * i);
   }
-  if (lane < PDIM) s.packed[row * group_stride * PDIM + lane] = word;
-  if (lane == 0) s.norms[row * group_stride] = nrm;
+  int64_t dst = row * group_stride;
+  if (pos_dev) {
+    const int64_t pos = *pos_dev;
+    if (pos < 0 || pos >= group_stride) return;
+    dst += pos;
+  }
+  if (lane < PDIM) s.packed[dst * PDIM + lane] = word;
+  if (lane == 0) s.norms[dst] = nrm;
 }
 
 namespace tq {
 int encode_pair(const void* k_new, int k_dtype, const float* k_signs, uint32_t* k_packed, float* k_norms,
                 const void* v_new, int v_dtype, const float* v_signs, uint32_t* v_packed, float* v_norms,
-                const float* boundaries, int64_t n_rows, int64_t group_stride, int variant, tq_stream_t stream_) {
+                const float* boundaries, int64_t n_rows, int64_t group_stride, int variant, tq_stream_t stream_,
+                const int64_t* pos_dev) {
   Thresholds thr;
   for (int i = 0; i < 15; ++i) thr.t[i] = INFINITY;
   encode_thresholds(boundaries, 128, 3, variant, thr.t);
   PairSide k{k_new, k_signs, k_packed, k_norms, k_dtype}, v{v_new, v_signs, v_packed, v_norms, v_dtype};
   const int grid = (int)((2 * n_rows + kWavesPerBlock - 1) / kWavesPerBlock);
-  encode_pair_kernel<<<grid, kBlock, 0, (hipStream_t)stream_>>>(k, v, thr, n_rows, group_stride);
+  encode_pair_kernel<<<grid, kBlock, 0, (hipStream_t)stream_>>>(k, v, thr, n_rows, group_stride, pos_dev);
   TQ_CHECK_LAUNCH("encode_pair launch");
   return TQ_OK;
 }

@@ -64,7 +64,8 @@ void encode_thresholds(const float* boundaries, int dim, int bits, int variant, 
 // encoder; the caller has validated pointers and dtypes).
 int encode_pair(const void* k_new, int k_dtype, const float* k_signs, uint32_t* k_packed, float* k_norms,
                 const void* v_new, int v_dtype, const float* v_signs, uint32_t* v_packed, float* v_norms,
-                const float* boundaries, int64_t n_rows, int64_t group_stride, int variant, tq_stream_t stream);
+                const float* boundaries, int64_t n_rows, int64_t group_stride, int variant, tq_stream_t stream,
+                const int64_t* pos_dev = nullptr);   // set: row g goes to g * group_stride + *pos_dev (device value)
 
 inline size_t dtype_size(int dt) { return dt == TQ_F32 ? 4 : 2; }
 

@@ -38,6 +38,8 @@ struct PackedArgs {
   const uint32_t* v_packed;
   const float* v_norms;
   const int32_t* seq_offsets;
+  const int64_t* len_dev;     // optional (no seq_offsets): every sequence attends
+  int64_t len_bias;           // min(max(*len_dev + len_bias, 0), seq_len) positions, read when the kernel runs
   const float* mask;
   float* scores;              // kScores: [n_q, T] f32; kSoftScores: [n_seq * n_q, w_stride] f32, log2 units
   float* stats_out;           // kSoftScores: [n_seq * n_kv, n_tiles_max, n_rep, 2] (maximum, sum of 2^(s - maximum)) per tile
@@ -179,6 +181,9 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
   if (a.seq_offsets) {
     first = a.seq_offsets[seq];
     len = (int64_t)a.seq_offsets[seq + 1] - first;
+  } else if (a.len_dev) {
+    const int64_t want = *a.len_dev + a.len_bias;
+    len = want < 0 ? 0 : (want < len ? want : len);
   }
   const int64_t tile_p0 = (int64_t)tile * kTilePos;
   if (tile_p0 >= len) return;
@@ -610,6 +615,9 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
   if (a.seq_offsets) {
     first = a.seq_offsets[seq];
     len = (int64_t)a.seq_offsets[seq + 1] - first;
+  } else if (a.len_dev) {
+    const int64_t want = *a.len_dev + a.len_bias;
+    len = want < 0 ? 0 : (want < len ? want : len);
   }
   const int64_t wg_p0 = (int64_t)wg * kSStepPos * n_steps;
   if (wg_p0 >= len) return;

@@ -81,6 +81,7 @@ PROTOTYPES = {
     "tq_packed_decode_step": (_i, [C.POINTER(PackedCacheDesc), _p, _i, _p, _i, _p, _i, _p, _i, _l, _f, _p]),
     "tq_vonly_append_at": (_i, [_p, _i, _p, _i, _p, _fp, _p, _p, _p, _p, _l, _l, _l, _i, _i, _i, _p, _p]),
     "tq_vonly_decode_step_at": (_i, [C.POINTER(VOnlyCacheDesc), _p, _i, _p, _i, _p, _i, _p, _i, _p, _f, _p]),
+    "tq_packed_decode_step_at": (_i, [C.POINTER(PackedCacheDesc), _p, _i, _p, _i, _p, _i, _p, _i, _p, _f, _p]),
     "tq_vonly_decode_attn_phases": (_i, [_p, _i, _p, _p, _p, _fp, _p, _p, _p, _z, C.POINTER(DecodeShape), _i, _p]),
     "tq_vonly_sparse_decode_attn": (_i, [_p, _i, _p, _p, _p, _fp, _p, _f, _p, _p, _z, C.POINTER(DecodeShape), _p]),
     "tq_vonly_sparse_workspace_bytes": (_z, [_i, _i, _l]),

@@ -229,29 +229,32 @@ def bench_step(iters, dev):
             print(f"layer step, {kind}, {n_q}/{n_kv} heads, T~{T}: update_and_fetch + attention {us2:6.1f} us wall, "
                   f"decode_step {us1:6.1f} us wall", flush=True)
             del c
-        caches = [tqhip.VOnlyTurboQuantCache(bits=3, fused=True) for _ in range(L)]
-        k0 = torch.randn((1, 4, T, D), device=dev, dtype=torch.float16)
-        for c in caches:
-            c.reserve(1, 4, T + 2048, D)
-            c.update_and_fetch(k0, k0)
-        k1 = torch.randn((1, 4, 1, D), device=dev, dtype=torch.float16)
-        q = torch.randn((1, 28, 1, D), device=dev, dtype=torch.float16)
-        outs = [torch.empty((1, 28, D), device=dev, dtype=torch.float16) for _ in range(L)]
-        pos = torch.tensor([T], dtype=torch.int64, device=dev)
+        for kind, n_q, n_kv in (("V-only cache", 28, 4), ("packed cache", 32, 8)):
+            mk = (lambda: tqhip.VOnlyTurboQuantCache(bits=3, fused=True)) if kind == "V-only cache" else \
+                 (lambda: tqhip.TurboQuantKVCache(bits=3, fused=True))
+            caches = [mk() for _ in range(L)]
+            k0 = torch.randn((1, n_kv, T, D), device=dev, dtype=torch.float16)
+            for c in caches:
+                c.reserve(1, n_kv, T + 2048, D)
+                c.update_and_fetch(k0, k0)
+            k1 = torch.randn((1, n_kv, 1, D), device=dev, dtype=torch.float16)
+            q = torch.randn((1, n_q, 1, D), device=dev, dtype=torch.float16)
+            outs = [torch.empty((1, n_q, D), device=dev, dtype=torch.float16) for _ in range(L)]
+            pos = torch.tensor([T], dtype=torch.int64, device=dev)
 
-        def token():
-            for i, c in enumerate(caches):
-                c.decode_step(q, k1, k1, sc, position=pos, out=outs[i])
-            pos.add_(1)
-        token()
-        torch.cuda.synchronize()
-        g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g):
+            def token():
+                for i, c in enumerate(caches):
+                    c.decode_step(q, k1, k1, sc, position=pos, out=outs[i])
+                pos.add_(1)
             token()
-        us = wall(g.replay, n) / L
-        print(f"layer step, V-only cache, 28/4 heads, T~{T}: {L} layers recorded in a HIP graph, position in device "
-              f"memory: {us:6.1f} us per layer step", flush=True)
-        del g, caches
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                token()
+            us = wall(g.replay, n) / L
+            print(f"layer step, {kind}, {n_q}/{n_kv} heads, T~{T}: {L} layers recorded in a HIP graph, position in "
+                  f"device memory: {us:6.1f} us per layer step", flush=True)
+            del g, caches
 
 
 CASES = {"step": bench_step, "prefill": bench_prefill, "encode": bench_encode, "scores": bench_scores, "sparse_v": bench_sparse_v, "flash": bench_flash,

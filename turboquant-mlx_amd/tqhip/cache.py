@@ -193,12 +193,25 @@ class TurboQuantKVCache:
             z = self._zero_scalars[key] = t.new_zeros(())
         return z
 
-    def decode_step(self, queries: torch.Tensor, keys: torch.Tensor, values: torch.Tensor, attn_scale: float):
+    def reserve(self, B: int, H: int, n_positions: int, dim: int, device="cuda"):
+        """Allocate storage for `n_positions` more positions now, so that steps recorded in a HIP graph keep
+        their addresses for that long (storage otherwise grows in steps of 256, which reallocates)."""
+        device = torch.device(device)
+        self._ensure_quantizer(dim, dim, device)
+        self._ensure_storage(B, H, n_positions, device)
+
+    def decode_step(self, queries: torch.Tensor, keys: torch.Tensor, values: torch.Tensor, attn_scale: float,
+                    position: torch.Tensor | None = None, out: torch.Tensor | None = None):
         """Encode one token and attend in one library call: the result of `update_and_fetch(keys, values)`
         followed by `turboquant_attention(queries, self, attn_scale, fused=True)` (no mask, no threshold) on
         a cache with packed keys and values.  queries (B, n_heads, 1, dim), keys / values (B, n_kv, 1, dim)
         -> (B, n_heads, 1, dim) in queries.dtype.  Not in the reference, where the two halves are separate
-        calls of the model's attention layer (cache.py:131-165, fused_attention.py:20-125)."""
+        calls of the model's attention layer (cache.py:131-165, fused_attention.py:20-125).
+
+        With `position` (one-element int64 GPU tensor holding the cache's current offset) the kernels read the
+        insert position and the attended length from it when they run, so the step can be recorded in a HIP
+        graph once and replayed while the caller advances the tensor; set `offset` afterwards.  `out`
+        (B, n_heads, dim) receives the result when given."""
         from . import attention
         B, n_q, S_q, dim = queries.shape
         H = values.shape[1]
@@ -222,10 +235,13 @@ class TurboQuantKVCache:
                 except ValueError:                 # storage handed in through `state` as slices
                     ok = False
         if not ok:
+            if position is not None:
+                raise ValueError("a step with a device-side position needs one new token, dim 128, 3-bit codes, "
+                                 "n_rep <= 16 and contiguous storage")
             self.update_and_fetch(keys, values)
             return attention.turboquant_attention(queries, self, attn_scale, fused=True)
         out = ops.packed_decode_step(self._step, keys[:, :, 0, :], values[:, :, 0, :], queries[:, :, 0, :],
-                                     self.offset, attn_scale)
+                                     self.offset if position is None else position, attn_scale, out=out)
         self.offset += 1          # _deq_offset stays behind: the next unfused fetch dequantises the whole cache
         return out[:, :, None, :]
 

@@ -838,29 +838,38 @@ class PackedStep:
         self._need = _lib.load().tq_workspace_bytes(_lib.TQ_OP_FLASH_DECODE, B, H * n_rep, T, dim)
 
 
-def packed_decode_step(step: PackedStep, keys: torch.Tensor, values: torch.Tensor, q: torch.Tensor, position: int,
-                       attn_scale: float, out_dtype=None) -> torch.Tensor:
+def packed_decode_step(step: PackedStep, keys: torch.Tensor, values: torch.Tensor, q: torch.Tensor, position,
+                       attn_scale: float, out_dtype=None, out: torch.Tensor | None = None) -> torch.Tensor:
     """One decode step of a packed cache in one library call (tq_packed_decode_step): encode the new token
     keys / values (B, n_kv, dim) at time index `position`, then attend with q (B, n_kv * n_rep, dim; not
     pre-rotated) over positions 0 .. position.  Same result as two encode_into calls followed by
-    flash_decode_from_q.  Returns (B, n_q, dim) in out_dtype (default q.dtype)."""
-    _need_gpu(keys, values, q)
+    flash_decode_from_q.  Returns (B, n_q, dim) in out_dtype (default q.dtype), written into `out` when given.
+    `position` may be a one-element int64 GPU tensor (tq_packed_decode_step_at), as in vonly_decode_step."""
+    _need_gpu(keys, values, q, out)
     B, H, T, D = step.shape
     n_q = H * step.n_rep
     if tuple(keys.shape) != (B, H, D) or tuple(values.shape) != (B, H, D) or tuple(q.shape) != (B, n_q, D):
         raise ValueError(f"expected keys / values {(B, H, D)} and q {(B, n_q, D)}, got {tuple(keys.shape)}, "
                          f"{tuple(values.shape)}, {tuple(q.shape)}")
-    if not 0 <= position < T:
+    on_device = isinstance(position, torch.Tensor)
+    if on_device:
+        if position.dtype != torch.int64 or position.numel() != 1 or not position.is_cuda:
+            raise ValueError("a device-side position must be a one-element int64 tensor on the GPU")
+    elif not 0 <= position < T:
         raise ValueError(f"position {position} outside the storage of {T} positions")
     keys, values, q = keys.contiguous(), values.contiguous(), q.contiguous()
-    out = torch.empty((B, n_q, D), dtype=out_dtype or q.dtype, device=q.device)
+    if out is None:
+        out = torch.empty((B, n_q, D), dtype=out_dtype or q.dtype, device=q.device)
+    elif tuple(out.shape) != (B, n_q, D) or not out.is_contiguous():
+        raise ValueError(f"out must be a contiguous {(B, n_q, D)} tensor")
     stream = _stream(q)
     ws = _workspace(q.device, stream.value or 0, step._need)
     d = step.desc
     d.workspace, d.workspace_bytes = ws.data_ptr(), ws.numel()
-    _lib.check(_lib.load().tq_packed_decode_step(
-        step._ref, _ptr(keys), _dt(keys), _ptr(values), _dt(values), _ptr(q), _dt(q), _ptr(out), _dt(out),
-        position, attn_scale, stream))
+    lib = _lib.load()
+    fn = lib.tq_packed_decode_step_at if on_device else lib.tq_packed_decode_step
+    _lib.check(fn(step._ref, _ptr(keys), _dt(keys), _ptr(values), _dt(values), _ptr(q), _dt(q), _ptr(out), _dt(out),
+                  _ptr(position) if on_device else position, attn_scale, stream))
     return out
 
 
