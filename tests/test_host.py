@@ -34,6 +34,37 @@ def test_decode_shape_struct_matches_header_size():
     assert ctypes.sizeof(_lib.DecodeShape) == 6 * 4 + 8 + 8 + 8 * 8 + 8 + 2 * 8 + 4 + 4 + 4 + 4
 
 
+def test_struct_mirrors_match_the_header_as_a_c_compiler_lays_it_out(tmp_path):
+    """include/tqhip.h is plain C: gcc compiles a probe that prints size and field offsets of every struct
+    the binding mirrors, and the ctypes mirrors must agree field by field."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no C compiler")
+    mirrors = {"tq_decode_shape": _lib.DecodeShape, "tq_vonly_cache_desc": _lib.VOnlyCacheDesc,
+               "tq_packed_cache_desc": _lib.PackedCacheDesc}
+    lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "tqhip.h"', 'int main(void) {']
+    for cname, mirror in mirrors.items():
+        lines.append(f'  printf("{cname} size %zu\\n", sizeof({cname}));')
+        for fname, _ in mirror._fields_:
+            lines.append(f'  printf("{cname} {fname} %zu\\n", offsetof({cname}, {fname}));')
+    lines += ['  return 0;', '}']
+    src = tmp_path / "abi_probe.c"
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "abi_probe"
+    inc = os.path.join(ROOT, "include")
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-I", inc, str(src), "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout
+    seen = 0
+    for line in out.splitlines():
+        cname, fname, value = line.split()
+        mirror = mirrors[cname]
+        want = ctypes.sizeof(mirror) if fname == "size" else getattr(mirror, fname).offset
+        assert int(value) == want, (cname, fname, value, want)
+        seen += 1
+    assert seen == sum(len(m._fields_) + 1 for m in mirrors.values())
+
+
 def test_argument_errors_without_launch():
     lib = _lib.load()
     null = ctypes.c_void_p(0)
