@@ -91,6 +91,22 @@ def test_argument_errors_without_launch():
         _lib.check(-8)
     assert lib.tq_workspace_bytes(0, 1, 28, 32768, 128) == 28 * 128 * 130 * 4
     assert lib.tq_workspace_bytes(2, 1, 28, 32768, 128) == 28 * 128 * 130 * 4
+    # the single-call decode steps validate descriptor, position and pointers before any launch
+    for name, desc_t in (("tq_vonly_decode_step", _lib.VOnlyCacheDesc), ("tq_packed_decode_step", _lib.PackedCacheDesc)):
+        fn, fn_at = getattr(lib, name), getattr(lib, name + "_at")
+        assert fn(None, null, 1, null, 1, null, 1, null, 1, 0, 0.1, null) == -1
+        assert fn_at(None, null, 1, null, 1, null, 1, null, 1, null, 0.1, null) == -1
+        d = desc_t()
+        d.n_seq, d.n_kv_heads, d.n_rep, d.dim, d.bits, d.t_alloc = 1, 4, 7, 128, 3, 256
+        assert fn(ctypes.byref(d), null, 1, null, 1, null, 1, null, 1, 256, 0.1, null) == -9
+        assert b"outside the storage" in lib.tq_last_error()
+        assert fn(ctypes.byref(d), null, 1, null, 1, null, 1, null, 1, 5, 0.1, null) == -1     # null storage
+        assert fn_at(ctypes.byref(d), null, 1, null, 1, null, 1, null, 1, null, 0.1, null) == -1
+        d.bits = 5
+        assert fn(ctypes.byref(d), null, 1, null, 1, null, 1, null, 1, 5, 0.1, null) == -3
+    assert lib.tq_vonly_append(null, 1, null, 9, null, b, null, null, null, null, 1, 1, 0, 0, 0, 0, 128, 3, 0, null) == -6
+    assert lib.tq_vonly_append(null, 1, null, 1, null, b, null, null, null, null, 0, 1, 0, 0, 0, 0, 128, 3, 0, null) == 0
+    assert lib.tq_vonly_append_at(null, 1, null, 1, null, b, null, null, null, null, 1, 1, 8, 128, 3, 0, null, null) == -1
 
 
 def test_kernels_refuse_cpu_tensors():
