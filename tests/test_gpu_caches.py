@@ -635,7 +635,7 @@ def test_vonly_decode_step_replayed_from_a_hip_graph(tq):
     (tq_vonly_decode_step_at) and replayed for ten tokens, with eager work and synchronisations between the
     replays: every replay matches the eager step on a twin cache and the float64 oracle, and the two caches
     end in the same state bit for bit.  An insert past the storage is dropped."""
-    B, n_q, n_kv, D, S0, N = 1, 28, 4, 128, 300, 10
+    B, n_q, n_kv, D, S0, N = 2, 28, 4, 128, 300, 10
     sc = 1 / math.sqrt(D)
     k0, v0 = rand((B, n_kv, S0, D), 900), rand((B, n_kv, S0, D), 901)
     cg, ce = tq.VOnlyTurboQuantCache(bits=3, fused=True), tq.VOnlyTurboQuantCache(bits=3, fused=True)
@@ -675,10 +675,11 @@ def test_vonly_decode_step_replayed_from_a_hip_graph(tq):
         assert torch.equal(x, y)
     st = cg.state
     vq = cg._v_tq._v_q
-    ref = o.vonly_decode_attention(host(q[0, :, 0]), st[0][0].cpu().numpy(), st[2][0].cpu().numpy().view(np.uint32),
-                                   st[3][0].cpu().numpy(), np.asarray(vq.centroids.cpu()), vq.signs.cpu().numpy(), D, 3, sc)
-    err = np.abs(host(got[0]).astype(np.float64) - ref)
-    assert (err <= 1e-3 + 2e-3 * np.abs(ref)).all(), err.max()
+    for s_ in range(B):
+        ref = o.vonly_decode_attention(host(q[s_, :, 0]), st[0][s_].cpu().numpy(), st[2][s_].cpu().numpy().view(np.uint32),
+                                       st[3][s_].cpu().numpy(), np.asarray(vq.centroids.cpu()), vq.signs.cpu().numpy(), D, 3, sc)
+        err = np.abs(host(got[s_]).astype(np.float64) - ref)
+        assert (err <= 1e-3 + 2e-3 * np.abs(ref)).all(), err.max()
     # past the storage: nothing is written, the step still runs
     before = [t.clone() for t in (cg._k_cache.keys, cg._v_tq.v_packed, cg._v_tq.v_norms)]
     pos.fill_(t_alloc)
