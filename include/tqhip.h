@@ -342,9 +342,12 @@ typedef struct tq_packed_cache_desc {
 } tq_packed_cache_desc;
 
 /*
- * One decode step of a packed cache in one library call: tq_encode of ONE new key and value row
- * per sequence and kv head at time index `position`, then tq_flash_decode_from_q (no mask, no
- * threshold) of the query token over positions 0 .. position; results identical to the three calls.
+ * One decode step of a packed cache in one library call: ONE new key and value row per sequence
+ * and kv head is encoded and stored at time index `position` and the query token attends over
+ * positions 0 .. position (no mask, no threshold).  Two launches: the packed tile pass over
+ * positions 0 .. position - 1, and a merge pass that encodes both new rows with the encoder's own
+ * arithmetic, rotates the query, scores the new key from its codes and folds both in (stored state
+ * bit-identical to tq_encode's, output equal to the separate calls up to the rounding of one score).
  * Replaces, for a single-token step, TurboQuantKVCache.update_and_fetch (cache.py:131-165) followed
  * by turboquant_attention (fused_attention.py:20-125).  Shapes and errors as tq_vonly_decode_step;
  * TQ_ERR_UNSUPPORTED where tq_flash_decode_from_q has no kernel (it needs dim 128, 3 bits, n_rep <= 16).

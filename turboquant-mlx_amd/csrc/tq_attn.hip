@@ -863,9 +863,11 @@ int launch_packed_mfma(const float* q_rot_or_weights, const uint32_t* k_packed, 
                        const float* v_centroids, const float* v_signs, void* out, void* workspace,
                        size_t workspace_bytes, const tq_decode_shape& sh, float threshold, hipStream_t stream,
                        const char* who, const void* q_raw = nullptr, int q_dtype = TQ_F32,
-                       const float* k_signs = nullptr, const int64_t* len_dev = nullptr, int64_t len_bias = 0) {
+                       const float* k_signs = nullptr, const int64_t* len_dev = nullptr, int64_t len_bias = 0,
+                       const tqm::FreshToken* fresh = nullptr) {
   const int n_q = sh.n_kv_heads * sh.n_rep;
-  const int n_tiles = (int)((sh.seq_len + tqm::kTilePos - 1) / tqm::kTilePos);
+  const int n_tiles_real = (int)((sh.seq_len + tqm::kTilePos - 1) / tqm::kTilePos);   // 0: empty cache, merge pass only (fresh)
+  const int n_tiles = n_tiles_real > 0 ? n_tiles_real : 1;
   const size_t need = (size_t)sh.n_seq * n_q * n_tiles * (tqm::kD + 2) * sizeof(float);
   if (!workspace || workspace_bytes < need)
     return tq::fail(TQ_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, need, workspace_bytes);
@@ -900,7 +902,7 @@ int launch_packed_mfma(const float* q_rot_or_weights, const uint32_t* k_packed, 
     a.n_tiles_max = (int)((sh.seq_len + tile_pos - 1) / tile_pos);
     dim3 grid(a.n_tiles_max, sh.n_kv_heads, sh.n_seq);
     tqm::packed_stream_kernel<<<grid, tqm::kSThreads, 0, stream>>>(a, kcb, vcb, n_steps);
-  } else {
+  } else if (n_tiles_real > 0) {
     dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
     tqm::packed_tile_mfma_kernel<MODE><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, kcb, vcb);
   }
@@ -908,6 +910,24 @@ int launch_packed_mfma(const float* q_rot_or_weights, const uint32_t* k_packed, 
   dim3 mgrid(n_q, sh.n_seq);
   const float inv_dim = 1.0f / (float)sh.dim;
   const int n_parts = a.n_tiles_max;
+  if (fresh) {                                             // kFlash only: the merge pass inserts the token
+#define LAUNCH_FRESH_P(TO, U_)                                                                                \
+  tqm::decode_merge_fresh_kernel<TO, U_><<<mgrid, tqm::kMergeThreads + 64, 0, stream>>>(                        \
+      a.ws_S, a.ws_ml, sh.seq_len, n_parts, sh.n_kv_heads, sh.n_rep, v_signs, inv_dim, (TO*)out, tile_pos, len_dev, *fresh)
+#define LAUNCH_FRESH_PM(TO)                                                                                   \
+  do {                                                                                                        \
+    if (n_parts <= 64) LAUNCH_FRESH_P(TO, 8);                                                                 \
+    else if (n_parts <= 128) LAUNCH_FRESH_P(TO, 16);                                                          \
+    else LAUNCH_FRESH_P(TO, 32);                                                                              \
+  } while (0)
+    if (sh.out_dtype == TQ_F16) { LAUNCH_FRESH_PM(__half); }
+    else if (sh.out_dtype == TQ_BF16) { LAUNCH_FRESH_PM(__hip_bfloat16); }
+    else { LAUNCH_FRESH_PM(float); }
+#undef LAUNCH_FRESH_PM
+#undef LAUNCH_FRESH_P
+    TQ_CHECK_LAUNCH(who);
+    return TQ_OK;
+  }
 #define LAUNCH_MERGE_P(TO)                                                                                    \
   tqm::decode_merge_rows_kernel<TO, MODE == tqm::kFlash><<<mgrid, tqm::kMergeThreads, 0, stream>>>(            \
       a.ws_S, a.ws_ml, sh.seq_offsets, sh.seq_len, n_parts, sh.n_kv_heads, sh.n_rep, v_signs, inv_dim, (TO*)out, tile_pos, \
@@ -1440,6 +1460,30 @@ int packed_step(const tq_packed_cache_desc* c, const void* k_new, int k_dtype, c
       !tq::aligned(c->k_signs, 4) || !tq::aligned(c->v_signs, 4) || !tq::aligned(c->k_packed, 4) ||
       !tq::aligned(c->v_packed, 4) || !tq::aligned(c->k_norms, 4) || !tq::aligned(c->v_norms, 4))
     return tq::fail(TQ_ERR_ALIGN, "%s: misaligned pointer", who);
+  if (q && out && !tq::check_dtype(q_dtype) && !tq::check_dtype(out_dtype) && tq::aligned(q, (int)tq::dtype_size(q_dtype)) &&
+      (!position_dev || tq::aligned(position_dev, 8)) && c->n_seq <= 65535 && c->n_kv_heads <= 65535) {
+    // two launches: the tile pass over the positions before the new one, and a merge pass that encodes both new
+    // rows, scores the new key and stores them (tqm::FreshToken with packed keys)
+    tqm::FreshToken f{};
+    f.k_new = k_new; f.v_new = v_new; f.q = q;
+    f.v_packed = c->v_packed; f.v_norms = c->v_norms; f.k_packed = c->k_packed; f.k_norms = c->k_norms;
+    f.k_signs = c->k_signs;
+    f.pos_dev = position_dev; f.pos = position; f.t_alloc = c->t_alloc;
+    tq::encode_thresholds(c->boundaries, c->dim, c->bits, c->variant, f.thr);
+    for (int i = 0; i < 8; ++i) f.cent[i] = c->centroids[i];
+    f.cs = attn_scale * tqm::kLog2e;
+    f.k_dtype = k_dtype; f.v_dtype = v_dtype; f.q_dtype = q_dtype;
+    tq_decode_shape fs{};
+    fs.n_seq = c->n_seq; fs.n_kv_heads = c->n_kv_heads; fs.n_rep = c->n_rep; fs.dim = c->dim; fs.bits = c->bits;
+    fs.block_size = 16;
+    fs.seq_len = position_dev ? c->t_alloc : position;     // positions before the new one (device: upper bound)
+    fs.k_head_stride = fs.kn_head_stride = fs.v_head_stride = fs.vn_head_stride = c->t_alloc;
+    fs.k_seq_stride = fs.kn_seq_stride = fs.v_seq_stride = fs.vn_seq_stride = c->t_alloc * c->n_kv_heads;
+    fs.attn_scale = attn_scale; fs.out_dtype = out_dtype; fs.allow_mma = 1;
+    return launch_packed_mfma<tqm::kFlash>(nullptr, c->k_packed, c->k_norms, c->v_packed, c->v_norms, c->centroids,
+                                           c->centroids, c->v_signs, out, c->workspace, c->workspace_bytes, fs, 0.0f,
+                                           (hipStream_t)stream_, who, q, q_dtype, c->k_signs, position_dev, 0, &f);
+  }
   if (int rc = tq::encode_pair(k_new, k_dtype, c->k_signs, c->k_packed + position * pdim, c->k_norms + position, v_new,
                                v_dtype, c->v_signs, c->v_packed + position * pdim, c->v_norms + position, c->boundaries,
                                groups, c->t_alloc, c->variant, stream_, position_dev))

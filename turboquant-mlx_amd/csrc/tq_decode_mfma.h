@@ -1053,6 +1053,12 @@ struct FreshToken {
   float cent[8];
   float cs;                   // attn_scale * log2 e
   int32_t k_dtype, v_dtype, q_dtype;
+  // Cache with packed keys (k_packed set; k_f16 / v_raw unused): the new key row is encoded as well (signs
+  // k_signs, same thresholds and centroids), the query is rotated (raw butterfly of q * k_signs) and the
+  // score is sum_e c[idx_k[e]] * q_rot[e] * k_norm / dim, as the packed tile pass takes it.
+  const float* k_signs;
+  uint32_t* k_packed;
+  float* k_norms;
 };
 
 __device__ __forceinline__ float load_any(const void* p, int dtype, int64_t at) {
@@ -1093,8 +1099,8 @@ __device__ __forceinline__ void merge_rows_body(
   bool fresh_wave = false;
   if constexpr (FRESH) fresh_wave = tid >= 256;
   // what the wavefront of the inserted token keeps for its stores, which wait until the fold is under way
-  float x[2] = {0.f, 0.f}, kx[2] = {0.f, 0.f}, fresh_nrm = 0.0f;
-  int idx[2] = {0, 0};
+  float x[2] = {0.f, 0.f}, kx[2] = {0.f, 0.f}, fresh_nrm = 0.0f, fresh_knrm = 0.0f;
+  int idx[2] = {0, 0}, kidx[2] = {0, 0};
   int64_t fresh_row = -1;
   if constexpr (FRESH) { if (fresh_wave) {
     // ---- the inserted token (one wavefront) ------------------------------------------------------------
@@ -1107,10 +1113,13 @@ __device__ __forceinline__ void merge_rows_body(
     for (int i = 0; i < 2; ++i) {
       const int e = lane + 64 * i;
       x[i] = load_any(f.v_new, f.v_dtype, src + e);
-      kx[i] = __half2float(__float2half_rn(load_any(f.k_new, f.k_dtype, src + e)));
+      kx[i] = load_any(f.k_new, f.k_dtype, src + e);
+      if (!f.k_packed) kx[i] = __half2float(__float2half_rn(kx[i]));
       qx[i] = load_any(f.q, f.q_dtype, ((int64_t)seq * gridDim.x + head) * kD + e);
       sq[i] = x[i] * x[i];
     }
+    float ksg[2] = {0.f, 0.f};
+    if (f.k_packed) { ksg[0] = f.k_signs[lane]; ksg[1] = f.k_signs[lane + 64]; }
     const float ss = tree_sum<kD>(sq);
     const float nrm = sqrtf(ss);
     const float safe = fmaxf(nrm, 1e-8f);
@@ -1129,9 +1138,37 @@ __device__ __forceinline__ void merge_rows_body(
       for (int k = 1; k < 8; ++k) c = (n == (uint32_t)k) ? f.cent[k] : c;
       acc_s[8][lane + 64 * i] = nrm * c;
     }
-    float d = qx[0] * kx[0] + qx[1] * kx[1];
+    float d;
+    if (f.k_packed) {
+      float ksq[2] = {kx[0] * kx[0], kx[1] * kx[1]};
+      const float kss = tree_sum<kD>(ksq);
+      const float knrm = sqrtf(kss);
+      const float ksafe = fmaxf(knrm, 1e-8f);
+      float kv[2] = {(kx[0] / ksafe) * ksg[0], (kx[1] / ksafe) * ksg[1]};
+      raw_butterfly<kD>(kv, lane);
+      float qr[2] = {qx[0] * ksg[0], qx[1] * ksg[1]};
+      raw_butterfly<kD>(qr, lane);
+      fresh_knrm = knrm;
+      d = 0.0f;
 #pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) d += shfl_xor_f(d, m);
+      for (int i = 0; i < 2; ++i) {
+        uint32_t n = 0;
+#pragma unroll
+        for (int b = 0; b < 7; ++b) n += (kv[i] > f.thr[b]) ? 1u : 0u;
+        kidx[i] = (int)n;
+        float c = f.cent[0];
+#pragma unroll
+        for (int k = 1; k < 8; ++k) c = (n == (uint32_t)k) ? f.cent[k] : c;
+        d += c * qr[i];
+      }
+#pragma unroll
+      for (int m = 32; m >= 1; m >>= 1) d += shfl_xor_f(d, m);
+      d = (d * knrm) * inv_dim;
+    } else {
+      d = qx[0] * kx[0] + qx[1] * kx[1];
+#pragma unroll
+      for (int m = 32; m >= 1; m >>= 1) d += shfl_xor_f(d, m);
+    }
     if (lane == 0) {
       ml_s[8][0] = ok ? d * f.cs : -INFINITY;
       ml_s[8][1] = 1.0f;
@@ -1174,18 +1211,27 @@ __device__ __forceinline__ void merge_rows_body(
   if constexpr (FRESH) { if (fresh_wave) {
     // packed word `lane` holds elements 10 * lane .. 10 * lane + 9 (3-bit fields, lowest first)
     const FreshToken& f = *ft;
-    uint32_t word = 0;
+    uint32_t word = 0, kword = 0;
 #pragma unroll
     for (int i = 0; i < 10; ++i) {
       const int e = min(10 * lane + i, kD - 1);
       const int lo = __shfl(idx[0], e & 63), hi = __shfl(idx[1], e & 63);
       const uint32_t fld = (uint32_t)((e >> 6) ? hi : lo);
       if (10 * lane + i < kD) word |= fld << (3 * i);
+      if (f.k_packed) {
+        const int klo = __shfl(kidx[0], e & 63), khi = __shfl(kidx[1], e & 63);
+        const uint32_t kfld = (uint32_t)((e >> 6) ? khi : klo);
+        if (10 * lane + i < kD) kword |= kfld << (3 * i);
+      }
     }
     if (fresh_row >= 0) {                                  // first query head of the kv head, position inside the storage
       const int64_t row = fresh_row;
       if (lane < kPdim) f.v_packed[row * kPdim + lane] = word;
       if (lane == 0) f.v_norms[row] = fresh_nrm;
+      if (f.k_packed) {
+        if (lane < kPdim) f.k_packed[row * kPdim + lane] = kword;
+        if (lane == 0) f.k_norms[row] = fresh_knrm;
+      } else {
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         const int e = lane + 64 * i;
@@ -1195,6 +1241,7 @@ __device__ __forceinline__ void merge_rows_body(
           else if (f.v_dtype == TQ_F16) ((__half*)f.v_raw)[row * kD + e] = __float2half_rn(x[i]);
           else ((__hip_bfloat16*)f.v_raw)[row * kD + e] = __float2bfloat16(x[i]);
         }
+      }
       }
     }
   } }
