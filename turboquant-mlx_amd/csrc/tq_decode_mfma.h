@@ -1061,10 +1061,19 @@ struct FreshToken {
   float* k_norms;
 };
 
-__device__ __forceinline__ float load_any(const void* p, int dtype, int64_t at) {
-  if (dtype == TQ_F16) return __half2float(((const __half*)p)[at]);
-  if (dtype == TQ_F32) return ((const float*)p)[at];
-  return __bfloat162float(((const __hip_bfloat16*)p)[at]);
+// An element of a tensor whose dtype is a run-time value, in two steps so that a wavefront can have the loads of
+// several such tensors in flight together: the raw bits first (one uniform branch on the element size, no use of
+// the value), the conversion (selects, no branch) once everything has been requested.
+__device__ __forceinline__ uint32_t load_raw(const void* p, int dtype, int64_t at) {
+  if (dtype == TQ_F32) return ((const uint32_t*)p)[at];
+  return ((const uint16_t*)p)[at];
+}
+__device__ __forceinline__ float raw_to_float(uint32_t raw, int dtype) {
+  const float f32 = __uint_as_float(raw);
+  const float bf = __uint_as_float(raw << 16);
+  const unsigned short hbits = (unsigned short)(raw & 0xFFFFu);
+  const float f16 = __half2float(__ushort_as_half(hbits));
+  return dtype == TQ_F32 ? f32 : (dtype == TQ_F16 ? f16 : bf);
 }
 
 // Merge pass: grid = (n_q, n_seq), 256 threads (320 with FRESH).  Lane group ph = tid / 32 folds tiles ph, ph + 8, ...
@@ -1109,17 +1118,21 @@ __device__ __forceinline__ void merge_rows_body(
     const bool ok = pos >= 0 && pos < f.t_alloc;
     const int64_t src = grp * kD;
     float qx[2], sq[2];
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int e = lane + 64 * i;
-      x[i] = load_any(f.v_new, f.v_dtype, src + e);
-      kx[i] = load_any(f.k_new, f.k_dtype, src + e);
-      if (!f.k_packed) kx[i] = __half2float(__float2half_rn(kx[i]));
-      qx[i] = load_any(f.q, f.q_dtype, ((int64_t)seq * gridDim.x + head) * kD + e);
-      sq[i] = x[i] * x[i];
-    }
+    uint32_t rv[2], rk[2], rq[2];
+    const int64_t qsrc = ((int64_t)seq * gridDim.x + head) * kD;
+    rv[0] = load_raw(f.v_new, f.v_dtype, src + lane); rv[1] = load_raw(f.v_new, f.v_dtype, src + lane + 64);
+    rk[0] = load_raw(f.k_new, f.k_dtype, src + lane); rk[1] = load_raw(f.k_new, f.k_dtype, src + lane + 64);
+    rq[0] = load_raw(f.q, f.q_dtype, qsrc + lane); rq[1] = load_raw(f.q, f.q_dtype, qsrc + lane + 64);
     float ksg[2] = {0.f, 0.f};
     if (f.k_packed) { ksg[0] = f.k_signs[lane]; ksg[1] = f.k_signs[lane + 64]; }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      x[i] = raw_to_float(rv[i], f.v_dtype);
+      kx[i] = raw_to_float(rk[i], f.k_dtype);
+      if (!f.k_packed) kx[i] = __half2float(__float2half_rn(kx[i]));
+      qx[i] = raw_to_float(rq[i], f.q_dtype);
+      sq[i] = x[i] * x[i];
+    }
     const float ss = tree_sum<kD>(sq);
     const float nrm = sqrtf(ss);
     const float safe = fmaxf(nrm, 1e-8f);
