@@ -829,3 +829,28 @@ def test_packed_decode_step_from_an_empty_cache_and_at_a_tile_boundary(tq, dtype
             err = np.abs(host(got[s_, :, 0]).astype(np.float64) - ref)
             assert (err <= 1e-3 + 2e-3 * np.abs(ref)).all(), (a.offset, err.max())
     assert a.offset == 513
+
+
+def test_vonly_append_with_a_device_side_position(tq):
+    """tq_vonly_append_at: three tokens inserted at a position held in device memory give the storage of the
+    host-position call bit for bit; rows that would land past the storage are dropped, the others kept."""
+    from tqhip import ops
+    B, H, T, S, D = 2, 3, 64, 3, 128
+    sg = o.random_diagonal_sign(D, 43)
+    signs = torch.from_numpy(sg).cuda()
+    c = o.gaussian_codebook(3)
+    bnd = o.gaussian_boundaries(c)
+    k, v = rand((B, H, S, D), 1400, torch.bfloat16), rand((B, H, S, D), 1401)
+
+    def storage():
+        return (torch.zeros((B, H, T, D), dtype=torch.float16, device="cuda"), torch.zeros((B, H, T, D), dtype=torch.float16, device="cuda"),
+                torch.zeros((B, H, T, 13), dtype=torch.int32, device="cuda").view(torch.uint32), torch.zeros((B, H, T), device="cuda"))
+    for pos in (17, T - 2):
+        a, b = storage(), storage()
+        n_fit = min(S, T - pos)
+        ops.vonly_append_into(k[:, :, :n_fit], v[:, :, :n_fit], signs, bnd, a[0], a[1], a[2], a[3], position=pos, bits=3)
+        ops.vonly_append_into(k, v, signs, bnd, b[0], b[1], b[2], b[3],
+                              position=torch.tensor([pos], dtype=torch.int64, device="cuda"), bits=3)
+        for x, y in zip(a, b):
+            assert torch.equal(x, y), pos
+        assert float(a[3][:, :, pos:pos + n_fit].min()) > 0.0

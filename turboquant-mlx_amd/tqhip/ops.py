@@ -179,7 +179,7 @@ def encode_into(x: torch.Tensor, signs: torch.Tensor, boundaries, packed: torch.
 
 def vonly_append_into(keys: torch.Tensor, values: torch.Tensor, signs: torch.Tensor, boundaries,
                       k_f16: torch.Tensor, v_raw, v_packed: torch.Tensor, v_norms: torch.Tensor, *,
-                      position: int, bits: int, variant: str = "mlx") -> None:
+                      position, bits: int, variant: str = "mlx") -> None:
     """Insert the S new tokens `keys`, `values` [B, H, S, D] at time index `position` of a cache with
     float16 keys `k_f16` [B, H, T_alloc, D], optional unencoded values `v_raw` (same dtype as
     `values`, or None) and packed values `v_packed` [B, H, T_alloc, pdim] / `v_norms` [B, H, T_alloc]
@@ -187,6 +187,15 @@ def vonly_append_into(keys: torch.Tensor, values: torch.Tensor, signs: torch.Ten
     VOnlyTurboQuantCache.update_and_fetch (v_only_cache.py:52-53)."""
     _need_gpu(keys, values, signs, k_f16, v_packed, v_norms)
     B, H, S, D = values.shape
+    on_device = isinstance(position, torch.Tensor)
+    if on_device:
+        # tq_vonly_append_at: the position is read on the GPU when the kernel runs (one-element int64 tensor); all
+        # four tensors must then hold the same number of positions, and rows past the storage are dropped
+        if position.dtype != torch.int64 or position.numel() != 1 or not position.is_cuda:
+            raise ValueError("a device-side position must be a one-element int64 tensor on the GPU")
+        pos_dev, position = position, 0
+        if len({k_f16.shape[2], v_packed.shape[2], v_norms.shape[2]} | ({v_raw.shape[2]} if v_raw is not None else set())) != 1:
+            raise ValueError("a device-side position needs key, value, packed and norm storage of one length")
     if keys.shape != values.shape:
         raise ValueError(f"keys {tuple(keys.shape)} and values {tuple(values.shape)} must have one shape")
     if k_f16.dtype != torch.float16 or not k_f16.is_contiguous():
@@ -204,6 +213,12 @@ def vonly_append_into(keys: torch.Tensor, values: torch.Tensor, signs: torch.Ten
     pd = packed_dim(D, bits)
     var = {"mlx": _lib.TQ_ENCODE_MLX, "metal": _lib.TQ_ENCODE_METAL}[variant]
     lib = _lib.load()
+    if on_device:
+        _lib.check(lib.tq_vonly_append_at(
+            _ptr(keys), _dt(keys), _ptr(values), _dt(values), _ptr(signs), _host_table(boundaries),
+            _ptr(k_f16), _ptr(v_raw), _ptr(v_packed), _ptr(v_norms), B * H, S, k_f16.shape[2], D, bits, var,
+            _ptr(pos_dev), _stream(values)))
+        return
     _lib.check(lib.tq_vonly_append(
         _ptr(keys), _dt(keys), _ptr(values), _dt(values), _ptr(signs), _host_table(boundaries),
         C.c_void_p(k_f16.data_ptr() + position * D * 2),
