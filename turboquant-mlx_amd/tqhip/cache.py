@@ -217,7 +217,7 @@ class TurboQuantKVCache:
         H = values.shape[1]
         ok = (not self.v_only and S_q == 1 and values.shape[2] == 1 and keys.shape == values.shape
               and keys.shape[3] == dim and n_q % H == 0 and values.is_cuda
-              and queries.dtype in (torch.float16, torch.bfloat16, torch.float32)
+              and queries.dtype in ops._DTYPES and keys.dtype in ops._DTYPES and values.dtype in ops._DTYPES
               and ops.vonly_sparse_supported(dim, self.quant_bits, n_q // H))
         if ok:
             self._dtype = keys.dtype
@@ -240,10 +240,22 @@ class TurboQuantKVCache:
                                  "n_rep <= 16 and contiguous storage")
             self.update_and_fetch(keys, values)
             return attention.turboquant_attention(queries, self, attn_scale, fused=True)
-        out = ops.packed_decode_step(self._step, keys[:, :, 0, :], values[:, :, 0, :], queries[:, :, 0, :],
-                                     self.offset if position is None else position, attn_scale, out=out)
+        if position is not None and (position.dtype != torch.int64 or position.numel() != 1 or not position.is_cuda):
+            raise ValueError("a device-side position must be a one-element int64 tensor on the GPU")
+        sb, sh_, _, sd = self._step.shape
+        if (sb, sh_, sd) != (B, H, dim) or values.shape[0] != B or not (queries.is_cuda and keys.is_cuda):
+            raise ValueError(f"the cache stores {sb} x {sh_} groups of dim {sd} on the GPU; got queries {tuple(queries.shape)}, "
+                             f"keys {tuple(keys.shape)} on {keys.device}")
+        if out is None:
+            res = torch.empty((B, n_q, 1, dim), dtype=queries.dtype, device=queries.device)
+        elif out.numel() != B * n_q * dim or not out.is_contiguous() or not out.is_cuda or out.dtype not in ops._DTYPES:
+            raise ValueError(f"out must be a contiguous GPU tensor of {B} x {n_q} x {dim} elements")
+        else:
+            res = out
+        ops.step_call_unchecked(self._step, keys.contiguous(), values.contiguous(), queries.contiguous(),
+                                self.offset if position is None else position, attn_scale, res, packed=True)
         self.offset += 1          # _deq_offset stays behind: the next unfused fetch dequantises the whole cache
-        return out[:, :, None, :]
+        return res if res.dim() == 4 else res[:, :, None, :]
 
     def update_and_fetch(self, keys: torch.Tensor, values: torch.Tensor):
         B, H, S, k_dim = keys.shape

@@ -808,6 +808,26 @@ def vonly_decode_step(step: VOnlyStep, keys: torch.Tensor, values: torch.Tensor,
     return out
 
 
+def step_call_unchecked(step, keys: torch.Tensor, values: torch.Tensor, q: torch.Tensor, position, attn_scale: float,
+                        out: torch.Tensor, packed: bool) -> None:
+    """The library call of vonly_decode_step / packed_decode_step without their argument checks, for the cache
+    objects, which have established shapes, dtypes and devices themselves: keys / values / q / out are contiguous
+    and hold (B, heads, dim) elements in any view of that memory (a (B, heads, 1, dim) tensor qualifies)."""
+    stream = _stream(q)
+    ws = _workspace(q.device, stream.value or 0, step._need)
+    d = step.desc
+    d.workspace, d.workspace_bytes = ws.data_ptr(), ws.numel()
+    lib = _lib.load()
+    if isinstance(position, torch.Tensor):
+        fn = lib.tq_packed_decode_step_at if packed else lib.tq_vonly_decode_step_at
+        pos = C.c_void_p(position.data_ptr())
+    else:
+        fn = lib.tq_packed_decode_step if packed else lib.tq_vonly_decode_step
+        pos = position
+    _lib.check(fn(step._ref, keys.data_ptr(), _DTYPES[keys.dtype], values.data_ptr(), _DTYPES[values.dtype],
+                  q.data_ptr(), _DTYPES[q.dtype], out.data_ptr(), _DTYPES[out.dtype], pos, attn_scale, stream))
+
+
 def _fill_table(dst, values, n, what):
     vals = [float(x) for x in (values.tolist() if isinstance(values, torch.Tensor) else values)]
     if len(vals) != n:

@@ -103,7 +103,7 @@ class VOnlyTurboQuantCache:
         B, n_q, S_q, dim = queries.shape
         H = values.shape[1]
         if (S_q != 1 or values.shape[2] != 1 or keys.shape != values.shape or n_q % H or not values.is_cuda
-                or queries.dtype not in (torch.float16, torch.bfloat16, torch.float32)
+                or queries.dtype not in ops._DTYPES or keys.dtype not in ops._DTYPES or values.dtype not in ops._DTYPES
                 or (kc.values is not None and kc.values.dtype != values.dtype)
                 or (kc.keys is not None and kc.keys.dtype != torch.float16) or kc.offset != tq.offset):
             if position is not None:
@@ -128,11 +128,23 @@ class VOnlyTurboQuantCache:
                 self.update_and_fetch(keys, values)
                 return attention.vonly_decode_attention(queries, self, attn_scale)
             self._step_key = key
-        out = ops.vonly_decode_step(self._step, keys[:, :, 0, :], values[:, :, 0, :], queries[:, :, 0, :],
-                                    kc.offset if position is None else position, attn_scale, out=out)
+        if position is not None and (position.dtype != torch.int64 or position.numel() != 1 or not position.is_cuda):
+            raise ValueError("a device-side position must be a one-element int64 tensor on the GPU")
+        sb, sh_, _, sd = self._step.shape
+        if (sb, sh_, sd) != (B, H, dim) or values.shape[0] != B or not (queries.is_cuda and keys.is_cuda):
+            raise ValueError(f"the cache stores {sb} x {sh_} groups of dim {sd} on the GPU; got queries {tuple(queries.shape)}, "
+                             f"keys {tuple(keys.shape)} on {keys.device}")
+        if out is None:
+            res = torch.empty((B, n_q, 1, dim), dtype=queries.dtype, device=queries.device)
+        elif out.numel() != B * n_q * dim or not out.is_contiguous() or not out.is_cuda or out.dtype not in ops._DTYPES:
+            raise ValueError(f"out must be a contiguous GPU tensor of {B} x {n_q} x {dim} elements")
+        else:
+            res = out
+        ops.step_call_unchecked(self._step, keys.contiguous(), values.contiguous(), queries.contiguous(),
+                                kc.offset if position is None else position, attn_scale, res, packed=False)
         kc.offset += 1
         tq.offset += 1
-        return out[:, :, None, :]
+        return res if res.dim() == 4 else res[:, :, None, :]
 
     def dequantized_values(self, dtype=None) -> torch.Tensor:
         """All cached values, dequantised: [B, H, offset, D]."""
