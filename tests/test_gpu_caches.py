@@ -854,3 +854,29 @@ def test_vonly_append_with_a_device_side_position(tq):
         for x, y in zip(a, b):
             assert torch.equal(x, y), pos
         assert float(a[3][:, :, pos:pos + n_fit].min()) > 0.0
+
+
+def test_decode_step_after_from_state_and_trim(tq):
+    """decode_step on caches rebuilt with from_state (storage handed in as slices, possibly of unequal
+    allocated lengths) and after trim: same state as the two calls, output within the bar."""
+    B, n_q, n_kv, D, S0 = 1, 8, 2, 128, 300
+    sc = 1 / math.sqrt(D)
+    k0, v0 = rand((B, n_kv, S0, D), 1500), rand((B, n_kv, S0, D), 1501)
+    for make, attend in ((lambda: tq.VOnlyTurboQuantCache(bits=3, fused=True), tq.vonly_decode_attention),
+                         (lambda: tq.TurboQuantKVCache(bits=3, fused=True), lambda q, c, s: tq.turboquant_attention(q, c, s, fused=True))):
+        src = make()
+        src.update_and_fetch(k0, v0)
+        a = type(src).from_state(src.state, src.meta_state)
+        b = type(src).from_state(src.state, src.meta_state)
+        a.fused = b.fused = True
+        a.trim(7), b.trim(7)
+        for i in range(3):
+            k1, v1, q1 = rand((B, n_kv, 1, D), 1510 + 3 * i), rand((B, n_kv, 1, D), 1511 + 3 * i), rand((B, n_q, 1, D), 1512 + 3 * i)
+            got = a.decode_step(q1, k1, v1, sc)
+            b.update_and_fetch(k1, v1)
+            want = attend(q1, b, sc)
+            err = (got.float() - want.float()).abs()
+            assert bool((err <= 1e-3 + 2e-3 * want.float().abs()).all()), float(err.max())
+        assert a.offset == b.offset == S0 - 7 + 3
+        for x, y in zip(a.state, b.state):
+            assert torch.equal(x, y)
