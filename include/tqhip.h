@@ -258,6 +258,26 @@ int tq_vonly_decode_attn(const void* q, int q_dtype, const void* k_f16,
                          const tq_decode_shape* shape /* host */, tq_stream_t stream);
 
 /*
+ * tq_vonly_decode_attn without a workspace argument and without any allocation.  No counterpart in the
+ * reference (its runtime allocates every kernel output, e.g. sparse_v.py:169-185): this entry point is for
+ * callers that cannot allocate device memory -- code under HIP-graph capture, tight serving loops,
+ * harnesses that forbid it.  The per-tile partial sums that tq_vonly_decode_attn keeps in the caller's
+ * workspace go to an array of TQ_STATIC_SCRATCH_BYTES bytes inside the library (one copy per GPU, held
+ * until the process ends; its address is looked up on the first call on a device, so make that call
+ * outside a capture).  Arguments, kernels and results are those of tq_vonly_decode_attn (bit-identical
+ * output).  Fails with TQ_ERR_WORKSPACE when tq_workspace_bytes(TQ_OP_VONLY_DECODE, n_seq, n_q_heads,
+ * seq_len, dim) exceeds TQ_STATIC_SCRATCH_BYTES (e.g. more than 8065 tiles of 256 positions x query heads
+ * at dim 128).  Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two
+ * streams, two threads) race; order them on one stream.  Nothing in the array has to be cleared
+ * between calls -- every partial that a call's merge pass reads has been written by its tile pass.
+ */
+#define TQ_STATIC_SCRATCH_BYTES ((size_t)4 << 20)
+int tq_vonly_decode_attn_static(const void* q, int q_dtype, const void* k_f16,
+                                const uint32_t* v_packed, const float* v_norms,
+                                const float* v_centroids, const float* v_signs,
+                                void* out, const tq_decode_shape* shape /* host */, tq_stream_t stream);
+
+/*
  * A V-only cache as the library sees it between two growths of its storage: what a caller fills in
  * once and reuses for every decode step (all four tensors share n_seq, n_kv_heads and t_alloc).
  */

@@ -1257,6 +1257,51 @@ extern "C" int tq_vonly_decode_attn(const void* q, int q_dtype, const void* k_f1
                                      workspace_bytes, shape, 3, stream_);
 }
 
+// ---- the entry point that allocates nothing -------------------------------------------------------------
+// Per-tile partial sums of tq_vonly_decode_attn_static live in this array instead of a caller's workspace.
+// Every GPU the library runs on holds its own copy at its own address until the process ends; in host code
+// the array's name is only a handle for hipGetSymbolAddress, never a device address.
+constexpr size_t kStaticScratchBytes = TQ_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices];      // device address of `scratch` per device ordinal, resolved once
+std::mutex g_scratch_mutex;
+
+// Device address of `scratch` on the current device: hipGetSymbolAddress on the first call per device.
+int static_scratch(void** ptr, const char* who) {
+  int dev = -1;
+  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return tq::hip_fail(e, who);
+  if (dev < 0 || dev >= kMaxDevices) return tq::fail(TQ_ERR_ARG, "%s: device ordinal %d outside 0..%d", who, dev, kMaxDevices - 1);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    if (hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)); e != hipSuccess) return tq::hip_fail(e, who);
+    if (!p) return tq::fail(TQ_ERR_HIP, "%s: hipGetSymbolAddress returned a null address", who);
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr = g_scratch_ptr[dev];
+  return TQ_OK;
+}
+}  // namespace
+
+extern "C" int tq_vonly_decode_attn_static(const void* q, int q_dtype, const void* k_f16, const uint32_t* v_packed,
+                                           const float* v_norms, const float* v_centroids, const float* v_signs,
+                                           void* out, const tq_decode_shape* shape, tq_stream_t stream_) {
+  const char* who = "tq_vonly_decode_attn_static";
+  if (int rc = check_shape(shape, who, 256)) return rc;
+  const size_t need = ws_bytes(shape->n_seq, shape->n_kv_heads * shape->n_rep, shape->seq_len, shape->dim);
+  if (need > kStaticScratchBytes)
+    return tq::fail(TQ_ERR_WORKSPACE,
+                    "%s: this shape needs %zu bytes of per-tile partial sums, the static scratch holds %zu; "
+                    "call tq_vonly_decode_attn with a workspace instead", who, need, kStaticScratchBytes);
+  void* ptr = nullptr;
+  if (int rc = static_scratch(&ptr, who)) return rc;
+  return tq_vonly_decode_attn_phases(q, q_dtype, k_f16, v_packed, v_norms, v_centroids, v_signs, out, ptr,
+                                     kStaticScratchBytes, shape, 3, stream_);
+}
+
 namespace {
 constexpr int kNotFused = 1;   // not an error: the caller takes the append + attention route
 

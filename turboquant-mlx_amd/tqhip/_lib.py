@@ -77,6 +77,7 @@ PROTOTYPES = {
     "tq_flash_decode": (_i, [_p, _p, _p, _p, _p, _fp, _fp, _p, _p, _p, _z, C.POINTER(DecodeShape), _p]),
     "tq_flash_decode_plan": (_i, [_i, _i, _l, _i, _i]),
     "tq_vonly_decode_attn": (_i, [_p, _i, _p, _p, _p, _fp, _p, _p, _p, _z, C.POINTER(DecodeShape), _p]),
+    "tq_vonly_decode_attn_static": (_i, [_p, _i, _p, _p, _p, _fp, _p, _p, C.POINTER(DecodeShape), _p]),
     "tq_vonly_decode_step": (_i, [C.POINTER(VOnlyCacheDesc), _p, _i, _p, _i, _p, _i, _p, _i, _l, _f, _p]),
     "tq_packed_decode_step": (_i, [C.POINTER(PackedCacheDesc), _p, _i, _p, _i, _p, _i, _p, _i, _l, _f, _p]),
     "tq_vonly_append_at": (_i, [_p, _i, _p, _i, _p, _fp, _p, _p, _p, _p, _l, _l, _l, _i, _i, _i, _p, _p]),
@@ -118,6 +119,7 @@ def load():
 # (sparse_v.py:147-157, flash_attention.py:224-234, metal_kernels_v4.py:138-139,188-191,
 #  quantizer.py:37-38)
 _VALUE_ERRORS = {-2, -3, -4, -7, -9}
+STATIC_SCRATCH_BYTES = 4 << 20     # TQ_STATIC_SCRATCH_BYTES of include/tqhip.h
 
 
 def check(status: int) -> None:

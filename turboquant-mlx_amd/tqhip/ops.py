@@ -656,7 +656,8 @@ def vonly_sparse_supported(dim: int, bits: int, n_rep: int) -> bool:
 def vonly_decode(q: torch.Tensor, k: torch.Tensor, v_packed, v_norms, v_centroids, v_signs, dim: int,
                  bits: int, attn_scale: float, *, n_rep: int = 1, seq_len: int | None = None,
                  seq_offsets: torch.Tensor | None = None, max_seq_len: int | None = None, mask=None,
-                 out_dtype=torch.float32, precision: str = "fp16", sparse_v_threshold: float = 0.0) -> torch.Tensor:
+                 out_dtype=torch.float32, precision: str = "fp16", sparse_v_threshold: float = 0.0,
+                 out: torch.Tensor | None = None, static_scratch: bool = False) -> torch.Tensor:
     """Dense-softmax decode attention over fp16 keys and packed values (tq_vonly_decode_attn).
     precision as in flash_decode (on the matrix-core path fp16 queries enter as they are, bf16 converted to
     fp16, float32 as an fp16 value plus the fp16 remainder of that rounding).
@@ -664,6 +665,12 @@ def vonly_decode(q: torch.Tensor, k: torch.Tensor, v_packed, v_norms, v_centroid
     sparse_v_threshold > 0: softmax weights below it are dropped from the value sum (threshold rule of
     sparse_v.py:59-65 on the final weights, as in hybrid_attention.py:52-88) -- tq_vonly_sparse_decode_attn,
     matrix-core shape only (see vonly_sparse_supported).
+
+    out: a contiguous (n_seq, n_q, dim) tensor to write into (its dtype is the output dtype) instead of a new one.
+    static_scratch=True takes tq_vonly_decode_attn_static: the per-tile partial sums go to an array inside the
+    library instead of a torch workspace, so with `out` given and inputs already in the kernel's layout the call
+    allocates no device memory (for callers under HIP-graph capture or in loops that must not allocate); shapes
+    whose partial sums exceed that array raise, and calls that overlap on one GPU would race on it.
 
     q (n_seq, n_q, dim) fp16/bf16/fp32; k [n_seq, n_kv, T_alloc, dim] or ragged [n_kv, sum(L), dim] fp16;
     V as in flash_decode.  Returns (n_seq, n_q, dim) `out_dtype`.
@@ -691,13 +698,26 @@ def vonly_decode(q: torch.Tensor, k: torch.Tensor, v_packed, v_norms, v_centroid
     _check_rows(T, ragged, n_seq, k=k, v_packed=v_packed, v_norms=v_norms)
     v_signs = _as_f32_dev(v_signs, q)
     mask, ms = _mask_layout(mask, n_seq, n_q, T, q.device)
-    out = torch.empty((n_seq, n_q, dim), dtype=out_dtype, device=q.device)
+    if out is None:
+        out = torch.empty((n_seq, n_q, dim), dtype=out_dtype, device=q.device)
+    else:
+        _need_gpu(out)
+        if tuple(out.shape) != (n_seq, n_q, dim) or not out.is_contiguous() or out.dtype not in _DTYPES:
+            raise ValueError(f"out must be a contiguous ({n_seq}, {n_q}, {dim}) float32/float16/bfloat16 tensor")
+        out_dtype = out.dtype
     sh = _decode_shape(n_seq=n_seq, n_kv=n_kv, n_rep=n_rep, dim=dim, bits=bits, block_size=16, seq_len=T,
                        seq_offsets=seq_offsets, k_strides=ks, kn_strides=(0, 0), v_strides=vs, vn_strides=vns,
                        mask=mask, mask_strides=ms, attn_scale=attn_scale, out_dtype=out_dtype,
                        allow_mma=bool(_mma_flag(precision)))
     lib = _lib.load()
     stream = _stream(q)
+    if static_scratch:
+        if sparse_v_threshold and sparse_v_threshold > 0.0:
+            raise ValueError("static_scratch serves the dense step only (sparse_v_threshold = 0)")
+        _lib.check(lib.tq_vonly_decode_attn_static(
+            _ptr(q), _dt(q), _ptr(k), _ptr(v_packed), _ptr(v_norms), _host_table(v_centroids), _ptr(v_signs),
+            _ptr(out), C.byref(sh), stream))
+        return out
     if sparse_v_threshold and sparse_v_threshold > 0.0:
         if not (vonly_sparse_supported(dim, bits, n_rep) and T > 0):
             raise ValueError("thresholded V-only decode needs dim 128, 3-bit values, n_rep <= 16 and a non-empty cache; "
