@@ -6,8 +6,10 @@ packed V[4,32768,13]+norms[4,32768], dense softmax, out[28,128] -- the fused tq_
 entry point of libtqhip.so, called through the C ABI.  Inputs are resident in HBM before the timed
 region; the steps rotate over N_SETS independent (q, K, V) sets totalling > 400 MB so that neither
 the L2s nor the 256 MB Infinity Cache can serve the reads.  The K timed steps are captured once
-into a HIP graph and replayed (back-to-back launches, no host gaps); HIP events on the launch
-stream bracket the replay.
+into a HIP graph (back-to-back launches, no host gaps) and the graph is replayed until at least
+MIN_TIMED_MS of GPU time has passed, every replay bracketed by HIP events on the launch stream:
+`ms_per_step` is the MEDIAN replay divided by K (a single replay of 20 steps is a 0.3 ms sample),
+the fastest and slowest replay are reported beside it.
 
 Prints ONE JSON line (see the fields below).  `roofline.achieved` = algorithmic bytes per step
 (40 908 800 B: q 7 168 + K 33 554 432 + V packed 6 815 744 + V norms 524 288 + out 7 168)
@@ -32,6 +34,8 @@ PDIM = 13
 ALGO_BYTES = N_Q * D * 2 + N_KV * T * D * 2 + N_KV * T * PDIM * 4 + N_KV * T * 4 + N_Q * D * 2
 HBM_PEAK_GBS = 8000.0
 N_SETS = 10
+MIN_TIMED_MS = 50.0       # GPU time every timed quantity is measured over (at least 5 replays)
+READ_WGS = 2048           # workgroups of the plain-read probe (8 per CU)
 
 # HBM bytes per launch of the dominant kernel (the tile pass), from two rocprofv3 --pmc runs of
 # `python bench.py --steps 60 --warmup 6 --no-cpu --no-graph` (FETCH_SIZE, then WRITE_SIZE), each
@@ -100,6 +104,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph")
+    ap.add_argument("--no-ceiling", action="store_true", help="skip the plain-read probe (`read_ceiling` of the line)")
+    ap.add_argument("--calibrate-read", action="store_true",
+                    help="instead of the benchmark, time tq_probe_read: one launch that only streams the K / packed-V / "
+                         "norm bytes of a step (and an empty launch), with the benchmark's rotation and launch pattern")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="instead of the benchmark, run --steps plain device copies of ALGO_BYTES bytes each "
                          "(known traffic: ALGO_BYTES read + ALGO_BYTES written) to scale rocprofv3's "
@@ -159,7 +167,7 @@ def main():
     torch.cuda.synchronize()
     checked = outs[0].clone()
     cpu = None
-    if not args.no_cpu:
+    if not args.no_cpu and not args.calibrate_read:
         ref, cpu = cpu_baseline(torch, sets, cb, signs)
         err = np.abs(outs[0][0].cpu().numpy() - ref)
         if not np.all(err <= 1e-3 + 2e-3 * np.abs(ref)):
@@ -168,43 +176,94 @@ def main():
 
     side = torch.cuda.Stream(device=dev)
 
-    def timed(phases, rot=N_SETS):
-        """ms per launch of `args.steps` back-to-back calls (HIP graph replay unless --no-graph),
-        bracketed by HIP events on the launch stream, rotating over the first `rot` buffer sets."""
-        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    def timed(one_step):
+        """(median, min, max, replays): ms per step of `one_step(i, stream)` over replays of a HIP graph of
+        `args.steps` back-to-back steps (eager launches once with --no-graph), HIP events on the launch stream."""
         with torch.cuda.stream(side):
-            s_args = [bound(i, side.cuda_stream) for i in range(N_SETS)]
             for i in range(args.warmup):
-                step(i, s_args, phases, rot)
+                one_step(i, side.cuda_stream)
             side.synchronize()
             if args.no_graph:
+                ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 ev0.record(side)
                 for i in range(args.steps):
-                    step(i, s_args, phases, rot)
+                    one_step(i, side.cuda_stream)
                 ev1.record(side)
                 side.synchronize()
-            else:
-                graph = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(graph, stream=side):
-                    g_stream = torch.cuda.current_stream(dev)
-                    g_args = [bound(i, g_stream.cuda_stream) for i in range(N_SETS)]
-                    for i in range(args.steps):
-                        step(i, g_args, phases, rot)
-                graph.replay()                  # one untimed replay: instantiation, page-in
-                torch.cuda.synchronize()
-                ev0.record(side)
+                per = ev0.elapsed_time(ev1) / args.steps
+                return per, per, per, 1
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                g_stream = torch.cuda.current_stream(dev).cuda_stream
+                for i in range(args.steps):
+                    one_step(i, g_stream)
+            graph.replay()                      # untimed: instantiation, page-in
+            side.synchronize()
+            ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+            ev[0].record(side)
+            graph.replay()
+            ev[1].record(side)
+            side.synchronize()
+            est = max(ev[0].elapsed_time(ev[1]), 1e-3)
+            n_rep = int(min(max(5, math.ceil(MIN_TIMED_MS / est)), 4000))
+            ev = [torch.cuda.Event(enable_timing=True) for _ in range(n_rep + 1)]
+            ev[0].record(side)
+            for r in range(n_rep):
                 graph.replay()
-                ev1.record(side)
-                side.synchronize()
+                ev[r + 1].record(side)
+            side.synchronize()
         torch.cuda.synchronize()
-        return ev0.elapsed_time(ev1) / args.steps
+        per = sorted(ev[r].elapsed_time(ev[r + 1]) / args.steps for r in range(n_rep))
+        return per[n_rep // 2], per[0], per[-1], n_rep
+
+    arg_cache = {}
+
+    def decode_step(phases, rot=N_SETS):
+        def one(i, stream):
+            if stream not in arg_cache:
+                arg_cache[stream] = [bound(j, stream) for j in range(N_SETS)]
+            step(i, arg_cache[stream], phases, rot)
+        return one
+
+    def read_ceiling():
+        """One launch that only streams the K, packed-V and norm bytes of a step (tq_probe_read, rotating over
+        copies of the buffer sets), and an empty launch, timed like the decode step."""
+        sink = torch.zeros(1, dtype=torch.int32, device=dev)
+        srcs = [torch.cat([k.reshape(-1).view(torch.uint8), vp.reshape(-1).view(torch.uint8),
+                           vn.reshape(-1).view(torch.uint8)]) for (_, k, vp, vn) in sets]
+        nbytes = srcs[0].numel() // 16 * 16
+
+        def read_step(nb):
+            def one(i, stream):
+                rc = lib.tq_probe_read(C.c_void_p(srcs[i % N_SETS].data_ptr()), nb, C.c_void_p(sink.data_ptr()),
+                                       READ_WGS, C.c_void_p(stream))
+                if rc != 0:
+                    _lib.check(rc)
+            return one
+        r_med, r_min, r_max, r_n = timed(read_step(nbytes))
+        e_med, e_min, e_max, _ = timed(read_step(0))
+        return {
+            "bytes_per_launch": nbytes, "workgroups": READ_WGS,
+            "us_per_launch": round(r_med * 1e3, 3), "min": round(r_min * 1e3, 3), "max": round(r_max * 1e3, 3),
+            "replays": r_n, "GB/s": round(nbytes / (r_med * 1e-3) / 1e9, 1),
+            "frac_of_peak": round(nbytes / (r_med * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            "empty_launch_us": round(e_med * 1e3, 3), "empty_launch_min": round(e_min * 1e3, 3),
+            "empty_launch_max": round(e_max * 1e3, 3),
+            "note": "one launch that only reads the K, packed-V and norm bytes of a step (rotating buffer sets, the "
+                    "benchmark's launch pattern): the practical ceiling for a launch of this size on this box"}
+
+    if args.calibrate_read:
+        print(json.dumps({"calibrate_read": True, "buffer_sets": N_SETS, "steps": args.steps, "warmup": args.warmup,
+                          "launch": "eager" if args.no_graph else "hipgraph", "read": read_ceiling()}))
+        return
 
     mode = "eager" if args.no_graph else "hipgraph"
-    ms_per_step = timed(3)                      # whole step: tile pass + merge pass
-    ms_tile = timed(1)                          # dominant kernel alone, same launch pattern
-    ms_warm = timed(3, rot=1)                   # one buffer set over and over: its 41 MB stay in the 256 MB Infinity Cache
+    ms_per_step, ms_min, ms_max, n_replays = timed(decode_step(3))    # whole step: tile pass + merge pass
+    ms_tile, tile_min, tile_max, _ = timed(decode_step(1))            # dominant kernel alone, same launch pattern
+    ms_warm = timed(decode_step(3, rot=1))[0]   # one buffer set over and over: its 41 MB stay in the 256 MB Infinity Cache
     gbs = ALGO_BYTES / (ms_per_step * 1e-3) / 1e9
     gbs_tile = ALGO_BYTES / (ms_tile * 1e-3) / 1e9
+    ceiling = None if args.no_ceiling else read_ceiling()
     step(0, eager_args)                         # leave outs[0] = the full result of set 0
     torch.cuda.synchronize()
 
@@ -229,6 +288,11 @@ def main():
                      "note": "algorithmic bytes / event-timed launch period of the tile pass alone; "
                              "`value` covers the whole step (tile pass + merge pass)"},
         "cpu_baseline": cpu,
+        "read_ceiling": ceiling,
+        "timing": {"method": "median over HIP-graph replays of `steps` steps each, >= %d ms of GPU time" % int(MIN_TIMED_MS)
+                   if not args.no_graph else "one pass of eager launches",
+                   "replays": n_replays, "us_per_layer_min": round(ms_min * 1e3, 3), "us_per_layer_max": round(ms_max * 1e3, 3),
+                   "tile_us_min": round(tile_min * 1e3, 3), "tile_us_max": round(tile_max * 1e3, 3)},
         "warm_cache": {"us_per_layer": round(ms_warm * 1e3, 3), "value": round(ALGO_BYTES / (ms_warm * 1e-3) / 1e9, 1),
                        "unit": "GB/s", "note": "same step on ONE buffer set (inputs served from the Infinity Cache); "
                                                "reported beside `value`, never as it"},

@@ -486,6 +486,16 @@ int tq_prefill_attn(const void* q, int q_dtype,
 
 size_t tq_prefill_workspace_bytes(int n_q_heads, int64_t n_rows, int64_t kv_len, int dim);
 
+/*
+ * Measurement aid, no counterpart in the reference (its benches time whole kernels with mx.eval,
+ * scripts/bench_sparse_v.py:49-57): ONE launch that streams `bytes` bytes from `src` (16-byte aligned,
+ * a multiple of 16) through n_workgroups workgroups of 256 threads and writes nothing -- the practical
+ * ceiling for a launch that reads this much on the machine at hand, launch overhead and tail included.
+ * bytes == 0 launches an empty kernel (the cost of a launch alone).  `sink` (device, 4 bytes, may be NULL)
+ * is never written in practice.  bench.py --calibrate-read times both beside the decode step.
+ */
+int tq_probe_read(const void* src, size_t bytes, uint32_t* sink, int n_workgroups, tq_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
