@@ -880,3 +880,209 @@ def test_decode_step_after_from_state_and_trim(tq):
         assert a.offset == b.offset == S0 - 7 + 3
         for x, y in zip(a.state, b.state):
             assert torch.equal(x, y)
+
+
+# ------------------------------------------------------------------ explicit sign vectors
+
+def _pm1(dim, seed):
+    rng = np.random.default_rng(seed)
+    return np.where(rng.random(dim) < 0.5, -1.0, 1.0).astype(F32)
+
+
+def test_packed_cache_with_explicit_signs_round_trips(tq):
+    """A cache built with caller-supplied sign vectors (cache.py:33-39,90-98 take them from the seed): packed
+    state equals the oracle's for THOSE signs, differs from the seed-derived one, survives state / meta_state /
+    from_state(..., k_signs, v_signs) bit for bit, and attends within the bar both before and after."""
+    B, n_q, n_kv, D, S = 1, 8, 2, 128, 300
+    sc = 1 / math.sqrt(D)
+    ks, vs = _pm1(D, 901), _pm1(D, 902)
+    k, v = rand((B, n_kv, S, D), 910), rand((B, n_kv, S, D), 911)
+    q = rand((B, n_q, 1, D), 912)
+    c = tq.TurboQuantKVCache(bits=3, fused=True, k_signs=ks, v_signs=torch.from_numpy(vs))
+    c.update_and_fetch(k, v)
+    cb = o.gaussian_codebook(3)
+    bd = o.gaussian_boundaries(cb)
+    kp, kn = o.fused_quantize(host(k).reshape(-1, D), ks, bd, D, 3)
+    vp, vn = o.fused_quantize(host(v).reshape(-1, D), vs, bd, D, 3)
+    assert np.array_equal(c.k_packed[..., :S, :].cpu().numpy().reshape(-1, 13), kp)
+    assert np.array_equal(c.v_packed[..., :S, :].cpu().numpy().reshape(-1, 13), vp)
+    assert np.array_equal(c.k_norms[..., :S].cpu().numpy().ravel(), kn)
+    seeded = tq.TurboQuantKVCache(bits=3, fused=True)
+    seeded.update_and_fetch(k, v)
+    assert not torch.equal(seeded.k_packed, c.k_packed)
+    want = np.stack([o.flash_attention_turboquant(
+        o.prerotate_query(host(q)[0, :, 0, :], ks), kp.reshape(n_kv, S, 13), kn.reshape(n_kv, S), vp.reshape(n_kv, S, 13),
+        vn.reshape(n_kv, S), cb, cb, vs, D, 3, n_rep=n_q // n_kv, attn_scale=sc)])
+    got = host(tq.turboquant_attention(q, c, sc, fused=True))[:, :, 0, :]
+    err = np.abs(got - want)
+    assert np.all(err <= 1e-3 + 2e-3 * np.abs(want)), err.max()
+    # serialise and restore: with the signs the restored cache is the same cache
+    r = tq.TurboQuantKVCache.from_state([t.clone() for t in c.state], c.meta_state, k_signs=ks, v_signs=vs)
+    for x, y in zip(r.state, c.state):
+        assert torch.equal(x, y)
+    assert r.meta_state == c.meta_state
+    got_r = host(tq.turboquant_attention(q, r, sc, fused=True))[:, :, 0, :]
+    assert np.array_equal(got_r, got)
+    # ... and can extend: the new rows are encoded with the given signs
+    k1, v1 = rand((B, n_kv, 5, D), 913), rand((B, n_kv, 5, D), 914)
+    r.fused = True
+    r.update_and_fetch(k1, v1)
+    kp1, _ = o.fused_quantize(host(k1).reshape(-1, D), ks, bd, D, 3)
+    assert np.array_equal(r.k_packed[..., S:S + 5, :].cpu().numpy().reshape(-1, 13), kp1)
+    # without the signs the restored cache decodes with the seed's vector: a different (wrong) result
+    wrong = tq.TurboQuantKVCache.from_state([t.clone() for t in c.state], c.meta_state)
+    got_w = host(tq.turboquant_attention(q, wrong, sc, fused=True))[:, :, 0, :]
+    assert np.abs(got_w - want).max() > 0.05
+    with pytest.raises(ValueError):
+        tq.TurboQuantKVCache(bits=3, k_signs=np.ones(64, F32)).update_and_fetch(k, v)
+    with pytest.raises(ValueError):
+        tq.TurboQuantKVCache(bits=3, v_signs=np.zeros(D, F32)).update_and_fetch(k, v)
+
+
+def test_vonly_cache_with_explicit_signs_round_trips(tq):
+    """VOnlyTurboQuantCache(v_signs=...) and from_state(..., v_signs=...): values dequantise to the oracle's for
+    those signs, the restored cache is bit-identical and attends like the original."""
+    B, n_q, n_kv, D, S = 1, 14, 2, 128, 260
+    sc = 1 / math.sqrt(D)
+    vs = _pm1(D, 921)
+    k, v = rand((B, n_kv, S, D), 930), rand((B, n_kv, S, D), 931)
+    q = rand((B, n_q, 1, D), 932)
+    c = tq.VOnlyTurboQuantCache(bits=3, v_signs=vs)
+    _, v_deq = c.update_and_fetch(k, v)
+    cb = o.gaussian_codebook(3)
+    vp, vn = o.fused_quantize(host(v).reshape(-1, D), vs, o.gaussian_boundaries(cb), D, 3)
+    assert np.array_equal(c._v_tq.v_packed[..., :S, :].cpu().numpy().reshape(-1, 13), vp)
+    want_deq = o.packed_dequantize(vp, vn, cb, vs, D, 3).reshape(B, n_kv, S, D)
+    assert np.abs(host(v_deq) - want_deq).max() <= 2e-3           # fp16 output of exact float32 values
+    want = o.vonly_decode_attention(host(q)[0, :, 0, :], host(k)[0].astype(np.float16), vp.reshape(n_kv, S, 13),
+                                    vn.reshape(n_kv, S), cb, vs, D, 3, sc)
+    got = host(tq.vonly_decode_attention(q, c, sc))[0, :, 0, :]
+    assert np.all(np.abs(got - want) <= 1e-3 + 2e-3 * np.abs(want))
+    r = tq.VOnlyTurboQuantCache.from_state([t.clone() for t in c.state], c.meta_state, v_signs=vs)
+    assert r.offset == S and r.meta_state == c.meta_state
+    for x, y in zip(r.state, c.state):
+        assert torch.equal(x, y)
+    assert np.array_equal(host(tq.vonly_decode_attention(q, r, sc))[0, :, 0, :], got)
+    k1, v1, q1 = rand((B, n_kv, 1, D), 933), rand((B, n_kv, 1, D), 934), rand((B, n_q, 1, D), 935)
+    o1 = host(r.decode_step(q1, k1, v1, sc))[0, :, 0, :]
+    c.update_and_fetch(k1, v1)
+    o2 = host(tq.vonly_decode_attention(q1, c, sc))[0, :, 0, :]
+    assert np.all(np.abs(o1 - o2) <= 1e-3 + 2e-3 * np.abs(o2))
+    for x, y in zip(r.state, c.state):
+        assert torch.equal(x, y)
+
+
+# ------------------------------------------------------------------ one capacity for keys and values
+
+def _vonly_filled(tq, chunks, seed, **kw):
+    B, n_kv, D = 1, 2, 128
+    c = tq.VOnlyTurboQuantCache(bits=3, **kw)
+    for i, S in enumerate(chunks):
+        c.update_and_fetch(rand((B, n_kv, S, D), seed + 2 * i), rand((B, n_kv, S, D), seed + 2 * i + 1))
+    return c
+
+
+@pytest.mark.parametrize("chunks,fused", [((1000,), False), ((1000, 500), False), ((1000,), True), ((700, 300, 3), True)])
+def test_vonly_single_call_step_after_real_prompts(tq, chunks, fused):
+    """A prompt through update_and_fetch leaves the key cache and the packed values with different capacities
+    (they grow by different rules); reserve() and decode_step() must bring them to one capacity so that the
+    single-call step (host position AND device-side position) runs on its descriptor, not on the two-call
+    fallback: the descriptor is asserted to exist, results and state are compared with the two calls."""
+    B, n_q, n_kv, D = 1, 14, 2, 128
+    sc = 1 / math.sqrt(D)
+    a = _vonly_filled(tq, chunks, 1700, fused=fused)
+    b = _vonly_filled(tq, chunks, 1700, fused=True)
+    n0 = sum(chunks)
+    a.reserve(B, n_kv, 2000, D)
+    assert a._k_cache.keys.shape[2] == a._v_tq.v_packed.shape[2] >= n0 + 2000
+    assert a._k_cache.keys.shape[2] % 256 == 0
+    for x, y in zip(a.state, b.state):
+        assert torch.equal(x, y)
+    pos = torch.tensor([n0], dtype=torch.int64, device="cuda")
+    out = torch.empty((B, n_q, D), dtype=torch.float16, device="cuda")
+    for i in range(3):
+        k1, v1, q1 = rand((B, n_kv, 1, D), 1710 + 3 * i), rand((B, n_kv, 1, D), 1711 + 3 * i), rand((B, n_q, 1, D), 1712 + 3 * i)
+        if i < 2:
+            a.decode_step(q1, k1, v1, sc, position=pos, out=out)
+            pos.add_(1)
+            got = out.clone()[:, :, None, :]
+        else:
+            a.set_offset(int(pos.item()))
+            got = a.decode_step(q1, k1, v1, sc)
+        assert a._step is not None and a._step.shape[2] == a._k_cache.keys.shape[2], "the two-call fallback ran"
+        b.update_and_fetch(k1, v1)
+        want = tq.vonly_decode_attention(q1, b, sc)
+        err = (got.float() - want.float()).abs()
+        assert bool((err <= 1e-3 + 2e-3 * want.float().abs()).all()), float(err.max())
+    assert a.offset == b.offset == n0 + 3
+    for x, y in zip(a.state, b.state):
+        assert torch.equal(x, y)
+
+
+def test_vonly_single_call_step_after_from_state(tq):
+    """from_state hands the storage in as slices (300 positions; the key cache would grow to 556, the packed
+    values to 512): the first decode_step realigns both to one contiguous capacity and runs on the descriptor,
+    also with a device-side position."""
+    B, n_q, n_kv, D, S0 = 1, 8, 2, 128, 300
+    sc = 1 / math.sqrt(D)
+    src = _vonly_filled(tq, (S0,), 1800, fused=True)
+    a = tq.VOnlyTurboQuantCache.from_state(src.state, src.meta_state)
+    a.fused = True
+    a.reserve(B, n_kv, 1, D)
+    assert a._k_cache.keys.shape[2] == a._v_tq.v_packed.shape[2] == 512 and a._k_cache.keys.is_contiguous()
+    pos = torch.tensor([S0], dtype=torch.int64, device="cuda")
+    for i in range(2):
+        k1, v1, q1 = rand((B, n_kv, 1, D), 1810 + 3 * i), rand((B, n_kv, 1, D), 1811 + 3 * i), rand((B, n_q, 1, D), 1812 + 3 * i)
+        got = a.decode_step(q1, k1, v1, sc, position=pos)
+        pos.add_(1)
+        assert a._step is not None
+        src.update_and_fetch(k1, v1)
+        want = tq.vonly_decode_attention(q1, src, sc)
+        err = (got.float() - want.float()).abs()
+        assert bool((err <= 1e-3 + 2e-3 * want.float().abs()).all()), float(err.max())
+    a.set_offset(int(pos.item()))
+    for x, y in zip(a.state, src.state):
+        assert torch.equal(x, y)
+    with pytest.raises(ValueError):
+        a.set_offset(513)
+
+
+def test_step_descriptor_keeps_its_workspace_alive(tq):
+    """The workspace address goes into every call of a step descriptor (and into a HIP graph that records one).
+    When a later, larger op replaces the shared per-stream workspace, the descriptor must still hold the buffer
+    it used: its graph replays keep writing there."""
+    from tqhip import ops
+    B, n_q, n_kv, D = 1, 14, 2, 128
+    sc = 1 / math.sqrt(D)
+    a = _vonly_filled(tq, (600,), 1900, fused=True)
+    b = _vonly_filled(tq, (600,), 1900, fused=True)
+    a.reserve(B, n_kv, 64, D)
+    pos = torch.tensor([600], dtype=torch.int64, device="cuda")
+    ks, vs_, qs = rand((B, n_kv, 1, D), 1910), rand((B, n_kv, 1, D), 1911), rand((B, n_q, 1, D), 1912)
+    out = torch.empty((B, n_q, D), dtype=torch.float16, device="cuda")
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        a.decode_step(qs, ks, vs_, sc, position=pos, out=out)      # warm-up on the capture stream
+        side.synchronize()
+        first_ws = a._step._ws
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            a.decode_step(qs, ks, vs_, sc, position=pos, out=out)
+    torch.cuda.synchronize()
+    key = (first_ws.device, side.cuda_stream)
+    assert ops._workspaces[key] is first_ws
+    with torch.cuda.stream(side):                                  # a larger request on that stream replaces the shared buffer
+        ops._workspace(first_ws.device, side.cuda_stream, first_ws.numel() * 4 + 1)
+    assert ops._workspaces[key] is not first_ws
+    assert any(w is first_ws for w in a._step._ws_refs), "the descriptor dropped the workspace its graph writes to"
+    filler = torch.full((first_ws.numel() * 2,), 7, dtype=torch.uint8, device="cuda")   # would land in freed memory
+    for i in range(3):
+        g.replay()
+        torch.cuda.synchronize()
+        pos.add_(1)
+        torch.cuda.synchronize()
+        b.update_and_fetch(ks, vs_)
+        want = tq.vonly_decode_attention(qs, b, sc)[:, :, 0, :]
+        err = (out.float() - want.float()).abs()
+        assert bool((err <= 1e-3 + 2e-3 * want.float().abs()).all()), (i, float(err.max()))
+    assert int(filler.sum()) == 7 * filler.numel()

@@ -709,7 +709,7 @@ def test_prefill_attention_matches_oracle(tq, n_kv, n_rep, T, n_rows, pos0):
     got = tq.prefill_attention(dev(q), dev(kp), dev(kn), dev(vp), dev(vn), c, c, dev(ks), dev(vs), 128, 3, sc,
                                n_rep=n_rep, q_pos0=pos0, out_dtype=torch.float32)
     assert got.shape == (n_kv * n_rep, n_rows, 128)
-    close(host(got).reshape(-1, 128), want.reshape(-1, 128), row_scale=True)
+    close(host(got).reshape(-1, 128), want.reshape(-1, 128))      # N(0,1) data, no outlier channels: elementwise 2e-3 / 1e-3
     rel = np.abs(host(got) - want).max() / np.abs(want).max()
     assert rel < 1e-3, rel
 
@@ -1136,8 +1136,11 @@ def test_flash_streaming_pass_group_sizes_and_leading_offset(tq, n_kv, n_rep):
 def test_config4_full_size_paths_agree(tq):
     """benchmark configuration 4 at full size (16 sequences of 4096..32768 positions, 32 q / 8 kv heads, fp16
     out): the streaming pass, the one-tile-per-workgroup pass (forced by an all-zero mask) and the float32
-    kernels are three separate code paths and must agree; the two shortest sequences are also checked
-    against the oracle."""
+    kernels are three separate code paths and must agree; the two shortest sequences and the LONGEST one (the most
+    steps of the streaming pass) are also checked against the oracle.  Tolerances: the inputs are random packed
+    words with key norms of 7 .. 15, i.e. peaked softmax rows whose outputs span decades inside a row, so the
+    relative term is taken against the row maximum (the reference's own measure, tests/test_flash_attention.py),
+    plus the fp16 rounding of the output."""
     rng = np.random.default_rng(4)
     n_kv, n_rep, D, bits, n_seq = 8, 4, 128, 3, 16
     lens = rng.integers(4096, 32769, size=n_seq)
@@ -1166,11 +1169,13 @@ def test_config4_full_size_paths_agree(tq):
     close(t.reshape(-1, D), f.reshape(-1, D), rel=3e-3, row_scale=True)
     close(a.reshape(-1, D), t.reshape(-1, D), rel=2e-3, row_scale=True)
     hk, hkn, hv, hvn = host(kp), host(kn), host(vp), host(vn)
-    for i in np.argsort(lens)[:2]:
+    order = np.argsort(lens)
+    for i in (order[0], order[1], order[-1]):
         s0, s1 = offs[i], offs[i + 1]
         want = o.flash_attention_turboquant(o.prerotate_query(q[i], ks), hk[:, s0:s1], hkn[:, s0:s1], hv[:, s0:s1],
                                             hvn[:, s0:s1], c, c, vs, D, bits, sc, 16, n_rep)
         close(a[i], want, rel=3e-3, row_scale=True)
+        close(f[i], want, row_scale=True)                          # the float32 kernels: no fp16 anywhere
 
 
 def test_config5_full_size_encode_paths_agree(tq):
@@ -1196,7 +1201,9 @@ def test_config5_full_size_encode_paths_agree(tq):
 def test_config5_full_size_prefill_rows_are_decode_steps(tq):
     """benchmark configuration 5, attention half, at full size: a 512-row causal chunk at the end of a 131 072-position
     packed cache, 32 q / 8 kv heads.  Row i of the chunk is one decode step over positions 0 .. T-512+i: three
-    rows are compared with the float32 flash-decode kernels (a separate code path) over those prefixes."""
+    rows are compared with the float32 flash-decode kernels (a separate code path) over those prefixes, and with
+    the ORACLE's flash attention over the same prefixes -- the last row (all 131 072 positions) on kv heads 0 and 7,
+    the first and the middle row on kv head 3 (the float64 oracle takes ~8 s per kv head at this length)."""
     g = torch.Generator(device="cuda")
     g.manual_seed(55)
     n_kv, n_rep, T, n_rows, D, bits = 8, 4, 131072, 512, 128, 3
@@ -1215,6 +1222,15 @@ def test_config5_full_size_prefill_rows_are_decode_steps(tq):
         ref = tq.flash_attention_turboquant(q_rot, kp[:, :L], kn[:, :L], vp[:, :L], vn[:, :L], c, c, vs, D, bits, sc,
                                             n_rep=n_rep, precision="fp32")
         close(host(got[:, i]), host(ref), row_scale=True)
+    hks = o.random_diagonal_sign(D, 42)
+    hvs = o.random_diagonal_sign(D, 43)
+    for i, heads in ((511, (0, 7)), (0, (3,)), (255, (3,))):
+        L = T - n_rows + i + 1
+        for h in heads:
+            qh = host(q[h * n_rep:(h + 1) * n_rep, i]).astype(F32)
+            want = o.flash_attention_turboquant(o.prerotate_query(qh, hks), host(kp[h:h + 1, :L]), host(kn[h:h + 1, :L]),
+                                                host(vp[h:h + 1, :L]), host(vn[h:h + 1, :L]), c, c, hvs, D, bits, sc, 16, n_rep)
+            close(host(got[h * n_rep:(h + 1) * n_rep, i]), want, row_scale=True)
 
 
 def test_config3_full_size_scores(tq):
@@ -1729,3 +1745,39 @@ def test_attended_length_beyond_the_tensors_is_refused(tq):
                              c, c, dev(ks), dev(vs), 128, 3, 0.1, n_rep=1, kv_len=101)
     with pytest.raises(ValueError, match="holds 1 sequences"):
         tq.vonly_decode(torch.cat([q, q]), dev(K[None]), dev(vp[None]), dev(vn[None]), c, dev(vs), 128, 3, 0.1)
+
+
+def test_seq_offsets_are_checked_by_every_ragged_wrapper(tq):
+    """An int64 offsets tensor (torch.cumsum's default) would be read as int32 pairs by the kernels: all three ragged
+    wrappers refuse it, as they refuse a wrong count; validate_offsets=True also checks order and range."""
+    rng = np.random.default_rng(77)
+    n_kv, n_rep, D, bits = 2, 2, 128, 3
+    lens = [100, 60]
+    total = sum(lens)
+    c, b = tables(bits)
+    ks, vs = o.random_diagonal_sign(D, 42), o.random_diagonal_sign(D, 43)
+    X = rng.standard_normal((n_kv * total, D)).astype(np.float16)
+    kp, kn = tq.fused_quantize(dev(X), dev(ks), b, D, bits)
+    kp, kn = kp.reshape(n_kv, total, -1), kn.reshape(n_kv, total)
+    K16 = dev(X.reshape(n_kv, total, D))
+    q = dev(rng.standard_normal((2, n_kv * n_rep, D)).astype(np.float32))
+    good = torch.tensor([0, 100, 160], dtype=torch.int32, device="cuda")
+    calls = {
+        "flash_decode": lambda off, **kw: tq.flash_decode(q, kp, kn, kp, kn, c, c, dev(vs), D, bits, 0.1, n_rep=n_rep,
+                                                          seq_offsets=off, max_seq_len=100, **kw),
+        "flash_decode_from_q": lambda off, **kw: tq.flash_decode_from_q(q, dev(ks), kp, kn, kp, kn, c, c, dev(vs), D, bits, 0.1,
+                                                                        n_rep=n_rep, seq_offsets=off, max_seq_len=100, **kw),
+        "vonly_decode": lambda off, **kw: tq.vonly_decode(q, K16, kp, kn, c, dev(vs), D, bits, 0.1, n_rep=n_rep,
+                                                          seq_offsets=off, max_seq_len=100, **kw),
+    }
+    for name, call in calls.items():
+        ref = call(good, validate_offsets=True)
+        assert torch.isfinite(ref).all(), name
+        with pytest.raises(ValueError, match="int32"):
+            call(torch.cumsum(torch.tensor([0, 100, 60], device="cuda"), 0))             # int64
+        with pytest.raises(ValueError, match="n_seq"):
+            call(torch.tensor([0, 160], dtype=torch.int32, device="cuda"))
+        with pytest.raises(ValueError, match="never decrease"):
+            call(torch.tensor([0, 120, 100], dtype=torch.int32, device="cuda"), validate_offsets=True)
+        with pytest.raises(ValueError, match="holds"):
+            call(torch.tensor([0, 100, 161], dtype=torch.int32, device="cuda"), validate_offsets=True)

@@ -13,13 +13,27 @@ from .quantizer import gaussian_boundaries, gaussian_codebook
 from .rotation import random_diagonal_sign
 
 
-class _Quantizer:
-    """cache.py:33-39: signs (device) + codebook tables (host)."""
+def _checked_signs(signs, dim, device) -> torch.Tensor:
+    """A caller's sign vector as the kernels take it: float32 [dim] of +-1 on `device`."""
+    t = torch.as_tensor(signs)
+    if t.dim() != 1 or t.numel() != dim:
+        raise ValueError(f"a sign vector must have shape ({dim},), got {tuple(t.shape)}")
+    t = t.detach().to(device=device, dtype=torch.float32).contiguous()
+    if not bool((t.abs() == 1.0).all()):
+        raise ValueError("a sign vector holds +1 and -1 only")
+    return t
 
-    def __init__(self, dim, bits, seed, device):
+
+class _Quantizer:
+    """cache.py:33-39: signs (device) + codebook tables (host).  `signs` overrides the vector that
+    random_diagonal_sign derives from `seed` (whose generator is this package's own, not MLX's): the way to
+    read a cache written by the reference, which stores only the seed (cache.py:286)."""
+
+    def __init__(self, dim, bits, seed, device, signs=None):
         self.dim = dim
         self.bits = bits
-        self.signs = random_diagonal_sign(dim, seed=seed, device=device)
+        self.signs = (random_diagonal_sign(dim, seed=seed, device=device) if signs is None
+                      else _checked_signs(signs, dim, device))
         self.centroids = gaussian_codebook(bits)
         self.boundaries = gaussian_boundaries(self.centroids)
 
@@ -60,7 +74,9 @@ class TurboQuantKVCache:
 
     def __init__(self, bits: int = 3, seed: int = 42, fused: bool = False,
                  sparse_v_threshold: float | None = None, v_only: bool = False,
-                 encode_variant: str = "mlx"):
+                 encode_variant: str = "mlx", k_signs=None, v_signs=None):
+        """k_signs / v_signs ([dim] of +-1, any tensor-like): the rotation's sign vectors, used instead of the ones
+        derived from `seed` / `seed + 1` (cache.py:92,96).  Everything else as the reference (cache.py:54-61)."""
         self.quant_bits = bits
         self.seed = seed
         self.offset = 0
@@ -72,6 +88,7 @@ class TurboQuantKVCache:
         # The two differ only for values within an ulp of a decision boundary.
         self.encode_variant = encode_variant
         self._reset_fields()
+        self._k_signs_given, self._v_signs_given = k_signs, v_signs
 
     def _reset_fields(self):
         self.k_packed = None
@@ -90,6 +107,7 @@ class TurboQuantKVCache:
         self._v_pdim = None
         self._dtype = None
         self._step, self._step_key = None, None
+        self._k_signs_given, self._v_signs_given = None, None
 
     # ---------------------------------------------------------------- setup (cache.py:90-123)
     def _device(self):
@@ -101,11 +119,11 @@ class TurboQuantKVCache:
     def _ensure_quantizer(self, k_dim, v_dim, device=None):
         device = device if device is not None else self._device()
         if not self.v_only and self._k_q is None:
-            self._k_q = _Quantizer(k_dim, self.quant_bits, self.seed, device)
+            self._k_q = _Quantizer(k_dim, self.quant_bits, self.seed, device, self._k_signs_given)
             self._k_dim = k_dim
             self._k_pdim = ops.packed_dim(k_dim, self.quant_bits)
         if self._v_q is None:
-            self._v_q = _Quantizer(v_dim, self.quant_bits, self.seed + 1, device)
+            self._v_q = _Quantizer(v_dim, self.quant_bits, self.seed + 1, device, self._v_signs_given)
             self._v_dim = v_dim
             self._v_pdim = ops.packed_dim(v_dim, self.quant_bits)
 
@@ -121,12 +139,16 @@ class TurboQuantKVCache:
         prev = self.offset
         needed = prev + num_new
         if self.v_packed is None or needed > self.v_packed.shape[2]:
-            n = _round_up(needed, self.step)
-            if not self.v_only:
-                self.k_packed, self.k_norms = self._grow(self.k_packed, self.k_norms, B, H, n,
-                                                         self._k_pdim, prev, device)
-            self.v_packed, self.v_norms = self._grow(self.v_packed, self.v_norms, B, H, n,
-                                                     self._v_pdim, prev, device)
+            self._reallocate(B, H, _round_up(needed, self.step), device)
+
+    def _reallocate(self, B, H, n, device):
+        """Fresh contiguous storage of n positions per (b, h) holding the first `offset` positions."""
+        prev = self.offset
+        if not self.v_only:
+            self.k_packed, self.k_norms = self._grow(self.k_packed, self.k_norms, B, H, n,
+                                                     self._k_pdim, prev, device)
+        self.v_packed, self.v_norms = self._grow(self.v_packed, self.v_norms, B, H, n,
+                                                 self._v_pdim, prev, device)
 
     # ---------------------------------------------------------------- codec calls
     def _encode(self, x, q, packed, norms, B, H, S, dim, prev):
@@ -393,9 +415,13 @@ class TurboQuantKVCache:
 
     # ---------------------------------------------------------------- cache.py:336-369
     @classmethod
-    def from_state(cls, state, meta_state):
+    def from_state(cls, state, meta_state, k_signs=None, v_signs=None):
+        """cache.py:336-369.  The serialised cache carries its seed, not its sign vectors (cache.py:286): a cache
+        written with explicit signs -- or by the reference, whose seed-to-signs generator is MLX's -- restores
+        correctly only with the same k_signs / v_signs given here."""
         obj = cls.__new__(cls)
         obj._reset_fields()
+        obj._k_signs_given, obj._v_signs_given = k_signs, v_signs
         obj.fused = False
         obj.sparse_v_threshold = None
         obj.v_only = False

@@ -58,6 +58,16 @@ class KVCache:
             else:
                 self.keys, self.values = new_k, new_v
 
+    def reallocate(self, B, H, n, k_dim, v_dim, k_dtype, v_dtype, device):
+        """Fresh contiguous storage of exactly n positions holding the first `offset` positions (a capacity
+        chosen by the caller, for an owner that keeps this cache in step with a second storage)."""
+        new_k = torch.zeros((B, H, n, k_dim), dtype=k_dtype, device=device)
+        new_v = torch.zeros((B, H, n, v_dim), dtype=v_dtype, device=device)
+        if self.keys is not None and self.offset > 0:
+            new_k[..., :self.offset, :] = self.keys[..., :self.offset, :]
+            new_v[..., :self.offset, :] = self.values[..., :self.offset, :]
+        self.keys, self.values = new_k, new_v
+
     def update_and_fetch(self, keys: torch.Tensor, values: torch.Tensor):
         prev = self.offset
         B, H, S, k_dim = keys.shape

@@ -472,6 +472,26 @@ def _check_rows(T: int, ragged: bool, n_seq: int, **tensors):
             raise ValueError(f"{name} holds {t.shape[0]} sequences, the query {n_seq}")
 
 
+def _check_offsets(seq_offsets: torch.Tensor, n_seq: int, validate: bool, **tensors) -> None:
+    """The kernels read seq_offsets as n_seq + 1 int32 values and trust them: sequence s occupies rows
+    seq_offsets[s] .. seq_offsets[s + 1] - 1 of the ragged tensors.  Dtype, count and layout are checked here
+    (an int64 tensor, torch.cumsum's default, would be read as int32 pairs: zero or negative lengths and
+    silently wrong outputs).  That the offsets start at >= 0, never decrease and end inside the tensors is the
+    caller's contract; validate=True checks it too, at the price of one device-to-host synchronisation."""
+    if (seq_offsets.dtype != torch.int32 or seq_offsets.dim() != 1 or seq_offsets.numel() != n_seq + 1
+            or not seq_offsets.is_contiguous()):
+        raise ValueError(f"seq_offsets must be a contiguous int32 tensor with n_seq + 1 = {n_seq + 1} entries, got "
+                         f"{seq_offsets.dtype} {tuple(seq_offsets.shape)}")
+    if validate:
+        off = seq_offsets.cpu().tolist()
+        if off[0] < 0 or any(b < a for a, b in zip(off, off[1:])):
+            raise ValueError("seq_offsets must start at >= 0 and never decrease")
+        for name, t in tensors.items():
+            rows = t.shape[-2] if name in ("k", "k_packed", "v_packed") else t.shape[-1]
+            if off[-1] > rows:
+                raise ValueError(f"seq_offsets end at row {off[-1]}, {name} holds {rows}")
+
+
 def _kv_layout(t: torch.Tensor, inner: int, ragged: bool):
     """Strides in rows for KV addressing.  Accepts [H, T, inner] (one sequence or ragged batch) or
     [B, H, T, inner] (cache layout); the last two axes must be row-contiguous."""
@@ -515,7 +535,8 @@ def flash_decode(q_rot: torch.Tensor, k_packed, k_norms, v_packed, v_norms, k_ce
                  v_signs, dim: int, bits: int, attn_scale: float, *, n_rep: int = 1, block_size: int = 16,
                  seq_len: int | None = None, seq_offsets: torch.Tensor | None = None,
                  max_seq_len: int | None = None, mask=None, out_dtype=torch.float32,
-                 precision: str = "fp16", sparse_v_threshold: float = 0.0) -> torch.Tensor:
+                 precision: str = "fp16", sparse_v_threshold: float = 0.0,
+                 validate_offsets: bool = False) -> torch.Tensor:
     """Batched form of flash_attention_turboquant (tq_flash_decode).
 
     sparse_v_threshold > 0: softmax weights below it are dropped from the value sum (the threshold of
@@ -527,7 +548,9 @@ def flash_decode(q_rot: torch.Tensor, k_packed, k_norms, v_packed, v_norms, k_ce
 
     q_rot (n_seq, n_q, dim) float32.  K/V either cache layout [n_seq, n_kv, T_alloc, *] with the
     uniform valid length `seq_len`, or ragged [n_kv, sum(L), *] with int32 `seq_offsets`
-    (n_seq + 1 entries on the GPU) and `max_seq_len`.  Returns (n_seq, n_q, dim) `out_dtype`.
+    (n_seq + 1 entries on the GPU, non-decreasing, ending inside the tensors: the caller's contract, checked
+    only with validate_offsets=True, which synchronises once) and `max_seq_len`.  Returns (n_seq, n_q, dim)
+    `out_dtype`.
     """
     _need_gpu(q_rot, k_packed, k_norms, v_packed, v_norms, seq_offsets)
     if dim > 128 or dim & (dim - 1):
@@ -547,8 +570,8 @@ def flash_decode(q_rot: torch.Tensor, k_packed, k_norms, v_packed, v_norms, k_ce
     if ragged:
         if max_seq_len is None:
             raise ValueError("max_seq_len is required with seq_offsets")
-        if seq_offsets.dtype != torch.int32 or seq_offsets.numel() != n_seq + 1:
-            raise ValueError("seq_offsets must be int32 with n_seq + 1 entries")
+        _check_offsets(seq_offsets, n_seq, validate_offsets, k_packed=k_packed, k_norms=k_norms, v_packed=v_packed,
+                       v_norms=v_norms)
         T = int(max_seq_len)
     else:
         T = int(seq_len if seq_len is not None else k_norms.shape[-1])
@@ -586,7 +609,7 @@ def flash_decode_from_q(q: torch.Tensor, k_signs, k_packed, k_norms, v_packed, v
                         v_signs, dim: int, bits: int, attn_scale: float, *, n_rep: int = 1,
                         seq_len: int | None = None, seq_offsets: torch.Tensor | None = None,
                         max_seq_len: int | None = None, mask=None, out_dtype=torch.float32,
-                        sparse_v_threshold: float = 0.0) -> torch.Tensor:
+                        sparse_v_threshold: float = 0.0, validate_offsets: bool = False) -> torch.Tensor:
     """The decode step of turboquant_attention (fused_attention.py:56-121) in ONE library call from the query
     itself: the pre-rotation of prerotate_query happens inside the attention kernels (tq_flash_decode_from_q).
     q (n_seq, n_q, dim) fp16 / bf16 / float32; other arguments as flash_decode.  Matrix-core shapes only
@@ -609,8 +632,8 @@ def flash_decode_from_q(q: torch.Tensor, k_signs, k_packed, k_norms, v_packed, v
     if ragged:
         if max_seq_len is None:
             raise ValueError("max_seq_len is required with seq_offsets")
-        if seq_offsets.dtype != torch.int32 or seq_offsets.numel() != n_seq + 1:
-            raise ValueError("seq_offsets must be int32 with n_seq + 1 entries")
+        _check_offsets(seq_offsets, n_seq, validate_offsets, k_packed=k_packed, k_norms=k_norms, v_packed=v_packed,
+                       v_norms=v_norms)
         T = int(max_seq_len)
     else:
         T = int(seq_len if seq_len is not None else k_norms.shape[-1])
@@ -657,7 +680,8 @@ def vonly_decode(q: torch.Tensor, k: torch.Tensor, v_packed, v_norms, v_centroid
                  bits: int, attn_scale: float, *, n_rep: int = 1, seq_len: int | None = None,
                  seq_offsets: torch.Tensor | None = None, max_seq_len: int | None = None, mask=None,
                  out_dtype=torch.float32, precision: str = "fp16", sparse_v_threshold: float = 0.0,
-                 out: torch.Tensor | None = None, static_scratch: bool = False) -> torch.Tensor:
+                 out: torch.Tensor | None = None, static_scratch: bool = False,
+                 validate_offsets: bool = False) -> torch.Tensor:
     """Dense-softmax decode attention over fp16 keys and packed values (tq_vonly_decode_attn).
     precision as in flash_decode (on the matrix-core path fp16 queries enter as they are, bf16 converted to
     fp16, float32 as an fp16 value plus the fp16 remainder of that rounding).
@@ -692,6 +716,7 @@ def vonly_decode(q: torch.Tensor, k: torch.Tensor, v_packed, v_norms, v_centroid
     if ragged:
         if max_seq_len is None:
             raise ValueError("max_seq_len is required with seq_offsets")
+        _check_offsets(seq_offsets, n_seq, validate_offsets, k=k, v_packed=v_packed, v_norms=v_norms)
         T = int(max_seq_len)
     else:
         T = int(seq_len if seq_len is not None else v_norms.shape[-1])
@@ -780,6 +805,7 @@ class VOnlyStep:
         self.desc = d
         self._ref = C.byref(d)
         self._need = _lib.load().tq_workspace_bytes(_lib.TQ_OP_VONLY_DECODE, B, H * n_rep, T, D)
+        self._ws, self._ws_refs = None, []
 
 
 def vonly_decode_step(step: VOnlyStep, keys: torch.Tensor, values: torch.Tensor, q: torch.Tensor, position,
@@ -813,9 +839,7 @@ def vonly_decode_step(step: VOnlyStep, keys: torch.Tensor, values: torch.Tensor,
     elif tuple(out.shape) != (B, n_q, D) or not out.is_contiguous():
         raise ValueError(f"out must be a contiguous {(B, n_q, D)} tensor")
     stream = _stream(q)
-    ws = _workspace(q.device, stream.value or 0, step._need)
-    d = step.desc
-    d.workspace, d.workspace_bytes = ws.data_ptr(), ws.numel()
+    _step_workspace(step, q.device, stream.value or 0)
     lib = _lib.load()
     if on_device:
         _lib.check(lib.tq_vonly_decode_step_at(
@@ -828,15 +852,24 @@ def vonly_decode_step(step: VOnlyStep, keys: torch.Tensor, values: torch.Tensor,
     return out
 
 
+def _step_workspace(step, device, stream_id: int) -> None:
+    """Point the descriptor at the (device, stream) workspace.  The descriptor keeps every buffer it has ever
+    handed to the library alive: a call recorded in a HIP graph has the address baked in, and the shared
+    buffer is replaced (not grown in place) when a later, larger op needs more."""
+    ws = _workspace(device, stream_id, step._need)
+    if step._ws is not ws:
+        step._ws_refs.append(ws)
+        step._ws = ws
+        step.desc.workspace, step.desc.workspace_bytes = ws.data_ptr(), ws.numel()
+
+
 def step_call_unchecked(step, keys: torch.Tensor, values: torch.Tensor, q: torch.Tensor, position, attn_scale: float,
                         out: torch.Tensor, packed: bool) -> None:
     """The library call of vonly_decode_step / packed_decode_step without their argument checks, for the cache
     objects, which have established shapes, dtypes and devices themselves: keys / values / q / out are contiguous
     and hold (B, heads, dim) elements in any view of that memory (a (B, heads, 1, dim) tensor qualifies)."""
     stream = _stream(q)
-    ws = _workspace(q.device, stream.value or 0, step._need)
-    d = step.desc
-    d.workspace, d.workspace_bytes = ws.data_ptr(), ws.numel()
+    _step_workspace(step, q.device, stream.value or 0)
     lib = _lib.load()
     if isinstance(position, torch.Tensor):
         fn = lib.tq_packed_decode_step_at if packed else lib.tq_vonly_decode_step_at
@@ -891,6 +924,7 @@ class PackedStep:
         self.desc = d
         self._ref = C.byref(d)
         self._need = _lib.load().tq_workspace_bytes(_lib.TQ_OP_FLASH_DECODE, B, H * n_rep, T, dim)
+        self._ws, self._ws_refs = None, []
 
 
 def packed_decode_step(step: PackedStep, keys: torch.Tensor, values: torch.Tensor, q: torch.Tensor, position,
@@ -918,9 +952,7 @@ def packed_decode_step(step: PackedStep, keys: torch.Tensor, values: torch.Tenso
     elif tuple(out.shape) != (B, n_q, D) or not out.is_contiguous():
         raise ValueError(f"out must be a contiguous {(B, n_q, D)} tensor")
     stream = _stream(q)
-    ws = _workspace(q.device, stream.value or 0, step._need)
-    d = step.desc
-    d.workspace, d.workspace_bytes = ws.data_ptr(), ws.numel()
+    _step_workspace(step, q.device, stream.value or 0)
     lib = _lib.load()
     fn = lib.tq_packed_decode_step_at if on_device else lib.tq_packed_decode_step
     _lib.check(fn(step._ref, _ptr(keys), _dt(keys), _ptr(values), _dt(values), _ptr(q), _dt(q), _ptr(out), _dt(out),

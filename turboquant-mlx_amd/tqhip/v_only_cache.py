@@ -4,7 +4,7 @@ from __future__ import annotations
 
 import torch
 
-from .cache import TurboQuantKVCache
+from .cache import TurboQuantKVCache, _round_up
 from .kvcache import KVCache
 
 
@@ -19,9 +19,11 @@ class VOnlyTurboQuantCache:
     packed values directly (vonly_decode_attention, tqhip.patch); `dequantized_values()` gives the
     fp16 values when a multi-token step needs them."""
 
-    def __init__(self, bits: int = 3, seed: int = 42, no_v_buffer: bool = False, fused: bool = False):
+    def __init__(self, bits: int = 3, seed: int = 42, no_v_buffer: bool = False, fused: bool = False, v_signs=None):
+        """v_signs ([dim] of +-1): the value rotation's sign vector, used instead of the one derived from
+        `seed + 1` (cache.py:96).  Everything else as the reference (v_only_cache.py:41-49) plus `fused`."""
         self._k_cache = KVCache()
-        self._v_tq = TurboQuantKVCache(bits=bits, seed=seed, v_only=True)
+        self._v_tq = TurboQuantKVCache(bits=bits, seed=seed, v_only=True, v_signs=v_signs)
         self._v_bits = bits
         self._no_v_buffer = no_v_buffer
         self.fused = fused
@@ -37,6 +39,26 @@ class VOnlyTurboQuantCache:
         tq._encode(values, tq._v_q, tq.v_packed, tq.v_norms, B, H, S, v_dim, tq.offset)
         tq.offset += S
 
+    def _align_storage(self, B, H, S, dim, v_dtype, device):
+        """Room for S more positions with ONE capacity for the key cache and the packed values, both
+        contiguous: the single-call decode step describes all four tensors by one t_alloc.  The two storages
+        grow by different rules when they are filled through their own update_and_fetch (the key cache trims
+        to its offset and appends whole steps, the packed storage rounds offset + S up to a step) or are
+        restored from `state` slices, so they are brought to round_up(max(needed, either capacity), 256)
+        here; nothing moves when they already agree and have room."""
+        kc, tq = self._k_cache, self._v_tq
+        need = kc.offset + S
+        have_k = 0 if kc.keys is None else kc.keys.shape[2]
+        have_v = 0 if tq.v_packed is None else tq.v_packed.shape[2]
+        n = _round_up(max(need, have_k, have_v), tq.step)
+        if (have_k != n or not kc.keys.is_contiguous() or not kc.values.is_contiguous()
+                or kc.keys.dtype != torch.float16 or kc.values.dtype != v_dtype):
+            if kc.keys is not None and (kc.keys.dtype != torch.float16 or kc.values.dtype != v_dtype):
+                raise ValueError("the stored keys must be float16 and the stored values of the new values' dtype")
+            kc.reallocate(B, H, n, dim, dim, torch.float16, v_dtype, device)
+        if have_v != n or not tq.v_packed.is_contiguous() or not tq.v_norms.is_contiguous():
+            tq._reallocate(B, H, n, device)
+
     # Decode-sized inserts of a fused cache go through one launch (key rows to float16, value rows
     # raw and encoded) instead of two slice assignments, a cast and the encoder.
     _FUSED_APPEND_MAX_TOKENS = 16
@@ -50,13 +72,9 @@ class VOnlyTurboQuantCache:
                 or (kc.keys is not None and kc.keys.dtype != torch.float16)
                 or kc.offset != tq.offset):
             return False
-        kc.reserve(B, H, S, keys.shape[3], v_dim, torch.float16, values.dtype, values.device)
         tq._dtype = keys.dtype
         tq._ensure_quantizer(keys.shape[-1], v_dim, values.device)
-        tq._ensure_storage(B, H, S, values.device)
-        if not (kc.keys.is_contiguous() and kc.values.is_contiguous() and tq.v_packed.is_contiguous()
-                and tq.v_norms.is_contiguous()):
-            return False                  # storage handed in through `state` as slices: the general path copes
+        self._align_storage(B, H, S, v_dim, values.dtype, values.device)
         ops.vonly_append_into(keys, values, tq._v_q.signs, tq._v_q.boundaries, kc.keys, kc.values,
                               tq.v_packed, tq.v_norms, position=kc.offset, bits=tq.quant_bits,
                               variant=tq.encode_variant)
@@ -70,17 +88,16 @@ class VOnlyTurboQuantCache:
         kc, tq = self._k_cache, self._v_tq
         device = torch.device(device)
         tq._ensure_quantizer(dim, dim, device)
-        need = kc.offset + n_positions
-        have = 0 if kc.keys is None else kc.keys.shape[2]
-        if need > have:
-            kc.reserve(B, H, need - kc.offset, dim, dim, torch.float16, dtype, device)
-        if tq.v_packed is None or need > tq.v_packed.shape[2]:
-            tq._ensure_storage(B, H, need - tq.offset, device)
+        if kc.offset != tq.offset:
+            raise ValueError("keys and values hold different numbers of positions")
+        self._align_storage(B, H, n_positions, dim, dtype if kc.values is None else kc.values.dtype, device)
 
     def set_offset(self, n: int):
         """Set the number of valid positions (keys and values alike): for a caller that replayed recorded steps
         with a device-side position and now tells the host-side bookkeeping how far the cache has got."""
-        if not 0 <= n <= (0 if self._k_cache.keys is None else self._k_cache.keys.shape[2]):
+        have_k = 0 if self._k_cache.keys is None else self._k_cache.keys.shape[2]
+        have_v = 0 if self._v_tq.v_packed is None else self._v_tq.v_packed.shape[2]
+        if not 0 <= n <= min(have_k, have_v):
             raise ValueError(f"offset {n} outside the storage")
         self._k_cache.offset = n
         self._v_tq.offset = n
@@ -111,10 +128,9 @@ class VOnlyTurboQuantCache:
                                  "queries and a cache whose stored values have the dtype of the new ones")
             self.update_and_fetch(keys, values)
             return attention.vonly_decode_attention(queries, self, attn_scale)
-        kc.reserve(B, H, 1, dim, dim, torch.float16, values.dtype, values.device)
         tq._dtype = keys.dtype
         tq._ensure_quantizer(dim, dim, values.device)
-        tq._ensure_storage(B, H, 1, values.device)
+        self._align_storage(B, H, 1, dim, values.dtype, values.device)
         key = (kc.keys.data_ptr(), kc.values.data_ptr(), tq.v_packed.data_ptr(), tq.v_norms.data_ptr(),
                kc.keys.shape[2], n_q)
         if self._step_key != key:
@@ -122,7 +138,7 @@ class VOnlyTurboQuantCache:
                 self._step = ops.VOnlyStep(kc.keys, kc.values, tq.v_packed, tq.v_norms, tq._v_q.signs,
                                            tq._v_q.boundaries, tq._v_q.centroids, n_rep=n_q // H,
                                            bits=tq.quant_bits, variant=tq.encode_variant)
-            except ValueError:                     # storage handed in through `state` as slices
+            except ValueError:                     # a shape the single call does not serve
                 if position is not None:
                     raise
                 self.update_and_fetch(keys, values)
@@ -198,18 +214,25 @@ class VOnlyTurboQuantCache:
         return f"VOnlyTQ,{self._v_bits},{self._v_tq.seed},{self._v_tq.meta_state}"
 
     @classmethod
-    def from_state(cls, state, meta_state):
-        parts = meta_state.split(",", 3)                        # v_only_cache.py:95-111
+    def from_state(cls, state, meta_state, v_signs=None):
+        """v_only_cache.py:95-111.  The serialised cache carries its seed, not its sign vector: pass the
+        v_signs the cache was written with when they were given explicitly (or come from the reference,
+        whose seed-to-signs generator is MLX's)."""
+        parts = meta_state.split(",", 3)
         bits = int(parts[1])
         seed = int(parts[2])
-        obj = cls(bits=bits, seed=seed)
+        obj = cls(bits=bits, seed=seed, v_signs=v_signs)
         if len(state) >= 2:
             obj._k_cache.keys = state[0]
             obj._k_cache.values = state[1]
             obj._k_cache.offset = state[0].shape[2]
         if len(state) > 2:
-            obj._v_tq.state = state[2:]
-            obj._v_tq.meta_state = parts[3]
+            tq = obj._v_tq
+            tq.state = state[2:]
+            tq.meta_state = parts[3]
+            tq._v_pdim = tq.v_packed.shape[-1]
+            if tq._v_dim is not None:                     # usable at once (attention straight off the restored cache),
+                tq._ensure_quantizer(tq._v_dim, tq._v_dim, tq.v_packed.device)   # not only after the next insert
         return obj
 
     @classmethod
