@@ -781,13 +781,6 @@ int launch_vonly_mfma(const void* q, int q_dtype, const void* k_f16, const uint3
   a.mask_seq_stride = sh.mask_seq_stride; a.mask_head_stride = sh.mask_head_stride;
   a.n_kv = sh.n_kv_heads; a.n_rep = sh.n_rep; a.n_tiles_max = n_tiles;
   a.attn_scale = sh.attn_scale;
-#ifdef TQ_TRACE
-  {  // timeline goes behind the regular workspace when the caller left room for it
-    const size_t tbytes = (size_t)n_tiles * sh.n_kv_heads * sh.n_seq * 16 * sizeof(unsigned long long);
-    const size_t off = (need + 255) / 256 * 256;
-    a.trace = (workspace_bytes >= off + tbytes) ? (unsigned long long*)((char*)workspace + off) : nullptr;
-  }
-#endif
   Codebook vcb;
   a.v_unscale = tq::fill_codebook_fp16(vcb, v_centroids, sh.bits);
   if ((phases & 1) && n_tiles_real > 0) {

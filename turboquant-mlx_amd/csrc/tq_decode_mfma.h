@@ -76,34 +76,7 @@ struct MfmaArgs {
   int32_t q_bf16;
   float* scores;              // vonly_scores_kernel: [n_seq * n_q, scores_stride] f32, log2 units
   int64_t scores_stride;      // floats per score row (a multiple of 4)
-#ifdef TQ_TRACE
-  unsigned long long* trace;
-#endif
 };
-
-// Optional phase timeline for tuning (compile with -DTQ_TRACE): thread 0 of every workgroup
-// stores the 100 MHz real-time counter at each phase boundary into a.trace[workgroup][16].
-#ifdef TQ_TRACE
-#define TQ_STAMP(slot)                                                                              \
-  do {                                                                                              \
-    if (a.trace && threadIdx.x == 0)                                                                \
-      a.trace[((blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 16 + (slot)] =     \
-          __builtin_amdgcn_s_memrealtime();                                                         \
-  } while (0)
-// per-wave variant: lane 0 of wave w > 0 writes slot `base_slot_of[w]` (spare slots of the record)
-#define TQ_STAMP_WAVE()                                                                             \
-  do {                                                                                              \
-    const int w_ = threadIdx.x >> 6;                                                                \
-    if (a.trace && (threadIdx.x & 63) == 0 && w_ > 0) {                                             \
-      const int slot_ = (w_ <= 3) ? 3 + w_ : 7 + w_;          /* waves 1..3 -> 4..6, 4..7 -> 11..14 */ \
-      a.trace[((blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 16 + slot_] =      \
-          __builtin_amdgcn_s_memrealtime();                                                         \
-    }                                                                                               \
-  } while (0)
-#else
-#define TQ_STAMP(slot) do {} while (0)
-#define TQ_STAMP_WAVE() do {} while (0)
-#endif
 
 // additive mask of four consecutive positions row0 .. row0 + 3 of one head: one 16-byte load where the row is
 // aligned and the positions are inside the tile, else element by element; positions past the tile read as 0
@@ -122,6 +95,72 @@ __device__ __forceinline__ void load_mask4(const float* src, int row0, int rows_
 __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
   __half2 h = __floats2half2_rn(a, b);
   return *reinterpret_cast<uint32_t*>(&h);
+}
+
+// Cross-wave merge of a workgroup's tile.  Every wave leaves, per head, the maximum m of its scores (log2 units)
+// and its weight sum l, its power-of-two accumulator scale, and its RAW accumulator rows in an LDS area of its
+// own (`area`, 4 KB: eight rows of 128 floats; nothing of another wave lives there, so no barrier is needed
+// before the deposit).  After ONE barrier one thread per (head, four elements) folds the NW deposits with the
+// factors 2^(m_w - M) * scale_w, which it derives itself: NW exponentials per thread instead of two more
+// barriers around a shared table of factors.  The partial of the tile goes to pS / pml.
+template <int NW>
+struct MergeLds {
+  float m[kHeadsMax][NW];
+  float l[kHeadsMax][NW];
+  float ts[NW];
+};
+
+template <int NW>
+__device__ __forceinline__ void merge_waves(MergeLds<NW>& mg, unsigned char* areas, int area_stride, const f4 (&accS)[8],
+                                            float m, float l, float inv_tscale, float v_unscale, int n_rep,
+                                            float* __restrict__ pS, float* __restrict__ pml) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n16 = lane & 15, g = lane >> 4;
+  if (g == 0) {
+    mg.m[n16][wave] = m;
+    mg.l[n16][wave] = l;
+  }
+  if (lane == 0) mg.ts[wave] = inv_tscale;
+  float (*mine)[kD] = reinterpret_cast<float (*)[kD]>(areas + wave * area_stride);
+  for (int h0 = 0; h0 < n_rep; h0 += 8) {
+    if (h0) __syncthreads();                             // the previous round has been summed
+    if ((g >> 1) == (h0 >> 3)) {                         // lanes whose rows 4g+j fall in this round
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float4* dst = reinterpret_cast<float4*>(&mine[(4 * g + j) & 7][8 * n16]);
+        dst[0] = make_float4(accS[0][j], accS[1][j], accS[2][j], accS[3][j]);
+        dst[1] = make_float4(accS[4][j], accS[5][j], accS[6][j], accS[7][j]);
+      }
+    }
+    __syncthreads();
+    const int rows = min(8, n_rep - h0);
+    if (tid < rows * (kD / 4)) {                         // one float4 of one head per thread
+      const int hl = tid >> 5, e4 = tid & 31, h = h0 + hl;
+      float mw[NW], fw[NW];
+      float M = -INFINITY;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) {
+        mw[w] = mg.m[h][w];
+        M = fmaxf(M, mw[w]);
+      }
+      float L = 0.0f;
+      f4 sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int w = 0; w < NW; ++w) {
+        const float e = (mw[w] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(mw[w] - M);
+        fw[w] = e * mg.ts[w];
+        L += e * mg.l[h][w];
+        const f4 x = *reinterpret_cast<const f4*>(areas + w * area_stride + (hl * kD + 4 * e4) * 4);
+        sum = sum + x * fw[w];
+      }
+      sum = sum * v_unscale;
+      *reinterpret_cast<f4*>(pS + h * kD + 4 * e4) = sum;
+      if (e4 == 0) {
+        pml[2 * h] = M;
+        pml[2 * h + 1] = L;
+      }
+    }
+  }
 }
 
 // grid = (n_tiles_max, n_kv, n_seq), NW * 64 threads: a workgroup of NW waves owns NW * 64 consecutive positions.
@@ -145,8 +184,7 @@ __device__ __forceinline__ void vonly_tile_body(const MfmaArgs& a, const Codeboo
   __shared__ __align__(16) uint32_t q_s[kHeadsMax][kD / 2];   // fp16 pairs, rows >= n_rep are zero
   __shared__ __align__(16) uint32_t ql_s[QF32 ? kHeadsMax : 1][kD / 2];   // QF32: what rounding the query to fp16 lost
   __shared__ __align__(16) float nrm_s[NW][kWavePos];
-  __shared__ float m_s[NW][kHeadsMax], l_s[NW][kHeadsMax], M_s[kHeadsMax];
-  __shared__ __align__(16) float f_s[NW][kHeadsMax];
+  __shared__ __align__(16) MergeLds<NW> mg_s;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -157,7 +195,6 @@ __device__ __forceinline__ void vonly_tile_body(const MfmaArgs& a, const Codeboo
   const int64_t q_row0 = (int64_t)seq * n_q + (int64_t)kvh * n_rep;
 
   const int64_t tile_p0 = (int64_t)tile * kTPos;
-  TQ_STAMP(0);
   if (tile_p0 >= len) return;                          // the merge pass never reads this tile
   const int rows_here = PLAIN ? kTPos : (int)min((int64_t)kTPos, len - tile_p0);   // valid rows of this tile
   const int last_row = rows_here - 1;
@@ -179,7 +216,6 @@ __device__ __forceinline__ void vonly_tile_body(const MfmaArgs& a, const Codeboo
       my_ql[i] = pack_h2(f.x - back.x, f.y - back.y);
     } else {
       my_q[i] = (w < n_rep * (kD / 2)) ? reinterpret_cast<const uint32_t*>(a.q + q_row0 * kD)[w] : 0u;
-      if (a.q_bf16) my_q[i] = pack_h2(__uint_as_float(my_q[i] << 16), __uint_as_float(my_q[i] & 0xFFFF0000u));
     }
   }
   float my_norm;
@@ -244,7 +280,6 @@ __device__ __forceinline__ void vonly_tile_body(const MfmaArgs& a, const Codeboo
 #pragma unroll
   for (int i = 0; i < 8; ++i) issue_k(i);
   __builtin_amdgcn_sched_barrier(0);
-  TQ_STAMP(15);
   if (tid < 64) {
     float clo = 0.0f, chi = 0.0f;                        // selects, not a dynamic index into kernel arguments
 #pragma unroll
@@ -256,12 +291,14 @@ __device__ __forceinline__ void vonly_tile_body(const MfmaArgs& a, const Codeboo
   }
 #pragma unroll
   for (int i = 0; i < kQIt; ++i) {
+    // bf16 queries become fp16 here, after every load of the pass has been requested: converting where the word
+    // is loaded would wait for it before anything else is in flight
+    if (!QF32 && a.q_bf16) my_q[i] = pack_h2(__uint_as_float(my_q[i] << 16), __uint_as_float(my_q[i] & 0xFFFF0000u));
     (&q_s[0][0])[tid + i * kThr] = my_q[i];
     if (QF32) (&ql_s[0][0])[tid + i * kThr] = my_ql[i];
   }
   nrm_s[wave][lane] = my_norm;
   __syncthreads();
-  TQ_STAMP(1);
 
   // ---- Q operand and the V norms of this lane's 16 positions ----------------------------------------
   u4 qreg[4], qlow[4];
@@ -377,11 +414,9 @@ __device__ __forceinline__ void vonly_tile_body(const MfmaArgs& a, const Codeboo
 #pragma unroll
   for (int i = 12; i < 16; ++i) issue_k(i);
   __builtin_amdgcn_sched_barrier(0);
-  TQ_STAMP(7);
   qk_tile(1);
   qk_tile(2);
   qk_tile(3);
-  TQ_STAMP(2);
 
   // ---- softmax statistics of head n16 over the wave's 64 positions ----------------------------------
   float m = -INFINITY;
@@ -426,71 +461,12 @@ __device__ __forceinline__ void vonly_tile_body(const MfmaArgs& a, const Codeboo
       accS[et] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, A), __builtin_bit_cast(h8, breg[kb2][et]),
                                                         accS[et], 0, 0, 0);
   }
-  TQ_STAMP(3);
-  TQ_STAMP_WAVE();
 
-  // ---- merge the eight waves ----------------------------------------------------------------------------
-  // (1) every wave publishes (m, l) per head; (2) 128 threads turn them into one factor
-  // e^(m_w - M_h) per (wave, head); (3) every wave scales its own accumulator rows by its factors
-  // and deposits them; (4) a float4 sum over the eight deposits goes to the workspace.  The
-  // exponentials are evaluated once per (wave, head), not once per element.
-  float (*S_all)[8][kD] = reinterpret_cast<float (*)[8][kD]>(big_s);    // [wave][head in round][128]: NW x 4 KB
+  // ---- merge the waves of the workgroup (merge_waves): one partial per workgroup goes to the workspace -----------
   const int64_t grp = (int64_t)seq * a.n_kv + kvh;
   float* pS = a.ws_S + (grp * a.n_tiles_max + tile) * (int64_t)(n_rep * kD);
   float* pml = a.ws_ml + (grp * a.n_tiles_max + tile) * (int64_t)(n_rep * 2);
-  if (g == 0) {
-    m_s[wave][n16] = m;
-    l_s[wave][n16] = l;
-  }
-  __syncthreads();                                       // (m, l) visible; the staging area is free
-  if (tid < NW * kHeadsMax) {
-    const int w = tid >> 4, h = tid & 15;
-    float M = m_s[0][h];
-#pragma unroll
-    for (int ww = 1; ww < NW; ++ww) M = fmaxf(M, m_s[ww][h]);
-    const float mw = m_s[w][h];
-    f_s[w][h] = (mw == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(mw - M);
-    if (w == 0) M_s[h] = M;
-  }
-  __syncthreads();
-  TQ_STAMP(8);
-  const float4 f4own = *reinterpret_cast<const float4*>(&f_s[wave][4 * g]);   // heads 4g .. 4g+3 of this lane's rows
-  const float wscale = inv_tscale * a.v_unscale;
-  const float fown[4] = {f4own.x * wscale, f4own.y * wscale, f4own.z * wscale, f4own.w * wscale};
-  for (int h0 = 0; h0 < n_rep; h0 += 8) {
-    if (h0) __syncthreads();                             // the previous round has been summed
-    if ((g >> 1) == (h0 >> 3)) {                         // lanes whose rows 4g+j fall in this round
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        float4* dst = reinterpret_cast<float4*>(&S_all[wave][(4 * g + j) & 7][8 * n16]);
-        const float f = fown[j];
-        dst[0] = make_float4(accS[0][j] * f, accS[1][j] * f, accS[2][j] * f, accS[3][j] * f);
-        dst[1] = make_float4(accS[4][j] * f, accS[5][j] * f, accS[6][j] * f, accS[7][j] * f);
-      }
-    }
-    __syncthreads();
-    const int rows = min(8, n_rep - h0);
-    if (tid < rows * (kD / 4)) {                         // one float4 of one head per thread
-      const int hl = tid >> 5, e4 = tid & 31;
-      float4 sum = *reinterpret_cast<const float4*>(&S_all[0][hl][4 * e4]);
-#pragma unroll
-      for (int w = 1; w < NW; ++w) {
-        const float4 x = *reinterpret_cast<const float4*>(&S_all[w][hl][4 * e4]);
-        sum.x += x.x; sum.y += x.y; sum.z += x.z; sum.w += x.w;
-      }
-      *reinterpret_cast<float4*>(pS + (h0 + hl) * kD + 4 * e4) = sum;
-    }
-  }
-  TQ_STAMP(9);
-  if (tid < n_rep) {
-    const int h = tid;
-    float L = 0.0f;
-#pragma unroll
-    for (int w = 0; w < NW; ++w) L += f_s[w][h] * l_s[w][h];
-    pml[2 * h] = M_s[h];
-    pml[2 * h + 1] = L;
-  }
-  TQ_STAMP(10);
+  merge_waves<NW>(mg_s, big_s, 4096, accS, m, l, inv_tscale, a.v_unscale, n_rep, pS, pml);
 }
 
 template <bool PLAIN, bool QF32, int NW>
@@ -574,7 +550,6 @@ __global__ __launch_bounds__(WAVES * 64) void vonly_scores_kernel(MfmaArgs a) {
       my_ql[i] = pack_h2(f.x - back.x, f.y - back.y);
     } else {
       my_q[i] = (w < n_rep * (kD / 2)) ? reinterpret_cast<const uint32_t*>(a.q + q_row0 * kD)[w] : 0u;
-      if (a.q_bf16) my_q[i] = pack_h2(__uint_as_float(my_q[i] << 16), __uint_as_float(my_q[i] & 0xFFFF0000u));
     }
   }
   // K: instruction i reads rows 4i .. 4i+3 of the wave (1 KB contiguous); lane L takes 16-byte piece
@@ -592,6 +567,9 @@ __global__ __launch_bounds__(WAVES * 64) void vonly_scores_kernel(MfmaArgs a) {
   }
 #pragma unroll
   for (int i = 0; i < kQIt; ++i) {
+    // bf16 queries become fp16 here, after every load of the pass has been requested: converting where the word
+    // is loaded would wait for it before anything else is in flight
+    if (!QF32 && a.q_bf16) my_q[i] = pack_h2(__uint_as_float(my_q[i] << 16), __uint_as_float(my_q[i] & 0xFFFF0000u));
     (&q_s[0][0])[tid + i * kThr] = my_q[i];
     if (QF32) (&ql_s[0][0])[tid + i * kThr] = my_ql[i];
   }
@@ -719,8 +697,7 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
   __shared__ __align__(16) uint32_t ql_s[QF32 ? kHeadsMax : 1][kD / 2];
   __shared__ __align__(16) float nrm_s[kWaves][kStepPos];
   __shared__ __align__(16) float alpha_s[kWaves][kHeadsMax];
-  __shared__ float m_s[kWaves][kHeadsMax], l_s[kWaves][kHeadsMax], M_s[kHeadsMax];
-  __shared__ __align__(16) float f_s[kWaves][kHeadsMax];
+  __shared__ __align__(16) MergeLds<kWaves> mg_s;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -794,7 +771,6 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
       my_ql[i] = pack_h2(f.x - back.x, f.y - back.y);
     } else {
       my_q[i] = (w < n_rep * (kD / 2)) ? reinterpret_cast<const uint32_t*>(a.q + q_row0 * kD)[w] : 0u;
-      if (a.q_bf16) my_q[i] = pack_h2(__uint_as_float(my_q[i] << 16), __uint_as_float(my_q[i] & 0xFFFF0000u));
     }
   }
   float nrmA, nrmB = 0.0f;
@@ -818,6 +794,9 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
   }
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
+    // bf16 queries become fp16 here, after every load of the pass has been requested: converting where the word
+    // is loaded would wait for it before anything else is in flight
+    if (!QF32 && a.q_bf16) my_q[i] = pack_h2(__uint_as_float(my_q[i] << 16), __uint_as_float(my_q[i] & 0xFFFF0000u));
     (&q_s[0][0])[tid + i * kMfmaThreads] = my_q[i];
     if (QF32) (&ql_s[0][0])[tid + i * kMfmaThreads] = my_ql[i];
   }
@@ -970,66 +949,16 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
     });
   }
 
-  // ---- merge the eight waves (as in vonly_tile_mfma_kernel): m is the running maximum, the weight sum
-  // and the accumulators carry 2^kexp of the last step
+  // ---- merge the eight waves (merge_waves): m is the running maximum, the weight sum and the accumulators carry
+  // 2^kexp of the last step
   float l = l_run;
   l += shfl_xor_f(l, 16);
   l += shfl_xor_f(l, 32);
   l *= inv_tscale;
-  const float m = m_run;
-  float (*S_all)[8][kD] = reinterpret_cast<float (*)[8][kD]>(big_s);
   const int64_t grp = (int64_t)seq * a.n_kv + kvh;
   float* pS = a.ws_S + (grp * a.n_tiles_max + tile) * (int64_t)(n_rep * kD);
   float* pml = a.ws_ml + (grp * a.n_tiles_max + tile) * (int64_t)(n_rep * 2);
-  if (g == 0) {
-    m_s[wave][n16] = m;
-    l_s[wave][n16] = l;
-  }
-  __syncthreads();
-  if (tid < kWaves * kHeadsMax) {
-    const int w = tid >> 4, h = tid & 15;
-    float M = m_s[0][h];
-#pragma unroll
-    for (int ww = 1; ww < kWaves; ++ww) M = fmaxf(M, m_s[ww][h]);
-    f_s[w][h] = __builtin_amdgcn_exp2f(m_s[w][h] - M);
-    if (w == 0) M_s[h] = M;
-  }
-  __syncthreads();
-  const float4 f4own = *reinterpret_cast<const float4*>(&f_s[wave][4 * g]);
-  const float wscale = inv_tscale * a.v_unscale;
-  const float fown[4] = {f4own.x * wscale, f4own.y * wscale, f4own.z * wscale, f4own.w * wscale};
-  for (int h0 = 0; h0 < n_rep; h0 += 8) {
-    if (h0) __syncthreads();
-    if ((g >> 1) == (h0 >> 3)) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        float4* dst = reinterpret_cast<float4*>(&S_all[wave][(4 * g + j) & 7][8 * n16]);
-        const float f = fown[j];
-        dst[0] = make_float4(accS[0][j] * f, accS[1][j] * f, accS[2][j] * f, accS[3][j] * f);
-        dst[1] = make_float4(accS[4][j] * f, accS[5][j] * f, accS[6][j] * f, accS[7][j] * f);
-      }
-    }
-    __syncthreads();
-    const int rows = min(8, n_rep - h0);
-    if (tid < rows * (kD / 4)) {
-      const int hl = tid >> 5, e4 = tid & 31;
-      float4 sum = *reinterpret_cast<const float4*>(&S_all[0][hl][4 * e4]);
-#pragma unroll
-      for (int w = 1; w < kWaves; ++w) {
-        const float4 x = *reinterpret_cast<const float4*>(&S_all[w][hl][4 * e4]);
-        sum.x += x.x; sum.y += x.y; sum.z += x.z; sum.w += x.w;
-      }
-      *reinterpret_cast<float4*>(pS + (h0 + hl) * kD + 4 * e4) = sum;
-    }
-  }
-  if (tid < n_rep) {
-    const int h = tid;
-    float L = 0.0f;
-#pragma unroll
-    for (int w = 0; w < kWaves; ++w) L += f_s[w][h] * l_s[w][h];
-    pml[2 * h] = M_s[h];
-    pml[2 * h + 1] = L;
-  }
+  merge_waves<kWaves>(mg_s, big_s, 4096, accS, m_run, l, inv_tscale, a.v_unscale, n_rep, pS, pml);
 }
 
 // The token a decode step inserts, handled by the merge pass instead of a launch of its own ahead of the

@@ -166,7 +166,7 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
   __shared__ __align__(16) uint32_t ql_s[kHeadsMax][kD / 2];     // ... and what the rounding lost
   __shared__ __align__(16) float kn_s[kWaves][kWavePos], vn_s[kWaves][kWavePos];
   __shared__ float m_s[kWaves][kHeadsMax], l_s[kWaves][kHeadsMax], M_s[kHeadsMax];
-  __shared__ __align__(16) float f_s[kWaves][kHeadsMax];
+  __shared__ __align__(16) MergeLds<kWaves> mg_s;
   __shared__ float iL_s[kHeadsMax];
 
   const int tid = threadIdx.x;
@@ -514,62 +514,11 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
     }
   }
 
-  // ---- merge the eight waves, as in the dense-key kernel: one factor per (wave, head), scaled deposits,
-  // float4 sum -------------------------------------------------------------------------------------------
-  float (*S_all)[8][kD] = reinterpret_cast<float (*)[8][kD]>(big_s);
+  // ---- merge the eight waves (merge_waves, tq_decode_mfma.h) ------------------------------------------------
   const int64_t grp = (int64_t)seq * a.n_kv + kvh;
   float* pS = a.ws_S + (grp * a.n_tiles_max + tile) * (int64_t)(n_rep * kD);
   float* pml = a.ws_ml + (grp * a.n_tiles_max + tile) * (int64_t)(n_rep * 2);
-  if (g == 0) {
-    m_s[wave][n16] = m;
-    l_s[wave][n16] = l;
-  }
-  __syncthreads();
-  if (tid < kWaves * kHeadsMax) {
-    const int w = tid >> 4, h = tid & 15;
-    float M = m_s[0][h];
-#pragma unroll
-    for (int ww = 1; ww < kWaves; ++ww) M = fmaxf(M, m_s[ww][h]);
-    const float mw = m_s[w][h];
-    f_s[w][h] = (mw == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(mw - M);
-    if (w == 0) M_s[h] = M;
-  }
-  __syncthreads();
-  const float4 f4own = *reinterpret_cast<const float4*>(&f_s[wave][4 * g]);
-  const float wscale = inv_tscale * a.v_unscale;
-  const float fown[4] = {f4own.x * wscale, f4own.y * wscale, f4own.z * wscale, f4own.w * wscale};
-  for (int h0 = 0; h0 < n_rep; h0 += 8) {
-    if (h0) __syncthreads();
-    if ((g >> 1) == (h0 >> 3)) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        float4* dst = reinterpret_cast<float4*>(&S_all[wave][(4 * g + j) & 7][8 * n16]);
-        const float f = fown[j];
-        dst[0] = make_float4(accS[0][j] * f, accS[1][j] * f, accS[2][j] * f, accS[3][j] * f);
-        dst[1] = make_float4(accS[4][j] * f, accS[5][j] * f, accS[6][j] * f, accS[7][j] * f);
-      }
-    }
-    __syncthreads();
-    const int rows = min(8, n_rep - h0);
-    if (tid < rows * (kD / 4)) {
-      const int hl = tid >> 5, e4 = tid & 31;
-      float4 sum = *reinterpret_cast<const float4*>(&S_all[0][hl][4 * e4]);
-#pragma unroll
-      for (int w = 1; w < kWaves; ++w) {
-        const float4 x = *reinterpret_cast<const float4*>(&S_all[w][hl][4 * e4]);
-        sum.x += x.x; sum.y += x.y; sum.z += x.z; sum.w += x.w;
-      }
-      *reinterpret_cast<float4*>(pS + (h0 + hl) * kD + 4 * e4) = sum;
-    }
-  }
-  if (tid < n_rep) {
-    const int h = tid;
-    float L = 0.0f;
-#pragma unroll
-    for (int w = 0; w < kWaves; ++w) L += f_s[w][h] * l_s[w][h];
-    pml[2 * h] = M_s[h];
-    pml[2 * h + 1] = L;
-  }
+  merge_waves<kWaves>(mg_s, big_s, 4096, accS, m, l, inv_tscale, a.v_unscale, n_rep, pS, pml);
 }
 
 // Streaming flash-decode pass (packed K and V, no mask): a workgroup of FOUR waves runs through
@@ -600,8 +549,7 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
   __shared__ __align__(16) uint32_t ql_s[kHeadsMax][kD / 2];
   __shared__ __align__(16) float kn_s[kSWaves][kWavePos], vn_s[kSWaves][kWavePos];
   __shared__ __align__(16) float alpha_s[kSWaves][kHeadsMax];
-  __shared__ float m_s[kSWaves][kHeadsMax], l_s[kSWaves][kHeadsMax], M_s[kHeadsMax];
-  __shared__ __align__(16) float f_s[kSWaves][kHeadsMax];
+  __shared__ __align__(16) MergeLds<kSWaves> mg_s;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -833,66 +781,17 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
       });
   }
 
-  // ---- merge the four waves: one factor per (wave, head), scaled deposits, float4 sum.  A wave that saw
-  // no valid row has m = -inf, l = 0 and zero accumulators.
+  // ---- merge the four waves (merge_waves): a wave deposits into its own image area.  A wave that saw no valid
+  // row has m = -inf, l = 0 and zero accumulators.
   float l = l_run;
   l += shfl_xor_f(l, 16);
   l += shfl_xor_f(l, 32);
   l *= inv_tscale;
-  float (*S_all)[8][kD] = reinterpret_cast<float (*)[8][kD]>(big_s);
   const int64_t grp = (int64_t)seq * a.n_kv + kvh;
   float* pS = a.ws_S + (grp * a.n_tiles_max + wg) * (int64_t)(n_rep * kD);
   float* pml = a.ws_ml + (grp * a.n_tiles_max + wg) * (int64_t)(n_rep * 2);
-  if (g == 0) {
-    m_s[wave][n16] = m_run;
-    l_s[wave][n16] = l;
-  }
-  __syncthreads();                                         // also: every wave is done with its images
-  if (tid < kSWaves * kHeadsMax) {
-    const int w = tid >> 4, h = tid & 15;
-    float M = m_s[0][h];
-#pragma unroll
-    for (int ww = 1; ww < kSWaves; ++ww) M = fmaxf(M, m_s[ww][h]);
-    const float mw = m_s[w][h];
-    f_s[w][h] = (mw == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(mw - M);
-    if (w == 0) M_s[h] = M;
-  }
-  __syncthreads();
-  const float4 f4own = *reinterpret_cast<const float4*>(&f_s[wave][4 * g]);
-  const float wscale = inv_tscale * a.v_unscale;
-  const float fown[4] = {f4own.x * wscale, f4own.y * wscale, f4own.z * wscale, f4own.w * wscale};
-  for (int h0 = 0; h0 < n_rep; h0 += 8) {
-    if (h0) __syncthreads();
-    if ((g >> 1) == (h0 >> 3)) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        float4* dst = reinterpret_cast<float4*>(&S_all[wave][(4 * g + j) & 7][8 * n16]);
-        const float f = fown[j];
-        dst[0] = make_float4(accS[0][j] * f, accS[1][j] * f, accS[2][j] * f, accS[3][j] * f);
-        dst[1] = make_float4(accS[4][j] * f, accS[5][j] * f, accS[6][j] * f, accS[7][j] * f);
-      }
-    }
-    __syncthreads();
-    const int rows = min(8, n_rep - h0);
-    if (tid < rows * (kD / 4)) {
-      const int hl = tid >> 5, e4 = tid & 31;
-      float4 sum = *reinterpret_cast<const float4*>(&S_all[0][hl][4 * e4]);
-#pragma unroll
-      for (int w = 1; w < kSWaves; ++w) {
-        const float4 x = *reinterpret_cast<const float4*>(&S_all[w][hl][4 * e4]);
-        sum.x += x.x; sum.y += x.y; sum.z += x.z; sum.w += x.w;
-      }
-      *reinterpret_cast<float4*>(pS + (h0 + hl) * kD + 4 * e4) = sum;
-    }
-  }
-  if (tid < n_rep) {
-    const int h = tid;
-    float L = 0.0f;
-#pragma unroll
-    for (int w = 0; w < kSWaves; ++w) L += f_s[w][h] * l_s[w][h];
-    pml[2 * h] = M_s[h];
-    pml[2 * h + 1] = L;
-  }
+  static_assert(2 * kSImageBytes >= 8 * kD * 4 && (2 * kSImageBytes) % 16 == 0, "a wave's image area holds its eight deposit rows");
+  merge_waves<kSWaves>(mg_s, big_s, 2 * kSImageBytes, accS, m_run, l, inv_tscale, a.v_unscale, n_rep, pS, pml);
 }
 
 }  // namespace tqm
