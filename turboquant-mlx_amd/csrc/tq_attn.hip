@@ -1234,7 +1234,7 @@ extern "C" int tq_vonly_decode_attn_phases(const void* q, int q_dtype, const voi
     return tq::fail(TQ_ERR_NULL, "tq_vonly_decode_attn: null pointer");
   if (!tq::aligned(k_f16, 16)) return tq::fail(TQ_ERR_ALIGN, "tq_vonly_decode_attn: k must be 16-byte aligned");
   // d = 128, 3-bit, at most 16 query heads per kv head: matrix-core tile pass (float32 queries as fp16 value + remainder).
-  if (mma_shape(*shape) && tq::aligned(q, q_dtype == TQ_F32 ? 8 : 4))
+  if (mma_shape(*shape) && tq::aligned(q, 16))
     return launch_vonly_mfma(q, q_dtype, k_f16, v_packed, v_norms, v_centroids, v_signs, out, workspace, workspace_bytes,
                              *shape, (hipStream_t)stream_, phases);
   return launch_decode<kDenseK>(q, q_dtype, nullptr, nullptr, k_f16, v_packed, v_norms, nullptr, v_centroids,
@@ -1304,7 +1304,7 @@ int vonly_step_fused(const tq_vonly_cache_desc* c, const void* k_new, int k_dtyp
                      const void* q, int q_dtype, void* out, int out_dtype, int64_t position, const int64_t* position_dev,
                      float attn_scale, tq_stream_t stream_, const char* who) {
   if (!(c->dim == 128 && c->bits == 3 && c->n_rep >= 1 && c->n_rep <= tqm::kHeadsMax && c->allow_mma &&
-        tq::aligned(q, q_dtype == TQ_F32 ? 8 : 4) && tq::aligned(c->k_f16, 16)))
+        tq::aligned(q, 16) && tq::aligned(c->k_f16, 16)))
     return kNotFused;
   if (tq::check_dtype(k_dtype) || tq::check_dtype(v_dtype) || tq::check_dtype(q_dtype) || tq::check_dtype(out_dtype))
     return tq::fail(TQ_ERR_DTYPE, "%s: unknown dtype", who);
@@ -1388,7 +1388,7 @@ extern "C" int tq_vonly_sparse_decode_attn(const void* q, int q_dtype, const voi
   if (!tq::aligned(k_f16, 16)) return tq::fail(TQ_ERR_ALIGN, "%s: k must be 16-byte aligned", who);
   if (!(threshold >= 0.0f)) return tq::fail(TQ_ERR_ARG, "%s: threshold must be >= 0", who);
   if (!(shape->dim == 128 && shape->bits == 3 && shape->n_rep <= tqm::kHeadsMax && shape->seq_len > 0 &&
-        tq::aligned(q, q_dtype == TQ_F32 ? 8 : 4)))
+        tq::aligned(q, 16)))
     return tq::fail(TQ_ERR_UNSUPPORTED, "%s: dim 128, 3-bit values, n_rep <= 16 and a non-empty cache only "
                                         "(compose tq_dense_qk_scores, tq_softmax_rows and tq_sparse_v_matvec otherwise)", who);
   return launch_vonly_sparse(q, q_dtype, k_f16, v_packed, v_norms, v_centroids, v_signs, threshold, out, workspace,
@@ -1459,7 +1459,7 @@ extern "C" int tq_vonly_decode_step_at(const tq_vonly_cache_desc* c, const void*
   sh.attn_scale = attn_scale; sh.out_dtype = out_dtype; sh.allow_mma = 1;
   if (int rc = check_shape(&sh, who, 256)) return rc;
   if (tq::check_dtype(q_dtype)) return tq::fail(TQ_ERR_DTYPE, "%s: unknown q_dtype %d", who, q_dtype);
-  if (!(mma_shape(sh) && tq::aligned(q, q_dtype == TQ_F32 ? 8 : 4) && tq::aligned(c->k_f16, 16)))
+  if (!(mma_shape(sh) && tq::aligned(q, 16) && tq::aligned(c->k_f16, 16)))
     return tq::fail(TQ_ERR_UNSUPPORTED, "%s: dim 128, 3-bit values, n_rep <= 16 and aligned q / k only", who);
   const int n_q = c->n_kv_heads * c->n_rep;
   if (c->workspace_bytes < tq_workspace_bytes(TQ_OP_VONLY_DECODE, c->n_seq, n_q, c->t_alloc, c->dim))

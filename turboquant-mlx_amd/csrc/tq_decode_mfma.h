@@ -180,9 +180,7 @@ __device__ __forceinline__ void vonly_tile_body(const MfmaArgs& a, const Codeboo
   // 4 KB per wave used three ways: per-wave staging first for the packed V block, then for K
   // tiles; finally the cross-wave merge buffer S_all[NW][8][128].
   __shared__ __align__(16) unsigned char big_s[NW * 4096];
-  __shared__ uint32_t lut_s[64];                       // half2(c[i & 7], c[i >> 3])
-  __shared__ __align__(16) uint32_t q_s[kHeadsMax][kD / 2];   // fp16 pairs, rows >= n_rep are zero
-  __shared__ __align__(16) uint32_t ql_s[QF32 ? kHeadsMax : 1][kD / 2];   // QF32: what rounding the query to fp16 lost
+  __shared__ uint32_t lut_s[NW][64];                   // per wave: half2(c[i & 7], c[i >> 3])
   __shared__ __align__(16) float nrm_s[NW][kWavePos];
   __shared__ __align__(16) MergeLds<NW> mg_s;
 
@@ -201,21 +199,22 @@ __device__ __forceinline__ void vonly_tile_body(const MfmaArgs& a, const Codeboo
   const int wrow0 = wave * kWavePos;                                  // wave's first row inside the tile
 
   // ---- issue every global load of this wave, small ones first -------------------------------------
-  constexpr int kQIt = kHeadsMax * (kD / 2) / kThr;
-  uint32_t my_q[kQIt], my_ql[kQIt];                    // Q rows of this kv head: n_rep x 64 words, <= 1024
+  // Q operand of the score products, straight from global memory (the rows of a kv head are a few KB that
+  // every workgroup of the head reads: cache hits): lane (n16, g) takes piece 4 kb + g of row n16 for kb = 0 .. 3,
+  // 16 bytes of fp16 / bf16 or 32 bytes of float32.  Rows >= n_rep read row 0 and are zeroed.  Nothing here
+  // goes through LDS, so no wave waits for another before the merge.
+  const bool q_row_ok = n16 < n_rep;
+  u4 qraw[QF32 ? 8 : 4];
+  {
+    const char* qrow = reinterpret_cast<const char*>(a.q) + (q_row0 + (q_row_ok ? n16 : 0)) * (int64_t)(kD * (QF32 ? 4 : 2));
 #pragma unroll
-  for (int i = 0; i < kQIt; ++i) {
-    my_ql[i] = 0u;
-    const int w = tid + i * kThr;
-    if (QF32) {
-      const float2 f = (w < n_rep * (kD / 2)) ? reinterpret_cast<const float2*>(reinterpret_cast<const float*>(a.q) + q_row0 * kD)[w]
-                                              : make_float2(0.f, 0.f);
-      const __half2 h = __floats2half2_rn(f.x, f.y);
-      const float2 back = __half22float2(h);
-      my_q[i] = *reinterpret_cast<const uint32_t*>(&h);
-      my_ql[i] = pack_h2(f.x - back.x, f.y - back.y);
-    } else {
-      my_q[i] = (w < n_rep * (kD / 2)) ? reinterpret_cast<const uint32_t*>(a.q + q_row0 * kD)[w] : 0u;
+    for (int kb = 0; kb < 4; ++kb) {
+      if (QF32) {
+        qraw[2 * kb] = *reinterpret_cast<const u4*>(qrow + (4 * kb + g) * 32);
+        qraw[2 * kb + 1] = *reinterpret_cast<const u4*>(qrow + (4 * kb + g) * 32 + 16);
+      } else {
+        qraw[kb] = *reinterpret_cast<const u4*>(qrow + (4 * kb + g) * 16);
+      }
     }
   }
   float my_norm;
@@ -280,32 +279,40 @@ __device__ __forceinline__ void vonly_tile_body(const MfmaArgs& a, const Codeboo
 #pragma unroll
   for (int i = 0; i < 8; ++i) issue_k(i);
   __builtin_amdgcn_sched_barrier(0);
-  if (tid < 64) {
+  {
     float clo = 0.0f, chi = 0.0f;                        // selects, not a dynamic index into kernel arguments
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      clo = ((tid & 7) == i) ? vcb.c[i] : clo;
-      chi = ((tid >> 3) == i) ? vcb.c[i] : chi;
+      clo = ((lane & 7) == i) ? vcb.c[i] : clo;
+      chi = ((lane >> 3) == i) ? vcb.c[i] : chi;
     }
-    lut_s[tid] = pack_h2(clo, chi);
-  }
-#pragma unroll
-  for (int i = 0; i < kQIt; ++i) {
-    // bf16 queries become fp16 here, after every load of the pass has been requested: converting where the word
-    // is loaded would wait for it before anything else is in flight
-    if (!QF32 && a.q_bf16) my_q[i] = pack_h2(__uint_as_float(my_q[i] << 16), __uint_as_float(my_q[i] & 0xFFFF0000u));
-    (&q_s[0][0])[tid + i * kThr] = my_q[i];
-    if (QF32) (&ql_s[0][0])[tid + i * kThr] = my_ql[i];
+    lut_s[wave][lane] = pack_h2(clo, chi);
   }
   nrm_s[wave][lane] = my_norm;
-  __syncthreads();
+  const uint32_t* lut_w = lut_s[wave];
 
-  // ---- Q operand and the V norms of this lane's 16 positions ----------------------------------------
+  // ---- Q operand (converted now that every early load is in flight) and the V norms of this lane's 16 positions
   u4 qreg[4], qlow[4];
 #pragma unroll
   for (int kb = 0; kb < 4; ++kb) {
-    qreg[kb] = *reinterpret_cast<const u4*>(&q_s[n16][(4 * kb + g) * 4]);
-    if (QF32) qlow[kb] = *reinterpret_cast<const u4*>(&ql_s[n16][(4 * kb + g) * 4]);
+    if (QF32) {
+      const f4 lo4 = __builtin_bit_cast(f4, qraw[2 * kb]), hi4 = __builtin_bit_cast(f4, qraw[2 * kb + 1]);
+      const float f[8] = {lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const __half2 h = __floats2half2_rn(f[2 * i], f[2 * i + 1]);
+        const float2 back = __half22float2(h);
+        qreg[kb][i] = q_row_ok ? *reinterpret_cast<const uint32_t*>(&h) : 0u;
+        qlow[kb][i] = q_row_ok ? pack_h2(f[2 * i] - back.x, f[2 * i + 1] - back.y) : 0u;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        uint32_t w = qraw[kb][i];
+        if (a.q_bf16) w = pack_h2(__uint_as_float(w << 16), __uint_as_float(w & 0xFFFF0000u));
+        qreg[kb][i] = q_row_ok ? w : 0u;
+      }
+    }
   }
   float vn[4][4];
   float nmax = 0.0f;
@@ -363,7 +370,7 @@ __device__ __forceinline__ void vonly_tile_body(const MfmaArgs& a, const Codeboo
 #pragma unroll
       for (int qd = 0; qd < 4; ++qd) {
         const uint32_t src = (et & 1) ? Y[kb2][qd] : X[kb2][qd];
-        breg[kb2][et][qd] = lut_s[(src >> (6 * (et >> 1))) & 63u];
+        breg[kb2][et][qd] = lut_w[(src >> (6 * (et >> 1))) & 63u];
       }
   };
   // one 16-position score tile: K pieces through the wave's staging area, 4 matrix instructions
