@@ -38,12 +38,12 @@ MIN_TIMED_MS = 50.0       # GPU time every timed quantity is measured over (at l
 READ_WGS = 2048           # workgroups of the plain-read probe (8 per CU)
 
 # HBM bytes per launch of the dominant kernel (the tile pass), from two rocprofv3 --pmc runs of
-# `python bench.py --steps 60 --warmup 6 --no-cpu --no-graph` (FETCH_SIZE, then WRITE_SIZE), each
+# `python bench.py --steps 60 --warmup 6 --no-cpu --no-graph --no-ceiling` (FETCH_SIZE, then WRITE_SIZE), each
 # scaled by what the same counter reads for `python bench.py --calibrate-copy --steps 40`, a plain
-# copy of ALGO_BYTES bytes (FETCH_SIZE reads 19986.7 for 39950 KiB -> factor 1.9988; WRITE_SIZE
-# reads 39950.0 -> factor 1.0000).  Tile pass: FETCH_SIZE 20059.2 -> 40095 KiB, WRITE_SIZE 916.0
+# copy of ALGO_BYTES bytes (FETCH_SIZE reads 19986.6 for 39950 KiB -> factor 1.9988; WRITE_SIZE
+# reads 39950.0 -> factor 1.0000).  Tile pass: FETCH_SIZE 20071.6 -> 40120 KiB, WRITE_SIZE 916.0
 # -> 916 KiB.  Summary: profiles/vonly_decode_c2_pmc_traffic.md.
-MEASURED_TRAFFIC_BYTES = 41994390  # (20058.7 * 39950.0 / 19986.6 + 916.0) KiB
+MEASURED_TRAFFIC_BYTES = 42020792  # (20071.6 * 39950.0 / 19986.6 + 916.0) KiB
 
 
 def make_sets(torch, tqhip, dev):
