@@ -1781,3 +1781,31 @@ def test_seq_offsets_are_checked_by_every_ragged_wrapper(tq):
             call(torch.tensor([0, 120, 100], dtype=torch.int32, device="cuda"), validate_offsets=True)
         with pytest.raises(ValueError, match="holds"):
             call(torch.tensor([0, 100, 161], dtype=torch.int32, device="cuda"), validate_offsets=True)
+
+
+@pytest.mark.parametrize("spike_pos", [5, 40, 63, 64 + 33, 300, 511, 700])
+@pytest.mark.parametrize("q_dtype", [np.float16, np.float32])
+def test_vonly_decode_with_one_dominant_key(tq, spike_pos, q_dtype):
+    """One key row equal to 3 q (its score exceeds every other by some 50 log2 units) at positions that fall into
+    the first or the second 32-position half of a wave's run, in full and in ragged tiles: the tile pass takes
+    the softmax reference of a run from its first half and must fall back to the true maximum here (weights would
+    leave the fp16 range otherwise).  Against the oracle, at the 2e-3 / 1e-3 bar."""
+    rng = np.random.default_rng(900 + spike_pos)
+    n_kv, n_rep, T, D, bits = 2, 4, 777, 128, 3
+    c, b = tables(bits)
+    vs = o.random_diagonal_sign(D, 43)
+    K = rng.standard_normal((n_kv, T, D)).astype(np.float16)
+    V = rng.standard_normal((n_kv, T, D)).astype(np.float16)
+    q = rng.standard_normal((1, n_kv * n_rep, D)).astype(q_dtype)
+    K[0, spike_pos] = (3.0 * q[0, 1]).astype(np.float16)             # head 1 of kv head 0
+    K[1, spike_pos] = (3.0 * q[0, n_rep + 2]).astype(np.float16)     # head 2 of kv head 1
+    sc = 1 / math.sqrt(D)
+    gp, gn = tq.fused_quantize(dev(V.reshape(-1, D)), dev(vs), b, D, bits)
+    vp, vn = gp.reshape(n_kv, T, -1), gn.reshape(n_kv, T)
+    for L in (T, 512):
+        if spike_pos >= L:
+            continue
+        got = host(tq.vonly_decode(dev(q), dev(K), vp, vn, c, dev(vs), D, bits, sc, n_rep=n_rep, seq_len=L))
+        want = o.vonly_decode_attention(q[0], K[:, :L], host(vp)[:, :L], host(vn)[:, :L], c, vs, D, bits, sc)
+        assert np.isfinite(got).all()
+        close(got[0], want)
