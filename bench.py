@@ -227,30 +227,38 @@ def main():
 
     def read_ceiling():
         """One launch that only streams the K, packed-V and norm bytes of a step (tq_probe_read, rotating over
-        copies of the buffer sets), and an empty launch, timed like the decode step."""
-        sink = torch.zeros(1, dtype=torch.int32, device=dev)
+        copies of the buffer sets), the same with the launch shape of the tile pass (256 workgroups) with and
+        without a 3.5 KB store per workgroup at the end, and an empty launch -- all timed like the decode step."""
+        part = N_REP * (D + 2) * 4 // 16 * 16               # bytes of one workgroup's partial result
+        sink = torch.zeros(16 + READ_WGS * part, dtype=torch.uint8, device=dev)
         srcs = [torch.cat([k.reshape(-1).view(torch.uint8), vp.reshape(-1).view(torch.uint8),
                            vn.reshape(-1).view(torch.uint8)]) for (_, k, vp, vn) in sets]
         nbytes = srcs[0].numel() // 16 * 16
 
-        def read_step(nb):
+        def read_step(nb, wgs=READ_WGS, store=0):
             def one(i, stream):
                 rc = lib.tq_probe_read(C.c_void_p(srcs[i % N_SETS].data_ptr()), nb, C.c_void_p(sink.data_ptr()),
-                                       READ_WGS, C.c_void_p(stream))
+                                       wgs, store, C.c_void_p(stream))
                 if rc != 0:
                     _lib.check(rc)
             return one
         r_med, r_min, r_max, r_n = timed(read_step(nbytes))
+        t_med = timed(read_step(nbytes, 256))[0]
+        s_med = timed(read_step(nbytes, 256, part))[0]
         e_med, e_min, e_max, _ = timed(read_step(0))
         return {
             "bytes_per_launch": nbytes, "workgroups": READ_WGS,
             "us_per_launch": round(r_med * 1e3, 3), "min": round(r_min * 1e3, 3), "max": round(r_max * 1e3, 3),
             "replays": r_n, "GB/s": round(nbytes / (r_med * 1e-3) / 1e9, 1),
             "frac_of_peak": round(nbytes / (r_med * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            "us_256_workgroups": round(t_med * 1e3, 3),
+            "us_256_workgroups_storing_a_partial_each": round(s_med * 1e3, 3), "partial_bytes": part,
             "empty_launch_us": round(e_med * 1e3, 3), "empty_launch_min": round(e_min * 1e3, 3),
             "empty_launch_max": round(e_max * 1e3, 3),
             "note": "one launch that only reads the K, packed-V and norm bytes of a step (rotating buffer sets, the "
-                    "benchmark's launch pattern): the practical ceiling for a launch of this size on this box"}
+                    "benchmark's launch pattern): the practical ceiling for a launch of this size on this box; the "
+                    "256-workgroup figures use the grid of the tile pass, the second one ends every workgroup with "
+                    "the store of a partial result"}
 
     if args.calibrate_read:
         print(json.dumps({"calibrate_read": True, "buffer_sets": N_SETS, "steps": args.steps, "warmup": args.warmup,

@@ -489,12 +489,18 @@ size_t tq_prefill_workspace_bytes(int n_q_heads, int64_t n_rows, int64_t kv_len,
 /*
  * Measurement aid, no counterpart in the reference (its benches time whole kernels with mx.eval,
  * scripts/bench_sparse_v.py:49-57): ONE launch that streams `bytes` bytes from `src` (16-byte aligned,
- * a multiple of 16) through n_workgroups workgroups of 256 threads and writes nothing -- the practical
- * ceiling for a launch that reads this much on the machine at hand, launch overhead and tail included.
- * bytes == 0 launches an empty kernel (the cost of a launch alone).  `sink` (device, 4 bytes, may be NULL)
- * is never written in practice.  bench.py --calibrate-read times both beside the decode step.
+ * a multiple of 16) through n_workgroups workgroups (256 threads with eight loads in flight each; 512 threads with
+ * every load requested up front when a workgroup's share is between 32 and 160 KB) -- the practical ceiling for a launch
+ * that reads this much on the machine at hand, launch overhead and tail included.  With
+ * store_bytes_per_workgroup > 0 (a multiple of 16, at most 4096) every workgroup ends with a store of that
+ * many bytes at sink + 16 + workgroup * store_bytes_per_workgroup, as a split-KV tile pass ends with the
+ * store of its partial result; `sink` (device, 16-byte aligned) must then hold 16 + n_workgroups *
+ * store_bytes_per_workgroup bytes, else 4 bytes suffice (never written in practice) and it may be NULL.
+ * bytes == 0 launches an empty kernel (the cost of a launch alone).  bench.py --calibrate-read times these
+ * beside the decode step.
  */
-int tq_probe_read(const void* src, size_t bytes, uint32_t* sink, int n_workgroups, tq_stream_t stream);
+int tq_probe_read(const void* src, size_t bytes, uint32_t* sink, int n_workgroups,
+                  size_t store_bytes_per_workgroup, tq_stream_t stream);
 
 #ifdef __cplusplus
 }

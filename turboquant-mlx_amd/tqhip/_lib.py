@@ -92,7 +92,7 @@ PROTOTYPES = {
     "tq_prefill_attn": (_i, [_p, _i, _p, _p, _p, _p, _fp, _fp, _p, _p, _p, _i, _p, _z, _i, _i, _l, _l, _l,
                             _l, _l, _l, _l, _i, _i, _f, _i, _p]),
     "tq_prefill_workspace_bytes": (_z, [_i, _l, _l, _i]),
-    "tq_probe_read": (_i, [_p, _z, _p, _i, _p]),
+    "tq_probe_read": (_i, [_p, _z, _p, _i, _z, _p]),
 }
 
 _lib = None
