@@ -51,10 +51,12 @@ def close(got, want, rel=REL, abs_=ABS, row_scale=False, extra=0.0):
 
 
 def threshold_slack(w, thr, vp, vn, c, vs, n_rep, band):
-    """Extra tolerance for a thresholded value sum: a weight within `band` (relative) of the threshold may fall on
-    either side when the scores behind it differ in the last places (fp16 operands, summation order); such a
+    """Extra tolerance for a thresholded value sum over PACKED keys (the only users): the scores of that step come
+    from fp16 operands (about 3e-4 relative per score, i.e. up to ~2e-3 relative per weight at |score| ~ 6), so a
+    weight within `band` (relative; 3e-3 in the tests) of the threshold may fall on either side of it; such a
     position moves the output by its whole contribution w * |dequantised V row|.  Returns (n_q, dim): the sum of
-    those contributions over the ambiguous positions of each head (zero when there are none)."""
+    those contributions over the ambiguous positions of each head -- zero when no weight is that close, in which
+    case the plain 2e-3 / 1e-3 bar applies.  The thresholded steps over fp16 keys do not use it."""
     amb = np.abs(w.astype(np.float64) - thr) <= band * thr                      # (n_q, T)
     if not amb.any():
         return np.zeros((w.shape[0], 128))
@@ -1526,7 +1528,7 @@ def test_flash_sparse_decode_matches_oracle(tq, n_seq, n_kv, n_rep, T, thr, mask
         want = o.turboquant_attention_single(q[i], kp[i, :, :T], kn[i, :, :T], vp[i, :, :T], vn[i, :, :T], c, ks, c, vs,
                                              D, bits, sc, sparse_v_threshold=thr, mask=mi)
         w = _packed_weights(q[i], kp[i, :, :T], kn[i, :, :T], c, ks, sc, n_rep, mi)
-        close(got[i], want, extra=threshold_slack(w, thr, vp[i, :, :T], vn[i, :, :T], c, vs, n_rep, 1e-2))
+        close(got[i], want, extra=threshold_slack(w, thr, vp[i, :, :T], vn[i, :, :T], c, vs, n_rep, 3e-3))
 
 
 def test_flash_sparse_decode_ragged_and_limits(tq):
@@ -1546,7 +1548,7 @@ def test_flash_sparse_decode_ragged_and_limits(tq):
         want = o.turboquant_attention_single(q[i], kp[:, a:e], kn[:, a:e], vp[:, a:e], vn[:, a:e], c, ks, c, vs,
                                              D, bits, sc, sparse_v_threshold=1e-4)
         w = _packed_weights(q[i], kp[:, a:e], kn[:, a:e], c, ks, sc, n_rep, None)
-        close(got[i], want, extra=threshold_slack(w, 1e-4, vp[:, a:e], vn[:, a:e], c, vs, n_rep, 1e-2))
+        close(got[i], want, extra=threshold_slack(w, 1e-4, vp[:, a:e], vn[:, a:e], c, vs, n_rep, 3e-3))
     assert (host(tq.flash_decode(*args, sparse_v_threshold=2.0, **kw)) == 0).all()
     close(host(tq.flash_decode(*args, sparse_v_threshold=1e-37, **kw)), host(tq.flash_decode(*args, **kw)),
           rel=1e-3, abs_=2e-4)
@@ -1590,7 +1592,7 @@ def test_decode_sweep_flash_sparse(tq, seed):
         w = _packed_weights(q[i], kpi, kni, c, ks, sc, n_rep, mi)
         close(got[i], o.turboquant_attention_single(q[i], kpi, kni, vpi, vni, c, ks, c, vs, D, bits, sc,
                                                     sparse_v_threshold=thr, mask=mi),
-              extra=threshold_slack(w, thr, vpi, vni, c, vs, n_rep, 1e-2))
+              extra=threshold_slack(w, thr, vpi, vni, c, vs, n_rep, 3e-3))
 
 
 # ------------------------------------------------------------------ decode step from the query itself (rotation in-kernel)
