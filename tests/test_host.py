@@ -184,3 +184,78 @@ def test_patch_install_and_restore_on_host():
     tqhip.remove_patch()
     assert a.scaled_dot_product_attention is len and not hasattr(b, "scaled_dot_product_attention")
     tqhip.remove_patch()                                   # nothing left to undo
+
+
+def test_offsets_check_on_host():
+    """The ragged wrappers' offsets check: dtype, count and layout always; order and range with validate=True."""
+    good = torch.tensor([0, 5, 9], dtype=torch.int32)
+    rows = torch.zeros((2, 9, 13), dtype=torch.int32)
+    ops._check_offsets(good, 2, True, k_packed=rows)
+    with pytest.raises(ValueError, match="int32"):
+        ops._check_offsets(torch.cumsum(torch.tensor([0, 5, 4]), 0), 2, False)
+    with pytest.raises(ValueError, match="n_seq"):
+        ops._check_offsets(good, 3, False)
+    with pytest.raises(ValueError, match="int32"):
+        ops._check_offsets(torch.tensor([0, 1, 5, 2, 9], dtype=torch.int32)[::2], 2, False)      # not contiguous
+    with pytest.raises(ValueError, match="never decrease"):
+        ops._check_offsets(torch.tensor([0, 7, 5], dtype=torch.int32), 2, True)
+    with pytest.raises(ValueError, match="never decrease"):
+        ops._check_offsets(torch.tensor([-1, 2, 5], dtype=torch.int32), 2, True)
+    with pytest.raises(ValueError, match="holds 9"):
+        ops._check_offsets(torch.tensor([0, 5, 10], dtype=torch.int32), 2, True, k_packed=rows)
+    ops._check_offsets(torch.tensor([0, 5, 10], dtype=torch.int32), 2, False, k_packed=rows)      # unchecked by default
+
+
+def test_explicit_sign_vectors_are_validated_on_host():
+    from tqhip.cache import _Quantizer, _checked_signs
+    s = np.where(np.arange(128) % 3 == 0, -1.0, 1.0).astype(np.float32)
+    q = _Quantizer(128, 3, seed=42, device="cpu", signs=s)
+    assert q.signs.dtype == torch.float32 and np.array_equal(q.signs.numpy(), s)
+    assert not np.array_equal(_Quantizer(128, 3, seed=42, device="cpu").signs.numpy(), s)
+    assert np.array_equal(_checked_signs(torch.from_numpy(s).double(), 128, "cpu").numpy(), s)    # any float dtype
+    for bad in (np.ones(64, np.float32), np.zeros(128, np.float32), np.ones((2, 64), np.float32), 0.5 * s):
+        with pytest.raises(ValueError):
+            _checked_signs(bad, 128, "cpu")
+    c = tqhip.TurboQuantKVCache(bits=3, k_signs=s, v_signs=-s)
+    c._ensure_quantizer(128, 128, torch.device("cpu"))
+    assert np.array_equal(c._k_q.signs.numpy(), s) and np.array_equal(c._v_q.signs.numpy(), -s)
+    v = tqhip.VOnlyTurboQuantCache(bits=3, v_signs=s)
+    v._v_tq._ensure_quantizer(128, 128, torch.device("cpu"))
+    assert np.array_equal(v._v_tq._v_q.signs.numpy(), s)
+
+
+@pytest.mark.parametrize("have_k,have_v,offset,extra", [(1024, 1024, 1000, 2000), (1512, 1536, 1500, 1),
+                                                         (300, 300, 300, 1), (556, 512, 301, 1), (0, 0, 0, 5)])
+def test_vonly_cache_brings_keys_and_values_to_one_capacity(have_k, have_v, offset, extra):
+    """The capacity rule of the V-only cache on host tensors (no kernel involved): whatever capacities the key
+    cache and the packed values have drifted to (1000-token prompt; 1000 + 500 chunks; from_state slices; from_state
+    then one insert through the two storages' own growth rules), reserve() leaves both contiguous with ONE capacity,
+    a multiple of 256 with room for the request, and the first `offset` positions unchanged."""
+    B, H, D = 1, 2, 128
+    c = tqhip.VOnlyTurboQuantCache(bits=3)
+    kc, tq = c._k_cache, c._v_tq
+    g = torch.Generator().manual_seed(have_k + offset)
+    if have_k:
+        kc.keys = torch.randn((B, H, have_k + 3, D), generator=g).to(torch.float16)[:, :, :have_k]     # a slice, not contiguous
+        kc.values = torch.randn((B, H, have_k + 3, D), generator=g).to(torch.float16)[:, :, :have_k]
+        tq.v_packed = torch.randint(0, 2 ** 30, (B, H, have_v + 5, 13), generator=g, dtype=torch.int32)[:, :, :have_v].view(torch.uint32)
+        tq.v_norms = torch.rand((B, H, have_v + 5), generator=g)[:, :, :have_v]
+        tq._v_pdim, tq._v_dim = 13, D
+    kc.offset = tq.offset = offset
+    before = [t[..., :offset, :].clone() if t.dim() == 4 else t[..., :offset].clone()
+              for t in (kc.keys, kc.values, tq.v_packed, tq.v_norms)] if have_k else None
+    c.reserve(B, H, extra, D, device="cpu")
+    n = kc.keys.shape[2]
+    assert n == tq.v_packed.shape[2] == tq.v_norms.shape[2] == kc.values.shape[2]
+    assert n % 256 == 0 and n >= offset + extra and n >= max(have_k, have_v)
+    assert all(t.is_contiguous() for t in (kc.keys, kc.values, tq.v_packed, tq.v_norms))
+    if before:
+        after = [kc.keys[..., :offset, :], kc.values[..., :offset, :], tq.v_packed[..., :offset, :], tq.v_norms[..., :offset]]
+        for x, y in zip(before, after):
+            assert torch.equal(x.view(torch.int32) if x.dtype == torch.uint32 else x, y.view(torch.int32) if y.dtype == torch.uint32 else y)
+    addr = kc.keys.data_ptr()
+    c.reserve(B, H, extra, D, device="cpu")                  # nothing moves when both agree and have room
+    assert kc.keys.data_ptr() == addr
+    c.set_offset(n)
+    with pytest.raises(ValueError):
+        c.set_offset(n + 1)
