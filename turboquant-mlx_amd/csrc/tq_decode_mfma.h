@@ -422,73 +422,52 @@ __device__ __forceinline__ void vonly_tile_body(const MfmaArgs& a, const Codeboo
   for (int i = 12; i < 16; ++i) issue_k(i);
   __builtin_amdgcn_sched_barrier(0);
   qk_tile(1);
-
-  // ---- softmax and value product in two halves of 32 positions ---------------------------------------------
-  // The first half (score tiles 0, 1) is finished while the K rows of the second are still arriving: its
-  // maximum is the wave's reference R for BOTH halves (weights 2^(s - R); any reference serves a softmax as
-  // long as nothing overflows), so the second half adds its weights and products without rescaling the first.
-  // Weights travel as fp16 scaled to [1, 2) by the norm scale, so a second-half score may exceed R by up to
-  // 14 (log2 units) -- a factor of 16 000 inside one run of 64 positions.  Beyond that (or when the first half
-  // is fully masked) the wave redoes both halves against the true maximum; the check is wave-uniform.
-  // PLAIN: s is the raw product and attn_scale > 0 (host check), so the maximum commutes with the scaling;
-  // weights = 2^(s * cs - R + kexp) in one fma + v_exp_f32.
-  const float arg_scale = PLAIN ? cs : 1.0f;
-  uint32_t pa[2][4];                                     // A operands of the value product
-  f4 accS[8];
-  auto half_max = [&](int kb2) {
-    float mx = -INFINITY;
-#pragma unroll
-    for (int t = 2 * kb2; t < 2 * kb2 + 2; ++t)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) mx = fmaxf(mx, s[t][j]);
-    mx = fmaxf(mx, shfl_xor_f(mx, 16));
-    mx = fmaxf(mx, shfl_xor_f(mx, 32));
-    return mx * arg_scale;                               // log2 units (-inf stays -inf)
-  };
-  auto half_weights = [&](int kb2, float bias) {         // returns this lane's part of the weight sum
-    float lsum = 0.0f;
-#pragma unroll
-    for (int t = 2 * kb2; t < 2 * kb2 + 2; ++t) {
-      float p[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        p[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][j], arg_scale, bias));   // weight * 2^kexp
-        lsum += p[j];
-        p[j] *= vn[t][j];
-      }
-      pa[kb2][2 * (t & 1)] = pack_h2(p[0], p[1]);
-      pa[kb2][2 * (t & 1) + 1] = pack_h2(p[2], p[3]);
-    }
-    return lsum;
-  };
-  auto half_values = [&](int kb2, bool fresh) {
-    const u4 A = {pa[kb2][0], pa[kb2][1], pa[kb2][2], pa[kb2][3]};
-#pragma unroll
-    for (int et = 0; et < 8; ++et)
-      accS[et] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, A), __builtin_bit_cast(h8, breg[kb2][et]),
-                                                        fresh ? f4{0.f, 0.f, 0.f, 0.f} : accS[et], 0, 0, 0);
-  };
-  float m = half_max(0);                                 // the reference R
-  float l = half_weights(0, kexp - ((m == -INFINITY) ? 0.0f : m));
-  half_values(0, true);
-  __builtin_amdgcn_sched_barrier(0);
   qk_tile(2);
   qk_tile(3);
-  const float mB = half_max(1);
-  if (!__any(m == -INFINITY || mB > m + 14.0f)) {
-    l += half_weights(1, kexp - m);
-    half_values(1, false);
-  } else {                                               // rare: both halves against the true maximum
-    m = fmaxf(m, mB);
-    const float bias = kexp - ((m == -INFINITY) ? 0.0f : m);
-    l = half_weights(0, bias);
-    half_values(0, true);
-    l += half_weights(1, bias);
-    half_values(1, false);
+
+  // ---- softmax statistics of head n16 over the wave's 64 positions ----------------------------------
+  float m = -INFINITY;
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) m = fmaxf(m, s[t][j]);
+  m = fmaxf(m, shfl_xor_f(m, 16));
+  m = fmaxf(m, shfl_xor_f(m, 32));
+  // PLAIN: s is the raw product and attn_scale > 0 (host check), so the maximum commutes with the
+  // scaling; weights = 2^(s * cs - m * cs + kexp) in one fma + v_exp_f32.
+  const float arg_scale = PLAIN ? cs : 1.0f;
+  m = m * arg_scale;                                     // log2 units from here on (-inf stays -inf)
+  const float bias = kexp - ((m == -INFINITY) ? 0.0f : m);
+  float l = 0.0f;
+  uint32_t pa[2][4];                                     // A operands of the value product
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    float p[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      p[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][j], arg_scale, bias));   // weight * 2^kexp
+      l += p[j];
+      p[j] *= vn[t][j];
+    }
+    pa[t >> 1][2 * (t & 1)] = pack_h2(p[0], p[1]);
+    pa[t >> 1][2 * (t & 1) + 1] = pack_h2(p[2], p[3]);
   }
   l += shfl_xor_f(l, 16);
   l += shfl_xor_f(l, 32);
   l *= inv_tscale;
+
+  // ---- values ------------------------------------------------------------------------------------------
+  f4 accS[8];
+#pragma unroll
+  for (int et = 0; et < 8; ++et) accS[et] = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int kb2 = 0; kb2 < 2; ++kb2) {
+    const u4 A = {pa[kb2][0], pa[kb2][1], pa[kb2][2], pa[kb2][3]};
+#pragma unroll
+    for (int et = 0; et < 8; ++et)
+      accS[et] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, A), __builtin_bit_cast(h8, breg[kb2][et]),
+                                                        accS[et], 0, 0, 0);
+  }
 
   // ---- merge the waves of the workgroup (merge_waves): one partial per workgroup goes to the workspace -----------
   const int64_t grp = (int64_t)seq * a.n_kv + kvh;
