@@ -1789,9 +1789,9 @@ def test_seq_offsets_are_checked_by_every_ragged_wrapper(tq):
 @pytest.mark.parametrize("q_dtype", [np.float16, np.float32])
 def test_vonly_decode_with_one_dominant_key(tq, spike_pos, q_dtype):
     """One key row equal to 3 q (its score exceeds every other by some 50 log2 units) at positions that fall into
-    the first or the second 32-position half of a wave's run, in full and in ragged tiles: the tile pass takes
-    the softmax reference of a run from its first half and must fall back to the true maximum here (weights would
-    leave the fp16 range otherwise).  Against the oracle, at the 2e-3 / 1e-3 bar."""
+    different waves, score tiles and halves of a wave's run, in full and in ragged tiles: weights travel as fp16
+    relative to a per-wave reference, and a reference taken from anything but the true maximum of the run would
+    push them out of range here.  Against the oracle, at the 2e-3 / 1e-3 bar."""
     rng = np.random.default_rng(900 + spike_pos)
     n_kv, n_rep, T, D, bits = 2, 4, 777, 128, 3
     c, b = tables(bits)
