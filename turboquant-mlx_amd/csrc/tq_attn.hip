@@ -510,8 +510,13 @@ __global__ __launch_bounds__(kThreads) void decode_tile_kernel(DecodeArgs a, Cod
   stage_rows<PDIM>(a.v_packed + (vrow0 + t_begin) * PDIM, n_here, vrows_s[wave], lane);
   const float my_nrm = (lane < n_here) ? a.v_norms[vnrow0 + t_begin + lane] : 0.0f;
   __builtin_amdgcn_wave_barrier();                      // the rows are read back by this wave only; LDS operations of a wave complete in order
-  // software pipeline: the packed words of position j + 2 and the centroids of position j + 1 are fetched from
-  // LDS while the multiply-adds of position j run (rows 64 and 65 of the wave's area exist and are never used)
+  // The norm of a position rides on its weights (same lane): (w * norm) * centroid, the order of
+  // sparse_v.py:64.  Software pipeline: the packed words of position j + 2 and the centroids of position j + 1
+  // are fetched from LDS while the multiply-adds of position j run (rows 64 and 65 of the wave's area exist and
+  // are never used).  Four positions per trip with a wave-uniform trip count: positions past n_here carry
+  // weight 0 and whatever codes their rows hold select finite centroids.
+#pragma unroll
+  for (int r = 0; r < kRMax; ++r) pw[r] *= my_nrm;
   const uint32_t* vrows = vrows_s[wave];
   uint32_t wnext[EPL];
   float cnext[EPL];
@@ -519,21 +524,26 @@ __global__ __launch_bounds__(kThreads) void decode_tile_kernel(DecodeArgs a, Cod
   for (int i = 0; i < EPL; ++i) cnext[i] = cbv_s[(vrows[widx[i]] >> wsh[i]) & Pk<BITS>::MASK];
 #pragma unroll
   for (int i = 0; i < EPL; ++i) wnext[i] = vrows[(PDIM | 1) + widx[i]];
-  for (int j = 0; j < n_here; ++j) {
-    float cn[EPL];
-    const float nrm = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_nrm), j));
+  const int n_trips = __builtin_amdgcn_readfirstlane((n_here + 3) >> 2);
+  for (int jj = 0; jj < n_trips; ++jj) {
 #pragma unroll
-    for (int i = 0; i < EPL; ++i) cn[i] = cnext[i] * nrm;
+    for (int u = 0; u < 4; ++u) {
+      const int j = 4 * jj + u;
+      float cn[EPL];
 #pragma unroll
-    for (int i = 0; i < EPL; ++i) cnext[i] = cbv_s[(wnext[i] >> wsh[i]) & Pk<BITS>::MASK];
+      for (int i = 0; i < EPL; ++i) cn[i] = cnext[i];
 #pragma unroll
-    for (int i = 0; i < EPL; ++i) wnext[i] = vrows[(j + 2) * (PDIM | 1) + widx[i]];
+      for (int i = 0; i < EPL; ++i) cnext[i] = cbv_s[(wnext[i] >> wsh[i]) & Pk<BITS>::MASK];
 #pragma unroll
-    for (int r = 0; r < kRMax; ++r) {
-      const float w = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, pw[r]), j));
+      for (int i = 0; i < EPL; ++i) wnext[i] = vrows[(u + 2) * (PDIM | 1) + widx[i]];
 #pragma unroll
-      for (int i = 0; i < EPL; ++i) acc[r][i] = __builtin_fmaf(w, cn[i], acc[r][i]);
+      for (int r = 0; r < kRMax; ++r) {
+        const float w = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, pw[r]), j));
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) acc[r][i] = __builtin_fmaf(w, cn[i], acc[r][i]);
+      }
     }
+    vrows += 4 * (PDIM | 1);
   }
 #pragma unroll
   for (int r = 0; r < kRMax; ++r)
