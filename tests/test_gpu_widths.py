@@ -1,0 +1,185 @@
+"""GPU parity tests of the V-only decode step at value widths of 1, 2 and 4 bits (the reference takes
+bits 1-4, adaptive.py:26, v_only_cache.py:41): the matrix-core tile pass against the CPU oracle and
+against the float32 kernels, over every launch shape the host picks from (one tile per workgroup of
+four or eight waves, full or ragged; the streaming pass, full or ragged), with masks, ragged batches
+and the three query dtypes.  Tolerance: 2e-3 relative + 1e-3 absolute, elementwise, as for 3 bits.
+"""
+import math
+
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+
+from oracle import polarquant_oracle as o  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+
+F32 = np.float32
+REL, ABS = 2e-3, 1e-3
+D = 128
+
+
+@pytest.fixture(scope="module")
+def tq():
+    if not torch.cuda.is_available():
+        pytest.fail("GPU tests need a GPU: torch.cuda.is_available() is False")
+    import tqhip
+    return tqhip
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    return t.detach().float().cpu().numpy()
+
+
+def close(got, want, rel=REL, abs_=ABS):
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    ok = err <= abs_ + rel * np.abs(want)
+    assert ok.all(), f"max err {err.max():.3e} (want scale {np.abs(want).max():.3e}), {(~ok).sum()} bad"
+
+
+def fixture(rng, n_kv, T, bits):
+    """fp16 keys, values encoded by the oracle at `bits` bits (norms spread over two decades)."""
+    c = o.gaussian_codebook(bits)
+    b = o.gaussian_boundaries(c)
+    vs = o.random_diagonal_sign(D, 43)
+    K = rng.standard_normal((n_kv, T, D)).astype(np.float16)
+    V = (rng.standard_normal((n_kv, T, D)) * np.exp(rng.uniform(-2.3, 2.3, size=(n_kv, T, 1)))).astype(np.float16)
+    vp, vn = o.fused_quantize(V.reshape(-1, D), vs, b, D, bits)
+    pd = o.packed_dim(D, bits)
+    return c, vs, K, vp.reshape(n_kv, T, pd), vn.reshape(n_kv, T)
+
+
+@pytest.mark.parametrize("bits", [1, 2, 4])
+@pytest.mark.parametrize("n_kv,n_rep,T,qdt", [(4, 7, 1000, np.float16), (2, 1, 64, np.float16), (1, 9, 257, np.float32),
+                                              (8, 4, 513, np.float16), (3, 16, 1, np.float32), (2, 5, 4096, np.float16),
+                                              (4, 7, 5000, np.float32)])
+def test_vonly_decode_other_widths_match_oracle(tq, bits, n_kv, n_rep, T, qdt):
+    rng = np.random.default_rng(300 + bits)
+    c, vs, K, vp, vn = fixture(rng, n_kv, T, bits)
+    q = rng.standard_normal((1, n_kv * n_rep, D)).astype(qdt)
+    sc = 1 / math.sqrt(D)
+    got = host(tq.vonly_decode(dev(q), dev(K), dev(vp), dev(vn), c, dev(vs), D, bits, sc, n_rep=n_rep))
+    want = o.vonly_decode_attention(q[0], K, vp, vn, c, vs, D, bits, sc)
+    close(got[0], want)
+    ref32 = host(tq.vonly_decode(dev(q), dev(K), dev(vp), dev(vn), c, dev(vs), D, bits, sc, n_rep=n_rep, precision="fp32"))
+    close(got[0], ref32[0])
+
+
+@pytest.mark.parametrize("bits", [1, 2, 4])
+def test_vonly_decode_other_widths_bf16_queries_and_output_dtypes(tq, bits):
+    rng = np.random.default_rng(310 + bits)
+    n_kv, n_rep, T = 4, 7, 777
+    c, vs, K, vp, vn = fixture(rng, n_kv, T, bits)
+    qt = torch.from_numpy(rng.standard_normal((1, n_kv * n_rep, D)).astype(F32)).to(torch.bfloat16)
+    sc = 1 / math.sqrt(D)
+    want = o.vonly_decode_attention(qt[0].float().numpy(), K, vp, vn, c, vs, D, bits, sc)
+    for od, rel, abs_ in ((torch.float32, REL, ABS), (torch.float16, REL, ABS), (torch.bfloat16, 1e-2, 1e-3)):
+        got = host(tq.vonly_decode(qt.cuda(), dev(K), dev(vp), dev(vn), c, dev(vs), D, bits, sc, n_rep=n_rep, out_dtype=od))
+        close(got[0], want, rel, abs_)                     # bf16 outputs carry their own 2^-8 rounding
+
+
+@pytest.mark.parametrize("bits", [1, 2, 4])
+def test_vonly_decode_other_widths_ragged_batch_and_mask(tq, bits):
+    rng = np.random.default_rng(320 + bits)
+    n_kv, n_rep, n_seq = 4, 7, 4
+    sc = 1 / math.sqrt(D)
+    lens = rng.integers(10, 900, size=n_seq)
+    offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    c, vs, K, vp, vn = fixture(rng, n_kv, int(offs[-1]), bits)
+    q = rng.standard_normal((n_seq, n_kv * n_rep, D)).astype(np.float16)
+    got = host(tq.vonly_decode(dev(q), dev(K), dev(vp), dev(vn), c, dev(vs), D, bits, sc, n_rep=n_rep,
+                               seq_offsets=dev(offs), max_seq_len=int(lens.max())))
+    for i in range(n_seq):
+        a, e = offs[i], offs[i + 1]
+        close(got[i], o.vonly_decode_attention(q[i], K[:, a:e], vp[:, a:e], vn[:, a:e], c, vs, D, bits, sc))
+    # cache layout (B, H, T_alloc, ...) read up to seq_len, with an additive mask per head
+    B, T_alloc, total = 2, 1024, 701
+    Kb = rng.standard_normal((B, n_kv, T_alloc, D)).astype(np.float16)
+    cs, vss, _, vpb, vnb = fixture(rng, B * n_kv, T_alloc, bits)
+    vpb, vnb = vpb.reshape(B, n_kv, T_alloc, -1), vnb.reshape(B, n_kv, T_alloc)
+    qb = rng.standard_normal((B, n_kv * n_rep, D)).astype(np.float16)
+    mask = np.where(rng.random((B, n_kv * n_rep, total)) < 0.3, -np.inf, 0.0).astype(F32)
+    mask[..., 5] = 0.0
+    got = host(tq.vonly_decode(dev(qb), dev(Kb), dev(vpb), dev(vnb), cs, dev(vss), D, bits, sc, n_rep=n_rep,
+                               seq_len=total, mask=dev(mask)))
+    for i in range(B):
+        close(got[i], o.vonly_decode_attention(qb[i], Kb[i, :, :total], vpb[i, :, :total], vnb[i, :, :total], cs, vss,
+                                               D, bits, sc, mask=mask[i]))
+
+
+@pytest.mark.parametrize("bits", [1, 2, 4])
+def test_vonly_decode_other_widths_masked_eight_wave_tiles(tq, bits):
+    """20 000 masked positions of 4 kv heads: 160 tiles of 512, the eight-wave shape with the mask reads."""
+    rng = np.random.default_rng(325 + bits)
+    n_kv, n_rep, T = 4, 7, 20000
+    sc = 1 / math.sqrt(D)
+    c, vs, K, vp, vn = fixture(rng, n_kv, T, bits)
+    q = rng.standard_normal((1, n_kv * n_rep, D)).astype(np.float16)
+    mask = np.where(rng.random((1, 1, T)) < 0.3, -np.inf, 0.0).astype(F32)
+    mask += (rng.standard_normal((1, 1, T)) * 0.5).astype(F32) * np.isfinite(mask)
+    got = host(tq.vonly_decode(dev(q), dev(K), dev(vp), dev(vn), c, dev(vs), D, bits, sc, n_rep=n_rep, mask=dev(mask)))
+    close(got[0], o.vonly_decode_attention(q[0], K, vp, vn, c, vs, D, bits, sc, mask=mask[0]))
+
+
+# one case per launch shape (28 query / 4 kv heads): eight-wave full tiles, four-wave full tiles, the ragged tile of
+# either, the streaming pass over whole blocks and with a ragged end
+SHAPES = [(32768, "eight waves, full tiles"), (4096, "four waves, full tiles"), (32769 - 200, "eight waves, ragged end"),
+          (40000, "four waves, ragged end"), (65536, "streaming, whole blocks"), (50000, "streaming, ragged end")]
+
+
+@pytest.mark.parametrize("bits", [1, 2, 4])
+@pytest.mark.parametrize("T,shape", SHAPES)
+def test_vonly_decode_other_widths_every_launch_shape(tq, bits, T, shape):
+    """Values are encoded on the GPU (the generic encoder, bit-exact against the oracle elsewhere) with norms that
+    jump by 2^+-6 between 512-position blocks, so the power-of-two norm scale of the streaming pass changes from
+    block to block; the oracle sees the same packed words and norms."""
+    rng = np.random.default_rng(330 + bits)
+    n_kv, n_rep = 4, 7
+    c = o.gaussian_codebook(bits)
+    b = o.gaussian_boundaries(c)
+    vs = o.random_diagonal_sign(D, 43)
+    sc = 1 / math.sqrt(D)
+    K = rng.standard_normal((n_kv, T, D)).astype(np.float16)
+    V = rng.standard_normal((n_kv, T, D)).astype(F32)
+    V *= (2.0 ** rng.integers(-6, 7, size=(n_kv, (T + 511) // 512, 1))).repeat(512, axis=1)[:, :T]
+    vp, vn = tq.fused_quantize(dev(V.astype(np.float16)).reshape(-1, D), dev(vs), b, D, bits)
+    vp, vn = vp.reshape(n_kv, T, -1), vn.reshape(n_kv, T)
+    hp, hn = vp.cpu().numpy(), vn.cpu().numpy()
+    for qdt in (np.float16, np.float32):
+        q = rng.standard_normal((1, n_kv * n_rep, D)).astype(qdt)
+        got = host(tq.vonly_decode(dev(q), dev(K), vp, vn, c, dev(vs), D, bits, sc, n_rep=n_rep))
+        want = o.vonly_decode_attention(q[0], K, hp, hn, c, vs, D, bits, sc)
+        close(got[0], want)
+
+
+@pytest.mark.parametrize("bits", [2, 4])
+def test_vonly_cache_other_widths_decode_through_the_cache(tq, bits):
+    """A VOnlyTurboQuantCache of another width: prompt, a few decode steps, attention after each against the oracle
+    on the cache's own packed state."""
+    rng = np.random.default_rng(340 + bits)
+    B, n_kv, n_rep, S = 2, 4, 7, 300
+    sc = 1 / math.sqrt(D)
+    cache = tq.VOnlyTurboQuantCache(bits=bits, seed=11, no_v_buffer=True)
+    k = torch.from_numpy(rng.standard_normal((B, n_kv, S, D)).astype(np.float16)).cuda()
+    v = torch.from_numpy(rng.standard_normal((B, n_kv, S, D)).astype(np.float16)).cuda()
+    cache.update_and_fetch(k, v)
+    for step in range(3):
+        k1 = torch.from_numpy(rng.standard_normal((B, n_kv, 1, D)).astype(np.float16)).cuda()
+        v1 = torch.from_numpy(rng.standard_normal((B, n_kv, 1, D)).astype(np.float16)).cuda()
+        cache.update_and_fetch(k1, v1)
+        q = torch.from_numpy(rng.standard_normal((B, n_kv * n_rep, 1, D)).astype(np.float16)).cuda()
+        got = host(tq.vonly_decode_attention(q, cache, sc))[:, :, 0, :]
+        total = cache.offset
+        assert total == S + step + 1
+        tqc = cache._v_tq
+        keys = cache._k_cache.keys[:, :, :total].cpu().numpy()
+        vp, vn = tqc.v_packed[:, :, :total].cpu().numpy(), tqc.v_norms[:, :, :total].cpu().numpy()
+        cen, sg = np.asarray(tqc._v_q.centroids, dtype=F32), tqc._v_q.signs.cpu().numpy()
+        for bi in range(B):
+            want = o.vonly_decode_attention(q[bi, :, 0].cpu().numpy(), keys[bi], vp[bi], vn[bi], cen, sg, D, bits, sc)
+            close(got[bi], want)

@@ -795,18 +795,16 @@ int launch_vonly_mfma(const void* q, int q_dtype, const void* k_f16, const uint3
   a.v_unscale = tq::fill_codebook_fp16(vcb, v_centroids, sh.bits);
   if ((phases & 1) && n_tiles_real > 0) {
     dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
-    const bool plain4 = plain_base && sh.seq_len % 256 == 0;           // full 256-position tiles
-#define LAUNCH_TILE(QF)                                                                                          \
-    if (n_blocks > 1 && ragged_stream) tqm::vonly_stream_kernel<QF, true><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb, n_blocks); \
-    else if (n_blocks > 1) tqm::vonly_stream_kernel<QF, false><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, vcb, n_blocks); \
-    else if (nw == 8 && plain) tqm::vonly_tile_mfma_kernel<true, QF, 8><<<grid, 512, 0, stream>>>(a, vcb);           \
-    else if (nw == 8 && plain_any) tqm::vonly_tile_anylen_kernel<QF, 8><<<grid, 512, 0, stream>>>(a, vcb);           \
-    else if (nw == 8) tqm::vonly_tile_mfma_kernel<false, QF, 8><<<grid, 512, 0, stream>>>(a, vcb);                   \
-    else if (plain4) tqm::vonly_tile_mfma_kernel<true, QF, 4><<<grid, 256, 0, stream>>>(a, vcb);                     \
-    else if (plain_any) tqm::vonly_tile_anylen_kernel<QF, 4><<<grid, 256, 0, stream>>>(a, vcb);                      \
-    else tqm::vonly_tile_mfma_kernel<false, QF, 4><<<grid, 256, 0, stream>>>(a, vcb)
-    if (q_f32) { LAUNCH_TILE(true); } else { LAUNCH_TILE(false); }
-#undef LAUNCH_TILE
+    tqm::VonlyTileChoice ch{};
+    ch.nw = nw; ch.n_blocks = n_blocks; ch.ragged_stream = ragged_stream; ch.plain = plain;
+    ch.plain4 = plain_base && sh.seq_len % 256 == 0;                    // full 256-position tiles
+    ch.plain_any = plain_any; ch.q_f32 = q_f32;
+    switch (sh.bits) {
+      case 1: tqm::launch_vonly_tiles<1>(grid, ch, a, vcb, stream); break;
+      case 2: tqm::launch_vonly_tiles<2>(grid, ch, a, vcb, stream); break;
+      case 4: tqm::launch_vonly_tiles<4>(grid, ch, a, vcb, stream); break;
+      default: tqm::launch_vonly_tiles<3>(grid, ch, a, vcb, stream); break;
+    }
     TQ_CHECK_LAUNCH(who);
   }
   if (!(phases & 2)) return TQ_OK;
@@ -1074,6 +1072,11 @@ bool mma_shape(const tq_decode_shape& sh) {
   return sh.allow_mma && sh.dim == 128 && sh.bits == 3 && sh.n_rep <= tqm::kHeadsMax && sh.seq_len > 0;
 }
 
+// the tile pass over fp16 keys and packed values exists for every value width
+bool vonly_mma_shape(const tq_decode_shape& sh) {
+  return sh.allow_mma && sh.dim == 128 && sh.bits >= 1 && sh.bits <= 4 && sh.n_rep <= tqm::kHeadsMax && sh.seq_len > 0;
+}
+
 int check_shape(const tq_decode_shape* sh, const char* who, int max_dim) {
   if (!sh) return tq::fail(TQ_ERR_NULL, "%s: null shape", who);
   if (int rc = tq::check_dim_bits(sh->dim, sh->bits)) return rc;
@@ -1243,8 +1246,8 @@ extern "C" int tq_vonly_decode_attn_phases(const void* q, int q_dtype, const voi
   if (shape->seq_len > 0 && (!k_f16 || !v_packed || !v_norms))
     return tq::fail(TQ_ERR_NULL, "tq_vonly_decode_attn: null pointer");
   if (!tq::aligned(k_f16, 16)) return tq::fail(TQ_ERR_ALIGN, "tq_vonly_decode_attn: k must be 16-byte aligned");
-  // d = 128, 3-bit, at most 16 query heads per kv head: matrix-core tile pass (float32 queries as fp16 value + remainder).
-  if (mma_shape(*shape) && tq::aligned(q, 16))
+  // d = 128, at most 16 query heads per kv head: matrix-core tile pass (float32 queries as fp16 value + remainder).
+  if (vonly_mma_shape(*shape) && tq::aligned(q, 16))
     return launch_vonly_mfma(q, q_dtype, k_f16, v_packed, v_norms, v_centroids, v_signs, out, workspace, workspace_bytes,
                              *shape, (hipStream_t)stream_, phases);
   return launch_decode<kDenseK>(q, q_dtype, nullptr, nullptr, k_f16, v_packed, v_norms, nullptr, v_centroids,

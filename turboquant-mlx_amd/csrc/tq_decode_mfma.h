@@ -97,6 +97,55 @@ __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
   return *reinterpret_cast<uint32_t*>(&h);
 }
 
+// Packed values of one bit width (d = 128): words per row, and how a lane gets at the 8 * BITS bits that hold
+// elements 8 pc .. 8 pc + 7 of a row.  Three-bit rows hold ten fields per word, so a piece may straddle two
+// words; the other widths divide the word.
+template <int BITS>
+struct VField {
+  static constexpr int kPd = BITS == 3 ? 13 : 4 * BITS;                  // words per packed row
+  static constexpr uint32_t kEven = BITS == 3 ? 0x1C71C7u : BITS == 4 ? 0x0F0F0F0Fu : BITS == 2 ? 0x3333u : 0x55u;   // fields 0, 2, 4, 6
+  static constexpr int kLut = 1 << (2 * BITS);                            // entries of the centroid-pair table
+  __device__ static __forceinline__ void pos(int pc, int& w0, int& sh_lo, int& sh_hi) {
+    if (BITS == 3) {
+      w0 = (pc == 15) ? 11 : (8 * pc) / 10;                               // piece 15: word 11 >> 30 is 0, all of word 12
+      const int s0 = (pc == 15) ? 10 : (8 * pc) % 10;
+      sh_lo = 3 * s0;
+      sh_hi = 30 - 3 * s0;
+    } else {
+      constexpr int kPerWord = 4 / BITS;                                  // pieces per word: 1, 2, 4 for 4, 2, 1 bits
+      w0 = pc / kPerWord;
+      sh_lo = (pc % kPerWord) * 8 * BITS;
+      sh_hi = 0;
+    }
+  }
+  __device__ static __forceinline__ uint32_t field(const uint32_t* at_w0, int sh_lo, int sh_hi) {
+    if (BITS == 3) return ((at_w0[0] >> sh_lo) | (at_w0[1] << sh_hi)) & 0xFFFFFFu;
+    if (BITS == 4) return at_w0[0];
+    return (at_w0[0] >> sh_lo) & ((1u << (8 * BITS)) - 1u);
+  }
+  // even / odd fields of two rows interleaved into table indices at bit offsets 0, 2 BITS, 4 BITS, 6 BITS
+  __device__ static __forceinline__ void interleave(uint32_t fa, uint32_t fb, uint32_t& X, uint32_t& Y) {
+    X = (fa & kEven) | ((fb & kEven) << BITS);
+    Y = ((fa >> BITS) & kEven) | (fb & (kEven << BITS));
+  }
+  __device__ static __forceinline__ uint32_t index(uint32_t src, int i) { return (src >> (2 * BITS * i)) & (uint32_t)(kLut - 1); }
+  // this lane's entries of a table of kLut centroid pairs half2(c[i & mask], c[i >> BITS]); selects, not a dynamic
+  // index into kernel arguments
+  __device__ static __forceinline__ void fill(uint32_t* lut, const Codebook& cb, int lane) {
+#pragma unroll
+    for (int base = 0; base < kLut; base += 64) {
+      const int idx = base + lane;
+      float clo = 0.0f, chi = 0.0f;
+#pragma unroll
+      for (int i = 0; i < (1 << BITS); ++i) {
+        clo = ((idx & ((1 << BITS) - 1)) == i) ? cb.c[i] : clo;
+        chi = ((idx >> BITS) == i) ? cb.c[i] : chi;
+      }
+      if (kLut >= 64 || idx < kLut) lut[idx] = pack_h2(clo, chi);
+    }
+  }
+};
+
 // Cross-wave merge of a workgroup's tile.  Every wave leaves, per head, the maximum m of its scores (log2 units)
 // and its weight sum l, its power-of-two accumulator scale, and its RAW accumulator rows in an LDS area of its
 // own (`area`, 4 KB: eight rows of 128 floats; nothing of another wave lives there, so no barrier is needed
@@ -172,15 +221,17 @@ __device__ __forceinline__ void merge_waves(MergeLds<NW>& mg, unsigned char* are
 // narrow V path drop out, and K / V addresses are a uniform base plus a lane-constant offset.
 // QF32: the queries are float32 and enter as an fp16 value plus the fp16 remainder of that rounding (two
 // matrix instructions per key operand), which keeps float32-query fidelity; otherwise fp16 (or bf16) queries.
-template <bool PLAIN, bool QF32, int NW>
+template <bool PLAIN, bool QF32, int NW, int BITS>
 __device__ __forceinline__ void vonly_tile_body(const MfmaArgs& a, const Codebook& vcb, const int64_t first,
                                                 const int64_t len) {
+  using VF = VField<BITS>;
+  constexpr int kPd = VF::kPd;                         // words per packed value row
   constexpr int kTPos = NW * kWavePos;                 // positions per workgroup
   constexpr int kThr = NW * 64;
   // 4 KB per wave used three ways: per-wave staging first for the packed V block, then for K
   // tiles; finally the cross-wave merge buffer S_all[NW][8][128].
   __shared__ __align__(16) unsigned char big_s[NW * 4096];
-  __shared__ uint32_t lut_s[NW][64];                   // per wave: half2(c[i & 7], c[i >> 3])
+  __shared__ uint32_t lut_s[NW][VF::kLut < 64 ? 64 : VF::kLut];   // per wave: half2(c[i & mask], c[i >> BITS])
   __shared__ __align__(16) float nrm_s[NW][kWavePos];
   __shared__ __align__(16) MergeLds<NW> mg_s;
 
@@ -224,24 +275,26 @@ __device__ __forceinline__ void vonly_tile_body(const MfmaArgs& a, const Codeboo
     if (!PLAIN) row = row < last_row ? row : last_row;
     my_norm = nb[(unsigned)row];
   }
-  // packed V of the wave: 64 rows x 52 bytes, contiguous.  Full, 16-byte aligned blocks take four
-  // 16-byte loads per lane; ragged or unaligned ones take thirteen 4-byte loads with the index
+  // packed V of the wave: 64 rows x 4 kPd bytes (52 at three bits), contiguous.  Full, 16-byte aligned blocks
+  // take up to four 16-byte loads per lane; ragged or unaligned ones take kPd 4-byte loads with the index
   // clamped to the last valid word.  Either way the LDS image is the plain copy of the block.
+  constexpr int kVFull = (16 * kPd) / 64;              // whole-wave 16-byte loads: 3 at three bits (then 16 more pieces)
+  constexpr int kVTail = 16 * kPd - 64 * kVFull;       // pieces of the last, partial load (0 or 16)
   const uint32_t* vblock = a.v_packed +
-      ((int64_t)seq * a.v_seq_stride + (int64_t)kvh * a.v_head_stride + first + tile_p0 + wrow0) * kPdim;
+      ((int64_t)seq * a.v_seq_stride + (int64_t)kvh * a.v_head_stride + first + tile_p0 + wrow0) * kPd;
   const bool v_wide = PLAIN || ((wrow0 + kWavePos <= rows_here) && ((reinterpret_cast<uintptr_t>(vblock) & 15) == 0));
   u4 vq[4];
-  uint32_t vd[13];
+  uint32_t vd[kPd];
   if (v_wide) {
     const char* vb = reinterpret_cast<const char*>(vblock);
 #pragma unroll
-    for (int i = 0; i < 3; ++i) vq[i] = *reinterpret_cast<const u4*>(vb + i * 1024 + (uint32_t)(lane * 16));
-    vq[3] = *reinterpret_cast<const u4*>(vb + 3072 + (uint32_t)((lane & 15) * 16));   // 208 pieces in all; lanes >= 16 repeat
+    for (int i = 0; i < kVFull; ++i) vq[i] = *reinterpret_cast<const u4*>(vb + i * 1024 + (uint32_t)(lane * 16));
+    if (kVTail) vq[kVFull] = *reinterpret_cast<const u4*>(vb + kVFull * 1024 + (uint32_t)((lane & (kVTail - 1)) * 16));   // lanes >= kVTail repeat
   } else {
-    const int valid_words = max(0, rows_here - wrow0) * kPdim;       // words of the block inside the sequence
-    const uint32_t* tile_base = vblock - (int64_t)wrow0 * kPdim;     // row 0 of the tile: always valid
+    const int valid_words = max(0, rows_here - wrow0) * kPd;         // words of the block inside the sequence
+    const uint32_t* tile_base = vblock - (int64_t)wrow0 * kPd;       // row 0 of the tile: always valid
 #pragma unroll
-    for (int i = 0; i < 13; ++i) {
+    for (int i = 0; i < kPd; ++i) {
       const int w = i * 64 + lane;
       vd[i] = (w < valid_words) ? vblock[w] : tile_base[0];
     }
@@ -279,15 +332,7 @@ __device__ __forceinline__ void vonly_tile_body(const MfmaArgs& a, const Codeboo
 #pragma unroll
   for (int i = 0; i < 8; ++i) issue_k(i);
   __builtin_amdgcn_sched_barrier(0);
-  {
-    float clo = 0.0f, chi = 0.0f;                        // selects, not a dynamic index into kernel arguments
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      clo = ((lane & 7) == i) ? vcb.c[i] : clo;
-      chi = ((lane >> 3) == i) ? vcb.c[i] : chi;
-    }
-    lut_s[wave][lane] = pack_h2(clo, chi);
-  }
+  VF::fill(lut_s[wave], vcb, lane);
   nrm_s[wave][lane] = my_norm;
   const uint32_t* lut_w = lut_s[wave];
 
@@ -337,31 +382,26 @@ __device__ __forceinline__ void vonly_tile_body(const MfmaArgs& a, const Codeboo
   if (v_wide) {
     u4* st4 = reinterpret_cast<u4*>(stage);
 #pragma unroll
-    for (int i = 0; i < 3; ++i) st4[i * 64 + lane] = vq[i];
-    if (lane < 16) st4[192 + lane] = vq[3];
+    for (int i = 0; i < kVFull; ++i) st4[i * 64 + lane] = vq[i];
+    if (kVTail) { if (lane < kVTail) st4[kVFull * 64 + lane] = vq[kVFull]; }
   } else {
 #pragma unroll
-    for (int i = 0; i < 13; ++i) stage[i * 64 + lane] = vd[i];
+    for (int i = 0; i < kPd; ++i) stage[i * 64 + lane] = vd[i];
   }
-  // lane (n16, g) decodes elements 8*n16 .. 8*n16+7 of positions 16t + 4g + j: 24 bits that start in
-  // word w0 at field s0 and may spill into word w0 + 1 (lane 15 reads words 11, 12 and takes
+  // lane (n16, g) decodes elements 8*n16 .. 8*n16+7 of positions 16t + 4g + j: 8 * BITS bits that start in
+  // word w0 (at three bits they may spill into word w0 + 1; lane 15 then reads words 11, 12 and takes
   // everything from the second).  X / Y interleave the even / odd fields of two positions into
-  // 6-bit table indices at bit offsets 0, 6, 12, 18; each index fetches a centroid pair.
-  const int w0 = (n16 == 15) ? 11 : (8 * n16) / 10;
-  const int s0 = (n16 == 15) ? 10 : (8 * n16) % 10;
-  const int sh_lo = 3 * s0, sh_hi = 30 - 3 * s0;
-  constexpr uint32_t kEven = 0x1C71C7u;        // fields 0, 2, 4, 6
+  // table indices of 2 * BITS bits each; each index fetches a centroid pair.
+  int w0, sh_lo, sh_hi;
+  VF::pos(n16, w0, sh_lo, sh_hi);
   uint32_t X[2][4], Y[2][4];
 #pragma unroll
   for (int kb2 = 0; kb2 < 2; ++kb2)
 #pragma unroll
     for (int qd = 0; qd < 4; ++qd) {
       const int t = 2 * kb2 + (qd >> 1), jp = qd & 1;
-      const uint32_t* ra = stage + (16 * t + 4 * g + 2 * jp) * kPdim + w0;
-      const uint32_t fa = ((ra[0] >> sh_lo) | (ra[1] << sh_hi)) & 0xFFFFFFu;
-      const uint32_t fb = ((ra[kPdim] >> sh_lo) | (ra[kPdim + 1] << sh_hi)) & 0xFFFFFFu;
-      X[kb2][qd] = (fa & kEven) | ((fb & kEven) << 3);
-      Y[kb2][qd] = ((fa >> 3) & kEven) | (fb & (kEven << 3));
+      const uint32_t* ra = stage + (16 * t + 4 * g + 2 * jp) * kPd + w0;
+      VF::interleave(VF::field(ra, sh_lo, sh_hi), VF::field(ra + kPd, sh_lo, sh_hi), X[kb2][qd], Y[kb2][qd]);
     }
   u4 breg[2][8];
   auto lookups = [&](int kb2) {
@@ -370,7 +410,7 @@ __device__ __forceinline__ void vonly_tile_body(const MfmaArgs& a, const Codeboo
 #pragma unroll
       for (int qd = 0; qd < 4; ++qd) {
         const uint32_t src = (et & 1) ? Y[kb2][qd] : X[kb2][qd];
-        breg[kb2][et][qd] = lut_w[(src >> (6 * (et >> 1))) & 63u];
+        breg[kb2][et][qd] = lut_w[VF::index(src, et >> 1)];
       }
   };
   // one 16-position score tile: K pieces through the wave's staging area, 4 matrix instructions
@@ -476,7 +516,7 @@ __device__ __forceinline__ void vonly_tile_body(const MfmaArgs& a, const Codeboo
   merge_waves<NW>(mg_s, big_s, 4096, accS, m, l, inv_tscale, a.v_unscale, n_rep, pS, pml);
 }
 
-template <bool PLAIN, bool QF32, int NW>
+template <bool PLAIN, bool QF32, int NW, int BITS = 3>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 8 ? 2 : 3, NW == 8 ? 2 : 3)))
 void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
   int64_t first = 0, len = a.seq_len;
@@ -487,14 +527,14 @@ void vonly_tile_mfma_kernel(MfmaArgs a, Codebook vcb) {
     const int64_t want = *a.len_dev + a.len_bias;
     len = want < 0 ? 0 : (want < len ? want : len);
   }
-  vonly_tile_body<PLAIN, QF32, NW>(a, vcb, first, len);
+  vonly_tile_body<PLAIN, QF32, NW, BITS>(a, vcb, first, len);
 }
 
 // The same pass for unmasked caches of ANY length (host-checked: no mask, no ragged offsets, positive scale,
 // 16-byte aligned value rows): a workgroup whose tile lies wholly inside the sequence runs the PLAIN body, the one
 // tile that straddles the end runs the general body, tiles past the end leave at once.  The length may live in
 // device memory (len_dev), which is what a step recorded in a HIP graph needs.
-template <bool QF32, int NW>
+template <bool QF32, int NW, int BITS = 3>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 8 ? 2 : 3, NW == 8 ? 2 : 3)))
 void vonly_tile_anylen_kernel(MfmaArgs a, Codebook vcb) {
   int64_t len = a.seq_len;
@@ -503,8 +543,8 @@ void vonly_tile_anylen_kernel(MfmaArgs a, Codebook vcb) {
     len = want < 0 ? 0 : (want < len ? want : len);
   }
   const int64_t tile_end = ((int64_t)blockIdx.x + 1) * (NW * kWavePos);
-  if (tile_end <= len) vonly_tile_body<true, QF32, NW>(a, vcb, 0, len);
-  else vonly_tile_body<false, QF32, NW>(a, vcb, 0, len);
+  if (tile_end <= len) vonly_tile_body<true, QF32, NW, BITS>(a, vcb, 0, len);
+  else vonly_tile_body<false, QF32, NW, BITS>(a, vcb, 0, len);
 }
 
 // Scores pass of the thresholded decode step (weights below a threshold are dropped, and the threshold
@@ -695,11 +735,14 @@ __global__ __launch_bounds__(WAVES * 64) void vonly_scores_kernel(MfmaArgs a) {
 // 16-byte piece that holds a valid byte never crosses a page) and the scores of those rows are set to -inf.
 constexpr int kStepPos = 32;
 
-template <bool QF32, bool RAGGED>
+template <bool QF32, bool RAGGED, int BITS = 3>
 __global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
+  using VF = VField<BITS>;
+  constexpr int kPd = VF::kPd;                           // words per packed value row
+  constexpr int kPieces = 8 * kPd;                       // 16-byte pieces of a step's 32 packed rows: 104 at three bits
   __shared__ __align__(16) unsigned char big_s[32768];
-  __shared__ uint32_t lut_s[64];
+  __shared__ uint32_t lut_s[VF::kLut < 64 ? 64 : VF::kLut];
   __shared__ __align__(16) uint32_t q_s[kHeadsMax][kD / 2];
   __shared__ __align__(16) uint32_t ql_s[QF32 ? kHeadsMax : 1][kD / 2];
   __shared__ __align__(16) float nrm_s[kWaves][kStepPos];
@@ -725,10 +768,13 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
   const float* nbase = a.v_norms + (int64_t)seq * a.vn_seq_stride + (int64_t)kvh * a.vn_head_stride + tile_p0 +
                        (RAGGED ? 0 : (lane & 31));
   const char* vbase = reinterpret_cast<const char*>(
-      a.v_packed + ((int64_t)seq * a.v_seq_stride + (int64_t)kvh * a.v_head_stride + tile_p0) * kPdim);
+      a.v_packed + ((int64_t)seq * a.v_seq_stride + (int64_t)kvh * a.v_head_stride + tile_p0) * kPd);
   const char* kbase = reinterpret_cast<const char*>(
       a.k + ((int64_t)seq * a.k_seq_stride + (int64_t)kvh * a.k_head_stride + tile_p0) * kD);
-  const uint32_t voff0 = (uint32_t)(lane * 16), voff1 = (uint32_t)((lane < 40 ? 64 + lane : 103) * 16);   // 104 pieces
+  // pieces lane and 64 + lane of a step's block (the second load only where a block has more than 64 pieces);
+  // lanes past the last piece repeat an earlier one
+  const uint32_t voff0 = (uint32_t)((kPieces >= 64 ? lane : (lane & (kPieces - 1))) * 16);
+  const uint32_t voff1 = (uint32_t)((64 + lane < kPieces ? 64 + lane : kPieces - 1) * 16);
   const uint32_t koff_even = (uint32_t)(((lane >> 4) * 16 + ((lane & 15) ^ ((lane >> 4) & 7))) * 16);
   const uint32_t koff_odd = (uint32_t)(((4 + (lane >> 4)) * 16 + ((lane & 15) ^ ((4 + (lane >> 4)) & 7))) * 16);
   auto issue_nv = [&](int s, float& nrm, u4 (&vqx)[2]) {
@@ -736,15 +782,15 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
     if (RAGGED) {
       nrm = nbase[min(r + (lane & 31), last_valid)];
       const int rc = min(r, last_step_row);                             // a step with no valid row re-reads the last one that has
-      const uint32_t limit = (uint32_t)((valid - rc) * (kPdim * 4));     // bytes of valid rows from rc on (> 0)
-      const char* vb = vbase + (int64_t)rc * (kPdim * 4);
+      const uint32_t limit = (uint32_t)((valid - rc) * (kPd * 4));       // bytes of valid rows from rc on (> 0)
+      const char* vb = vbase + (int64_t)rc * (kPd * 4);
       vqx[0] = *reinterpret_cast<const u4*>(vb + (voff0 < limit ? voff0 : 0u));
-      vqx[1] = *reinterpret_cast<const u4*>(vb + (voff1 < limit ? voff1 : 0u));
+      if (kPieces > 64) vqx[1] = *reinterpret_cast<const u4*>(vb + (voff1 < limit ? voff1 : 0u));
     } else {
       nrm = nbase[r];
-      const char* vb = vbase + (int64_t)r * (kPdim * 4);
+      const char* vb = vbase + (int64_t)r * (kPd * 4);
       vqx[0] = *reinterpret_cast<const u4*>(vb + voff0);
-      vqx[1] = *reinterpret_cast<const u4*>(vb + voff1);
+      if (kPieces > 64) vqx[1] = *reinterpret_cast<const u4*>(vb + voff1);
     }
   };
   auto issue_k4 = [&](int s, u4 (&kx)[8], int part) {     // instructions 4*part .. 4*part+3: rows 16*part .. +15 of the step
@@ -790,15 +836,7 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
   issue_k4(0, kA, 1);
   __builtin_amdgcn_sched_barrier(0);
 
-  if (tid < 64) {
-    float clo = 0.0f, chi = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      clo = ((tid & 7) == i) ? vcb.c[i] : clo;
-      chi = ((tid >> 3) == i) ? vcb.c[i] : chi;
-    }
-    lut_s[tid] = pack_h2(clo, chi);
-  }
+  if (tid < 64) VF::fill(lut_s, vcb, tid);
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     // bf16 queries become fp16 here, after every load of the pass has been requested: converting where the word
@@ -818,10 +856,8 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
   const float cs = a.attn_scale * kLog2e;
   uint32_t* stage = reinterpret_cast<uint32_t*>(big_s) + wave * 1024;   // this wave's 4 KB
   u4* kst = reinterpret_cast<u4*>(stage);
-  const int w0 = (n16 == 15) ? 11 : (8 * n16) / 10;
-  const int s0 = (n16 == 15) ? 10 : (8 * n16) % 10;
-  const int sh_lo = 3 * s0, sh_hi = 30 - 3 * s0;
-  constexpr uint32_t kEven = 0x1C71C7u;
+  int w0, sh_lo, sh_hi;
+  VF::pos(n16, w0, sh_lo, sh_hi);
 
   f4 accS[8];
 #pragma unroll
@@ -849,8 +885,8 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
     // ---- packed V -> table indices -> centroid pairs
     {
       u4* st4 = reinterpret_cast<u4*>(stage);
-      st4[lane] = vqx[0];
-      if (lane < 40) st4[64 + lane] = vqx[1];
+      if (kPieces >= 64 || lane < kPieces) st4[lane] = vqx[0];
+      if (kPieces > 64) { if (64 + lane < kPieces) st4[64 + lane] = vqx[1]; }
     }
     __builtin_amdgcn_sched_barrier(0);
     next(0);
@@ -859,11 +895,8 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
 #pragma unroll
     for (int qd = 0; qd < 4; ++qd) {
       const int t = qd >> 1, jp = qd & 1;
-      const uint32_t* ra = stage + (16 * t + 4 * g + 2 * jp) * kPdim + w0;
-      const uint32_t fa = ((ra[0] >> sh_lo) | (ra[1] << sh_hi)) & 0xFFFFFFu;
-      const uint32_t fb = ((ra[kPdim] >> sh_lo) | (ra[kPdim + 1] << sh_hi)) & 0xFFFFFFu;
-      X[qd] = (fa & kEven) | ((fb & kEven) << 3);
-      Y[qd] = ((fa >> 3) & kEven) | (fb & (kEven << 3));
+      const uint32_t* ra = stage + (16 * t + 4 * g + 2 * jp) * kPd + w0;
+      VF::interleave(VF::field(ra, sh_lo, sh_hi), VF::field(ra + kPd, sh_lo, sh_hi), X[qd], Y[qd]);
     }
     u4 breg[8];
 #pragma unroll
@@ -871,7 +904,7 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
 #pragma unroll
       for (int qd = 0; qd < 4; ++qd) {
         const uint32_t src = (et & 1) ? Y[qd] : X[qd];
-        breg[et][qd] = lut_s[(src >> (6 * (et >> 1))) & 63u];
+        breg[et][qd] = lut_s[VF::index(src, et >> 1)];
       }
     __builtin_amdgcn_sched_barrier(0);
     next(1);
@@ -1237,5 +1270,38 @@ __global__ __launch_bounds__(kMergeThreads + 64) void decode_merge_fresh_kernel(
   merge_rows_body<TO, true, U, true>(ws_S, ws_ml, nullptr, seq_len, n_tiles_max, n_kv, n_rep, signs, inv_dim, out,
                                      tile_pos, len_dev, 0, &ft);
 }
+
+// Which tile kernel a launch uses (chosen by the host from the length, the mask / offsets and the alignment).
+struct VonlyTileChoice {
+  int nw;                     // waves per workgroup of the single-tile shapes: 8 or 4
+  int n_blocks;               // > 1: streaming pass, that many 512-position blocks per workgroup
+  bool ragged_stream;         // the streaming pass with a ragged end
+  bool plain;                 // full 512-position tiles, no mask, no offsets
+  bool plain4;                // full 256-position tiles, no mask, no offsets
+  bool plain_any;             // no mask, no offsets, any length
+  bool q_f32;
+};
+
+// The tile pass for values of BITS bits.  Instantiated once per width: 3 beside the host code of the decode
+// entry points, 1, 2 and 4 in a translation unit of their own.
+template <int BITS>
+void launch_vonly_tiles(dim3 grid, const VonlyTileChoice& c, const MfmaArgs& a, const Codebook& vcb, hipStream_t stream) {
+#define TQ_LAUNCH_TILE(QF)                                                                                              \
+  if (c.n_blocks > 1 && c.ragged_stream) vonly_stream_kernel<QF, true, BITS><<<grid, kMfmaThreads, 0, stream>>>(a, vcb, c.n_blocks); \
+  else if (c.n_blocks > 1) vonly_stream_kernel<QF, false, BITS><<<grid, kMfmaThreads, 0, stream>>>(a, vcb, c.n_blocks);  \
+  else if (c.nw == 8 && c.plain) vonly_tile_mfma_kernel<true, QF, 8, BITS><<<grid, 512, 0, stream>>>(a, vcb);           \
+  else if (c.nw == 8 && c.plain_any) vonly_tile_anylen_kernel<QF, 8, BITS><<<grid, 512, 0, stream>>>(a, vcb);           \
+  else if (c.nw == 8) vonly_tile_mfma_kernel<false, QF, 8, BITS><<<grid, 512, 0, stream>>>(a, vcb);                     \
+  else if (c.plain4) vonly_tile_mfma_kernel<true, QF, 4, BITS><<<grid, 256, 0, stream>>>(a, vcb);                       \
+  else if (c.plain_any) vonly_tile_anylen_kernel<QF, 4, BITS><<<grid, 256, 0, stream>>>(a, vcb);                        \
+  else vonly_tile_mfma_kernel<false, QF, 4, BITS><<<grid, 256, 0, stream>>>(a, vcb)
+  if (c.q_f32) { TQ_LAUNCH_TILE(true); } else { TQ_LAUNCH_TILE(false); }
+#undef TQ_LAUNCH_TILE
+}
+#ifndef TQ_VONLY_OTHER_WIDTHS_HERE
+extern template void launch_vonly_tiles<1>(dim3, const VonlyTileChoice&, const MfmaArgs&, const Codebook&, hipStream_t);
+extern template void launch_vonly_tiles<2>(dim3, const VonlyTileChoice&, const MfmaArgs&, const Codebook&, hipStream_t);
+extern template void launch_vonly_tiles<4>(dim3, const VonlyTileChoice&, const MfmaArgs&, const Codebook&, hipStream_t);
+#endif
 
 }  // namespace tqm

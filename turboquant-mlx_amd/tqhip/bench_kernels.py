@@ -6,7 +6,7 @@ back-to-back launches, and rotation over several independent input sets so that 
 Infinity Cache cannot serve the reads.  Prints one line per case: us per call, GB/s of algorithmic
 bytes and the fraction of 8 TB/s.
 
-    python -m tqhip.bench_kernels [--iters 200] [--cases encode,scores,flash,flash_long,sparse_v,vonly,prefill,step]
+    python -m tqhip.bench_kernels [--iters 200] [--cases encode,scores,flash,flash_long,sparse_v,vonly,widths,prefill,step]
 """
 from __future__ import annotations
 
@@ -166,6 +166,57 @@ def bench_vonly(iters, dev):
                    timeit(fns, iters), nbytes)
 
 
+def timeit_graph(fns, iters):
+    """Like timeit, but the calls are recorded once into a HIP graph (one round over the input sets) and the
+    graph is replayed: kernel time without the cost of the Python calls."""
+    for f in fns:
+        f()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        for f in fns:
+            f()
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            for f in fns:
+                f()
+    reps = max(3, iters // len(fns))
+    graph.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / (reps * len(fns))
+
+
+def bench_widths(iters, dev):
+    """V-only decode at the other value widths (1, 2 and 4 bits): the matrix-core tile pass against the
+    float32 kernels that served these widths before it (precision="fp32"), HIP-graph replay."""
+    signs = tqhip.random_diagonal_sign(128, 43, device=dev)
+    g = torch.Generator(device=dev)
+    g.manual_seed(8)
+    for bits in (1, 2, 3, 4):
+        cb = gaussian_codebook(bits)
+        pd = tqhip.packed_dim(128, bits)
+        for T in (32768, 131072):
+            nbytes = 4 * T * (256 + 4 * pd + 4) + 28 * 256 * 2
+            n_sets = n_sets_for(nbytes)
+            ks = [torch.randn((4, T, 128), device=dev, dtype=torch.float16) for _ in range(n_sets)]
+            codes = [torch.randint(0, 2 ** bits, (4 * T, 128), generator=g, device=dev, dtype=torch.uint8) for _ in range(n_sets)]
+            ps = [tqhip.pack_indices(c, bits).reshape(4, T, pd) for c in codes]
+            ns = [torch.rand((4, T), generator=g, device=dev) + 0.1 for _ in range(n_sets)]
+            q = torch.randn((1, 28, 128), device=dev, dtype=torch.float16)
+            for prec in ("fp16", "fp32"):
+                fns = [(lambda k=k, p=p, n=n: tqhip.vonly_decode(q, k, p, n, cb, signs, 128, bits, 1 / math.sqrt(128),
+                                                                 n_rep=7, precision=prec)) for k, p, n in zip(ks, ps, ns)]
+                kind = "matrix cores" if prec == "fp16" else "float32 kernels"
+                report(f"V-only decode 28/4 heads, {bits}-bit values, T={T}, {kind} (graph)", timeit_graph(fns, iters), nbytes)
+
+
 def bench_prefill(iters, dev):
     """benchmark configuration 5, attention half: a chunk of 512 query rows x 32 heads at the end of a
     131072-position packed cache (8 kv heads), causal.  Matrix-core bound: reported in TFLOP/s of
@@ -258,7 +309,7 @@ def bench_step(iters, dev):
 
 
 CASES = {"step": bench_step, "prefill": bench_prefill, "encode": bench_encode, "scores": bench_scores, "sparse_v": bench_sparse_v, "flash": bench_flash,
-         "flash_long": bench_flash_long, "vonly": bench_vonly}
+         "flash_long": bench_flash_long, "vonly": bench_vonly, "widths": bench_widths}
 
 
 def main():
