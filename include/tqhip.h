@@ -216,7 +216,8 @@ typedef struct tq_decode_shape {
   float attn_scale;
   int32_t out_dtype;         /* TQ_F32, TQ_F16 or TQ_BF16 */
   int32_t allow_mma;         /* 1: use the fp16 matrix-core kernels where the shape allows (d = 128,
-                                3-bit, n_rep <= 16; operands rounded to fp16, float32 accumulation);
+                                n_rep <= 16; 3-bit keys and values for packed keys, values of any width
+                                1-4 beside fp16 keys; operands rounded to fp16, float32 accumulation);
                                 0: float32 vector-ALU kernels only */
 } tq_decode_shape;
 
@@ -250,6 +251,8 @@ int tq_flash_decode_plan(int n_seq, int n_kv_heads, int64_t max_seq_len, int rag
  * The composition dense-K scores -> softmax -> sparse_v_matvec of hybrid_attention.py:52-88 /
  * fused_attention.py:50-121 in one launch for the cache of v_only_cache.py:24-127.
  *   q [n_seq, n_kv*n_rep, dim] dtype q_dtype;  k_f16 rows of dim halfs;  out as tq_flash_decode.
+ * With allow_mma, d = 128 and n_rep <= 16 the tile pass runs on the matrix cores for values of every
+ * width (bits 1-4, as adaptive.py:26 / v_only_cache.py:41 take them); other shapes take the float32 kernels.
  */
 int tq_vonly_decode_attn(const void* q, int q_dtype, const void* k_f16,
                          const uint32_t* v_packed, const float* v_norms,

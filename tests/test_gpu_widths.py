@@ -183,3 +183,18 @@ def test_vonly_cache_other_widths_decode_through_the_cache(tq, bits):
         for bi in range(B):
             want = o.vonly_decode_attention(q[bi, :, 0].cpu().numpy(), keys[bi], vp[bi], vn[bi], cen, sg, D, bits, sc)
             close(got[bi], want)
+    # the single-call step (insert + attend): same result as the two halves
+    for step in range(2):
+        k1 = torch.from_numpy(rng.standard_normal((B, n_kv, 1, D)).astype(np.float16)).cuda()
+        v1 = torch.from_numpy(rng.standard_normal((B, n_kv, 1, D)).astype(np.float16)).cuda()
+        q = torch.from_numpy(rng.standard_normal((B, n_kv * n_rep, 1, D)).astype(np.float16)).cuda()
+        got = host(cache.decode_step(q, k1, v1, sc))[:, :, 0, :]
+        total = cache.offset
+        assert total == S + 3 + step + 1
+        tqc = cache._v_tq
+        keys = cache._k_cache.keys[:, :, :total].cpu().numpy()
+        vp, vn = tqc.v_packed[:, :, :total].cpu().numpy(), tqc.v_norms[:, :, :total].cpu().numpy()
+        assert np.array_equal(keys[:, :, -1], k1[:, :, 0].cpu().numpy())
+        for bi in range(B):
+            want = o.vonly_decode_attention(q[bi, :, 0].cpu().numpy(), keys[bi], vp[bi], vn[bi], cen, sg, D, bits, sc)
+            close(got[bi], want)
