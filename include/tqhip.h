@@ -411,8 +411,8 @@ int tq_vonly_decode_attn_phases(const void* q, int q_dtype, const void* k_f16,
  * a scores pass, a weights-and-values pass and the merge pass, with the scores of the step held in `workspace`
  * (tq_vonly_sparse_workspace_bytes) instead of three tensors of the caller.  Arguments as tq_vonly_decode_attn;
  * threshold >= 0 (0 = dense: every position contributes).  Rows whose positions are all masked out yield zeros.
- * Matrix-core shape only: dim 128, 3-bit values, n_rep <= 16, non-empty cache (TQ_ERR_UNSUPPORTED otherwise:
- * compose tq_dense_qk_scores, tq_softmax_rows and tq_sparse_v_matvec for those).
+ * Matrix-core shape only: dim 128, values of any width (bits 1-4), n_rep <= 16, non-empty cache
+ * (TQ_ERR_UNSUPPORTED otherwise: compose tq_dense_qk_scores, tq_softmax_rows and tq_sparse_v_matvec for those).
  */
 int tq_vonly_sparse_decode_attn(const void* q, int q_dtype, const void* k_f16,
                                 const uint32_t* v_packed, const float* v_norms,

@@ -1453,7 +1453,7 @@ def test_vonly_sparse_decode_threshold_limits(tq):
 
 
 def test_vonly_sparse_decode_rejects_other_shapes(tq):
-    """dim 64 / 4-bit caches have no one-call thresholded step: the wrapper says which ops to compose."""
+    """dim 64 caches have no one-call thresholded step: the wrapper says which ops to compose."""
     rng = np.random.default_rng(403)
     c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, 2, 64, 64, 4)
     q = rng.standard_normal((1, 2, 64)).astype(np.float16)

@@ -2,7 +2,8 @@
 bits 1-4, adaptive.py:26, v_only_cache.py:41): the matrix-core tile pass against the CPU oracle and
 against the float32 kernels, over every launch shape the host picks from (one tile per workgroup of
 four or eight waves, full or ragged; the streaming pass, full or ragged), with masks, ragged batches
-and the three query dtypes.  Tolerance: 2e-3 relative + 1e-3 absolute, elementwise, as for 3 bits.
+and the three query dtypes; the thresholded one-call step and sparse_v_matvec on the matrix cores at
+the same widths.  Tolerance: 2e-3 relative + 1e-3 absolute, elementwise, as for 3 bits.
 """
 import math
 
@@ -198,3 +199,51 @@ def test_vonly_cache_other_widths_decode_through_the_cache(tq, bits):
         for bi in range(B):
             want = o.vonly_decode_attention(q[bi, :, 0].cpu().numpy(), keys[bi], vp[bi], vn[bi], cen, sg, D, bits, sc)
             close(got[bi], want)
+
+
+# ------------------------------------------------------------------ given weights and the thresholded step
+
+@pytest.mark.parametrize("bits", [1, 2, 4])
+@pytest.mark.parametrize("n_seq,n_kv,n_rep,T,thr,qdt", [(1, 4, 7, 1500, 1e-5, np.float16), (2, 2, 4, 513, 1e-3, np.float32),
+                                                        (3, 1, 16, 77, 1e-2, np.float16), (1, 4, 7, 4099, 1e-5, np.float32),
+                                                        (2, 3, 5, 1, 1e-5, np.float16)])
+def test_vonly_thresholded_decode_other_widths_match_oracle(tq, bits, n_seq, n_kv, n_rep, T, thr, qdt):
+    """The one-call thresholded step (scores pass, weights-and-values pass, merge; sparse_v.py:59-65 on the final
+    weights) at the other widths, cache layout with an allocation longer than the valid length."""
+    rng = np.random.default_rng(7 * T + n_rep + bits)
+    sc = 1 / math.sqrt(D)
+    T_alloc = T + 37
+    c, vs, K, vp, vn = fixture(rng, n_seq * n_kv, T_alloc, bits)
+    K, vp, vn = (a.reshape(n_seq, n_kv, *a.shape[1:]) for a in (K, vp, vn))
+    q = rng.standard_normal((n_seq, n_kv * n_rep, D)).astype(qdt)
+    got = host(tq.vonly_decode(dev(q), dev(K), dev(vp), dev(vn), c, dev(vs), D, bits, sc, n_rep=n_rep, seq_len=T,
+                               sparse_v_threshold=thr))
+    dropped = 0
+    for i in range(n_seq):
+        want = o.vonly_decode_attention(q[i], K[i, :, :T], vp[i, :, :T], vn[i, :, :T], c, vs, D, bits, sc, threshold=thr)
+        dense = o.vonly_decode_attention(q[i], K[i, :, :T], vp[i, :, :T], vn[i, :, :T], c, vs, D, bits, sc)
+        dropped += int(np.abs(want - dense).max() > 0)
+        close(got[i], want)
+    if T >= 500:
+        assert dropped > 0                         # the threshold did remove something in these cases
+
+
+@pytest.mark.parametrize("bits", [1, 2, 4])
+def test_sparse_v_matvec_other_widths_on_the_matrix_cores(tq, bits):
+    """sparse_v_matvec(precision="fp16") (sparse_v.py:94-186) at the other widths: dense, thresholded, and the
+    threshold above every weight; against the oracle and the float32 kernel."""
+    rng = np.random.default_rng(350 + bits)
+    n_kv, n_rep, T = 4, 7, 3000
+    c, vs, K, vp, vn = fixture(rng, n_kv, T, bits)
+    x = rng.standard_normal((n_kv * n_rep, T)) * 3
+    w = np.exp(x - x.max(-1, keepdims=True))
+    w = (w / w.sum(-1, keepdims=True)).astype(F32)
+    args = (dev(vp), dev(vn), c, dev(vs), D, bits)
+    for thr in (0.0, 1e-4):
+        want = o.sparse_v_matvec(w, vp, vn, c, vs, D, bits, thr, n_rep)
+        got = host(tq.sparse_v_matvec(dev(w), *args, threshold=thr, n_rep=n_rep, precision="fp16"))
+        close(got, want)
+        ref = host(tq.sparse_v_matvec(dev(w), *args, threshold=thr, n_rep=n_rep, precision="fp32"))
+        assert np.abs(ref - want).max() <= 1e-5 * np.abs(want).max()
+    zero = host(tq.sparse_v_matvec(dev(w), *args, threshold=2.0, n_rep=n_rep, precision="fp16"))
+    assert (zero == 0).all()

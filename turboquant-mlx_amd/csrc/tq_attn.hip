@@ -845,6 +845,18 @@ int launch_vonly_mfma(const void* q, int q_dtype, const void* k_f16, const uint3
   return TQ_OK;
 }
 
+// the width as a run-time value
+void launch_given_tiles_bits(int bits, int mode, dim3 grid, const tqm::PackedArgs& a, const Codebook& kcb,
+                                    const Codebook& vcb, hipStream_t stream) {
+  switch (bits) {
+    case 1: tqm::launch_given_tiles<1>(mode, grid, a, kcb, vcb, stream); break;
+    case 2: tqm::launch_given_tiles<2>(mode, grid, a, kcb, vcb, stream); break;
+    case 4: tqm::launch_given_tiles<4>(mode, grid, a, kcb, vcb, stream); break;
+    default: tqm::launch_given_tiles<3>(mode, grid, a, kcb, vcb, stream); break;
+  }
+}
+
+
 // Steps of 256 positions that one workgroup of the streaming flash pass runs through, or 0 for the
 // single-tile pass.  The streaming pass wants at least two workgroups per CU (512 on this part) so
 // that the set-up of one overlaps the arithmetic of another: the largest step count up to 8 that
@@ -905,7 +917,8 @@ int launch_packed_mfma(const float* q_rot_or_weights, const uint32_t* k_packed, 
     tqm::packed_stream_kernel<<<grid, tqm::kSThreads, 0, stream>>>(a, kcb, vcb, n_steps);
   } else if (n_tiles_real > 0) {
     dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
-    tqm::packed_tile_mfma_kernel<MODE><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, kcb, vcb);
+    if (MODE == tqm::kWeights) launch_given_tiles_bits(sh.bits, MODE, grid, a, kcb, vcb, stream);   // values of any width
+    else tqm::packed_tile_mfma_kernel<MODE><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, kcb, vcb);
   }
   TQ_CHECK_LAUNCH(who);
   dim3 mgrid(n_q, sh.n_seq);
@@ -963,7 +976,7 @@ int launch_soft_weights(const float* scores, const float* stats, int stats_tile_
   Codebook kcb, vcb;
   fill_codebook(kcb, nullptr, sh.bits);
   a.v_unscale = tq::fill_codebook_fp16(vcb, v_centroids, sh.bits);
-  tqm::packed_tile_mfma_kernel<tqm::kSoftWeights><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, kcb, vcb);
+  launch_given_tiles_bits(sh.bits, tqm::kSoftWeights, grid, a, kcb, vcb, stream);
   TQ_CHECK_LAUNCH(who);
 
   dim3 mgrid(n_q, sh.n_seq);
@@ -1203,7 +1216,7 @@ extern "C" int tq_sparse_v_matvec(const float* weights, const uint32_t* v_packed
     return tq::fail(TQ_ERR_NULL, "tq_sparse_v_matvec: null pointer");
   const float thr = threshold > 0.0f ? threshold : 0.0f;
   sh.allow_mma = allow_mma;
-  if (mma_shape(sh))
+  if (vonly_mma_shape(sh))                                   // packed values only: every width
     return launch_packed_mfma<tqm::kWeights>(weights, nullptr, nullptr, v_packed, v_norms, centroids, centroids,
                                              signs, out, workspace, workspace_bytes, sh, thr,
                                              (hipStream_t)stream_, "tq_sparse_v_matvec");
@@ -1400,9 +1413,8 @@ extern "C" int tq_vonly_sparse_decode_attn(const void* q, int q_dtype, const voi
   if (shape->seq_len > 0 && (!k_f16 || !v_packed || !v_norms)) return tq::fail(TQ_ERR_NULL, "%s: null pointer", who);
   if (!tq::aligned(k_f16, 16)) return tq::fail(TQ_ERR_ALIGN, "%s: k must be 16-byte aligned", who);
   if (!(threshold >= 0.0f)) return tq::fail(TQ_ERR_ARG, "%s: threshold must be >= 0", who);
-  if (!(shape->dim == 128 && shape->bits == 3 && shape->n_rep <= tqm::kHeadsMax && shape->seq_len > 0 &&
-        tq::aligned(q, 16)))
-    return tq::fail(TQ_ERR_UNSUPPORTED, "%s: dim 128, 3-bit values, n_rep <= 16 and a non-empty cache only "
+  if (!(shape->dim == 128 && shape->n_rep <= tqm::kHeadsMax && shape->seq_len > 0 && tq::aligned(q, 16)))
+    return tq::fail(TQ_ERR_UNSUPPORTED, "%s: dim 128, n_rep <= 16 and a non-empty cache only "
                                         "(compose tq_dense_qk_scores, tq_softmax_rows and tq_sparse_v_matvec otherwise)", who);
   return launch_vonly_sparse(q, q_dtype, k_f16, v_packed, v_norms, v_centroids, v_signs, threshold, out, workspace,
                              workspace_bytes, *shape, (hipStream_t)stream_);

@@ -55,40 +55,50 @@ struct PackedArgs {
   float threshold;            // kWeights
 };
 
-// copy one wave's 64 packed rows (3328 bytes) from global memory into its LDS area
-struct PackedBlock {
-  u4 q[4];
-  uint32_t d[13];
+// copy one wave's 64 packed rows of PD words each (3328 bytes at three bits) from global memory into its LDS area:
+// wave-wide 16-byte loads where the block is whole and aligned (three and a quarter of them at three bits), else
+// PD 4-byte loads per lane with the index clamped into the tile
+template <int PD>
+struct PackedBlockT {
+  static constexpr int kFull = (16 * PD) / 64;            // whole-wave 16-byte loads
+  static constexpr int kTail = 16 * PD - 64 * kFull;      // pieces of the last, partial one (0 or 16)
+  u4 q[kFull + (kTail ? 1 : 0)];
+  uint32_t d[PD];
   bool wide;
 };
+using PackedBlock = PackedBlockT<kPdim>;
 
-__device__ __forceinline__ void load_block(PackedBlock& b, const uint32_t* block, int lane, int wrow0, int rows_here) {
+template <int PD>
+__device__ __forceinline__ void load_block(PackedBlockT<PD>& b, const uint32_t* block, int lane, int wrow0, int rows_here) {
+  constexpr int kFull = PackedBlockT<PD>::kFull, kTail = PackedBlockT<PD>::kTail;
   b.wide = (wrow0 + kWavePos <= rows_here) && ((reinterpret_cast<uintptr_t>(block) & 15) == 0);
   if (b.wide) {
     const u4* b4 = reinterpret_cast<const u4*>(block);
 #pragma unroll
-    for (int i = 0; i < 3; ++i) b.q[i] = b4[i * 64 + lane];
-    b.q[3] = b4[192 + (lane & 15)];
+    for (int i = 0; i < kFull; ++i) b.q[i] = b4[i * 64 + lane];
+    if (kTail) b.q[kFull] = b4[kFull * 64 + (lane & (kTail - 1))];
   } else {
-    const int valid_words = max(0, rows_here - wrow0) * kPdim;
-    const uint32_t* tile_base = block - (int64_t)wrow0 * kPdim;       // row 0 of the tile: always valid
+    const int valid_words = max(0, rows_here - wrow0) * PD;
+    const uint32_t* tile_base = block - (int64_t)wrow0 * PD;          // row 0 of the tile: always valid
 #pragma unroll
-    for (int i = 0; i < 13; ++i) {
+    for (int i = 0; i < PD; ++i) {
       const int w = i * 64 + lane;
       b.d[i] = (w < valid_words) ? block[w] : tile_base[0];
     }
   }
 }
 
-__device__ __forceinline__ void stage_block(const PackedBlock& b, uint32_t* stage, int lane) {
+template <int PD>
+__device__ __forceinline__ void stage_block(const PackedBlockT<PD>& b, uint32_t* stage, int lane) {
+  constexpr int kFull = PackedBlockT<PD>::kFull, kTail = PackedBlockT<PD>::kTail;
   if (b.wide) {
     u4* st4 = reinterpret_cast<u4*>(stage);
 #pragma unroll
-    for (int i = 0; i < 3; ++i) st4[i * 64 + lane] = b.q[i];
-    if (lane < 16) st4[192 + lane] = b.q[3];
+    for (int i = 0; i < kFull; ++i) st4[i * 64 + lane] = b.q[i];
+    if (kTail) { if (lane < kTail) st4[kFull * 64 + lane] = b.q[kFull]; }
   } else {
 #pragma unroll
-    for (int i = 0; i < 13; ++i) stage[i * 64 + lane] = b.d[i];
+    for (int i = 0; i < PD; ++i) stage[i * 64 + lane] = b.d[i];
   }
 }
 
@@ -152,16 +162,20 @@ __device__ __forceinline__ void rotate_query_rows(const void* q_raw, int q_dtype
   }
 }
 
-// grid = (n_tiles_max, n_kv, n_seq), 512 threads.
-template <int MODE>
+// grid = (n_tiles_max, n_kv, n_seq), 512 threads.  VBITS: width of the packed values; the modes that read packed
+// keys exist for three bits only (keys and values share the width there).
+template <int MODE, int VBITS = 3>
 __global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(4, 4)))
 void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
+  using VF = VField<VBITS>;
+  constexpr int kVPd = VF::kPd;                                      // words per packed value row
   constexpr bool GIVEN = MODE == kWeights || MODE == kSoftWeights;   // weights come from memory, no keys
+  static_assert(GIVEN || VBITS == 3, "packed keys are three-bit here");
   constexpr bool HAS_K = !GIVEN;
   constexpr bool HAS_V = MODE != kScores && MODE != kSoftScores;
   constexpr bool SOFT = MODE == kFlash || MODE == kSoftScores;        // scores carry attn_scale * log2 e and the mask
   __shared__ __align__(16) unsigned char big_s[32768];      // per-wave 4 KB areas, later S_all[8][8][128]
-  __shared__ uint32_t lutk_s[64], lutv_s[64];
+  __shared__ uint32_t lutk_s[64], lutv_s[VF::kLut < 64 ? 64 : VF::kLut];
   __shared__ __align__(16) uint32_t q_s[kHeadsMax][kD / 2];      // rotated queries as half2: rounded value ...
   __shared__ __align__(16) uint32_t ql_s[kHeadsMax][kD / 2];     // ... and what the rounding lost
   __shared__ __align__(16) float kn_s[kWaves][kWavePos], vn_s[kWaves][kWavePos];
@@ -204,11 +218,12 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
     }
   }
   float my_kn = 0.0f, my_vn = 0.0f;
-  PackedBlock kb_, vb_;
+  PackedBlock kb_;
+  PackedBlockT<kVPd> vb_;
   if (HAS_V) {
     my_vn = a.v_norms[(int64_t)seq * a.vn_seq_stride + (int64_t)kvh * a.vn_head_stride + first + tile_p0 + crow];
     load_block(vb_, a.v_packed + ((int64_t)seq * a.v_seq_stride + (int64_t)kvh * a.v_head_stride + first +
-                                  tile_p0 + wrow0) * kPdim, lane, wrow0, rows_here);
+                                  tile_p0 + wrow0) * kVPd, lane, wrow0, rows_here);
   }
   if (HAS_K) {
     my_kn = a.k_norms[(int64_t)seq * a.kn_seq_stride + (int64_t)kvh * a.kn_head_stride + first + tile_p0 + crow];
@@ -289,7 +304,7 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
       }
   }
   if (HAS_K) fill_lut(lutk_s, kcb, tid);
-  if (HAS_V) fill_lut(lutv_s, vcb, tid);
+  if (HAS_V) { if (tid < 64) VF::fill(lutv_s, vcb, tid); }
   if (HAS_K) {
     if (a.q_raw) {
       rotate_query_rows<kWaves>(a.q_raw, a.q_dtype, a.k_signs, q_row0, n_rep, wave, lane, q_s, ql_s);
@@ -338,18 +353,14 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
 
     stage_block(vb_, stage, lane);
     int w0, sh_lo, sh_hi;
-    piece_bits(n16, w0, sh_lo, sh_hi);
-    constexpr uint32_t kEven = 0x1C71C7u;
+    VF::pos(n16, w0, sh_lo, sh_hi);
 #pragma unroll
     for (int kb2 = 0; kb2 < 2; ++kb2)
 #pragma unroll
       for (int qd = 0; qd < 4; ++qd) {
         const int t = 2 * kb2 + (qd >> 1), jp = qd & 1;
-        const uint32_t* ra = stage + (16 * t + 4 * g + 2 * jp) * kPdim + w0;
-        const uint32_t fa = ((ra[0] >> sh_lo) | (ra[1] << sh_hi)) & 0xFFFFFFu;
-        const uint32_t fb = ((ra[kPdim] >> sh_lo) | (ra[kPdim + 1] << sh_hi)) & 0xFFFFFFu;
-        X[kb2][qd] = (fa & kEven) | ((fb & kEven) << 3);
-        Y[kb2][qd] = ((fa >> 3) & kEven) | (fb & (kEven << 3));
+        const uint32_t* ra = stage + (16 * t + 4 * g + 2 * jp) * kVPd + w0;
+        VF::interleave(VF::field(ra, sh_lo, sh_hi), VF::field(ra + kVPd, sh_lo, sh_hi), X[kb2][qd], Y[kb2][qd]);
       }
   }
 
@@ -507,7 +518,7 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
 #pragma unroll
       for (int qd = 0; qd < 4; ++qd) {
         const uint32_t src = (et & 1) ? Y[kb2][qd] : X[kb2][qd];
-        B[qd] = lutv_s[(src >> (6 * (et >> 1))) & 63u];
+        B[qd] = lutv_s[VF::index(src, et >> 1)];
       }
       accS[et] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, A), __builtin_bit_cast(h8, B),
                                                         accS[et], 0, 0, 0);
@@ -521,6 +532,7 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
   merge_waves<kWaves>(mg_s, big_s, 4096, accS, m, l, inv_tscale, a.v_unscale, n_rep, pS, pml);
 }
 
+#ifndef TQ_VONLY_OTHER_WIDTHS_HERE      // a plain (non-template) kernel: defined in one translation unit only
 // Streaming flash-decode pass (packed K and V, no mask): a workgroup of FOUR waves runs through
 // n_steps consecutive 256-position steps of one (sequence, kv head), a wave 64 positions per step,
 // with the online-softmax recurrence in registers, and writes one partial at the end.  Two such
@@ -793,5 +805,21 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
   static_assert(2 * kSImageBytes >= 8 * kD * 4 && (2 * kSImageBytes) % 16 == 0, "a wave's image area holds its eight deposit rows");
   merge_waves<kSWaves>(mg_s, big_s, 2 * kSImageBytes, accS, m_run, l, inv_tscale, a.v_unscale, n_rep, pS, pml);
 }
+
+#endif
+
+// The given-weights tile pass (mode kWeights or kSoftWeights: packed values only) for values of VBITS bits.
+// Instantiated once per width: 3 beside the host code of the entry points, 1, 2 and 4 in a translation unit of their own.
+template <int VBITS>
+void launch_given_tiles(int mode, dim3 grid, const PackedArgs& a, const Codebook& kcb, const Codebook& vcb,
+                        hipStream_t stream) {
+  if (mode == kWeights) packed_tile_mfma_kernel<kWeights, VBITS><<<grid, kMfmaThreads, 0, stream>>>(a, kcb, vcb);
+  else packed_tile_mfma_kernel<kSoftWeights, VBITS><<<grid, kMfmaThreads, 0, stream>>>(a, kcb, vcb);
+}
+#ifndef TQ_VONLY_OTHER_WIDTHS_HERE
+extern template void launch_given_tiles<1>(int, dim3, const PackedArgs&, const Codebook&, const Codebook&, hipStream_t);
+extern template void launch_given_tiles<2>(int, dim3, const PackedArgs&, const Codebook&, const Codebook&, hipStream_t);
+extern template void launch_given_tiles<4>(int, dim3, const PackedArgs&, const Codebook&, const Codebook&, hipStream_t);
+#endif
 
 }  // namespace tqm

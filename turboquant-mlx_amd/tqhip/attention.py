@@ -101,7 +101,7 @@ def vonly_decode_attention(queries: torch.Tensor, cache, attn_scale: float, mask
     queries (B, n_heads, 1, dim) -> (B, n_heads, 1, dim) in queries.dtype.  With no positive
     threshold the step is one fused launch; with one it is one call of three passes (scores, weights
     and values, merge) so that the threshold applies to the final weights (sparse_v.py:60-61); shapes
-    outside the matrix-core kernels (dim != 128, bits != 3) run scores, softmax and sparse-V separately.
+    outside the matrix-core kernels (dim != 128, more than 16 query heads per kv head) run scores, softmax and sparse-V separately.
     """
     B, n_q, S_q, dim = queries.shape
     if S_q != 1:
@@ -113,7 +113,7 @@ def vonly_decode_attention(queries: torch.Tensor, cache, attn_scale: float, mask
     vq = tq._v_q
     bits = tq.quant_bits
     thr = sparse_v_threshold if (sparse_v_threshold is not None and sparse_v_threshold >= 0.0) else 0.0
-    if thr == 0.0 or (ops.vonly_sparse_supported(dim, bits, n_rep) and total > 0):
+    if thr == 0.0 or (ops.vonly_threshold_supported(dim, bits, n_rep) and total > 0):
         m = None
         if mask is not None:
             m = torch.stack([_mask_rows(mask, b, n_q, total).expand(n_q, total) for b in range(B)])

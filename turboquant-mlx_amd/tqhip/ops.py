@@ -672,8 +672,14 @@ def flash_attention_turboquant(q_rot, k_packed, k_norms, v_packed, v_norms, k_ce
 
 
 def vonly_sparse_supported(dim: int, bits: int, n_rep: int) -> bool:
-    """Shapes the thresholded one-call V-only decode step covers (the matrix-core kernels)."""
+    """Shapes the one-call steps over PACKED keys cover (the matrix-core kernels: flash decode from the raw query,
+    its thresholded form, the packed cache's decode_step)."""
     return dim == 128 and bits == 3 and 1 <= n_rep <= 16
+
+
+def vonly_threshold_supported(dim: int, bits: int, n_rep: int) -> bool:
+    """Shapes the thresholded one-call V-only decode step covers: fp16 keys, packed values of any width."""
+    return dim == 128 and 1 <= bits <= 4 and 1 <= n_rep <= 16
 
 
 def vonly_decode(q: torch.Tensor, k: torch.Tensor, v_packed, v_norms, v_centroids, v_signs, dim: int,
@@ -744,8 +750,8 @@ def vonly_decode(q: torch.Tensor, k: torch.Tensor, v_packed, v_norms, v_centroid
             _ptr(out), C.byref(sh), stream))
         return out
     if sparse_v_threshold and sparse_v_threshold > 0.0:
-        if not (vonly_sparse_supported(dim, bits, n_rep) and T > 0):
-            raise ValueError("thresholded V-only decode needs dim 128, 3-bit values, n_rep <= 16 and a non-empty cache; "
+        if not (vonly_threshold_supported(dim, bits, n_rep) and T > 0):
+            raise ValueError("thresholded V-only decode needs dim 128, n_rep <= 16 and a non-empty cache; "
                              "compose dense_qk_scores, softmax_rows and sparse_v_matvec for other shapes")
         need = lib.tq_vonly_sparse_workspace_bytes(n_seq, n_q, T)
         ws = _workspace(q.device, stream.value or 0, need)
