@@ -172,8 +172,8 @@ __device__ __forceinline__ void merge_waves(MergeLds<NW>& mg, unsigned char* are
   if (lane == 0) mg.ts[wave] = inv_tscale;
   float (*mine)[kD] = reinterpret_cast<float (*)[kD]>(areas + wave * area_stride);
   for (int h0 = 0; h0 < n_rep; h0 += 8) {
-    if (h0) __syncthreads();                             // the previous round has been summed
-    if ((g >> 1) == (h0 >> 3)) {                         // lanes whose rows 4g+j fall in this round
+    if (h0) __syncthreads();                             // the previous eight heads have been summed
+    if ((g >> 1) == (h0 >> 3)) {                         // lanes whose rows 4g+j are among these eight heads
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         float4* dst = reinterpret_cast<float4*>(&mine[(4 * g + j) & 7][8 * n16]);
