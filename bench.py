@@ -7,9 +7,10 @@ entry point of libtqhip.so, called through the C ABI.  Inputs are resident in HB
 region; the steps rotate over N_SETS independent (q, K, V) sets totalling > 400 MB so that neither
 the L2s nor the 256 MB Infinity Cache can serve the reads.  The K timed steps are captured once
 into a HIP graph (back-to-back launches, no host gaps) and the graph is replayed until at least
-MIN_TIMED_MS of GPU time has passed, every replay bracketed by HIP events on the launch stream:
-`ms_per_step` is the MEDIAN replay divided by K (a single replay of 20 steps is a 0.3 ms sample),
-the fastest and slowest replay are reported beside it.
+MIN_TIMED_MS of GPU time has passed, with a HIP event on the launch stream after every MIN_SAMPLE_MS
+worth of replays: `ms_per_step` is the MEDIAN sample divided by its steps (a single replay of 20
+steps is a 0.3 ms sample, and an event record per replay would add 0.2 us to each of its steps),
+the fastest and slowest sample are reported beside it.
 
 Prints ONE JSON line (see the fields below).  `roofline.achieved` = algorithmic bytes per step
 (40 908 800 B: q 7 168 + K 33 554 432 + V packed 6 815 744 + V norms 524 288 + out 7 168)
@@ -35,6 +36,7 @@ ALGO_BYTES = N_Q * D * 2 + N_KV * T * D * 2 + N_KV * T * PDIM * 4 + N_KV * T * 4
 HBM_PEAK_GBS = 8000.0
 N_SETS = 10
 MIN_TIMED_MS = 50.0       # GPU time every timed quantity is measured over (at least 5 replays)
+MIN_SAMPLE_MS = 2.0      # GPU time between two event records of the timed region
 READ_WGS = 2048           # workgroups of the plain-read probe (8 per CU)
 
 # HBM bytes per launch of the dominant kernel (the tile pass), from two rocprofv3 --pmc runs of
@@ -177,7 +179,7 @@ def main():
     side = torch.cuda.Stream(device=dev)
 
     def timed(one_step):
-        """(median, min, max, replays): ms per step of `one_step(i, stream)` over replays of a HIP graph of
+        """(median, min, max, replays): ms per step of `one_step(i, stream)` over samples of replays of a HIP graph of
         `args.steps` back-to-back steps (eager launches once with --no-graph), HIP events on the launch stream."""
         with torch.cuda.stream(side):
             for i in range(args.warmup):
@@ -205,16 +207,20 @@ def main():
             ev[1].record(side)
             side.synchronize()
             est = max(ev[0].elapsed_time(ev[1]), 1e-3)
-            n_rep = int(min(max(5, math.ceil(MIN_TIMED_MS / est)), 4000))
+            # a sample = `per_sample` replays between two event records (at least MIN_SAMPLE_MS of GPU time, so that
+            # the records themselves, a few microseconds each, do not show in a short graph's figure)
+            per_sample = int(max(1, math.ceil(MIN_SAMPLE_MS / est)))
+            n_rep = int(min(max(5, math.ceil(MIN_TIMED_MS / (est * per_sample))), 4000))
             ev = [torch.cuda.Event(enable_timing=True) for _ in range(n_rep + 1)]
             ev[0].record(side)
             for r in range(n_rep):
-                graph.replay()
+                for _ in range(per_sample):
+                    graph.replay()
                 ev[r + 1].record(side)
             side.synchronize()
         torch.cuda.synchronize()
-        per = sorted(ev[r].elapsed_time(ev[r + 1]) / args.steps for r in range(n_rep))
-        return per[n_rep // 2], per[0], per[-1], n_rep
+        per = sorted(ev[r].elapsed_time(ev[r + 1]) / (args.steps * per_sample) for r in range(n_rep))
+        return per[n_rep // 2], per[0], per[-1], n_rep * per_sample
 
     arg_cache = {}
 
@@ -297,7 +303,8 @@ def main():
                              "`value` covers the whole step (tile pass + merge pass)"},
         "cpu_baseline": cpu,
         "read_ceiling": ceiling,
-        "timing": {"method": "median over HIP-graph replays of `steps` steps each, >= %d ms of GPU time" % int(MIN_TIMED_MS)
+        "timing": {"method": "median over samples of back-to-back HIP-graph replays of `steps` steps each (>= %g ms of GPU "
+                             "time per sample, >= %d ms in all)" % (MIN_SAMPLE_MS, int(MIN_TIMED_MS))
                    if not args.no_graph else "one pass of eager launches",
                    "replays": n_replays, "us_per_layer_min": round(ms_min * 1e3, 3), "us_per_layer_max": round(ms_max * 1e3, 3),
                    "tile_us_min": round(tile_min * 1e3, 3), "tile_us_max": round(tile_max * 1e3, 3)},
