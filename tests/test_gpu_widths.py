@@ -3,7 +3,8 @@ bits 1-4, adaptive.py:26, v_only_cache.py:41): the matrix-core tile pass against
 against the float32 kernels, over every launch shape the host picks from (one tile per workgroup of
 four or eight waves, full or ragged; the streaming pass, full or ragged), with masks, ragged batches
 and the three query dtypes; the thresholded one-call step and sparse_v_matvec on the matrix cores at
-the same widths.  Tolerance: 2e-3 relative + 1e-3 absolute, elementwise, as for 3 bits.
+the same widths.  Tolerance: 2e-3 relative + 1e-3 absolute, elementwise, as for 3 bits.  Last, the streaming
+encoder and dequantiser at these widths: bit-exact against the oracle and the generic kernels.
 """
 import math
 
@@ -247,3 +248,115 @@ def test_sparse_v_matvec_other_widths_on_the_matrix_cores(tq, bits):
         assert np.abs(ref - want).max() <= 1e-5 * np.abs(want).max()
     zero = host(tq.sparse_v_matvec(dev(w), *args, threshold=2.0, n_rep=n_rep, precision="fp16"))
     assert (zero == 0).all()
+
+
+# ------------------------------------------------------------------ streaming encoder / dequantiser at d = 128
+
+def _special_rows(rng, n, b):
+    """n x 128 float32 rows: random scales, a zero row, one-hot rows, and 200 rows whose butterfly outputs sit
+    within a few ulp of a decision boundary of the given width."""
+    x = (rng.standard_normal((n, 128)) * rng.choice([1e-3, 1.0, 300.0], size=(n, 1))).astype(F32)
+    x[5] = 0.0
+    x[6] = 0.0
+    x[6, 127] = -2.5
+    x[7] = 0.0
+    x[7, 64] = 1e-3
+    H = np.array([[1.0 if bin(j & k).count("1") % 2 == 0 else -1.0 for k in range(128)] for j in range(128)])
+    for r in range(32, 232):
+        z = rng.standard_normal(128)
+        z[rng.integers(0, 128)] = float(b[rng.integers(0, len(b))]) * (1 + rng.integers(-3, 4) * 2.0 ** -23) \
+            + (rng.integers(-3, 4) * 2.0 ** -24 if len(b) == 1 else 0.0)          # the one-bit boundary is 0
+        z *= math.sqrt(128) / np.linalg.norm(z)
+        x[r] = (H @ z) / 128.0
+    return x
+
+
+@pytest.mark.parametrize("variant", ["mlx", "metal"])
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("bits", [1, 2, 4])
+def test_streaming_encoder_other_widths_bit_exact(tq, bits, dtype, variant):
+    """A row count that is a multiple of 16 takes the streaming encoder at every width (metal.py:14-101 /
+    quantizer.py:85-106 for bits 1-4): level = thresholds below a guess cell + one compare, the cell table derived
+    from the thresholds on the GPU.  Its words and norms must be the oracle's and those of the generic
+    one-wavefront-per-vector kernel (ragged count), special rows included."""
+    rng = np.random.default_rng(40 + bits)
+    c = o.gaussian_codebook(bits)
+    b = o.gaussian_boundaries(c)
+    s = o.random_diagonal_sign(128, 43)
+    n = 16 * 261
+    x = _special_rows(rng, n, b)
+    xt = torch.from_numpy(x)
+    if dtype == "f16":
+        xt = xt.to(torch.float16)
+    elif dtype == "bf16":
+        xt = xt.to(torch.bfloat16)
+    xt[100] = float("nan")
+    xt[101, 3] = float("nan")
+    if dtype == "f32":
+        xt[102] = 3e19                                          # sum of squares overflows float32: the norm is inf
+    ref_in = xt.float().numpy()
+    ok = ~np.isnan(ref_in).any(axis=1)
+    with np.errstate(over="ignore"):
+        wp, wn = o.fused_quantize(ref_in[ok], s, b, 128, bits, variant)
+    gp, gn = tq.fused_quantize(xt.cuda(), dev(s), b, 128, bits, variant=variant)
+    gp, gn = gp.cpu().numpy(), gn.cpu().numpy()
+    assert gp.shape == (n, o.packed_dim(128, bits))
+    assert np.array_equal(gp[ok], wp) and np.array_equal(gn[ok], wn)
+    assert (gp[~ok] == 0).all() and np.isnan(gn[~ok]).all()          # NaN compares false with every threshold
+    gp2, gn2 = tq.fused_quantize(xt[: n - 3].cuda(), dev(s), b, 128, bits, variant=variant)
+    assert np.array_equal(gp2.cpu().numpy(), gp[: n - 3])
+    assert np.array_equal(gn2.cpu().numpy()[ok[: n - 3]], gn[: n - 3][ok[: n - 3]])
+
+
+@pytest.mark.parametrize("bits", [1, 2, 4])
+def test_streaming_encoder_other_widths_every_level_and_custom_tables(tq, bits):
+    """Every level of the width is produced on a sweep of one coordinate through the whole range, and a codebook
+    whose thresholds admit no guess line (two of them 1e-3 apart) still encodes exactly (generic kernel)."""
+    c = o.gaussian_codebook(bits)
+    b = o.gaussian_boundaries(c)
+    ones = np.ones(128, F32)
+    n = 4096
+    H = np.array([[1.0 if bin(j & k).count("1") % 2 == 0 else -1.0 for k in range(128)] for j in range(128)])
+    rng = np.random.default_rng(60 + bits)
+    z = rng.standard_normal((n, 128)) * 0.05
+    z[:, 9] = np.linspace(-3.2, 3.2, n)
+    x = ((z @ H) / 128.0).astype(F32)
+    wp, wn = o.fused_quantize(x, ones, b, 128, bits, "metal")
+    gp, gn = tq.fused_quantize(dev(x), dev(ones), b, 128, bits, variant="metal")
+    assert np.array_equal(gp.cpu().numpy(), wp) and np.array_equal(gn.cpu().numpy(), wn)
+    idx = o.unpack_indices(wp, bits, 128)
+    assert set(np.unique(idx[:, 9]).tolist()) == set(range(2 ** bits))
+    if bits > 1:
+        b2 = np.array(b, dtype=F32).copy()
+        b2[1] = b2[0] + 1e-3
+        b2 = np.sort(b2)
+        wp, wn = o.fused_quantize(x, ones, b2, 128, bits, "metal")
+        gp, gn = tq.fused_quantize(dev(x), dev(ones), b2, 128, bits, variant="metal")
+        assert np.array_equal(gp.cpu().numpy(), wp) and np.array_equal(gn.cpu().numpy(), wn)
+
+
+@pytest.mark.parametrize("out", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("bits", [1, 2, 4])
+def test_streaming_dequantiser_other_widths_bit_exact(tq, bits, out):
+    """packed_dequantize / dequant_fp16 (kernels.py:14-55, metal.py:104-141) at a row count that takes the streaming
+    kernel: float32 output equal to the oracle's, 16-bit outputs equal to its rounding, and equal to the generic
+    kernel (ragged count)."""
+    rng = np.random.default_rng(70 + bits)
+    c = o.gaussian_codebook(bits)
+    s = o.random_diagonal_sign(128, 43)
+    n = 16 * 130
+    idx = rng.integers(0, 2 ** bits, size=(n, 128)).astype(np.uint8)
+    wp = o.pack_indices(idx, bits)
+    wn = (rng.random(n) * 10 + 0.01).astype(F32)
+    want = o.packed_dequantize(wp, wn, c, s, 128, bits)
+    if out == "f32":
+        got = tq.packed_dequantize(dev(wp), dev(wn), c, dev(s), 128, bits)
+        assert np.array_equal(got.cpu().numpy(), want)
+        rag = tq.packed_dequantize(dev(wp[: n - 5]), dev(wn[: n - 5]), c, dev(s), 128, bits)
+        assert np.array_equal(rag.cpu().numpy(), want[: n - 5])
+    else:
+        td = torch.float16 if out == "f16" else torch.bfloat16
+        outbuf = torch.empty((n, 128), dtype=td, device="cuda")
+        tq.dequant_into(dev(wp), dev(wn), c, dev(s), outbuf, n_groups=1, rows_per_group=n, packed_group_stride=n,
+                        norms_group_stride=n, out_group_stride=n, dim=128, bits=bits)
+        assert torch.equal(outbuf.cpu(), torch.from_numpy(want).to(td))

@@ -136,8 +136,9 @@ __global__ __launch_bounds__(kBlock) void encode_kernel(const T* __restrict__ x,
   }
 }
 
-// ---------------------------------------------------------------- encode, d = 128, 3-bit
-// The streaming encoder for the cache's own shape.  Four lanes own one vector, so a wavefront
+// ---------------------------------------------------------------- encode, d = 128
+// The streaming encoder for the cache's own head dimension (every width; the notes below describe three bits,
+// the width-dependent parts are the level table and the word assembly at the end of a pass).  Four lanes own one vector, so a wavefront
 // encodes 16 vectors per pass: lane ls = lane % 4 of a vector holds the four 8-element chunks
 // c = ls + 4k (k = 0..3), element e = 32k + 8ls + j.  Each load instruction therefore reads 64
 // contiguous bytes per vector; butterfly stages 1, 2, 4, 32 and 64 and five of the seven levels of
@@ -180,19 +181,54 @@ __device__ __forceinline__ float mix_fma_addend(float a, float b, uint32_t h2) {
   return d;
 }
 
+// The 8 * BITS bits that hold elements 8c .. 8c+7 (chunk c) of a packed d = 128 row: word and shifts.  Three-bit
+// rows hold ten fields per word, so a chunk may straddle two words (chunk 15 is all of word 12: taken as word
+// 11 >> 30, which is 0, | word 12); the other widths divide the word.
+template <int BITS>
+struct Chunk {
+  static constexpr int kPd = BITS == 3 ? 13 : 4 * BITS;       // words per row
+  static constexpr uint32_t kPairMask = (1u << (2 * BITS)) - 1u;
+  __device__ static __forceinline__ void pos(int c, int& w0, int& sh_lo, int& sh_hi) {
+    if (BITS == 3) {
+      w0 = (c == 15) ? 11 : (8 * c) / 10;
+      const int s0 = (c == 15) ? 10 : (8 * c) % 10;
+      sh_lo = 3 * s0;
+      sh_hi = 30 - 3 * s0;
+    } else {
+      constexpr int kPerWord = 4 / BITS;
+      w0 = c / kPerWord;
+      sh_lo = (c % kPerWord) * 8 * BITS;
+      sh_hi = 0;
+    }
+  }
+  __device__ static __forceinline__ uint32_t field(const uint32_t* at_w0, int sh_lo, int sh_hi) {
+    if (BITS == 3) return ((at_w0[0] >> sh_lo) | (at_w0[1] << sh_hi)) & 0xFFFFFFu;
+    if (BITS == 4) return at_w0[0];
+    return (at_w0[0] >> sh_lo) & ((1u << (8 * BITS)) - 1u);
+  }
+};
+
 constexpr int kEncVecs = 16;      // vectors per wavefront pass
 constexpr int kEncPasses = 4;     // passes per wavefront once there are rows enough to fill the chip
 
-struct EncodeGuess { float alpha, beta; };
+// alpha and beta of the level guess; beta0 = beta without the 2^20 + 32 that places the guess in the mantissa
+struct EncodeGuess { float alpha, beta, beta0; };
 
-template <typename T>
+// BITS = 3: every threshold j sits in cell j of the guess (level_guess_search), and the table is written down
+// directly.  Other widths: any guess line under which no cell holds two thresholds (level_cells_search); cell
+// c = floor(alpha * w + beta0) then knows the count g of thresholds below its lower edge and the one threshold it
+// may hold (else +inf: nothing to compare with), both derived here from the thresholds themselves.
+template <typename T, int BITS = 3>
 __global__ __launch_bounds__(kBlock) void encode128x3_kernel(const T* __restrict__ x,
                                                              const float* __restrict__ signs, Thresholds thr,
                                                              EncodeGuess gs, uint32_t* __restrict__ packed,
                                                              float* __restrict__ norms, RowMap rm, int passes) {
   constexpr bool kHalfWidth = sizeof(T) == 2;
   constexpr int NM = kHalfWidth ? 4 : 8;                       // sign masks per chunk
-  __shared__ __align__(8) uint2 lvl_s[64];                     // (threshold bits, guess) by 32 + floor(alpha*w + beta)
+  constexpr int NB = (1 << BITS) - 1;                          // thresholds
+  constexpr int kPd = Chunk<BITS>::kPd;
+  constexpr int kCells = BITS == 4 ? 128 : 64;                 // cells of the level guess (fifteen thresholds need finer ones)
+  __shared__ __align__(8) uint2 lvl_s[kCells];                 // (threshold bits, guess) by kCells / 2 + floor(alpha*w + beta0)
   __shared__ __align__(16) float sg_s[128];
   __shared__ uint32_t chunk_s[kWavesPerBlock][kEncVecs * 16 + 4];
 
@@ -200,12 +236,23 @@ __global__ __launch_bounds__(kBlock) void encode128x3_kernel(const T* __restrict
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ls = lane & 3, v = lane >> 2;
-  if (tid < 64) {
-    const int gq = tid - 32;
-    float t = gq < 0 ? INFINITY : -INFINITY;
+  if (tid < kCells) {
+    const int gq = tid - kCells / 2;
+    if (BITS == 3) {
+      float t = gq < 0 ? INFINITY : -INFINITY;
 #pragma unroll
-    for (int i = 0; i < 7; ++i) t = (gq == i) ? thr.t[i] : t;
-    lvl_s[tid] = make_uint2(__float_as_uint(t), (uint32_t)(gq < 0 ? 0 : (gq > 6 ? 6 : gq)));
+      for (int i = 0; i < 7; ++i) t = (gq == i) ? thr.t[i] : t;
+      lvl_s[tid] = make_uint2(__float_as_uint(t), (uint32_t)(gq < 0 ? 0 : (gq > 6 ? 6 : gq)));
+    } else {
+      int g = 0;                                               // thresholds below the cell's lower edge
+#pragma unroll
+      for (int i = 0; i < NB; ++i) g += (__fmaf_rn(thr.t[i], gs.alpha, gs.beta0) < (float)gq) ? 1 : 0;
+      float t = INFINITY;                                      // threshold number g, if it lies inside the cell
+#pragma unroll
+      for (int i = 0; i < NB; ++i)
+        t = (i == g && __fmaf_rn(thr.t[i], gs.alpha, gs.beta0) < (float)(gq + 1)) ? thr.t[i] : t;
+      lvl_s[tid] = make_uint2(__float_as_uint(t), (uint32_t)g);
+    }
   }
   if (tid < 128) sg_s[tid] = signs[tid];
   __syncthreads();
@@ -322,30 +369,41 @@ __global__ __launch_bounds__(kBlock) void encode128x3_kernel(const T* __restrict
         }
       }
     butterfly_4lane(xs, flip1, flip2);
-    // ---- levels, 24 bits per chunk
+    // ---- levels, 8 * BITS bits per chunk
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       uint32_t bits24 = 0;
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const float w = xs[k][j];
-        const uint32_t off = __float_as_uint(__fmaf_rn(w, gs.alpha, gs.beta)) & 0x1F8u;
+        const uint32_t off = __float_as_uint(__fmaf_rn(w, gs.alpha, gs.beta)) & (uint32_t)((kCells - 1) << 3);
         const uint2 lv = *reinterpret_cast<const uint2*>(reinterpret_cast<const unsigned char*>(lvl_s) + off);
         const uint32_t idx = lv.y + ((w > __uint_as_float(lv.x)) ? 1u : 0u);
-        bits24 |= idx << (3 * j);
+        bits24 |= idx << (BITS * j);
       }
       chunks[v * 16 + ls + 4 * k] = (nrm != nrm) ? 0u : bits24;
     }
-    // ---- words: word wd of a row holds elements 10wd .. 10wd+9 = chunks (5wd)/4 and the next
-    uint32_t* prow = packed + ((int64_t)grp * rm.packed_group_stride + rin) * 13;
+    // ---- words.  Three bits: word wd of a row holds elements 10wd .. 10wd+9 = chunks (5wd)/4 and the next;
+    // four bits: a chunk is a word; two bits / one bit: two / four chunks make a word
+    uint32_t* prow = packed + ((int64_t)grp * rm.packed_group_stride + rin) * kPd;
 #pragma unroll
-    for (int it = 0; it < 4; ++it) {
+    for (int it = 0; it < (kEncVecs * kPd + 63) / 64; ++it) {
       const int id = it * 64 + lane;
-      if (id < kEncVecs * 13) {
-        const int vv = id / 13, wd = id - 13 * vv;
-        const int a = (5 * wd) >> 2, sh = 3 * ((10 * wd) & 7);
-        const uint32_t lo = chunks[vv * 16 + a], hi = chunks[vv * 16 + a + 1];
-        const uint32_t word = ((lo >> sh) | (hi << (24 - sh))) & (wd == 12 ? 0xFFFFFFu : 0x3FFFFFFFu);
+      if (id < kEncVecs * kPd) {
+        const int vv = id / kPd, wd = id - kPd * vv;
+        uint32_t word;
+        if (BITS == 3) {
+          const int a = (5 * wd) >> 2, sh = 3 * ((10 * wd) & 7);
+          const uint32_t lo = chunks[vv * 16 + a], hi = chunks[vv * 16 + a + 1];
+          word = ((lo >> sh) | (hi << (24 - sh))) & (wd == 12 ? 0xFFFFFFu : 0x3FFFFFFFu);
+        } else if (BITS == 4) {
+          word = chunks[vv * 16 + wd];
+        } else if (BITS == 2) {
+          word = chunks[vv * 16 + 2 * wd] | (chunks[vv * 16 + 2 * wd + 1] << 16);
+        } else {
+          word = chunks[vv * 16 + 4 * wd] | (chunks[vv * 16 + 4 * wd + 1] << 8) | (chunks[vv * 16 + 4 * wd + 2] << 16) |
+                 (chunks[vv * 16 + 4 * wd + 3] << 24);
+        }
         prow[id] = word;
       }
     }
@@ -411,19 +469,23 @@ __global__ __launch_bounds__(kBlock) void dequant_kernel(const uint32_t* __restr
   }
 }
 
-// ---------------------------------------------------------------- dequant, d = 128, 3-bit
-// Same four-lanes-per-vector layout as encode128x3_kernel.  The 208 packed words of a pass are
-// read with coalesced loads into LDS; a lane cuts the 24 bits of each of its chunks out of two
-// words and looks centroid pairs up in a 64-entry table of (c[a]*s, c[b]*s).  Arithmetic per
+// ---------------------------------------------------------------- dequant, d = 128
+// Same four-lanes-per-vector layout as encode128x3_kernel, every width.  The packed words of a pass (208 at
+// three bits) are read with coalesced loads into LDS; a lane cuts the 8 * BITS bits of each of its chunks out
+// of one or two words and looks centroid pairs up in a table of 4^BITS entries (c[a]*s, c[b]*s).  Arithmetic per
 // element, in this order, as in dequant_kernel: butterfly, * s, * sign, * norm, round to TO.
-template <typename TO>
+template <typename TO, int BITS = 3>
 __global__ __launch_bounds__(kBlock) void dequant128x3_kernel(const uint32_t* __restrict__ packed,
                                                               const float* __restrict__ norms, Codebook cbk,
                                                               const float* __restrict__ signs, float s,
                                                               TO* __restrict__ out, RowMap rm, int passes) {
+  using CK = Chunk<BITS>;
+  constexpr int kPd = CK::kPd;
+  constexpr int kPairs = 1 << (2 * BITS);                      // entries of the centroid-pair table
+  constexpr int kWordLoads = (kEncVecs * kPd + 63) / 64;       // wave-wide loads of a pass's packed words
   __shared__ __align__(16) float sg_s[128];
-  __shared__ __align__(8) float2 pair_s[64];
-  __shared__ uint32_t words_s[kWavesPerBlock][kEncVecs * 13 + 3];
+  __shared__ __align__(8) float2 pair_s[kPairs < 64 ? 64 : kPairs];
+  __shared__ uint32_t words_s[kWavesPerBlock][kEncVecs * kPd + 3];
   // Outputs leave through LDS: 16 rows of 256 (16-bit) or 512 (float32) bytes at a padded pitch (conflict-free
   // 16-byte writes per lane and reads per row segment), so that every store instruction writes 1 KB of
   // contiguous memory
@@ -434,12 +496,12 @@ __global__ __launch_bounds__(kBlock) void dequant128x3_kernel(const uint32_t* __
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ls = lane & 3, v = lane >> 2;
-  if (tid < 64) {
+  if (tid < kPairs) {                                          // kBlock = 256 threads cover the largest table
     float clo = 0.0f, chi = 0.0f;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      clo = ((tid & 7) == i) ? cbk.c[i] : clo;
-      chi = ((tid >> 3) == i) ? cbk.c[i] : chi;
+    for (int i = 0; i < (1 << BITS); ++i) {
+      clo = ((tid & ((1 << BITS) - 1)) == i) ? cbk.c[i] : clo;
+      chi = ((tid >> BITS) == i) ? cbk.c[i] : chi;
     }
     pair_s[tid] = make_float2(clo * s, chi * s);
   }
@@ -458,17 +520,10 @@ __global__ __launch_bounds__(kBlock) void dequant128x3_kernel(const uint32_t* __
   const uint32_t flip1 = (ls & 1) ? 0x80000000u : 0u;
   const uint32_t flip2 = (ls & 2) ? 0x80000000u : 0u;
   uint32_t* words = words_s[wave];
-  // words / shifts of the 24 bits of chunk c = ls + 4k: elements 8c .. 8c+7 start in word 8c/10
-  // (chunk 15, the last 8 elements, is all of word 12: taken as word 11 >> 30, which is 0, | word 12)
+  // words / shifts of the bits of chunk c = ls + 4k (elements 8c .. 8c+7)
   int cw[4], csl[4], csh[4];
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    const int c = ls + 4 * k;
-    cw[k] = (c == 15) ? 11 : (8 * c) / 10;
-    const int s0 = (c == 15) ? 10 : (8 * c) % 10;
-    csl[k] = 3 * s0;
-    csh[k] = 30 - 3 * s0;
-  }
+  for (int k = 0; k < 4; ++k) CK::pos(ls + 4 * k, cw[k], csl[k], csh[k]);
 
   const uint32_t batch0 = ((uint32_t)blockIdx.x * kWavesPerBlock + wave) * (uint32_t)passes;
   uint32_t row0 = batch0 * kEncVecs;
@@ -476,15 +531,15 @@ __global__ __launch_bounds__(kBlock) void dequant128x3_kernel(const uint32_t* __
   uint32_t rin = row0 - grp * (uint32_t)rm.rows_per_group;
 
   // the packed words and the norm of the next pass are fetched while the current one is computed
-  uint32_t pw[4];
+  uint32_t pw[kWordLoads];
   float pn = 0.0f;
   auto fetch = [&](uint32_t g_, uint32_t r_) {
-    const uint32_t* prow = packed + ((int64_t)g_ * rm.packed_group_stride + r_) * 13;
+    const uint32_t* prow = packed + ((int64_t)g_ * rm.packed_group_stride + r_) * kPd;
     pn = norms[(int64_t)g_ * rm.norms_group_stride + r_ + v];
 #pragma unroll
-    for (int it = 0; it < 4; ++it) {
+    for (int it = 0; it < kWordLoads; ++it) {
       const int id = it * 64 + lane;
-      pw[it] = (id < kEncVecs * 13) ? prow[id] : 0u;
+      pw[it] = (id < kEncVecs * kPd) ? prow[id] : 0u;
     }
   };
   if (row0 < (uint32_t)rm.n_rows) fetch(grp, rin);
@@ -492,9 +547,9 @@ __global__ __launch_bounds__(kBlock) void dequant128x3_kernel(const uint32_t* __
     if (row0 >= (uint32_t)rm.n_rows) break;                    // uniform over the wavefront
     const float nrm = pn;
 #pragma unroll
-    for (int it = 0; it < 4; ++it) {
+    for (int it = 0; it < kWordLoads; ++it) {
       const int id = it * 64 + lane;
-      if (id < kEncVecs * 13) words[id] = pw[it];
+      if (id < kEncVecs * kPd) words[id] = pw[it];
     }
     uint32_t nrin = rin + kEncVecs, ngrp = grp;
     if (nrin >= (uint32_t)rm.rows_per_group) { nrin = 0; ++ngrp; }
@@ -502,11 +557,10 @@ __global__ __launch_bounds__(kBlock) void dequant128x3_kernel(const uint32_t* __
     float xs[4][8];
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-      const uint32_t* rw = words + v * 13 + cw[k];
-      const uint32_t f = ((rw[0] >> csl[k]) | (rw[1] << csh[k])) & 0xFFFFFFu;
+      const uint32_t f = CK::field(words + v * kPd + cw[k], csl[k], csh[k]);
 #pragma unroll
       for (int jp = 0; jp < 4; ++jp) {
-        const float2 c2 = pair_s[(f >> (6 * jp)) & 63u];
+        const float2 c2 = pair_s[(f >> (2 * BITS * jp)) & CK::kPairMask];
         xs[k][2 * jp] = c2.x;
         xs[k][2 * jp + 1] = c2.y;
       }
@@ -664,9 +718,47 @@ float double_rounding_threshold(float b, float s) {
 // further margin of 0.01), beta a multiple of 1/8.  The kernel evaluates v = fma(w, alpha, beta + 2^20 + 32)
 // in float: one rounding, to a multiple of 1/8, i.e. at most 1/16 away from alpha*w + beta, so
 // floor(v) - 2^20 - 32 is the count of thresholds below w or one less for every w.  |w| <= sqrt(128)
-// (raw butterfly of a unit vector), so the guess must stay within +-32 of zero for the 64-entry table.
+// (raw butterfly of a unit vector), so the guess must stay within +-32 of zero for the 64-entry table (three bits).
 // False when no such line exists (then the generic kernel counts the thresholds one by one).
 bool level_guess_search(const float* t, int nb, EncodeGuess& out);
+
+// Widths other than three bits: any line u = alpha * t + beta0 (beta0 a multiple of 1/8) under which no cell
+// [c, c + 1) of u holds two thresholds and every threshold keeps the margin above from both edges of its cell.
+// The kernel's cell of w is floor(alpha * w + beta0) or, for w within 1/16 below a cell edge, the next one; with no
+// threshold that close below an edge the count "thresholds below the cell + (w > the threshold inside it)" is the
+// count of thresholds below w either way.  The candidate with the widest margin is taken.
+bool level_cells_search(const float* t, int nb, EncodeGuess& out) {
+  for (int i = 0; i < nb; ++i)
+    if (!std::isfinite(t[i]) || (i > 0 && !(t[i] > t[i - 1]))) return false;
+  const int half = nb == 15 ? 64 : 32;                              // the kernel's table has 2 * half cells
+  const double margin = 1.0 / 16.0 + 0.01;
+  double best = -1.0, best_b = 0.0;
+  float best_a = 0.0f;
+  for (int ai = 4000; ai >= 100; --ai) {
+    const float af = (float)(ai * ((half - 1) / 11.4 / 4000.0));    // up to (half - 1) / 11.4 cells per unit of w
+    const double a = (double)af;
+    for (int bi = -64; bi <= 64; ++bi) {
+      const double b = bi / 8.0;
+      if (!(a * 11.4 + std::fabs(b) < half - 1.0)) continue;
+      double slack = 1e9, prev_cell = -1e9;
+      bool ok = true;
+      for (int j = 0; j < nb && ok; ++j) {
+        const double u = a * (double)t[j] + b;
+        const double c = std::floor(u), f = u - c;
+        if (f < margin || f > 1.0 - margin || c <= prev_cell) ok = false;
+        prev_cell = c;
+        slack = std::fmin(slack, std::fmin(f - margin, 1.0 - margin - f));
+      }
+      if (ok && slack > best) { best = slack; best_a = af; best_b = b; }
+    }
+    if (best > 0.15) break;                                         // good enough: finer cells gain nothing
+  }
+  if (best < 0.0) return false;
+  out.alpha = best_a;
+  out.beta0 = (float)best_b;
+  out.beta = (float)(best_b + 1048576.0 + (double)half);            // exact: a multiple of 1/8 below 2^21
+  return true;
+}
 
 // The search result is kept for the last threshold set seen.
 bool level_guess(const float* t, int nb, EncodeGuess& out) {
@@ -677,7 +769,7 @@ bool level_guess(const float* t, int nb, EncodeGuess& out) {
   static EncodeGuess last_out;
   std::lock_guard<std::mutex> lock(mu);
   if (last_nb != nb || memcmp(last_t, t, nb * sizeof(float)) != 0) {
-    last_ok = level_guess_search(t, nb, last_out);
+    last_ok = (nb == 7) ? level_guess_search(t, nb, last_out) : level_cells_search(t, nb, last_out);
     memcpy(last_t, t, nb * sizeof(float));
     last_nb = nb;
   }
@@ -713,6 +805,7 @@ bool level_guess_search(const float* t, int nb, EncodeGuess& out) {
   if (!(b - lo >= margin && hi - b >= margin)) return false;
   if (!(a * 11.4 + std::fabs(b) < 31.0)) return false;
   out.beta = (float)(b + 1048576.0 + 32.0);                  // exact: a multiple of 1/8 below 2^21
+  out.beta0 = (float)b;
   return true;
 }
 
@@ -867,18 +960,18 @@ extern "C" int tq_encode(const void* x, int x_dtype, const float* signs, const f
   hipStream_t stream = (hipStream_t)stream_;
   const int grid = grid_for_rows(n_rows);
   EncodeGuess gs{};
-  if (dim == 128 && bits == 3 && rows_per_group % kEncVecs == 0 && n_rows < (int64_t)1 << 31 &&
+  if (dim == 128 && rows_per_group % kEncVecs == 0 && n_rows < (int64_t)1 << 31 &&
       tq::aligned(x, 16) && level_guess(thr.t, nb, gs)) {
     const int passes = fast_passes(n_rows);
     const int64_t rows_per_block = (int64_t)kEncVecs * passes * kWavesPerBlock;
     const int fgrid = (int)((n_rows + rows_per_block - 1) / rows_per_block);
-    if (x_dtype == TQ_F32)
-      encode128x3_kernel<float><<<fgrid, kBlock, 0, stream>>>((const float*)x, signs, thr, gs, packed, norms, rm, passes);
-    else if (x_dtype == TQ_F16)
-      encode128x3_kernel<__half><<<fgrid, kBlock, 0, stream>>>((const __half*)x, signs, thr, gs, packed, norms, rm, passes);
-    else
-      encode128x3_kernel<__hip_bfloat16><<<fgrid, kBlock, 0, stream>>>((const __hip_bfloat16*)x, signs, thr, gs,
-                                                                      packed, norms, rm, passes);
+#define LAUNCH_ENC128(T)                                                                                          \
+    TQ_DISPATCH_BITS(bits, (encode128x3_kernel<T, B_><<<fgrid, kBlock, 0, stream>>>((const T*)x, signs, thr, gs, packed, \
+                                                                                   norms, rm, passes)))
+    if (x_dtype == TQ_F32) { LAUNCH_ENC128(float); }
+    else if (x_dtype == TQ_F16) { LAUNCH_ENC128(__half); }
+    else { LAUNCH_ENC128(__hip_bfloat16); }
+#undef LAUNCH_ENC128
     TQ_CHECK_LAUNCH("tq_encode launch");
     return TQ_OK;
   }
@@ -981,18 +1074,18 @@ extern "C" int tq_dequant(const uint32_t* packed, const float* norms, const floa
   RowMap rm{n_rows, rows_per_group, packed_group_stride, norms_group_stride, out_group_stride};
   hipStream_t stream = (hipStream_t)stream_;
   const int grid = grid_for_rows(n_rows);
-  if (dim == 128 && bits == 3 && rows_per_group % kEncVecs == 0 && n_rows < (int64_t)1 << 31 &&
+  if (dim == 128 && rows_per_group % kEncVecs == 0 && n_rows < (int64_t)1 << 31 &&
       tq::aligned(out, 16) && (out_group_stride * 128 * (int64_t)tq::dtype_size(out_dtype)) % 16 == 0) {
     const int passes = fast_passes(n_rows);
     const int64_t rows_per_block = (int64_t)kEncVecs * passes * kWavesPerBlock;
     const int fgrid = (int)((n_rows + rows_per_block - 1) / rows_per_block);
-    if (out_dtype == TQ_F32)
-      dequant128x3_kernel<float><<<fgrid, kBlock, 0, stream>>>(packed, norms, cb, signs, s, (float*)out, rm, passes);
-    else if (out_dtype == TQ_F16)
-      dequant128x3_kernel<__half><<<fgrid, kBlock, 0, stream>>>(packed, norms, cb, signs, s, (__half*)out, rm, passes);
-    else
-      dequant128x3_kernel<__hip_bfloat16><<<fgrid, kBlock, 0, stream>>>(packed, norms, cb, signs, s,
-                                                                       (__hip_bfloat16*)out, rm, passes);
+#define LAUNCH_DEQ128(TO)                                                                                       \
+    TQ_DISPATCH_BITS(bits, (dequant128x3_kernel<TO, B_><<<fgrid, kBlock, 0, stream>>>(packed, norms, cb, signs, s, \
+                                                                                     (TO*)out, rm, passes)))
+    if (out_dtype == TQ_F32) { LAUNCH_DEQ128(float); }
+    else if (out_dtype == TQ_F16) { LAUNCH_DEQ128(__half); }
+    else { LAUNCH_DEQ128(__hip_bfloat16); }
+#undef LAUNCH_DEQ128
     TQ_CHECK_LAUNCH("tq_dequant launch");
     return TQ_OK;
   }

@@ -6,7 +6,7 @@ back-to-back launches, and rotation over several independent input sets so that 
 Infinity Cache cannot serve the reads.  Prints one line per case: us per call, GB/s of algorithmic
 bytes and the fraction of 8 TB/s.
 
-    python -m tqhip.bench_kernels [--iters 200] [--cases encode,scores,flash,flash_long,sparse_v,vonly,widths,prefill,step]
+    python -m tqhip.bench_kernels [--iters 200] [--cases encode,scores,flash,flash_long,sparse_v,vonly,widths,codec_widths,prefill,step]
 """
 from __future__ import annotations
 
@@ -217,6 +217,24 @@ def bench_widths(iters, dev):
                 report(f"V-only decode 28/4 heads, {bits}-bit values, T={T}, {kind} (graph)", timeit_graph(fns, iters), nbytes)
 
 
+def bench_codec_widths(iters, dev):
+    """Encode / dequantise 1 048 576 vectors at every width: the streaming kernels (row count a multiple of 16)
+    against the generic one-wavefront-per-vector kernels (one row fewer)."""
+    signs = tqhip.random_diagonal_sign(128, 43, device=dev)
+    n = 131072 * 8
+    xs = [torch.randn((n, 128), device=dev, dtype=torch.float16) for _ in range(2)]
+    for bits in (1, 2, 3, 4):
+        cb = gaussian_codebook(bits)
+        bd = gaussian_boundaries(cb)
+        pd = tqhip.packed_dim(128, bits)
+        for rows, kind in ((n, "streaming kernel"), (n - 1, "generic kernel")):
+            fns = [(lambda x=x: tqhip.fused_quantize(x[:rows], signs, bd, 128, bits)) for x in xs]
+            report(f"encode d=128 {bits}-bit, {rows} vectors, {kind}", timeit(fns, max(10, iters // 4)), rows * (256 + 4 * pd + 4))
+            p, nr = tqhip.fused_quantize(xs[0][:rows], signs, bd, 128, bits)
+            fns = [(lambda: tqhip.dequant_fp16(p, nr, cb, signs, 128, bits))]
+            report(f"dequant_fp16 d=128 {bits}-bit, {rows} vectors, {kind}", timeit(fns, max(10, iters // 4)), rows * (256 + 4 * pd + 4))
+
+
 def bench_prefill(iters, dev):
     """benchmark configuration 5, attention half: a chunk of 512 query rows x 32 heads at the end of a
     131072-position packed cache (8 kv heads), causal.  Matrix-core bound: reported in TFLOP/s of
@@ -309,7 +327,7 @@ def bench_step(iters, dev):
 
 
 CASES = {"step": bench_step, "prefill": bench_prefill, "encode": bench_encode, "scores": bench_scores, "sparse_v": bench_sparse_v, "flash": bench_flash,
-         "flash_long": bench_flash_long, "vonly": bench_vonly, "widths": bench_widths}
+         "flash_long": bench_flash_long, "vonly": bench_vonly, "widths": bench_widths, "codec_widths": bench_codec_widths}
 
 
 def main():
