@@ -302,8 +302,8 @@ typedef struct tq_vonly_cache_desc {
 
 /*
  * One decode step of a V-only cache in one library call: ONE new token per sequence is inserted at
- * time index `position` and the query token attends over positions 0 .. position.  For dim 128,
- * 3-bit values and n_rep <= 16 that is two launches: the tile pass over positions 0 .. position - 1,
+ * time index `position` and the query token attends over positions 0 .. position.  For dim 128
+ * (values of any width, bits 1-4) and n_rep <= 16 that is two launches: the tile pass over positions 0 .. position - 1,
  * and a merge pass that encodes the new value row with the encoder's own arithmetic, scores the new
  * key, folds both in and stores the key row, the raw value row, the packed words and the norm (the
  * stored state is bit-identical to tq_vonly_append's, the output agrees with the two calls to the
@@ -336,7 +336,7 @@ int tq_vonly_append_at(const void* k_new, int k_dtype, const void* v_new, int v_
  * *position_dev and attends over positions 0 .. *position_dev (clamped to the storage).  Grids and the
  * workspace are sized for t_alloc positions, so the same recorded launches serve every step until the
  * storage is reallocated; the caller advances the counter between steps (on the same stream).
- * dim 128, 3-bit values, n_rep <= 16 only (TQ_ERR_UNSUPPORTED otherwise).
+ * dim 128 (values of any width) and n_rep <= 16 only (TQ_ERR_UNSUPPORTED otherwise).
  */
 int tq_vonly_decode_step_at(const tq_vonly_cache_desc* cache /* host */,
                             const void* k_new, int k_dtype, const void* v_new, int v_dtype,

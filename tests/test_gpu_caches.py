@@ -729,7 +729,7 @@ def test_vonly_decode_step_from_an_empty_cache_and_at_tile_boundaries(tq, dtype)
 
 
 def test_vonly_decode_step_other_shapes_take_the_append_route(tq):
-    """d = 64 / 4-bit values: tq_vonly_decode_step has no two-launch form there and runs tq_vonly_append +
+    """d = 64: tq_vonly_decode_step has no two-launch form there and runs tq_vonly_append +
     tq_vonly_decode_attn inside the one call: the very bits of the two calls of the Python surface."""
     B, n_q, n_kv, D, S0 = 1, 6, 2, 64, 70
     sc = 1 / math.sqrt(D)
@@ -745,7 +745,7 @@ def test_vonly_decode_step_other_shapes_take_the_append_route(tq):
         assert torch.equal(x, y)
     pos = torch.tensor([a.offset], dtype=torch.int64, device="cuda")
     with pytest.raises((ValueError, RuntimeError)):
-        a.decode_step(q1, k1, v1, sc, position=pos)                  # the device-side position needs d = 128 / 3-bit
+        a.decode_step(q1, k1, v1, sc, position=pos)                  # the device-side position needs d = 128
 
 
 @pytest.mark.parametrize("S0,want_alloc", [(300, 1024), (31000, 32768)])

@@ -360,3 +360,58 @@ def test_streaming_dequantiser_other_widths_bit_exact(tq, bits, out):
         tq.dequant_into(dev(wp), dev(wn), c, dev(s), outbuf, n_groups=1, rows_per_group=n, packed_group_stride=n,
                         norms_group_stride=n, out_group_stride=n, dim=128, bits=bits)
         assert torch.equal(outbuf.cpu(), torch.from_numpy(want).to(td))
+
+
+# ------------------------------------------------------------------ the step that inserts its own token
+
+@pytest.mark.parametrize("bits", [1, 2, 4])
+def test_vonly_step_with_in_merge_insert_other_widths_hip_graph(tq, bits):
+    """decode_step at the other widths is the two-launch form as well (the merge pass encodes and stores the new
+    token), with the position in device memory it can be recorded in a HIP graph: every replay matches the float64
+    oracle on the cache's own state, and the state is, bit for bit, the one update_and_fetch (the encoder kernels)
+    builds from the same tokens."""
+    rng = np.random.default_rng(380 + bits)
+    B, n_kv, n_rep, S0, N = 2, 4, 7, 300, 6
+    n_q = n_kv * n_rep
+    sc = 1 / math.sqrt(D)
+
+    def rnd(shape):
+        return torch.from_numpy(rng.standard_normal(shape).astype(np.float16)).cuda()
+    k0, v0 = rnd((B, n_kv, S0, D)), rnd((B, n_kv, S0, D))
+    cg, ce = tq.VOnlyTurboQuantCache(bits=bits, fused=True), tq.VOnlyTurboQuantCache(bits=bits, fused=True)
+    cg.reserve(B, n_kv, 1024, D)
+    cg.update_and_fetch(k0, v0), ce.update_and_fetch(k0, v0)
+    pos = torch.tensor([S0], dtype=torch.int64, device="cuda")
+    qs, ks, vs = rnd((B, n_q, 1, D)), rnd((B, n_kv, 1, D)), rnd((B, n_kv, 1, D))
+    out_s = torch.empty((B, n_q, D), dtype=torch.float16, device="cuda")
+
+    def check(step_no, q):
+        st = ce.state
+        vq = ce._v_tq._v_q
+        for s_ in range(B):
+            ref = o.vonly_decode_attention(q[s_, :, 0].cpu().numpy(), st[0][s_].cpu().numpy(),
+                                           st[2][s_].cpu().numpy().view(np.uint32), st[3][s_].cpu().numpy(),
+                                           np.asarray(vq.centroids.cpu()), vq.signs.cpu().numpy(), D, bits, sc)
+            close(out_s[s_].float().cpu().numpy(), ref)
+
+    cg.decode_step(qs, ks, vs, sc, position=pos, out=out_s)          # eager once: workspace, descriptor
+    pos.add_(1)
+    ce.update_and_fetch(ks, vs)                                      # the twin goes through the encoder kernels
+    check(-1, qs)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        cg.decode_step(qs, ks, vs, sc, position=pos, out=out_s)
+        pos.add_(1)
+    for i in range(N):
+        q, k, v = rnd((B, n_q, 1, D)), rnd((B, n_kv, 1, D)), rnd((B, n_kv, 1, D))
+        qs.copy_(q), ks.copy_(k), vs.copy_(v)
+        graph.replay()
+        ce.update_and_fetch(k, v)
+        check(i, q)
+        torch.cuda.synchronize()
+        assert int(pos.item()) == S0 + 2 + i
+    cg.set_offset(S0 + 1 + N)
+    assert cg.offset == ce.offset == S0 + 1 + N
+    for x, y in zip(cg.state, ce.state):
+        assert torch.equal(x, y)

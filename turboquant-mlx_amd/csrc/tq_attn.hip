@@ -1325,11 +1325,11 @@ namespace {
 constexpr int kNotFused = 1;   // not an error: the caller takes the append + attention route
 
 // A decode step as two launches: the tile pass over the positions before the new one, and a merge pass that
-// encodes and stores the new token itself (tqm::FreshToken).  dim 128, 3-bit values, n_rep <= 16.
+// encodes and stores the new token itself (tqm::FreshToken).  dim 128, values of any width, n_rep <= 16.
 int vonly_step_fused(const tq_vonly_cache_desc* c, const void* k_new, int k_dtype, const void* v_new, int v_dtype,
                      const void* q, int q_dtype, void* out, int out_dtype, int64_t position, const int64_t* position_dev,
                      float attn_scale, tq_stream_t stream_, const char* who) {
-  if (!(c->dim == 128 && c->bits == 3 && c->n_rep >= 1 && c->n_rep <= tqm::kHeadsMax && c->allow_mma &&
+  if (!(c->dim == 128 && c->bits >= 1 && c->bits <= 4 && c->n_rep >= 1 && c->n_rep <= tqm::kHeadsMax && c->allow_mma &&
         tq::aligned(q, 16) && tq::aligned(c->k_f16, 16)))
     return kNotFused;
   if (tq::check_dtype(k_dtype) || tq::check_dtype(v_dtype) || tq::check_dtype(q_dtype) || tq::check_dtype(out_dtype))
@@ -1346,8 +1346,10 @@ int vonly_step_fused(const tq_vonly_cache_desc* c, const void* k_new, int k_dtyp
   f.k_new = k_new; f.v_new = v_new; f.q = q;
   f.k_f16 = (__half*)c->k_f16; f.v_raw = c->v_raw; f.v_packed = c->v_packed; f.v_norms = c->v_norms;
   f.pos_dev = position_dev; f.pos = position; f.t_alloc = c->t_alloc;
+  for (int i = 0; i < 15; ++i) f.thr[i] = INFINITY;         // past the width: never exceeded
   tq::encode_thresholds(c->boundaries, c->dim, c->bits, c->variant, f.thr);
-  for (int i = 0; i < 8; ++i) f.cent[i] = c->centroids[i];
+  for (int i = 0; i < 16; ++i) f.cent[i] = i < (1 << c->bits) ? c->centroids[i] : 0.0f;
+  f.bits = c->bits;
   f.cs = attn_scale * tqm::kLog2e;
   f.k_dtype = k_dtype; f.v_dtype = v_dtype; f.q_dtype = q_dtype;
   tq_decode_shape sh{};
@@ -1484,8 +1486,8 @@ extern "C" int tq_vonly_decode_step_at(const tq_vonly_cache_desc* c, const void*
   sh.attn_scale = attn_scale; sh.out_dtype = out_dtype; sh.allow_mma = 1;
   if (int rc = check_shape(&sh, who, 256)) return rc;
   if (tq::check_dtype(q_dtype)) return tq::fail(TQ_ERR_DTYPE, "%s: unknown q_dtype %d", who, q_dtype);
-  if (!(mma_shape(sh) && tq::aligned(q, 16) && tq::aligned(c->k_f16, 16)))
-    return tq::fail(TQ_ERR_UNSUPPORTED, "%s: dim 128, 3-bit values, n_rep <= 16 and aligned q / k only", who);
+  if (!(vonly_mma_shape(sh) && tq::aligned(q, 16) && tq::aligned(c->k_f16, 16)))
+    return tq::fail(TQ_ERR_UNSUPPORTED, "%s: dim 128, n_rep <= 16 and aligned q / k only", who);
   const int n_q = c->n_kv_heads * c->n_rep;
   if (c->workspace_bytes < tq_workspace_bytes(TQ_OP_VONLY_DECODE, c->n_seq, n_q, c->t_alloc, c->dim))
     return tq::fail(TQ_ERR_WORKSPACE, "%s: workspace too small for %lld positions", who, (long long)c->t_alloc);
@@ -1532,8 +1534,10 @@ int packed_step(const tq_packed_cache_desc* c, const void* k_new, int k_dtype, c
     f.v_packed = c->v_packed; f.v_norms = c->v_norms; f.k_packed = c->k_packed; f.k_norms = c->k_norms;
     f.k_signs = c->k_signs;
     f.pos_dev = position_dev; f.pos = position; f.t_alloc = c->t_alloc;
+    for (int i = 0; i < 15; ++i) f.thr[i] = INFINITY;
     tq::encode_thresholds(c->boundaries, c->dim, c->bits, c->variant, f.thr);
-    for (int i = 0; i < 8; ++i) f.cent[i] = c->centroids[i];
+    for (int i = 0; i < 16; ++i) f.cent[i] = i < (1 << c->bits) ? c->centroids[i] : 0.0f;
+    f.bits = c->bits;
     f.cs = attn_scale * tqm::kLog2e;
     f.k_dtype = k_dtype; f.v_dtype = v_dtype; f.q_dtype = q_dtype;
     tq_decode_shape fs{};

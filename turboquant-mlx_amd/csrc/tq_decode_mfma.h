@@ -1018,8 +1018,9 @@ struct FreshToken {
   float* v_norms;
   const int64_t* pos_dev;     // insert position in device memory, or null: `pos`
   int64_t pos, t_alloc;
-  float thr[7];               // decision thresholds in the domain of the raw butterfly output
-  float cent[8];
+  float thr[15];              // decision thresholds in the domain of the raw butterfly output; +inf past the 2^bits - 1 real ones
+  float cent[16];
+  int32_t bits;               // width of the packed fields, 1-4 (packed keys: 3)
   float cs;                   // attn_scale * log2 e
   int32_t k_dtype, v_dtype, q_dtype;
   // Cache with packed keys (k_packed set; k_f16 / v_raw unused): the new key row is encoded as well (signs
@@ -1029,6 +1030,35 @@ struct FreshToken {
   uint32_t* k_packed;
   float* k_norms;
 };
+
+// Level of one butterfly output (count of thresholds it exceeds, strictly) and the centroid of that level, for a
+// token inserted by the merge pass.  NB = thresholds looked at: 7 serves widths up to three bits (entries past the
+// width are +inf), 15 the four-bit width; selects, not a dynamic index into kernel arguments.
+template <int NB>
+__device__ __forceinline__ void fresh_level(const FreshToken& f, float w, uint32_t& n, float& c) {
+  n = 0;
+#pragma unroll
+  for (int b = 0; b < NB; ++b) n += (w > f.thr[b]) ? 1u : 0u;
+  c = f.cent[0];
+#pragma unroll
+  for (int k = 1; k <= NB; ++k) c = (n == (uint32_t)k) ? f.cent[k] : c;
+}
+
+// Packed word `lane` of a row whose 128 indices sit two per lane (idx[0] = element lane, idx[1] = element
+// lane + 64): elements VPW * lane .. VPW * lane + VPW - 1, fields of BITS bits, lowest first (packing.py:26-56).
+template <int BITS>
+__device__ __forceinline__ uint32_t fresh_word(const int (&idx)[2], int lane) {
+  constexpr int VPW = BITS == 3 ? 10 : 32 / BITS;
+  uint32_t word = 0;
+#pragma unroll
+  for (int i = 0; i < VPW; ++i) {
+    const int e = min(VPW * lane + i, kD - 1);
+    const int lo = __shfl(idx[0], e & 63), hi = __shfl(idx[1], e & 63);
+    const uint32_t fld = (uint32_t)((e >> 6) ? hi : lo);
+    if (VPW * lane + i < kD) word |= fld << (BITS * i);
+  }
+  return word;
+}
 
 // An element of a tensor whose dtype is a run-time value, in two steps so that a wavefront can have the loads of
 // several such tensors in flight together: the raw bits first (one uniform branch on the element size, no use of
@@ -1111,13 +1141,10 @@ __device__ __forceinline__ void merge_rows_body(
     if (ok && r == 0) fresh_row = grp * f.t_alloc + pos;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      uint32_t n = 0;
-#pragma unroll
-      for (int b = 0; b < 7; ++b) n += (v[i] > f.thr[b]) ? 1u : 0u;
+      uint32_t n;
+      float c;
+      if (f.bits <= 3) fresh_level<7>(f, v[i], n, c); else fresh_level<15>(f, v[i], n, c);      // uniform
       idx[i] = (int)n;
-      float c = f.cent[0];                               // selects, not a dynamic index into kernel arguments
-#pragma unroll
-      for (int k = 1; k < 8; ++k) c = (n == (uint32_t)k) ? f.cent[k] : c;
       acc_s[8][lane + 64 * i] = nrm * c;
     }
     float d;
@@ -1134,13 +1161,10 @@ __device__ __forceinline__ void merge_rows_body(
       d = 0.0f;
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
-        uint32_t n = 0;
-#pragma unroll
-        for (int b = 0; b < 7; ++b) n += (kv[i] > f.thr[b]) ? 1u : 0u;
+        uint32_t n;
+        float c;
+        fresh_level<7>(f, kv[i], n, c);                    // packed keys are three-bit
         kidx[i] = (int)n;
-        float c = f.cent[0];
-#pragma unroll
-        for (int k = 1; k < 8; ++k) c = (n == (uint32_t)k) ? f.cent[k] : c;
         d += c * qr[i];
       }
 #pragma unroll
@@ -1191,27 +1215,23 @@ __device__ __forceinline__ void merge_rows_body(
   }
   __syncthreads();
   if constexpr (FRESH) { if (fresh_wave) {
-    // packed word `lane` holds elements 10 * lane .. 10 * lane + 9 (3-bit fields, lowest first)
+    // packed word `lane` holds elements vpw * lane .. vpw * lane + vpw - 1 (fields of `bits` bits, lowest first;
+    // 10 per word at three bits, else 32 / bits)
     const FreshToken& f = *ft;
-    uint32_t word = 0, kword = 0;
-#pragma unroll
-    for (int i = 0; i < 10; ++i) {
-      const int e = min(10 * lane + i, kD - 1);
-      const int lo = __shfl(idx[0], e & 63), hi = __shfl(idx[1], e & 63);
-      const uint32_t fld = (uint32_t)((e >> 6) ? hi : lo);
-      if (10 * lane + i < kD) word |= fld << (3 * i);
-      if (f.k_packed) {
-        const int klo = __shfl(kidx[0], e & 63), khi = __shfl(kidx[1], e & 63);
-        const uint32_t kfld = (uint32_t)((e >> 6) ? khi : klo);
-        if (10 * lane + i < kD) kword |= kfld << (3 * i);
-      }
-    }
+    const int bits = f.bits;                               // uniform
+    const int pd = bits == 3 ? kPdim : 4 * bits;           // words per row: 4, 8, 13, 16
+    uint32_t word, kword = 0;
+    if (bits == 3) word = fresh_word<3>(idx, lane);
+    else if (bits == 4) word = fresh_word<4>(idx, lane);
+    else if (bits == 2) word = fresh_word<2>(idx, lane);
+    else word = fresh_word<1>(idx, lane);
+    if (f.k_packed) kword = fresh_word<3>(kidx, lane);     // packed keys are three-bit
     if (fresh_row >= 0) {                                  // first query head of the kv head, position inside the storage
       const int64_t row = fresh_row;
-      if (lane < kPdim) f.v_packed[row * kPdim + lane] = word;
+      if (lane < pd) f.v_packed[row * pd + lane] = word;
       if (lane == 0) f.v_norms[row] = fresh_nrm;
       if (f.k_packed) {
-        if (lane < kPdim) f.k_packed[row * kPdim + lane] = kword;
+        if (lane < pd) f.k_packed[row * pd + lane] = kword;
         if (lane == 0) f.k_norms[row] = fresh_knrm;
       } else {
 #pragma unroll

@@ -298,8 +298,10 @@ def bench_step(iters, dev):
             print(f"layer step, {kind}, {n_q}/{n_kv} heads, T~{T}: update_and_fetch + attention {us2:6.1f} us wall, "
                   f"decode_step {us1:6.1f} us wall", flush=True)
             del c
-        for kind, n_q, n_kv in (("V-only cache", 28, 4), ("packed cache", 32, 8)):
-            mk = (lambda: tqhip.VOnlyTurboQuantCache(bits=3, fused=True)) if kind == "V-only cache" else \
+        for kind, n_q, n_kv in (("V-only cache", 28, 4), ("packed cache", 32, 8), ("V-only cache, 4-bit values", 28, 4),
+                                ("V-only cache, 2-bit values", 28, 4)):
+            vb = 4 if "4-bit" in kind else 2 if "2-bit" in kind else 3
+            mk = (lambda: tqhip.VOnlyTurboQuantCache(bits=vb, fused=True)) if kind.startswith("V-only cache") else \
                  (lambda: tqhip.TurboQuantKVCache(bits=3, fused=True))
             caches = [mk() for _ in range(L)]
             k0 = torch.randn((1, n_kv, T, D), device=dev, dtype=torch.float16)
