@@ -415,3 +415,37 @@ def test_vonly_step_with_in_merge_insert_other_widths_hip_graph(tq, bits):
     assert cg.offset == ce.offset == S0 + 1 + N
     for x, y in zip(cg.state, ce.state):
         assert torch.equal(x, y)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("bits", [1, 2, 4])
+def test_vonly_step_other_widths_from_an_empty_cache_and_at_tile_boundaries(tq, bits, dtype):
+    """The merge pass that inserts the token, at the other widths: from an empty cache (no tile pass at all), and at
+    lengths around the 256- and 512-position tile boundaries, with keys, values and queries of every dtype; the state
+    equals the two-call cache's bit for bit and the output matches the float64 oracle."""
+    rng = np.random.default_rng(390 + bits)
+    B, n_q, n_kv = 2, 8, 2
+    sc = 1 / math.sqrt(D)
+
+    def rnd(shape):
+        return torch.from_numpy(rng.standard_normal(shape).astype(F32)).to(dtype).cuda()
+    a, b = tq.VOnlyTurboQuantCache(bits=bits, fused=True), tq.VOnlyTurboQuantCache(bits=bits, fused=True)
+    for grow in (0, 254, 255, 2, 253, 1):                           # steps at lengths 0, 255, 511, 512, 513, 767, 768, 769
+        if grow:
+            k0, v0 = rnd((B, n_kv, grow, D)), rnd((B, n_kv, grow, D))
+            a.update_and_fetch(k0, v0), b.update_and_fetch(k0, v0)
+        for _ in range(2 if grow in (2, 1) else 1):
+            k1, v1, q1 = rnd((B, n_kv, 1, D)), rnd((B, n_kv, 1, D)), rnd((B, n_q, 1, D))
+            got = a.decode_step(q1, k1, v1, sc)
+            b.update_and_fetch(k1, v1)
+            assert a.offset == b.offset
+            st = a.state
+            for x, y in zip(st, b.state):
+                assert x.dtype == y.dtype and torch.equal(x, y), a.offset
+            vq = a._v_tq._v_q
+            for s_ in range(B):
+                ref = o.vonly_decode_attention(q1[s_, :, 0].float().cpu().numpy(), st[0][s_].cpu().numpy(),
+                                               st[2][s_].cpu().numpy().view(np.uint32), st[3][s_].cpu().numpy(),
+                                               np.asarray(vq.centroids.cpu()), vq.signs.cpu().numpy(), D, bits, sc)
+                close(got[s_, :, 0].float().cpu().numpy(), ref, 8e-3 if dtype == torch.bfloat16 else REL, ABS)
+    assert a.offset == 0 + 1 + 254 + 1 + 255 + 1 + 2 + 2 + 253 + 1 + 1 + 2
