@@ -917,8 +917,13 @@ int launch_packed_mfma(const float* q_rot_or_weights, const uint32_t* k_packed, 
     tqm::packed_stream_kernel<<<grid, tqm::kSThreads, 0, stream>>>(a, kcb, vcb, n_steps);
   } else if (n_tiles_real > 0) {
     dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
-    if (MODE == tqm::kWeights) launch_given_tiles_bits(sh.bits, MODE, grid, a, kcb, vcb, stream);   // values of any width
-    else tqm::packed_tile_mfma_kernel<MODE><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, kcb, vcb);
+    if constexpr (MODE == tqm::kWeights) {
+      launch_given_tiles_bits(sh.bits, MODE, grid, a, kcb, vcb, stream);   // values of any width
+    } else if ((int64_t)n_tiles * sh.n_kv_heads * sh.n_seq <= 256) {   // one workgroup per CU at most: the variant without spills
+      tqm::packed_tile_mfma_kernel<MODE, 3, 3><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, kcb, vcb);
+    } else {
+      tqm::packed_tile_mfma_kernel<MODE><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, kcb, vcb);
+    }
   }
   TQ_CHECK_LAUNCH(who);
   dim3 mgrid(n_q, sh.n_seq);

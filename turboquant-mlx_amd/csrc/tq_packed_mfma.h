@@ -163,9 +163,11 @@ __device__ __forceinline__ void rotate_query_rows(const void* q_raw, int q_dtype
 }
 
 // grid = (n_tiles_max, n_kv, n_seq), 512 threads.  VBITS: width of the packed values; the modes that read packed
-// keys exist for three bits only (keys and values share the width there).
-template <int MODE, int VBITS = 3>
-__global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(4, 4)))
+// keys exist for three bits only (keys and values share the width there).  WPE = waves per SIMD the registers are
+// budgeted for: 4 lets two workgroups share a CU (the flash mode then spills 20 registers, which large grids repay);
+// 3 is the flash mode without spills, for grids that give a CU one workgroup at most.
+template <int MODE, int VBITS = 3, int WPE = 4>
+__global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
 void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
   using VF = VField<VBITS>;
   constexpr int kVPd = VF::kPd;                                      // words per packed value row
