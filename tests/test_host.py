@@ -262,11 +262,11 @@ def test_vonly_cache_brings_keys_and_values_to_one_capacity(have_k, have_v, offs
 
 
 def test_matrix_core_shape_predicates():
-    """Packed KEYS run on the matrix cores at three bits only; the steps over fp16 keys take packed values of
-    every width the reference's caches accept (v_only_cache.py:41, adaptive.py:26)."""
+    """The one-call steps (packed or fp16 keys) cover d = 128 at every width the reference's caches accept
+    (cache.py:60, v_only_cache.py:41, adaptive.py:26)."""
     for bits in (1, 2, 3, 4):
         assert ops.vonly_threshold_supported(128, bits, 7)
-        assert ops.vonly_sparse_supported(128, bits, 7) == (bits == 3)
+        assert ops.vonly_sparse_supported(128, bits, 7)
     for dim, bits, n_rep in ((64, 3, 1), (256, 3, 4), (128, 3, 17), (128, 3, 0), (128, 5, 1), (128, 0, 1)):
         assert not ops.vonly_threshold_supported(dim, bits, n_rep)
         assert not ops.vonly_sparse_supported(dim, bits, n_rep)

@@ -846,13 +846,23 @@ int launch_vonly_mfma(const void* q, int q_dtype, const void* k_f16, const uint3
 }
 
 // the width as a run-time value
-void launch_given_tiles_bits(int bits, int mode, dim3 grid, const tqm::PackedArgs& a, const Codebook& kcb,
-                                    const Codebook& vcb, hipStream_t stream) {
+void launch_packed_tiles_bits(int bits, int mode, bool one_per_cu, dim3 grid, const tqm::PackedArgs& a, const Codebook& kcb,
+                              const Codebook& vcb, hipStream_t stream) {
   switch (bits) {
-    case 1: tqm::launch_given_tiles<1>(mode, grid, a, kcb, vcb, stream); break;
-    case 2: tqm::launch_given_tiles<2>(mode, grid, a, kcb, vcb, stream); break;
-    case 4: tqm::launch_given_tiles<4>(mode, grid, a, kcb, vcb, stream); break;
-    default: tqm::launch_given_tiles<3>(mode, grid, a, kcb, vcb, stream); break;
+    case 1: tqm::launch_packed_tiles<1>(mode, one_per_cu, grid, a, kcb, vcb, stream); break;
+    case 2: tqm::launch_packed_tiles<2>(mode, one_per_cu, grid, a, kcb, vcb, stream); break;
+    case 4: tqm::launch_packed_tiles<4>(mode, one_per_cu, grid, a, kcb, vcb, stream); break;
+    default: tqm::launch_packed_tiles<3>(mode, one_per_cu, grid, a, kcb, vcb, stream); break;
+  }
+}
+
+void launch_packed_stream_bits(int bits, dim3 grid, const tqm::PackedArgs& a, const Codebook& kcb, const Codebook& vcb,
+                               int n_steps, hipStream_t stream) {
+  switch (bits) {
+    case 1: tqm::launch_packed_stream<1>(grid, a, kcb, vcb, n_steps, stream); break;
+    case 2: tqm::launch_packed_stream<2>(grid, a, kcb, vcb, n_steps, stream); break;
+    case 4: tqm::launch_packed_stream<4>(grid, a, kcb, vcb, n_steps, stream); break;
+    default: tqm::launch_packed_stream<3>(grid, a, kcb, vcb, n_steps, stream); break;
   }
 }
 
@@ -908,22 +918,20 @@ int launch_packed_mfma(const float* q_rot_or_weights, const uint32_t* k_packed, 
   a.v_unscale = tq::fill_codebook_fp16(vcb, v_centroids, sh.bits);
   int tile_pos = tqm::kTilePos;
   a.len_dev = len_dev; a.len_bias = len_bias;             // a length read on the device: an upper bound on the host, like a ragged batch
-  const int n_steps = (MODE == tqm::kFlash && !sh.mask)
-                          ? flash_stream_steps(sh.n_seq, sh.n_kv_heads, sh.seq_len, sh.seq_offsets != nullptr || len_dev != nullptr) : 0;
+  // the streaming pass takes rows at any 4-byte offset at three bits only (the other widths: 16-byte aligned tensors)
+  const bool stream_ok = MODE == tqm::kFlash && !sh.mask &&
+                         (sh.bits == 3 || (tq::aligned(k_packed, 16) && tq::aligned(v_packed, 16)));
+  const int n_steps = stream_ok ? flash_stream_steps(sh.n_seq, sh.n_kv_heads, sh.seq_len,
+                                                     sh.seq_offsets != nullptr || len_dev != nullptr) : 0;
   if (n_steps >= 2) {
     tile_pos = tqm::kSStepPos * n_steps;
     a.n_tiles_max = (int)((sh.seq_len + tile_pos - 1) / tile_pos);
     dim3 grid(a.n_tiles_max, sh.n_kv_heads, sh.n_seq);
-    tqm::packed_stream_kernel<<<grid, tqm::kSThreads, 0, stream>>>(a, kcb, vcb, n_steps);
+    launch_packed_stream_bits(sh.bits, grid, a, kcb, vcb, n_steps, stream);
   } else if (n_tiles_real > 0) {
     dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
-    if constexpr (MODE == tqm::kWeights) {
-      launch_given_tiles_bits(sh.bits, MODE, grid, a, kcb, vcb, stream);   // values of any width
-    } else if ((int64_t)n_tiles * sh.n_kv_heads * sh.n_seq <= 256) {   // one workgroup per CU at most: the variant without spills
-      tqm::packed_tile_mfma_kernel<MODE, 3, 3><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, kcb, vcb);
-    } else {
-      tqm::packed_tile_mfma_kernel<MODE><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, kcb, vcb);
-    }
+    // at most one workgroup per CU: the flash variant without spills
+    launch_packed_tiles_bits(sh.bits, MODE, (int64_t)n_tiles * sh.n_kv_heads * sh.n_seq <= 256, grid, a, kcb, vcb, stream);
   }
   TQ_CHECK_LAUNCH(who);
   dim3 mgrid(n_q, sh.n_seq);
@@ -981,7 +989,7 @@ int launch_soft_weights(const float* scores, const float* stats, int stats_tile_
   Codebook kcb, vcb;
   fill_codebook(kcb, nullptr, sh.bits);
   a.v_unscale = tq::fill_codebook_fp16(vcb, v_centroids, sh.bits);
-  launch_given_tiles_bits(sh.bits, tqm::kSoftWeights, grid, a, kcb, vcb, stream);
+  launch_packed_tiles_bits(sh.bits, tqm::kSoftWeights, false, grid, a, kcb, vcb, stream);
   TQ_CHECK_LAUNCH(who);
 
   dim3 mgrid(n_q, sh.n_seq);
@@ -1080,20 +1088,18 @@ int launch_flash_sparse(const float* q_rot, const uint32_t* k_packed, const floa
   Codebook kcb;
   a.score_scale = sh.attn_scale / (float)sh.dim * tq::fill_codebook_fp16(kcb, k_centroids, sh.bits);
   dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
-  tqm::packed_tile_mfma_kernel<tqm::kSoftScores><<<grid, tqm::kMfmaThreads, 0, stream>>>(a, kcb, kcb);
+  launch_packed_tiles_bits(sh.bits, tqm::kSoftScores, false, grid, a, kcb, kcb, stream);
   TQ_CHECK_LAUNCH(who);
   return launch_soft_weights(scores, stats, tqm::kTilePos, ws_S, ws_ml, t_pad, n_tiles, v_packed, v_norms, v_centroids,
                              v_signs, threshold, out, sh, stream, who);
 }
 
+// the matrix-core tile passes exist for d = 128 at every width
 bool mma_shape(const tq_decode_shape& sh) {
-  return sh.allow_mma && sh.dim == 128 && sh.bits == 3 && sh.n_rep <= tqm::kHeadsMax && sh.seq_len > 0;
-}
-
-// the tile pass over fp16 keys and packed values exists for every value width
-bool vonly_mma_shape(const tq_decode_shape& sh) {
   return sh.allow_mma && sh.dim == 128 && sh.bits >= 1 && sh.bits <= 4 && sh.n_rep <= tqm::kHeadsMax && sh.seq_len > 0;
 }
+
+bool vonly_mma_shape(const tq_decode_shape& sh) { return mma_shape(sh); }
 
 int check_shape(const tq_decode_shape* sh, const char* who, int max_dim) {
   if (!sh) return tq::fail(TQ_ERR_NULL, "%s: null shape", who);
@@ -1136,7 +1142,7 @@ extern "C" int tq_prerot_qk_scores(const float* q_rot, const uint32_t* k_packed,
     return tq::fail(TQ_ERR_NULL, "tq_prerot_qk_scores: null pointer");
   Codebook cb;
   fill_codebook(cb, centroids, bits);
-  if (allow_mma && dim == 128 && bits == 3 && n_rep <= tqm::kHeadsMax && tq::aligned(q_rot, 8)) {
+  if (allow_mma && dim == 128 && bits >= 1 && bits <= 4 && n_rep <= tqm::kHeadsMax && tq::aligned(q_rot, 8)) {
     tqm::PackedArgs a{};
     a.q_rot = q_rot; a.k_packed = k_packed; a.k_norms = k_norms; a.scores = scores;
     a.seq_len = seq_len; a.k_head_stride = packed_head_stride; a.kn_head_stride = norms_head_stride;
@@ -1144,7 +1150,7 @@ extern "C" int tq_prerot_qk_scores(const float* q_rot, const uint32_t* k_packed,
     Codebook cbh;
     a.score_scale = tq::fill_codebook_fp16(cbh, centroids, bits) / (float)dim;
     dim3 grid((unsigned)((seq_len + tqm::kTilePos - 1) / tqm::kTilePos), n_kv_heads, 1);
-    tqm::packed_tile_mfma_kernel<tqm::kScores><<<grid, tqm::kMfmaThreads, 0, (hipStream_t)stream_>>>(a, cbh, cbh);
+    launch_packed_tiles_bits(bits, tqm::kScores, false, grid, a, cbh, cbh, (hipStream_t)stream_);
     TQ_CHECK_LAUNCH("tq_prerot_qk_scores launch");
     return TQ_OK;
   }
@@ -1438,9 +1444,9 @@ extern "C" int tq_flash_sparse_decode(const float* q_rot, const uint32_t* k_pack
   if (shape->seq_len > 0 && (!k_packed || !k_norms || !v_packed || !v_norms))
     return tq::fail(TQ_ERR_NULL, "%s: null pointer", who);
   if (!(threshold >= 0.0f)) return tq::fail(TQ_ERR_ARG, "%s: threshold must be >= 0", who);
-  if (!(shape->dim == 128 && shape->bits == 3 && shape->n_rep <= tqm::kHeadsMax && shape->seq_len > 0 &&
+  if (!(shape->dim == 128 && shape->bits >= 1 && shape->bits <= 4 && shape->n_rep <= tqm::kHeadsMax && shape->seq_len > 0 &&
         tq::aligned(q_rot, 8)))
-    return tq::fail(TQ_ERR_UNSUPPORTED, "%s: dim 128, 3-bit, n_rep <= 16 and a non-empty cache only "
+    return tq::fail(TQ_ERR_UNSUPPORTED, "%s: dim 128, n_rep <= 16 and a non-empty cache only "
                                         "(compose tq_prerot_qk_scores, tq_softmax_rows and tq_sparse_v_matvec otherwise)", who);
   return launch_flash_sparse(q_rot, k_packed, k_norms, v_packed, v_norms, k_centroids, v_centroids, v_signs, threshold,
                              out, workspace, workspace_bytes, *shape, (hipStream_t)stream_);
@@ -1458,9 +1464,9 @@ extern "C" int tq_flash_decode_from_q(const void* q, int q_dtype, const float* k
   if (shape->seq_len > 0 && (!k_packed || !k_norms || !v_packed || !v_norms))
     return tq::fail(TQ_ERR_NULL, "%s: null pointer", who);
   if (!(threshold >= 0.0f)) return tq::fail(TQ_ERR_ARG, "%s: threshold must be >= 0", who);
-  if (!(shape->dim == 128 && shape->bits == 3 && shape->n_rep <= tqm::kHeadsMax && shape->seq_len > 0 &&
+  if (!(shape->dim == 128 && shape->bits >= 1 && shape->bits <= 4 && shape->n_rep <= tqm::kHeadsMax && shape->seq_len > 0 &&
         tq::aligned(q, (int)tq::dtype_size(q_dtype))))
-    return tq::fail(TQ_ERR_UNSUPPORTED, "%s: dim 128, 3-bit, n_rep <= 16 and a non-empty cache only "
+    return tq::fail(TQ_ERR_UNSUPPORTED, "%s: dim 128, n_rep <= 16 and a non-empty cache only "
                                         "(call tq_prerotate_query and tq_flash_decode otherwise)", who);
   hipStream_t stream = (hipStream_t)stream_;
   if (threshold > 0.0f)
@@ -1516,8 +1522,8 @@ int packed_step(const tq_packed_cache_desc* c, const void* k_new, int k_dtype, c
     return tq::fail(TQ_ERR_ARG, "%s: position %lld outside the storage of %lld positions", who, (long long)position,
                     (long long)c->t_alloc);
   if (!c->k_packed || !c->k_norms || !c->v_packed || !c->v_norms) return tq::fail(TQ_ERR_NULL, "%s: null pointer", who);
-  if (!(c->dim == 128 && c->bits == 3 && c->n_rep >= 1 && c->n_rep <= tqm::kHeadsMax))
-    return tq::fail(TQ_ERR_UNSUPPORTED, "%s: dim 128, 3-bit and n_rep <= 16 only (call tq_encode, "
+  if (!(c->dim == 128 && c->bits >= 1 && c->bits <= 4 && c->n_rep >= 1 && c->n_rep <= tqm::kHeadsMax))
+    return tq::fail(TQ_ERR_UNSUPPORTED, "%s: dim 128 and n_rep <= 16 only (call tq_encode, "
                                         "tq_prerotate_query and tq_flash_decode otherwise)", who);
   const int pdim = tq::packed_dim(c->dim, c->bits);
   const int64_t groups = (int64_t)c->n_seq * c->n_kv_heads;
@@ -1558,7 +1564,7 @@ int packed_step(const tq_packed_cache_desc* c, const void* k_new, int k_dtype, c
   }
   if (int rc = tq::encode_pair(k_new, k_dtype, c->k_signs, c->k_packed + position * pdim, c->k_norms + position, v_new,
                                v_dtype, c->v_signs, c->v_packed + position * pdim, c->v_norms + position, c->boundaries,
-                               groups, c->t_alloc, c->variant, stream_, position_dev))
+                               c->bits, groups, c->t_alloc, c->variant, stream_, position_dev))
     return rc;
   tq_decode_shape sh{};
   sh.n_seq = c->n_seq; sh.n_kv_heads = c->n_kv_heads; sh.n_rep = c->n_rep; sh.dim = c->dim; sh.bits = c->bits;

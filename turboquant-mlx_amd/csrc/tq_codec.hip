@@ -826,7 +826,7 @@ int grid_for_rows(int64_t rows) {
 
 }  // namespace
 
-// Key and value rows of one decode step in one launch (d = 128, 3-bit, one wavefront per row): rows
+// Key and value rows of one decode step in one launch (d = 128, BITS bits, one wavefront per row): rows
 // 0 .. n_rows - 1 are the keys (signs, destination 0), rows n_rows .. 2 n_rows - 1 the values.  Same
 // arithmetic, operation for operation, as encode_kernel.
 struct PairSide {
@@ -839,9 +839,10 @@ struct PairSide {
 
 // With pos_dev set the destination row of group g is g * group_stride + *pos_dev (read when the kernel runs;
 // nothing is stored when that position is outside 0 .. group_stride - 1).
+template <int BITS>
 __global__ __launch_bounds__(kBlock) void encode_pair_kernel(PairSide k, PairSide v, Thresholds thr, int64_t n_rows,
                                                              int64_t group_stride, const int64_t* pos_dev) {
-  constexpr int D = 128, PDIM = 13;
+  constexpr int D = 128, PDIM = BITS == 3 ? 13 : 4 * BITS, VPW = BITS == 3 ? 10 : 32 / BITS, NB = (1 << BITS) - 1;
   const int lane = threadIdx.x & (TQ_WAVE - 1);
   const int wave = threadIdx.x >> 6;
   const int64_t slot = (int64_t)blockIdx.x * kWavesPerBlock + wave;
@@ -868,16 +869,16 @@ __global__ __launch_bounds__(kBlock) void encode_pair_kernel(PairSide k, PairSid
   for (int i = 0; i < 2; ++i) {
     uint32_t n = 0;
 #pragma unroll
-    for (int b = 0; b < 7; ++b) n += (w[i] > thr.t[b]) ? 1u : 0u;
+    for (int b = 0; b < NB; ++b) n += (w[i] > thr.t[b]) ? 1u : 0u;
     idx[i] = (int)n;
   }
-  uint32_t word = 0;                                       // word `lane`: elements 10 * lane .. 10 * lane + 9
+  uint32_t word = 0;                                       // word `lane`: elements VPW * lane .. VPW * lane + VPW - 1
 #pragma unroll
-  for (int i = 0; i < 10; ++i) {
-    const int e = min(10 * lane + i, D - 1);
+  for (int i = 0; i < VPW; ++i) {
+    const int e = min(VPW * lane + i, D - 1);
     const int lo = __shfl(idx[0], e & 63), hi = __shfl(idx[1], e & 63);
     const uint32_t fld = (uint32_t)((e >> 6) ? hi : lo);
-    if (10 * lane + i < D) word |= fld << (3 * i);
+    if (VPW * lane + i < D) word |= fld << (BITS * i);
   }
   int64_t dst = row * group_stride;
   if (pos_dev) {
@@ -892,14 +893,14 @@ __global__ __launch_bounds__(kBlock) void encode_pair_kernel(PairSide k, PairSid
 namespace tq {
 int encode_pair(const void* k_new, int k_dtype, const float* k_signs, uint32_t* k_packed, float* k_norms,
                 const void* v_new, int v_dtype, const float* v_signs, uint32_t* v_packed, float* v_norms,
-                const float* boundaries, int64_t n_rows, int64_t group_stride, int variant, tq_stream_t stream_,
+                const float* boundaries, int bits, int64_t n_rows, int64_t group_stride, int variant, tq_stream_t stream_,
                 const int64_t* pos_dev) {
   Thresholds thr;
   for (int i = 0; i < 15; ++i) thr.t[i] = INFINITY;
-  encode_thresholds(boundaries, 128, 3, variant, thr.t);
+  encode_thresholds(boundaries, 128, bits, variant, thr.t);
   PairSide k{k_new, k_signs, k_packed, k_norms, k_dtype}, v{v_new, v_signs, v_packed, v_norms, v_dtype};
   const int grid = (int)((2 * n_rows + kWavesPerBlock - 1) / kWavesPerBlock);
-  encode_pair_kernel<<<grid, kBlock, 0, (hipStream_t)stream_>>>(k, v, thr, n_rows, group_stride, pos_dev);
+  TQ_DISPATCH_BITS(bits, (encode_pair_kernel<B_><<<grid, kBlock, 0, (hipStream_t)stream_>>>(k, v, thr, n_rows, group_stride, pos_dev)));
   TQ_CHECK_LAUNCH("encode_pair launch");
   return TQ_OK;
 }

@@ -59,12 +59,12 @@ inline int check_dtype(int dt) { return (dt == TQ_F32 || dt == TQ_F16 || dt == T
 // fl(fl(w * s) / s) with the boundary, TQ_ENCODE_METAL compares w itself.
 void encode_thresholds(const float* boundaries, int dim, int bits, int variant, float* thr_out);
 
-// One new key row and one new value row per group (d = 128, 3-bit) encoded by ONE launch: row g of either
-// tensor goes to packed + g * group_stride * 13 words and norms + g * group_stride (defined beside the
-// encoder; the caller has validated pointers and dtypes).
+// One new key row and one new value row per group (d = 128, `bits` bits) encoded by ONE launch: row g of either
+// tensor goes to packed + g * group_stride rows and norms + g * group_stride (defined beside the
+// encoder; the caller has validated pointers, dtypes and the width).
 int encode_pair(const void* k_new, int k_dtype, const float* k_signs, uint32_t* k_packed, float* k_norms,
                 const void* v_new, int v_dtype, const float* v_signs, uint32_t* v_packed, float* v_norms,
-                const float* boundaries, int64_t n_rows, int64_t group_stride, int variant, tq_stream_t stream,
+                const float* boundaries, int bits, int64_t n_rows, int64_t group_stride, int variant, tq_stream_t stream,
                 const int64_t* pos_dev = nullptr);   // set: row g goes to g * group_stride + *pos_dev (device value)
 
 inline size_t dtype_size(int dt) { return dt == TQ_F32 ? 4 : 2; }
@@ -263,6 +263,60 @@ __device__ __forceinline__ float wave_sum(float v) {
   for (int m = 32; m >= 1; m >>= 1) v += shfl_xor_f(v, m);
   return v;
 }
+
+__device__ __forceinline__ uint32_t pack_h2(float a, float b) {
+  __half2 h = __floats2half2_rn(a, b);
+  return *reinterpret_cast<uint32_t*>(&h);
+}
+
+// Packed rows of one bit width (d = 128): words per row, and how a lane gets at the 8 * BITS bits that hold
+// elements 8 pc .. 8 pc + 7 of a row.  Three-bit rows hold ten fields per word, so a piece may straddle two
+// words; the other widths divide the word.
+template <int BITS>
+struct PackedField {
+  static constexpr int kPd = BITS == 3 ? 13 : 4 * BITS;                  // words per packed row
+  static constexpr uint32_t kEven = BITS == 3 ? 0x1C71C7u : BITS == 4 ? 0x0F0F0F0Fu : BITS == 2 ? 0x3333u : 0x55u;   // fields 0, 2, 4, 6
+  static constexpr int kLut = 1 << (2 * BITS);                            // entries of the centroid-pair table
+  __device__ static __forceinline__ void pos(int pc, int& w0, int& sh_lo, int& sh_hi) {
+    if (BITS == 3) {
+      w0 = (pc == 15) ? 11 : (8 * pc) / 10;                               // piece 15: word 11 >> 30 is 0, all of word 12
+      const int s0 = (pc == 15) ? 10 : (8 * pc) % 10;
+      sh_lo = 3 * s0;
+      sh_hi = 30 - 3 * s0;
+    } else {
+      constexpr int kPerWord = 4 / BITS;                                  // pieces per word: 1, 2, 4 for 4, 2, 1 bits
+      w0 = pc / kPerWord;
+      sh_lo = (pc % kPerWord) * 8 * BITS;
+      sh_hi = 0;
+    }
+  }
+  __device__ static __forceinline__ uint32_t field(const uint32_t* at_w0, int sh_lo, int sh_hi) {
+    if (BITS == 3) return ((at_w0[0] >> sh_lo) | (at_w0[1] << sh_hi)) & 0xFFFFFFu;
+    if (BITS == 4) return at_w0[0];
+    return (at_w0[0] >> sh_lo) & ((1u << (8 * BITS)) - 1u);
+  }
+  // even / odd fields of two rows interleaved into table indices at bit offsets 0, 2 BITS, 4 BITS, 6 BITS
+  __device__ static __forceinline__ void interleave(uint32_t fa, uint32_t fb, uint32_t& X, uint32_t& Y) {
+    X = (fa & kEven) | ((fb & kEven) << BITS);
+    Y = ((fa >> BITS) & kEven) | (fb & (kEven << BITS));
+  }
+  __device__ static __forceinline__ uint32_t index(uint32_t src, int i) { return (src >> (2 * BITS * i)) & (uint32_t)(kLut - 1); }
+  // this lane's entries of a table of kLut centroid pairs half2(c[i & mask], c[i >> BITS]); selects, not a dynamic
+  // index into kernel arguments
+  __device__ static __forceinline__ void fill(uint32_t* lut, const Codebook& cb, int lane) {
+#pragma unroll
+    for (int base = 0; base < kLut; base += 64) {
+      const int idx = base + lane;
+      float clo = 0.0f, chi = 0.0f;
+#pragma unroll
+      for (int i = 0; i < (1 << BITS); ++i) {
+        clo = ((idx & ((1 << BITS) - 1)) == i) ? cb.c[i] : clo;
+        chi = ((idx >> BITS) == i) ? cb.c[i] : chi;
+      }
+      if (kLut >= 64 || idx < kLut) lut[idx] = pack_h2(clo, chi);
+    }
+  }
+};
 
 }  // namespace tqd
 

@@ -92,59 +92,9 @@ __device__ __forceinline__ void load_mask4(const float* src, int row0, int rows_
   }
 }
 
-__device__ __forceinline__ uint32_t pack_h2(float a, float b) {
-  __half2 h = __floats2half2_rn(a, b);
-  return *reinterpret_cast<uint32_t*>(&h);
-}
-
-// Packed values of one bit width (d = 128): words per row, and how a lane gets at the 8 * BITS bits that hold
-// elements 8 pc .. 8 pc + 7 of a row.  Three-bit rows hold ten fields per word, so a piece may straddle two
-// words; the other widths divide the word.
+// packed rows of one width: words per row, field extraction, centroid-pair table (tq_common.h)
 template <int BITS>
-struct VField {
-  static constexpr int kPd = BITS == 3 ? 13 : 4 * BITS;                  // words per packed row
-  static constexpr uint32_t kEven = BITS == 3 ? 0x1C71C7u : BITS == 4 ? 0x0F0F0F0Fu : BITS == 2 ? 0x3333u : 0x55u;   // fields 0, 2, 4, 6
-  static constexpr int kLut = 1 << (2 * BITS);                            // entries of the centroid-pair table
-  __device__ static __forceinline__ void pos(int pc, int& w0, int& sh_lo, int& sh_hi) {
-    if (BITS == 3) {
-      w0 = (pc == 15) ? 11 : (8 * pc) / 10;                               // piece 15: word 11 >> 30 is 0, all of word 12
-      const int s0 = (pc == 15) ? 10 : (8 * pc) % 10;
-      sh_lo = 3 * s0;
-      sh_hi = 30 - 3 * s0;
-    } else {
-      constexpr int kPerWord = 4 / BITS;                                  // pieces per word: 1, 2, 4 for 4, 2, 1 bits
-      w0 = pc / kPerWord;
-      sh_lo = (pc % kPerWord) * 8 * BITS;
-      sh_hi = 0;
-    }
-  }
-  __device__ static __forceinline__ uint32_t field(const uint32_t* at_w0, int sh_lo, int sh_hi) {
-    if (BITS == 3) return ((at_w0[0] >> sh_lo) | (at_w0[1] << sh_hi)) & 0xFFFFFFu;
-    if (BITS == 4) return at_w0[0];
-    return (at_w0[0] >> sh_lo) & ((1u << (8 * BITS)) - 1u);
-  }
-  // even / odd fields of two rows interleaved into table indices at bit offsets 0, 2 BITS, 4 BITS, 6 BITS
-  __device__ static __forceinline__ void interleave(uint32_t fa, uint32_t fb, uint32_t& X, uint32_t& Y) {
-    X = (fa & kEven) | ((fb & kEven) << BITS);
-    Y = ((fa >> BITS) & kEven) | (fb & (kEven << BITS));
-  }
-  __device__ static __forceinline__ uint32_t index(uint32_t src, int i) { return (src >> (2 * BITS * i)) & (uint32_t)(kLut - 1); }
-  // this lane's entries of a table of kLut centroid pairs half2(c[i & mask], c[i >> BITS]); selects, not a dynamic
-  // index into kernel arguments
-  __device__ static __forceinline__ void fill(uint32_t* lut, const Codebook& cb, int lane) {
-#pragma unroll
-    for (int base = 0; base < kLut; base += 64) {
-      const int idx = base + lane;
-      float clo = 0.0f, chi = 0.0f;
-#pragma unroll
-      for (int i = 0; i < (1 << BITS); ++i) {
-        clo = ((idx & ((1 << BITS) - 1)) == i) ? cb.c[i] : clo;
-        chi = ((idx >> BITS) == i) ? cb.c[i] : chi;
-      }
-      if (kLut >= 64 || idx < kLut) lut[idx] = pack_h2(clo, chi);
-    }
-  }
-};
+using VField = PackedField<BITS>;
 
 // Cross-wave merge of a workgroup's tile.  Every wave leaves, per head, the maximum m of its scores (log2 units)
 // and its weight sum l, its power-of-two accumulator scale, and its RAW accumulator rows in an LDS area of its
@@ -1020,7 +970,7 @@ struct FreshToken {
   int64_t pos, t_alloc;
   float thr[15];              // decision thresholds in the domain of the raw butterfly output; +inf past the 2^bits - 1 real ones
   float cent[16];
-  int32_t bits;               // width of the packed fields, 1-4 (packed keys: 3)
+  int32_t bits;               // width of the packed fields, 1-4 (keys, where packed, and values alike)
   float cs;                   // attn_scale * log2 e
   int32_t k_dtype, v_dtype, q_dtype;
   // Cache with packed keys (k_packed set; k_f16 / v_raw unused): the new key row is encoded as well (signs
@@ -1163,7 +1113,7 @@ __device__ __forceinline__ void merge_rows_body(
       for (int i = 0; i < 2; ++i) {
         uint32_t n;
         float c;
-        fresh_level<7>(f, kv[i], n, c);                    // packed keys are three-bit
+        if (f.bits <= 3) fresh_level<7>(f, kv[i], n, c); else fresh_level<15>(f, kv[i], n, c);  // uniform
         kidx[i] = (int)n;
         d += c * qr[i];
       }
@@ -1221,11 +1171,10 @@ __device__ __forceinline__ void merge_rows_body(
     const int bits = f.bits;                               // uniform
     const int pd = bits == 3 ? kPdim : 4 * bits;           // words per row: 4, 8, 13, 16
     uint32_t word, kword = 0;
-    if (bits == 3) word = fresh_word<3>(idx, lane);
-    else if (bits == 4) word = fresh_word<4>(idx, lane);
-    else if (bits == 2) word = fresh_word<2>(idx, lane);
-    else word = fresh_word<1>(idx, lane);
-    if (f.k_packed) kword = fresh_word<3>(kidx, lane);     // packed keys are three-bit
+    if (bits == 3) { word = fresh_word<3>(idx, lane); if (f.k_packed) kword = fresh_word<3>(kidx, lane); }
+    else if (bits == 4) { word = fresh_word<4>(idx, lane); if (f.k_packed) kword = fresh_word<4>(kidx, lane); }
+    else if (bits == 2) { word = fresh_word<2>(idx, lane); if (f.k_packed) kword = fresh_word<2>(kidx, lane); }
+    else { word = fresh_word<1>(idx, lane); if (f.k_packed) kword = fresh_word<1>(kidx, lane); }
     if (fresh_row >= 0) {                                  // first query head of the kv head, position inside the storage
       const int64_t row = fresh_row;
       if (lane < pd) f.v_packed[row * pd + lane] = word;
@@ -1303,7 +1252,7 @@ struct VonlyTileChoice {
 };
 
 // The tile pass for values of BITS bits.  Instantiated once per width: 3 beside the host code of the decode
-// entry points, 1, 2 and 4 in a translation unit of their own.
+// entry points, 1, 2 and 4 in translation units of their own (those define TQ_WIDTH_HERE).
 template <int BITS>
 void launch_vonly_tiles(dim3 grid, const VonlyTileChoice& c, const MfmaArgs& a, const Codebook& vcb, hipStream_t stream) {
 #define TQ_LAUNCH_TILE(QF)                                                                                              \
@@ -1318,7 +1267,7 @@ void launch_vonly_tiles(dim3 grid, const VonlyTileChoice& c, const MfmaArgs& a, 
   if (c.q_f32) { TQ_LAUNCH_TILE(true); } else { TQ_LAUNCH_TILE(false); }
 #undef TQ_LAUNCH_TILE
 }
-#ifndef TQ_VONLY_OTHER_WIDTHS_HERE
+#ifndef TQ_WIDTH_HERE
 extern template void launch_vonly_tiles<1>(dim3, const VonlyTileChoice&, const MfmaArgs&, const Codebook&, hipStream_t);
 extern template void launch_vonly_tiles<2>(dim3, const VonlyTileChoice&, const MfmaArgs&, const Codebook&, hipStream_t);
 extern template void launch_vonly_tiles<4>(dim3, const VonlyTileChoice&, const MfmaArgs&, const Codebook&, hipStream_t);

@@ -1,4 +1,4 @@
-// Matrix-core tile pass over PACKED keys and/or values (d = 128, 3-bit, n_rep <= 16).
+// Matrix-core tile pass over PACKED keys and/or values (d = 128, 1 to 4 bits, n_rep <= 16).
 // Included by tq_attn.hip after tq_decode_mfma.h, whose conventions it shares: a workgroup of 8
 // waves owns 512 positions of one kv head, a wave 64 of them; partials go to the workspace and
 // the merge pass finishes.  Three modes:
@@ -9,12 +9,13 @@
 //   kWeights  packed V only: the weights are given, positions below the threshold contribute
 //             nothing (tq_sparse_v_matvec).
 //
-// Packed rows are 52 bytes, so the wave's 64 rows of K (and of V) are one contiguous 3328-byte
-// block: 4 coalesced 16-byte loads per lane, copied into the wave's LDS area.  A lane then needs, per
-// row, the 24 bits holding 8 consecutive elements: two words, one shift-or.  For K the 8 elements
-// are 4 ADJACENT pairs, i.e. four contiguous 6-bit fields, each of which indexes the centroid-pair
-// table directly and yields one register of the A operand; for V two positions are interleaved
-// first (see tq_decode_mfma.h).  Scores are (sum_e c_k[idx] q_rot[e]) * k_norm * (1/d) [* scale].
+// Packed rows are 52 bytes at three bits, so the wave's 64 rows of K (and of V) are one contiguous
+// 3328-byte block: 4 coalesced 16-byte loads per lane, copied into the wave's LDS area.  A lane then
+// needs, per row, the 24 bits holding 8 consecutive elements: two words, one shift-or (the other
+// widths divide the word: one shift).  For K the 8 elements are 4 ADJACENT pairs, i.e. four
+// contiguous fields of 2 * bits bits, each of which indexes the centroid-pair table directly and
+// yields one register of the A operand; for V two positions are interleaved first (see
+// tq_decode_mfma.h).  Scores are (sum_e c_k[idx] q_rot[e]) * k_norm * (1/d) [* scale].
 #pragma once
 
 #include "tq_decode_mfma.h"
@@ -102,26 +103,6 @@ __device__ __forceinline__ void stage_block(const PackedBlockT<PD>& b, uint32_t*
   }
 }
 
-// word index / shifts of the 24 bits that hold elements 8*pc .. 8*pc+7 of a packed row
-__device__ __forceinline__ void piece_bits(int pc, int& w0, int& sh_lo, int& sh_hi) {
-  w0 = (pc == 15) ? 11 : (8 * pc) / 10;
-  const int s0 = (pc == 15) ? 10 : (8 * pc) % 10;
-  sh_lo = 3 * s0;
-  sh_hi = 30 - 3 * s0;
-}
-
-__device__ __forceinline__ void fill_lut(uint32_t* lut, const Codebook& cb, int tid) {
-  if ((unsigned)tid < 64u) {
-    float clo = 0.0f, chi = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      clo = ((tid & 7) == i) ? cb.c[i] : clo;
-      chi = ((tid >> 3) == i) ? cb.c[i] : chi;
-    }
-    lut[tid] = pack_h2(clo, chi);
-  }
-}
-
 // Query rows of one kv head, rotated in place of a separate pre-rotation launch: wave w takes rows w, w + N_WAVES, ...
 // of the 16 (rows at or past n_rep are zeros), lane l the elements l and l + 64; q * signs, the raw butterfly of
 // tq_prerotate_query (same stage order, hence the same bits), then the fp16 value and the fp16 remainder of that
@@ -162,22 +143,21 @@ __device__ __forceinline__ void rotate_query_rows(const void* q_raw, int q_dtype
   }
 }
 
-// grid = (n_tiles_max, n_kv, n_seq), 512 threads.  VBITS: width of the packed values; the modes that read packed
-// keys exist for three bits only (keys and values share the width there).  WPE = waves per SIMD the registers are
-// budgeted for: 4 lets two workgroups share a CU (the flash mode then spills 20 registers, which large grids repay);
-// 3 is the flash mode without spills, for grids that give a CU one workgroup at most.
-template <int MODE, int VBITS = 3, int WPE = 4>
+// grid = (n_tiles_max, n_kv, n_seq), 512 threads.  BITS: width of the packed keys and values (a cache has one
+// width for both).  WPE = waves per SIMD the registers are budgeted for: 4 lets two workgroups share a CU (the
+// flash mode then spills some registers, which large grids repay); 3 is the flash mode without spills, for
+// grids that give a CU one workgroup at most.
+template <int MODE, int BITS = 3, int WPE = 4>
 __global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
 void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
-  using VF = VField<VBITS>;
-  constexpr int kVPd = VF::kPd;                                      // words per packed value row
+  using VF = VField<BITS>;
+  constexpr int kVPd = VF::kPd;                                      // words per packed row
   constexpr bool GIVEN = MODE == kWeights || MODE == kSoftWeights;   // weights come from memory, no keys
-  static_assert(GIVEN || VBITS == 3, "packed keys are three-bit here");
   constexpr bool HAS_K = !GIVEN;
   constexpr bool HAS_V = MODE != kScores && MODE != kSoftScores;
   constexpr bool SOFT = MODE == kFlash || MODE == kSoftScores;        // scores carry attn_scale * log2 e and the mask
   __shared__ __align__(16) unsigned char big_s[32768];      // per-wave 4 KB areas, later S_all[8][8][128]
-  __shared__ uint32_t lutk_s[64], lutv_s[VF::kLut < 64 ? 64 : VF::kLut];
+  __shared__ uint32_t lutk_s[VF::kLut < 64 ? 64 : VF::kLut], lutv_s[VF::kLut < 64 ? 64 : VF::kLut];
   __shared__ __align__(16) uint32_t q_s[kHeadsMax][kD / 2];      // rotated queries as half2: rounded value ...
   __shared__ __align__(16) uint32_t ql_s[kHeadsMax][kD / 2];     // ... and what the rounding lost
   __shared__ __align__(16) float kn_s[kWaves][kWavePos], vn_s[kWaves][kWavePos];
@@ -220,8 +200,7 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
     }
   }
   float my_kn = 0.0f, my_vn = 0.0f;
-  PackedBlock kb_;
-  PackedBlockT<kVPd> vb_;
+  PackedBlockT<kVPd> kb_, vb_;
   if (HAS_V) {
     my_vn = a.v_norms[(int64_t)seq * a.vn_seq_stride + (int64_t)kvh * a.vn_head_stride + first + tile_p0 + crow];
     load_block(vb_, a.v_packed + ((int64_t)seq * a.v_seq_stride + (int64_t)kvh * a.v_head_stride + first +
@@ -230,7 +209,7 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
   if (HAS_K) {
     my_kn = a.k_norms[(int64_t)seq * a.kn_seq_stride + (int64_t)kvh * a.kn_head_stride + first + tile_p0 + crow];
     load_block(kb_, a.k_packed + ((int64_t)seq * a.k_seq_stride + (int64_t)kvh * a.k_head_stride + first +
-                                  tile_p0 + wrow0) * kPdim, lane, wrow0, rows_here);
+                                  tile_p0 + wrow0) * kVPd, lane, wrow0, rows_here);
   }
   // given weights: lane (head n16, group g) takes positions 16t + 4g + j
   float wgt[4][4];
@@ -305,7 +284,7 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
         wgt[t][j] = (w < a.threshold) ? 0.0f : w;
       }
   }
-  if (HAS_K) fill_lut(lutk_s, kcb, tid);
+  if (HAS_K) { if (tid >= 64 && tid < 128) VF::fill(lutk_s, kcb, tid - 64); }
   if (HAS_V) { if (tid < 64) VF::fill(lutv_s, vcb, tid); }
   if (HAS_K) {
     if (a.q_raw) {
@@ -380,17 +359,17 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
     stage_block(kb_, stage, lane);                       // the V image has been consumed
     int kw0[4], ksl[4], ksh[4];
 #pragma unroll
-    for (int kb = 0; kb < 4; ++kb) piece_bits(4 * kb + g, kw0[kb], ksl[kb], ksh[kb]);
+    for (int kb = 0; kb < 4; ++kb) VF::pos(4 * kb + g, kw0[kb], ksl[kb], ksh[kb]);
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       f4 acc = {0.f, 0.f, 0.f, 0.f};
-      const uint32_t* krow = stage + (16 * t + n16) * kPdim;
+      const uint32_t* krow = stage + (16 * t + n16) * kVPd;
 #pragma unroll
       for (int kb = 0; kb < 4; ++kb) {
-        const uint32_t f = ((krow[kw0[kb]] >> ksl[kb]) | (krow[kw0[kb] + 1] << ksh[kb])) & 0xFFFFFFu;
+        const uint32_t f = VF::field(krow + kw0[kb], ksl[kb], ksh[kb]);
         u4 ka;
 #pragma unroll
-        for (int k = 0; k < 4; ++k) ka[k] = lutk_s[(f >> (6 * k)) & 63u];
+        for (int k = 0; k < 4; ++k) ka[k] = lutk_s[VF::index(f, k)];
         acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, ka), __builtin_bit_cast(h8, qreg[kb]),
                                                      acc, 0, 0, 0);
         acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, ka), __builtin_bit_cast(h8, qlow[kb]),
@@ -534,7 +513,6 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
   merge_waves<kWaves>(mg_s, big_s, 4096, accS, m, l, inv_tscale, a.v_unscale, n_rep, pS, pml);
 }
 
-#ifndef TQ_VONLY_OTHER_WIDTHS_HERE      // a plain (non-template) kernel: defined in one translation unit only
 // Streaming flash-decode pass (packed K and V, no mask): a workgroup of FOUR waves runs through
 // n_steps consecutive 256-position steps of one (sequence, kv head), a wave 64 positions per step,
 // with the online-softmax recurrence in registers, and writes one partial at the end.  Two such
@@ -543,22 +521,29 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
 // computed.  The fixed work of a tile (query staging, tables, merge, partial store) is paid once
 // per n_steps * 256 positions and the merge pass sees that many fewer partials.
 //
-// Loads: a wave's 64 rows of 52 bytes start at an arbitrary multiple of 4 bytes (ragged batches
-// start a sequence at any row).  They are fetched as ALIGNED 16-byte pieces from the 16-byte
+// Loads: at three bits a wave's 64 rows of 52 bytes start at an arbitrary multiple of 4 bytes (ragged
+// batches start a sequence at any row).  They are fetched as ALIGNED 16-byte pieces from the 16-byte
 // boundary at or below the first row (at most 209 pieces) into the wave's LDS image, and rows are
 // read from the image at the misalignment offset.  An aligned 16-byte piece never crosses a page,
 // so a piece that holds at least one valid byte is readable in full; pieces with no valid byte
 // (rows past the end of the sequence) are not fetched and read as zero, and their positions get
-// -inf scores.
+// -inf scores.  Rows of the other widths are 16, 32 or 64 bytes: every row of a 16-byte aligned
+// tensor is aligned (the host sends other tensors to the tile pass), and a block is 64, 128 or 256 pieces.
 constexpr int kSWaves = 4;
 constexpr int kSThreads = kSWaves * 64;
 constexpr int kSStepPos = kSWaves * kWavePos;     // 256 positions per workgroup step
-constexpr int kSImageBytes = 4096;                // 209 pieces of 16 bytes, rounded up
+constexpr int kSImageBytes = 4096;                // 209 pieces of 16 bytes, rounded up; 256 pieces at four bits
 
+template <int BITS>
 __global__ __launch_bounds__(kSThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps) {
+  using VF = VField<BITS>;
+  constexpr int kPd = VF::kPd;                                  // words per packed row
+  constexpr int kPieces = BITS == 3 ? 209 : 16 * kPd;           // 16-byte pieces of a wave's 64 rows (three bits: + misalignment)
+  constexpr int kWhole = kPieces / 64, kRest = kPieces % 64;    // whole-wave stores into the image, lanes of the last one
+  constexpr int kLoads = kWhole + (kRest ? 1 : 0);
   __shared__ __align__(16) unsigned char big_s[kSWaves * 2 * kSImageBytes];   // per wave: K image, V image; later S_all[4][8][128]
-  __shared__ uint32_t lutk_s[64], lutv_s[64];
+  __shared__ uint32_t lutk_s[VF::kLut < 64 ? 64 : VF::kLut], lutv_s[VF::kLut < 64 ? 64 : VF::kLut];
   __shared__ __align__(16) uint32_t q_s[kHeadsMax][kD / 2];
   __shared__ __align__(16) uint32_t ql_s[kHeadsMax][kD / 2];
   __shared__ __align__(16) float kn_s[kSWaves][kWavePos], vn_s[kSWaves][kWavePos];
@@ -586,12 +571,12 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
 
   // ---- addresses: row 0 of the sequence for this kv head, misalignment of the wave's blocks
   const char* krow0 = reinterpret_cast<const char*>(
-      a.k_packed + ((int64_t)seq * a.k_seq_stride + (int64_t)kvh * a.k_head_stride + first) * kPdim);
+      a.k_packed + ((int64_t)seq * a.k_seq_stride + (int64_t)kvh * a.k_head_stride + first) * kPd);
   const char* vrow0 = reinterpret_cast<const char*>(
-      a.v_packed + ((int64_t)seq * a.v_seq_stride + (int64_t)kvh * a.v_head_stride + first) * kPdim);
+      a.v_packed + ((int64_t)seq * a.v_seq_stride + (int64_t)kvh * a.v_head_stride + first) * kPd);
   // every block of this workgroup starts a multiple of 64 rows = 208 pieces after row wg_p0: one misalignment
-  const int kmis = (int)((reinterpret_cast<uintptr_t>(krow0) + (uint64_t)wg_p0 * (kPdim * 4)) & 15);
-  const int vmis = (int)((reinterpret_cast<uintptr_t>(vrow0) + (uint64_t)wg_p0 * (kPdim * 4)) & 15);
+  const int kmis = BITS == 3 ? (int)((reinterpret_cast<uintptr_t>(krow0) + (uint64_t)wg_p0 * (kPd * 4)) & 15) : 0;
+  const int vmis = BITS == 3 ? (int)((reinterpret_cast<uintptr_t>(vrow0) + (uint64_t)wg_p0 * (kPd * 4)) & 15) : 0;
   const float* knrow0 = a.k_norms + (int64_t)seq * a.kn_seq_stride + (int64_t)kvh * a.kn_head_stride + first;
   const float* vnrow0 = a.v_norms + (int64_t)seq * a.vn_seq_stride + (int64_t)kvh * a.vn_head_stride + first;
 
@@ -600,15 +585,15 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
     const int64_t left = len - p0w;
     return (int)(left < 0 ? 0 : (left > kWavePos ? kWavePos : left));
   };
-  auto issue = [&](int s, u4 (&kq)[4], u4 (&vq)[4], float& kn, float& vn) {
+  auto issue = [&](int s, u4 (&kq)[kLoads], u4 (&vq)[kLoads], float& kn, float& vn) {
     const int64_t p0w = wg_p0 + (int64_t)s * kSStepPos + wave * kWavePos;
     const int rows = rows_left_of(s);
-    const int kbytes = rows ? kmis + rows * (kPdim * 4) : 0;
-    const int vbytes = rows ? vmis + rows * (kPdim * 4) : 0;
-    const char* kb = krow0 + p0w * (kPdim * 4) - kmis;
-    const char* vb = vrow0 + p0w * (kPdim * 4) - vmis;
+    const int kbytes = rows ? kmis + rows * (kPd * 4) : 0;
+    const int vbytes = rows ? vmis + rows * (kPd * 4) : 0;
+    const char* kb = krow0 + p0w * (kPd * 4) - kmis;
+    const char* vb = vrow0 + p0w * (kPd * 4) - vmis;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < kLoads; ++i) {
       const int off = (i * 64 + lane) * 16;
       kq[i] = (off < kbytes) ? *reinterpret_cast<const u4*>(kb + off) : u4{0u, 0u, 0u, 0u};
       vq[i] = (off < vbytes) ? *reinterpret_cast<const u4*>(vb + off) : u4{0u, 0u, 0u, 0u};
@@ -625,12 +610,12 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
       my_q[i] = (w < n_rep * (kD / 2)) ? reinterpret_cast<const float2*>(a.q_rot + q_row0 * kD)[w] : make_float2(0.f, 0.f);
     }
   }
-  u4 kqA[4], vqA[4], kqB[4], vqB[4];
+  u4 kqA[kLoads], vqA[kLoads], kqB[kLoads], vqB[kLoads];
   float knA, vnA, knB = 0.0f, vnB = 0.0f;
   issue(0, kqA, vqA, knA, vnA);
 
-  fill_lut(lutk_s, kcb, tid);
-  fill_lut(lutv_s, vcb, tid - 64);
+  if (tid < 64) VF::fill(lutk_s, kcb, tid);
+  else if (tid < 128) VF::fill(lutv_s, vcb, tid - 64);
   if (a.q_raw) {
     rotate_query_rows<kSWaves>(a.q_raw, a.q_dtype, a.k_signs, q_row0, n_rep, wave, lane, q_s, ql_s);
   } else {
@@ -655,10 +640,9 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
   const uint32_t* vimg = reinterpret_cast<const uint32_t*>(image + kSImageBytes + vmis);
   int kw0[4], ksl[4], ksh[4];
 #pragma unroll
-  for (int kb = 0; kb < 4; ++kb) piece_bits(4 * kb + g, kw0[kb], ksl[kb], ksh[kb]);
+  for (int kb = 0; kb < 4; ++kb) VF::pos(4 * kb + g, kw0[kb], ksl[kb], ksh[kb]);
   int vw0, vsl, vsh;
-  piece_bits(n16, vw0, vsl, vsh);
-  constexpr uint32_t kEven = 0x1C71C7u;
+  VF::pos(n16, vw0, vsl, vsh);
   const float kscale = a.score_scale * kLog2e;           // scores in log2 units
 
   f4 accS[8];
@@ -667,7 +651,7 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
   float m_run = -INFINITY, R_run = -INFINITY, l_run = 0.0f, inv_tscale = 1.0f;
 
   // one step on the buffers (kq, vq, kn, vn); `next()` issues the loads of the following step
-  auto step = [&](int sidx, u4 (&kq)[4], u4 (&vq)[4], float kn, float vn_, auto&& next) {
+  auto step = [&](int sidx, u4 (&kq)[kLoads], u4 (&vq)[kLoads], float kn, float vn_, auto&& next) {
     const int rows = rows_left_of(sidx);                 // uniform over the wave
     if (rows <= 0) return;                               // steps only run out at the end: nothing follows
     // ---- images and norms into the wave's LDS area
@@ -675,8 +659,8 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
       u4* k4 = reinterpret_cast<u4*>(image);
       u4* v4 = reinterpret_cast<u4*>(image + kSImageBytes);
 #pragma unroll
-      for (int i = 0; i < 3; ++i) { k4[i * 64 + lane] = kq[i]; v4[i * 64 + lane] = vq[i]; }
-      if (lane < 17) { k4[192 + lane] = kq[3]; v4[192 + lane] = vq[3]; }
+      for (int i = 0; i < kWhole; ++i) { k4[i * 64 + lane] = kq[i]; v4[i * 64 + lane] = vq[i]; }
+      if (kRest) { if (lane < kRest) { k4[kWhole * 64 + lane] = kq[kLoads - 1]; v4[kWhole * 64 + lane] = vq[kLoads - 1]; } }
       kn_s[wave][lane] = kn * kscale;
       vn_s[wave][lane] = vn_;
     }
@@ -688,13 +672,13 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       f4 acc = {0.f, 0.f, 0.f, 0.f};
-      const uint32_t* krow = kimg + (16 * t + n16) * kPdim;
+      const uint32_t* krow = kimg + (16 * t + n16) * kPd;
 #pragma unroll
       for (int kb = 0; kb < 4; ++kb) {
-        const uint32_t f = ((krow[kw0[kb]] >> ksl[kb]) | (krow[kw0[kb] + 1] << ksh[kb])) & 0xFFFFFFu;
+        const uint32_t f = VF::field(krow + kw0[kb], ksl[kb], ksh[kb]);
         u4 ka;
 #pragma unroll
-        for (int k = 0; k < 4; ++k) ka[k] = lutk_s[(f >> (6 * k)) & 63u];
+        for (int k = 0; k < 4; ++k) ka[k] = lutk_s[VF::index(f, k)];
         acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, ka), __builtin_bit_cast(h8, qreg[kb]),
                                                      acc, 0, 0, 0);
         acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, ka), __builtin_bit_cast(h8, qlow[kb]),
@@ -764,11 +748,8 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
 #pragma unroll
       for (int qd = 0; qd < 4; ++qd) {
         const int t = 2 * kb2 + (qd >> 1), jp = qd & 1;
-        const uint32_t* ra = vimg + (16 * t + 4 * g + 2 * jp) * kPdim + vw0;
-        const uint32_t fa = ((ra[0] >> vsl) | (ra[1] << vsh)) & 0xFFFFFFu;
-        const uint32_t fb = ((ra[kPdim] >> vsl) | (ra[kPdim + 1] << vsh)) & 0xFFFFFFu;
-        X[qd] = (fa & kEven) | ((fb & kEven) << 3);
-        Y[qd] = ((fa >> 3) & kEven) | (fb & (kEven << 3));
+        const uint32_t* ra = vimg + (16 * t + 4 * g + 2 * jp) * kPd + vw0;
+        VF::interleave(VF::field(ra, vsl, vsh), VF::field(ra + kPd, vsl, vsh), X[qd], Y[qd]);
       }
       const u4 A = {pa[kb2][0], pa[kb2][1], pa[kb2][2], pa[kb2][3]};
 #pragma unroll
@@ -777,7 +758,7 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
 #pragma unroll
         for (int qd = 0; qd < 4; ++qd) {
           const uint32_t src = (et & 1) ? Y[qd] : X[qd];
-          B[qd] = lutv_s[(src >> (6 * (et >> 1))) & 63u];
+          B[qd] = lutv_s[VF::index(src, et >> 1)];
         }
         accS[et] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, A), __builtin_bit_cast(h8, B),
                                                           accS[et], 0, 0, 0);
@@ -808,20 +789,39 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
   merge_waves<kSWaves>(mg_s, big_s, 2 * kSImageBytes, accS, m_run, l, inv_tscale, a.v_unscale, n_rep, pS, pml);
 }
 
-#endif
-
-// The given-weights tile pass (mode kWeights or kSoftWeights: packed values only) for values of VBITS bits.
-// Instantiated once per width: 3 beside the host code of the entry points, 1, 2 and 4 in a translation unit of their own.
-template <int VBITS>
-void launch_given_tiles(int mode, dim3 grid, const PackedArgs& a, const Codebook& kcb, const Codebook& vcb,
-                        hipStream_t stream) {
-  if (mode == kWeights) packed_tile_mfma_kernel<kWeights, VBITS><<<grid, kMfmaThreads, 0, stream>>>(a, kcb, vcb);
-  else packed_tile_mfma_kernel<kSoftWeights, VBITS><<<grid, kMfmaThreads, 0, stream>>>(a, kcb, vcb);
+// Launchers of the kernels above for one width.  Instantiated once per width: 3 beside the host code of the entry
+// points, 1, 2 and 4 in translation units of their own (the widths compile in parallel).
+//   launch_packed_tiles: the tile pass in `mode`; one_per_cu: the grid gives a CU one workgroup at most
+//   launch_packed_stream: the streaming flash pass (no mask); rows of widths other than 3 must be 16-byte aligned
+template <int BITS>
+void launch_packed_tiles(int mode, bool one_per_cu, dim3 grid, const PackedArgs& a, const Codebook& kcb, const Codebook& vcb,
+                         hipStream_t stream) {
+  switch (mode) {
+    case kFlash:
+      if (one_per_cu) packed_tile_mfma_kernel<kFlash, BITS, 3><<<grid, kMfmaThreads, 0, stream>>>(a, kcb, vcb);
+      else packed_tile_mfma_kernel<kFlash, BITS><<<grid, kMfmaThreads, 0, stream>>>(a, kcb, vcb);
+      break;
+    case kScores: packed_tile_mfma_kernel<kScores, BITS><<<grid, kMfmaThreads, 0, stream>>>(a, kcb, vcb); break;
+    case kSoftScores: packed_tile_mfma_kernel<kSoftScores, BITS><<<grid, kMfmaThreads, 0, stream>>>(a, kcb, vcb); break;
+    case kWeights: packed_tile_mfma_kernel<kWeights, BITS><<<grid, kMfmaThreads, 0, stream>>>(a, kcb, vcb); break;
+    default: packed_tile_mfma_kernel<kSoftWeights, BITS><<<grid, kMfmaThreads, 0, stream>>>(a, kcb, vcb); break;
+  }
 }
-#ifndef TQ_VONLY_OTHER_WIDTHS_HERE
-extern template void launch_given_tiles<1>(int, dim3, const PackedArgs&, const Codebook&, const Codebook&, hipStream_t);
-extern template void launch_given_tiles<2>(int, dim3, const PackedArgs&, const Codebook&, const Codebook&, hipStream_t);
-extern template void launch_given_tiles<4>(int, dim3, const PackedArgs&, const Codebook&, const Codebook&, hipStream_t);
+
+template <int BITS>
+void launch_packed_stream(dim3 grid, const PackedArgs& a, const Codebook& kcb, const Codebook& vcb, int n_steps,
+                          hipStream_t stream) {
+  packed_stream_kernel<BITS><<<grid, kSThreads, 0, stream>>>(a, kcb, vcb, n_steps);
+}
+
+#define TQ_PACKED_LAUNCHERS(KEYWORD, B_)                                                                               \
+  KEYWORD template void launch_packed_tiles<B_>(int, bool, dim3, const PackedArgs&, const Codebook&, const Codebook&,  \
+                                                hipStream_t);                                                          \
+  KEYWORD template void launch_packed_stream<B_>(dim3, const PackedArgs&, const Codebook&, const Codebook&, int, hipStream_t);
+#ifndef TQ_WIDTH_HERE
+TQ_PACKED_LAUNCHERS(extern, 1)
+TQ_PACKED_LAUNCHERS(extern, 2)
+TQ_PACKED_LAUNCHERS(extern, 4)
 #endif
 
 }  // namespace tqm

@@ -1,8 +1,8 @@
-// Chunked-prefill attention over PACKED keys and values (d = 128, 3-bit) on the gfx950 matrix
+// Chunked-prefill attention over PACKED keys and values (d = 128, 1 to 4 bits) on the gfx950 matrix
 // cores: a chunk of query rows (all q heads) against the packed cache up to the chunk's end,
 // causal inside the chunk.  The reference has no kernel for this step: its prefill dequantises
 // the whole cache to fp16 (cache.py:125-129, 209-210) and calls stock SDPA, i.e. it moves
-// 256 B per cached vector where this path moves 56 B and never materialises K or V.
+// 256 B per cached vector where this path moves 56 B (at three bits) and never materialises K or V.
 //
 // Everything happens in the rotated domain, as in flash_attention.py:79-162:
 //   q_rot = B(q * signs_K)                                  (one pass, rounded to fp16)
@@ -24,7 +24,6 @@ typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef float f4 __attribute__((ext_vector_type(4)));
 
 constexpr int kD = 128;
-constexpr int kPdim = 13;
 constexpr int kBlkPos = 64;                     // key positions decoded into LDS per step
 constexpr int kWaves = 8;
 constexpr int kWaveRows = 32;                   // query rows per wavefront
@@ -33,20 +32,14 @@ constexpr int kWgRows = kWaves * kWaveRows;     // 256 query rows per workgroup
 constexpr int kThreads = kWaves * 64;
 constexpr int kKStride = 136;                   // halfs per decoded key row in LDS (272 B: conflict-free b128 reads)
 constexpr int kVStride = 72;                    // halfs per row of the transposed value block (144 B)
-constexpr int kStageWords = kBlkPos * kPdim;    // 832 packed words per block and tensor
 constexpr float kVnScale = 0.0625f;             // value norms enter the fp16 weights times 2^-4 (norms up to 1e6)
 constexpr float kLog2e = 1.44269504088896340736f;
 constexpr int kRowsPerWavePass = 16;            // four lanes per row in the pre-rotation and merge kernels
 
-__device__ __forceinline__ uint32_t pack_h2(float a, float b) {
-  const __half2 h = __floats2half2_rn(a, b);
-  return *reinterpret_cast<const uint32_t*>(&h);
-}
-
 struct PrefillArgs {
   const __half* q_rot;          // [n_q, n_rows, 128] fp16, pre-rotated
   const __half* q_rot_lo;       // same shape: what rounding q_rot to fp16 lost, as fp16
-  const uint32_t* k_packed;     // [n_kv, k_head_stride rows, 13]
+  const uint32_t* k_packed;     // [n_kv, k_head_stride rows, words per packed row]
   const float* k_norms;
   const uint32_t* v_packed;
   const float* v_norms;
@@ -59,23 +52,10 @@ struct PrefillArgs {
   float score_scale;            // attn_scale / d / key-table scale * log2(e)
 };
 
-// words / shifts of the 24 bits that hold elements 8c .. 8c+7 of a packed row (chunk 15 is all of
-// word 12: taken as word 11 >> 30, which is 0, | word 12)
-__device__ __forceinline__ void chunk_bits(int c, int& w0, int& sh_lo, int& sh_hi) {
-  w0 = (c == 15) ? 11 : (8 * c) / 10;
-  const int s0 = (c == 15) ? 10 : (8 * c) % 10;
-  sh_lo = 3 * s0;
-  sh_hi = 30 - 3 * s0;
-}
-
-__device__ __forceinline__ uint32_t chunk_field(const uint32_t* row, int w0, int sh_lo, int sh_hi) {
-  return ((row[w0] >> sh_lo) | (row[w0 + 1] << sh_hi)) & 0xFFFFFFu;
-}
-
 // grid = (n_splits, ceil(n_rows / 256), n_q), 512 threads: two wavefronts per SIMD, so that one's
 // matrix instructions overlap the other's LDS reads and softmax arithmetic.
 // Wavefront w owns query rows 32w .. 32w+31 of the workgroup's 256.  Per block of 64 key
-// positions: all threads decode the packed rows through 64-entry centroid-pair tables into LDS
+// positions: all threads decode the packed rows (BITS bits per field) through centroid-pair tables into LDS
 //   Ks[p][e]   keys, row-major, fp16
 //   Vt[e][s]   values, transposed; position p = 32b + 16h + 4g + j sits in slot s = 32b + 8g + 4h + j,
 //              the order in which the weights come out of the score accumulators
@@ -84,14 +64,19 @@ __device__ __forceinline__ uint32_t chunk_field(const uint32_t* row, int w0, int
 // cancels in the average), the online softmax on its accumulators, and O += P V with the
 // accumulator registers of S^T reused as the A operand.  The packed words of the next block are
 // fetched while the current one is computed.
+template <int BITS>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void prefill_tile_kernel(PrefillArgs a, Codebook kcb, Codebook vcb) {
+  using PF = PackedField<BITS>;
+  constexpr int kPdim = PF::kPd;                    // words per packed row
+  constexpr int kStageWords = kBlkPos * kPdim;      // packed words per block and tensor (832 at three bits)
+  constexpr int kLut = PF::kLut < 64 ? 64 : PF::kLut;
   __shared__ __align__(16) _Float16 Ks2[2][kBlkPos * kKStride];
   __shared__ __align__(16) _Float16 Vt2[2][kD * kVStride];
   __shared__ uint32_t stK2[2][kStageWords + 4], stV2[2][kStageWords + 4];
   __shared__ float stN2[2][2 * kBlkPos];                       // raw key norms, then raw value norms
   __shared__ __align__(16) float kn_s2[2][kBlkPos], vn_s2[2][kBlkPos];
-  __shared__ uint32_t lutk_s[64], lutv_s[64];
+  __shared__ uint32_t lutk_s[kLut], lutv_s[kLut];
   __shared__ __align__(16) float alpha_s[kWaves][kWaveRows];
 
   const int tid = threadIdx.x;
@@ -112,17 +97,8 @@ void prefill_tile_kernel(PrefillArgs a, Codebook kcb, Codebook vcb) {
   }
   const int64_t part = ((int64_t)split * a.n_q + head) * a.n_rows;       // first row of this (split, head) in the workspace
 
-  if (tid < 128) {
-    const int t = tid & 63;
-    float clo = 0.0f, chi = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const float ci = (tid < 64) ? kcb.c[i] : vcb.c[i];
-      clo = ((t & 7) == i) ? ci : clo;
-      chi = ((t >> 3) == i) ? ci : chi;
-    }
-    if (tid < 64) lutk_s[t] = pack_h2(clo, chi); else lutv_s[t] = pack_h2(clo, chi);
-  }
+  if (tid < 64) PF::fill(lutk_s, kcb, tid);
+  else if (tid < 128) PF::fill(lutv_s, vcb, tid - 64);
 
   // ---- query operands: B[k = element][n = row], 8 consecutive elements per lane; value and remainder
   u4 qhi[kRowTiles][4], qlo[kRowTiles][4];
@@ -155,10 +131,10 @@ void prefill_tile_kernel(PrefillArgs a, Codebook kcb, Codebook vcb) {
   const int kpos = tid >> 3, kq = tid & 7;
   int kcw[2], kcl[2], kch[2];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) chunk_bits(2 * kq + i, kcw[i], kcl[i], kch[i]);
+  for (int i = 0; i < 2; ++i) PF::pos(2 * kq + i, kcw[i], kcl[i], kch[i]);
   const int vpp = tid & 31, vc = tid >> 5;
   int vcw, vcl, vch;
-  chunk_bits(vc, vcw, vcl, vch);
+  PF::pos(vc, vcw, vcl, vch);
   // slot of the even position 2*vpp: p = 32b + 16h + 4gg + j  ->  32b + 8gg + 4h + j
   const int vp = 2 * vpp;
   const int vslot = (vp & 32) + 8 * ((vp >> 2) & 3) + 4 * ((vp >> 4) & 1) + (vp & 3);
@@ -206,25 +182,22 @@ void prefill_tile_kernel(PrefillArgs a, Codebook kcb, Codebook vcb) {
       const uint32_t* row = stK + kpos * kPdim;
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
-        const uint32_t f = chunk_field(row, kcw[i], kcl[i], kch[i]);
+        const uint32_t f = PF::field(row + kcw[i], kcl[i], kch[i]);
         u4 w;
 #pragma unroll
-        for (int jp = 0; jp < 4; ++jp) w[jp] = lutk_s[(f >> (6 * jp)) & 63u];
+        for (int jp = 0; jp < 4; ++jp) w[jp] = lutk_s[PF::index(f, jp)];
         *reinterpret_cast<u4*>(&Ks[kpos * kKStride + 8 * (2 * kq + i)]) = w;
       }
     }
     // ---- decode values: two positions x 8 elements, written transposed
     {
-      constexpr uint32_t kEven = 0x1C71C7u;
-      const uint32_t* ra = stV + vp * kPdim;
-      const uint32_t fa = chunk_field(ra, vcw, vcl, vch);
-      const uint32_t fb = chunk_field(ra + kPdim, vcw, vcl, vch);
-      const uint32_t X = (fa & kEven) | ((fb & kEven) << 3);            // elements 8c + 0, 2, 4, 6
-      const uint32_t Y = ((fa >> 3) & kEven) | (fb & (kEven << 3));     // elements 8c + 1, 3, 5, 7
+      const uint32_t* ra = stV + vp * kPdim + vcw;
+      uint32_t X, Y;                                                    // elements 8c + 0, 2, 4, 6 / 8c + 1, 3, 5, 7
+      PF::interleave(PF::field(ra, vcl, vch), PF::field(ra + kPdim, vcl, vch), X, Y);
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        *reinterpret_cast<uint32_t*>(&Vt[(8 * vc + 2 * i) * kVStride + vslot]) = lutv_s[(X >> (6 * i)) & 63u];
-        *reinterpret_cast<uint32_t*>(&Vt[(8 * vc + 2 * i + 1) * kVStride + vslot]) = lutv_s[(Y >> (6 * i)) & 63u];
+        *reinterpret_cast<uint32_t*>(&Vt[(8 * vc + 2 * i) * kVStride + vslot]) = lutv_s[PF::index(X, i)];
+        *reinterpret_cast<uint32_t*>(&Vt[(8 * vc + 2 * i + 1) * kVStride + vslot]) = lutv_s[PF::index(Y, i)];
       }
     }
   };
@@ -532,8 +505,8 @@ extern "C" int tq_prefill_attn(const void* q, int q_dtype, const uint32_t* k_pac
                                int bits, float attn_scale, int causal, tq_stream_t stream_) {
   const char* who = "tq_prefill_attn";
   if (int rc = tq::check_dim_bits(dim, bits)) return rc;
-  if (dim != kD || bits != 3)
-    return tq::fail(TQ_ERR_UNSUPPORTED, "%s: only dim 128 / 3-bit has a kernel, got dim %d bits %d", who, dim, bits);
+  if (dim != kD)
+    return tq::fail(TQ_ERR_UNSUPPORTED, "%s: only dim 128 has a kernel, got dim %d", who, dim);
   if (n_kv_heads < 1) return tq::fail(TQ_ERR_ARG, "%s: n_kv_heads must be >= 1, got %d", who, n_kv_heads);
   if (n_rep < 1) return tq::fail(TQ_ERR_NREP, "%s: n_rep must be >= 1, got %d", who, n_rep);
   if (tq::check_dtype(q_dtype) || tq::check_dtype(out_dtype)) return tq::fail(TQ_ERR_DTYPE, "%s: unknown dtype", who);
@@ -589,7 +562,7 @@ extern "C" int tq_prefill_attn(const void* q, int q_dtype, const uint32_t* k_pac
   const float v_unscale = tq::fill_codebook_fp16(vcb, v_centroids, bits);
   a.score_scale = attn_scale / (float)dim * k_unscale * kLog2e;
   dim3 grid(plan.n_splits, (unsigned)((n_rows + kWgRows - 1) / kWgRows), n_q);
-  prefill_tile_kernel<<<grid, kThreads, 0, stream>>>(a, kcb, vcb);
+  TQ_DISPATCH_BITS(bits, (prefill_tile_kernel<B_><<<grid, kThreads, 0, stream>>>(a, kcb, vcb)));
   TQ_CHECK_LAUNCH("tq_prefill_attn tile pass");
 
   const float unscale = v_unscale / kVnScale / (float)dim;

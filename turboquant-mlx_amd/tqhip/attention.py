@@ -37,7 +37,7 @@ def turboquant_attention(queries: torch.Tensor, cache, attn_scale: float, mask=N
     packed K and V; returns (B, n_heads, 1, dim) in queries.dtype.
 
     fused=True runs the whole step as one library call (pre-rotation aside) when no v_buffer is given: one
-    launch + merge without a sparse-V threshold, three passes with one (d = 128 / 3-bit / n_rep <= 16; other
+    launch + merge without a sparse-V threshold, three passes with one (d = 128 / n_rep <= 16; other
     shapes compose the separate ops); the result is the same up to summation order and operand rounding.
     """
     B, n_q, S_q, dim = queries.shape

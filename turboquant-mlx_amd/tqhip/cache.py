@@ -258,7 +258,7 @@ class TurboQuantKVCache:
                     ok = False
         if not ok:
             if position is not None:
-                raise ValueError("a step with a device-side position needs one new token, dim 128, 3-bit codes, "
+                raise ValueError("a step with a device-side position needs one new token, dim 128, "
                                  "n_rep <= 16 and contiguous storage")
             self.update_and_fetch(keys, values)
             return attention.turboquant_attention(queries, self, attn_scale, fused=True)

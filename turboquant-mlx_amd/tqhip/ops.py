@@ -543,7 +543,7 @@ def flash_decode(q_rot: torch.Tensor, k_packed, k_norms, v_packed, v_norms, k_ce
     sparse_v.py:59-65 on the final weights, as turboquant_attention applies it, fused_attention.py:109-121)
     -- tq_flash_sparse_decode, matrix-core shape only (see vonly_sparse_supported).
 
-    precision="fp16" (default): matrix-core kernels where the shape allows (d = 128, 3-bit,
+    precision="fp16" (default): matrix-core kernels where the shape allows (d = 128, any width,
     n_rep <= 16), operands rounded to half, float32 accumulation; "fp32": float32 kernels.
 
     q_rot (n_seq, n_q, dim) float32.  K/V either cache layout [n_seq, n_kv, T_alloc, *] with the
@@ -587,7 +587,7 @@ def flash_decode(q_rot: torch.Tensor, k_packed, k_norms, v_packed, v_norms, k_ce
     stream = _stream(q_rot)
     if sparse_v_threshold and sparse_v_threshold > 0.0:
         if not (vonly_sparse_supported(dim, bits, n_rep) and T > 0):
-            raise ValueError("thresholded flash decode needs dim 128, 3-bit, n_rep <= 16 and a non-empty cache; "
+            raise ValueError("thresholded flash decode needs dim 128, n_rep <= 16 and a non-empty cache; "
                              "compose prerot_fused_qk_scores, softmax_rows and sparse_v_matvec for other shapes")
         need = lib.tq_vonly_sparse_workspace_bytes(n_seq, n_q, T)
         ws = _workspace(q_rot.device, stream.value or 0, need)
@@ -620,7 +620,7 @@ def flash_decode_from_q(q: torch.Tensor, k_signs, k_packed, k_norms, v_packed, v
     n_kv = k_norms.shape[-2]
     _check_gqa(n_q, n_kv, n_rep)
     if not vonly_sparse_supported(dim, bits, n_rep):
-        raise ValueError("flash_decode_from_q needs dim 128, 3-bit, n_rep <= 16; use prerotate_query + flash_decode")
+        raise ValueError("flash_decode_from_q needs dim 128 and n_rep <= 16; use prerotate_query + flash_decode")
     pd = packed_dim(dim, bits)
     if q.dtype not in _DTYPES:
         q = q.float()
@@ -673,8 +673,8 @@ def flash_attention_turboquant(q_rot, k_packed, k_norms, v_packed, v_norms, k_ce
 
 def vonly_sparse_supported(dim: int, bits: int, n_rep: int) -> bool:
     """Shapes the one-call steps over PACKED keys cover (the matrix-core kernels: flash decode from the raw query,
-    its thresholded form, the packed cache's decode_step)."""
-    return dim == 128 and bits == 3 and 1 <= n_rep <= 16
+    its thresholded form, the packed cache's decode_step): d = 128 at every width."""
+    return dim == 128 and 1 <= bits <= 4 and 1 <= n_rep <= 16
 
 
 def vonly_threshold_supported(dim: int, bits: int, n_rep: int) -> bool:
