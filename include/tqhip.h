@@ -143,7 +143,7 @@ int tq_prerotate_query(const void* q, int q_dtype, const float* signs, float* q_
  *   scores [n_kv*n_rep, seq_len] f32 contiguous.
  * allow_mma = 0: float32 arithmetic throughout (the reference's numerics); 1: q_rot and the
  * centroids are rounded to fp16 and multiplied on the matrix cores with float32 accumulation
- * (about 3e-4 relative per score) where the shape allows (d = 128, 3-bit, n_rep <= 16).
+ * (about 3e-4 relative per score) where the shape allows (d = 128, any width, n_rep <= 16).
  */
 int tq_prerot_qk_scores(const float* q_rot, const uint32_t* k_packed, const float* k_norms,
                         const float* centroids, float* scores,
@@ -216,8 +216,8 @@ typedef struct tq_decode_shape {
   float attn_scale;
   int32_t out_dtype;         /* TQ_F32, TQ_F16 or TQ_BF16 */
   int32_t allow_mma;         /* 1: use the fp16 matrix-core kernels where the shape allows (d = 128,
-                                n_rep <= 16; 3-bit keys and values for packed keys, values of any width
-                                1-4 beside fp16 keys; operands rounded to fp16, float32 accumulation);
+                                n_rep <= 16, every width 1-4; operands rounded to fp16, float32
+                                accumulation);
                                 0: float32 vector-ALU kernels only */
 } tq_decode_shape;
 
@@ -373,7 +373,7 @@ typedef struct tq_packed_cache_desc {
  * bit-identical to tq_encode's, output equal to the separate calls up to the rounding of one score).
  * Replaces, for a single-token step, TurboQuantKVCache.update_and_fetch (cache.py:131-165) followed
  * by turboquant_attention (fused_attention.py:20-125).  Shapes and errors as tq_vonly_decode_step;
- * TQ_ERR_UNSUPPORTED where tq_flash_decode_from_q has no kernel (it needs dim 128, 3 bits, n_rep <= 16).
+ * TQ_ERR_UNSUPPORTED where tq_flash_decode_from_q has no kernel (it needs dim 128 and n_rep <= 16).
  */
 int tq_packed_decode_step(const tq_packed_cache_desc* cache /* host */,
                           const void* k_new, int k_dtype, const void* v_new, int v_dtype,
@@ -444,7 +444,7 @@ int tq_flash_sparse_decode(const float* q_rot,
  * of tq_prerotate_query done inside the kernels (same bits), which saves the separate launch and the q_rot
  * tensor.  q [n_seq, n_kv*n_rep, dim] of q_dtype; k_signs [dim] f32 on the device.  Workspace:
  * tq_workspace_bytes(TQ_OP_FLASH_DECODE, ...) for threshold == 0, tq_vonly_sparse_workspace_bytes otherwise.
- * Matrix-core shape only (dim 128, 3-bit, n_rep <= 16, non-empty cache; TQ_ERR_UNSUPPORTED otherwise: call
+ * Matrix-core shape only (dim 128, n_rep <= 16, non-empty cache; TQ_ERR_UNSUPPORTED otherwise: call
  * tq_prerotate_query and tq_flash_decode).
  */
 int tq_flash_decode_from_q(const void* q, int q_dtype, const float* k_signs,
@@ -473,7 +473,7 @@ size_t tq_workspace_bytes(int op, int n_seq, int n_q_heads, int64_t max_seq_len,
  *   k_packed / v_packed [n_kv, *_head_stride rows, pdim], k_norms / v_norms [n_kv, *_head_stride]
  *   out [n_kv*n_rep, n_rows, dim] out_dtype, contiguous
  * Matrix-core kernel: q_rot, the centroids and softmax weights * value norm are fp16 operands,
- * accumulation is float32.  dim 128 / 3-bit only (TQ_ERR_UNSUPPORTED otherwise).  The workspace
+ * accumulation is float32.  dim 128 only, every width (TQ_ERR_UNSUPPORTED otherwise).  The workspace
  * (tq_prefill_workspace_bytes, 256-byte aligned) is scratch as for the decode ops.
  */
 int tq_prefill_attn(const void* q, int q_dtype,

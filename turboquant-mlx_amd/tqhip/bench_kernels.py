@@ -6,7 +6,7 @@ back-to-back launches, and rotation over several independent input sets so that 
 Infinity Cache cannot serve the reads.  Prints one line per case: us per call, GB/s of algorithmic
 bytes and the fraction of 8 TB/s.
 
-    python -m tqhip.bench_kernels [--iters 200] [--cases encode,scores,flash,flash_long,sparse_v,vonly,widths,codec_widths,prefill,step]
+    python -m tqhip.bench_kernels [--iters 200] [--cases encode,scores,flash,flash_long,sparse_v,vonly,widths,packed_widths,codec_widths,prefill,step]
 """
 from __future__ import annotations
 
@@ -217,6 +217,47 @@ def bench_widths(iters, dev):
                 report(f"V-only decode 28/4 heads, {bits}-bit values, T={T}, {kind} (graph)", timeit_graph(fns, iters), nbytes)
 
 
+def bench_packed_widths(iters, dev):
+    """The steps over PACKED keys at every width (32/8 heads): scores, flash decode (single sequence, HIP-graph
+    replay) and a 512-row prefill chunk, matrix cores against the float32 kernels (none for prefill)."""
+    ks_ = tqhip.random_diagonal_sign(128, 42, device=dev)
+    vs_ = tqhip.random_diagonal_sign(128, 43, device=dev)
+    g = torch.Generator(device=dev)
+    g.manual_seed(9)
+    sc = 1 / math.sqrt(128)
+    for bits in (1, 2, 3, 4):
+        cb = gaussian_codebook(bits)
+        pd = tqhip.packed_dim(128, bits)
+        row = 4 * pd + 4
+        for T in (32768, 131072):
+            n_sets = n_sets_for(2 * 8 * T * row)
+
+            def packed():
+                codes = torch.randint(0, 2 ** bits, (8 * T, 128), generator=g, device=dev, dtype=torch.uint8)
+                return tqhip.pack_indices(codes, bits).reshape(8, T, pd), torch.rand((8, T), generator=g, device=dev) + 0.5
+            sets = [(packed(), packed()) for _ in range(n_sets)]
+            q_rot = torch.randn((1, 32, 128), device=dev)
+            for prec in ("fp16", "fp32"):
+                kind = "matrix cores" if prec == "fp16" else "float32 kernels"
+                fns = [(lambda k=k: tqhip.prerot_fused_qk_scores(q_rot[0], k[0], k[1], cb, 128, bits, n_rep=4, precision=prec))
+                       for k, _ in sets]
+                report(f"scores 32/8 heads, {bits}-bit keys, T={T}, {kind} (graph)", timeit_graph(fns, iters),
+                       8 * T * row + 32 * T * 4)
+                fns = [(lambda k=k, v=v: tqhip.flash_decode(q_rot, k[0][None], k[1][None], v[0][None], v[1][None], cb, cb, vs_,
+                                                            128, bits, sc, n_rep=4, seq_len=T, precision=prec))
+                       for k, v in sets]
+                report(f"flash decode 32/8 heads, {bits}-bit, T={T}, {kind} (graph)", timeit_graph(fns, iters), 2 * 8 * T * row)
+        T, n_rows = 32768, 512
+        (kp, kn), (vp, vn) = sets[0][0], sets[0][1]
+        kp, kn, vp, vn = kp[:, :T], kn[:, :T], vp[:, :T], vn[:, :T]
+        q = torch.randn((32, n_rows, 128), device=dev, dtype=torch.float16)
+        us = timeit([lambda: tqhip.prefill_attention(q, kp, kn, vp, vn, cb, cb, ks_, vs_, 128, bits, sc, n_rep=4)],
+                    max(5, iters // 20), warmup=2)
+        flops = 4.0 * 32 * 128 * sum(T - n_rows + i + 1 for i in range(n_rows))
+        print(f"prefill chunk 512 rows x 32/8 heads, {bits}-bit, T={T:<7d} {us:10.1f} us  {flops / us / 1e6:8.1f} TFLOP/s  "
+              f"{100 * flops / us / 1e6 / 2500:5.1f} % of 2.5 PFLOP/s", flush=True)
+
+
 def bench_codec_widths(iters, dev):
     """Encode / dequantise 1 048 576 vectors at every width: the streaming kernels (row count a multiple of 16)
     against the generic one-wavefront-per-vector kernels (one row fewer)."""
@@ -329,7 +370,8 @@ def bench_step(iters, dev):
 
 
 CASES = {"step": bench_step, "prefill": bench_prefill, "encode": bench_encode, "scores": bench_scores, "sparse_v": bench_sparse_v, "flash": bench_flash,
-         "flash_long": bench_flash_long, "vonly": bench_vonly, "widths": bench_widths, "codec_widths": bench_codec_widths}
+         "flash_long": bench_flash_long, "vonly": bench_vonly, "widths": bench_widths, "codec_widths": bench_codec_widths,
+         "packed_widths": bench_packed_widths}
 
 
 def main():
