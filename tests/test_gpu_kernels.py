@@ -1729,6 +1729,40 @@ def test_vonly_streaming_pass_with_a_ragged_end(tq, n_seq, n_kv, n_rep, T, qdt):
         close(got[i], want, rel=(1e-2 if qdt == "bfloat16" else REL), abs_=(4e-3 if qdt == "bfloat16" else ABS), row_scale=True)
 
 
+@pytest.mark.parametrize("qdt", ["float16", "float32", "bfloat16"])
+@pytest.mark.parametrize("n_kv,n_rep,lens", [
+    (4, 7, [4097, 2561, 1025, 7000, 1, 3333, 5121, 6143]),       # every row misalignment; ends inside a step, a wave, a block
+    (2, 16, [33000, 511, 512, 513, 20000]),                       # a sequence past 32 768 beside ones around one block
+    (8, 1, [9000, 1, 1, 8193])])
+def test_vonly_streaming_pass_over_a_ragged_batch(tq, qdt, n_kv, n_rep, lens):
+    """An unmasked ragged batch long enough for the streaming pass: sequences start at arbitrary rows (packed rows of
+    52 bytes at every multiple of 4 bytes), workgroups past a sequence's end leave at once, the last workgroup of a
+    sequence runs through fewer blocks.  Exactly sum(L) rows are stored: nothing may be read past the end.  Each
+    sequence against the oracle; and the same batch with an all-zero mask (the single-tile kernels) to the bar."""
+    rng = np.random.default_rng(len(lens) * 1000 + n_kv)
+    D, bits, sc = 128, 3, 1 / math.sqrt(128)
+    lens = np.asarray(lens)
+    n_seq = len(lens)
+    offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    tot = int(offs[-1])
+    c, b = tables(bits)
+    vs = o.random_diagonal_sign(D, 43)
+    K = rng.standard_normal((n_kv, tot, D)).astype(np.float16)
+    vp = o.pack_indices(rng.integers(0, 8, size=(n_kv, tot, D)).astype(np.uint8), bits)
+    vn = ((rng.random((n_kv, tot)) + 0.5) * np.exp(rng.uniform(-3, 3, size=(n_kv, tot)))).astype(F32)
+    q = torch.from_numpy(rng.standard_normal((n_seq, n_kv * n_rep, D)).astype(F32)).to(getattr(torch, qdt))
+    kw = dict(n_rep=n_rep, seq_offsets=dev(offs), max_seq_len=int(lens.max()))
+    got = host(tq.vonly_decode(q.cuda(), dev(K), dev(vp), dev(vn), c, dev(vs), D, bits, sc, **kw).float())
+    rel, ab = (1e-2, 4e-3) if qdt == "bfloat16" else (REL, ABS)
+    for i in range(n_seq):
+        a, e = offs[i], offs[i + 1]
+        want = o.vonly_decode_attention(q[i].float().numpy(), K[:, a:e], vp[:, a:e], vn[:, a:e], c, vs, D, bits, sc)
+        close(got[i], want, rel=rel, abs_=ab, row_scale=True)
+    zero = torch.zeros((n_seq, 1, int(lens.max())), device="cuda")
+    tiles = host(tq.vonly_decode(q.cuda(), dev(K), dev(vp), dev(vn), c, dev(vs), D, bits, sc, mask=zero, **kw).float())
+    close(got, tiles, rel=rel, abs_=ab, row_scale=True)
+
+
 def test_attended_length_beyond_the_tensors_is_refused(tq):
     """The kernels trust seq_len / kv_len: the wrappers refuse a length that the K/V tensors do not hold."""
     rng = np.random.default_rng(12)

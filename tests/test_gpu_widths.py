@@ -115,6 +115,35 @@ def test_vonly_decode_other_widths_ragged_batch_and_mask(tq, bits):
 
 
 @pytest.mark.parametrize("bits", [1, 2, 4])
+def test_vonly_streaming_pass_other_widths_over_a_ragged_batch(tq, bits):
+    """An unmasked ragged batch long enough for the streaming pass (rows of 16, 32 or 64 bytes: always aligned);
+    and from storage 4 bytes off alignment, which goes to the single-tile kernels."""
+    rng = np.random.default_rng(330 + bits)
+    n_kv, n_rep = 4, 7
+    sc = 1 / math.sqrt(D)
+    lens = np.array([4097, 2561, 1025, 7000, 1, 3333, 5121, 6143])
+    n_seq = len(lens)
+    offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    tot = int(offs[-1])
+    c = o.gaussian_codebook(bits)
+    vs = o.random_diagonal_sign(D, 43)
+    K = rng.standard_normal((n_kv, tot, D)).astype(np.float16)
+    vp = o.pack_indices(rng.integers(0, 1 << bits, size=(n_kv, tot, D)).astype(np.uint8), bits)
+    vn = ((rng.random((n_kv, tot)) + 0.5) * np.exp(rng.uniform(-2, 2, size=(n_kv, tot)))).astype(F32)
+    q = rng.standard_normal((n_seq, n_kv * n_rep, D)).astype(np.float16)
+    kw = dict(n_rep=n_rep, seq_offsets=dev(offs), max_seq_len=int(lens.max()))
+    got = host(tq.vonly_decode(dev(q), dev(K), dev(vp), dev(vn), c, dev(vs), D, bits, sc, **kw))
+    for i in range(n_seq):
+        a, e = offs[i], offs[i + 1]
+        close(got[i], o.vonly_decode_attention(q[i], K[:, a:e], vp[:, a:e], vn[:, a:e], c, vs, D, bits, sc))
+    flat = torch.zeros(vp.size + 4, dtype=torch.int32, device="cuda")
+    shifted = flat[1:1 + vp.size].view(torch.uint32).reshape(vp.shape)
+    shifted.copy_(dev(vp))
+    assert shifted.data_ptr() % 16 == 4
+    close(host(tq.vonly_decode(dev(q), dev(K), shifted, dev(vn), c, dev(vs), D, bits, sc, **kw)), got)
+
+
+@pytest.mark.parametrize("bits", [1, 2, 4])
 def test_vonly_decode_other_widths_masked_eight_wave_tiles(tq, bits):
     """20 000 masked positions of 4 kv heads: 160 tiles of 512, the eight-wave shape with the mask reads."""
     rng = np.random.default_rng(325 + bits)

@@ -763,12 +763,35 @@ int launch_vonly_mfma(const void* q, int q_dtype, const void* k_f16, const uint3
     }
     ragged_stream = true;
   }
+  // Ragged batches (unmasked): the streaming pass as well, once the longest sequence alone would give every CU three
+  // four-wave tiles.  True lengths are not known here, so at most 4 blocks per workgroup (a short tail), the count
+  // with the fewest rounds for the longest sequence.  Three-bit rows start at any multiple of 4 bytes; rows of the
+  // other widths are multiples of 16 bytes and need a 16-byte aligned tensor.
+  const bool ragged_batch = sh.seq_offsets && !sh.mask && !len_dev && sh.attn_scale > 0.0f &&
+                            (sh.bits == 3 || tq::aligned(v_packed, 16));
+  if (ragged_batch && wgs4 > 768) {
+    const int64_t blocks = (sh.seq_len + tqm::kTilePos - 1) / tqm::kTilePos;
+    int64_t best_cost = INT64_MAX;
+    for (int nb = 2; nb <= 4; ++nb) {
+      const int64_t wgs = ((blocks + nb - 1) / nb) * sh.n_kv_heads * sh.n_seq;
+      const int64_t cost = ((wgs + 255) / 256) * nb;
+      if (cost <= best_cost) { best_cost = cost; n_blocks = nb; }         // ties: fewer workgroups, fewer set-ups
+    }
+    ragged_stream = true;
+  }
   // One tile per workgroup, as measured over lengths from 4 096 to 65 537 (28/4 heads): eight-wave workgroups
   // (512 positions, one per CU) are the faster shape when they fill between half and all of the CUs in one round;
   // four-wave workgroups (256 positions, up to three per CU) fill more CUs on short caches and, from 257 to 768
   // of them, avoid the nearly empty second round of the eight-wave shape; beyond that the eight-wave shape again.
   int nw = 8;
   if (n_blocks == 1 && (wgs8 <= 128 || (wgs8 > 256 && wgs4 <= 768))) nw = 4;
+  // The streaming pass in more than one round of eight-wave workgroups: four-wave workgroups over the same ranges
+  // (twice the blocks of half the size), two to a CU, so that the set-up and the merge of one run under the steps of
+  // the other.
+  if (n_blocks > 1) {
+    const int64_t blocks = (sh.seq_len + tqm::kTilePos - 1) / tqm::kTilePos;
+    if (((blocks + n_blocks - 1) / n_blocks) * sh.n_kv_heads * sh.n_seq > 256) { nw = 4; n_blocks *= 2; }
+  }
   const int tile_pos = nw * tqm::kWavePos * n_blocks;
   const int n_tiles_real = (int)((sh.seq_len + tile_pos - 1) / tile_pos);     // 0: an empty cache, merge pass only
   const int n_tiles = n_tiles_real > 0 ? n_tiles_real : 1;

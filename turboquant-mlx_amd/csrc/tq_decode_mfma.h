@@ -683,21 +683,32 @@ __global__ __launch_bounds__(WAVES * 64) void vonly_scores_kernel(MfmaArgs a) {
 // through fewer blocks, loads of rows past the end are redirected to valid rows (norms and K rows to the last
 // valid row, packed-V pieces with no valid byte to the first piece of the last partly valid step; an aligned
 // 16-byte piece that holds a valid byte never crosses a page) and the scores of those rows are set to -inf.
+// RAGGED also serves ragged batches (seq_offsets): a sequence starts at any row, so its packed three-bit rows of
+// 52 bytes start at any multiple of 4 bytes; every step's 32 rows are 104 pieces, hence ONE misalignment per
+// sequence: pieces are fetched from the 16-byte boundary at or below the step's first row (105 of them) and the
+// rows are read from the wave's LDS image at that offset.  Workgroups past a sequence's end leave at once.
 constexpr int kStepPos = 32;
 
-template <bool QF32, bool RAGGED, int BITS = 3>
-__global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
-void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
+// MODE 0: every range is whole and starts 16-byte aligned (no offsets); 1: the general ragged body (per-row checks);
+// 2: a whole range of a ragged launch (rows may start misaligned, no per-row checks).
+// NW waves per workgroup (a block is NW * 64 positions): 8 where one round of workgroups covers the launch, 4
+// where there are several, so that two workgroups share a CU and the set-up of one runs under the steps of the other.
+template <bool QF32, int MODE, int BITS, int NW>
+__device__ __forceinline__ void vonly_stream_body(const MfmaArgs& a, const Codebook& vcb, int n_blocks, int64_t first, int64_t len) {
   using VF = VField<BITS>;
+  constexpr bool RAGGED = MODE == 1;                     // per-row checks
+  constexpr bool MISALIGNED = MODE != 0 && BITS == 3;    // rows may start at any multiple of 4 bytes
   constexpr int kPd = VF::kPd;                           // words per packed value row
-  constexpr int kPieces = 8 * kPd;                       // 16-byte pieces of a step's 32 packed rows: 104 at three bits
-  __shared__ __align__(16) unsigned char big_s[32768];
+  constexpr int kBlk = NW * kWavePos;                    // positions of a block
+  constexpr int kThr = NW * 64;
+  constexpr int kPieces = 8 * kPd + (MISALIGNED ? 1 : 0);   // 16-byte pieces of a step's 32 packed rows: 104 at three bits (+ 1 misaligned)
+  __shared__ __align__(16) unsigned char big_s[NW * 4096];
   __shared__ uint32_t lut_s[VF::kLut < 64 ? 64 : VF::kLut];
   __shared__ __align__(16) uint32_t q_s[kHeadsMax][kD / 2];
   __shared__ __align__(16) uint32_t ql_s[QF32 ? kHeadsMax : 1][kD / 2];
-  __shared__ __align__(16) float nrm_s[kWaves][kStepPos];
-  __shared__ __align__(16) float alpha_s[kWaves][kHeadsMax];
-  __shared__ __align__(16) MergeLds<kWaves> mg_s;
+  __shared__ __align__(16) float nrm_s[NW][kStepPos];
+  __shared__ __align__(16) float alpha_s[NW][kHeadsMax];
+  __shared__ __align__(16) MergeLds<NW> mg_s;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -706,25 +717,30 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
   const int n_rep = a.n_rep;
   const int n_q = a.n_kv * n_rep;
   const int64_t q_row0 = (int64_t)seq * n_q + (int64_t)kvh * n_rep;
-  const int64_t tile_p0 = (int64_t)tile * kTilePos * n_blocks;
+  const int64_t tile_p0 = (int64_t)tile * kBlk * n_blocks;
   // positions of this workgroup's range that exist (RAGGED: the last workgroup has fewer)
-  const int valid = RAGGED ? (int)min((int64_t)kTilePos * n_blocks, a.seq_len - tile_p0) : kTilePos * n_blocks;
-  const int n_steps = RAGGED ? 2 * ((valid + kTilePos - 1) / kTilePos) : 2 * n_blocks;
+  const int valid = RAGGED ? (int)min((int64_t)kBlk * n_blocks, len - tile_p0) : kBlk * n_blocks;
+  const int n_steps = RAGGED ? 2 * ((valid + kBlk - 1) / kBlk) : 2 * n_blocks;
   const int last_valid = valid - 1;
   const int last_step_row = last_valid & ~(kStepPos - 1);               // first row of the last partly valid step
 
   // row of step s inside the workgroup's range: block s/2, this wave's 64 rows, half s%2
-  auto step_row = [&](int s) { return (s >> 1) * kTilePos + wave * kWavePos + (s & 1) * kStepPos; };
-  const float* nbase = a.v_norms + (int64_t)seq * a.vn_seq_stride + (int64_t)kvh * a.vn_head_stride + tile_p0 +
-                       (RAGGED ? 0 : (lane & 31));
-  const char* vbase = reinterpret_cast<const char*>(
-      a.v_packed + ((int64_t)seq * a.v_seq_stride + (int64_t)kvh * a.v_head_stride + tile_p0) * kPd);
+  auto step_row = [&](int s) { return (s >> 1) * kBlk + wave * kWavePos + (s & 1) * kStepPos; };
+  const float* nbase = a.v_norms + (int64_t)seq * a.vn_seq_stride + (int64_t)kvh * a.vn_head_stride + first + tile_p0;
+  const float* nbase_l = nbase + (lane & 31);
+  const char* vrow0 = reinterpret_cast<const char*>(
+      a.v_packed + ((int64_t)seq * a.v_seq_stride + (int64_t)kvh * a.v_head_stride + first + tile_p0) * kPd);
+  // bytes between the 16-byte boundary below the range's first row and that row (uniform; 0 unless RAGGED at three bits)
+  const int vmis = MISALIGNED ? (int)(reinterpret_cast<uintptr_t>(vrow0) & 15) : 0;
+  const char* vbase = vrow0 - vmis;
   const char* kbase = reinterpret_cast<const char*>(
-      a.k + ((int64_t)seq * a.k_seq_stride + (int64_t)kvh * a.k_head_stride + tile_p0) * kD);
+      a.k + ((int64_t)seq * a.k_seq_stride + (int64_t)kvh * a.k_head_stride + first + tile_p0) * kD);
   // pieces lane and 64 + lane of a step's block (the second load only where a block has more than 64 pieces);
   // lanes past the last piece repeat an earlier one
   const uint32_t voff0 = (uint32_t)((kPieces >= 64 ? lane : (lane & (kPieces - 1))) * 16);
   const uint32_t voff1 = (uint32_t)((64 + lane < kPieces ? 64 + lane : kPieces - 1) * 16);
+  // the same for a full range: the extra piece of a misaligned step exists only where it holds a valid byte
+  const uint32_t voff1_full = (MISALIGNED && voff1 >= (uint32_t)(8 * kPd * 16) && vmis == 0) ? 0u : voff1;
   const uint32_t koff_even = (uint32_t)(((lane >> 4) * 16 + ((lane & 15) ^ ((lane >> 4) & 7))) * 16);
   const uint32_t koff_odd = (uint32_t)(((4 + (lane >> 4)) * 16 + ((lane & 15) ^ ((4 + (lane >> 4)) & 7))) * 16);
   auto issue_nv = [&](int s, float& nrm, u4 (&vqx)[2]) {
@@ -732,15 +748,15 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
     if (RAGGED) {
       nrm = nbase[min(r + (lane & 31), last_valid)];
       const int rc = min(r, last_step_row);                             // a step with no valid row re-reads the last one that has
-      const uint32_t limit = (uint32_t)((valid - rc) * (kPd * 4));       // bytes of valid rows from rc on (> 0)
+      const uint32_t limit = (uint32_t)(vmis + (valid - rc) * (kPd * 4));   // bytes from the piece boundary to the end of the valid rows (> 0)
       const char* vb = vbase + (int64_t)rc * (kPd * 4);
       vqx[0] = *reinterpret_cast<const u4*>(vb + (voff0 < limit ? voff0 : 0u));
       if (kPieces > 64) vqx[1] = *reinterpret_cast<const u4*>(vb + (voff1 < limit ? voff1 : 0u));
     } else {
-      nrm = nbase[r];
+      nrm = nbase_l[r];
       const char* vb = vbase + (int64_t)r * (kPd * 4);
       vqx[0] = *reinterpret_cast<const u4*>(vb + voff0);
-      if (kPieces > 64) vqx[1] = *reinterpret_cast<const u4*>(vb + voff1);
+      if (kPieces > 64) vqx[1] = *reinterpret_cast<const u4*>(vb + voff1_full);
     }
   };
   auto issue_k4 = [&](int s, u4 (&kx)[8], int part) {     // instructions 4*part .. 4*part+3: rows 16*part .. +15 of the step
@@ -761,10 +777,12 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
     }
   };
 
-  uint32_t my_q[2], my_ql[2] = {0u, 0u};
+  constexpr int kQIt = kHeadsMax * (kD / 2) / kThr;      // words of the staged queries per thread
+  uint32_t my_q[kQIt], my_ql[kQIt];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int w = tid + i * kMfmaThreads;
+  for (int i = 0; i < kQIt; ++i) {
+    my_ql[i] = 0u;
+    const int w = tid + i * kThr;
     if (QF32) {
       const float2 f = (w < n_rep * (kD / 2)) ? reinterpret_cast<const float2*>(reinterpret_cast<const float*>(a.q) + q_row0 * kD)[w]
                                               : make_float2(0.f, 0.f);
@@ -788,12 +806,12 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
 
   if (tid < 64) VF::fill(lut_s, vcb, tid);
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < kQIt; ++i) {
     // bf16 queries become fp16 here, after every load of the pass has been requested: converting where the word
     // is loaded would wait for it before anything else is in flight
     if (!QF32 && a.q_bf16) my_q[i] = pack_h2(__uint_as_float(my_q[i] << 16), __uint_as_float(my_q[i] & 0xFFFF0000u));
-    (&q_s[0][0])[tid + i * kMfmaThreads] = my_q[i];
-    if (QF32) (&ql_s[0][0])[tid + i * kMfmaThreads] = my_ql[i];
+    (&q_s[0][0])[tid + i * kThr] = my_q[i];
+    if (QF32) (&ql_s[0][0])[tid + i * kThr] = my_ql[i];
   }
   __syncthreads();
 
@@ -845,7 +863,7 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
 #pragma unroll
     for (int qd = 0; qd < 4; ++qd) {
       const int t = qd >> 1, jp = qd & 1;
-      const uint32_t* ra = stage + (16 * t + 4 * g + 2 * jp) * kPd + w0;
+      const uint32_t* ra = stage + (vmis >> 2) + (16 * t + 4 * g + 2 * jp) * kPd + w0;
       VF::interleave(VF::field(ra, sh_lo, sh_hi), VF::field(ra + kPd, sh_lo, sh_hi), X[qd], Y[qd]);
     }
     u4 breg[8];
@@ -948,7 +966,26 @@ void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
   const int64_t grp = (int64_t)seq * a.n_kv + kvh;
   float* pS = a.ws_S + (grp * a.n_tiles_max + tile) * (int64_t)(n_rep * kD);
   float* pml = a.ws_ml + (grp * a.n_tiles_max + tile) * (int64_t)(n_rep * 2);
-  merge_waves<kWaves>(mg_s, big_s, 4096, accS, m_run, l, inv_tscale, a.v_unscale, n_rep, pS, pml);
+  merge_waves<NW>(mg_s, big_s, 4096, accS, m_run, l, inv_tscale, a.v_unscale, n_rep, pS, pml);
+}
+
+template <bool QF32, bool RAGGED, int BITS = 3, int NW = 8>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void vonly_stream_kernel(MfmaArgs a, Codebook vcb, int n_blocks) {
+  if (!RAGGED) {
+    vonly_stream_body<QF32, 0, BITS, NW>(a, vcb, n_blocks, 0, a.seq_len);
+    return;
+  }
+  int64_t first = 0, len = a.seq_len;
+  if (a.seq_offsets) {
+    first = a.seq_offsets[blockIdx.z];
+    len = (int64_t)a.seq_offsets[blockIdx.z + 1] - first;
+  }
+  const int64_t range = (int64_t)(NW * kWavePos) * n_blocks;
+  const int64_t tile_p0 = (int64_t)blockIdx.x * range;
+  if (tile_p0 >= len) return;                             // uniform over the workgroup, ahead of every barrier
+  if (tile_p0 + range <= len) vonly_stream_body<QF32, 2, BITS, NW>(a, vcb, n_blocks, first, len);
+  else vonly_stream_body<QF32, 1, BITS, NW>(a, vcb, n_blocks, first, len);
 }
 
 // The token a decode step inserts, handled by the merge pass instead of a launch of its own ahead of the
@@ -1242,7 +1279,7 @@ __global__ __launch_bounds__(kMergeThreads + 64) void decode_merge_fresh_kernel(
 
 // Which tile kernel a launch uses (chosen by the host from the length, the mask / offsets and the alignment).
 struct VonlyTileChoice {
-  int nw;                     // waves per workgroup of the single-tile shapes: 8 or 4
+  int nw;                     // waves per workgroup: 8 or 4
   int n_blocks;               // > 1: streaming pass, that many 512-position blocks per workgroup
   bool ragged_stream;         // the streaming pass with a ragged end
   bool plain;                 // full 512-position tiles, no mask, no offsets
@@ -1256,8 +1293,10 @@ struct VonlyTileChoice {
 template <int BITS>
 void launch_vonly_tiles(dim3 grid, const VonlyTileChoice& c, const MfmaArgs& a, const Codebook& vcb, hipStream_t stream) {
 #define TQ_LAUNCH_TILE(QF)                                                                                              \
-  if (c.n_blocks > 1 && c.ragged_stream) vonly_stream_kernel<QF, true, BITS><<<grid, kMfmaThreads, 0, stream>>>(a, vcb, c.n_blocks); \
-  else if (c.n_blocks > 1) vonly_stream_kernel<QF, false, BITS><<<grid, kMfmaThreads, 0, stream>>>(a, vcb, c.n_blocks);  \
+  if (c.n_blocks > 1 && c.ragged_stream && c.nw == 4) vonly_stream_kernel<QF, true, BITS, 4><<<grid, 256, 0, stream>>>(a, vcb, c.n_blocks); \
+  else if (c.n_blocks > 1 && c.ragged_stream) vonly_stream_kernel<QF, true, BITS, 8><<<grid, 512, 0, stream>>>(a, vcb, c.n_blocks); \
+  else if (c.n_blocks > 1 && c.nw == 4) vonly_stream_kernel<QF, false, BITS, 4><<<grid, 256, 0, stream>>>(a, vcb, c.n_blocks);  \
+  else if (c.n_blocks > 1) vonly_stream_kernel<QF, false, BITS, 8><<<grid, 512, 0, stream>>>(a, vcb, c.n_blocks);  \
   else if (c.nw == 8 && c.plain) vonly_tile_mfma_kernel<true, QF, 8, BITS><<<grid, 512, 0, stream>>>(a, vcb);           \
   else if (c.nw == 8 && c.plain_any) vonly_tile_anylen_kernel<QF, 8, BITS><<<grid, 512, 0, stream>>>(a, vcb);           \
   else if (c.nw == 8) vonly_tile_mfma_kernel<false, QF, 8, BITS><<<grid, 512, 0, stream>>>(a, vcb);                     \

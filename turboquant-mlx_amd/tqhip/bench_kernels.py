@@ -6,12 +6,14 @@ back-to-back launches, and rotation over several independent input sets so that 
 Infinity Cache cannot serve the reads.  Prints one line per case: us per call, GB/s of algorithmic
 bytes and the fraction of 8 TB/s.
 
-    python -m tqhip.bench_kernels [--iters 200] [--cases encode,scores,flash,flash_long,sparse_v,vonly,widths,packed_widths,codec_widths,prefill,step]
+    python -m tqhip.bench_kernels [--iters 200] [--cases encode,scores,flash,flash_long,sparse_v,vonly,vonly_batch,widths,packed_widths,codec_widths,prefill,step]
 """
 from __future__ import annotations
 
 import argparse
 import math
+
+import numpy as np
 
 import torch
 
@@ -217,6 +219,42 @@ def bench_widths(iters, dev):
                 report(f"V-only decode 28/4 heads, {bits}-bit values, T={T}, {kind} (graph)", timeit_graph(fns, iters), nbytes)
 
 
+def bench_vonly_batch(iters, dev):
+    """V-only decode over batches (28/4 heads, 3-bit values, HIP-graph replay): cache layout with one length, and
+    ragged batches (seq_offsets) with lengths drawn uniformly from a range, as a serving loop holds them."""
+    cb = gaussian_codebook(3)
+    signs = tqhip.random_diagonal_sign(128, 43, device=dev)
+    g = torch.Generator(device=dev)
+    g.manual_seed(11)
+    sc = 1 / math.sqrt(128)
+
+    def make(shape):
+        n = int(np.prod(shape))
+        K = torch.randn(shape + (128,), device=dev, dtype=torch.float16)
+        codes = torch.randint(0, 8, (n, 128), generator=g, device=dev, dtype=torch.uint8)
+        return K, tqhip.pack_indices(codes, 3).reshape(*shape, 13), torch.rand(shape, generator=g, device=dev) + 0.5
+
+    for n_seq, T in ((16, 8192), (16, 16384), (8, 32768), (64, 2048)):
+        nbytes = n_seq * 4 * T * 312
+        sets = [make((n_seq, 4, T)) for _ in range(n_sets_for(nbytes))]
+        q = torch.randn((n_seq, 28, 128), device=dev, dtype=torch.float16)
+        fns = [(lambda K=K, p=p, n=n: tqhip.vonly_decode(q, K, p, n, cb, signs, 128, 3, sc, n_rep=7, seq_len=T)) for K, p, n in sets]
+        report(f"V-only decode 28/4 heads, {n_seq} sequences x {T} (graph)", timeit_graph(fns, iters), nbytes)
+        del sets
+    for seed, n_seq, lo, hi in ((4, 16, 4096, 32768), (5, 32, 1024, 8192), (6, 8, 16384, 65536), (7, 64, 256, 4096)):
+        lens = np.random.default_rng(seed).integers(lo, hi + 1, size=n_seq)
+        offs = torch.tensor(np.concatenate([[0], np.cumsum(lens)]), dtype=torch.int32, device=dev)
+        tot = int(lens.sum())
+        nbytes = tot * 4 * 312
+        sets = [make((4, tot)) for _ in range(n_sets_for(nbytes))]
+        q = torch.randn((n_seq, 28, 128), device=dev, dtype=torch.float16)
+        fns = [(lambda K=K, p=p, n=n: tqhip.vonly_decode(q, K, p, n, cb, signs, 128, 3, sc, n_rep=7, seq_offsets=offs,
+                                                         max_seq_len=int(lens.max()))) for K, p, n in sets]
+        report(f"V-only decode 28/4 heads, ragged batch of {n_seq}, L ~ U({lo}, {hi}), sum L={tot} (graph)",
+               timeit_graph(fns, iters), nbytes)
+        del sets
+
+
 def bench_packed_widths(iters, dev):
     """The steps over PACKED keys at every width (32/8 heads): scores, flash decode (single sequence, HIP-graph
     replay) and a 512-row prefill chunk, matrix cores against the float32 kernels (none for prefill)."""
@@ -371,7 +409,7 @@ def bench_step(iters, dev):
 
 CASES = {"step": bench_step, "prefill": bench_prefill, "encode": bench_encode, "scores": bench_scores, "sparse_v": bench_sparse_v, "flash": bench_flash,
          "flash_long": bench_flash_long, "vonly": bench_vonly, "widths": bench_widths, "codec_widths": bench_codec_widths,
-         "packed_widths": bench_packed_widths}
+         "packed_widths": bench_packed_widths, "vonly_batch": bench_vonly_batch}
 
 
 def main():
