@@ -21,6 +21,9 @@ parity unpinned (only an MLX install could pin them):
     PRNG stream (rotation.py:47-49); MLX is not available, so this module
     uses its own documented generator.  Every function takes `signs`
     explicitly, so the rest of the path is independent of the generator.
+    mlx_random_diagonal_sign restates MLX's stream from its published
+    algorithm: its hash (threefry2x32) is pinned by the Random123
+    known-answer vectors, the word layout and the float conversion are not.
   * the float32 summation order inside mx.linalg.norm (quantizer.py:89) is
     backend-defined; this oracle fixes it to the only order the reference
     specifies, the stride-halving tree of its Metal encoder (metal.py:33-38).
@@ -103,6 +106,45 @@ def random_diagonal_sign(d: int, seed: int = 42) -> np.ndarray:
     for i in range(d):
         out[i] = 1.0 if (_splitmix64((base + i) & 0xFFFFFFFFFFFFFFFF) >> 63) else -1.0
     return out
+
+
+def threefry2x32(key0, key1, x0, x1):
+    """Threefry-2x32-20 (Salmon et al., SC'11) on uint32 arrays: the counter-based hash of MLX's `mx.random`
+    (third-party, mlx >= 0.20, pyproject.toml:13; absent here).  Pinned by the Random123 known-answer vectors."""
+    u32 = np.uint32
+    key0, key1 = u32(key0), u32(key1)
+    ks = (key0, key1, u32(0x1BD11BDA) ^ key0 ^ key1)
+    x0 = np.asarray(x0, dtype=u32).copy()
+    x1 = np.asarray(x1, dtype=u32).copy()
+    rot = ((13, 15, 26, 6), (17, 29, 16, 24))
+    with np.errstate(over="ignore"):
+        x0 += ks[0]
+        x1 += ks[1]
+        for block in range(5):
+            for r in rot[block & 1]:
+                x0 += x1
+                x1 = (x1 << u32(r)) | (x1 >> u32(32 - r))
+                x1 ^= x0
+            x0 += ks[(block + 1) % 3]
+            x1 += ks[(block + 2) % 3] + u32(block + 1)
+    return x0, x1
+
+
+def mlx_random_diagonal_sign(d: int, seed: int = 42) -> np.ndarray:
+    """rotation.py:47-49 with MLX's generator restated from its published source: key (seed >> 32, seed & 2^32-1);
+    word i and word i + ceil(d/2) are the two outputs of threefry2x32(key, (i, i + ceil(d/2))) (odd d: the middle
+    word is the first output of (floor(d/2), 0)); uniform = float32(word) / float32(2^32 - 1), capped below 1;
+    +1 where uniform < 0.5.  PARITY UNPINNED beyond the hash: only an MLX install could confirm the layout."""
+    half, odd = d // 2, d & 1
+    i = np.arange(half, dtype=np.uint32)
+    a, b = threefry2x32((seed >> 32) & 0xFFFFFFFF, seed & 0xFFFFFFFF, i, i + np.uint32(half + odd))
+    words = np.empty(d, dtype=np.uint32)
+    words[:half] = a
+    words[half + odd:] = b
+    if odd:
+        words[half] = threefry2x32((seed >> 32) & 0xFFFFFFFF, seed & 0xFFFFFFFF, [half], [0])[0][0]
+    u = np.minimum(words.astype(F32) / F32(4294967295.0), np.nextafter(F32(1.0), F32(0.0)))
+    return np.where(u < F32(0.5), F32(1.0), F32(-1.0)).astype(F32)
 
 
 def randomized_hadamard_transform(x: np.ndarray, signs: np.ndarray) -> np.ndarray:

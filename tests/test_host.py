@@ -123,6 +123,30 @@ def test_kernels_refuse_cpu_tensors():
                               torch.ones(96), 96, 3)
 
 
+def test_mlx_sign_stream_hash_known_answers_and_restatements_agree():
+    """Threefry-2x32-20 against the Random123 known-answer vectors (zero, all-ones, digits of pi), in the package's
+    scalar form and the oracle's vectorised one; the two restatements of MLX's sign stream (rotation.py:47-49) agree
+    for even and odd d and seeds above 2^32; the default generator is unchanged.  The word layout of that stream is
+    not pinned by anything available offline."""
+    from tqhip.rotation import mlx_sign_pattern, threefry2x32
+    kats = (((0, 0), (0, 0), (0x6B200159, 0x99BA4EFE)),
+            ((0xFFFFFFFF, 0xFFFFFFFF), (0xFFFFFFFF, 0xFFFFFFFF), (0x1CB996FC, 0xBB002BE7)),
+            ((0x13198A2E, 0x03707344), (0x243F6A88, 0x85A308D3), (0xC4923A9C, 0x483DF7A0)))
+    for key, count, want in kats:
+        assert threefry2x32(key, count) == want
+        a, b = o.threefry2x32(key[0], key[1], [count[0]], [count[1]])
+        assert (int(a[0]), int(b[0])) == want
+    for d, seed in ((128, 42), (128, 43), (64, 7), (256, 0), (33, 5), (128, (3 << 32) + 9)):
+        got = tqhip.random_diagonal_sign(d, seed, stream="mlx").numpy()
+        assert np.array_equal(got, o.mlx_random_diagonal_sign(d, seed))
+        assert got.dtype == np.float32 and set(np.unique(got)) <= {-1.0, 1.0}
+        assert mlx_sign_pattern(d, seed) == got.tolist()
+    assert abs(float(tqhip.random_diagonal_sign(4096, 1, stream="mlx").mean())) < 0.08
+    assert not np.array_equal(tqhip.random_diagonal_sign(128, 42, stream="mlx").numpy(), tqhip.random_diagonal_sign(128, 42).numpy())
+    with pytest.raises(ValueError, match="stream"):
+        tqhip.random_diagonal_sign(128, 42, stream="jax")
+
+
 def test_sign_generator_and_tables_match_oracle():
     for d, seed in ((128, 42), (128, 43), (64, 7), (256, 0)):
         assert np.array_equal(tqhip.random_diagonal_sign(d, seed).numpy(), o.random_diagonal_sign(d, seed))
