@@ -667,8 +667,8 @@ __global__ __launch_bounds__(WAVES * 64) void vonly_scores_kernel(MfmaArgs a) {
   }
 }
 
-// Streaming variant for unmasked full tiles: one workgroup runs through n_blocks CONSECUTIVE
-// 512-position blocks; a wave walks its 64 rows of every block in STEPS of 32 positions with an
+// Streaming variant for unmasked caches: one workgroup of NW waves runs through n_blocks CONSECUTIVE
+// blocks of NW * 64 positions; a wave walks its 64 rows of every block in STEPS of 32 positions with an
 // online softmax in registers (the flash recurrence: running maximum, rescale of the accumulators
 // when it moves).  Loads are double-buffered: the norm, packed-V and K loads of step s+1 are
 // issued in three instalments between the phases of step s, so memory streams while the ALUs and
@@ -678,8 +678,8 @@ __global__ __launch_bounds__(WAVES * 64) void vonly_scores_kernel(MfmaArgs a) {
 // The partial of a workgroup is taken relative to R = m - kexp (running maximum in log2 units minus
 // the exponent of the power-of-two norm scale of the step that set it): weights are
 // 2^(s*cs - R), and moving from R_old to R_new multiplies accumulators and weight sum by 2^(R_old - R_new).
-// grid = (ceil(seq_len / (512 * n_blocks)), n_kv, n_seq), 512 threads.
-// RAGGED = the length is not a multiple of 512 * n_blocks: the last workgroup of a (sequence, kv head) runs
+// grid = (ceil(seq_len / (NW * 64 * n_blocks)), n_kv, n_seq), NW * 64 threads.
+// RAGGED = the length is not a multiple of a workgroup's range: the last workgroup of a (sequence, kv head) runs
 // through fewer blocks, loads of rows past the end are redirected to valid rows (norms and K rows to the last
 // valid row, packed-V pieces with no valid byte to the first piece of the last partly valid step; an aligned
 // 16-byte piece that holds a valid byte never crosses a page) and the scores of those rows are set to -inf.
@@ -1280,8 +1280,8 @@ __global__ __launch_bounds__(kMergeThreads + 64) void decode_merge_fresh_kernel(
 // Which tile kernel a launch uses (chosen by the host from the length, the mask / offsets and the alignment).
 struct VonlyTileChoice {
   int nw;                     // waves per workgroup: 8 or 4
-  int n_blocks;               // > 1: streaming pass, that many 512-position blocks per workgroup
-  bool ragged_stream;         // the streaming pass with a ragged end
+  int n_blocks;               // > 1: streaming pass, that many blocks of nw * 64 positions per workgroup
+  bool ragged_stream;         // the streaming pass with a ragged end and / or over a ragged batch
   bool plain;                 // full 512-position tiles, no mask, no offsets
   bool plain4;                // full 256-position tiles, no mask, no offsets
   bool plain_any;             // no mask, no offsets, any length
