@@ -252,6 +252,26 @@ __device__ __forceinline__ void butterfly_4lane(float (&xs)[4][8], uint32_t flip
   }
 }
 
+// Reductions over the four 16-lane rows of a wave (lanes l, l ^ 16, l ^ 32, l ^ 48), result in every lane: row
+// swaps in the vector ALU (v_permlane16_swap: rows 1, 3 of the first operand change places with rows 0, 2 of the
+// second; v_permlane32_swap: the upper half of the first with the lower half of the second) instead of two trips
+// through the LDS permute path.  Both operands start as the value itself, so after a swap the two results hold the
+// value of this lane's row and of its partner row in some order; max and + do not care which.
+__device__ __forceinline__ float max_over_rows(float v) {
+  typedef unsigned int u2_t __attribute__((ext_vector_type(2)));
+  u2_t r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+  r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float sum_over_rows(float v) {
+  typedef unsigned int u2_t __attribute__((ext_vector_type(2)));
+  u2_t r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+  r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
   for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, shfl_xor_f(v, m));
@@ -301,6 +321,21 @@ struct PackedField {
     Y = ((fa >> BITS) & kEven) | (fb & (kEven << BITS));
   }
   __device__ static __forceinline__ uint32_t index(uint32_t src, int i) { return (src >> (2 * BITS * i)) & (uint32_t)(kLut - 1); }
+
+  // bits of a packed row that start in word at_w0[0] at bit sh_lo, NOT cut to the 8 * BITS bits of the piece: for
+  // consumers that mask every index they take out anyway
+  __device__ static __forceinline__ uint32_t field_raw(const uint32_t* at_w0, int sh_lo, int sh_hi) {
+    if (BITS == 3) return (at_w0[1] << sh_hi) | (at_w0[0] >> sh_lo);
+    if (BITS == 4) return at_w0[0];
+    return at_w0[0] >> sh_lo;
+  }
+  // interleave() on raw fields: bits of X / Y above 8 * BITS are garbage; four operations (two shifts, two selects
+  // under the mask of the even fields)
+  __device__ static __forceinline__ void interleave_raw(uint32_t fa, uint32_t fb, uint32_t& X, uint32_t& Y) {
+    X = (fa & kEven) | ((fb << BITS) & ~kEven);
+    Y = ((fa >> BITS) & kEven) | (fb & ~kEven);
+  }
+
   // this lane's entries of a table of kLut centroid pairs half2(c[i & mask], c[i >> BITS]); selects, not a dynamic
   // index into kernel arguments
   __device__ static __forceinline__ void fill(uint32_t* lut, const Codebook& cb, int lane) {
@@ -315,6 +350,42 @@ struct PackedField {
       }
       if (kLut >= 64 || idx < kLut) lut[idx] = pack_h2(clo, chi);
     }
+  }
+
+  // ---- centroid QUADS: one 8-byte look-up decodes four fields ----------------------------------------------------
+  // Entry i of the quad table is {pair[i mod kLut], pair[i / kLut]}: the four centroids of four adjacent fields of a
+  // source word (keys: four consecutive elements of a row; values: the same two elements of two rows, interleaved).
+  // 16 / 256 / 4096 entries at 1 / 2 / 3 bits (32 KB at three bits, one table for keys and values when their
+  // codebooks are equal); four bits would need 65536 entries and stay with pairs.  Per four fields: two vector
+  // instructions (bit-field extract, shift) and one 8-byte LDS read, against four and two 4-byte reads with pairs.
+  static constexpr bool kQuad = BITS <= 3;
+  static constexpr int kQuadBits = 4 * BITS;
+  static constexpr int kQuadEntries = kQuad ? (1 << kQuadBits) : 1;
+  // built by the whole workgroup from the pair table (which must be visible: barrier before, barrier after)
+  __device__ static __forceinline__ void fill_quad(uint2* qlut, const uint32_t* pair_lut, int tid, int n_threads) {
+    for (int i = tid; i < kQuadEntries; i += n_threads)
+      qlut[i] = make_uint2(pair_lut[i & (kLut - 1)], pair_lut[i >> (2 * BITS)]);
+  }
+  // Value side: four positions a, b, c, d interleaved so that the 4 * BITS bits of ONE element at the four positions
+  // are adjacent (a lowest): from the raw fields of the four rows, Z[0] holds elements 0 and 4 (quads 0 and 1), Z[1]
+  // elements 2 and 6, Z[2] elements 1 and 5, Z[3] elements 3 and 7.  Two levels of interleave_raw's shift-and-select:
+  // 16 operations for 32 fields.  Bits above 8 * BITS are garbage.
+  static constexpr uint32_t kEven2 = BITS == 3 ? 0x03F03Fu : BITS == 2 ? 0x0F0Fu : BITS == 1 ? 0x33u : 0x00FF00FFu;
+  __device__ static __forceinline__ void interleave4_raw(uint32_t fa, uint32_t fb, uint32_t fc, uint32_t fd, uint32_t (&Z)[4]) {
+    uint32_t Xab, Yab, Xcd, Ycd;
+    interleave_raw(fa, fb, Xab, Yab);
+    interleave_raw(fc, fd, Xcd, Ycd);
+    Z[0] = (Xab & kEven2) | ((Xcd << (2 * BITS)) & ~kEven2);
+    Z[1] = ((Xab >> (2 * BITS)) & kEven2) | (Xcd & ~kEven2);
+    Z[2] = (Yab & kEven2) | ((Ycd << (2 * BITS)) & ~kEven2);
+    Z[3] = ((Yab >> (2 * BITS)) & kEven2) | (Ycd & ~kEven2);
+  }
+  // element et (0 .. 7) of the piece: which Z word and which quad of it
+  __device__ static constexpr int z_word(int et) { return ((et & 1) << 1) | ((et >> 1) & 1); }
+  __device__ static constexpr int z_quad(int et) { return et >> 2; }
+  __device__ static __forceinline__ uint2 quad_lookup(const uint2* qlut, uint32_t src, int j) {
+    const uint32_t off = __builtin_amdgcn_ubfe(src, kQuadBits * j, kQuadBits) << 3;
+    return *reinterpret_cast<const uint2*>(reinterpret_cast<const char*>(qlut) + off);
   }
 };
 

@@ -143,10 +143,80 @@ __device__ __forceinline__ void rotate_query_rows(const void* q_raw, int q_dtype
   }
 }
 
+// A operand of a score product: the centroids of the 8 consecutive key elements in the low 8 * BITS bits of f,
+// as two quad look-ups or four pair look-ups
+template <int BITS, bool QUAD>
+__device__ __forceinline__ u4 key_operand(uint32_t f, const uint2* quad_lut, const uint32_t* pair_lut) {
+  using VF = VField<BITS>;
+  u4 ka;
+  if constexpr (QUAD) {
+    const uint2 lo = VF::quad_lookup(quad_lut, f, 0), hi = VF::quad_lookup(quad_lut, f, 1);
+    ka = u4{lo.x, lo.y, hi.x, hi.y};
+  } else {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) ka[k] = pair_lut[VF::index(f, k)];
+  }
+  return ka;
+}
+
+// Table indices of the value products of 32 positions (kb2 = which 32 of the wave's 64): lane (n16, g) decodes
+// elements 8 n16 .. 8 n16 + 7 (piece at word w0, shifts sh_lo / sh_hi of a row) of positions 16 t + 4 g + j,
+// t = 2 kb2, 2 kb2 + 1, j = 0 .. 3 -- the eight contraction slots of this lane in the matrix instruction.
+// Pairs: VI[qd] / VI[4 + qd] = even / odd elements of positions (2 jp, 2 jp + 1) of t, qd = 2 (t - 2 kb2) + jp.
+// Quads: VI[4 th + w] = word w of interleave4_raw over the four positions of t = 2 kb2 + th.
+template <int BITS, bool QUAD>
+__device__ __forceinline__ void value_indices(const uint32_t* rows, int kb2, int g, int w0, int sh_lo, int sh_hi,
+                                              uint32_t (&VI)[8]) {
+  using VF = VField<BITS>;
+  constexpr int kPd = VF::kPd;
+  if constexpr (QUAD) {
+#pragma unroll
+    for (int th = 0; th < 2; ++th) {
+      const uint32_t* r = rows + (16 * (2 * kb2 + th) + 4 * g) * kPd + w0;
+      uint32_t Z[4];
+      VF::interleave4_raw(VF::field_raw(r, sh_lo, sh_hi), VF::field_raw(r + kPd, sh_lo, sh_hi),
+                          VF::field_raw(r + 2 * kPd, sh_lo, sh_hi), VF::field_raw(r + 3 * kPd, sh_lo, sh_hi), Z);
+#pragma unroll
+      for (int w = 0; w < 4; ++w) VI[4 * th + w] = Z[w];
+    }
+  } else {
+#pragma unroll
+    for (int qd = 0; qd < 4; ++qd) {
+      const int t = 2 * kb2 + (qd >> 1), jp = qd & 1;
+      const uint32_t* ra = rows + (16 * t + 4 * g + 2 * jp) * kPd + w0;
+      VF::interleave_raw(VF::field_raw(ra, sh_lo, sh_hi), VF::field_raw(ra + kPd, sh_lo, sh_hi), VI[qd], VI[4 + qd]);
+    }
+  }
+}
+
+// Value products of 32 positions: accS[et] += A x B[et], B[et] = the centroids of element et of this lane's piece at
+// its eight positions: two quad look-ups (four positions each) or four pair look-ups.
+template <int BITS, bool QUAD>
+__device__ __forceinline__ void value_products(const u4& A, const uint32_t (&VI)[8], const uint2* quad_lut,
+                                               const uint32_t* pair_lut, f4 (&accS)[8]) {
+  using VF = VField<BITS>;
+#pragma unroll
+  for (int et = 0; et < 8; ++et) {
+    u4 B;
+    if constexpr (QUAD) {
+      const uint2 lo = VF::quad_lookup(quad_lut, VI[VF::z_word(et)], VF::z_quad(et));
+      const uint2 hi = VF::quad_lookup(quad_lut, VI[4 + VF::z_word(et)], VF::z_quad(et));
+      B = u4{lo.x, lo.y, hi.x, hi.y};
+    } else {
+#pragma unroll
+      for (int qd = 0; qd < 4; ++qd) B[qd] = pair_lut[VF::index(VI[(et & 1) * 4 + qd], et >> 1)];
+    }
+    accS[et] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, A), __builtin_bit_cast(h8, B),
+                                                      accS[et], 0, 0, 0);
+  }
+}
+
 // grid = (n_tiles_max, n_kv, n_seq), 512 threads.  BITS: width of the packed keys and values (a cache has one
 // width for both).  WPE = waves per SIMD the registers are budgeted for: 4 lets two workgroups share a CU (the
 // flash mode then spills some registers, which large grids repay); 3 is the flash mode without spills, for
 // grids that give a CU one workgroup at most.
+// Centroids come from the pair tables here: a workgroup decodes 512 positions once, which does not repay building the
+// 32 KB quad table (measured: scores over 65 536 positions 10.65 us with pairs, 10.95 us with quads).
 template <int MODE, int BITS = 3, int WPE = 4>
 __global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
 void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
@@ -156,8 +226,10 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
   constexpr bool HAS_K = !GIVEN;
   constexpr bool HAS_V = MODE != kScores && MODE != kSoftScores;
   constexpr bool SOFT = MODE == kFlash || MODE == kSoftScores;        // scores carry attn_scale * log2 e and the mask
+  constexpr bool KQUAD = false, VQUAD = false;
   __shared__ __align__(16) unsigned char big_s[32768];      // per-wave 4 KB areas, later S_all[8][8][128]
   __shared__ uint32_t lutk_s[VF::kLut < 64 ? 64 : VF::kLut], lutv_s[VF::kLut < 64 ? 64 : VF::kLut];
+  const uint2* quad_s = nullptr;
   __shared__ __align__(16) uint32_t q_s[kHeadsMax][kD / 2];      // rotated queries as half2: rounded value ...
   __shared__ __align__(16) uint32_t ql_s[kHeadsMax][kD / 2];     // ... and what the rounding lost
   __shared__ __align__(16) float kn_s[kWaves][kWavePos], vn_s[kWaves][kWavePos];
@@ -309,7 +381,7 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
   // ---- V: norms, table indices --------------------------------------------------------------------------
   float vn[4][4];
   float inv_tscale = 1.0f, kexp = 0.0f;
-  uint32_t X[2][4], Y[2][4];
+  uint32_t VI[2][8];
   if (HAS_V) {
     float nmax = 0.0f;
 #pragma unroll
@@ -336,13 +408,7 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
     int w0, sh_lo, sh_hi;
     VF::pos(n16, w0, sh_lo, sh_hi);
 #pragma unroll
-    for (int kb2 = 0; kb2 < 2; ++kb2)
-#pragma unroll
-      for (int qd = 0; qd < 4; ++qd) {
-        const int t = 2 * kb2 + (qd >> 1), jp = qd & 1;
-        const uint32_t* ra = stage + (16 * t + 4 * g + 2 * jp) * kVPd + w0;
-        VF::interleave(VF::field(ra, sh_lo, sh_hi), VF::field(ra + kVPd, sh_lo, sh_hi), X[kb2][qd], Y[kb2][qd]);
-      }
+    for (int kb2 = 0; kb2 < 2; ++kb2) value_indices<BITS, VQUAD>(stage, kb2, g, w0, sh_lo, sh_hi, VI[kb2]);
   }
 
   // ---- K: scores ----------------------------------------------------------------------------------------
@@ -366,10 +432,8 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
       const uint32_t* krow = stage + (16 * t + n16) * kVPd;
 #pragma unroll
       for (int kb = 0; kb < 4; ++kb) {
-        const uint32_t f = VF::field(krow + kw0[kb], ksl[kb], ksh[kb]);
-        u4 ka;
-#pragma unroll
-        for (int k = 0; k < 4; ++k) ka[k] = lutk_s[VF::index(f, k)];
+        const uint32_t f = VF::field_raw(krow + kw0[kb], ksl[kb], ksh[kb]);
+        const u4 ka = key_operand<BITS, KQUAD>(f, quad_s, lutk_s);
         acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, ka), __builtin_bit_cast(h8, qreg[kb]),
                                                      acc, 0, 0, 0);
         acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, ka), __builtin_bit_cast(h8, qlow[kb]),
@@ -493,17 +557,7 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
 #pragma unroll
   for (int kb2 = 0; kb2 < 2; ++kb2) {
     const u4 A = {pa[kb2][0], pa[kb2][1], pa[kb2][2], pa[kb2][3]};
-#pragma unroll
-    for (int et = 0; et < 8; ++et) {
-      u4 B;
-#pragma unroll
-      for (int qd = 0; qd < 4; ++qd) {
-        const uint32_t src = (et & 1) ? Y[kb2][qd] : X[kb2][qd];
-        B[qd] = lutv_s[VF::index(src, et >> 1)];
-      }
-      accS[et] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, A), __builtin_bit_cast(h8, B),
-                                                        accS[et], 0, 0, 0);
-    }
+    value_products<BITS, VQUAD>(A, VI[kb2], quad_s, lutv_s, accS);
   }
 
   // ---- merge the eight waves (merge_waves, tq_decode_mfma.h) ------------------------------------------------
@@ -534,16 +588,20 @@ constexpr int kSThreads = kSWaves * 64;
 constexpr int kSStepPos = kSWaves * kWavePos;     // 256 positions per workgroup step
 constexpr int kSImageBytes = 4096;                // 209 pieces of 16 bytes, rounded up; 256 pieces at four bits
 
-template <int BITS>
+template <int BITS, bool VQ = true>
 __global__ __launch_bounds__(kSThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps) {
   using VF = VField<BITS>;
+  // A workgroup decodes up to 8 x 256 positions, which repays building the quad table (one for keys and values when
+  // their codebooks are equal, VQ; else the values use their pair table).
+  constexpr bool KQUAD = VF::kQuad, VQUAD = VF::kQuad && VQ;
   constexpr int kPd = VF::kPd;                                  // words per packed row
   constexpr int kPieces = BITS == 3 ? 209 : 16 * kPd;           // 16-byte pieces of a wave's 64 rows (three bits: + misalignment)
   constexpr int kWhole = kPieces / 64, kRest = kPieces % 64;    // whole-wave stores into the image, lanes of the last one
   constexpr int kLoads = kWhole + (kRest ? 1 : 0);
   __shared__ __align__(16) unsigned char big_s[kSWaves * 2 * kSImageBytes];   // per wave: K image, V image; later S_all[4][8][128]
   __shared__ uint32_t lutk_s[VF::kLut < 64 ? 64 : VF::kLut], lutv_s[VF::kLut < 64 ? 64 : VF::kLut];
+  __shared__ __align__(16) uint2 quad_s[KQUAD ? VF::kQuadEntries : 1];
   __shared__ __align__(16) uint32_t q_s[kHeadsMax][kD / 2];
   __shared__ __align__(16) uint32_t ql_s[kHeadsMax][kD / 2];
   __shared__ __align__(16) float kn_s[kSWaves][kWavePos], vn_s[kSWaves][kWavePos];
@@ -582,24 +640,34 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
 
   auto rows_left_of = [&](int s) {
     const int64_t p0w = wg_p0 + (int64_t)s * kSStepPos + wave * kWavePos;
-    const int64_t left = len - p0w;
+    const int64_t left = s < n_steps ? len - p0w : 0;      // steps past the workgroup's last have no rows
     return (int)(left < 0 ? 0 : (left > kWavePos ? kWavePos : left));
   };
+  // Requests the rows of step s.  Every call issues the same loads whatever s is: a piece or norm past the end of
+  // the sequence (or a step past the workgroup's last) is fetched from the first piece / row of the workgroup's
+  // range instead, which exists, so that no branch surrounds a load -- the compiler can then count the requests in
+  // flight and wait for one buffer's rows while the other buffer's are still on their way.  What comes back for a
+  // row that does not exist is real data of another row: finite, and its score is set to -inf.
+  // Addresses are a base that is the same for the whole workgroup (its first piece / first norm) plus a 32-bit
+  // offset per lane: one register per load instead of a 64-bit pointer.
+  const char* k_base = krow0 + wg_p0 * (kPd * 4) - kmis;
+  const char* v_base = vrow0 + wg_p0 * (kPd * 4) - vmis;
+  const float* kn_base = knrow0 + wg_p0;
+  const float* vn_base = vnrow0 + wg_p0;
   auto issue = [&](int s, u4 (&kq)[kLoads], u4 (&vq)[kLoads], float& kn, float& vn) {
-    const int64_t p0w = wg_p0 + (int64_t)s * kSStepPos + wave * kWavePos;
+    const uint32_t row0 = (uint32_t)(s * kSStepPos + wave * kWavePos);   // first row of the wave's block, from wg_p0
     const int rows = rows_left_of(s);
-    const int kbytes = rows ? kmis + rows * (kPd * 4) : 0;
-    const int vbytes = rows ? vmis + rows * (kPd * 4) : 0;
-    const char* kb = krow0 + p0w * (kPd * 4) - kmis;
-    const char* vb = vrow0 + p0w * (kPd * 4) - vmis;
+    const uint32_t kbytes = rows ? kmis + rows * (kPd * 4) : 0;
+    const uint32_t vbytes = rows ? vmis + rows * (kPd * 4) : 0;
 #pragma unroll
     for (int i = 0; i < kLoads; ++i) {
-      const int off = (i * 64 + lane) * 16;
-      kq[i] = (off < kbytes) ? *reinterpret_cast<const u4*>(kb + off) : u4{0u, 0u, 0u, 0u};
-      vq[i] = (off < vbytes) ? *reinterpret_cast<const u4*>(vb + off) : u4{0u, 0u, 0u, 0u};
+      const uint32_t off = (uint32_t)(i * 64 + lane) * 16;
+      kq[i] = *reinterpret_cast<const u4*>(k_base + (off < kbytes ? row0 * (kPd * 4) + off : 0u));
+      vq[i] = *reinterpret_cast<const u4*>(v_base + (off < vbytes ? row0 * (kPd * 4) + off : 0u));
     }
-    kn = (lane < rows) ? knrow0[p0w + lane] : 0.0f;
-    vn = (lane < rows) ? vnrow0[p0w + lane] : 0.0f;
+    const uint32_t nrow = (lane < rows) ? row0 + lane : 0u;
+    kn = kn_base[nrow];
+    vn = vn_base[nrow];
   };
 
   float2 my_q[4];
@@ -628,6 +696,10 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
     }
   }
   __syncthreads();
+  if (KQUAD) {
+    VF::fill_quad(quad_s, lutk_s, tid, kSThreads);
+    __syncthreads();
+  }
 
   u4 qreg[4], qlow[4];
 #pragma unroll
@@ -652,8 +724,12 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
 
   // one step on the buffers (kq, vq, kn, vn); `next()` issues the loads of the following step
   auto step = [&](int sidx, u4 (&kq)[kLoads], u4 (&vq)[kLoads], float kn, float vn_, auto&& next) {
-    const int rows = rows_left_of(sidx);                 // uniform over the wave
-    if (rows <= 0) return;                               // steps only run out at the end: nothing follows
+    const int rows = rows_left_of(sidx);                 // uniform over the wave, at least 1 (the caller checks)
+    // ---- the request for the next step's rows goes out first (the other buffer is free): what separates the arrival
+    // of one step's rows from the request for the next is on the critical path of a loop that a memory round trip bounds
+    __builtin_amdgcn_sched_barrier(0);
+    next();
+    __builtin_amdgcn_sched_barrier(0);
     // ---- images and norms into the wave's LDS area
     {
       u4* k4 = reinterpret_cast<u4*>(image);
@@ -664,9 +740,6 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
       kn_s[wave][lane] = kn * kscale;
       vn_s[wave][lane] = vn_;
     }
-    __builtin_amdgcn_sched_barrier(0);
-    next();
-    __builtin_amdgcn_sched_barrier(0);
     // ---- scores of the 64 rows (log2 units)
     float s[4][4];
 #pragma unroll
@@ -675,10 +748,8 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
       const uint32_t* krow = kimg + (16 * t + n16) * kPd;
 #pragma unroll
       for (int kb = 0; kb < 4; ++kb) {
-        const uint32_t f = VF::field(krow + kw0[kb], ksl[kb], ksh[kb]);
-        u4 ka;
-#pragma unroll
-        for (int k = 0; k < 4; ++k) ka[k] = lutk_s[VF::index(f, k)];
+        const uint32_t f = VF::field_raw(krow + kw0[kb], ksl[kb], ksh[kb]);
+        const u4 ka = key_operand<BITS, KQUAD>(f, quad_s, lutk_s);
         acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, ka), __builtin_bit_cast(h8, qreg[kb]),
                                                      acc, 0, 0, 0);
         acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, ka), __builtin_bit_cast(h8, qlow[kb]),
@@ -698,8 +769,7 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
       vn[t][0] = n4.x; vn[t][1] = n4.y; vn[t][2] = n4.z; vn[t][3] = n4.w;
       nmax = fmaxf(nmax, fmaxf(fmaxf(n4.x, n4.y), fmaxf(n4.z, n4.w)));
     }
-    nmax = fmaxf(nmax, shfl_xor_f(nmax, 16));
-    nmax = fmaxf(nmax, shfl_xor_f(nmax, 32));
+    nmax = max_over_rows(nmax);
     int ex = (int)((__float_as_uint(nmax) >> 23) & 0xFF);
     ex = ex < 27 ? (ex < 1 ? 127 : 27) : (ex > 227 ? 227 : ex);
     const float kexp = (float)(127 - ex);
@@ -710,8 +780,7 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
     for (int t = 0; t < 4; ++t)
 #pragma unroll
       for (int j = 0; j < 4; ++j) mb = fmaxf(mb, s[t][j]);
-    mb = fmaxf(mb, shfl_xor_f(mb, 16));
-    mb = fmaxf(mb, shfl_xor_f(mb, 32));
+    mb = max_over_rows(mb);
     const float m_new = fmaxf(m_run, mb);
     const float R_new = m_new - kexp;
     const float factor = __builtin_amdgcn_exp2f(R_run - R_new);      // 0 on the wave's first step
@@ -741,40 +810,26 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
 #pragma unroll
         for (int j = 0; j < 4; ++j) accS[et][j] *= av[j];
     }
-    // ---- values: packed V -> interleaved table indices -> centroid pairs, 32 positions at a time
+    // ---- values: packed V -> interleaved table indices -> centroids, 32 positions at a time
 #pragma unroll
     for (int kb2 = 0; kb2 < 2; ++kb2) {
-      uint32_t X[4], Y[4];
-#pragma unroll
-      for (int qd = 0; qd < 4; ++qd) {
-        const int t = 2 * kb2 + (qd >> 1), jp = qd & 1;
-        const uint32_t* ra = vimg + (16 * t + 4 * g + 2 * jp) * kPd + vw0;
-        VF::interleave(VF::field(ra, vsl, vsh), VF::field(ra + kPd, vsl, vsh), X[qd], Y[qd]);
-      }
+      uint32_t VI[8];
+      value_indices<BITS, VQUAD>(vimg, kb2, g, vw0, vsl, vsh, VI);
       const u4 A = {pa[kb2][0], pa[kb2][1], pa[kb2][2], pa[kb2][3]};
-#pragma unroll
-      for (int et = 0; et < 8; ++et) {
-        u4 B;
-#pragma unroll
-        for (int qd = 0; qd < 4; ++qd) {
-          const uint32_t src = (et & 1) ? Y[qd] : X[qd];
-          B[qd] = lutv_s[VF::index(src, et >> 1)];
-        }
-        accS[et] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, A), __builtin_bit_cast(h8, B),
-                                                          accS[et], 0, 0, 0);
-      }
+      value_products<BITS, VQUAD>(A, VI, quad_s, lutv_s, accS);
     }
   };
 
-  for (int sidx = 0; sidx < n_steps; sidx += 2) {          // steps come in pairs: buffers A and B stay in fixed registers
-    step(sidx, kqA, vqA, knA, vnA, [&]() {
-      if (sidx + 1 < n_steps) issue(sidx + 1, kqB, vqB, knB, vnB);
-    });
-    if (sidx + 1 < n_steps)
-      step(sidx + 1, kqB, vqB, knB, vnB, [&]() {
-        if (sidx + 2 < n_steps) issue(sidx + 2, kqA, vqA, knA, vnA);
-      });
+  // Steps come in pairs so that the two register buffers keep their names; the rows of step s + 1 are requested as
+  // the first thing step s does.  A wave stops at its first step without rows (steps only run out at the end of the
+  // sequence).
+  for (int sidx = 0; sidx < n_steps; sidx += 2) {
+    if (rows_left_of(sidx) <= 0) break;
+    step(sidx, kqA, vqA, knA, vnA, [&]() { issue(sidx + 1, kqB, vqB, knB, vnB); });
+    if (sidx + 1 >= n_steps || rows_left_of(sidx + 1) <= 0) break;
+    step(sidx + 1, kqB, vqB, knB, vnB, [&]() { issue(sidx + 2, kqA, vqA, knA, vnA); });
   }
+
 
   // ---- merge the four waves (merge_waves): a wave deposits into its own image area.  A wave that saw no valid
   // row has m = -inf, l = 0 and zero accumulators.
@@ -811,6 +866,12 @@ void launch_packed_tiles(int mode, bool one_per_cu, dim3 grid, const PackedArgs&
 template <int BITS>
 void launch_packed_stream(dim3 grid, const PackedArgs& a, const Codebook& kcb, const Codebook& vcb, int n_steps,
                           hipStream_t stream) {
+  if constexpr (VField<BITS>::kQuad) {
+    if (std::memcmp(kcb.c, vcb.c, sizeof(kcb.c)) != 0) {
+      packed_stream_kernel<BITS, false><<<grid, kSThreads, 0, stream>>>(a, kcb, vcb, n_steps);
+      return;
+    }
+  }
   packed_stream_kernel<BITS><<<grid, kSThreads, 0, stream>>>(a, kcb, vcb, n_steps);
 }
 
