@@ -64,6 +64,13 @@ enum tq_encode_variant {
                           compares the raw butterfly output w */
 };
 
+/* values of the `allow_mma` argument of tq_prerot_qk_scores and tq_sparse_v_matvec */
+enum tq_mma_mode {
+  TQ_MMA_OFF = 0,      /* float32 vector kernels */
+  TQ_MMA_FP16 = 1,     /* matrix cores, operands rounded to fp16 */
+  TQ_MMA_SPLIT = 2     /* matrix cores, operands as fp16 value + fp16 remainder: float32 fidelity */
+};
+
 /* which fused decode kernel a workspace query is for */
 enum tq_op {
   TQ_OP_SPARSE_V = 0,
@@ -141,9 +148,13 @@ int tq_prerotate_query(const void* q, int q_dtype, const float* signs, float* q_
  * Replaces prerot_fused_qk_scores (metal_kernels_v4.py:153-221, kernel 71-113).
  *   q_rot [n_kv*n_rep, dim] f32; k_packed / k_norms: one sequence, head_stride in rows;
  *   scores [n_kv*n_rep, seq_len] f32 contiguous.
- * allow_mma = 0: float32 arithmetic throughout (the reference's numerics); 1: q_rot and the
- * centroids are rounded to fp16 and multiplied on the matrix cores with float32 accumulation
- * (about 3e-4 relative per score) where the shape allows (d = 128, any width, n_rep <= 16).
+ * allow_mma = TQ_MMA_OFF (0): float32 vector arithmetic throughout (the reference's operation
+ * order); TQ_MMA_FP16 (1): q_rot and the centroids are rounded to fp16 and multiplied on the matrix
+ * cores with float32 accumulation (about 3e-4 relative per score); TQ_MMA_SPLIT (2): matrix cores
+ * with every operand as an fp16 value plus the fp16 remainder of its rounding (three matrix
+ * instructions per tile, products exact in float32: float32 fidelity, ~1e-6 relative, inside the
+ * reference's own bar of 1e-4 absolute, tests/test_prerot.py:90-95).  The matrix-core forms need
+ * d = 128, n_rep <= 16 (any width); other shapes run the float32 vector kernels whatever the flag.
  */
 int tq_prerot_qk_scores(const float* q_rot, const uint32_t* k_packed, const float* k_norms,
                         const float* centroids, float* scores,
@@ -187,7 +198,9 @@ int tq_softmax_rows(const float* scores, const float* mask, int64_t mask_row_str
  * Replaces sparse_v_matvec (sparse_v.py:94-186, kernel 32-88).  KV positions are split
  * across workgroups; partial sums go through `workspace` and a second pass applies the one
  * butterfly.   weights [n_kv*n_rep, seq_len] f32; out [n_kv*n_rep, dim] f32.
- * allow_mma as in tq_prerot_qk_scores (weights * norm and centroids rounded to fp16).
+ * allow_mma as in tq_prerot_qk_scores (TQ_MMA_FP16: weights * norm and centroids rounded to fp16;
+ * TQ_MMA_SPLIT: both as value + remainder, within the reference's bar of 1e-5 of the largest
+ * output, tests/test_sparse_v.py:70-75).
  */
 int tq_sparse_v_matvec(const float* weights, const uint32_t* v_packed, const float* v_norms,
                        const float* centroids, const float* signs, float* out,

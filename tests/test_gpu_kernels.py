@@ -309,9 +309,15 @@ def test_polar_quantizer_object(tq):
 
 # ------------------------------------------------------------------ scores
 
+# the default (precision=None: split operands on the matrix cores where the shape allows) and the float32
+# vector kernels are held to the same bars, the reference's own
+PRECS = pytest.mark.parametrize("prec", [None, "fp32"])
+
+
+@PRECS
 @pytest.mark.parametrize("H,S,D,bits", [(4, 64, 128, 3), (8, 256, 128, 3), (2, 16, 64, 4), (1, 128, 32, 2),
-                                        (3, 1000, 128, 3)])
-def test_prerot_scores_match_oracle_and_full_kernel(tq, H, S, D, bits):
+                                        (3, 1000, 128, 3), (2, 700, 128, 4), (2, 513, 128, 2), (1, 64, 128, 1)])
+def test_prerot_scores_match_oracle_and_full_kernel(tq, H, S, D, bits, prec):
     rng = np.random.default_rng(8)
     c, b = tables(bits)
     s = o.random_diagonal_sign(D, 42)
@@ -319,7 +325,7 @@ def test_prerot_scores_match_oracle_and_full_kernel(tq, H, S, D, bits):
     kn = (rng.random((H, S)) * 10 + 1).astype(F32)
     q = rng.standard_normal((H, D)).astype(F32)
     q_rot = tq.prerotate_query(dev(q), dev(s))
-    pre = host(tq.prerot_fused_qk_scores(q_rot, dev(kp), dev(kn), c, D, bits))
+    pre = host(tq.prerot_fused_qk_scores(q_rot, dev(kp), dev(kn), c, D, bits, precision=prec))
     full = host(tq.packed_fused_qk_scores(dev(q), dev(kp), dev(kn), c, dev(s), D, bits))
     want = o.prerot_fused_qk_scores(o.prerotate_query(q, s), kp, kn, c, D, bits)
     scale = max(1.0, np.abs(want).max())
@@ -328,19 +334,20 @@ def test_prerot_scores_match_oracle_and_full_kernel(tq, H, S, D, bits):
     assert np.abs(pre - full).max() < 1e-4 * scale                       # test_prerot.py:62-97
 
 
-@pytest.mark.parametrize("n_kv,n_rep", [(4, 2), (2, 4), (4, 7), (1, 12)])
-def test_prerot_scores_gqa(tq, n_kv, n_rep):
+@PRECS
+@pytest.mark.parametrize("n_kv,n_rep", [(4, 2), (2, 4), (4, 7), (1, 12), (1, 16), (1, 17)])
+def test_prerot_scores_gqa(tq, n_kv, n_rep, prec):
     rng = np.random.default_rng(9)
     D, S, bits = 128, 300, 3
     c, b = tables(bits)
     kp = o.pack_indices(rng.integers(0, 8, size=(n_kv, S, D)).astype(np.uint8), bits)
     kn = (rng.random((n_kv, S)) + 0.5).astype(F32)
     qr = rng.standard_normal((n_kv * n_rep, D)).astype(F32)
-    got = host(tq.prerot_fused_qk_scores(dev(qr), dev(kp), dev(kn), c, D, bits, n_rep=n_rep))
+    got = host(tq.prerot_fused_qk_scores(dev(qr), dev(kp), dev(kn), c, D, bits, n_rep=n_rep, precision=prec))
     want = o.prerot_fused_qk_scores(qr, kp, kn, c, D, bits, n_rep)
     assert np.abs(got - want).max() < 1e-5 * max(1.0, np.abs(want).max())
     with pytest.raises(ValueError, match="must equal n_kv_heads"):
-        tq.prerot_fused_qk_scores(dev(qr[:-1]), dev(kp), dev(kn), c, D, bits, n_rep=n_rep)
+        tq.prerot_fused_qk_scores(dev(qr[:-1]), dev(kp), dev(kn), c, D, bits, n_rep=n_rep, precision=prec)
 
 
 def test_scores_on_cache_slices(tq):
@@ -389,18 +396,21 @@ def softmax_np(x):
     return (e / e.sum(-1, keepdims=True)).astype(F32)
 
 
+@PRECS
 @pytest.mark.parametrize("H,S,D,bits", [(4, 128, 128, 3), (2, 512, 128, 3), (8, 64, 64, 4), (2, 777, 256, 3),
-                                        (3, 100, 32, 2), (1, 5000, 128, 3)])
-def test_sparse_v_dense_threshold(tq, H, S, D, bits):
+                                        (3, 100, 32, 2), (1, 5000, 128, 3), (2, 1300, 128, 4), (2, 515, 128, 2),
+                                        (1, 70, 128, 1)])
+def test_sparse_v_dense_threshold(tq, H, S, D, bits, prec):
     rng = np.random.default_rng(12)
     c, s, vp, vn = v_fixture(rng, H, S, D, bits)
     w = softmax_np(rng.standard_normal((H, S)) * 3)
     want = o.sparse_v_matvec(w, vp, vn, c, s, D, bits, threshold=0.0)
-    got = host(tq.sparse_v_matvec(dev(w), dev(vp), dev(vn), c, dev(s), D, bits, threshold=0.0))
+    got = host(tq.sparse_v_matvec(dev(w), dev(vp), dev(vn), c, dev(s), D, bits, threshold=0.0, precision=prec))
     assert np.abs(got - want).max() / np.abs(want).max() < 1e-5         # test_sparse_v.py:47-76
 
 
-def test_sparse_v_threshold_semantics(tq):
+@PRECS
+def test_sparse_v_threshold_semantics(tq, prec):
     rng = np.random.default_rng(13)
     H, S, D, bits = 4, 2048, 128, 3
     c, s, vp, vn = v_fixture(rng, H, S, D, bits)
@@ -408,26 +418,28 @@ def test_sparse_v_threshold_semantics(tq):
     args = (dev(vp), dev(vn), c, dev(s), D, bits)
     for thr in (1e-5, 1e-4, 1e-3):
         want = o.sparse_v_matvec(w, vp, vn, c, s, D, bits, threshold=thr)
-        got = host(tq.sparse_v_matvec(dev(w), *args, threshold=thr))
+        got = host(tq.sparse_v_matvec(dev(w), *args, threshold=thr, precision=prec))
         assert np.abs(got - want).max() < 1e-5 * np.abs(want).max()
-    dense = host(tq.sparse_v_matvec(dev(w), *args, threshold=0.0))
-    sp = host(tq.sparse_v_matvec(dev(w), *args))                         # default threshold 1e-5
+    dense = host(tq.sparse_v_matvec(dev(w), *args, threshold=0.0, precision=prec))
+    sp = host(tq.sparse_v_matvec(dev(w), *args, precision=prec))         # default threshold 1e-5
     assert (sp * dense).sum() / np.linalg.norm(sp) / np.linalg.norm(dense) > 0.999
-    zero = host(tq.sparse_v_matvec(dev(w), *args, threshold=2.0))
+    zero = host(tq.sparse_v_matvec(dev(w), *args, threshold=2.0, precision=prec))
     assert (zero == 0).all()                                             # test_sparse_v.py:150-168
-    neg = host(tq.sparse_v_matvec(dev(w), *args, threshold=-1.0))
+    neg = host(tq.sparse_v_matvec(dev(w), *args, threshold=-1.0, precision=prec))
     assert np.array_equal(neg, dense)
     assert tq.count_active_positions(dev(w), 1e-5) == o.count_active_positions(w, 1e-5)
 
 
-@pytest.mark.parametrize("n_kv,n_rep", [(4, 2), (2, 4), (4, 7), (2, 9)])
-def test_sparse_v_gqa(tq, n_kv, n_rep):
+@PRECS
+@pytest.mark.parametrize("n_kv,n_rep", [(4, 2), (2, 4), (4, 7), (2, 9), (1, 16), (1, 17)])
+def test_sparse_v_gqa(tq, n_kv, n_rep, prec):
     rng = np.random.default_rng(14)
     S, D, bits = 400, 128, 3
     c, s, vp, vn = v_fixture(rng, n_kv, S, D, bits)
     w = softmax_np(rng.standard_normal((n_kv * n_rep, S)))
     want = o.sparse_v_matvec(w, vp, vn, c, s, D, bits, 0.0, n_rep)
-    got = host(tq.sparse_v_matvec(dev(w), dev(vp), dev(vn), c, dev(s), D, bits, threshold=0.0, n_rep=n_rep))
+    got = host(tq.sparse_v_matvec(dev(w), dev(vp), dev(vn), c, dev(s), D, bits, threshold=0.0, n_rep=n_rep,
+                                  precision=prec))
     assert np.abs(got - want).max() < 1e-5 * np.abs(want).max()
     with pytest.raises(ValueError, match="power of 2"):
         tq.sparse_v_matvec(dev(w), dev(vp), dev(vn), c, dev(s), 96, bits)
@@ -930,10 +942,14 @@ def test_decode_sweep_scores_and_sparse_v(tq, seed):
     w = (w / w.sum(axis=-1, keepdims=True)).astype(F32)
     thr = float(rng.choice([0.0, 1e-5, 1e-3]))
     wantv = o.sparse_v_matvec(w, vp, vn, c, vs, D, bits, threshold=thr, n_rep=n_rep)
-    for precision in ("fp32", "fp16"):
+    for precision in ("fp32", "fp16", None):
         gotv = host(tq.sparse_v_matvec(dev(w), dev(vp), dev(vn), c, dev(vs), D, bits, threshold=thr,
                                        n_rep=n_rep, precision=precision))
         close(gotv, wantv)
+        if precision != "fp16":                         # the reference's bar (tests/test_sparse_v.py:70-75)
+            assert np.abs(gotv - wantv).max() <= 1e-5 * np.abs(wantv).max()
+    s32 = host(tq.prerot_fused_qk_scores(dev(q_rot), dev(kp), dev(kn), c, D, bits, n_rep, precision="fp32"))
+    close(s32, want, rel=1e-5, abs_=max(1e-5, 1e-6 * float(np.abs(want).max())))
 
 
 @pytest.mark.parametrize("seed", range(10))

@@ -9,6 +9,7 @@
 #include "tq_common.h"
 #include "tq_decode_mfma.h"
 #include "tq_packed_mfma.h"
+#include "tq_split_mfma.h"
 
 #include <math.h>
 #include <cmath>
@@ -879,6 +880,16 @@ void launch_packed_tiles_bits(int bits, int mode, bool one_per_cu, dim3 grid, co
   }
 }
 
+
+void launch_split_tiles_bits(int bits, int mode, dim3 grid, const tqm::SplitArgs& a, const Codebook& cb, hipStream_t stream) {
+  switch (bits) {
+    case 1: tqm::launch_split_tiles<1>(mode, grid, a, cb, stream); break;
+    case 2: tqm::launch_split_tiles<2>(mode, grid, a, cb, stream); break;
+    case 4: tqm::launch_split_tiles<4>(mode, grid, a, cb, stream); break;
+    default: tqm::launch_split_tiles<3>(mode, grid, a, cb, stream); break;
+  }
+}
+
 void launch_packed_stream_bits(int bits, dim3 grid, const tqm::PackedArgs& a, const Codebook& kcb, const Codebook& vcb,
                                int n_steps, hipStream_t stream) {
   switch (bits) {
@@ -1165,6 +1176,18 @@ extern "C" int tq_prerot_qk_scores(const float* q_rot, const uint32_t* k_packed,
     return tq::fail(TQ_ERR_NULL, "tq_prerot_qk_scores: null pointer");
   Codebook cb;
   fill_codebook(cb, centroids, bits);
+  if (allow_mma == TQ_MMA_SPLIT && dim == 128 && bits >= 1 && bits <= 4 && n_rep <= tqm::kHeadsMax && tq::aligned(q_rot, 8)) {
+    // split operands (value + remainder, three matrix instructions per tile): float32 fidelity
+    tqm::SplitArgs a{};
+    a.q_rot = q_rot; a.packed = k_packed; a.norms = k_norms; a.scores = scores;
+    a.seq_len = seq_len; a.head_stride = packed_head_stride; a.norms_head_stride = norms_head_stride;
+    a.n_kv = n_kv_heads; a.n_rep = n_rep; a.scale = 1.0f / (float)dim;
+    dim3 grid((unsigned)((seq_len + tqm::kTilePos - 1) / tqm::kTilePos), n_kv_heads);
+    a.n_tiles = (int)grid.x;
+    launch_split_tiles_bits(bits, tqm::kScores, grid, a, cb, (hipStream_t)stream_);
+    TQ_CHECK_LAUNCH("tq_prerot_qk_scores launch");
+    return TQ_OK;
+  }
   if (allow_mma && dim == 128 && bits >= 1 && bits <= 4 && n_rep <= tqm::kHeadsMax && tq::aligned(q_rot, 8)) {
     tqm::PackedArgs a{};
     a.q_rot = q_rot; a.k_packed = k_packed; a.k_norms = k_norms; a.scores = scores;
@@ -1250,6 +1273,29 @@ extern "C" int tq_sparse_v_matvec(const float* weights, const uint32_t* v_packed
     return tq::fail(TQ_ERR_NULL, "tq_sparse_v_matvec: null pointer");
   const float thr = threshold > 0.0f ? threshold : 0.0f;
   sh.allow_mma = allow_mma;
+  if (allow_mma == TQ_MMA_SPLIT && vonly_mma_shape(sh)) {
+    // split operands (value + remainder, three matrix instructions per tile): float32 fidelity
+    const int n_q = n_kv_heads * n_rep;
+    const int n_tiles = (int)((seq_len + tqm::kTilePos - 1) / tqm::kTilePos);
+    const size_t need = (size_t)n_q * n_tiles * (tqm::kD + 2) * sizeof(float);
+    if (!workspace || workspace_bytes < need)
+      return tq::fail(TQ_ERR_WORKSPACE, "tq_sparse_v_matvec: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    if (!tq::aligned(workspace, 16)) return tq::fail(TQ_ERR_ALIGN, "tq_sparse_v_matvec: workspace must be 16-byte aligned");
+    tqm::SplitArgs a{};
+    a.weights = weights; a.w_stride = seq_len; a.packed = v_packed; a.norms = v_norms;
+    a.ws_S = (float*)workspace; a.ws_ml = a.ws_S + (size_t)n_q * n_tiles * tqm::kD;
+    a.seq_len = seq_len; a.head_stride = packed_head_stride; a.norms_head_stride = norms_head_stride;
+    a.n_kv = n_kv_heads; a.n_rep = n_rep; a.n_tiles = n_tiles; a.threshold = thr;
+    Codebook cb;
+    fill_codebook(cb, centroids, bits);
+    hipStream_t stream = (hipStream_t)stream_;
+    launch_split_tiles_bits(bits, tqm::kWeights, dim3(n_tiles, n_kv_heads), a, cb, stream);
+    TQ_CHECK_LAUNCH("tq_sparse_v_matvec launch");
+    tqm::decode_merge_rows_kernel<float, false><<<dim3(n_q, 1), tqm::kMergeThreads, 0, stream>>>(
+        a.ws_S, a.ws_ml, nullptr, seq_len, n_tiles, n_kv_heads, n_rep, signs, 1.0f / (float)dim, out, tqm::kTilePos);
+    TQ_CHECK_LAUNCH("tq_sparse_v_matvec merge launch");
+    return TQ_OK;
+  }
   if (vonly_mma_shape(sh))                                   // packed values only: every width
     return launch_packed_mfma<tqm::kWeights>(weights, nullptr, nullptr, v_packed, v_norms, centroids, centroids,
                                              signs, out, workspace, workspace_bytes, sh, thr,

@@ -13,6 +13,7 @@ LIB_PATH = os.environ.get("TQHIP_LIB", os.path.join(_HERE, "lib", "libtqhip.so")
 
 TQ_F32, TQ_F16, TQ_BF16 = 0, 1, 2
 TQ_ENCODE_MLX, TQ_ENCODE_METAL = 0, 1
+TQ_MMA_OFF, TQ_MMA_FP16, TQ_MMA_SPLIT = 0, 1, 2
 TQ_OP_SPARSE_V, TQ_OP_FLASH_DECODE, TQ_OP_VONLY_DECODE = 0, 1, 2
 
 _p = C.c_void_p

@@ -319,14 +319,27 @@ def _mma_flag(precision: str) -> int:
     return 1 if precision == "fp16" else 0
 
 
+def _mma_mode(precision) -> int:
+    """allow_mma of the two reference-named wrappers: None = float32 fidelity on the fastest kernel
+    (split operands on the matrix cores where the shape allows), "fp32" = the float32 vector kernels,
+    "fp16" = fp16 operands."""
+    if precision is None:
+        return _lib.TQ_MMA_SPLIT
+    return _lib.TQ_MMA_FP16 if _mma_flag(precision) else _lib.TQ_MMA_OFF
+
+
 def prerot_fused_qk_scores(q_rot: torch.Tensor, k_packed: torch.Tensor, k_norms: torch.Tensor,
                            centroids, dim: int, bits: int, n_rep: int = 1,
-                           precision: str = "fp32") -> torch.Tensor:
+                           precision=None) -> torch.Tensor:
     """metal_kernels_v4.py:153-221.  Scores of pre-rotated queries against packed K, GQA-aware.
 
     q_rot (n_q, dim); k_packed (n_kv, seq, pdim); k_norms (n_kv, seq) -> (n_q, seq) float32.
-    precision="fp32" keeps the reference's float32 arithmetic; "fp16" rounds q_rot and the
-    centroids to half and runs on the matrix cores (float32 accumulation, ~3e-4 relative).
+    precision=None (default): float32 fidelity -- at d = 128 and n_rep <= 16 on the matrix cores with
+    every operand as an fp16 value plus the fp16 remainder of its rounding (products exact in float32,
+    ~1e-6 relative; the reference's bar is 1e-4 absolute, tests/test_prerot.py:90-95), other shapes on
+    the float32 vector kernels.  "fp32": the float32 vector kernels for every shape (the reference's
+    operation order).  "fp16": q_rot and the centroids rounded to half on the matrix cores (~3e-4
+    relative).
     """
     _need_gpu(q_rot, k_packed, k_norms)
     n_q = q_rot.shape[0]
@@ -339,7 +352,7 @@ def prerot_fused_qk_scores(q_rot: torch.Tensor, k_packed: torch.Tensor, k_norms:
     out = torch.empty((n_q, seq_len), dtype=torch.float32, device=q_rot.device)
     _lib.check(_lib.load().tq_prerot_qk_scores(
         _ptr(q_rot), _ptr(k_packed), _ptr(k_norms), _host_table(centroids), _ptr(out),
-        n_kv, n_rep, seq_len, phs, nhs, dim, bits, _mma_flag(precision), _stream(q_rot)))
+        n_kv, n_rep, seq_len, phs, nhs, dim, bits, _mma_mode(precision), _stream(q_rot)))
     return out
 
 
@@ -403,12 +416,14 @@ def softmax_rows(scores: torch.Tensor, scale: float = 1.0, mask: torch.Tensor | 
 
 def sparse_v_matvec(weights: torch.Tensor, v_packed: torch.Tensor, v_norms: torch.Tensor, centroids,
                     signs, dim: int, bits: int, threshold: float = 1e-5, n_rep: int = 1,
-                    precision: str = "fp32") -> torch.Tensor:
+                    precision=None) -> torch.Tensor:
     """sparse_v.py:94-186.  Weighted sum of dequantised V rows with the butterfly pulled out of
     the position loop; positions with weight < threshold are skipped; threshold <= 0 is dense.
 
     weights (n_q, seq); v_packed (n_kv, seq, pdim); v_norms (n_kv, seq) -> (n_q, dim) float32.
-    precision as in prerot_fused_qk_scores ("fp16": weights * norm and centroids rounded to half).
+    precision as in prerot_fused_qk_scores (None: weights * norm and centroids as value + remainder on
+    the matrix cores, within the reference's 1e-5 of the largest output, tests/test_sparse_v.py:70-75;
+    "fp16": both rounded to half).
     """
     if dim & (dim - 1):
         raise ValueError(f"dim must be a power of 2, got {dim}")
@@ -431,7 +446,7 @@ def sparse_v_matvec(weights: torch.Tensor, v_packed: torch.Tensor, v_norms: torc
     _lib.check(lib.tq_sparse_v_matvec(
         _ptr(weights), _ptr(v_packed), _ptr(v_norms), _host_table(centroids), _ptr(signs), _ptr(out),
         _ptr(ws), ws.numel(), n_kv, n_rep, seq_len, phs, nhs, dim, bits, float(max(threshold, 0.0)),
-        _mma_flag(precision), stream))
+        _mma_mode(precision), stream))
     return out
 
 
