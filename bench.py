@@ -38,6 +38,7 @@ N_SETS = 10
 MIN_TIMED_MS = 50.0       # GPU time every timed quantity is measured over (at least 5 replays)
 MIN_SAMPLE_MS = 2.0      # GPU time between two event records of the timed region
 READ_WGS = 2048           # workgroups of the plain-read probe (8 per CU)
+THRESHOLD = 1e-5          # sparse-V threshold of the secondary figure: the reference's default (sparse_v.py:102)
 
 # HBM bytes per launch of the dominant kernel (the tile pass), from two rocprofv3 --pmc runs of
 # `python bench.py --steps 60 --warmup 6 --no-cpu --no-graph --no-ceiling` (FETCH_SIZE, then WRITE_SIZE), each
@@ -77,6 +78,7 @@ def cpu_baseline(torch, sets, cb, signs, budget_s=12.0):
     def run():
         return orc.vonly_decode_attention(q[0], k, vp, vn, cbn, sg, D, BITS, sc)
     ref = run()                       # warm-up, and the reference output for the check below
+    ref_thr = orc.vonly_decode_attention(q[0], k, vp, vn, cbn, sg, D, BITS, sc, threshold=THRESHOLD)
     t0 = time.perf_counter()
     n = 0
     while True:
@@ -91,7 +93,7 @@ def cpu_baseline(torch, sets, cb, signs, budget_s=12.0):
         threads = max([p.get("num_threads", 1) for p in threadpool_info()] or [1])
     except Exception:
         threads = 1
-    return ref, {
+    return ref, ref_thr, {
         "value": round(ALGO_BYTES / per / 1e9, 3), "unit": "GB/s", "us_per_layer": round(per * 1e6, 1),
         "cores": threads, "kind": "port",
         "sample": f"{n} full-size steps (28/4 heads, d=128, T=32768) of the numpy oracle; its matmuls run "
@@ -168,12 +170,35 @@ def main():
     step(0, eager_args)
     torch.cuda.synchronize()
     checked = outs[0].clone()
+
+    # secondary: the same step with the reference's default sparse-V threshold on the FINAL softmax weights
+    # (tq_vonly_sparse_decode_attn: scores pass, weights + values pass, merge pass)
+    thr_ws_bytes = lib.tq_vonly_sparse_workspace_bytes(1, N_Q, T)
+    thr_ws = torch.zeros(thr_ws_bytes, dtype=torch.uint8, device=dev)
+    thr_out = torch.empty((1, N_Q, D), dtype=torch.float32, device=dev)
+
+    def thr_step(i, stream):
+        q, k, vp, vn = sets[i % N_SETS]
+        rc = lib.tq_vonly_sparse_decode_attn(
+            C.c_void_p(q.data_ptr()), _lib.TQ_F16, C.c_void_p(k.data_ptr()), C.c_void_p(vp.data_ptr()),
+            C.c_void_p(vn.data_ptr()), cb_host, C.c_void_p(signs.data_ptr()), C.c_float(THRESHOLD),
+            C.c_void_p(thr_out.data_ptr()), C.c_void_p(thr_ws.data_ptr()), thr_ws.numel(), C.byref(shape),
+            C.c_void_p(stream))
+        if rc != 0:
+            _lib.check(rc)
+    thr_step(0, cur.cuda_stream)
+    torch.cuda.synchronize()
+    thr_checked = thr_out.clone()
     cpu = None
     if not args.no_cpu and not args.calibrate_read:
-        ref, cpu = cpu_baseline(torch, sets, cb, signs)
+        ref, ref_thr, cpu = cpu_baseline(torch, sets, cb, signs)
         err = np.abs(outs[0][0].cpu().numpy() - ref)
         if not np.all(err <= 1e-3 + 2e-3 * np.abs(ref)):
             print(f"bench: GPU output disagrees with the oracle (max err {err.max():.3e})", file=sys.stderr)
+            sys.exit(1)
+        err = np.abs(thr_checked[0].cpu().numpy() - ref_thr)
+        if not np.all(err <= 1e-3 + 2e-3 * np.abs(ref_thr)):
+            print(f"bench: thresholded GPU output disagrees with the oracle (max err {err.max():.3e})", file=sys.stderr)
             sys.exit(1)
 
     side = torch.cuda.Stream(device=dev)
@@ -275,9 +300,17 @@ def main():
     ms_per_step, ms_min, ms_max, n_replays = timed(decode_step(3))    # whole step: tile pass + merge pass
     ms_tile, tile_min, tile_max, _ = timed(decode_step(1))            # dominant kernel alone, same launch pattern
     ms_warm = timed(decode_step(3, rot=1))[0]   # one buffer set over and over: its 41 MB stay in the 256 MB Infinity Cache
+    ms_thr, thr_min, thr_max, _ = timed(thr_step)
     gbs = ALGO_BYTES / (ms_per_step * 1e-3) / 1e9
     gbs_tile = ALGO_BYTES / (ms_tile * 1e-3) / 1e9
     ceiling = None if args.no_ceiling else read_ceiling()
+    if ceiling is not None:
+        ceiling["frac_of_step"] = round(ceiling["us_per_launch"] / (ms_per_step * 1e3), 4)
+    thr_step(0, cur.cuda_stream)
+    torch.cuda.synchronize()
+    if not torch.equal(thr_out, thr_checked):
+        print("bench: the timed thresholded steps left a result that differs from the checked one", file=sys.stderr)
+        sys.exit(1)
     step(0, eager_args)                         # leave outs[0] = the full result of set 0
     torch.cuda.synchronize()
 
@@ -308,6 +341,13 @@ def main():
                    if not args.no_graph else "one pass of eager launches",
                    "replays": n_replays, "us_per_layer_min": round(ms_min * 1e3, 3), "us_per_layer_max": round(ms_max * 1e3, 3),
                    "tile_us_min": round(tile_min * 1e3, 3), "tile_us_max": round(tile_max * 1e3, 3)},
+        "threshold_1e-5": {"us_per_layer": round(ms_thr * 1e3, 3), "min": round(thr_min * 1e3, 3), "max": round(thr_max * 1e3, 3),
+                           "value": round(ALGO_BYTES / (ms_thr * 1e-3) / 1e9, 1), "unit": "GB/s",
+                           "pct_hbm_peak": round(100 * ALGO_BYTES / (ms_thr * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
+                           "note": "the same step with the reference's default sparse-V threshold (sparse_v.py:102) applied to "
+                                   "the final softmax weights: tq_vonly_sparse_decode_attn (scores pass, weights + values "
+                                   "pass, merge pass), timed like `value`, checked against the oracle; algorithmic bytes as for "
+                                   "the dense step (the scores written and re-read between the passes are not counted)"},
         "warm_cache": {"us_per_layer": round(ms_warm * 1e3, 3), "value": round(ALGO_BYTES / (ms_warm * 1e-3) / 1e9, 1),
                        "unit": "GB/s", "note": "same step on ONE buffer set (inputs served from the Infinity Cache); "
                                                "reported beside `value`, never as it"},

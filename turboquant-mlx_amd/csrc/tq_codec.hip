@@ -273,8 +273,14 @@ __global__ __launch_bounds__(kBlock) void encode128x3_kernel(const T* __restrict
       for (int j = 0; j < NM; ++j) sm[k][j] = __float_as_uint(sv[j & 7]) & 0x80000000u;
     }
   }
-  const uint32_t flip1 = (ls & 1) ? 0x80000000u : 0u;          // upper lane of a pair computes partner - own
-  const uint32_t flip2 = (ls & 2) ? 0x80000000u : 0u;
+  // lanes 1 and 2 of a vector take their inputs negated (folded into the sign masks): butterfly_4lane_neg12
+  if (ls == 1 || ls == 2) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+#pragma unroll
+      for (int j = 0; j < NM; ++j) sm[k][j] ^= kHalfWidth ? 0x80008000u : 0x80000000u;
+  }
+  const float m1 = (ls & 1) ? 1.0f : -1.0f, m2 = (ls & 2) ? 1.0f : -1.0f;
   uint32_t* chunks = chunk_s[wave];
 
   // first batch of 16 rows of this wavefront and its place in the (group, row) map
@@ -368,7 +374,7 @@ __global__ __launch_bounds__(kBlock) void encode128x3_kernel(const T* __restrict
           xs[k][j] = __fmaf_rn(rem, rinv, q0);
         }
       }
-    butterfly_4lane(xs, flip1, flip2);
+    butterfly_4lane_neg12(xs, m1, m2);
     // ---- levels, 8 * BITS bits per chunk
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
@@ -484,7 +490,8 @@ __global__ __launch_bounds__(kBlock) void dequant128x3_kernel(const uint32_t* __
   constexpr int kPairs = 1 << (2 * BITS);                      // entries of the centroid-pair table
   constexpr int kWordLoads = (kEncVecs * kPd + 63) / 64;       // wave-wide loads of a pass's packed words
   __shared__ __align__(16) float sg_s[128];
-  __shared__ __align__(8) float2 pair_s[kPairs < 64 ? 64 : kPairs];
+  // centroid pairs, and after them the same pairs negated: lanes 1 and 2 of a vector read those (butterfly_4lane_neg12)
+  __shared__ __align__(8) float2 pair_s[2 * kPairs];
   __shared__ uint32_t words_s[kWavesPerBlock][kEncVecs * kPd + 3];
   // Outputs leave through LDS: 16 rows of 256 (16-bit) or 512 (float32) bytes at a padded pitch (conflict-free
   // 16-byte writes per lane and reads per row segment), so that every store instruction writes 1 KB of
@@ -504,6 +511,7 @@ __global__ __launch_bounds__(kBlock) void dequant128x3_kernel(const uint32_t* __
       chi = ((tid >> BITS) == i) ? cbk.c[i] : chi;
     }
     pair_s[tid] = make_float2(clo * s, chi * s);
+    pair_s[kPairs + tid] = make_float2(-(clo * s), -(chi * s));
   }
   if (tid >= 128) sg_s[tid - 128] = signs[tid - 128];
   __syncthreads();
@@ -517,8 +525,8 @@ __global__ __launch_bounds__(kBlock) void dequant128x3_kernel(const uint32_t* __
 #pragma unroll
     for (int j = 0; j < 8; ++j) sm[k][j] = __float_as_uint(sv[j]) & 0x80000000u;
   }
-  const uint32_t flip1 = (ls & 1) ? 0x80000000u : 0u;
-  const uint32_t flip2 = (ls & 2) ? 0x80000000u : 0u;
+  const float m1 = (ls & 1) ? 1.0f : -1.0f, m2 = (ls & 2) ? 1.0f : -1.0f;
+  const float2* my_pairs = pair_s + ((ls == 1 || ls == 2) ? kPairs : 0);
   uint32_t* words = words_s[wave];
   // words / shifts of the bits of chunk c = ls + 4k (elements 8c .. 8c+7)
   int cw[4], csl[4], csh[4];
@@ -560,12 +568,12 @@ __global__ __launch_bounds__(kBlock) void dequant128x3_kernel(const uint32_t* __
       const uint32_t f = CK::field(words + v * kPd + cw[k], csl[k], csh[k]);
 #pragma unroll
       for (int jp = 0; jp < 4; ++jp) {
-        const float2 c2 = pair_s[(f >> (2 * BITS * jp)) & CK::kPairMask];
+        const float2 c2 = my_pairs[(f >> (2 * BITS * jp)) & CK::kPairMask];
         xs[k][2 * jp] = c2.x;
         xs[k][2 * jp + 1] = c2.y;
       }
     }
-    butterfly_4lane(xs, flip1, flip2);
+    butterfly_4lane_neg12(xs, m1, m2);
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       float r[8];

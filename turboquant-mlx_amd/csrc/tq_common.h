@@ -252,6 +252,57 @@ __device__ __forceinline__ void butterfly_4lane(float (&xs)[4][8], uint32_t flip
   }
 }
 
+// butterfly_4lane for inputs that the lanes with ls = 1 and ls = 2 hold NEGATED -- a sign the caller folds into the
+// sign flip or the table it applies to its inputs anyway.  Each of the two lane-exchange stages is then ONE fused
+// multiply-add, own + partner * (+-1), instead of a sign flip and an add: with the value a of the lower lane and b
+// of the upper lane of a pair, (own, partner, factor) = (a, -b, -1) gives a + b and (-b, a, +1) gives a - b; in the
+// pairs whose results the next stage wants negated, (-a, b, -1) gives -(a + b) and (b, -a, +1) gives -(a - b).  A
+// product with +-1 is exact, so every output is the same single rounding of the same sum as in butterfly_4lane:
+// identical bits (the sign of a zero aside, which no consumer looks at).  m1 = (ls & 1) ? 1 : -1,
+// m2 = (ls & 2) ? 1 : -1.  Outputs are not negated in any lane.
+__device__ __forceinline__ void butterfly_4lane_neg12(float (&xs)[4][8], float m1, float m2) {
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+#pragma unroll
+    for (int h = 1; h < 8; h <<= 1)
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (!(j & h)) {
+          const float a = xs[k][j], b = xs[k][j + h];
+          xs[k][j] = a + b;
+          xs[k][j + h] = a - b;
+        }
+  }
+  // v_fmac_f32 with the partner lane's value as its DPP operand, eight registers per statement (the compiler does
+  // not form this instruction from a quad permute and a fused multiply-add: it leaves the permute a move of its
+  // own).  A DPP read of a register that a vector instruction has just written needs two wait states, which the
+  // compiler does not count across an asm statement: each statement starts with them.
+#define TQ_FMAC8(PERM, M, R)                                                                                        \
+  asm("s_nop 1\n\t"                                                                                                \
+      "v_fmac_f32_dpp %0, %0, %8 quad_perm:" PERM " row_mask:0xf bank_mask:0xf\n\t"                                 \
+      "v_fmac_f32_dpp %1, %1, %8 quad_perm:" PERM " row_mask:0xf bank_mask:0xf\n\t"                                 \
+      "v_fmac_f32_dpp %2, %2, %8 quad_perm:" PERM " row_mask:0xf bank_mask:0xf\n\t"                                 \
+      "v_fmac_f32_dpp %3, %3, %8 quad_perm:" PERM " row_mask:0xf bank_mask:0xf\n\t"                                 \
+      "v_fmac_f32_dpp %4, %4, %8 quad_perm:" PERM " row_mask:0xf bank_mask:0xf\n\t"                                 \
+      "v_fmac_f32_dpp %5, %5, %8 quad_perm:" PERM " row_mask:0xf bank_mask:0xf\n\t"                                 \
+      "v_fmac_f32_dpp %6, %6, %8 quad_perm:" PERM " row_mask:0xf bank_mask:0xf\n\t"                                 \
+      "v_fmac_f32_dpp %7, %7, %8 quad_perm:" PERM " row_mask:0xf bank_mask:0xf"                                      \
+      : "+v"(R[0]), "+v"(R[1]), "+v"(R[2]), "+v"(R[3]), "+v"(R[4]), "+v"(R[5]), "+v"(R[6]), "+v"(R[7])              \
+      : "v"(M))
+#pragma unroll
+  for (int k = 0; k < 4; ++k) TQ_FMAC8("[1,0,3,2]", m1, xs[k]);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) TQ_FMAC8("[2,3,0,1]", m2, xs[k]);
+#undef TQ_FMAC8
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const float a0 = xs[0][j] + xs[1][j], a1 = xs[0][j] - xs[1][j];
+    const float a2 = xs[2][j] + xs[3][j], a3 = xs[2][j] - xs[3][j];
+    xs[0][j] = a0 + a2; xs[2][j] = a0 - a2;
+    xs[1][j] = a1 + a3; xs[3][j] = a1 - a3;
+  }
+}
+
 // Reductions over the four 16-lane rows of a wave (lanes l, l ^ 16, l ^ 32, l ^ 48), result in every lane: row
 // swaps in the vector ALU (v_permlane16_swap: rows 1, 3 of the first operand change places with rows 0, 2 of the
 // second; v_permlane32_swap: the upper half of the first with the lower half of the second) instead of two trips
