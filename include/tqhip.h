@@ -488,7 +488,14 @@ size_t tq_workspace_bytes(int op, int n_seq, int n_q_heads, int64_t max_seq_len,
  * Matrix-core kernel: q_rot, the centroids and softmax weights * value norm are fp16 operands,
  * accumulation is float32.  dim 128 only, every width (TQ_ERR_UNSUPPORTED otherwise).  The workspace
  * (tq_prefill_workspace_bytes, 256-byte aligned) is scratch as for the decode ops.
+ * flags: TQ_PREFILL_CAUSAL (row i sees positions <= q_pos0 + i); TQ_PREFILL_FP16_QUERY: the rotated
+ * query enters as ONE fp16 number per element instead of value + remainder (a third fewer matrix
+ * instructions).  The logit error of that rounding (~4e-4) is harmless on ordinary data but reaches
+ * 1e-2 of an output row when an outlier channel of V cancels in the average, so it is off unless
+ * the caller sets it.
  */
+enum tq_prefill_flags { TQ_PREFILL_CAUSAL = 1, TQ_PREFILL_FP16_QUERY = 2 };
+
 int tq_prefill_attn(const void* q, int q_dtype,
                     const uint32_t* k_packed, const float* k_norms,
                     const uint32_t* v_packed, const float* v_norms,
@@ -498,7 +505,7 @@ int tq_prefill_attn(const void* q, int q_dtype,
                     int n_kv_heads, int n_rep, int64_t n_rows, int64_t kv_len, int64_t q_pos0,
                     int64_t k_head_stride, int64_t kn_head_stride,
                     int64_t v_head_stride, int64_t vn_head_stride,
-                    int dim, int bits, float attn_scale, int causal, tq_stream_t stream);
+                    int dim, int bits, float attn_scale, int flags, tq_stream_t stream);
 
 size_t tq_prefill_workspace_bytes(int n_q_heads, int64_t n_rows, int64_t kv_len, int dim);
 

@@ -745,6 +745,33 @@ def test_prefill_attention_noncausal_fp16_out_and_outliers(tq):
         assert (err <= 1e-3 + 3e-3 * scale).all(), (err / scale).max()     # + fp16 rounding of the output
 
 
+def test_prefill_attention_fp16_query_flag(tq):
+    """fp16_query=True (the rotated query as one fp16 number per element, a third fewer matrix instructions) meets
+    the elementwise bar on N(0,1) data -- and does NOT meet the outlier test's bar on data with x20 outlier channels,
+    which is why it is off by default: the default path must keep passing that test with its remainder in."""
+    rng = np.random.default_rng(51)
+    n_kv, n_rep, T, n_rows, pos0 = 2, 4, 1000, 256, 744
+    c, ks, vs, kp, kn, vp, vn, q = _prefill_case(rng, n_kv, n_rep, T, n_rows)
+    sc = 1 / math.sqrt(128)
+    want = o.prefill_attention(q, kp, kn, vp, vn, c, c, ks, vs, 128, 3, sc, pos0, n_rep)
+    got = tq.prefill_attention(dev(q), dev(kp), dev(kn), dev(vp), dev(vn), c, c, dev(ks), dev(vs), 128, 3, sc,
+                               n_rep=n_rep, q_pos0=pos0, out_dtype=torch.float32, fp16_query=True)
+    close(host(got).reshape(-1, 128), want.reshape(-1, 128))
+    rng = np.random.default_rng(52)
+    n_kv, n_rep, T, n_rows = 2, 4, 1500, 200
+    c, ks, vs, kp, kn, vp, vn, q = _prefill_case(rng, n_kv, n_rep, T, n_rows, outliers=True)
+    want = o.prefill_attention(q, kp, kn, vp, vn, c, c, ks, vs, 128, 3, sc, T - n_rows, n_rep)
+    errs = {}
+    for flag in (False, True):
+        got = tq.prefill_attention(dev(q), dev(kp), dev(kn), dev(vp), dev(vn), c, c, dev(ks), dev(vs), 128, 3, sc,
+                                   n_rep=n_rep, out_dtype=torch.float32, fp16_query=flag)
+        err = np.abs(host(got).astype(np.float64) - want)
+        scale = np.abs(want).max(axis=-1, keepdims=True)
+        errs[flag] = float(((err - 1e-3) / scale).max())
+    assert errs[False] <= 2e-3, errs
+    assert errs[True] > 2e-3, errs                    # the flag is refused by the bar of the outlier test
+
+
 def test_prefill_attention_equals_decode_rows(tq):
     """Each row of a prefill chunk is one decode step over its prefix: compare with the
     float32 flash decode kernel of this library (independent code path)."""

@@ -64,7 +64,9 @@ struct PrefillArgs {
 // cancels in the average), the online softmax on its accumulators, and O += P V with the
 // accumulator registers of S^T reused as the A operand.  The packed words of the next block are
 // fetched while the current one is computed.
-template <int BITS>
+// QLO = false leaves the query remainder out (one matrix instruction per key operand instead of two): for callers
+// that declare their data free of outlier channels.
+template <int BITS, bool QLO = true>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void prefill_tile_kernel(PrefillArgs a, Codebook kcb, Codebook vcb) {
   using PF = PackedField<BITS>;
@@ -111,7 +113,7 @@ void prefill_tile_kernel(PrefillArgs a, Codebook kcb, Codebook vcb) {
       if (r < a.n_rows) {
         const int64_t off = ((int64_t)head * a.n_rows + r) * kD + 32 * kb + 8 * g;
         vh = *reinterpret_cast<const u4*>(a.q_rot + off);
-        vl = *reinterpret_cast<const u4*>(a.q_rot_lo + off);
+        if (QLO) vl = *reinterpret_cast<const u4*>(a.q_rot_lo + off);
       }
       qhi[ct][kb] = vh;
       qlo[ct][kb] = vl;
@@ -231,9 +233,10 @@ void prefill_tile_kernel(PrefillArgs a, Codebook kcb, Codebook vcb) {
         const u4 A = kreg[i % 3];
 #pragma unroll
         for (int ct = 0; ct < kRowTiles; ++ct) {
-          sacc[i >> 2][ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, A),
-                                                                    __builtin_bit_cast(h8, qlo[ct][i & 3]),
-                                                                    sacc[i >> 2][ct], 0, 0, 0);
+          if (QLO)
+            sacc[i >> 2][ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, A),
+                                                                      __builtin_bit_cast(h8, qlo[ct][i & 3]),
+                                                                      sacc[i >> 2][ct], 0, 0, 0);
           sacc[i >> 2][ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, A),
                                                                     __builtin_bit_cast(h8, qhi[ct][i & 3]),
                                                                     sacc[i >> 2][ct], 0, 0, 0);
@@ -502,8 +505,11 @@ extern "C" int tq_prefill_attn(const void* q, int q_dtype, const uint32_t* k_pac
                                int out_dtype, void* workspace, size_t workspace_bytes, int n_kv_heads, int n_rep,
                                int64_t n_rows, int64_t kv_len, int64_t q_pos0, int64_t k_head_stride,
                                int64_t kn_head_stride, int64_t v_head_stride, int64_t vn_head_stride, int dim,
-                               int bits, float attn_scale, int causal, tq_stream_t stream_) {
+                               int bits, float attn_scale, int flags, tq_stream_t stream_) {
   const char* who = "tq_prefill_attn";
+  if (flags & ~(TQ_PREFILL_CAUSAL | TQ_PREFILL_FP16_QUERY))
+    return tq::fail(TQ_ERR_ARG, "%s: unknown flag bits 0x%x", who, flags);
+  const int causal = flags & TQ_PREFILL_CAUSAL;
   if (int rc = tq::check_dim_bits(dim, bits)) return rc;
   if (dim != kD)
     return tq::fail(TQ_ERR_UNSUPPORTED, "%s: only dim 128 has a kernel, got dim %d", who, dim);
@@ -562,7 +568,11 @@ extern "C" int tq_prefill_attn(const void* q, int q_dtype, const uint32_t* k_pac
   const float v_unscale = tq::fill_codebook_fp16(vcb, v_centroids, bits);
   a.score_scale = attn_scale / (float)dim * k_unscale * kLog2e;
   dim3 grid(plan.n_splits, (unsigned)((n_rows + kWgRows - 1) / kWgRows), n_q);
-  TQ_DISPATCH_BITS(bits, (prefill_tile_kernel<B_><<<grid, kThreads, 0, stream>>>(a, kcb, vcb)));
+  if (flags & TQ_PREFILL_FP16_QUERY) {
+    TQ_DISPATCH_BITS(bits, (prefill_tile_kernel<B_, false><<<grid, kThreads, 0, stream>>>(a, kcb, vcb)));
+  } else {
+    TQ_DISPATCH_BITS(bits, (prefill_tile_kernel<B_><<<grid, kThreads, 0, stream>>>(a, kcb, vcb)));
+  }
   TQ_CHECK_LAUNCH("tq_prefill_attn tile pass");
 
   const float unscale = v_unscale / kVnScale / (float)dim;

@@ -325,14 +325,16 @@ def bench_prefill(iters, dev):
     for T in (8192, 32768, 131072):
         (kp, kn), (vp, vn) = packed_sets(8, T, dev, 1, 8)[0], packed_sets(8, T, dev, 1, 9)[0]
         q = torch.randn((32, n_rows, 128), device=dev, dtype=torch.float16)
-        fn = lambda: tqhip.prefill_attention(q, kp, kn, vp, vn, cb, cb, ks, vs, 128, 3, 1 / math.sqrt(128), n_rep=4)
-        us = timeit([fn], max(5, iters // 20), warmup=2)
         visible = sum(T - n_rows + i + 1 for i in range(n_rows))
         flops = 4.0 * 32 * 128 * visible
         nbytes = 8 * T * 112 + 2 * 32 * n_rows * 256
-        print(f"config 5: prefill chunk 512 rows x 32/8 heads, T={T:<7d} {us:10.1f} us  {flops / us / 1e6:8.1f} TFLOP/s  "
-              f"{100 * flops / us / 1e6 / 2500:5.1f} % of 2.5 PFLOP/s  ({nbytes / us / 1e3:6.1f} GB/s of packed cache)",
-              flush=True)
+        for flag, label in ((False, "value + remainder query (default)"), (True, "fp16_query=True")):
+            fn = lambda: tqhip.prefill_attention(q, kp, kn, vp, vn, cb, cb, ks, vs, 128, 3, 1 / math.sqrt(128), n_rep=4,
+                                                 fp16_query=flag)
+            us = timeit([fn], max(5, iters // 20), warmup=2)
+            print(f"config 5: prefill chunk 512 rows x 32/8 heads, T={T:<7d} {label}: {us:10.1f} us  "
+                  f"{flops / us / 1e6:8.1f} TFLOP/s  {100 * flops / us / 1e6 / 2500:5.1f} % of 2.5 PFLOP/s  "
+                  f"({nbytes / us / 1e3:6.1f} GB/s of packed cache)", flush=True)
 
 
 def bench_step(iters, dev):
