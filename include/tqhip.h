@@ -254,7 +254,9 @@ int tq_flash_decode(const float* q_rot,
  * 0 = one workgroup per 512-position tile; n >= 2 = the streaming pass, one workgroup per
  * n * 256 consecutive positions (large unmasked batches).  Informational: lets a caller or a test
  * know which kernel a shape exercises.  No counterpart in the reference (one kernel per call,
- * flash_attention.py:168-274).
+ * flash_attention.py:168-274).  The plan sees no pointers: it describes three-bit tensors (rows at any
+ * 4-byte offset) and tensors of widths 1, 2 and 4 that are 16-byte aligned; tq_flash_decode sends a
+ * tensor of width 1, 2 or 4 at another offset to the tile pass whatever the plan says.
  */
 int tq_flash_decode_plan(int n_seq, int n_kv_heads, int64_t max_seq_len, int ragged, int masked);
 
@@ -266,6 +268,9 @@ int tq_flash_decode_plan(int n_seq, int n_kv_heads, int64_t max_seq_len, int rag
  *   q [n_seq, n_kv*n_rep, dim] dtype q_dtype;  k_f16 rows of dim halfs;  out as tq_flash_decode.
  * With allow_mma, d = 128 and n_rep <= 16 the tile pass runs on the matrix cores for values of every
  * width (bits 1-4, as adaptive.py:26 / v_only_cache.py:41 take them); other shapes take the float32 kernels.
+ * Alignment: k_f16 16 bytes (TQ_ERR_ALIGN otherwise).  The matrix-core pass reads q in 16-byte pieces: a q
+ * that is not 16-byte aligned (a view at an odd element offset) is served by the float32 kernels instead,
+ * same result to their rounding, several times slower.
  */
 int tq_vonly_decode_attn(const void* q, int q_dtype, const void* k_f16,
                          const uint32_t* v_packed, const float* v_norms,
@@ -325,6 +330,8 @@ typedef struct tq_vonly_cache_desc {
  * attention of hybrid_attention.py:52-88 / fused_attention.py:50-121 (v_only_cache.py:52-78).
  *   k_new, v_new [n_seq, n_kv_heads, dim];  q [n_seq, n_kv_heads*n_rep, dim];  out likewise, out_dtype
  * Fails with TQ_ERR_ARG when position is outside 0 .. t_alloc - 1.
+ * Alignment: the two-launch path needs q and cache->k_f16 16-byte aligned; with another q (or k_f16) the
+ * call runs tq_vonly_append followed by tq_vonly_decode_attn, whose own rules then apply.
  */
 int tq_vonly_decode_step(const tq_vonly_cache_desc* cache /* host */,
                          const void* k_new, int k_dtype, const void* v_new, int v_dtype,
@@ -349,7 +356,8 @@ int tq_vonly_append_at(const void* k_new, int k_dtype, const void* v_new, int v_
  * *position_dev and attends over positions 0 .. *position_dev (clamped to the storage).  Grids and the
  * workspace are sized for t_alloc positions, so the same recorded launches serve every step until the
  * storage is reallocated; the caller advances the counter between steps (on the same stream).
- * dim 128 (values of any width) and n_rep <= 16 only (TQ_ERR_UNSUPPORTED otherwise).
+ * dim 128 (values of any width), n_rep <= 16 and 16-byte aligned q and cache->k_f16 only (TQ_ERR_UNSUPPORTED
+ * otherwise: there is no fallback that reads the position on the device); position_dev 8-byte aligned.
  */
 int tq_vonly_decode_step_at(const tq_vonly_cache_desc* cache /* host */,
                             const void* k_new, int k_dtype, const void* v_new, int v_dtype,
@@ -424,8 +432,9 @@ int tq_vonly_decode_attn_phases(const void* q, int q_dtype, const void* k_f16,
  * a scores pass, a weights-and-values pass and the merge pass, with the scores of the step held in `workspace`
  * (tq_vonly_sparse_workspace_bytes) instead of three tensors of the caller.  Arguments as tq_vonly_decode_attn;
  * threshold >= 0 (0 = dense: every position contributes).  Rows whose positions are all masked out yield zeros.
- * Matrix-core shape only: dim 128, values of any width (bits 1-4), n_rep <= 16, non-empty cache
- * (TQ_ERR_UNSUPPORTED otherwise: compose tq_dense_qk_scores, tq_softmax_rows and tq_sparse_v_matvec for those).
+ * Matrix-core shape only: dim 128, values of any width (bits 1-4), n_rep <= 16, non-empty cache, 16-byte
+ * aligned q (TQ_ERR_UNSUPPORTED otherwise: compose tq_dense_qk_scores, tq_softmax_rows and tq_sparse_v_matvec
+ * for those); k_f16 16-byte aligned (TQ_ERR_ALIGN otherwise).
  */
 int tq_vonly_sparse_decode_attn(const void* q, int q_dtype, const void* k_f16,
                                 const uint32_t* v_packed, const float* v_norms,

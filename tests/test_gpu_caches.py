@@ -594,6 +594,63 @@ def test_vonly_decode_step_refuses_bad_positions(tq):
         assert np.allclose(host(out[0, h]), want[h // 2], rtol=2e-3, atol=1e-3)
 
 
+def _offset_view(t, n_elems=1):
+    """The same values in a contiguous tensor whose storage starts n_elems elements past a fresh allocation:
+    4 bytes off a 16-byte boundary for float32, 2 bytes for fp16."""
+    buf = torch.empty(t.numel() + n_elems, dtype=t.dtype, device=t.device)
+    view = buf[n_elems:].view(t.shape)
+    view.copy_(t)
+    assert view.is_contiguous() and view.data_ptr() % 16 == n_elems * t.element_size()
+    return view
+
+
+@pytest.mark.parametrize("qdt", [torch.float32, torch.float16])
+def test_vonly_entries_with_a_query_off_the_16_byte_boundary(tq, qdt):
+    """The matrix-core V-only kernels read q in 16-byte pieces.  A q view one element past a boundary must never
+    reach them: tq_vonly_decode_attn and tq_vonly_decode_step serve it through the float32 kernels (same result
+    to the bar), tq_vonly_sparse_decode_attn and tq_vonly_decode_step_at refuse it (UNSUPPORTED), and nothing is
+    written by a refused call."""
+    from tqhip import ops
+    B, n_kv, n_rep, T, D = 1, 2, 7, 700, 128
+    n_q = n_kv * n_rep
+    sc = 1 / math.sqrt(D)
+    c = tq.VOnlyTurboQuantCache(bits=3, fused=True)
+    c.update_and_fetch(rand((B, n_kv, T, D), 1700), rand((B, n_kv, T, D), 1701))
+    kc, vt = c._k_cache, c._v_tq
+    K, vp, vn = kc.keys[:, :, :T], vt.v_packed[:, :, :T], vt.v_norms[:, :, :T]
+    cb, sg = vt._v_q.centroids, vt._v_q.signs
+    q = rand((B, n_q, D), 1702, qdt)
+    q_off = _offset_view(q)
+    want = tq.vonly_decode(q, K, vp, vn, cb, sg, D, 3, sc, n_rep=n_rep, seq_len=T)
+    got = tq.vonly_decode(q_off, K, vp, vn, cb, sg, D, 3, sc, n_rep=n_rep, seq_len=T)
+    assert bool(((got - want).abs() <= 1e-3 + 2e-3 * want.abs()).all())
+    fp32 = tq.vonly_decode(q, K, vp, vn, cb, sg, D, 3, sc, n_rep=n_rep, seq_len=T, precision="fp32")
+    assert torch.equal(got, fp32), "a q off the boundary is served by the float32 kernels"
+    out = torch.full((B, n_q, D), 7.0, device="cuda")
+    with pytest.raises(RuntimeError, match="aligned q"):
+        tq.vonly_decode(q_off, K, vp, vn, cb, sg, D, 3, sc, n_rep=n_rep, seq_len=T, sparse_v_threshold=1e-5, out=out)
+    torch.cuda.synchronize()
+    assert bool((out == 7.0).all())
+    # the single-call step: host position -> two-call route, device position -> refused
+    k1, v1 = rand((B, n_kv, D), 1703), rand((B, n_kv, D), 1704)
+    twin = tq.VOnlyTurboQuantCache(bits=3, fused=True)
+    twin.update_and_fetch(rand((B, n_kv, T, D), 1700), rand((B, n_kv, T, D), 1701))
+    a = c.decode_step(q.view(B, n_q, 1, D), k1.view(B, n_kv, 1, D), v1.view(B, n_kv, 1, D), sc)
+    b = twin.decode_step(q_off.view(B, n_q, 1, D), k1.view(B, n_kv, 1, D), v1.view(B, n_kv, 1, D), sc)
+    assert bool(((a.float() - b.float()).abs() <= 1e-3 + 2e-3 * a.float().abs()).all())
+    for x, y in zip(c.state, twin.state):
+        assert torch.equal(x, y)
+    pos = torch.tensor([c.offset], dtype=torch.int64, device="cuda")
+    c.reserve(B, n_kv, 4, D)
+    before = [t.clone() for t in c.state]
+    with pytest.raises(RuntimeError, match="aligned q"):
+        c.decode_step(q_off.view(B, n_q, 1, D), k1.view(B, n_kv, 1, D), v1.view(B, n_kv, 1, D), sc, position=pos,
+                      out=torch.empty((B, n_q, 1, D), dtype=q.dtype, device="cuda"))
+    torch.cuda.synchronize()
+    for x, y in zip(c.state, before):
+        assert torch.equal(x, y)
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_packed_cache_decode_step_is_update_plus_attention(tq, dtype):
     """TurboQuantKVCache.decode_step (tq_packed_decode_step: the tile pass over the old positions + a merge pass

@@ -449,6 +449,30 @@ def test_sparse_v_gqa(tq, n_kv, n_rep, prec):
         tq.sparse_v_matvec(dev(w[:-1]), dev(vp), dev(vn), c, dev(s), D, bits, n_rep=n_rep)
 
 
+@pytest.mark.parametrize("S", [512, 2048, 8192, 16384])
+def test_sparse_v_reference_benchmark_grid(tq, S):
+    """The grid of the reference's micro-benchmark (scripts/bench_sparse_v.py:35-46, 148-171): 32 heads (MHA),
+    d = 128, 3-bit values from uniform random indices, norms U(0.1, 1.1), weights = softmax(5 * N(0,1)), sequence
+    lengths 512 .. 16384, thresholds 0 / 1e-5 / 1e-4.  Every point: the default sparse_v_matvec against the oracle
+    to the reference's bar (tests/test_sparse_v.py:70-75), against the script's own dense composition
+    (weights x packed_dequantize) by the cosine it reports, and the count of active positions."""
+    rng = np.random.default_rng(S)
+    H, D, bits = 32, 128, 3
+    c, s, vp, vn = v_fixture(rng, H, S, D, bits)
+    vn = (rng.random((H, S)) + 0.1).astype(F32)
+    w = softmax_np(rng.standard_normal((H, S)) * 5)
+    dw, dvp, dvn, ds = dev(w), dev(vp), dev(vn), dev(s)
+    vdeq = tq.packed_dequantize(dvp.reshape(H * S, -1), dvn.reshape(-1), c, ds, D, bits).reshape(H, S, D)
+    dense = host(torch.einsum("hs,hsd->hd", dw, vdeq))
+    for thr in (0.0, 1e-5, 1e-4):
+        want = o.sparse_v_matvec(w, vp, vn, c, s, D, bits, threshold=thr)
+        got = host(tq.sparse_v_matvec(dw, dvp, dvn, c, ds, D, bits, threshold=thr))
+        assert np.abs(got - want).max() <= 1e-5 * np.abs(want).max(), (S, thr)
+        cosine = float((got * dense).sum() / np.linalg.norm(got) / np.linalg.norm(dense))
+        assert cosine > (0.99999 if thr == 0.0 else 0.999), (S, thr, cosine)
+        assert tq.count_active_positions(dw, thr) == o.count_active_positions(w, thr)
+
+
 # ------------------------------------------------------------------ flash decode
 
 def kv_fixture(rng, n_kv, S, D, bits, outliers=False):
@@ -742,7 +766,7 @@ def test_prefill_attention_noncausal_fp16_out_and_outliers(tq):
         assert got.dtype == torch.float16
         err = np.abs(host(got).astype(np.float64) - want)
         scale = np.abs(want).max(axis=-1, keepdims=True)
-        assert (err <= 1e-3 + 3e-3 * scale).all(), (err / scale).max()     # + fp16 rounding of the output
+        assert (err <= 1e-3 + 2.5e-3 * scale).all(), (err / scale).max()   # 2e-3 + fp16 rounding of the output (4.9e-4)
 
 
 def test_prefill_attention_fp16_query_flag(tq):
@@ -1178,14 +1202,34 @@ def test_flash_streaming_pass_group_sizes_and_leading_offset(tq, n_kv, n_rep):
         close(got[i], want)
 
 
+def encoded_kv_on_gpu(tq, g, n_kv, n_rows, bits, signs, outlier_channel=None):
+    """K or V of a benchmark configuration at full size: seeded N(0,1) fp16 rows drawn on the GPU (optionally one
+    channel scaled x20), encoded by the library's own encoder -- whose words and norms at this size are compared
+    with the oracle bit for bit in test_config5_full_size_encode_paths_agree.  Returns (packed (n_kv, n_rows, pdim)
+    uint32, norms (n_kv, n_rows) float32) on the GPU."""
+    c, b = tables(bits)
+    packed, norms = [], []
+    for h in range(n_kv):
+        x = torch.randn((n_rows, 128), generator=g, device="cuda", dtype=torch.float32).to(torch.float16)
+        if outlier_channel is not None:
+            x[:, outlier_channel] *= 20
+        p, n = tq.fused_quantize(x, signs, b, 128, bits)
+        packed.append(p)
+        norms.append(n)
+        del x
+    return torch.stack(packed), torch.stack(norms)
+
+
 def test_config4_full_size_paths_agree(tq):
     """benchmark configuration 4 at full size (16 sequences of 4096..32768 positions, 32 q / 8 kv heads, fp16
     out): the streaming pass, the one-tile-per-workgroup pass (forced by an all-zero mask) and the float32
     kernels are three separate code paths and must agree; the two shortest sequences and the LONGEST one (the most
-    steps of the streaming pass) are also checked against the oracle.  Tolerances: the inputs are random packed
-    words with key norms of 7 .. 15, i.e. peaked softmax rows whose outputs span decades inside a row, so the
-    relative term is taken against the row maximum (the reference's own measure, tests/test_flash_attention.py),
-    plus the fp16 rounding of the output."""
+    steps of the streaming pass) are also checked against the oracle.  Data as the configuration states it: K and V
+    are the encoder's output for seeded N(0,1) fp16 rows.  Tolerances: 2e-3 of the row maximum (the reference's own
+    measure, tests/test_flash_attention.py) for fp16-operand against float32 arithmetic, 2.5e-3 where the fp16
+    rounding of the OUTPUT (at most 4.9e-4 of an element) comes on top; the absolute term is 1e-4 here, not 1e-3:
+    the rows of a flat softmax over thousands of N(0,1) values are of size 0.01 - 0.05, where 1e-3 would pass
+    anything."""
     rng = np.random.default_rng(4)
     n_kv, n_rep, D, bits, n_seq = 8, 4, 128, 3, 16
     lens = rng.integers(4096, 32769, size=n_seq)
@@ -1196,11 +1240,9 @@ def test_config4_full_size_paths_agree(tq):
     ks, vs = o.random_diagonal_sign(D, 42), o.random_diagonal_sign(D, 43)
     g = torch.Generator(device="cuda")
     g.manual_seed(4)
-    kp = torch.randint(0, 2 ** 30, (n_kv, total, 13), generator=g, device="cuda", dtype=torch.int32).view(torch.uint32)
-    vp = torch.randint(0, 2 ** 30, (n_kv, total, 13), generator=g, device="cuda", dtype=torch.int32).view(torch.uint32)
-    kn = torch.rand((n_kv, total), generator=g, device="cuda") * 8 + 7
-    vn = torch.rand((n_kv, total), generator=g, device="cuda") + 0.5
-    q = rng.standard_normal((n_seq, n_kv * n_rep, D)).astype(F32)
+    kp, kn = encoded_kv_on_gpu(tq, g, n_kv, total, bits, dev(ks))
+    vp, vn = encoded_kv_on_gpu(tq, g, n_kv, total, bits, dev(vs))
+    q = rng.standard_normal((n_seq, n_kv * n_rep, D)).astype(np.float16).astype(F32)
     sc = 1 / math.sqrt(D)
     q_rot = tq.prerotate_query(dev(q.reshape(-1, D)), dev(ks)).reshape(n_seq, n_kv * n_rep, D)
     kw = dict(n_rep=n_rep, seq_offsets=dev(offs), max_seq_len=max_len)
@@ -1210,17 +1252,17 @@ def test_config4_full_size_paths_agree(tq):
     f = tq.flash_decode(q_rot, kp, kn, vp, vn, c, c, dev(vs), D, bits, sc, precision="fp32", **kw)
     assert a.dtype == torch.float16
     a, t, f = host(a).astype(F32), host(t).astype(F32), host(f)
-    close(a.reshape(-1, D), f.reshape(-1, D), rel=3e-3, row_scale=True)     # + fp16 rounding of the output
-    close(t.reshape(-1, D), f.reshape(-1, D), rel=3e-3, row_scale=True)
-    close(a.reshape(-1, D), t.reshape(-1, D), rel=2e-3, row_scale=True)
+    close(a.reshape(-1, D), f.reshape(-1, D), rel=2.5e-3, abs_=1e-4, row_scale=True)     # 2e-3 + fp16 rounding of the output
+    close(t.reshape(-1, D), f.reshape(-1, D), rel=2.5e-3, abs_=1e-4, row_scale=True)
+    close(a.reshape(-1, D), t.reshape(-1, D), rel=2e-3, abs_=1e-4, row_scale=True)
     hk, hkn, hv, hvn = host(kp), host(kn), host(vp), host(vn)
     order = np.argsort(lens)
     for i in (order[0], order[1], order[-1]):
         s0, s1 = offs[i], offs[i + 1]
         want = o.flash_attention_turboquant(o.prerotate_query(q[i], ks), hk[:, s0:s1], hkn[:, s0:s1], hv[:, s0:s1],
                                             hvn[:, s0:s1], c, c, vs, D, bits, sc, 16, n_rep)
-        close(a[i], want, rel=3e-3, row_scale=True)
-        close(f[i], want, row_scale=True)                          # the float32 kernels: no fp16 anywhere
+        close(a[i], want, rel=2.5e-3, abs_=1e-4, row_scale=True)
+        close(f[i], want, abs_=1e-4, row_scale=True)               # the float32 kernels: no fp16 anywhere
 
 
 def test_config5_full_size_encode_paths_agree(tq):
@@ -1254,10 +1296,10 @@ def test_config5_full_size_prefill_rows_are_decode_steps(tq):
     n_kv, n_rep, T, n_rows, D, bits = 8, 4, 131072, 512, 128, 3
     c, b = tables(bits)
     ks, vs = dev(o.random_diagonal_sign(D, 42)), dev(o.random_diagonal_sign(D, 43))
-    kp = torch.randint(0, 2 ** 30, (n_kv, T, 13), generator=g, device="cuda", dtype=torch.int32).view(torch.uint32)
-    vp = torch.randint(0, 2 ** 30, (n_kv, T, 13), generator=g, device="cuda", dtype=torch.int32).view(torch.uint32)
-    kn = torch.rand((n_kv, T), generator=g, device="cuda") * 8 + 7
-    vn = torch.rand((n_kv, T), generator=g, device="cuda") + 0.5
+    # the configuration's data: N(0,1) fp16 rows with 1 % of the channels (one of 128, drawn from the seed) scaled x20
+    ch = int(torch.randint(0, D, (1,), generator=g, device="cuda").item())
+    kp, kn = encoded_kv_on_gpu(tq, g, n_kv, T, bits, ks, outlier_channel=ch)
+    vp, vn = encoded_kv_on_gpu(tq, g, n_kv, T, bits, vs, outlier_channel=ch)
     q = torch.randn((n_kv * n_rep, n_rows, D), generator=g, device="cuda", dtype=torch.float16)
     sc = 1 / math.sqrt(D)
     got = tq.prefill_attention(q, kp, kn, vp, vn, c, c, ks, vs, D, bits, sc, n_rep=n_rep, out_dtype=torch.float32)

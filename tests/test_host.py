@@ -248,6 +248,42 @@ def test_explicit_sign_vectors_are_validated_on_host():
     assert np.array_equal(v._v_tq._v_q.signs.numpy(), s)
 
 
+def test_sign_stream_argument_selects_the_generator_on_host():
+    """sign_stream='mlx' on the constructors and on from_state expands the seed (and seed + 1 for the values)
+    by the restated MLX stream; 'native' (default) by this package's; explicit vectors win; bad names raise."""
+    dev = torch.device("cpu")
+    mlx_k = tqhip.random_diagonal_sign(128, 7, stream="mlx").numpy()
+    mlx_v = tqhip.random_diagonal_sign(128, 8, stream="mlx").numpy()
+    nat_k = tqhip.random_diagonal_sign(128, 7).numpy()
+    c = tqhip.TurboQuantKVCache(bits=3, seed=7, sign_stream="mlx")
+    c._ensure_quantizer(128, 128, dev)
+    assert np.array_equal(c._k_q.signs.numpy(), mlx_k) and np.array_equal(c._v_q.signs.numpy(), mlx_v)
+    d = tqhip.TurboQuantKVCache(bits=3, seed=7)
+    d._ensure_quantizer(128, 128, dev)
+    assert d.sign_stream == "native" and np.array_equal(d._k_q.signs.numpy(), nat_k)
+    e = tqhip.TurboQuantKVCache(bits=3, seed=7, sign_stream="mlx", k_signs=nat_k)
+    e._ensure_quantizer(128, 128, dev)
+    assert np.array_equal(e._k_q.signs.numpy(), nat_k) and np.array_equal(e._v_q.signs.numpy(), mlx_v)
+    v = tqhip.VOnlyTurboQuantCache(bits=3, seed=7, sign_stream="mlx")
+    v._v_tq._ensure_quantizer(128, 128, dev)
+    assert np.array_equal(v._v_tq._v_q.signs.numpy(), mlx_v)
+    # an empty serialised cache restores on the host: the stream choice survives until the first insert
+    meta = "0,3,7,0,0,float16"                                # dims unknown: no quantiser (and no device) yet
+    r = tqhip.TurboQuantKVCache.from_state([], meta, sign_stream="mlx")
+    assert r.sign_stream == "mlx" and r.seed == 7
+    r._ensure_quantizer(128, 128, dev)
+    assert np.array_equal(r._k_q.signs.numpy(), mlx_k)
+    rv = tqhip.VOnlyTurboQuantCache.from_state([], f"VOnlyTQ,3,7,{meta}", sign_stream="mlx")
+    rv._v_tq._ensure_quantizer(128, 128, dev)
+    assert np.array_equal(rv._v_tq._v_q.signs.numpy(), mlx_v)
+    for make in (lambda: tqhip.TurboQuantKVCache(sign_stream="numpy"),
+                 lambda: tqhip.VOnlyTurboQuantCache(sign_stream=""),
+                 lambda: tqhip.TurboQuantKVCache.from_state([], meta, sign_stream="MLX"),
+                 lambda: tqhip.VOnlyTurboQuantCache.from_state([], f"VOnlyTQ,3,7,{meta}", sign_stream=None)):
+        with pytest.raises(ValueError, match="sign_stream"):
+            make()
+
+
 @pytest.mark.parametrize("have_k,have_v,offset,extra", [(1024, 1024, 1000, 2000), (1512, 1536, 1500, 1),
                                                          (300, 300, 300, 1), (556, 512, 301, 1), (0, 0, 0, 5)])
 def test_vonly_cache_brings_keys_and_values_to_one_capacity(have_k, have_v, offset, extra):

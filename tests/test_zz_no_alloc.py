@@ -93,6 +93,38 @@ def test_static_scratch_batch_dtypes_and_float32_path(tq):
     assert torch.equal(a, b)
 
 
+def test_static_scratch_leaves_device_memory_alone_and_replays_from_a_graph(tq):
+    """The driver's own count of free device memory (hipMemGetInfo) is the same before and after a run of
+    calls -- torch's allocator statistics would not see a hipMalloc made inside the library -- and the call can
+    be recorded in a HIP graph (a capture refuses allocation) and replayed: every replay, with eager work and
+    synchronisations in between and fresh query values each time, equals the workspace entry point bit for bit."""
+    rng = np.random.default_rng(9)
+    sc = 1.0 / math.sqrt(D)
+    case = _case(tq, rng, 2, 4, 7, 3000)
+    args = (case["K"], case["vp"], case["vn"], case["c"], case["vs"], D, BITS, sc)
+    q = case["q"].clone()
+    out = torch.empty((2, 28, D), dtype=torch.float32, device="cuda")
+    tq.vonly_decode(q, *args, n_rep=7, out=out, static_scratch=True)      # first call on the device: looks the array up,
+    torch.cuda.synchronize()                                              # loads the kernels' code
+    free_before, _ = torch.cuda.mem_get_info()
+    for _ in range(5):
+        tq.vonly_decode(q, *args, n_rep=7, out=out, static_scratch=True)
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before, f"free device memory moved by {free_before - free_after} bytes over five calls"
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        tq.vonly_decode(q, *args, n_rep=7, out=out, static_scratch=True)
+    for i in range(4):
+        q.copy_(torch.from_numpy(rng.standard_normal(tuple(q.shape)).astype(np.float16)).cuda())
+        out.fill_(float("nan"))
+        g.replay()
+        torch.cuda.synchronize()
+        want = tq.vonly_decode(q, *args, n_rep=7)                         # eager, caller's workspace
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), f"replay {i} differs from tq_vonly_decode_attn"
+
+
 def test_static_scratch_rejects_shapes_beyond_the_array(tq):
     """More partial sums than the 4 MiB array holds: a clear error before any launch, nothing written."""
     from tqhip import _lib, ops

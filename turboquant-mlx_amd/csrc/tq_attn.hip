@@ -1496,7 +1496,7 @@ extern "C" int tq_vonly_sparse_decode_attn(const void* q, int q_dtype, const voi
   if (!tq::aligned(k_f16, 16)) return tq::fail(TQ_ERR_ALIGN, "%s: k must be 16-byte aligned", who);
   if (!(threshold >= 0.0f)) return tq::fail(TQ_ERR_ARG, "%s: threshold must be >= 0", who);
   if (!(shape->dim == 128 && shape->n_rep <= tqm::kHeadsMax && shape->seq_len > 0 && tq::aligned(q, 16)))
-    return tq::fail(TQ_ERR_UNSUPPORTED, "%s: dim 128, n_rep <= 16 and a non-empty cache only "
+    return tq::fail(TQ_ERR_UNSUPPORTED, "%s: dim 128, n_rep <= 16, a non-empty cache and a 16-byte aligned q only "
                                         "(compose tq_dense_qk_scores, tq_softmax_rows and tq_sparse_v_matvec otherwise)", who);
   return launch_vonly_sparse(q, q_dtype, k_f16, v_packed, v_norms, v_centroids, v_signs, threshold, out, workspace,
                              workspace_bytes, *shape, (hipStream_t)stream_);

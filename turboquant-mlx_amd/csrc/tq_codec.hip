@@ -768,21 +768,36 @@ bool level_cells_search(const float* t, int nb, EncodeGuess& out) {
   return true;
 }
 
-// The search result is kept for the last threshold set seen.
+// Search results are kept for the last few threshold sets seen (a process that alternates widths or threshold
+// rules between calls -- caches of different bits, keys and values under different rules -- would otherwise repeat
+// a search of several milliseconds at every switch).  The lock covers the table only, not the search: two threads
+// that miss on the same set both search and store the same result.
 bool level_guess(const float* t, int nb, EncodeGuess& out) {
+  constexpr int kSlots = 8;
+  struct Slot { float t[15]; int nb; bool ok; EncodeGuess g; };
   static std::mutex mu;
-  static float last_t[15];
-  static int last_nb = 0;
-  static bool last_ok = false;
-  static EncodeGuess last_out;
-  std::lock_guard<std::mutex> lock(mu);
-  if (last_nb != nb || memcmp(last_t, t, nb * sizeof(float)) != 0) {
-    last_ok = (nb == 7) ? level_guess_search(t, nb, last_out) : level_cells_search(t, nb, last_out);
-    memcpy(last_t, t, nb * sizeof(float));
-    last_nb = nb;
+  static Slot slots[kSlots];
+  static int n_used = 0, next = 0;
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    for (int i = 0; i < n_used; ++i)
+      if (slots[i].nb == nb && memcmp(slots[i].t, t, nb * sizeof(float)) == 0) {
+        out = slots[i].g;
+        return slots[i].ok;
+      }
   }
-  out = last_out;
-  return last_ok;
+  Slot s{};
+  s.nb = nb;
+  memcpy(s.t, t, nb * sizeof(float));
+  s.ok = (nb == 7) ? level_guess_search(t, nb, s.g) : level_cells_search(t, nb, s.g);
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    slots[next] = s;
+    next = (next + 1) % kSlots;
+    if (n_used < kSlots) ++n_used;
+  }
+  out = s.g;
+  return s.ok;
 }
 
 bool level_guess_search(const float* t, int nb, EncodeGuess& out) {

@@ -448,35 +448,42 @@ namespace tq {
 // systematic error (the same few values at every position, so it does not average out over a
 // sequence); multiplying the table by a scale a in [1, 2) first and dividing the result by a
 // afterwards (in float32) leaves the mathematics alone, and a can be chosen so that every a*c[i]
-// lies within a few 2^-16 of an fp16 value.  Returns 1/a; the search result is kept for the last
-// table seen.
+// lies within a few 2^-16 of an fp16 value.  Returns 1/a; search results are kept for the last few
+// tables seen.
 inline float fill_codebook_fp16(tqd::Codebook& cb, const float* c, int bits) {
+  constexpr int kSlots = 4;                                   // one per width in use
+  struct Slot { float c[16]; int n; float scale; };
   static std::mutex mu;
-  static float last_c[16], last_scale = 0.0f;
-  static int last_n = 0;
+  static Slot slots[kSlots];
+  static int n_used = 0, next = 0;
   const int n = 1 << bits;
-  float scale = 1.0f;
+  float scale = 0.0f;
   {
     std::lock_guard<std::mutex> lock(mu);
-    if (last_n == n && last_scale != 0.0f && std::memcmp(last_c, c, n * sizeof(float)) == 0) {
-      scale = last_scale;
-    } else {
-      double best = 1e30;
-      for (int j = 0; j < 65536; ++j) {
-        const float a = 1.0f + (float)j * (1.0f / 65536.0f);
-        double worst = 0.0;
-        for (int i = 0; i < n && worst < best; ++i) {
-          const float v = a * c[i];
-          if (v == 0.0f) continue;
-          const float r = (float)(_Float16)v;
-          worst = std::fmax(worst, std::fabs(((double)r - (double)v) / (double)v));
-        }
-        if (worst < best) { best = worst; scale = a; }
+    for (int i = 0; i < n_used; ++i)
+      if (slots[i].n == n && std::memcmp(slots[i].c, c, n * sizeof(float)) == 0) scale = slots[i].scale;
+  }
+  if (scale == 0.0f) {                                        // the search runs outside the lock
+    scale = 1.0f;
+    double best = 1e30;
+    for (int j = 0; j < 65536; ++j) {
+      const float a = 1.0f + (float)j * (1.0f / 65536.0f);
+      double worst = 0.0;
+      for (int i = 0; i < n && worst < best; ++i) {
+        const float v = a * c[i];
+        if (v == 0.0f) continue;
+        const float r = (float)(_Float16)v;
+        worst = std::fmax(worst, std::fabs(((double)r - (double)v) / (double)v));
       }
-      std::memcpy(last_c, c, n * sizeof(float));
-      last_n = n;
-      last_scale = scale;
+      if (worst < best) { best = worst; scale = a; }
     }
+    std::lock_guard<std::mutex> lock(mu);
+    Slot& s = slots[next];
+    std::memcpy(s.c, c, n * sizeof(float));
+    s.n = n;
+    s.scale = scale;
+    next = (next + 1) % kSlots;
+    if (n_used < kSlots) ++n_used;
   }
   for (int i = 0; i < 16; ++i) cb.c[i] = (i < n) ? scale * c[i] : 0.0f;
   return 1.0f / scale;

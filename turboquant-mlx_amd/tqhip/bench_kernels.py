@@ -6,7 +6,7 @@ back-to-back launches, and rotation over several independent input sets so that 
 Infinity Cache cannot serve the reads.  Prints one line per case: us per call, GB/s of algorithmic
 bytes and the fraction of 8 TB/s.
 
-    python -m tqhip.bench_kernels [--iters 200] [--cases encode,scores,flash,flash_long,sparse_v,vonly,vonly_batch,widths,packed_widths,codec_widths,prefill,step]
+    python -m tqhip.bench_kernels [--iters 200] [--cases encode,scores,flash,flash_long,sparse_v,sparse_v_grid,vonly,vonly_batch,widths,packed_widths,codec_widths,prefill,step]
 """
 from __future__ import annotations
 
@@ -82,10 +82,11 @@ def bench_scores(iters, dev):
         nbytes = 224 * T + 112 * T + 14336
         sets = packed_sets(4, T, dev, n_sets_for(nbytes), 3)
         q_rot = torch.randn((28, 128), device=dev)
-        for prec in ("fp32", "fp16"):
+        for prec, label in ((None, "default (split operands, float32 fidelity)"), ("fp32", "float32 vector kernels"),
+                            ("fp16", "fp16 operands")):
             fns = [(lambda p=p, n=n: tqhip.prerot_fused_qk_scores(q_rot, p, n, cb, 128, 3, n_rep=7, precision=prec))
                    for p, n in sets]
-            report(f"config 3: prerot scores 28/4 heads, T={T}, {prec} operands", timeit(fns, iters), nbytes)
+            report(f"config 3: prerot scores 28/4 heads, T={T}, {label}", timeit_graph(fns, iters), nbytes)
 
 
 def bench_sparse_v(iters, dev):
@@ -95,10 +96,43 @@ def bench_sparse_v(iters, dev):
         nbytes = 28 * T * 4 + 4 * T * 56 + 28 * 128 * 4
         sets = packed_sets(4, T, dev, n_sets_for(nbytes), 4)
         w = torch.softmax(torch.randn((28, T), device=dev) * 5, dim=-1)
-        for thr, prec in ((0.0, "fp32"), (1e-5, "fp32"), (1e-5, "fp16")):
+        for thr, prec, label in ((0.0, None, "default (split operands)"), (1e-5, None, "default (split operands)"),
+                                 (1e-5, "fp32", "float32 vector kernels"), (1e-5, "fp16", "fp16 operands")):
             fns = [(lambda p=p, n=n: tqhip.sparse_v_matvec(w, p, n, cb, signs, 128, 3, threshold=thr, n_rep=7,
                                                            precision=prec)) for p, n in sets]
-            report(f"sparse_v_matvec 28/4 heads, T={T}, thr={thr:g}, {prec} operands", timeit(fns, iters), nbytes)
+            report(f"sparse_v_matvec 28/4 heads, T={T}, thr={thr:g}, {label}", timeit_graph(fns, iters), nbytes)
+
+
+def bench_sparse_v_grid(iters, dev):
+    """The reference's micro-benchmark grid (scripts/bench_sparse_v.py:148-171): dense (packed_dequantize, then
+    weights x V) against sparse_v_matvec over sequence lengths x thresholds; 32 heads (MHA), d = 128, 3-bit,
+    weights = softmax(5 * N(0,1)).  Same columns as the script's table: ms, speed-up over dense, active positions,
+    cosine against dense.  HIP-graph replays (GPU time of the calls, no host gaps)."""
+    cb = gaussian_codebook(3)
+    signs = tqhip.random_diagonal_sign(128, 43, device=dev)
+    H = 32
+    g = torch.Generator(device=dev)
+    g.manual_seed(0)
+    print("| seq_len | dense us | thr | sparse_v us | speed-up | active % | cosine |")
+    print("|---|---|---|---|---|---|---|")
+    for S in (512, 2048, 8192, 16384):
+        n_sets = n_sets_for(H * S * 56)
+        sets = packed_sets(H, S, dev, n_sets, 100 + S)
+        w = torch.softmax(torch.randn((H, S), generator=g, device=dev) * 5, dim=-1)
+
+        def dense(p, n):
+            v = tqhip.packed_dequantize(p.reshape(H * S, -1), n.reshape(-1), cb, signs, 128, 3).reshape(H, S, 128)
+            return torch.einsum("hs,hsd->hd", w, v)
+        d_us = timeit_graph([(lambda p=p, n=n: dense(p, n)) for p, n in sets], iters)
+        d_out = dense(*sets[0])
+        for thr in (0.0, 1e-5, 1e-4):
+            fns = [(lambda p=p, n=n: tqhip.sparse_v_matvec(w, p, n, cb, signs, 128, 3, threshold=thr)) for p, n in sets]
+            us = timeit_graph(fns, iters)
+            out = tqhip.sparse_v_matvec(w, sets[0][0], sets[0][1], cb, signs, 128, 3, threshold=thr)
+            cosine = float((out * d_out).sum() / (out.norm() * d_out.norm() + 1e-8))
+            active = tqhip.count_active_positions(w, thr)
+            print(f"| {S} | {d_us:.1f} | {thr:g} | {us:.1f} | {d_us / us:.2f}x | {100.0 * active / (H * S):.1f} | {cosine:.6f} |",
+                  flush=True)
 
 
 def bench_flash(iters, dev):
@@ -411,7 +445,7 @@ def bench_step(iters, dev):
 
 CASES = {"step": bench_step, "prefill": bench_prefill, "encode": bench_encode, "scores": bench_scores, "sparse_v": bench_sparse_v, "flash": bench_flash,
          "flash_long": bench_flash_long, "vonly": bench_vonly, "widths": bench_widths, "codec_widths": bench_codec_widths,
-         "packed_widths": bench_packed_widths, "vonly_batch": bench_vonly_batch}
+         "packed_widths": bench_packed_widths, "vonly_batch": bench_vonly_batch, "sparse_v_grid": bench_sparse_v_grid}
 
 
 def main():

@@ -24,15 +24,20 @@ def _checked_signs(signs, dim, device) -> torch.Tensor:
     return t
 
 
+def _check_sign_stream(sign_stream):
+    if sign_stream not in ("native", "mlx"):
+        raise ValueError(f"sign_stream must be 'native' or 'mlx', got {sign_stream!r}")
+
+
 class _Quantizer:
     """cache.py:33-39: signs (device) + codebook tables (host).  `signs` overrides the vector that
     random_diagonal_sign derives from `seed` (whose generator is this package's own, not MLX's): the way to
     read a cache written by the reference, which stores only the seed (cache.py:286)."""
 
-    def __init__(self, dim, bits, seed, device, signs=None):
+    def __init__(self, dim, bits, seed, device, signs=None, sign_stream="native"):
         self.dim = dim
         self.bits = bits
-        self.signs = (random_diagonal_sign(dim, seed=seed, device=device) if signs is None
+        self.signs = (random_diagonal_sign(dim, seed=seed, device=device, stream=sign_stream) if signs is None
                       else _checked_signs(signs, dim, device))
         self.centroids = gaussian_codebook(bits)
         self.boundaries = gaussian_boundaries(self.centroids)
@@ -74,9 +79,12 @@ class TurboQuantKVCache:
 
     def __init__(self, bits: int = 3, seed: int = 42, fused: bool = False,
                  sparse_v_threshold: float | None = None, v_only: bool = False,
-                 encode_variant: str = "mlx", k_signs=None, v_signs=None):
+                 encode_variant: str = "mlx", k_signs=None, v_signs=None, sign_stream: str = "native"):
         """k_signs / v_signs ([dim] of +-1, any tensor-like): the rotation's sign vectors, used instead of the ones
-        derived from `seed` / `seed + 1` (cache.py:92,96).  Everything else as the reference (cache.py:54-61)."""
+        derived from `seed` / `seed + 1` (cache.py:92,96).  sign_stream: which generator derives them when they
+        are not given -- "native" (this package's) or "mlx" (the restated stream of rotation.py:47-49, for a
+        cache the reference wrote with that seed).  Everything else as the reference (cache.py:54-61)."""
+        _check_sign_stream(sign_stream)
         self.quant_bits = bits
         self.seed = seed
         self.offset = 0
@@ -89,6 +97,7 @@ class TurboQuantKVCache:
         self.encode_variant = encode_variant
         self._reset_fields()
         self._k_signs_given, self._v_signs_given = k_signs, v_signs
+        self.sign_stream = sign_stream
 
     def _reset_fields(self):
         self.k_packed = None
@@ -108,6 +117,7 @@ class TurboQuantKVCache:
         self._dtype = None
         self._step, self._step_key = None, None
         self._k_signs_given, self._v_signs_given = None, None
+        self.sign_stream = "native"
 
     # ---------------------------------------------------------------- setup (cache.py:90-123)
     def _device(self):
@@ -119,11 +129,11 @@ class TurboQuantKVCache:
     def _ensure_quantizer(self, k_dim, v_dim, device=None):
         device = device if device is not None else self._device()
         if not self.v_only and self._k_q is None:
-            self._k_q = _Quantizer(k_dim, self.quant_bits, self.seed, device, self._k_signs_given)
+            self._k_q = _Quantizer(k_dim, self.quant_bits, self.seed, device, self._k_signs_given, self.sign_stream)
             self._k_dim = k_dim
             self._k_pdim = ops.packed_dim(k_dim, self.quant_bits)
         if self._v_q is None:
-            self._v_q = _Quantizer(v_dim, self.quant_bits, self.seed + 1, device, self._v_signs_given)
+            self._v_q = _Quantizer(v_dim, self.quant_bits, self.seed + 1, device, self._v_signs_given, self.sign_stream)
             self._v_dim = v_dim
             self._v_pdim = ops.packed_dim(v_dim, self.quant_bits)
 
@@ -415,13 +425,16 @@ class TurboQuantKVCache:
 
     # ---------------------------------------------------------------- cache.py:336-369
     @classmethod
-    def from_state(cls, state, meta_state, k_signs=None, v_signs=None):
+    def from_state(cls, state, meta_state, k_signs=None, v_signs=None, sign_stream: str = "native"):
         """cache.py:336-369.  The serialised cache carries its seed, not its sign vectors (cache.py:286): a cache
         written with explicit signs -- or by the reference, whose seed-to-signs generator is MLX's -- restores
-        correctly only with the same k_signs / v_signs given here."""
+        correctly only with the same k_signs / v_signs given here, or, for a reference-written cache whose
+        vectors were not kept, with sign_stream="mlx" (the seed is then expanded by the restated MLX stream)."""
+        _check_sign_stream(sign_stream)
         obj = cls.__new__(cls)
         obj._reset_fields()
         obj._k_signs_given, obj._v_signs_given = k_signs, v_signs
+        obj.sign_stream = sign_stream
         obj.fused = False
         obj.sparse_v_threshold = None
         obj.v_only = False

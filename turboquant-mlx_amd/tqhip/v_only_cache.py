@@ -19,11 +19,13 @@ class VOnlyTurboQuantCache:
     packed values directly (vonly_decode_attention, tqhip.patch); `dequantized_values()` gives the
     fp16 values when a multi-token step needs them."""
 
-    def __init__(self, bits: int = 3, seed: int = 42, no_v_buffer: bool = False, fused: bool = False, v_signs=None):
+    def __init__(self, bits: int = 3, seed: int = 42, no_v_buffer: bool = False, fused: bool = False, v_signs=None,
+                 sign_stream: str = "native"):
         """v_signs ([dim] of +-1): the value rotation's sign vector, used instead of the one derived from
-        `seed + 1` (cache.py:96).  Everything else as the reference (v_only_cache.py:41-49) plus `fused`."""
+        `seed + 1` (cache.py:96); sign_stream ("native" | "mlx"): the generator that derives it otherwise, as for
+        TurboQuantKVCache.  Everything else as the reference (v_only_cache.py:41-49) plus `fused`."""
         self._k_cache = KVCache()
-        self._v_tq = TurboQuantKVCache(bits=bits, seed=seed, v_only=True, v_signs=v_signs)
+        self._v_tq = TurboQuantKVCache(bits=bits, seed=seed, v_only=True, v_signs=v_signs, sign_stream=sign_stream)
         self._v_bits = bits
         self._no_v_buffer = no_v_buffer
         self.fused = fused
@@ -214,14 +216,15 @@ class VOnlyTurboQuantCache:
         return f"VOnlyTQ,{self._v_bits},{self._v_tq.seed},{self._v_tq.meta_state}"
 
     @classmethod
-    def from_state(cls, state, meta_state, v_signs=None):
+    def from_state(cls, state, meta_state, v_signs=None, sign_stream: str = "native"):
         """v_only_cache.py:95-111.  The serialised cache carries its seed, not its sign vector: pass the
         v_signs the cache was written with when they were given explicitly (or come from the reference,
-        whose seed-to-signs generator is MLX's)."""
+        whose seed-to-signs generator is MLX's), or sign_stream="mlx" to expand a reference-written cache's
+        seed by the restated MLX stream."""
         parts = meta_state.split(",", 3)
         bits = int(parts[1])
         seed = int(parts[2])
-        obj = cls(bits=bits, seed=seed, v_signs=v_signs)
+        obj = cls(bits=bits, seed=seed, v_signs=v_signs, sign_stream=sign_stream)
         if len(state) >= 2:
             obj._k_cache.keys = state[0]
             obj._k_cache.values = state[1]
