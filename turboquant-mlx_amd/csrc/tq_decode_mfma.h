@@ -43,6 +43,12 @@ using namespace tqd;
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef float f4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u4 __attribute__((ext_vector_type(4)));   // plain vector: stays in registers
+// 16 bytes of K / V that this launch reads once: a streaming load (the "nt" hint).  Measured on the tile pass of the
+// decode step (41 MB per launch over rotating buffers): 10.25 -> 9.35 us.  Operands that many workgroups share (the
+// query rows, the per-tile partials) keep the default policy.
+__device__ __forceinline__ u4 load_stream(const void* p) { return __builtin_nontemporal_load(reinterpret_cast<const u4*>(p)); }
+__device__ __forceinline__ uint32_t load_stream(const uint32_t* p) { return __builtin_nontemporal_load(p); }
+__device__ __forceinline__ float load_stream(const float* p) { return __builtin_nontemporal_load(p); }
 
 constexpr int kD = 128;
 constexpr int kPdim = 13;
@@ -223,7 +229,7 @@ __device__ __forceinline__ void vonly_tile_body(const MfmaArgs& a, const Codeboo
     const float* nb = a.v_norms + (int64_t)seq * a.vn_seq_stride + (int64_t)kvh * a.vn_head_stride + first + tile_p0;
     int row = wrow0 + lane;
     if (!PLAIN) row = row < last_row ? row : last_row;
-    my_norm = nb[(unsigned)row];
+    my_norm = load_stream(nb + (unsigned)row);
   }
   // packed V of the wave: 64 rows x 4 kPd bytes (52 at three bits), contiguous.  Full, 16-byte aligned blocks
   // take up to four 16-byte loads per lane; ragged or unaligned ones take kPd 4-byte loads with the index
@@ -238,15 +244,15 @@ __device__ __forceinline__ void vonly_tile_body(const MfmaArgs& a, const Codeboo
   if (v_wide) {
     const char* vb = reinterpret_cast<const char*>(vblock);
 #pragma unroll
-    for (int i = 0; i < kVFull; ++i) vq[i] = *reinterpret_cast<const u4*>(vb + i * 1024 + (uint32_t)(lane * 16));
-    if (kVTail) vq[kVFull] = *reinterpret_cast<const u4*>(vb + kVFull * 1024 + (uint32_t)((lane & (kVTail - 1)) * 16));   // lanes >= kVTail repeat
+    for (int i = 0; i < kVFull; ++i) vq[i] = load_stream(vb + i * 1024 + (uint32_t)(lane * 16));
+    if (kVTail) vq[kVFull] = load_stream(vb + kVFull * 1024 + (uint32_t)((lane & (kVTail - 1)) * 16));   // lanes >= kVTail repeat
   } else {
     const int valid_words = max(0, rows_here - wrow0) * kPd;         // words of the block inside the sequence
     const uint32_t* tile_base = vblock - (int64_t)wrow0 * kPd;       // row 0 of the tile: always valid
 #pragma unroll
     for (int i = 0; i < kPd; ++i) {
       const int w = i * 64 + lane;
-      vd[i] = (w < valid_words) ? vblock[w] : tile_base[0];
+      vd[i] = load_stream((w < valid_words) ? vblock + w : tile_base);
     }
   }
   // K: instruction i reads rows 4i .. 4i+3 of the wave; lane L takes 16-byte piece (L & 15) ^ (row & 7)
@@ -270,13 +276,13 @@ __device__ __forceinline__ void vonly_tile_body(const MfmaArgs& a, const Codeboo
   auto issue_k = [&](int i) {
     if (PLAIN) {
       const char* kb = reinterpret_cast<const char*>(kbase) + (i >> 1) * 2048;      // 8 rows of 256 bytes per pair
-      kreg[i] = *reinterpret_cast<const u4*>(kb + ((i & 1) ? koff_odd : koff_even));
+      kreg[i] = load_stream(kb + ((i & 1) ? koff_odd : koff_even));
     } else {
       const int r = 4 * i + (lane >> 4);
       const int piece = (lane & 15) ^ (r & 7);
       int row = wrow0 + r;
       row = row < last_row ? row : last_row;
-      kreg[i] = *reinterpret_cast<const u4*>(reinterpret_cast<const char*>(kbase) + (uint32_t)((row * 16 + piece) * 16));
+      kreg[i] = load_stream(reinterpret_cast<const char*>(kbase) + (uint32_t)((row * 16 + piece) * 16));
     }
   };
 #pragma unroll
@@ -560,7 +566,7 @@ __global__ __launch_bounds__(WAVES * 64) void vonly_scores_kernel(MfmaArgs a) {
     const int piece = (lane & 15) ^ (r & 7);
     int row = wrow0 + r;
     row = row < last_row ? row : last_row;
-    kreg[i] = *reinterpret_cast<const u4*>(kbase + (uint32_t)((row * 16 + piece) * 16));
+    kreg[i] = load_stream(kbase + (uint32_t)((row * 16 + piece) * 16));
   }
 #pragma unroll
   for (int i = 0; i < kQIt; ++i) {
@@ -746,17 +752,17 @@ __device__ __forceinline__ void vonly_stream_body(const MfmaArgs& a, const Codeb
   auto issue_nv = [&](int s, float& nrm, u4 (&vqx)[2]) {
     const int r = step_row(s);
     if (RAGGED) {
-      nrm = nbase[min(r + (lane & 31), last_valid)];
+      nrm = load_stream(nbase + min(r + (lane & 31), last_valid));
       const int rc = min(r, last_step_row);                             // a step with no valid row re-reads the last one that has
       const uint32_t limit = (uint32_t)(vmis + (valid - rc) * (kPd * 4));   // bytes from the piece boundary to the end of the valid rows (> 0)
       const char* vb = vbase + (int64_t)rc * (kPd * 4);
-      vqx[0] = *reinterpret_cast<const u4*>(vb + (voff0 < limit ? voff0 : 0u));
-      if (kPieces > 64) vqx[1] = *reinterpret_cast<const u4*>(vb + (voff1 < limit ? voff1 : 0u));
+      vqx[0] = load_stream(vb + (voff0 < limit ? voff0 : 0u));
+      if (kPieces > 64) vqx[1] = load_stream(vb + (voff1 < limit ? voff1 : 0u));
     } else {
-      nrm = nbase_l[r];
+      nrm = load_stream(nbase_l + r);
       const char* vb = vbase + (int64_t)r * (kPd * 4);
-      vqx[0] = *reinterpret_cast<const u4*>(vb + voff0);
-      if (kPieces > 64) vqx[1] = *reinterpret_cast<const u4*>(vb + voff1_full);
+      vqx[0] = load_stream(vb + voff0);
+      if (kPieces > 64) vqx[1] = load_stream(vb + voff1_full);
     }
   };
   auto issue_k4 = [&](int s, u4 (&kx)[8], int part) {     // instructions 4*part .. 4*part+3: rows 16*part .. +15 of the step
@@ -766,14 +772,14 @@ __device__ __forceinline__ void vonly_stream_body(const MfmaArgs& a, const Codeb
         const int rin = 16 * part + 4 * i + (lane >> 4);                  // row inside the step
         const int piece = (lane & 15) ^ (rin & 7);
         const int row = min(step_row(s) + rin, last_valid);
-        kx[4 * part + i] = *reinterpret_cast<const u4*>(kbase + (int64_t)row * (kD * 2) + piece * 16);
+        kx[4 * part + i] = load_stream(kbase + (int64_t)row * (kD * 2) + piece * 16);
       }
     } else {
       const char* kb = kbase + (int64_t)step_row(s) * (kD * 2) + part * 4096;
-      kx[4 * part + 0] = *reinterpret_cast<const u4*>(kb + koff_even);
-      kx[4 * part + 1] = *reinterpret_cast<const u4*>(kb + koff_odd);
-      kx[4 * part + 2] = *reinterpret_cast<const u4*>(kb + 2048 + koff_even);
-      kx[4 * part + 3] = *reinterpret_cast<const u4*>(kb + 2048 + koff_odd);
+      kx[4 * part + 0] = load_stream(kb + koff_even);
+      kx[4 * part + 1] = load_stream(kb + koff_odd);
+      kx[4 * part + 2] = load_stream(kb + 2048 + koff_even);
+      kx[4 * part + 3] = load_stream(kb + 2048 + koff_odd);
     }
   };
 

@@ -69,22 +69,25 @@ struct PackedBlockT {
 };
 using PackedBlock = PackedBlockT<kPdim>;
 
-template <int PD>
+// STREAM: streaming loads (load_stream).  They pay in the passes that decode values (given weights: 11.9 -> 11.7 us at
+// 32 768 positions) and cost where a pass only scores keys and writes as many bytes as it reads (65 536 positions:
+// 10.7 -> 11.0 us), so the score-only passes keep the default policy.
+template <bool STREAM, int PD>
 __device__ __forceinline__ void load_block(PackedBlockT<PD>& b, const uint32_t* block, int lane, int wrow0, int rows_here) {
   constexpr int kFull = PackedBlockT<PD>::kFull, kTail = PackedBlockT<PD>::kTail;
   b.wide = (wrow0 + kWavePos <= rows_here) && ((reinterpret_cast<uintptr_t>(block) & 15) == 0);
   if (b.wide) {
     const u4* b4 = reinterpret_cast<const u4*>(block);
 #pragma unroll
-    for (int i = 0; i < kFull; ++i) b.q[i] = b4[i * 64 + lane];
-    if (kTail) b.q[kFull] = b4[kFull * 64 + (lane & (kTail - 1))];
+    for (int i = 0; i < kFull; ++i) b.q[i] = STREAM ? load_stream(b4 + i * 64 + lane) : b4[i * 64 + lane];
+    if (kTail) b.q[kFull] = STREAM ? load_stream(b4 + kFull * 64 + (lane & (kTail - 1))) : b4[kFull * 64 + (lane & (kTail - 1))];
   } else {
     const int valid_words = max(0, rows_here - wrow0) * PD;
     const uint32_t* tile_base = block - (int64_t)wrow0 * PD;          // row 0 of the tile: always valid
 #pragma unroll
     for (int i = 0; i < PD; ++i) {
       const int w = i * 64 + lane;
-      b.d[i] = (w < valid_words) ? block[w] : tile_base[0];
+      b.d[i] = load_stream((w < valid_words) ? block + w : tile_base);
     }
   }
 }
@@ -274,13 +277,13 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
   float my_kn = 0.0f, my_vn = 0.0f;
   PackedBlockT<kVPd> kb_, vb_;
   if (HAS_V) {
-    my_vn = a.v_norms[(int64_t)seq * a.vn_seq_stride + (int64_t)kvh * a.vn_head_stride + first + tile_p0 + crow];
-    load_block(vb_, a.v_packed + ((int64_t)seq * a.v_seq_stride + (int64_t)kvh * a.v_head_stride + first +
+    my_vn = load_stream(a.v_norms + (int64_t)seq * a.vn_seq_stride + (int64_t)kvh * a.vn_head_stride + first + tile_p0 + crow);
+    load_block<true>(vb_, a.v_packed + ((int64_t)seq * a.v_seq_stride + (int64_t)kvh * a.v_head_stride + first +
                                   tile_p0 + wrow0) * kVPd, lane, wrow0, rows_here);
   }
   if (HAS_K) {
-    my_kn = a.k_norms[(int64_t)seq * a.kn_seq_stride + (int64_t)kvh * a.kn_head_stride + first + tile_p0 + crow];
-    load_block(kb_, a.k_packed + ((int64_t)seq * a.k_seq_stride + (int64_t)kvh * a.k_head_stride + first +
+    my_kn = load_stream(a.k_norms + (int64_t)seq * a.kn_seq_stride + (int64_t)kvh * a.kn_head_stride + first + tile_p0 + crow);
+    load_block<HAS_V>(kb_, a.k_packed + ((int64_t)seq * a.k_seq_stride + (int64_t)kvh * a.k_head_stride + first +
                                   tile_p0 + wrow0) * kVPd, lane, wrow0, rows_here);
   }
   // given weights: lane (head n16, group g) takes positions 16t + 4g + j
@@ -662,12 +665,12 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
 #pragma unroll
     for (int i = 0; i < kLoads; ++i) {
       const uint32_t off = (uint32_t)(i * 64 + lane) * 16;
-      kq[i] = *reinterpret_cast<const u4*>(k_base + (off < kbytes ? row0 * (kPd * 4) + off : 0u));
-      vq[i] = *reinterpret_cast<const u4*>(v_base + (off < vbytes ? row0 * (kPd * 4) + off : 0u));
+      kq[i] = load_stream(k_base + (off < kbytes ? row0 * (kPd * 4) + off : 0u));
+      vq[i] = load_stream(v_base + (off < vbytes ? row0 * (kPd * 4) + off : 0u));
     }
     const uint32_t nrow = (lane < rows) ? row0 + lane : 0u;
-    kn = kn_base[nrow];
-    vn = vn_base[nrow];
+    kn = load_stream(kn_base + nrow);
+    vn = load_stream(vn_base + nrow);
   };
 
   float2 my_q[4];

@@ -28,7 +28,13 @@ __global__ __launch_bounds__(THREADS) void probe_read_kernel(const uint4* __rest
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
       const size_t j = i + (size_t)u * THREADS;
-      v[u] = j < e ? p[j] : make_uint4(0, 0, 0, 0);
+      if (j < e) {                                             // streaming loads, as the decode kernels read K and V
+        typedef uint32_t piece_t __attribute__((ext_vector_type(4)));
+        const piece_t w = __builtin_nontemporal_load(reinterpret_cast<const piece_t*>(p + j));
+        v[u] = make_uint4(w[0], w[1], w[2], w[3]);
+      } else {
+        v[u] = make_uint4(0, 0, 0, 0);
+      }
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;

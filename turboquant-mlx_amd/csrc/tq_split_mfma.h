@@ -104,7 +104,7 @@ void split_tile_kernel(SplitArgs a, Codebook cb) {
   }
   const float my_n = a.norms[(int64_t)kvh * a.norms_head_stride + tile_p0 + crow];
   PackedBlockT<kPd> blk;
-  load_block(blk, a.packed + ((int64_t)kvh * a.head_stride + tile_p0 + wrow0) * kPd, lane, wrow0, rows_here);
+  load_block<MODE == kWeights>(blk, a.packed + ((int64_t)kvh * a.head_stride + tile_p0 + wrow0) * kPd, lane, wrow0, rows_here);
   // given weights: lane (head n16, group g) takes positions 16t + 4g + j
   float wgt[4][4];
   if (!SCORES) {
