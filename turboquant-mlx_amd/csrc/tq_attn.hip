@@ -211,7 +211,7 @@ __global__ __launch_bounds__(kThreads) void prerot_scores_kernel(const float* __
       const float nrm = k_norms[(int64_t)kvh * n_head_stride + p];
 #pragma unroll
       for (int r = 0; r < kRMax; ++r)
-        if (r < n_local) scores[(q_row0 + r) * seq_len + p] = (acc[u][r] * nrm) * inv_dim;
+        if (r < n_local) __builtin_nontemporal_store((acc[u][r] * nrm) * inv_dim, &scores[(q_row0 + r) * seq_len + p]);
     }
   }
 }

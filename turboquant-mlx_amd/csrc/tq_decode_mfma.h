@@ -1182,7 +1182,7 @@ __device__ __forceinline__ void merge_rows_body(
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int t = min(t0 + 8 * u, n_tiles - 1);
-      x[u] = *reinterpret_cast<const f4*>(gS + (int64_t)t * (n_rep * kD));
+      x[u] = __builtin_nontemporal_load(reinterpret_cast<const f4*>(gS + (int64_t)t * (n_rep * kD)));
       ml[u] = *reinterpret_cast<const float2*>(gml + (int64_t)t * (n_rep * 2));
     }
     // maximum of the round first, then one independent 2^(m - M) per tile

