@@ -6,7 +6,7 @@ back-to-back launches, and rotation over several independent input sets so that 
 Infinity Cache cannot serve the reads.  Prints one line per case: us per call, GB/s of algorithmic
 bytes and the fraction of 8 TB/s.
 
-    python -m tqhip.bench_kernels [--iters 200] [--cases encode,scores,flash,flash_long,sparse_v,sparse_v_grid,vonly,vonly_batch,widths,packed_widths,codec_widths,prefill,step]
+    python -m tqhip.bench_kernels [--iters 200] [--cases encode,scores,flash,flash_long,sparse_v,sparse_v_grid,vonly,vonly_batch,vonly_lengths,widths,packed_widths,codec_widths,prefill,step]
 """
 from __future__ import annotations
 
@@ -229,6 +229,23 @@ def timeit_graph(fns, iters):
     return e0.elapsed_time(e1) * 1e3 / (reps * len(fns))
 
 
+def bench_vonly_lengths(iters, dev):
+    """The decode step of configuration 2's heads (28 query / 4 kv, 3-bit values) over cache lengths from 4 096 to
+    131 072 positions, multiples of the tile and not: which launch shape the host picks changes along the way (four- or
+    eight-wave tiles, the streaming pass).  HIP-graph replay over 8 buffer sets, tile pass + merge pass."""
+    cb = gaussian_codebook(3)
+    signs = tqhip.random_diagonal_sign(128, 43, device=dev)
+    lengths = (4096, 8192, 16384, 20000, 30000, 32768, 32769, 40000, 49152, 50000, 65536, 65537, 100000, 131071, 131072)
+    t_max = max(lengths) + 8
+    sets = packed_sets(4, t_max, dev, 8, 7)
+    ks = [torch.randn((1, 4, t_max, 128), device=dev, dtype=torch.float16) for _ in sets]
+    q = torch.randn((1, 28, 128), device=dev, dtype=torch.float16)
+    for T in lengths:
+        fns = [(lambda k=k, p=p, n=n: tqhip.vonly_decode(q, k, p[None], n[None], cb, signs, 128, 3, 1 / math.sqrt(128),
+                                                         n_rep=7, seq_len=T)) for k, (p, n) in zip(ks, sets)]
+        report(f"V-only decode 28/4 heads, T={T} (graph)", timeit_graph(fns, max(iters, 160)), 4 * T * 312 + 28 * 256 * 2)
+
+
 def bench_widths(iters, dev):
     """V-only decode at the other value widths (1, 2 and 4 bits): the matrix-core tile pass against the
     float32 kernels that served these widths before it (precision="fp32"), HIP-graph replay."""
@@ -443,7 +460,7 @@ def bench_step(iters, dev):
             del g, caches
 
 
-CASES = {"step": bench_step, "prefill": bench_prefill, "encode": bench_encode, "scores": bench_scores, "sparse_v": bench_sparse_v, "flash": bench_flash,
+CASES = {"vonly_lengths": bench_vonly_lengths, "step": bench_step, "prefill": bench_prefill, "encode": bench_encode, "scores": bench_scores, "sparse_v": bench_sparse_v, "flash": bench_flash,
          "flash_long": bench_flash_long, "vonly": bench_vonly, "widths": bench_widths, "codec_widths": bench_codec_widths,
          "packed_widths": bench_packed_widths, "vonly_batch": bench_vonly_batch, "sparse_v_grid": bench_sparse_v_grid}
 
