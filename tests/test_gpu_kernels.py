@@ -1814,6 +1814,37 @@ def test_vonly_streaming_pass_with_a_ragged_end(tq, n_seq, n_kv, n_rep, T, qdt):
         close(got[i], want, rel=(1e-2 if qdt == "bfloat16" else REL), abs_=(4e-3 if qdt == "bfloat16" else ABS), row_scale=True)
 
 
+@pytest.mark.parametrize("n_seq,n_kv,n_rep,T,qdt", [(1, 4, 7, 32769, "float16"), (1, 4, 7, 36864, "float32"),
+                                                     (1, 4, 7, 40001, "float16"), (1, 4, 7, 49152, "bfloat16"),
+                                                     (2, 8, 4, 10241, "float16"), (1, 8, 2, 24576, "float32")])
+def test_vonly_wide_workgroups_just_above_a_full_round(tq, n_seq, n_kv, n_rep, T, qdt):
+    """Unmasked caches a little too long for one round of 512-position workgroups (more than 256 of them, at most 256
+    of 640 or 768 positions) take workgroups of ten or twelve wavefronts: lengths that end inside a workgroup, a
+    wavefront, at a tile boundary, and exact multiples; two sequences; against the oracle."""
+    rng = np.random.default_rng(T + 7)
+    D, bits, sc = 128, 3, 1 / math.sqrt(128)
+    c, b = tables(bits)
+    vs = o.random_diagonal_sign(D, 43)
+    tiles8 = -(-T // 512) * n_kv * n_seq
+    assert tiles8 > 256 and -(-T // 768) * n_kv * n_seq <= 256          # the shapes this test is about
+    K = rng.standard_normal((n_seq, n_kv, T, D)).astype(np.float16)
+    vp = o.pack_indices(rng.integers(0, 8, size=(n_seq, n_kv, T, D)).astype(np.uint8), bits)
+    vn = ((rng.random((n_seq, n_kv, T)) + 0.5) * np.exp(rng.uniform(-3, 3, size=(n_seq, n_kv, T)))).astype(F32)
+    q = torch.from_numpy(rng.standard_normal((n_seq, n_kv * n_rep, D)).astype(F32)).to(getattr(torch, qdt))
+    got = host(tq.vonly_decode(q.cuda(), dev(K), dev(vp), dev(vn), c, dev(vs), D, bits, sc, n_rep=n_rep).float())
+    for i in range(n_seq):
+        want = o.vonly_decode_attention(q[i].float().numpy(), K[i], vp[i], vn[i], c, vs, D, bits, sc)
+        close(got[i], want, rel=(1e-2 if qdt == "bfloat16" else REL), abs_=(4e-3 if qdt == "bfloat16" else ABS), row_scale=True)
+    # the same cache through a longer allocation (cache layout, seq_len < T_alloc): the any-length path with a tail
+    if n_seq == 1:
+        pad = 300
+        Kp = np.concatenate([K, np.zeros((1, n_kv, pad, D), np.float16)], axis=2)
+        vpp = np.concatenate([vp, np.zeros((1, n_kv, pad, vp.shape[-1]), vp.dtype)], axis=2)
+        vnp = np.concatenate([vn, np.ones((1, n_kv, pad), F32)], axis=2)
+        got2 = host(tq.vonly_decode(q.cuda(), dev(Kp), dev(vpp), dev(vnp), c, dev(vs), D, bits, sc, n_rep=n_rep, seq_len=T).float())
+        assert np.array_equal(got2, got)
+
+
 @pytest.mark.parametrize("qdt", ["float16", "float32", "bfloat16"])
 @pytest.mark.parametrize("n_kv,n_rep,lens", [
     (4, 7, [4097, 2561, 1025, 7000, 1, 3333, 5121, 6143]),       # every row misalignment; ends inside a step, a wave, a block

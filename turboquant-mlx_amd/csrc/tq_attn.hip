@@ -786,6 +786,15 @@ int launch_vonly_mfma(const void* q, int q_dtype, const void* k_f16, const uint3
   // of them, avoid the nearly empty second round of the eight-wave shape; beyond that the eight-wave shape again.
   int nw = 8;
   if (n_blocks == 1 && (wgs8 <= 128 || (wgs8 > 256 && wgs4 <= 768))) nw = 4;
+  // Just above one full round of eight-wave workgroups (32 769 ... 49 152 positions at 28/4 heads) the four-wave shape pays
+  // for a short last round: workgroups of ten or twelve waves (640 / 768 positions, three waves per SIMD, still one
+  // workgroup per CU) cover such a cache in ONE round.  Any-length kernel only (unmasked, no offsets).
+  if (n_blocks == 1 && plain_any && wgs8 > 256 && wgs4 <= 768) {
+    for (int cand = 10; cand <= 12; cand += 2) {
+      const int64_t tiles = (sh.seq_len + cand * tqm::kWavePos - 1) / (cand * tqm::kWavePos);
+      if (tiles * sh.n_kv_heads * sh.n_seq <= 256) { nw = cand; break; }
+    }
+  }
   // The streaming pass in more than one round of eight-wave workgroups: four-wave workgroups over the same ranges
   // (twice the blocks of half the size), two to a CU, so that the set-up and the merge of one run under the steps of
   // the other.

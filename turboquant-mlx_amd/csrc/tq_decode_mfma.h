@@ -288,8 +288,9 @@ __device__ __forceinline__ void vonly_tile_body(const MfmaArgs& a, const Codeboo
   // (instalments of 4 + 8 + 4 instructions: the first is what the first score tile needs.  With streaming loads a
   // smaller first instalment lets the value block and the first keys arrive sooner: 9.44 -> 9.02 us against 8 + 4 + 4;
   // 2 + 10 + 4 gives 9.54, 0 + 12 + 4 9.97, 6 + 6 + 4 9.26, 12 or 16 up front 10.1)
-  // The four-wave shape (short caches, two or three workgroups per CU) keeps 8 + 4 + 4: 10.7 against 11.1 us at 16 384.
-  constexpr int kFirstK = NW == 8 ? 4 : 8;
+  // The four-wave shape (short caches, two or three workgroups per CU) keeps 8 + 4 + 4: 10.7 against 11.1 us at 16 384;
+  // the ten- and twelve-wave shapes are one workgroup per CU like the eight-wave one.
+  constexpr int kFirstK = NW >= 8 ? 4 : 8;
 #pragma unroll
   for (int i = 0; i < kFirstK; ++i) issue_k(i);
   __builtin_amdgcn_sched_barrier(0);
@@ -1290,7 +1291,7 @@ __global__ __launch_bounds__(kMergeThreads + 64) void decode_merge_fresh_kernel(
 
 // Which tile kernel a launch uses (chosen by the host from the length, the mask / offsets and the alignment).
 struct VonlyTileChoice {
-  int nw;                     // waves per workgroup: 8 or 4
+  int nw;                     // waves per workgroup: 8 or 4; 10 or 12 (any-length kernel only) just above a full round of 8
   int n_blocks;               // > 1: streaming pass, that many blocks of nw * 64 positions per workgroup
   bool ragged_stream;         // the streaming pass with a ragged end and / or over a ragged batch
   bool plain;                 // full 512-position tiles, no mask, no offsets
@@ -1308,6 +1309,8 @@ void launch_vonly_tiles(dim3 grid, const VonlyTileChoice& c, const MfmaArgs& a, 
   else if (c.n_blocks > 1 && c.ragged_stream) vonly_stream_kernel<QF, true, BITS, 8><<<grid, 512, 0, stream>>>(a, vcb, c.n_blocks); \
   else if (c.n_blocks > 1 && c.nw == 4) vonly_stream_kernel<QF, false, BITS, 4><<<grid, 256, 0, stream>>>(a, vcb, c.n_blocks);  \
   else if (c.n_blocks > 1) vonly_stream_kernel<QF, false, BITS, 8><<<grid, 512, 0, stream>>>(a, vcb, c.n_blocks);  \
+  else if (c.nw == 12) vonly_tile_anylen_kernel<QF, 12, BITS><<<grid, 768, 0, stream>>>(a, vcb);                        \
+  else if (c.nw == 10) vonly_tile_anylen_kernel<QF, 10, BITS><<<grid, 640, 0, stream>>>(a, vcb);                        \
   else if (c.nw == 8 && c.plain) vonly_tile_mfma_kernel<true, QF, 8, BITS><<<grid, 512, 0, stream>>>(a, vcb);           \
   else if (c.nw == 8 && c.plain_any) vonly_tile_anylen_kernel<QF, 8, BITS><<<grid, 512, 0, stream>>>(a, vcb);           \
   else if (c.nw == 8) vonly_tile_mfma_kernel<false, QF, 8, BITS><<<grid, 512, 0, stream>>>(a, vcb);                     \
