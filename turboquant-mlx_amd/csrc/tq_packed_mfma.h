@@ -588,8 +588,8 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
 // batches start a sequence at any row).  They are fetched as ALIGNED 16-byte pieces from the 16-byte
 // boundary at or below the first row (at most 209 pieces) into the wave's LDS image, and rows are
 // read from the image at the misalignment offset.  An aligned 16-byte piece never crosses a page,
-// so a piece that holds at least one valid byte is readable in full; pieces with no valid byte
-// (rows past the end of the sequence) are not fetched and read as zero, and their positions get
+// so a piece that holds at least one valid byte is readable in full; a piece with no valid byte
+// (rows past the end of the sequence) is replaced by the last piece that has one, and such rows get
 // -inf scores.  Rows of the other widths are 16, 32 or 64 bytes: every row of a 16-byte aligned
 // tensor is aligned (the host sends other tensors to the tile pass), and a block is 64, 128 or 256 pieces.
 constexpr int kSWaves = 4;
@@ -652,11 +652,12 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
     const int64_t left = s < n_steps ? len - p0w : 0;      // steps past the workgroup's last have no rows
     return (int)(left < 0 ? 0 : (left > kWavePos ? kWavePos : left));
   };
-  // Requests the rows of step s.  Every call issues the same loads whatever s is: a piece or norm past the end of
-  // the sequence (or a step past the workgroup's last) is fetched from the first piece / row of the workgroup's
-  // range instead, which exists, so that no branch surrounds a load -- the compiler can then count the requests in
-  // flight and wait for one buffer's rows while the other buffer's are still on their way.  What comes back for a
-  // row that does not exist is real data of another row: finite, and its score is set to -inf.
+  // Requests the rows of step s.  Every call issues the same loads whatever s is: a piece past the end of the sequence
+  // is fetched from the last piece of the block that holds a valid byte, a norm past the end (and everything of a step
+  // past the workgroup's last) from the first piece / row of the workgroup's range, which exists, so that no branch
+  // surrounds a load -- the compiler can then count the requests in flight and wait for one buffer's rows while the
+  // other buffer's are still on their way.  What comes back for a row that does not exist is real data of another row:
+  // finite, and its score is set to -inf.
   // Addresses are a base that is the same for the whole workgroup (its first piece / first norm) plus a 32-bit
   // offset per lane: one register per load instead of a 64-bit pointer.
   const char* k_base = krow0 + wg_p0 * (kPd * 4) - kmis;
@@ -666,13 +667,15 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
   auto issue = [&](int s, u4 (&kq)[kLoads], u4 (&vq)[kLoads], float& kn, float& vn) {
     const uint32_t row0 = (uint32_t)(s * kSStepPos + wave * kWavePos);   // first row of the wave's block, from wg_p0
     const int rows = rows_left_of(s);
-    const uint32_t kbytes = rows ? kmis + rows * (kPd * 4) : 0;
-    const uint32_t vbytes = rows ? vmis + rows * (kPd * 4) : 0;
+    // offset of the last piece that holds a valid byte (pieces past it are fetched from there), first byte of the block
+    const uint32_t klast = rows ? ((uint32_t)(kmis + rows * (kPd * 4) - 1) & ~15u) : 0u;
+    const uint32_t vlast = rows ? ((uint32_t)(vmis + rows * (kPd * 4) - 1) & ~15u) : 0u;
+    const uint32_t blk = rows ? row0 * (kPd * 4) : 0u;
 #pragma unroll
     for (int i = 0; i < kLoads; ++i) {
       const uint32_t off = (uint32_t)(i * 64 + lane) * 16;
-      kq[i] = load_stream(k_base + (off < kbytes ? row0 * (kPd * 4) + off : 0u));
-      vq[i] = load_stream(v_base + (off < vbytes ? row0 * (kPd * 4) + off : 0u));
+      kq[i] = load_stream(k_base + (blk + min(off, klast)));
+      vq[i] = load_stream(v_base + (blk + min(off, vlast)));
     }
     const uint32_t nrow = (lane < rows) ? row0 + lane : 0u;
     kn = load_stream(kn_base + nrow);
@@ -767,7 +770,13 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
       const float4 kn4 = *reinterpret_cast<const float4*>(&kn_s[wave][16 * t + 4 * g]);
       const float knv[4] = {kn4.x, kn4.y, kn4.z, kn4.w};
 #pragma unroll
-      for (int j = 0; j < 4; ++j) s[t][j] = (16 * t + 4 * g + j < rows) ? acc[j] * knv[j] : -INFINITY;
+      for (int j = 0; j < 4; ++j) s[t][j] = acc[j] * knv[j];
+    }
+    if (rows < kWavePos) {                                 // only a sequence's last block has rows to mask
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) s[t][j] = (16 * t + 4 * g + j < rows) ? s[t][j] : -INFINITY;
     }
     // ---- value norms, their power-of-two scale
     float vn[4][4];
