@@ -236,9 +236,8 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
   __shared__ __align__(16) uint32_t q_s[kHeadsMax][kD / 2];      // rotated queries as half2: rounded value ...
   __shared__ __align__(16) uint32_t ql_s[kHeadsMax][kD / 2];     // ... and what the rounding lost
   __shared__ __align__(16) float kn_s[kWaves][kWavePos], vn_s[kWaves][kWavePos];
-  __shared__ float m_s[kWaves][kHeadsMax], l_s[kWaves][kHeadsMax], M_s[kHeadsMax];
+  __shared__ float m_s[kWaves][kHeadsMax], l_s[kWaves][kHeadsMax];
   __shared__ __align__(16) MergeLds<kWaves> mg_s;
-  __shared__ float iL_s[kHeadsMax];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -265,6 +264,22 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
   crow = crow < last_row ? crow : last_row;                           // clamped row of this lane
 
   // ---- loads ----------------------------------------------------------------------------------------
+  // kSoftWeights: the weights wait for the fold of the per-tile statistics, so those are requested before anything
+  // else, up to four tiles per thread at once (thread = head tid % 16, tiles tid / 16 + 32 u: 128 tiles per sweep)
+  float2 st_ml[4];
+  int st_tiles = 0;
+  const float* st_base = nullptr;
+  if (MODE == kSoftWeights) {
+    st_tiles = (int)((len + a.stats_tile_pos - 1) / a.stats_tile_pos);
+    st_base = a.stats + (((int64_t)seq * a.n_kv + kvh) * a.n_stats_max) * (int64_t)(n_rep * 2);
+    const int h = tid & 15, part = tid >> 4;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int t = part + 32 * u;
+      st_ml[u] = (h < n_rep && t < st_tiles) ? *reinterpret_cast<const float2*>(st_base + (int64_t)t * (n_rep * 2) + 2 * h)
+                                             : make_float2(-INFINITY, 0.0f);
+    }
+  }
   float2 my_q[2];
   if (HAS_K && !a.q_raw) {
 #pragma unroll
@@ -319,39 +334,48 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
     // out entirely (L = 0) get weight 0.
     float Mh = 0.0f, iL = 1.0f;
     if (MODE == kSoftWeights) {
-      float* part_m = reinterpret_cast<float*>(big_s);                  // [32 parts][16 heads]
-      float* part_l = part_m + 32 * kHeadsMax;
+      float* part_m = reinterpret_cast<float*>(big_s);                  // [8 waves][16 heads]
+      float* part_l = part_m + kWaves * kHeadsMax;
       const int h = tid & 15, part = tid >> 4;
-      const int n_t = (int)((len + a.stats_tile_pos - 1) / a.stats_tile_pos);
-      const float* st = a.stats + (((int64_t)seq * a.n_kv + kvh) * a.n_stats_max) * (int64_t)(n_rep * 2);
       float M = -INFINITY, L = 0.0f;
+      auto fold = [&](const float2 ml) {
+        const float Mn = fmaxf(M, ml.x);
+        if (Mn != -INFINITY) {
+          L = L * __builtin_amdgcn_exp2f(M - Mn) + ml.y * __builtin_amdgcn_exp2f(ml.x - Mn);
+          M = Mn;
+        }
+      };
+#pragma unroll
+      for (int u = 0; u < 4; ++u) fold(st_ml[u]);
       if (h < n_rep) {
-        for (int t = part; t < n_t; t += 32) {
-          const float2 ml = *reinterpret_cast<const float2*>(st + (int64_t)t * (n_rep * 2) + 2 * h);
-          const float Mn = fmaxf(M, ml.x);
-          if (Mn != -INFINITY) {
-            L = L * __builtin_amdgcn_exp2f(M - Mn) + ml.y * __builtin_amdgcn_exp2f(ml.x - Mn);
-            M = Mn;
-          }
-        }
+        for (int t = part + 128; t < st_tiles; t += 32)
+          fold(*reinterpret_cast<const float2*>(st_base + (int64_t)t * (n_rep * 2) + 2 * h));
       }
-      part_m[part * kHeadsMax + h] = M;
-      part_l[part * kHeadsMax + h] = L;
-      __syncthreads();
-      if (tid < kHeadsMax) {
-        float Mt = -INFINITY;
-        for (int p = 0; p < 32; ++p) Mt = fmaxf(Mt, part_m[p * kHeadsMax + tid]);
-        float Lt = 0.0f;
-        for (int p = 0; p < 32; ++p) {
-          const float pm = part_m[p * kHeadsMax + tid];
-          Lt += (pm == -INFINITY) ? 0.0f : part_l[p * kHeadsMax + tid] * __builtin_amdgcn_exp2f(pm - Mt);
-        }
-        M_s[tid] = (Mt == -INFINITY) ? 0.0f : Mt;
-        iL_s[tid] = (Lt > 0.0f) ? 1.0f / Lt : 0.0f;
+      // the four threads of a head in this wave (lanes h + 16 k), then the eight waves through LDS; every thread
+      // folds the eight pairs of ITS head (n16 = h) itself: one barrier, no serial pass over all parts
+#pragma unroll
+      for (int d = 16; d <= 32; d <<= 1) {
+        const float Mo = shfl_xor_f(M, d), Lo = shfl_xor_f(L, d);
+        const float Mn = fmaxf(M, Mo);
+        if (Mn != -INFINITY) L = L * __builtin_amdgcn_exp2f(M - Mn) + Lo * __builtin_amdgcn_exp2f(Mo - Mn);
+        M = Mn;
+      }
+      if (lane < kHeadsMax) {
+        part_m[wave * kHeadsMax + lane] = M;
+        part_l[wave * kHeadsMax + lane] = L;
       }
       __syncthreads();
-      Mh = M_s[n16];
-      iL = iL_s[n16];
+      float Mt = -INFINITY;
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) Mt = fmaxf(Mt, part_m[w * kHeadsMax + n16]);
+      float Lt = 0.0f;
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) {
+        const float pm = part_m[w * kHeadsMax + n16];
+        Lt += (pm == -INFINITY) ? 0.0f : part_l[w * kHeadsMax + n16] * __builtin_amdgcn_exp2f(pm - Mt);
+      }
+      Mh = (Mt == -INFINITY) ? 0.0f : Mt;
+      iL = (Lt > 0.0f) ? 1.0f / Lt : 0.0f;                // (the barrier before the value image is staged protects these reads)
     }
 #pragma unroll
     for (int t = 0; t < 4; ++t)
