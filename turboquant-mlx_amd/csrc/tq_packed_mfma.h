@@ -264,22 +264,6 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
   crow = crow < last_row ? crow : last_row;                           // clamped row of this lane
 
   // ---- loads ----------------------------------------------------------------------------------------
-  // kSoftWeights: the weights wait for the fold of the per-tile statistics, so those are requested before anything
-  // else, up to four tiles per thread at once (thread = head tid % 16, tiles tid / 16 + 32 u: 128 tiles per sweep)
-  float2 st_ml[4];
-  int st_tiles = 0;
-  const float* st_base = nullptr;
-  if (MODE == kSoftWeights) {
-    st_tiles = (int)((len + a.stats_tile_pos - 1) / a.stats_tile_pos);
-    st_base = a.stats + (((int64_t)seq * a.n_kv + kvh) * a.n_stats_max) * (int64_t)(n_rep * 2);
-    const int h = tid & 15, part = tid >> 4;
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int t = part + 32 * u;
-      st_ml[u] = (h < n_rep && t < st_tiles) ? *reinterpret_cast<const float2*>(st_base + (int64_t)t * (n_rep * 2) + 2 * h)
-                                             : make_float2(-INFINITY, 0.0f);
-    }
-  }
   float2 my_q[2];
   if (HAS_K && !a.q_raw) {
 #pragma unroll
@@ -303,10 +287,12 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
   }
   // given weights: lane (head n16, group g) takes positions 16t + 4g + j
   float wgt[4][4];
+  float2 st_ml[4];
+  int st_tiles = 0;
+  const float* st_base = nullptr;
   if (GIVEN) {
     // four consecutive positions per (lane, t): one 16-byte load where the row is aligned and inside the tile.
-    // kSoftWeights: the rows hold scores s in log2 units (absent positions count as -inf); they are fetched
-    // first, so that their latency overlaps the fold of the statistics below.
+    // kSoftWeights: the rows hold scores s in log2 units (absent positions count as -inf).
     const bool vec_ok = ((a.w_stride & 3) == 0) && ((reinterpret_cast<uintptr_t>(a.weights) & 15) == 0);   // uniform
     const float absent = (MODE == kSoftWeights) ? -INFINITY : 0.0f;     // positions outside the tile / heads past n_rep
 #pragma unroll
@@ -329,62 +315,21 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
         }
       }
     }
-    // kSoftWeights: the weight is 2^(s - M) / L with (M, L) of the whole sequence, folded here from the per-tile
-    // pairs the scores pass left (every workgroup folds them itself: a few KB from L2).  Rows that are masked
-    // out entirely (L = 0) get weight 0.
-    float Mh = 0.0f, iL = 1.0f;
+    // kSoftWeights: the per-tile statistics, up to four tiles per thread at once (thread = head tid % 16, tiles
+    // tid / 16 + 32 u: 128 tiles per sweep).  Requested LAST and folded after the value rows have been prepared: they
+    // come back later than the rows (every workgroup of a kv head asks for the same few lines), and a wait for an
+    // earlier request would wait for them too.
     if (MODE == kSoftWeights) {
-      float* part_m = reinterpret_cast<float*>(big_s);                  // [8 waves][16 heads]
-      float* part_l = part_m + kWaves * kHeadsMax;
+      st_tiles = (int)((len + a.stats_tile_pos - 1) / a.stats_tile_pos);
+      st_base = a.stats + (((int64_t)seq * a.n_kv + kvh) * a.n_stats_max) * (int64_t)(n_rep * 2);
       const int h = tid & 15, part = tid >> 4;
-      float M = -INFINITY, L = 0.0f;
-      auto fold = [&](const float2 ml) {
-        const float Mn = fmaxf(M, ml.x);
-        if (Mn != -INFINITY) {
-          L = L * __builtin_amdgcn_exp2f(M - Mn) + ml.y * __builtin_amdgcn_exp2f(ml.x - Mn);
-          M = Mn;
-        }
-      };
 #pragma unroll
-      for (int u = 0; u < 4; ++u) fold(st_ml[u]);
-      if (h < n_rep) {
-        for (int t = part + 128; t < st_tiles; t += 32)
-          fold(*reinterpret_cast<const float2*>(st_base + (int64_t)t * (n_rep * 2) + 2 * h));
+      for (int u = 0; u < 4; ++u) {
+        const int t = part + 32 * u;
+        st_ml[u] = (h < n_rep && t < st_tiles) ? *reinterpret_cast<const float2*>(st_base + (int64_t)t * (n_rep * 2) + 2 * h)
+                                               : make_float2(-INFINITY, 0.0f);
       }
-      // the four threads of a head in this wave (lanes h + 16 k), then the eight waves through LDS; every thread
-      // folds the eight pairs of ITS head (n16 = h) itself: one barrier, no serial pass over all parts
-#pragma unroll
-      for (int d = 16; d <= 32; d <<= 1) {
-        const float Mo = shfl_xor_f(M, d), Lo = shfl_xor_f(L, d);
-        const float Mn = fmaxf(M, Mo);
-        if (Mn != -INFINITY) L = L * __builtin_amdgcn_exp2f(M - Mn) + Lo * __builtin_amdgcn_exp2f(Mo - Mn);
-        M = Mn;
-      }
-      if (lane < kHeadsMax) {
-        part_m[wave * kHeadsMax + lane] = M;
-        part_l[wave * kHeadsMax + lane] = L;
-      }
-      __syncthreads();
-      float Mt = -INFINITY;
-#pragma unroll
-      for (int w = 0; w < kWaves; ++w) Mt = fmaxf(Mt, part_m[w * kHeadsMax + n16]);
-      float Lt = 0.0f;
-#pragma unroll
-      for (int w = 0; w < kWaves; ++w) {
-        const float pm = part_m[w * kHeadsMax + n16];
-        Lt += (pm == -INFINITY) ? 0.0f : part_l[w * kHeadsMax + n16] * __builtin_amdgcn_exp2f(pm - Mt);
-      }
-      Mh = (Mt == -INFINITY) ? 0.0f : Mt;
-      iL = (Lt > 0.0f) ? 1.0f / Lt : 0.0f;                // (the barrier before the value image is staged protects these reads)
     }
-#pragma unroll
-    for (int t = 0; t < 4; ++t)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        float w = wgt[t][j];
-        if (MODE == kSoftWeights) w = __builtin_amdgcn_exp2f(w - Mh) * iL;
-        wgt[t][j] = (w < a.threshold) ? 0.0f : w;
-      }
   }
   if (HAS_K) { if (tid >= 64 && tid < 128) VF::fill(lutk_s, kcb, tid - 64); }
   if (HAS_V) { if (tid < 64) VF::fill(lutv_s, vcb, tid); }
@@ -552,6 +497,63 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
       }
       return;
     }
+  }
+
+  if (GIVEN) {
+    // kSoftWeights: the weight is 2^(s - M) / L with (M, L) of the whole sequence, folded here from the per-tile
+    // pairs the scores pass left (every workgroup folds them itself: a few KB from L2).  Rows that are masked
+    // out entirely (L = 0) get weight 0.
+    float Mh = 0.0f, iL = 1.0f;
+    if (MODE == kSoftWeights) {
+      const int h = tid & 15, part = tid >> 4;
+      float M = -INFINITY, L = 0.0f;
+      auto fold = [&](const float2 ml) {
+        const float Mn = fmaxf(M, ml.x);
+        if (Mn != -INFINITY) {
+          L = L * __builtin_amdgcn_exp2f(M - Mn) + ml.y * __builtin_amdgcn_exp2f(ml.x - Mn);
+          M = Mn;
+        }
+      };
+#pragma unroll
+      for (int u = 0; u < 4; ++u) fold(st_ml[u]);
+      if (h < n_rep) {
+        for (int t = part + 128; t < st_tiles; t += 32)
+          fold(*reinterpret_cast<const float2*>(st_base + (int64_t)t * (n_rep * 2) + 2 * h));
+      }
+      // the four threads of a head in this wave (lanes h + 16 k), then the eight waves through LDS; every thread
+      // folds the eight pairs of ITS head (n16 = h) itself: one barrier, no serial pass over all parts
+#pragma unroll
+      for (int d = 16; d <= 32; d <<= 1) {
+        const float Mo = shfl_xor_f(M, d), Lo = shfl_xor_f(L, d);
+        const float Mn = fmaxf(M, Mo);
+        if (Mn != -INFINITY) L = L * __builtin_amdgcn_exp2f(M - Mn) + Lo * __builtin_amdgcn_exp2f(Mo - Mn);
+        M = Mn;
+      }
+      if (lane < kHeadsMax) {
+        m_s[wave][lane] = M;
+        l_s[wave][lane] = L;
+      }
+      __syncthreads();
+      float Mt = -INFINITY;
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) Mt = fmaxf(Mt, m_s[w][n16]);
+      float Lt = 0.0f;
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) {
+        const float pm = m_s[w][n16];
+        Lt += (pm == -INFINITY) ? 0.0f : l_s[w][n16] * __builtin_amdgcn_exp2f(pm - Mt);
+      }
+      Mh = (Mt == -INFINITY) ? 0.0f : Mt;
+      iL = (Lt > 0.0f) ? 1.0f / Lt : 0.0f;
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float w = wgt[t][j];
+        if (MODE == kSoftWeights) w = __builtin_amdgcn_exp2f(w - Mh) * iL;
+        wgt[t][j] = (w < a.threshold) ? 0.0f : w;
+      }
   }
 
   // ---- weights of the value product -------------------------------------------------------------------
