@@ -1202,6 +1202,33 @@ def test_flash_streaming_pass_group_sizes_and_leading_offset(tq, n_kv, n_rep):
         close(got[i], want)
 
 
+@pytest.mark.parametrize("n_seq,n_kv,n_rep,T,masked", [
+    (1, 8, 4, 5003, False),      # 80 eight-wave tiles: workgroups of four waves over 256-position tiles
+    (1, 8, 4, 10007, False),     # 160: one eight-wave workgroup per CU
+    (2, 8, 2, 9001, True),       # 288, masked: two eight-wave workgroups per CU
+    (1, 2, 16, 257, False), (3, 1, 7, 256, True)])
+def test_flash_tile_pass_workgroup_shapes(tq, n_seq, n_kv, n_rep, T, masked):
+    """The three shapes of the packed tile pass in its flash mode (chosen by how many tiles the call has), each
+    against the oracle, lengths that end inside a wave's rows and one row into a tile, with and without a mask."""
+    rng = np.random.default_rng(5 * T + n_rep)
+    D, bits, sc = 128, 3, 1 / math.sqrt(128)
+    n_q = n_kv * n_rep
+    assert _flash_plan(tq, n_seq, n_kv, T, False, masked) == 0       # the tile pass, not the streaming one
+    c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, n_seq * n_kv, T + 9, D, bits)
+    kp, kn, vp, vn = (a.reshape(n_seq, n_kv, *a.shape[1:]) for a in (kp, kn, vp, vn))
+    q = rng.standard_normal((n_seq, n_q, D)).astype(F32)
+    mask = _draw_mask(rng, "head" if masked else "none", n_seq, n_q, T)
+    kw = {} if mask is None else dict(mask=dev(mask))
+    q_rot = tq.prerotate_query(dev(q.reshape(-1, D)), dev(ks)).reshape(n_seq, n_q, D)
+    got = host(tq.flash_decode(q_rot, dev(kp), dev(kn), dev(vp), dev(vn), c, c, dev(vs), D, bits, sc, n_rep=n_rep,
+                               seq_len=T, **kw))
+    for i in range(n_seq):
+        mi = None if mask is None else np.broadcast_to(mask[i], (n_q, T))
+        want = o.turboquant_attention_single(q[i], kp[i, :, :T], kn[i, :, :T], vp[i, :, :T], vn[i, :, :T], c, ks, c, vs,
+                                             D, bits, sc, mask=mi)
+        close(got[i], want)
+
+
 def encoded_kv_on_gpu(tq, g, n_kv, n_rows, bits, signs, outlier_channel=None):
     """K or V of a benchmark configuration at full size: seeded N(0,1) fp16 rows drawn on the GPU (optionally one
     channel scaled x20), encoded by the library's own encoder -- whose words and norms at this size are compared

@@ -879,13 +879,13 @@ int launch_vonly_mfma(const void* q, int q_dtype, const void* k_f16, const uint3
 }
 
 // the width as a run-time value
-void launch_packed_tiles_bits(int bits, int mode, bool one_per_cu, dim3 grid, const tqm::PackedArgs& a, const Codebook& kcb,
+void launch_packed_tiles_bits(int bits, int mode, int shape, dim3 grid, const tqm::PackedArgs& a, const Codebook& kcb,
                               const Codebook& vcb, hipStream_t stream) {
   switch (bits) {
-    case 1: tqm::launch_packed_tiles<1>(mode, one_per_cu, grid, a, kcb, vcb, stream); break;
-    case 2: tqm::launch_packed_tiles<2>(mode, one_per_cu, grid, a, kcb, vcb, stream); break;
-    case 4: tqm::launch_packed_tiles<4>(mode, one_per_cu, grid, a, kcb, vcb, stream); break;
-    default: tqm::launch_packed_tiles<3>(mode, one_per_cu, grid, a, kcb, vcb, stream); break;
+    case 1: tqm::launch_packed_tiles<1>(mode, shape, grid, a, kcb, vcb, stream); break;
+    case 2: tqm::launch_packed_tiles<2>(mode, shape, grid, a, kcb, vcb, stream); break;
+    case 4: tqm::launch_packed_tiles<4>(mode, shape, grid, a, kcb, vcb, stream); break;
+    default: tqm::launch_packed_tiles<3>(mode, shape, grid, a, kcb, vcb, stream); break;
   }
 }
 
@@ -972,9 +972,23 @@ int launch_packed_mfma(const float* q_rot_or_weights, const uint32_t* k_packed, 
     dim3 grid(a.n_tiles_max, sh.n_kv_heads, sh.n_seq);
     launch_packed_stream_bits(sh.bits, grid, a, kcb, vcb, n_steps, stream);
   } else if (n_tiles_real > 0) {
-    dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
-    // at most one workgroup per CU: the flash variant without spills
-    launch_packed_tiles_bits(sh.bits, MODE, (int64_t)n_tiles * sh.n_kv_heads * sh.n_seq <= 256, grid, a, kcb, vcb, stream);
+    const int64_t wgs8 = (int64_t)n_tiles * sh.n_kv_heads * sh.n_seq;
+    // Short caches (the eight-wave tiles fill at most half of the CUs): workgroups of FOUR waves over tiles of 256
+    // positions, so that a wave has its SIMD to itself -- a tile's time is one wave's chain of key decode, softmax and
+    // value decode, which a second wave on the SIMD stretches.  The partials of the finer tiles must fit the workspace.
+    const int n_tiles4 = (int)((sh.seq_len + 4 * tqm::kWavePos - 1) / (4 * tqm::kWavePos));
+    const size_t need4 = (size_t)sh.n_seq * n_q * n_tiles4 * (tqm::kD + 2) * sizeof(float);
+    if (MODE == tqm::kFlash && wgs8 <= 128 && workspace_bytes >= need4) {
+      tile_pos = 4 * tqm::kWavePos;
+      a.n_tiles_max = n_tiles4;
+      a.ws_ml = a.ws_S + (size_t)sh.n_seq * n_q * n_tiles4 * tqm::kD;
+      dim3 grid(n_tiles4, sh.n_kv_heads, sh.n_seq);
+      launch_packed_tiles_bits(sh.bits, MODE, tqm::kTilesFourWaves, grid, a, kcb, vcb, stream);
+    } else {
+      dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
+      // at most one workgroup per CU: the flash variant without spills
+      launch_packed_tiles_bits(sh.bits, MODE, wgs8 <= 256 ? tqm::kTilesOnePerCu : tqm::kTilesDefault, grid, a, kcb, vcb, stream);
+    }
   }
   TQ_CHECK_LAUNCH(who);
   dim3 mgrid(n_q, sh.n_seq);
@@ -1032,7 +1046,7 @@ int launch_soft_weights(const float* scores, const float* stats, int stats_tile_
   Codebook kcb, vcb;
   fill_codebook(kcb, nullptr, sh.bits);
   a.v_unscale = tq::fill_codebook_fp16(vcb, v_centroids, sh.bits);
-  launch_packed_tiles_bits(sh.bits, tqm::kSoftWeights, false, grid, a, kcb, vcb, stream);
+  launch_packed_tiles_bits(sh.bits, tqm::kSoftWeights, tqm::kTilesDefault, grid, a, kcb, vcb, stream);
   TQ_CHECK_LAUNCH(who);
 
   dim3 mgrid(n_q, sh.n_seq);
@@ -1131,7 +1145,7 @@ int launch_flash_sparse(const float* q_rot, const uint32_t* k_packed, const floa
   Codebook kcb;
   a.score_scale = sh.attn_scale / (float)sh.dim * tq::fill_codebook_fp16(kcb, k_centroids, sh.bits);
   dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
-  launch_packed_tiles_bits(sh.bits, tqm::kSoftScores, false, grid, a, kcb, kcb, stream);
+  launch_packed_tiles_bits(sh.bits, tqm::kSoftScores, tqm::kTilesDefault, grid, a, kcb, kcb, stream);
   TQ_CHECK_LAUNCH(who);
   return launch_soft_weights(scores, stats, tqm::kTilePos, ws_S, ws_ml, t_pad, n_tiles, v_packed, v_norms, v_centroids,
                              v_signs, threshold, out, sh, stream, who);
@@ -1205,7 +1219,7 @@ extern "C" int tq_prerot_qk_scores(const float* q_rot, const uint32_t* k_packed,
     Codebook cbh;
     a.score_scale = tq::fill_codebook_fp16(cbh, centroids, bits) / (float)dim;
     dim3 grid((unsigned)((seq_len + tqm::kTilePos - 1) / tqm::kTilePos), n_kv_heads, 1);
-    launch_packed_tiles_bits(bits, tqm::kScores, false, grid, a, cbh, cbh, (hipStream_t)stream_);
+    launch_packed_tiles_bits(bits, tqm::kScores, tqm::kTilesDefault, grid, a, cbh, cbh, (hipStream_t)stream_);
     TQ_CHECK_LAUNCH("tq_prerot_qk_scores launch");
     return TQ_OK;
   }

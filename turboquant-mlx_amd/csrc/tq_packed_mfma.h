@@ -23,6 +23,7 @@
 namespace tqm {
 
 enum PackedMode { kFlash = 0, kScores = 1, kWeights = 2, kSoftWeights = 3, kSoftScores = 4 };
+enum PackedTileShape { kTilesDefault = 0, kTilesOnePerCu = 1, kTilesFourWaves = 2 };
 
 struct PackedArgs {
   const float* q_rot;         // kFlash / kScores: [n_seq, n_q, 128] f32, pre-rotated; or NULL with q_raw set
@@ -220,9 +221,11 @@ __device__ __forceinline__ void value_products(const u4& A, const uint32_t (&VI)
 // grids that give a CU one workgroup at most.
 // Centroids come from the pair tables here: a workgroup decodes 512 positions once, which does not repay building the
 // 32 KB quad table (measured: scores over 65 536 positions 10.65 us with pairs, 10.95 us with quads).
-template <int MODE, int BITS = 3, int WPE = 4>
-__global__ __launch_bounds__(kMfmaThreads) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
+template <int MODE, int BITS = 3, int WPE = 4, int NW = kWaves>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
 void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
+  static_assert(NW == kWaves || (NW == 4 && MODE == kFlash), "the four-wave shape exists for the flash mode");
+  constexpr int kThr = NW * 64, kPos = NW * kWavePos;               // threads and positions of a workgroup
   using VF = VField<BITS>;
   constexpr int kVPd = VF::kPd;                                      // words per packed row
   constexpr bool GIVEN = MODE == kWeights || MODE == kSoftWeights;   // weights come from memory, no keys
@@ -230,14 +233,14 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
   constexpr bool HAS_V = MODE != kScores && MODE != kSoftScores;
   constexpr bool SOFT = MODE == kFlash || MODE == kSoftScores;        // scores carry attn_scale * log2 e and the mask
   constexpr bool KQUAD = false, VQUAD = false;
-  __shared__ __align__(16) unsigned char big_s[32768];      // per-wave 4 KB areas, later S_all[8][8][128]
+  __shared__ __align__(16) unsigned char big_s[NW * 4096];    // per-wave 4 KB areas, later S_all[NW][8][128]
   __shared__ uint32_t lutk_s[VF::kLut < 64 ? 64 : VF::kLut], lutv_s[VF::kLut < 64 ? 64 : VF::kLut];
   const uint2* quad_s = nullptr;
   __shared__ __align__(16) uint32_t q_s[kHeadsMax][kD / 2];      // rotated queries as half2: rounded value ...
   __shared__ __align__(16) uint32_t ql_s[kHeadsMax][kD / 2];     // ... and what the rounding lost
-  __shared__ __align__(16) float kn_s[kWaves][kWavePos], vn_s[kWaves][kWavePos];
-  __shared__ float m_s[kWaves][kHeadsMax], l_s[kWaves][kHeadsMax];
-  __shared__ __align__(16) MergeLds<kWaves> mg_s;
+  __shared__ __align__(16) float kn_s[NW][kWavePos], vn_s[NW][kWavePos];
+  __shared__ float m_s[NW][kHeadsMax], l_s[NW][kHeadsMax];
+  __shared__ __align__(16) MergeLds<NW> mg_s;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -255,20 +258,21 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
     const int64_t want = *a.len_dev + a.len_bias;
     len = want < 0 ? 0 : (want < len ? want : len);
   }
-  const int64_t tile_p0 = (int64_t)tile * kTilePos;
+  const int64_t tile_p0 = (int64_t)tile * kPos;
   if (tile_p0 >= len) return;
-  const int rows_here = (int)min((int64_t)kTilePos, len - tile_p0);
+  const int rows_here = (int)min((int64_t)kPos, len - tile_p0);
   const int last_row = rows_here - 1;
   const int wrow0 = wave * kWavePos;
   int crow = wrow0 + lane;
   crow = crow < last_row ? crow : last_row;                           // clamped row of this lane
 
   // ---- loads ----------------------------------------------------------------------------------------
-  float2 my_q[2];
+  constexpr int kQIt = kHeadsMax * (kD / 2) / kThr;
+  float2 my_q[kQIt];
   if (HAS_K && !a.q_raw) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int w = tid + i * kMfmaThreads;                           // word = 2 consecutive elements
+    for (int i = 0; i < kQIt; ++i) {
+      const int w = tid + i * kThr;                           // word = 2 consecutive elements
       my_q[i] = (w < n_rep * (kD / 2)) ? reinterpret_cast<const float2*>(a.q_rot + q_row0 * kD)[w]
                                        : make_float2(0.f, 0.f);
     }
@@ -335,14 +339,14 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
   if (HAS_V) { if (tid < 64) VF::fill(lutv_s, vcb, tid); }
   if (HAS_K) {
     if (a.q_raw) {
-      rotate_query_rows<kWaves>(a.q_raw, a.q_dtype, a.k_signs, q_row0, n_rep, wave, lane, q_s, ql_s);
+      rotate_query_rows<NW>(a.q_raw, a.q_dtype, a.k_signs, q_row0, n_rep, wave, lane, q_s, ql_s);
     } else {
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
+      for (int i = 0; i < kQIt; ++i) {
         const __half2 h = __floats2half2_rn(my_q[i].x, my_q[i].y);
         const float2 back = __half22float2(h);
-        (&q_s[0][0])[tid + i * kMfmaThreads] = *reinterpret_cast<const uint32_t*>(&h);
-        (&ql_s[0][0])[tid + i * kMfmaThreads] = pack_h2(my_q[i].x - back.x, my_q[i].y - back.y);
+        (&q_s[0][0])[tid + i * kThr] = *reinterpret_cast<const uint32_t*>(&h);
+        (&ql_s[0][0])[tid + i * kThr] = pack_h2(my_q[i].x - back.x, my_q[i].y - back.y);
       }
     }
     // the score scale rides on the key norm: log2 units for the softmax, plain units for kScores
@@ -483,10 +487,10 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
         if (tid < n_rep) {
           float M = m_s[0][tid];
 #pragma unroll
-          for (int w = 1; w < kWaves; ++w) M = fmaxf(M, m_s[w][tid]);
+          for (int w = 1; w < NW; ++w) M = fmaxf(M, m_s[w][tid]);
           float L = 0.0f;
 #pragma unroll
-          for (int w = 0; w < kWaves; ++w) {
+          for (int w = 0; w < NW; ++w) {
             const float mw = m_s[w][tid];
             L += (mw == -INFINITY) ? 0.0f : l_s[w][tid] * __builtin_amdgcn_exp2f(mw - M);
           }
@@ -536,10 +540,10 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
       __syncthreads();
       float Mt = -INFINITY;
 #pragma unroll
-      for (int w = 0; w < kWaves; ++w) Mt = fmaxf(Mt, m_s[w][n16]);
+      for (int w = 0; w < NW; ++w) Mt = fmaxf(Mt, m_s[w][n16]);
       float Lt = 0.0f;
 #pragma unroll
-      for (int w = 0; w < kWaves; ++w) {
+      for (int w = 0; w < NW; ++w) {
         const float pm = m_s[w][n16];
         Lt += (pm == -INFINITY) ? 0.0f : l_s[w][n16] * __builtin_amdgcn_exp2f(pm - Mt);
       }
@@ -599,7 +603,7 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
   const int64_t grp = (int64_t)seq * a.n_kv + kvh;
   float* pS = a.ws_S + (grp * a.n_tiles_max + tile) * (int64_t)(n_rep * kD);
   float* pml = a.ws_ml + (grp * a.n_tiles_max + tile) * (int64_t)(n_rep * 2);
-  merge_waves<kWaves>(mg_s, big_s, 4096, accS, m, l, inv_tscale, a.v_unscale, n_rep, pS, pml);
+  merge_waves<NW>(mg_s, big_s, 4096, accS, m, l, inv_tscale, a.v_unscale, n_rep, pS, pml);
 }
 
 // Streaming flash-decode pass (packed K and V, no mask): a workgroup of FOUR waves runs through
@@ -890,14 +894,16 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
 
 // Launchers of the kernels above for one width.  Instantiated once per width: 3 beside the host code of the entry
 // points, 1, 2 and 4 in translation units of their own (the widths compile in parallel).
-//   launch_packed_tiles: the tile pass in `mode`; one_per_cu: the grid gives a CU one workgroup at most
+//   launch_packed_tiles: the tile pass in `mode`; shape (flash mode): kTilesOnePerCu when the grid gives a CU one
+//     workgroup at most, kTilesFourWaves for workgroups of four waves (tiles of 256 positions)
 //   launch_packed_stream: the streaming flash pass (no mask); rows of widths other than 3 must be 16-byte aligned
 template <int BITS>
-void launch_packed_tiles(int mode, bool one_per_cu, dim3 grid, const PackedArgs& a, const Codebook& kcb, const Codebook& vcb,
+void launch_packed_tiles(int mode, int shape, dim3 grid, const PackedArgs& a, const Codebook& kcb, const Codebook& vcb,
                          hipStream_t stream) {
   switch (mode) {
     case kFlash:
-      if (one_per_cu) packed_tile_mfma_kernel<kFlash, BITS, 3><<<grid, kMfmaThreads, 0, stream>>>(a, kcb, vcb);
+      if (shape == kTilesFourWaves) packed_tile_mfma_kernel<kFlash, BITS, 2, 4><<<grid, 256, 0, stream>>>(a, kcb, vcb);
+      else if (shape == kTilesOnePerCu) packed_tile_mfma_kernel<kFlash, BITS, 3><<<grid, kMfmaThreads, 0, stream>>>(a, kcb, vcb);
       else packed_tile_mfma_kernel<kFlash, BITS><<<grid, kMfmaThreads, 0, stream>>>(a, kcb, vcb);
       break;
     case kScores: packed_tile_mfma_kernel<kScores, BITS><<<grid, kMfmaThreads, 0, stream>>>(a, kcb, vcb); break;
@@ -920,7 +926,7 @@ void launch_packed_stream(dim3 grid, const PackedArgs& a, const Codebook& kcb, c
 }
 
 #define TQ_PACKED_LAUNCHERS(KEYWORD, B_)                                                                               \
-  KEYWORD template void launch_packed_tiles<B_>(int, bool, dim3, const PackedArgs&, const Codebook&, const Codebook&,  \
+  KEYWORD template void launch_packed_tiles<B_>(int, int, dim3, const PackedArgs&, const Codebook&, const Codebook&,  \
                                                 hipStream_t);                                                          \
   KEYWORD template void launch_packed_stream<B_>(dim3, const PackedArgs&, const Codebook&, const Codebook&, int, hipStream_t);
 #ifndef TQ_WIDTH_HERE
