@@ -1092,7 +1092,7 @@ def test_flash_streaming_pass_ragged(tq):
 
 
 @pytest.mark.parametrize("n_seq,n_kv,n_rep,T,outliers", [(2, 8, 2, 16500, False), (1, 4, 7, 70000, False),
-                                                          (3, 8, 1, 12289, True)])
+                                                          (3, 8, 1, 12289, True), (1, 8, 4, 24001, False)])
 def test_flash_streaming_pass_cache_layout(tq, n_seq, n_kv, n_rep, T, outliers):
     """Cache layout [n_seq, n_kv, T_alloc, *] with a valid length that is not a multiple of anything;
     value norms spread over six decades so that the running power-of-two scale moves between steps."""
@@ -1123,6 +1123,13 @@ def test_flash_plan_masked_and_small_batches_take_the_tile_pass(tq):
     assert _flash_plan(tq, 16, 8, 32768, True, masked=True) == 0
     assert _flash_plan(tq, 16, 8, 32768, True) == 4
     assert _flash_plan(tq, 1, 8, 131072, False) == 8
+    # one four-wave workgroup per CU where three steps reach that and two would leave 384 workgroups
+    assert _flash_plan(tq, 1, 8, 24576, False) == 3
+    assert _flash_plan(tq, 1, 8, 20480, False) == 3
+    assert _flash_plan(tq, 1, 8, 32768, False) == 2
+    assert _flash_plan(tq, 1, 8, 36864, False) == 3
+    assert _flash_plan(tq, 1, 8, 18432, False) == 3
+    assert _flash_plan(tq, 1, 8, 16384, False) == 0
 
 
 def test_encode_fp16_denormal_and_tiny_inputs(tq):

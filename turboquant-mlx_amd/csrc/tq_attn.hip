@@ -911,14 +911,28 @@ void launch_packed_stream_bits(int bits, dim3 grid, const tqm::PackedArgs& a, co
 
 
 // Steps of 256 positions that one workgroup of the streaming flash pass runs through, or 0 for the
-// single-tile pass.  The streaming pass wants at least two workgroups per CU (512 on this part) so
-// that the set-up of one overlaps the arithmetic of another: the largest step count up to 8 that
-// leaves that many; ragged batches (true lengths unknown on the host, max_seq_len is an upper bound)
-// stop at 4, which keeps the tail of the launch short.
+// single-tile pass (at most 512 steps in all).  A step of a wave that has its SIMD to itself (at most
+// one four-wave workgroup per CU, 256 on this part) takes about 2.7 us, a step that shares it (up to two
+// per CU) about 4.2 us, and with more workgroups than that the launch runs in rounds whose set-up overlaps.
+// So: the smallest step count that brings the launch down to 256 workgroups, or the smallest that brings it
+// down to 512, whichever costs less; at most 8 steps, and at most 4 for ragged batches (true lengths
+// unknown on the host, max_seq_len is an upper bound), which keeps the tail of the launch short.  Measured,
+// one sequence of 32 / 8 heads: 24 576 positions 16.7 us with 3 steps (256 workgroups) against 17.9 with 2
+// (384) and 22.4 as single tiles; 18 432 positions 17.0 with 3 steps, 18.2 with 2, 22.0 as single tiles; 36 864
+// positions 21.7 with 3 (384 workgroups), 26.5 with 2 (576), 22.3 with 5 (232).
 int flash_stream_steps(int n_seq, int n_kv, int64_t max_seq_len, bool ragged) {
-  const int64_t units = (int64_t)n_seq * n_kv * ((max_seq_len + tqm::kSStepPos - 1) / tqm::kSStepPos);
-  int n = (int)std::min<int64_t>(ragged ? 4 : 8, units / 512);
-  return n >= 2 ? n : 0;
+  const int64_t steps = (max_seq_len + tqm::kSStepPos - 1) / tqm::kSStepPos;
+  const int64_t groups = (int64_t)n_seq * n_kv;
+  if (groups * steps <= 512) return 0;            // up to 256 eight-wave tiles: the tile pass is as fast (14.7 against 14.9 us)
+  const int cap = ragged ? 4 : 8;
+  int alone = 0, shared = 0;                      // step counts that leave at most 256 / 512 workgroups
+  for (int n = 2; n <= cap; ++n) {
+    const int64_t wgs = groups * ((steps + n - 1) / n);
+    if (!alone && wgs <= 256) alone = n;
+    if (!shared && wgs <= 512) shared = n;
+  }
+  if (!shared) return cap;
+  return (alone && alone * 27 <= shared * 42) ? alone : shared;
 }
 
 // Matrix-core path over packed keys/values: MODE = tqm::kFlash (tq_flash_decode) or tqm::kWeights
