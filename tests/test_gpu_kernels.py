@@ -1681,6 +1681,47 @@ def test_flash_sparse_decode_ragged_and_limits(tq):
                         64, 4, 0.125, n_rep=1, sparse_v_threshold=1e-5)
 
 
+def test_flash_sparse_decode_streaming_scores_pass(tq):
+    """Calls large enough for the streaming form of the scores pass (one statistics entry per workgroup range of several
+    256-position steps): a ragged batch whose sequences start at every misalignment of the 52-byte rows and end inside
+    a step, inside a wave's rows and one row past a step; and a cache layout with an allocation longer than the length."""
+    rng = np.random.default_rng(413)
+    n_kv, n_rep, D, bits, sc, thr = 8, 4, 128, 3, 1 / math.sqrt(128), 1e-5
+    lens = np.array([4097, 2561, 1025, 7000, 1, 3333, 5121, 6143])
+    n_seq = len(lens)
+    assert _flash_plan(tq, n_seq, n_kv, int(lens.max()), True) >= 2
+    offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, n_kv, int(offs[-1]), D, bits)
+    q = rng.standard_normal((n_seq, n_kv * n_rep, D)).astype(F32)
+    q_rot = tq.prerotate_query(dev(q.reshape(-1, D)), dev(ks)).reshape(n_seq, -1, D)
+    got = host(tq.flash_decode(q_rot, dev(kp), dev(kn), dev(vp), dev(vn), c, c, dev(vs), D, bits, sc, n_rep=n_rep,
+                               seq_offsets=dev(offs), max_seq_len=int(lens.max()), sparse_v_threshold=thr))
+    dropped = 0
+    for i in range(n_seq):
+        a, e = offs[i], offs[i + 1]
+        want = o.turboquant_attention_single(q[i], kp[:, a:e], kn[:, a:e], vp[:, a:e], vn[:, a:e], c, ks, c, vs,
+                                             D, bits, sc, sparse_v_threshold=thr)
+        dense = o.turboquant_attention_single(q[i], kp[:, a:e], kn[:, a:e], vp[:, a:e], vn[:, a:e], c, ks, c, vs, D, bits, sc)
+        dropped += int(np.abs(want - dense).max() > 0)
+        w = _packed_weights(q[i], kp[:, a:e], kn[:, a:e], c, ks, sc, n_rep, None)
+        close(got[i], want, extra=threshold_slack(w, thr, vp[:, a:e], vn[:, a:e], c, vs, n_rep, 3e-3))
+    assert dropped >= 4                                      # the threshold removed something in the long sequences
+    # cache layout, two sequences of 9001 positions in an allocation of 9030
+    T, T_alloc = 9001, 9030
+    assert _flash_plan(tq, 2, n_kv, T, False) >= 2
+    c, ks, vs, K, V, kp, kn, vp, vn = kv_fixture(rng, 2 * n_kv, T_alloc, D, bits)
+    kp, kn, vp, vn = (x.reshape(2, n_kv, *x.shape[1:]) for x in (kp, kn, vp, vn))
+    q = rng.standard_normal((2, n_kv * n_rep, D)).astype(F32)
+    q_rot = tq.prerotate_query(dev(q.reshape(-1, D)), dev(ks)).reshape(2, -1, D)
+    got = host(tq.flash_decode(q_rot, dev(kp), dev(kn), dev(vp), dev(vn), c, c, dev(vs), D, bits, sc, n_rep=n_rep,
+                               seq_len=T, sparse_v_threshold=thr))
+    for i in range(2):
+        want = o.turboquant_attention_single(q[i], kp[i, :, :T], kn[i, :, :T], vp[i, :, :T], vn[i, :, :T], c, ks, c, vs,
+                                             D, bits, sc, sparse_v_threshold=thr)
+        w = _packed_weights(q[i], kp[i, :, :T], kn[i, :, :T], c, ks, sc, n_rep, None)
+        close(got[i], want, extra=threshold_slack(w, thr, vp[i, :, :T], vn[i, :, :T], c, vs, n_rep, 3e-3))
+
+
 @pytest.mark.parametrize("seed", range(12))
 def test_decode_sweep_flash_sparse(tq, seed):
     """The thresholded packed-key step on the drawn decode shapes."""

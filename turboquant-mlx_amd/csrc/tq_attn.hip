@@ -899,6 +899,16 @@ void launch_split_tiles_bits(int bits, int mode, dim3 grid, const tqm::SplitArgs
   }
 }
 
+void launch_packed_stream_scores_bits(int bits, dim3 grid, const tqm::PackedArgs& a, const Codebook& kcb, int n_steps,
+                                      hipStream_t stream) {
+  switch (bits) {
+    case 1: tqm::launch_packed_stream_scores<1>(grid, a, kcb, n_steps, stream); break;
+    case 2: tqm::launch_packed_stream_scores<2>(grid, a, kcb, n_steps, stream); break;
+    case 4: tqm::launch_packed_stream_scores<4>(grid, a, kcb, n_steps, stream); break;
+    default: tqm::launch_packed_stream_scores<3>(grid, a, kcb, n_steps, stream); break;
+  }
+}
+
 void launch_packed_stream_bits(int bits, dim3 grid, const tqm::PackedArgs& a, const Codebook& kcb, const Codebook& vcb,
                                int n_steps, hipStream_t stream) {
   switch (bits) {
@@ -1158,10 +1168,22 @@ int launch_flash_sparse(const float* q_rot, const uint32_t* k_packed, const floa
   a.n_kv = sh.n_kv_heads; a.n_rep = sh.n_rep; a.n_tiles_max = n_tiles;
   Codebook kcb;
   a.score_scale = sh.attn_scale / (float)sh.dim * tq::fill_codebook_fp16(kcb, k_centroids, sh.bits);
-  dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
-  launch_packed_tiles_bits(sh.bits, tqm::kSoftScores, tqm::kTilesDefault, grid, a, kcb, kcb, stream);
+  // Large unmasked calls: the scores pass in its streaming form (the rule of the dense step), one statistics entry per
+  // workgroup range of n_steps * 256 positions -- at most as many entries as the tile pass would write.
+  const bool stream_ok = !sh.mask && (sh.bits == 3 || tq::aligned(k_packed, 16));
+  const int n_steps = stream_ok ? flash_stream_steps(sh.n_seq, sh.n_kv_heads, sh.seq_len, sh.seq_offsets != nullptr) : 0;
+  int stats_pos = tqm::kTilePos;
+  if (n_steps >= 2) {
+    stats_pos = tqm::kSStepPos * n_steps;
+    a.n_tiles_max = (int)((sh.seq_len + stats_pos - 1) / stats_pos);
+    dim3 grid(a.n_tiles_max, sh.n_kv_heads, sh.n_seq);
+    launch_packed_stream_scores_bits(sh.bits, grid, a, kcb, n_steps, stream);
+  } else {
+    dim3 grid(n_tiles, sh.n_kv_heads, sh.n_seq);
+    launch_packed_tiles_bits(sh.bits, tqm::kSoftScores, tqm::kTilesDefault, grid, a, kcb, kcb, stream);
+  }
   TQ_CHECK_LAUNCH(who);
-  return launch_soft_weights(scores, stats, tqm::kTilePos, ws_S, ws_ml, t_pad, n_tiles, v_packed, v_norms, v_centroids,
+  return launch_soft_weights(scores, stats, stats_pos, ws_S, ws_ml, t_pad, n_tiles, v_packed, v_norms, v_centroids,
                              v_signs, threshold, out, sh, stream, who);
 }
 

@@ -892,6 +892,221 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
   merge_waves<kSWaves>(mg_s, big_s, 2 * kSImageBytes, accS, m_run, l, inv_tscale, a.v_unscale, n_rep, pS, pml);
 }
 
+// Scores pass of the thresholded flash step in the streaming form (packed K, no mask): the key half of
+// packed_stream_kernel.  A workgroup of four waves runs through n_steps consecutive 256-position steps of one
+// (sequence, kv head); a wave writes the scores of its 64 rows (log2 units) through its LDS area in 256-byte runs per
+// head and keeps the running (maximum, sum of 2^(s - maximum)) of its rows; at the end the four waves are folded into
+// ONE pair per head for the workgroup's range (a.stats_out, [n_seq * n_kv, n_tiles_max, n_rep, 2]), so the weights
+// pass has n_steps * 256 positions per statistics entry.
+template <int BITS>
+__global__ __launch_bounds__(kSThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void packed_stream_scores_kernel(PackedArgs a, Codebook kcb, int n_steps) {
+  using VF = VField<BITS>;
+  constexpr bool KQUAD = VF::kQuad;
+  constexpr int kPd = VF::kPd;
+  constexpr int kPieces = BITS == 3 ? 209 : 16 * kPd;
+  constexpr int kWhole = kPieces / 64, kRest = kPieces % 64;
+  constexpr int kLoads = kWhole + (kRest ? 1 : 0);
+  __shared__ __align__(16) unsigned char big_s[kSWaves * kSImageBytes];   // per wave: K image, then its 64 x 16 scores
+  __shared__ uint32_t lutk_s[VF::kLut < 64 ? 64 : VF::kLut];
+  __shared__ __align__(16) uint2 quad_s[KQUAD ? VF::kQuadEntries : 1];
+  __shared__ __align__(16) uint32_t q_s[kHeadsMax][kD / 2];
+  __shared__ __align__(16) uint32_t ql_s[kHeadsMax][kD / 2];
+  __shared__ __align__(16) float kn_s[kSWaves][kWavePos];
+  __shared__ float m_s[kSWaves][kHeadsMax], l_s[kSWaves][kHeadsMax];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int n16 = lane & 15, g = lane >> 4;
+  const int wg = blockIdx.x, kvh = blockIdx.y, seq = blockIdx.z;
+  const int n_rep = a.n_rep;
+  const int n_q = a.n_kv * n_rep;
+  const int64_t q_row0 = (int64_t)seq * n_q + (int64_t)kvh * n_rep;
+
+  int64_t first = 0, len = a.seq_len;
+  if (a.seq_offsets) {
+    first = a.seq_offsets[seq];
+    len = (int64_t)a.seq_offsets[seq + 1] - first;
+  }
+  const int64_t wg_p0 = (int64_t)wg * kSStepPos * n_steps;
+  if (wg_p0 >= len) return;                              // the weights pass never reads this entry
+
+  const char* krow0 = reinterpret_cast<const char*>(
+      a.k_packed + ((int64_t)seq * a.k_seq_stride + (int64_t)kvh * a.k_head_stride + first) * kPd);
+  const int kmis = BITS == 3 ? (int)((reinterpret_cast<uintptr_t>(krow0) + (uint64_t)wg_p0 * (kPd * 4)) & 15) : 0;
+  const float* knrow0 = a.k_norms + (int64_t)seq * a.kn_seq_stride + (int64_t)kvh * a.kn_head_stride + first;
+  auto rows_left_of = [&](int s) {
+    const int64_t p0w = wg_p0 + (int64_t)s * kSStepPos + wave * kWavePos;
+    const int64_t left = s < n_steps ? len - p0w : 0;
+    return (int)(left < 0 ? 0 : (left > kWavePos ? kWavePos : left));
+  };
+  // requests as in packed_stream_kernel: the same loads whatever s is, no branch around a load
+  const char* k_base = krow0 + wg_p0 * (kPd * 4) - kmis;
+  const float* kn_base = knrow0 + wg_p0;
+  auto issue = [&](int s, u4 (&kq)[kLoads], float& kn) {
+    const uint32_t row0 = (uint32_t)(s * kSStepPos + wave * kWavePos);
+    const int rows = rows_left_of(s);
+    const uint32_t klast = rows ? ((uint32_t)(kmis + rows * (kPd * 4) - 1) & ~15u) : 0u;
+    const uint32_t blk = rows ? row0 * (kPd * 4) : 0u;
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) {
+      const uint32_t off = (uint32_t)(i * 64 + lane) * 16;
+      kq[i] = load_stream(k_base + (blk + min(off, klast)));
+    }
+    kn = load_stream(kn_base + ((lane < rows) ? row0 + lane : 0u));
+  };
+
+  float2 my_q[4];
+  if (!a.q_raw) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int w = tid + i * kSThreads;
+      my_q[i] = (w < n_rep * (kD / 2)) ? reinterpret_cast<const float2*>(a.q_rot + q_row0 * kD)[w] : make_float2(0.f, 0.f);
+    }
+  }
+  u4 kqA[kLoads], kqB[kLoads];
+  float knA, knB = 0.0f;
+  issue(0, kqA, knA);
+
+  if (tid < 64) VF::fill(lutk_s, kcb, tid);
+  if (a.q_raw) {
+    rotate_query_rows<kSWaves>(a.q_raw, a.q_dtype, a.k_signs, q_row0, n_rep, wave, lane, q_s, ql_s);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const __half2 h = __floats2half2_rn(my_q[i].x, my_q[i].y);
+      const float2 back = __half22float2(h);
+      (&q_s[0][0])[tid + i * kSThreads] = *reinterpret_cast<const uint32_t*>(&h);
+      (&ql_s[0][0])[tid + i * kSThreads] = pack_h2(my_q[i].x - back.x, my_q[i].y - back.y);
+    }
+  }
+  __syncthreads();
+  if (KQUAD) {
+    VF::fill_quad(quad_s, lutk_s, tid, kSThreads);
+    __syncthreads();
+  }
+  u4 qreg[4], qlow[4];
+#pragma unroll
+  for (int kb = 0; kb < 4; ++kb) {
+    qreg[kb] = *reinterpret_cast<const u4*>(&q_s[n16][(4 * kb + g) * 4]);
+    qlow[kb] = *reinterpret_cast<const u4*>(&ql_s[n16][(4 * kb + g) * 4]);
+  }
+  unsigned char* image = big_s + wave * kSImageBytes;
+  const uint32_t* kimg = reinterpret_cast<const uint32_t*>(image + kmis);
+  int kw0[4], ksl[4], ksh[4];
+#pragma unroll
+  for (int kb = 0; kb < 4; ++kb) VF::pos(4 * kb + g, kw0[kb], ksl[kb], ksh[kb]);
+  const float kscale = a.score_scale * kLog2e;           // scores in log2 units
+  const bool vec_ok = ((a.w_stride & 3) == 0) && ((reinterpret_cast<uintptr_t>(a.scores) & 15) == 0);   // uniform
+  float m_run = -INFINITY, l_run = 0.0f;
+
+  auto step = [&](int sidx, u4 (&kq)[kLoads], float kn, auto&& next) {
+    const int rows = rows_left_of(sidx);                 // uniform over the wave, at least 1 (the caller checks)
+    __builtin_amdgcn_sched_barrier(0);
+    next();
+    __builtin_amdgcn_sched_barrier(0);
+    {
+      u4* k4 = reinterpret_cast<u4*>(image);
+#pragma unroll
+      for (int i = 0; i < kWhole; ++i) k4[i * 64 + lane] = kq[i];
+      if (kRest) { if (lane < kRest) k4[kWhole * 64 + lane] = kq[kLoads - 1]; }
+      kn_s[wave][lane] = kn * kscale;
+    }
+    float s[4][4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      f4 acc = {0.f, 0.f, 0.f, 0.f};
+      const uint32_t* krow = kimg + (16 * t + n16) * kPd;
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb) {
+        const uint32_t f = VF::field_raw(krow + kw0[kb], ksl[kb], ksh[kb]);
+        const u4 ka = key_operand<BITS, KQUAD>(f, quad_s, lutk_s);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, ka), __builtin_bit_cast(h8, qreg[kb]),
+                                                     acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, ka), __builtin_bit_cast(h8, qlow[kb]),
+                                                     acc, 0, 0, 0);
+      }
+      const float4 kn4 = *reinterpret_cast<const float4*>(&kn_s[wave][16 * t + 4 * g]);
+      const float knv[4] = {kn4.x, kn4.y, kn4.z, kn4.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) s[t][j] = acc[j] * knv[j];
+    }
+    if (rows < kWavePos) {
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) s[t][j] = (16 * t + 4 * g + j < rows) ? s[t][j] : -INFINITY;
+    }
+    // ---- running statistics of head n16 (rows >= 1: the maximum of the step is finite)
+    float mb = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) mb = fmaxf(mb, s[t][j]);
+    mb = max_over_rows(mb);
+    const float m_new = fmaxf(m_run, mb);
+    float lsum = 0.0f;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) lsum += __builtin_amdgcn_exp2f(s[t][j] - m_new);
+    l_run = l_run * __builtin_amdgcn_exp2f(m_run - m_new) + lsum;       // 2^(-inf) = 0 on the wave's first step
+    m_run = m_new;
+    // ---- the scores leave through the wave's LDS area (the key image has been consumed): [16 heads][16 units of
+    // four positions], the unit index xor-ed with the head, so that a store instruction writes 256-byte runs
+    f4* sc = reinterpret_cast<f4*>(image);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) sc[n16 * 16 + ((4 * t + g) ^ n16)] = f4{s[t][0], s[t][1], s[t][2], s[t][3]};
+    const int64_t p0w = wg_p0 + (int64_t)sidx * kSStepPos + wave * kWavePos;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int h = 4 * i + g, unit = n16;
+      if (h < n_rep) {
+        const f4 v = sc[h * 16 + (unit ^ h)];
+        float* dst = a.scores + (q_row0 + h) * a.w_stride + p0w + 4 * unit;
+        if (vec_ok && 4 * unit + 4 <= rows) {
+          *reinterpret_cast<f4*>(dst) = v;
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            if (4 * unit + j < rows) dst[j] = v[j];
+        }
+      }
+    }
+  };
+
+  for (int sidx = 0; sidx < n_steps; sidx += 2) {
+    if (rows_left_of(sidx) <= 0) break;
+    step(sidx, kqA, knA, [&]() { issue(sidx + 1, kqB, knB); });
+    if (sidx + 1 >= n_steps || rows_left_of(sidx + 1) <= 0) break;
+    step(sidx + 1, kqB, knB, [&]() { issue(sidx + 2, kqA, knA); });
+  }
+
+  // ---- one (maximum, sum) pair per head for the workgroup's range; a wave without rows has (-inf, 0)
+  float l = l_run;
+  l += shfl_xor_f(l, 16);
+  l += shfl_xor_f(l, 32);
+  if (g == 0) {
+    m_s[wave][n16] = m_run;
+    l_s[wave][n16] = l;
+  }
+  __syncthreads();
+  if (tid < n_rep) {
+    float M = m_s[0][tid];
+#pragma unroll
+    for (int w = 1; w < kSWaves; ++w) M = fmaxf(M, m_s[w][tid]);
+    float L = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kSWaves; ++w) {
+      const float mw = m_s[w][tid];
+      L += (mw == -INFINITY) ? 0.0f : l_s[w][tid] * __builtin_amdgcn_exp2f(mw - M);
+    }
+    float* pst = a.stats_out + ((((int64_t)seq * a.n_kv + kvh) * a.n_tiles_max) + wg) * (int64_t)(n_rep * 2);
+    pst[2 * tid] = M;
+    pst[2 * tid + 1] = L;
+  }
+}
+
 // Launchers of the kernels above for one width.  Instantiated once per width: 3 beside the host code of the entry
 // points, 1, 2 and 4 in translation units of their own (the widths compile in parallel).
 //   launch_packed_tiles: the tile pass in `mode`; shape (flash mode): kTilesOnePerCu when the grid gives a CU one
@@ -925,10 +1140,16 @@ void launch_packed_stream(dim3 grid, const PackedArgs& a, const Codebook& kcb, c
   packed_stream_kernel<BITS><<<grid, kSThreads, 0, stream>>>(a, kcb, vcb, n_steps);
 }
 
+template <int BITS>
+void launch_packed_stream_scores(dim3 grid, const PackedArgs& a, const Codebook& kcb, int n_steps, hipStream_t stream) {
+  packed_stream_scores_kernel<BITS><<<grid, kSThreads, 0, stream>>>(a, kcb, n_steps);
+}
+
 #define TQ_PACKED_LAUNCHERS(KEYWORD, B_)                                                                               \
   KEYWORD template void launch_packed_tiles<B_>(int, int, dim3, const PackedArgs&, const Codebook&, const Codebook&,  \
                                                 hipStream_t);                                                          \
-  KEYWORD template void launch_packed_stream<B_>(dim3, const PackedArgs&, const Codebook&, const Codebook&, int, hipStream_t);
+  KEYWORD template void launch_packed_stream<B_>(dim3, const PackedArgs&, const Codebook&, const Codebook&, int, hipStream_t); \
+  KEYWORD template void launch_packed_stream_scores<B_>(dim3, const PackedArgs&, const Codebook&, int, hipStream_t);
 #ifndef TQ_WIDTH_HERE
 TQ_PACKED_LAUNCHERS(extern, 1)
 TQ_PACKED_LAUNCHERS(extern, 2)
