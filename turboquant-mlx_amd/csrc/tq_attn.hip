@@ -909,6 +909,16 @@ void launch_packed_stream_scores_bits(int bits, dim3 grid, const tqm::PackedArgs
   }
 }
 
+void launch_packed_stream_weights_bits(int bits, dim3 grid, const tqm::PackedArgs& a, const Codebook& vcb, int n_steps,
+                                       hipStream_t stream) {
+  switch (bits) {
+    case 1: tqm::launch_packed_stream_weights<1>(grid, a, vcb, n_steps, stream); break;
+    case 2: tqm::launch_packed_stream_weights<2>(grid, a, vcb, n_steps, stream); break;
+    case 4: tqm::launch_packed_stream_weights<4>(grid, a, vcb, n_steps, stream); break;
+    default: tqm::launch_packed_stream_weights<3>(grid, a, vcb, n_steps, stream); break;
+  }
+}
+
 void launch_packed_stream_bits(int bits, dim3 grid, const tqm::PackedArgs& a, const Codebook& kcb, const Codebook& vcb,
                                int n_steps, hipStream_t stream) {
   switch (bits) {
@@ -1070,14 +1080,28 @@ int launch_soft_weights(const float* scores, const float* stats, int stats_tile_
   Codebook kcb, vcb;
   fill_codebook(kcb, nullptr, sh.bits);
   a.v_unscale = tq::fill_codebook_fp16(vcb, v_centroids, sh.bits);
-  launch_packed_tiles_bits(sh.bits, tqm::kSoftWeights, tqm::kTilesDefault, grid, a, kcb, vcb, stream);
+  // Large calls: the streaming form (the rule of the dense flash step; a mask only concerns the scores pass), one
+  // partial per workgroup range -- fewer than the tile pass would write, so they fit the same workspace section.
+  const int n_steps = (sh.bits == 3 || tq::aligned(v_packed, 16))
+                          ? flash_stream_steps(sh.n_seq, sh.n_kv_heads, sh.seq_len, sh.seq_offsets != nullptr) : 0;
+  int tile_pos = tqm::kTilePos, n_parts = n_tiles;
+  if (n_steps >= 2) {
+    tile_pos = tqm::kSStepPos * n_steps;
+    n_parts = (int)((sh.seq_len + tile_pos - 1) / tile_pos);
+    a.n_tiles_max = n_parts;
+    a.ws_ml = ws_ml = ws_S + (size_t)sh.n_seq * n_q * n_parts * tqm::kD;
+    dim3 sgrid(n_parts, sh.n_kv_heads, sh.n_seq);
+    launch_packed_stream_weights_bits(sh.bits, sgrid, a, vcb, n_steps, stream);
+  } else {
+    launch_packed_tiles_bits(sh.bits, tqm::kSoftWeights, tqm::kTilesDefault, grid, a, kcb, vcb, stream);
+  }
   TQ_CHECK_LAUNCH(who);
 
   dim3 mgrid(n_q, sh.n_seq);
   const float inv_dim = 1.0f / (float)sh.dim;
 #define LAUNCH_MERGE_S(TO)                                                                                  \
   tqm::decode_merge_rows_kernel<TO, false><<<mgrid, tqm::kMergeThreads, 0, stream>>>(                         \
-      ws_S, ws_ml, sh.seq_offsets, sh.seq_len, n_tiles, sh.n_kv_heads, sh.n_rep, v_signs, inv_dim, (TO*)out, tqm::kTilePos)
+      ws_S, ws_ml, sh.seq_offsets, sh.seq_len, n_parts, sh.n_kv_heads, sh.n_rep, v_signs, inv_dim, (TO*)out, tile_pos)
   if (sh.out_dtype == TQ_F16) { LAUNCH_MERGE_S(__half); }
   else if (sh.out_dtype == TQ_BF16) { LAUNCH_MERGE_S(__hip_bfloat16); }
   else { LAUNCH_MERGE_S(float); }

@@ -899,7 +899,7 @@ void packed_stream_kernel(PackedArgs a, Codebook kcb, Codebook vcb, int n_steps)
 // ONE pair per head for the workgroup's range (a.stats_out, [n_seq * n_kv, n_tiles_max, n_rep, 2]), so the weights
 // pass has n_steps * 256 positions per statistics entry.
 template <int BITS>
-__global__ __launch_bounds__(kSThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
+__global__ __launch_bounds__(kSThreads) __attribute__((amdgpu_waves_per_eu(3, 3)))
 void packed_stream_scores_kernel(PackedArgs a, Codebook kcb, int n_steps) {
   using VF = VField<BITS>;
   constexpr bool KQUAD = VF::kQuad;
@@ -910,8 +910,9 @@ void packed_stream_scores_kernel(PackedArgs a, Codebook kcb, int n_steps) {
   __shared__ __align__(16) unsigned char big_s[kSWaves * kSImageBytes];   // per wave: K image, then its 64 x 16 scores
   __shared__ uint32_t lutk_s[VF::kLut < 64 ? 64 : VF::kLut];
   __shared__ __align__(16) uint2 quad_s[KQUAD ? VF::kQuadEntries : 1];
-  __shared__ __align__(16) uint32_t q_s[kHeadsMax][kD / 2];
-  __shared__ __align__(16) uint32_t ql_s[kHeadsMax][kD / 2];
+  // the rotated query (fp16 value and remainder, 8 KB) is staged in the image area: it is in registers before any image is written
+  uint32_t (*q_s)[kD / 2] = reinterpret_cast<uint32_t (*)[kD / 2]>(big_s);
+  uint32_t (*ql_s)[kD / 2] = reinterpret_cast<uint32_t (*)[kD / 2]>(big_s + kHeadsMax * (kD / 2) * 4);
   __shared__ __align__(16) float kn_s[kSWaves][kWavePos];
   __shared__ float m_s[kSWaves][kHeadsMax], l_s[kSWaves][kHeadsMax];
 
@@ -981,16 +982,14 @@ void packed_stream_scores_kernel(PackedArgs a, Codebook kcb, int n_steps) {
     }
   }
   __syncthreads();
-  if (KQUAD) {
-    VF::fill_quad(quad_s, lutk_s, tid, kSThreads);
-    __syncthreads();
-  }
   u4 qreg[4], qlow[4];
 #pragma unroll
   for (int kb = 0; kb < 4; ++kb) {
     qreg[kb] = *reinterpret_cast<const u4*>(&q_s[n16][(4 * kb + g) * 4]);
     qlow[kb] = *reinterpret_cast<const u4*>(&ql_s[n16][(4 * kb + g) * 4]);
   }
+  if (KQUAD) VF::fill_quad(quad_s, lutk_s, tid, kSThreads);
+  __syncthreads();                                       // every wave has its query operands: the image area is free
   unsigned char* image = big_s + wave * kSImageBytes;
   const uint32_t* kimg = reinterpret_cast<const uint32_t*>(image + kmis);
   int kw0[4], ksl[4], ksh[4];
@@ -1107,6 +1106,238 @@ void packed_stream_scores_kernel(PackedArgs a, Codebook kcb, int n_steps) {
   }
 }
 
+// Weights-and-values pass of the thresholded steps in the streaming form (packed V, scores and per-range statistics
+// from a scores pass): the value half of packed_stream_kernel.  Every workgroup first folds the statistics of its
+// (sequence, kv head) into (M, L) per head; a wave then forms w = 2^(s - M) / L for its 64 rows per step, drops
+// w < threshold, and sums w * norm * centroids on the matrix cores.  No softmax recurrence: the weights are final.
+// What does move from step to step is the power-of-two scale that keeps w * norm inside fp16 (taken from the largest
+// value norm seen so far); the accumulators are rescaled when it grows.  The partial of a workgroup is a plain
+// weighted sum (maximum 0), folded by the merge pass without normalisation.
+template <int BITS>
+__global__ __launch_bounds__(kSThreads) __attribute__((amdgpu_waves_per_eu(3, 3)))
+void packed_stream_weights_kernel(PackedArgs a, Codebook vcb, int n_steps) {
+  using VF = VField<BITS>;
+  constexpr bool VQUAD = VF::kQuad;
+  constexpr int kPd = VF::kPd;
+  constexpr int kPieces = BITS == 3 ? 209 : 16 * kPd;
+  constexpr int kWhole = kPieces / 64, kRest = kPieces % 64;
+  constexpr int kLoads = kWhole + (kRest ? 1 : 0);
+  __shared__ __align__(16) unsigned char big_s[kSWaves * kSImageBytes];   // per wave: V image; later its eight deposit rows
+  __shared__ uint32_t lutv_s[VF::kLut < 64 ? 64 : VF::kLut];
+  __shared__ __align__(16) uint2 quad_s[VQUAD ? VF::kQuadEntries : 1];
+  __shared__ __align__(16) float vn_s[kSWaves][kWavePos];
+  __shared__ float m_s[kSWaves][kHeadsMax], l_s[kSWaves][kHeadsMax];
+  __shared__ __align__(16) MergeLds<kSWaves> mg_s;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int n16 = lane & 15, g = lane >> 4;
+  const int wg = blockIdx.x, kvh = blockIdx.y, seq = blockIdx.z;
+  const int n_rep = a.n_rep;
+  const int n_q = a.n_kv * n_rep;
+  const int64_t q_row0 = (int64_t)seq * n_q + (int64_t)kvh * n_rep;
+
+  int64_t first = 0, len = a.seq_len;
+  if (a.seq_offsets) {
+    first = a.seq_offsets[seq];
+    len = (int64_t)a.seq_offsets[seq + 1] - first;
+  }
+  const int64_t wg_p0 = (int64_t)wg * kSStepPos * n_steps;
+  if (wg_p0 >= len) return;
+
+  const char* vrow0 = reinterpret_cast<const char*>(
+      a.v_packed + ((int64_t)seq * a.v_seq_stride + (int64_t)kvh * a.v_head_stride + first) * kPd);
+  const int vmis = BITS == 3 ? (int)((reinterpret_cast<uintptr_t>(vrow0) + (uint64_t)wg_p0 * (kPd * 4)) & 15) : 0;
+  const float* vnrow0 = a.v_norms + (int64_t)seq * a.vn_seq_stride + (int64_t)kvh * a.vn_head_stride + first;
+  auto rows_left_of = [&](int s) {
+    const int64_t p0w = wg_p0 + (int64_t)s * kSStepPos + wave * kWavePos;
+    const int64_t left = s < n_steps ? len - p0w : 0;
+    return (int)(left < 0 ? 0 : (left > kWavePos ? kWavePos : left));
+  };
+  // Requests of a step: the same loads whatever s is, no branch around a load (see packed_stream_kernel).  The scores
+  // of head n16 (heads past n_rep: head 0) at positions 16 t + 4 g .. + 3 of the wave's rows come as one 16-byte
+  // piece per t (rows of `weights` are w_stride floats, a multiple of four, from a 16-byte aligned base; a row's
+  // padding and the pieces of blocks past the end are read and then masked).
+  const char* v_base = vrow0 + wg_p0 * (kPd * 4) - vmis;
+  const float* vn_base = vnrow0 + wg_p0;
+  const float* sc_base = a.weights + (q_row0 + (n16 < n_rep ? n16 : 0)) * a.w_stride + wg_p0;
+  const bool vec_ok = ((a.w_stride & 3) == 0) && ((reinterpret_cast<uintptr_t>(a.weights) & 15) == 0);   // uniform
+  auto issue = [&](int s, u4 (&vq)[kLoads], float& vn, f4 (&sc)[4]) {
+    const uint32_t row0 = (uint32_t)(s * kSStepPos + wave * kWavePos);
+    const int rows = rows_left_of(s);
+    const uint32_t vlast = rows ? ((uint32_t)(vmis + rows * (kPd * 4) - 1) & ~15u) : 0u;
+    const uint32_t blk = rows ? row0 * (kPd * 4) : 0u;
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) {
+      const uint32_t off = (uint32_t)(i * 64 + lane) * 16;
+      vq[i] = load_stream(v_base + (blk + min(off, vlast)));
+    }
+    vn = load_stream(vn_base + ((lane < rows) ? row0 + lane : 0u));
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const uint32_t at = (16 * t + 4 * g < rows) ? row0 + 16 * t + 4 * g : 0u;   // a piece with no valid position: the range's first
+      if (vec_ok) {
+        sc[t] = __builtin_nontemporal_load(reinterpret_cast<const f4*>(sc_base + at));
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) sc[t][j] = sc_base[at + (16 * t + 4 * g + j < rows ? j : 0)];
+      }
+    }
+  };
+
+  // ---- statistics of this (sequence, kv head): thread = head tid % 16, entries tid / 16 + 16 u
+  float2 st_ml[4];
+  const int st_tiles = (int)((len + a.stats_tile_pos - 1) / a.stats_tile_pos);
+  const float* st_base = a.stats + (((int64_t)seq * a.n_kv + kvh) * a.n_stats_max) * (int64_t)(n_rep * 2);
+  {
+    const int h = tid & 15, part = tid >> 4;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int t = part + 16 * u;
+      st_ml[u] = (h < n_rep && t < st_tiles) ? *reinterpret_cast<const float2*>(st_base + (int64_t)t * (n_rep * 2) + 2 * h)
+                                             : make_float2(-INFINITY, 0.0f);
+    }
+  }
+  u4 vqA[kLoads], vqB[kLoads];
+  float vnA, vnB = 0.0f;
+  f4 scA[4], scB[4];
+  issue(0, vqA, vnA, scA);
+
+  if (tid < 64) VF::fill(lutv_s, vcb, tid);
+  float Mh, iL;
+  {
+    const int h = tid & 15, part = tid >> 4;
+    float M = -INFINITY, L = 0.0f;
+    auto fold = [&](const float2 ml) {
+      const float Mn = fmaxf(M, ml.x);
+      if (Mn != -INFINITY) {
+        L = L * __builtin_amdgcn_exp2f(M - Mn) + ml.y * __builtin_amdgcn_exp2f(ml.x - Mn);
+        M = Mn;
+      }
+    };
+#pragma unroll
+    for (int u = 0; u < 4; ++u) fold(st_ml[u]);
+    if (h < n_rep) {
+      for (int t = part + 64; t < st_tiles; t += 16)
+        fold(*reinterpret_cast<const float2*>(st_base + (int64_t)t * (n_rep * 2) + 2 * h));
+    }
+#pragma unroll
+    for (int d = 16; d <= 32; d <<= 1) {
+      const float Mo = shfl_xor_f(M, d), Lo = shfl_xor_f(L, d);
+      const float Mn = fmaxf(M, Mo);
+      if (Mn != -INFINITY) L = L * __builtin_amdgcn_exp2f(M - Mn) + Lo * __builtin_amdgcn_exp2f(Mo - Mn);
+      M = Mn;
+    }
+    if (lane < kHeadsMax) {
+      m_s[wave][lane] = M;
+      l_s[wave][lane] = L;
+    }
+  }
+  __syncthreads();
+  {
+    float Mt = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < kSWaves; ++w) Mt = fmaxf(Mt, m_s[w][n16]);
+    float Lt = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kSWaves; ++w) {
+      const float pm = m_s[w][n16];
+      Lt += (pm == -INFINITY) ? 0.0f : l_s[w][n16] * __builtin_amdgcn_exp2f(pm - Mt);
+    }
+    Mh = (Mt == -INFINITY) ? 0.0f : Mt;
+    iL = (Lt > 0.0f) ? 1.0f / Lt : 0.0f;                  // rows that are masked out entirely: weight 0
+  }
+  if (VQUAD) {
+    VF::fill_quad(quad_s, lutv_s, tid, kSThreads);
+    __syncthreads();
+  }
+
+  unsigned char* image = big_s + wave * kSImageBytes;
+  const uint32_t* vimg = reinterpret_cast<const uint32_t*>(image + vmis);
+  int vw0, vsl, vsh;
+  VF::pos(n16, vw0, vsl, vsh);
+  const bool head_ok = n16 < n_rep;
+
+  f4 accS[8];
+#pragma unroll
+  for (int et = 0; et < 8; ++et) accS[et] = f4{0.f, 0.f, 0.f, 0.f};
+  int ex_run = 27;                                          // exponent of the scale of the value norms, only grows
+
+  auto step = [&](int sidx, u4 (&vq)[kLoads], float vn_, f4 (&sc)[4], auto&& next) {
+    const int rows = rows_left_of(sidx);                 // uniform over the wave, at least 1 (the caller checks)
+    __builtin_amdgcn_sched_barrier(0);
+    next();
+    __builtin_amdgcn_sched_barrier(0);
+    {
+      u4* v4 = reinterpret_cast<u4*>(image);
+#pragma unroll
+      for (int i = 0; i < kWhole; ++i) v4[i * 64 + lane] = vq[i];
+      if (kRest) { if (lane < kRest) v4[kWhole * 64 + lane] = vq[kLoads - 1]; }
+      vn_s[wave][lane] = vn_;
+    }
+    // ---- value norms, their power-of-two scale (as the tile pass takes it, here a running maximum)
+    float vn[4][4];
+    float nmax = 0.0f;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const float4 n4 = *reinterpret_cast<const float4*>(&vn_s[wave][16 * t + 4 * g]);
+      vn[t][0] = n4.x; vn[t][1] = n4.y; vn[t][2] = n4.z; vn[t][3] = n4.w;
+      nmax = fmaxf(nmax, fmaxf(fmaxf(n4.x, n4.y), fmaxf(n4.z, n4.w)));
+    }
+    nmax = max_over_rows(nmax);
+    int ex = (int)((__float_as_uint(nmax) >> 23) & 0xFF);
+    ex = ex < 27 ? (ex < 1 ? 127 : 27) : (ex > 227 ? 227 : ex);
+    if (sidx == 0) ex_run = ex;
+    if (ex > ex_run) {                                     // uniform: the scale grows, what has been summed shrinks
+      const float shrink = (ex - ex_run < 127) ? __uint_as_float((uint32_t)(127 - (ex - ex_run)) << 23) : 0.0f;
+#pragma unroll
+      for (int et = 0; et < 8; ++et)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) accS[et][j] *= shrink;
+      ex_run = ex;
+    }
+    const float tscale = __uint_as_float((uint32_t)(254 - ex_run) << 23);
+    // ---- weights
+    uint32_t pa[2][4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      float p[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float w = __builtin_amdgcn_exp2f(sc[t][j] - Mh) * iL;
+        w = (w < a.threshold) ? 0.0f : w;
+        w = (head_ok && 16 * t + 4 * g + j < rows) ? w : 0.0f;
+        p[j] = w * (vn[t][j] * tscale);
+      }
+      pa[t >> 1][2 * (t & 1)] = pack_h2(p[0], p[1]);
+      pa[t >> 1][2 * (t & 1) + 1] = pack_h2(p[2], p[3]);
+    }
+    // ---- values
+#pragma unroll
+    for (int kb2 = 0; kb2 < 2; ++kb2) {
+      uint32_t VI[8];
+      value_indices<BITS, VQUAD>(vimg, kb2, g, vw0, vsl, vsh, VI);
+      const u4 A = {pa[kb2][0], pa[kb2][1], pa[kb2][2], pa[kb2][3]};
+      value_products<BITS, VQUAD>(A, VI, quad_s, lutv_s, accS);
+    }
+  };
+
+  for (int sidx = 0; sidx < n_steps; sidx += 2) {
+    if (rows_left_of(sidx) <= 0) break;
+    step(sidx, vqA, vnA, scA, [&]() { issue(sidx + 1, vqB, vnB, scB); });
+    if (sidx + 1 >= n_steps || rows_left_of(sidx + 1) <= 0) break;
+    step(sidx + 1, vqB, vnB, scB, [&]() { issue(sidx + 2, vqA, vnA, scA); });
+  }
+
+  // ---- merge the four waves: plain weighted sums (maximum 0 everywhere), each with its own scale
+  const float inv_tscale = __uint_as_float((uint32_t)ex_run << 23);
+  const int64_t grp = (int64_t)seq * a.n_kv + kvh;
+  float* pS = a.ws_S + (grp * a.n_tiles_max + wg) * (int64_t)(n_rep * kD);
+  float* pml = a.ws_ml + (grp * a.n_tiles_max + wg) * (int64_t)(n_rep * 2);
+  static_assert(kSImageBytes >= 8 * kD * 4 && kSImageBytes % 16 == 0, "a wave's image area holds its eight deposit rows");
+  merge_waves<kSWaves>(mg_s, big_s, kSImageBytes, accS, 0.0f, 0.0f, inv_tscale, a.v_unscale, n_rep, pS, pml);
+}
+
 // Launchers of the kernels above for one width.  Instantiated once per width: 3 beside the host code of the entry
 // points, 1, 2 and 4 in translation units of their own (the widths compile in parallel).
 //   launch_packed_tiles: the tile pass in `mode`; shape (flash mode): kTilesOnePerCu when the grid gives a CU one
@@ -1145,11 +1376,17 @@ void launch_packed_stream_scores(dim3 grid, const PackedArgs& a, const Codebook&
   packed_stream_scores_kernel<BITS><<<grid, kSThreads, 0, stream>>>(a, kcb, n_steps);
 }
 
+template <int BITS>
+void launch_packed_stream_weights(dim3 grid, const PackedArgs& a, const Codebook& vcb, int n_steps, hipStream_t stream) {
+  packed_stream_weights_kernel<BITS><<<grid, kSThreads, 0, stream>>>(a, vcb, n_steps);
+}
+
 #define TQ_PACKED_LAUNCHERS(KEYWORD, B_)                                                                               \
   KEYWORD template void launch_packed_tiles<B_>(int, int, dim3, const PackedArgs&, const Codebook&, const Codebook&,  \
                                                 hipStream_t);                                                          \
   KEYWORD template void launch_packed_stream<B_>(dim3, const PackedArgs&, const Codebook&, const Codebook&, int, hipStream_t); \
-  KEYWORD template void launch_packed_stream_scores<B_>(dim3, const PackedArgs&, const Codebook&, int, hipStream_t);
+  KEYWORD template void launch_packed_stream_scores<B_>(dim3, const PackedArgs&, const Codebook&, int, hipStream_t);          \
+  KEYWORD template void launch_packed_stream_weights<B_>(dim3, const PackedArgs&, const Codebook&, int, hipStream_t);
 #ifndef TQ_WIDTH_HERE
 TQ_PACKED_LAUNCHERS(extern, 1)
 TQ_PACKED_LAUNCHERS(extern, 2)
