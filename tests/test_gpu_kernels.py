@@ -1897,6 +1897,27 @@ def test_vonly_streaming_pass_with_a_ragged_end(tq, n_seq, n_kv, n_rep, T, qdt):
         close(got[i], want, rel=(1e-2 if qdt == "bfloat16" else REL), abs_=(4e-3 if qdt == "bfloat16" else ABS), row_scale=True)
 
 
+@pytest.mark.parametrize("n_seq,n_kv,n_rep,T,qdt", [(4, 8, 2, 10240, "float16"), (3, 8, 1, 18432, "float32")])
+def test_vonly_streaming_pass_block_count_that_does_not_divide_the_length(tq, n_seq, n_kv, n_rep, T, qdt):
+    """Batches whose length is a multiple of 512 positions but where the block count the divisor rule arrives at leaves
+    a short second round of workgroups (20 blocks x 32 pairs in twos: 320 workgroups; 36 x 24 in threes: 288): the host
+    then takes the count with the fewest rounds times blocks (three, which does not divide 20: 224 workgroups; four: 216)
+    and the any-length form of the streaming pass.  Against the oracle."""
+    rng = np.random.default_rng(T + n_seq)
+    D, bits, sc = 128, 3, 1 / math.sqrt(128)
+    c, b = tables(bits)
+    vs = o.random_diagonal_sign(D, 43)
+    assert T % 512 == 0
+    K = rng.standard_normal((n_seq, n_kv, T, D)).astype(np.float16)
+    vp = o.pack_indices(rng.integers(0, 8, size=(n_seq, n_kv, T, D)).astype(np.uint8), bits)
+    vn = ((rng.random((n_seq, n_kv, T)) + 0.5) * np.exp(rng.uniform(-3, 3, size=(n_seq, n_kv, T)))).astype(F32)
+    q = torch.from_numpy(rng.standard_normal((n_seq, n_kv * n_rep, D)).astype(F32)).to(getattr(torch, qdt))
+    got = host(tq.vonly_decode(q.cuda(), dev(K), dev(vp), dev(vn), c, dev(vs), D, bits, sc, n_rep=n_rep).float())
+    for i in range(n_seq):
+        want = o.vonly_decode_attention(q[i].float().numpy(), K[i], vp[i], vn[i], c, vs, D, bits, sc)
+        close(got[i], want, row_scale=True)
+
+
 @pytest.mark.parametrize("n_seq,n_kv,n_rep,T,qdt", [(1, 4, 7, 32769, "float16"), (1, 4, 7, 36864, "float32"),
                                                      (1, 4, 7, 40001, "float16"), (1, 4, 7, 49152, "bfloat16"),
                                                      (2, 8, 4, 10241, "float16"), (1, 8, 2, 24576, "float32")])

@@ -750,6 +750,16 @@ int launch_vonly_mfma(const void* q, int q_dtype, const void* k_f16, const uint3
   if (plain) {
     for (int nb = (int)(wgs8 / 256 < 8 ? wgs8 / 256 : 8); nb > 1; --nb)
       if ((sh.seq_len / tqm::kTilePos) % nb == 0) { n_blocks = nb; break; }
+    // A divisor may leave a short second round (36 blocks x 32 (sequence, kv head) pairs in fours: 288 workgroups, so
+    // 32 CUs carry two): a count that does not divide the length takes the any-length form of the pass when it needs
+    // fewer rounds of 256 workgroups times blocks (there: five blocks, 256 workgroups -- 46.2 -> 36 us).
+    if (n_blocks > 1) {
+      const int64_t blocks = sh.seq_len / tqm::kTilePos, groups = (int64_t)sh.n_kv_heads * sh.n_seq;
+      auto cost = [&](int nb) { return ((((blocks + nb - 1) / nb) * groups + 255) / 256) * nb; };
+      int64_t best = cost(n_blocks);
+      for (int nb = 2; nb <= 8; ++nb)
+        if (cost(nb) < best) { best = cost(nb); n_blocks = nb; ragged_stream = true; }
+    }
   }
   const int64_t wgs4 = ((sh.seq_len + 255) / 256) * sh.n_kv_heads * sh.n_seq;
   if (n_blocks == 1 && plain_base && wgs4 > 768) {
