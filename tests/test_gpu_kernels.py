@@ -1130,6 +1130,8 @@ def test_flash_plan_masked_and_small_batches_take_the_tile_pass(tq):
     assert _flash_plan(tq, 1, 8, 36864, False) == 3
     assert _flash_plan(tq, 1, 8, 18432, False) == 3
     assert _flash_plan(tq, 1, 8, 16384, False) == 0
+    # more than 512 workgroups at any step count: whole rounds (1024 workgroups of five steps, not 640 of eight)
+    assert _flash_plan(tq, 16, 8, 10240, False) == 5
 
 
 def test_encode_fp16_denormal_and_tiny_inputs(tq):

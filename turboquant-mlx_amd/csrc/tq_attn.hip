@@ -961,7 +961,23 @@ int flash_stream_steps(int n_seq, int n_kv, int64_t max_seq_len, bool ragged) {
     if (!alone && wgs <= 256) alone = n;
     if (!shared && wgs <= 512) shared = n;
   }
-  if (!shared) return cap;
+  if (!shared) {
+    // More than two workgroups per CU even at the cap: the launch runs in rounds of 512 workgroups.  A full round costs
+    // the steps of a workgroup at the shared rate (4.2 us each) plus a set-up of about 5 us (the stamps of the kernel; a
+    // sweep of the count over a ragged batch of 16 sequences: 116 / 117 / 108 / 108 us at 2 / 3 / 4 / 6 steps); a last round of at most 256
+    // workgroups runs its steps at the rate of a wave that has its SIMD to itself.  The cheapest count, ties to the
+    // larger.  16 sequences x 8 kv heads x 40 steps: five steps (1024 workgroups, two full rounds) instead of eight
+    // (640: a second round that is a quarter full), 61 -> 54 us on one box.
+    int best_n = cap;
+    int64_t best = INT64_MAX;
+    for (int n = 2; n <= cap; ++n) {
+      const int64_t wgs = groups * ((steps + n - 1) / n);
+      const int64_t rest = wgs % 512;
+      const int64_t cost = (wgs / 512) * (42 * n + 50) + (rest == 0 ? 0 : (rest <= 256 ? 27 : 42) * n + 50);
+      if (cost <= best) { best = cost; best_n = n; }
+    }
+    return best_n;
+  }
   return (alone && alone * 27 <= shared * 42) ? alone : shared;
 }
 
