@@ -1506,8 +1506,8 @@ def test_softmax_rows_shapes(tq, n_rows, T, mask_kind):
     (1, 4, 7, 4099, 1e-5, np.float32, "head"), (2, 3, 5, 1, 1e-5, np.float16, "none"),
     # more than 128 statistics per kv head: the weights pass folds them in more than one sweep
     (1, 2, 7, 40001, 1e-5, np.float16, "none"), (1, 1, 4, 70000, 1e-6, np.float32, "none"),
-    # more than 512 steps of 256 positions in all: the weights pass in its streaming form
-    (2, 8, 2, 9001, 1e-5, np.float16, "none"), (3, 8, 1, 6000, 1e-4, np.float32, "head")])
+    # more than 1024 steps of 256 positions in all: the weights pass in its streaming form
+    (4, 8, 2, 9001, 1e-5, np.float16, "none"), (6, 8, 1, 6000, 1e-4, np.float32, "head")])
 def test_vonly_sparse_decode_matches_oracle(tq, n_seq, n_kv, n_rep, T, thr, qdt, mask_kind):
     """tq_vonly_sparse_decode_attn (scores pass, weights-and-values pass, merge) against the oracle's
     dense scores -> softmax -> thresholded value sum, cache layout with an allocation longer than the
@@ -1636,7 +1636,7 @@ def _packed_weights(q, kp, kn, c, ks, sc, n_rep, mask):
     # more than 128 tiles per kv head: the weights pass folds the statistics in more than one sweep
     (1, 1, 4, 70001, 1e-6, "none"),
     # masked and large: scores by the tile pass, weights and values by the streaming pass
-    (2, 8, 2, 9001, 1e-5, "head")])
+    (4, 8, 2, 9001, 1e-5, "head")])
 def test_flash_sparse_decode_matches_oracle(tq, n_seq, n_kv, n_rep, T, thr, mask_kind):
     """tq_flash_sparse_decode against the oracle's turboquant_attention with a sparse-V threshold
     (scores of packed K -> scale, mask, softmax -> thresholded value sum)."""

@@ -217,7 +217,7 @@ def test_flash_streaming_pass_other_widths_ragged_and_misaligned_storage(tq, bit
 @pytest.mark.parametrize("bits", WIDTHS)
 @pytest.mark.parametrize("n_seq,n_kv,n_rep,T,thr,masked", [(1, 8, 4, 1500, 1e-5, False), (2, 2, 7, 513, 1e-3, True),
                                                            (3, 1, 16, 77, 1e-2, False),
-                                                           (2, 8, 2, 9001, 1e-5, False)])   # streaming scores pass
+                                                           (4, 8, 2, 9001, 1e-5, False)])   # streaming passes
 def test_flash_sparse_decode_other_widths(tq, bits, n_seq, n_kv, n_rep, T, thr, masked):
     """The thresholded decode step over packed keys (scores pass, weights pass, merge pass) against the oracle's
     turboquant_attention with a sparse-V threshold (fused_attention.py:109-121).  A weight within 3e-3 (relative)
