@@ -1129,13 +1129,21 @@ int launch_soft_weights(const float* scores, const float* stats, int stats_tile_
 
   dim3 mgrid(n_q, sh.n_seq);
   const float inv_dim = 1.0f / (float)sh.dim;
-#define LAUNCH_MERGE_S(TO)                                                                                  \
-  tqm::decode_merge_rows_kernel<TO, false><<<mgrid, tqm::kMergeThreads, 0, stream>>>(                         \
+  // partials per lane group and round: one round of loads where 64, 128 or 256 partials cover the sequence
+#define LAUNCH_MERGE_SU(TO, U_)                                                                             \
+  tqm::decode_merge_rows_kernel<TO, false, U_><<<mgrid, tqm::kMergeThreads, 0, stream>>>(                     \
       ws_S, ws_ml, sh.seq_offsets, sh.seq_len, n_parts, sh.n_kv_heads, sh.n_rep, v_signs, inv_dim, (TO*)out, tile_pos)
+#define LAUNCH_MERGE_S(TO)                                                                                  \
+  do {                                                                                                      \
+    if (n_parts <= 64) LAUNCH_MERGE_SU(TO, 8);                                                              \
+    else if (n_parts <= 128) LAUNCH_MERGE_SU(TO, 16);                                                       \
+    else LAUNCH_MERGE_SU(TO, 32);                                                                           \
+  } while (0)
   if (sh.out_dtype == TQ_F16) { LAUNCH_MERGE_S(__half); }
   else if (sh.out_dtype == TQ_BF16) { LAUNCH_MERGE_S(__hip_bfloat16); }
   else { LAUNCH_MERGE_S(float); }
 #undef LAUNCH_MERGE_S
+#undef LAUNCH_MERGE_SU
   TQ_CHECK_LAUNCH(who);
   return TQ_OK;
 }
