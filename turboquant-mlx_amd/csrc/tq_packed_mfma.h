@@ -215,10 +215,12 @@ __device__ __forceinline__ void value_products(const u4& A, const uint32_t (&VI)
   }
 }
 
-// grid = (n_tiles_max, n_kv, n_seq), 512 threads.  BITS: width of the packed keys and values (a cache has one
-// width for both).  WPE = waves per SIMD the registers are budgeted for: 4 lets two workgroups share a CU (the
-// flash mode then spills some registers, which large grids repay); 3 is the flash mode without spills, for
-// grids that give a CU one workgroup at most.
+// grid = (n_tiles_max, n_kv, n_seq), NW * 64 threads, a tile of NW * 64 positions.  BITS: width of the packed keys and
+// values (a cache has one width for both).  WPE = waves per SIMD the registers are budgeted for: 4 lets two eight-wave
+// workgroups share a CU (the flash mode then spills some registers, which large grids repay); 3 is the flash mode
+// without spills, for grids that give a CU one workgroup at most.  NW = 4 (flash mode, budget of two waves per SIMD)
+// is for short caches whose eight-wave tiles would fill at most half of the CUs: twice the workgroups, each wave with
+// its SIMD to itself.
 // Centroids come from the pair tables here: a workgroup decodes 512 positions once, which does not repay building the
 // 32 KB quad table (measured: scores over 65 536 positions 10.65 us with pairs, 10.95 us with quads).
 template <int MODE, int BITS = 3, int WPE = 4, int NW = kWaves>
