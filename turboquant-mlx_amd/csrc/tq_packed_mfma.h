@@ -473,10 +473,9 @@ void packed_tile_mfma_kernel(PackedArgs a, Codebook kcb, Codebook vcb) {
           const int row0 = wrow0 + 4 * unit;
           float* dst = a.scores + ((MODE == kSoftScores ? q_row0 : (int64_t)kvh * n_rep) + h) * row_len + tile_p0 + row0;
           if (vec_ok && row0 + 4 <= rows_here) {
-            // scores handed to the caller leave as streaming stores (10.9 -> 10.3 us at 65 536 positions); those of the
-            // thresholded step are read back by its next pass and keep the default policy
-            if (MODE == kScores) __builtin_nontemporal_store(v, reinterpret_cast<f4*>(dst));
-            else *reinterpret_cast<f4*>(dst) = v;
+            // streaming stores: 10.9 -> 10.3 us for scores handed to the caller at 65 536 positions; the scores of a
+            // thresholded step are read back by its next pass, from the memory side in either case
+            __builtin_nontemporal_store(v, reinterpret_cast<f4*>(dst));
           } else {
 #pragma unroll
             for (int j = 0; j < 4; ++j)
@@ -1066,7 +1065,7 @@ void packed_stream_scores_kernel(PackedArgs a, Codebook kcb, int n_steps) {
         const f4 v = sc[h * 16 + (unit ^ h)];
         float* dst = a.scores + (q_row0 + h) * a.w_stride + p0w + 4 * unit;
         if (vec_ok && 4 * unit + 4 <= rows) {
-          *reinterpret_cast<f4*>(dst) = v;
+          __builtin_nontemporal_store(v, reinterpret_cast<f4*>(dst));
         } else {
 #pragma unroll
           for (int j = 0; j < 4; ++j)
