@@ -43,10 +43,10 @@ THRESHOLD = 1e-5          # sparse-V threshold of the secondary figure: the refe
 # HBM bytes per launch of the dominant kernel (the tile pass), from two rocprofv3 --pmc runs of
 # `python bench.py --steps 60 --warmup 6 --no-cpu --no-graph --no-ceiling` (FETCH_SIZE, then WRITE_SIZE), each
 # scaled by what the same counter reads for `python bench.py --calibrate-copy --steps 40`, a plain
-# copy of ALGO_BYTES bytes (FETCH_SIZE reads 19986.7 for 39950 KiB -> factor 1.9988; WRITE_SIZE
-# reads 39950.0 -> factor 1.0000).  Tile pass: FETCH_SIZE 20071.1 -> 40119 KiB, WRITE_SIZE 916.0
+# copy of ALGO_BYTES bytes (FETCH_SIZE reads 19986.6 for 39950 KiB -> factor 1.9988; WRITE_SIZE
+# reads 39950.0 -> factor 1.0000).  Tile pass: FETCH_SIZE 20071.2 -> 40119 KiB, WRITE_SIZE 916.0
 # -> 916 KiB (run to run the fetch figure moves by a few KiB).  Summary: profiles/vonly_decode_c2_pmc_traffic.md.
-MEASURED_TRAFFIC_BYTES = 42019703  # (20071.1 * 39950.0 / 19986.7 + 916.0) KiB, from the unrounded averages
+MEASURED_TRAFFIC_BYTES = 42019784  # (20071.2 * 39950.0 / 19986.6 + 916.0) KiB, from the unrounded averages
 
 
 def make_sets(torch, tqhip, dev):
