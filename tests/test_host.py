@@ -330,3 +330,50 @@ def test_matrix_core_shape_predicates():
     for dim, bits, n_rep in ((64, 3, 1), (256, 3, 4), (128, 3, 17), (128, 3, 0), (128, 5, 1), (128, 0, 1)):
         assert not ops.vonly_threshold_supported(dim, bits, n_rep)
         assert not ops.vonly_sparse_supported(dim, bits, n_rep)
+
+
+def _plan_restated(n_seq, n_kv, max_len, ragged, masked):
+    """The step rule of the streaming flash pass, restated: steps of 256 positions per workgroup, 0 for the tile pass."""
+    if masked:
+        return 0
+    steps, groups = -(-max_len // 256), n_seq * n_kv
+    if groups * steps <= 512:
+        return 0
+    cap = 4 if ragged else 8
+    wgs = lambda n: groups * -(-steps // n)
+    alone = next((n for n in range(2, cap + 1) if wgs(n) <= 256), 0)
+    shared = next((n for n in range(2, cap + 1) if wgs(n) <= 512), 0)
+    if shared:
+        return alone if alone and alone * 27 <= shared * 42 else shared
+    best, best_n = None, cap
+    for n in range(2, cap + 1):
+        rest = wgs(n) % 512
+        cost = (wgs(n) // 512) * (42 * n + 50) + (0 if rest == 0 else (27 if rest <= 256 else 42) * n + 50)
+        if best is None or cost <= best:
+            best, best_n = cost, n
+    return best_n
+
+
+def test_flash_decode_plan_follows_its_rule_on_host():
+    """tq_flash_decode_plan is host arithmetic (no launch): known picks, and a grid of shapes against the restated rule.
+    Every pick leaves no workgroup without work at the front of a sequence: steps * 256 * (workgroups - 1) < length."""
+    lib = _lib.load()
+    plan = lambda *a: lib.tq_flash_decode_plan(*a)
+    assert plan(1, 4, 4096, 0, 0) == 0                      # short: the tile pass
+    assert plan(16, 8, 32768, 1, 1) == 0                    # masked: the tile pass
+    assert plan(1, 8, 16384, 0, 0) == 0                     # exactly 512 steps: one eight-wave tile per CU
+    assert plan(1, 8, 18432, 0, 0) == 3                     # one four-wave workgroup per CU (192) beats two (288)
+    assert plan(1, 8, 32768, 0, 0) == 2
+    assert plan(1, 8, 131072, 0, 0) == 8
+    assert plan(16, 8, 32768, 1, 0) == 4                    # ragged batches stop at four steps
+    assert plan(16, 8, 10240, 0, 0) == 5                    # whole rounds: 1024 workgroups of five steps, not 640 of eight
+    for n_seq in (1, 2, 3, 5, 16):
+        for n_kv in (1, 4, 8):
+            for max_len in (1, 255, 256, 4097, 16384, 16385, 20000, 36864, 65536, 131072, 1000000):
+                for ragged in (0, 1):
+                    for masked in (0, 1):
+                        got = plan(n_seq, n_kv, max_len, ragged, masked)
+                        assert got == _plan_restated(n_seq, n_kv, max_len, ragged, masked), (n_seq, n_kv, max_len, ragged, masked)
+                        if got:
+                            assert 2 <= got <= (4 if ragged else 8)
+                            assert got * 256 * (-(-max_len // (got * 256)) - 1) < max_len
